@@ -1,0 +1,184 @@
+/*
+ * ema_hip.h -- C ABI of libema_hip.so: the EMA chunked scan (forward and backward) as
+ * hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Every entry point replaces one launcher of the reference repository
+ * kartiksrinivas007/triton-kernels (a Python function that allocates its output and starts
+ * one Triton kernel); the citation on each declaration is that launcher, with paths
+ * relative to the reference root.
+ *
+ * Conventions
+ *   - All pointers are DEVICE pointers.  The caller allocates every input, output and
+ *     workspace; the library never allocates, frees or keeps a pointer.
+ *   - Work is only enqueued on `stream` (a hipStream_t passed as void*; NULL = the null
+ *     stream).  No entry point synchronises or reads anything back, so all of them may be
+ *     captured into a HIP graph.
+ *   - Sequence tensors (x, y, dy, dx) are addressed as
+ *         ptr[b * s_b + l * s_l + h * s_h + t],   b < batch, l < seqlen, h < nheads, t < dim
+ *     with strides in ELEMENTS and a unit stride along `dim`.  The reference's flat
+ *     layout (B, L, T) is nheads = 1; the headed layout (b, L, nh, d) is s_b = L*nh*d,
+ *     s_l = nh*d, s_h = d.  The log-decay A (float32) is addressed the same way without
+ *     the `dim` axis.  A sequence index n = b * nheads + h numbers the independent scans;
+ *     N = batch * nheads.
+ *   - Chunked intermediates are dense float32: cs (N, C, Q), states / prev / ds / g
+ *     (N, C, T), final (N, T), per-chunk scalars (N, C); C = ceil(seqlen / chunk).
+ *   - `dtype` is the element type of the sequence tensors (ema_dtype); accumulation is
+ *     always float32.  dim must be a multiple of 8 (bf16) or 4 (f32) and row starts must
+ *     be 16-byte aligned.
+ *   - Return value: EMA_OK (0) or a negative ema_status.  Arguments are validated before
+ *     anything is launched; nothing is thrown across the boundary.
+ */
+#ifndef EMA_HIP_H
+#define EMA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  EMA_OK = 0,
+  EMA_ERR_NULL = -1,        /* a required pointer is NULL */
+  EMA_ERR_SHAPE = -2,       /* a dimension is <= 0 or out of the supported range */
+  EMA_ERR_ALIGN = -3,       /* dim / strides / pointers break the 16-byte rule */
+  EMA_ERR_DTYPE = -4,       /* unknown ema_dtype */
+  EMA_ERR_UNSUPPORTED = -5, /* a feature the reference also rejects */
+  EMA_ERR_LAUNCH = -6       /* hipGetLastError() after a launch was not hipSuccess */
+} ema_status;
+
+typedef enum { EMA_F32 = 0, EMA_BF16 = 1 } ema_dtype;
+
+/* Largest chunk size accepted by every entry point. */
+#define EMA_MAX_CHUNK 1024
+
+const char* ema_version(void);
+const char* ema_status_string(int status);
+
+/* ---------------------------------------------------------------- forward stages ---- */
+
+/* F1: cs[n,c,q] = sum_{j<=q} A[n, c*Q+j], restarting every chunk, positions past seqlen
+ * adding 0.  Replaces ema_chunk_cumsum_fwd, kernels/ema_kernels/ema_cumsum.py:66-80. */
+int ema_chunk_cumsum_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh,
+                         float* cs, int64_t batch, int64_t nheads, int64_t seqlen,
+                         int64_t chunk, void* stream);
+
+/* F2: states[n,c,t] = sum_q exp(min(cs[n,c,Q-1]-cs[n,c,q],0)) * x[n,c*Q+q,t].
+ * Replaces _ema_chunk_state_fwd, kernels/ema_kernels/ema_state_fwd.py:130-163. */
+int ema_chunk_state_fwd(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype,
+                        const float* cs, float* states, int64_t batch, int64_t nheads,
+                        int64_t seqlen, int64_t dim, int64_t chunk, void* stream);
+
+/* F3: S_0 = 0; prev[n,c] = S_c; S_{c+1} = exp(cs_last[n,c]) * S_c + states[n,c];
+ * final[n] = S_C.  cs_last is addressed as cs_last[n*cl_sn + c*cl_sc] so that the strided
+ * view cs[..., -1] can be passed without a copy.
+ * Replaces _ema_state_passing_fwd, kernels/ema_kernels/ema_state_pass.py:125-154. */
+int ema_state_passing_fwd(const float* states, const float* cs_last, int64_t cl_sn,
+                          int64_t cl_sc, float* prev, float* final_state, int64_t nseq,
+                          int64_t nchunks, int64_t dim, void* stream);
+
+/* F4: y[n,c*Q+m,t] = exp(min(cs[m],0)) * prev[n,c,t]
+ *                   + sum_{k<=m} exp(min(cs[m]-cs[k],0)) * x[n,c*Q+k,t].
+ * Replaces _ema_scan_fwd, kernels/ema_kernels/ema_scan_fwd.py:161-193. */
+int ema_scan_fwd(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype,
+                 const float* cs, const float* prev, void* y, int64_t y_sb, int64_t y_sl,
+                 int64_t y_sh, int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
+                 int64_t chunk, void* stream);
+
+/* Bytes of workspace ema_fwd needs (the chunk-local states). */
+size_t ema_fwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
+                               int64_t chunk);
+
+/* F1..F4 in sequence.  Outputs y, cs (N,C,Q), prev (N,C,T), final (N,T).
+ * Replaces _ema_matmul_scan_combined_fwd, kernels/ema_kernels/ema_combined_fwd.py:12-45. */
+int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void* x,
+            int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb,
+            int64_t y_sl, int64_t y_sh, float* cs, float* prev, float* final_state,
+            void* workspace, size_t workspace_bytes, int64_t batch, int64_t nheads,
+            int64_t seqlen, int64_t dim, int64_t chunk, void* stream);
+
+/* --------------------------------------------------------------- backward stages ---- */
+
+/* B1: ds[n,c,t] = sum_m exp(cs[n,c,m]) * dy[n,c*Q+m,t].
+ * Replaces _ema_chunk_scan_bwd_dstates, kernels/ema_kernels_bwd/ema_scan_bwd.py:132-153. */
+int ema_chunk_scan_bwd_dstates(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh,
+                               int dtype, const float* cs, float* ds, int64_t batch,
+                               int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk,
+                               void* stream);
+
+/* Bytes of workspace ema_state_passing_bwd needs (per-wave partial dot products). */
+size_t ema_state_passing_bwd_workspace_bytes(int64_t nseq, int64_t nchunks, int64_t dim);
+
+/* B2: g[n,C-1] = 0; g[n,c-1] = exp(cs_last[n,c]) * g[n,c] + ds[n,c];
+ * ddA_chunk[n,c] = exp(cs_last[n,c]) * <prev[n,c], g[n,c]>, ddA_chunk[n,0] = 0.
+ * Replaces _ema_state_passing_bwd,
+ * kernels/ema_kernels_bwd/ema_state_passing_bwd_dstates.py:103-183. */
+int ema_state_passing_bwd(const float* prev, const float* cs_last, int64_t cl_sn,
+                          int64_t cl_sc, const float* ds, float* g, float* ddA_chunk,
+                          void* workspace, size_t workspace_bytes, int64_t nseq,
+                          int64_t nchunks, int64_t dim, void* stream);
+
+/* B3: dx[n,c*Q+m,t] = exp(min(cs[Q-1]-cs[m],0)) * g[n,c,t]
+ *                    + sum_{k>=m} exp(min(cs[k]-cs[m],0)) * dy[n,c*Q+k,t].
+ * Replaces _chunk_scan_chunk_state_bwd_dx,
+ * kernels/ema_kernels_bwd/ema_chunk_scan_chunk_state_bwd_dx.py:208-262. */
+int ema_chunk_scan_chunk_state_bwd_dx(const void* dy, int64_t dy_sb, int64_t dy_sl,
+                                      int64_t dy_sh, int dtype, const float* cs,
+                                      const float* g, void* dx, int64_t dx_sb, int64_t dx_sl,
+                                      int64_t dx_sh, int64_t batch, int64_t nheads,
+                                      int64_t seqlen, int64_t dim, int64_t chunk,
+                                      void* stream);
+
+/* B4: r[m] = exp(min(cs[Q-1]-cs[m],0)) * <g[n,c], x[n,c*Q+m]> written to slot m+1
+ * (slot 0 = 0); when raw == 0 an inclusive cumsum along the chunk follows, giving
+ * ddA_next[j] = sum_{m<j} r[m].  Output (N,C,Q).
+ * Replaces _ema_chunk_state_bwd_db,
+ * kernels/ema_kernels_bwd/ema_chunk_state_bwd_db.py:122-152. */
+int ema_chunk_state_bwd_db(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
+                           int dtype, const float* cs, const float* g, float* ddA_next,
+                           int raw, int64_t batch, int64_t nheads, int64_t seqlen,
+                           int64_t dim, int64_t chunk, void* stream);
+
+/* B5: s[n,c,m] = exp(cs[n,c,m]) * <dy[n,c*Q+m], prev[n,c]> (0 past seqlen).  Output
+ * (N,C,Q), before the reverse cumsum.
+ * Replaces _ema_chunk_scan_bwd_dC, kernels/ema_kernels_bwd/ema_chunk_scan_bwd_dc.py:115-147. */
+int ema_chunk_scan_bwd_dc(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh,
+                          int dtype, const float* prev, const float* cs, float* ddA_prev,
+                          int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
+                          int64_t chunk, void* stream);
+
+/* Bytes of workspace ema_chunk_scan_bwd_ddAcs needs (per-row-tile partial sums). */
+size_t ema_chunk_scan_bwd_ddAcs_workspace_bytes(int64_t batch, int64_t nheads,
+                                                int64_t seqlen, int64_t chunk);
+
+/* B6: G[m,k] = exp(min(cs[m]-cs[k],0)) * <dy[m], x[k]> for k < m;
+ * ddA_intra[j] = sum_{m>=j} sum_{k<j} G[m,k], ddA_intra[0] = 0.  Output (N,C,Q).
+ * Replaces _ema_chunk_scan_bwd_ddAcs_stable,
+ * kernels/ema_kernels_bwd/ema_scan_da.py:113-137. */
+int ema_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
+                             const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh,
+                             int dtype, const float* cs, float* ddA_intra, void* workspace,
+                             size_t workspace_bytes, int64_t batch, int64_t nheads,
+                             int64_t seqlen, int64_t dim, int64_t chunk, void* stream);
+
+/* Bytes of workspace ema_bwd needs (cs, states, prev, ds, g and the partial sums). */
+size_t ema_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
+                               int64_t chunk);
+
+/* Whole backward: recomputes F1..F3, then B1..B6 and their sum.  Outputs dx (layout of x)
+ * and ddA (N,C,Q) float32 with ddA[n,c,q] = dL/dA[n, c*Q+q]; when y is not NULL the
+ * forward output is recomputed into it (the reference's recompute_output=True).
+ * Replaces _ema_chunk_scan_combined_bwd,
+ * kernels/ema_kernels_bwd/ema_combined_bwd.py:13-83. */
+int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const void* x,
+            int64_t x_sb, int64_t x_sl, int64_t x_sh, const float* A, int64_t a_sb,
+            int64_t a_sl, int64_t a_sh, int dtype, void* dx, int64_t dx_sb, int64_t dx_sl,
+            int64_t dx_sh, float* ddA, void* y, int64_t y_sb, int64_t y_sl, int64_t y_sh,
+            void* workspace, size_t workspace_bytes, int64_t batch, int64_t nheads,
+            int64_t seqlen, int64_t dim, int64_t chunk, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EMA_HIP_H */

@@ -1,0 +1,94 @@
+"""CPU-side checks of the C ABI: the built library loads, exports every symbol that
+include/ema_hip.h declares, and validates its arguments before launching anything (so the
+refusals can be exercised without a GPU)."""
+import os
+import re
+
+import pytest
+
+from kernels import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "ema_hip.h")
+
+
+def declared_functions():
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(ema_[a-z_A-Z0-9]+)\s*\(", src)))
+
+
+def test_header_and_binding_agree():
+    assert declared_functions() == _lib.exported_symbols()
+
+
+def test_library_exports_every_declared_symbol():
+    handle = _lib.lib()
+    for name in declared_functions():
+        assert hasattr(handle, name), name
+    assert b"gfx950" in handle.ema_version()
+
+
+def test_status_strings():
+    handle = _lib.lib()
+    assert handle.ema_status_string(0) == b"ok"
+    for code in range(-6, 0):
+        assert handle.ema_status_string(code) not in (b"ok", b"unknown status")
+
+
+def test_workspace_sizes():
+    handle = _lib.lib()
+    # config 2: N=32, C=32, T=1024, Q=128
+    assert handle.ema_fwd_workspace_bytes(16, 2, 4096, 1024, 128) == 32 * 32 * 1024 * 4
+    assert handle.ema_state_passing_bwd_workspace_bytes(32, 32, 1024) == 32 * 32 * 16 * 4
+    assert handle.ema_chunk_scan_bwd_ddAcs_workspace_bytes(16, 2, 4096, 128) == 2 * 32 * 32 * 128 * 4
+    assert handle.ema_bwd_workspace_bytes(16, 2, 4096, 1024, 128) > 4 * 32 * 32 * 1024 * 4
+    # refused shapes report 0 bytes
+    assert handle.ema_fwd_workspace_bytes(0, 2, 4096, 1024, 128) == 0
+    assert handle.ema_bwd_workspace_bytes(16, 2, 4096, 1024, _lib.EMA_MAX_CHUNK + 1) == 0
+
+
+def test_validation_happens_before_any_launch():
+    handle = _lib.lib()
+    fake = 0x1000  # 16-byte aligned, never dereferenced: every call below is refused
+    # null pointers
+    assert handle.ema_chunk_cumsum_fwd(None, 1, 1, 0, fake, 1, 1, 8, 4, None) == -1
+    # bad shapes
+    assert handle.ema_chunk_cumsum_fwd(fake, 8, 1, 0, fake, 0, 1, 8, 4, None) == -2
+    assert handle.ema_chunk_cumsum_fwd(fake, 8, 1, 0, fake, 1, 1, 8, 0, None) == -2
+    assert handle.ema_chunk_cumsum_fwd(fake, 8, 1, 0, fake, 1, 1, 8, 2048, None) == -2
+    # feature size / strides that break 16-byte rows
+    assert handle.ema_chunk_state_fwd(fake, 48, 6, 0, _lib.EMA_F32, fake, fake, 1, 1, 8, 6, 4, None) == -3
+    assert handle.ema_chunk_state_fwd(fake, 64, 8, 0, _lib.EMA_BF16, fake, fake, 1, 1, 8, 4, 4, None) == -3
+    assert handle.ema_chunk_state_fwd(fake + 2, 64, 8, 0, _lib.EMA_BF16, fake, fake, 1, 1, 8, 8, 4, None) == -3
+    # unknown dtype
+    assert handle.ema_chunk_state_fwd(fake, 64, 8, 0, 7, fake, fake, 1, 1, 8, 8, 4, None) == -4
+    # workspace too small
+    assert (
+        handle.ema_fwd(fake, 8, 1, 0, fake, 64, 8, 0, _lib.EMA_F32, fake, 64, 8, 0, fake, fake, fake,
+                       fake, 16, 1, 1, 8, 8, 4, None)
+        == -2
+    )
+
+
+def test_error_mapping():
+    with pytest.raises(AssertionError):
+        _lib.check(-2, "x")
+    with pytest.raises(AssertionError):
+        _lib.check(-3, "x")
+    with pytest.raises(TypeError):
+        _lib.check(-4, "x")
+    with pytest.raises(NotImplementedError):
+        _lib.check(-5, "x")
+    with pytest.raises(RuntimeError):
+        _lib.check(-6, "x")
+    _lib.check(0, "x")
+
+
+def test_ops_refuse_cpu_tensors():
+    import torch
+
+    from kernels.ema_kernels.ema_cumsum import ema_chunk_cumsum_fwd
+
+    with pytest.raises(RuntimeError):
+        ema_chunk_cumsum_fwd(torch.zeros(1, 8), 4)

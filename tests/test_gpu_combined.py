@@ -1,0 +1,185 @@
+"""GPU parity of the combined forward / backward and of the autograd entry point against
+the sequential CPU oracle, including BASELINE configurations 1-4 at their full sizes."""
+import pytest
+import torch
+
+from oracle import ema_oracle as O
+from parity_util import announce, check_close, flat_case
+
+pytestmark = pytest.mark.gpu
+
+F32, BF16 = torch.float32, torch.bfloat16
+
+
+def _run_flat(A, X, dy, Q, device, recompute_output=False):
+    from kernels.ema_kernels.ema_combined_fwd import _ema_matmul_scan_combined_fwd
+    from kernels.ema_kernels_bwd.ema_combined_bwd import _ema_chunk_scan_combined_bwd
+
+    Ad, Xd, dyd = A.to(device), X.to(device), dy.to(device)
+    y, cs, prev, final = _ema_matmul_scan_combined_fwd(Ad, Xd, Q)
+    res = _ema_chunk_scan_combined_bwd(dyd, Xd, Ad, Q, recompute_output=recompute_output)
+    torch.cuda.synchronize()
+    return y, cs, prev, final, res
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize(
+    "N,L,T,Q,kind",
+    [
+        (4, 2048, 512, 128, "neg_rand"),  # tests/ema_bwd/_ema_full_bwd.py:56-79, L shortened
+        (2, 1000, 64, 128, "sigmoid"),    # ragged
+        (2, 640, 136, 64, "sigmoid"),
+        (1, 2048, 128, 512, "sigmoid"),
+        (3, 200, 8, 256, "sigmoid"),      # one ragged chunk
+        (2, 1, 8, 128, "sigmoid"),        # L = 1
+    ],
+)
+def test_combined_vs_sequential(N, L, T, Q, kind, dtype, device):
+    announce(f"combined N{N} L{L} T{T} Q{Q} {kind} {dtype}")
+    A, X, dy = flat_case(N, L, T, seed=77 + L + T, dtype=dtype, kind=kind)
+    y, cs, prev, final, (dx, ddA, y2) = _run_flat(A, X, dy, Q, device, recompute_output=True)
+    y_ref = O.ema_loop(X.float(), A)
+    dx_ref, dA_ref = O.ema_loop_bwd(dy.float(), X.float(), A)
+    check_close("y", y, y_ref, dtype)
+    check_close("y (recomputed in bwd)", y2, y_ref, dtype)
+    check_close("final", final, y_ref[:, -1], F32 if dtype == F32 else BF16)
+    check_close("dx", dx, dx_ref, dtype)
+    assert ddA.shape == (N, -(-L // Q), Q) and ddA.dtype == F32
+    check_close("dA", ddA.reshape(N, -1)[:, :L], dA_ref, dtype)
+    C = cs.shape[1]
+    for c in range(1, C):
+        pass
+    ref_prev = torch.stack([y_ref[:, c * Q - 1] if c else torch.zeros(N, T) for c in range(C)], 1)
+    check_close("prev", prev, ref_prev, F32 if dtype == F32 else BF16)
+
+
+def _headed_reference(x, A, dy):
+    b, L, nh, d = x.shape
+    xf, Af = O.to_flat(x.float(), A)
+    dyf, _ = O.to_flat(dy.float(), A)
+    y = O.from_flat(O.ema_loop(xf, Af), b, nh)
+    dx, dA = O.ema_loop_bwd(dyf, xf, Af)
+    return y, O.from_flat(dx, b, nh), dA.reshape(b, nh, L).permute(0, 2, 1)
+
+
+def _autograd_headed(x, A, dy, Q, device):
+    from kernels.ema_kernels.ema_combined_fwd import ema_matmul_scan_combined
+
+    xg = x.to(device).requires_grad_()
+    Ag = A.to(device).requires_grad_()
+    y = ema_matmul_scan_combined(Ag, xg, Q)
+    y.backward(dy.to(device))
+    torch.cuda.synchronize()
+    return y, xg.grad, Ag.grad
+
+
+def test_config1_fp32_forward(device):
+    """BASELINE config 1: b1 nh2 L512 d64 Q128 fp32, input scaled by (1 - alpha), compared
+    with y_t = alpha_t y_{t-1} + (1 - alpha_t) x_t."""
+    from kernels.ema_kernels.ema_combined_fwd import ema_matmul_scan_combined
+
+    announce("config 1")
+    x, A, _ = O.make_inputs(1, 2, 512, 64, seed=11, scale_x=False)
+    xs, _, _ = O.make_inputs(1, 2, 512, 64, seed=11, scale_x=True)
+    alpha = torch.exp(A)
+    z = torch.zeros(1, 2, 64)
+    ref = torch.empty_like(x)
+    for t in range(512):
+        z = alpha[:, t, :, None] * z + (1 - alpha[:, t, :, None]) * x[:, t]
+        ref[:, t] = z
+    y = ema_matmul_scan_combined(A.to(device), xs.to(device), 128)
+    check_close("y", y, ref, F32)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+def test_autograd_headed_small(dtype, device):
+    announce(f"autograd headed b2 L300 nh2 d64 {dtype}")
+    x, A, dy = O.make_inputs(2, 2, 300, 64, seed=5, dtype=dtype)
+    y, dx, dA = _autograd_headed(x, A, dy, 128, device)
+    y_ref, dx_ref, dA_ref = _headed_reference(x, A, dy)
+    assert dA.shape == A.shape and dx.shape == x.shape
+    check_close("y", y, y_ref, dtype)
+    check_close("dx", dx, dx_ref, dtype)
+    check_close("dA", dA, dA_ref, dtype)
+
+
+@pytest.mark.parametrize("Q", [128, 256, 512])
+def test_config3_bf16_fwd_bwd_full_size(Q, device):
+    """BASELINE configs 2 and 3: b16 nh2 d1024 L4096, bf16, chunk size swept, seed fixed per
+    chunk size; forward, dx and dA against the sequential oracle at full size."""
+    announce(f"config 2/3 full size Q{Q}")
+    x, A, dy = O.make_inputs(16, 2, 4096, 1024, seed=1000 + Q, dtype=BF16)
+    y, dx, dA = _autograd_headed(x, A, dy, Q, device)
+    y_ref, dx_ref, dA_ref = _headed_reference(x, A, dy)
+    check_close("y", y, y_ref, BF16)
+    check_close("dx", dx, dx_ref, BF16)
+    check_close("dA", dA, dA_ref, BF16)
+
+
+def test_config4_long_sequence(device):
+    """BASELINE config 4: b4 nh2 d1024 L32768 Q256, bf16, u ~ N(4,1) (long memory)."""
+    announce("config 4 full size")
+    x, A, dy = O.make_inputs(4, 2, 32768, 1024, seed=4, dtype=BF16, u_mean=4.0)
+    y, dx, dA = _autograd_headed(x, A, dy, 256, device)
+    y_ref, dx_ref, dA_ref = _headed_reference(x, A, dy)
+    check_close("y", y, y_ref, BF16)
+    check_close("dx", dx, dx_ref, BF16)
+    check_close("dA", dA, dA_ref, BF16)
+
+
+def test_chunk_size_invariance_and_linearity_full_size(device):
+    """Size-independent properties at the bench shape: the output does not depend on the
+    chunk size, and the scan is linear in x."""
+    from kernels.ema_kernels.ema_combined_fwd import ema_matmul_scan_combined
+
+    announce("invariance / linearity at b16 nh2 d1024 L4096")
+    x, A, _ = O.make_inputs(16, 2, 4096, 1024, seed=21, dtype=F32, with_dy=False)
+    xd, Ad = x.to(device), A.to(device)
+    y128 = ema_matmul_scan_combined(Ad, xd, 128)
+    y512 = ema_matmul_scan_combined(Ad, xd, 512)
+    check_close("Q128 vs Q512", y128, y512, F32)
+    x2 = torch.roll(xd, 1, dims=0)
+    lhs = ema_matmul_scan_combined(Ad, 2.0 * xd - x2, 128)
+    rhs = 2.0 * y128 - ema_matmul_scan_combined(Ad, x2, 128)
+    check_close("linearity", lhs, rhs, F32)
+
+
+def test_zero_log_decay_is_cumsum(device):
+    from kernels.ema_kernels.ema_combined_fwd import ema_matmul_scan_combined
+
+    announce("A == 0")
+    X = torch.randn(2, 500, 64)
+    A = torch.zeros(2, 500)
+    y = ema_matmul_scan_combined(A.to(device), X.to(device), 128)
+    check_close("y", y, torch.cumsum(X, 1), F32)
+
+
+def test_strong_decay_no_nan(device):
+    """Very negative log-decays underflow to 0 instead of producing inf * 0."""
+    from kernels.ema_kernels.ema_combined_fwd import ema_matmul_scan_combined
+
+    announce("A = -60")
+    X = torch.randn(1, 256, 64)
+    A = torch.full((1, 256), -60.0)
+    y = ema_matmul_scan_combined(A.to(device), X.to(device), 128)
+    check_close("y", y, O.ema_loop(X, A), F32)
+
+
+def test_error_behaviour(device):
+    """Same refusals as the reference launchers."""
+    from kernels.ema_kernels.ema_state_pass import _ema_state_passing_fwd
+    from kernels.ema_kernels.ema_state_fwd import _ema_chunk_state_fwd
+    from kernels.ema_kernels_bwd.ema_state_passing_bwd_dstates import _ema_state_passing_bwd
+
+    st = torch.zeros(2, 3, 8, device=device)
+    cl = torch.zeros(2, 3, device=device)
+    with pytest.raises(NotImplementedError):  # kernels/ema_kernels/ema_state_pass.py:129-130
+        _ema_state_passing_fwd(st, cl, initial_states=torch.zeros(2, 8, device=device))
+    with pytest.raises(AssertionError):
+        _ema_state_passing_fwd(st, torch.zeros(2, 4, device=device))
+    with pytest.raises(AssertionError):  # ...state_passing_bwd_dstates.py:120-122
+        _ema_state_passing_bwd(st, cl, st, dfinal_states=torch.zeros(2, 8, device=device))
+    with pytest.raises(AssertionError):  # kernels/ema_kernels/ema_state_fwd.py:135-140
+        _ema_chunk_state_fwd(torch.zeros(2, 24, 8, device=device), torch.zeros(2, 2, 8, device=device))
+    with pytest.raises(AssertionError):  # feature size must allow 16-byte rows
+        _ema_chunk_state_fwd(torch.zeros(2, 16, 6, device=device), torch.zeros(2, 2, 8, device=device))

@@ -1,0 +1,465 @@
+// C ABI of libema_hip.so: argument validation and kernel launches.  Declarations and the
+// reference launcher each entry point replaces are in include/ema_hip.h.
+#include "../../include/ema_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include "ema_device.h"
+#include "ema_gemm_kernels.h"
+#include "ema_stream_kernels.h"
+
+using namespace ema;
+
+namespace {
+
+struct Dims {
+  int64_t batch, nh, L, T, Q, N, C;
+};
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+inline int elem_size(int dtype) { return dtype == EMA_BF16 ? 2 : 4; }
+
+// Shape checks shared by every entry point that sees the sequence axis.
+int check_dims(int64_t batch, int64_t nh, int64_t L, int64_t T, int64_t Q, bool has_T, Dims* d) {
+  if (batch <= 0 || nh <= 0 || L <= 0 || Q <= 0 || (has_T && T <= 0)) return EMA_ERR_SHAPE;
+  if (Q > EMA_MAX_CHUNK) return EMA_ERR_SHAPE;
+  if (batch > (1 << 24) || nh > (1 << 16) || L > (int64_t)1 << 30 || T > (1 << 24))
+    return EMA_ERR_SHAPE;
+  d->batch = batch;
+  d->nh = nh;
+  d->L = L;
+  d->T = T;
+  d->Q = Q;
+  d->N = batch * nh;
+  d->C = (L + Q - 1) / Q;
+  if (d->N * d->C > ((int64_t)1 << 30)) return EMA_ERR_SHAPE;
+  return EMA_OK;
+}
+
+int check_dtype(int dtype) { return (dtype == EMA_F32 || dtype == EMA_BF16) ? EMA_OK : EMA_ERR_DTYPE; }
+
+// A sequence tensor must allow 16-byte loads of every row segment.
+int check_seq(const void* p, int64_t sb, int64_t sl, int64_t sh, int dtype, int64_t T) {
+  if (!p) return EMA_ERR_NULL;
+  const int epl = 16 / elem_size(dtype);
+  if (T % epl || sb % epl || sl % epl || sh % epl) return EMA_ERR_ALIGN;
+  if (reinterpret_cast<uintptr_t>(p) % 16) return EMA_ERR_ALIGN;
+  return EMA_OK;
+}
+
+int check_f32(const void* p) {
+  if (!p) return EMA_ERR_NULL;
+  return reinterpret_cast<uintptr_t>(p) % 16 ? EMA_ERR_ALIGN : EMA_OK;
+}
+
+inline int launched() { return hipGetLastError() == hipSuccess ? EMA_OK : EMA_ERR_LAUNCH; }
+
+#define EMA_TRY(expr)            \
+  do {                           \
+    int _s = (expr);             \
+    if (_s != EMA_OK) return _s; \
+  } while (0)
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+// ---------------------------------------------------------------- launch helpers
+
+int launch_cumsum(const float* A, SeqStrides sa, float* cs, const Dims& d, hipStream_t st) {
+  const int64_t total = d.N * d.C;
+  const unsigned grid = (unsigned)((total + 3) / 4);
+  hipLaunchKernelGGL(cumsum_kernel, dim3(grid), dim3(256), 0, st, A, sa, cs, (int)d.nh, (int)d.L,
+                     (int)d.Q, (int)d.C, total);
+  return launched();
+}
+
+template <int MODE>
+int launch_chunk_reduce(const void* x, SeqStrides sx, int dtype, const float* cs, float* out,
+                        const Dims& d, hipStream_t st) {
+  const int epl = 16 / elem_size(dtype);
+  const int64_t vecs = d.T / epl;
+  int cg_log2 = 0;
+  while ((1 << cg_log2) < vecs && cg_log2 < 6) ++cg_log2;
+  const int cg = 1 << cg_log2;
+  const int ntiles = (int)((vecs + cg - 1) / cg);
+  const int64_t grid = d.N * d.C * ntiles;
+  if (grid > 0x7fffffff) return EMA_ERR_SHAPE;
+  if (dtype == EMA_BF16)
+    hipLaunchKernelGGL((chunk_reduce_kernel<bf16_t, MODE>), dim3((unsigned)grid), dim3(256), 0, st,
+                       (const bf16_t*)x, sx, cs, out, (int)d.nh, (int)d.L, (int)d.T, (int)d.Q,
+                       (int)d.C, cg_log2, ntiles);
+  else
+    hipLaunchKernelGGL((chunk_reduce_kernel<float, MODE>), dim3((unsigned)grid), dim3(256), 0, st,
+                       (const float*)x, sx, cs, out, (int)d.nh, (int)d.L, (int)d.T, (int)d.Q,
+                       (int)d.C, cg_log2, ntiles);
+  return launched();
+}
+
+int launch_state_passing_fwd(const float* states, const float* cs_last, int64_t cl_sn,
+                             int64_t cl_sc, float* prev, float* fin, int64_t N, int64_t C,
+                             int64_t T, hipStream_t st) {
+  const int tiles = (int)((T + 255) / 256);
+  hipLaunchKernelGGL(state_passing_fwd_kernel, dim3((unsigned)(N * tiles)), dim3(256), 0, st,
+                     states, cs_last, cl_sn, cl_sc, prev, fin, (int)C, (int)T, tiles);
+  return launched();
+}
+
+int launch_state_passing_bwd(const float* prev, const float* cs_last, int64_t cl_sn,
+                             int64_t cl_sc, const float* ds, float* g, float* ddA_chunk,
+                             float* part, int64_t N, int64_t C, int64_t T, hipStream_t st) {
+  const int tiles = (int)((T + 255) / 256);
+  const int nw = (int)((T + 63) / 64);
+  hipLaunchKernelGGL(state_passing_bwd_kernel, dim3((unsigned)(N * tiles)), dim3(256), 0, st, prev,
+                     cs_last, cl_sn, cl_sc, ds, g, part, (int)C, (int)T, tiles, nw);
+  EMA_TRY(launched());
+  const int64_t total = N * C;
+  hipLaunchKernelGGL(state_passing_bwd_finish_kernel, dim3((unsigned)((total + 255) / 256)),
+                     dim3(256), 0, st, part, cs_last, cl_sn, cl_sc, ddA_chunk, (int)C, nw, total);
+  return launched();
+}
+
+template <bool REVERSE>
+int launch_chunk_gemm(const void* in, SeqStrides si, int dtype, const float* cs, const float* vec,
+                      void* out, SeqStrides so, const Dims& d, hipStream_t st) {
+  const int MT = (int)((d.Q + kBM - 1) / kBM);
+  const int ntiles = (int)((d.T + kBN - 1) / kBN);
+  const int64_t grid = d.N * d.C * MT * ntiles;
+  if (grid > 0x7fffffff) return EMA_ERR_SHAPE;
+  if (dtype == EMA_BF16)
+    hipLaunchKernelGGL((chunk_gemm_kernel<bf16_t, REVERSE>), dim3((unsigned)grid), dim3(256), 0, st,
+                       (const bf16_t*)in, si, cs, vec, (bf16_t*)out, so, (int)d.nh, (int)d.L,
+                       (int)d.T, (int)d.Q, (int)d.C, MT, ntiles);
+  else
+    hipLaunchKernelGGL((chunk_gemm_kernel<float, REVERSE>), dim3((unsigned)grid), dim3(256), 0, st,
+                       (const float*)in, si, cs, vec, (float*)out, so, (int)d.nh, (int)d.L,
+                       (int)d.T, (int)d.Q, (int)d.C, MT, ntiles);
+  return launched();
+}
+
+template <int MODE>
+int launch_row_dot(const void* x, SeqStrides sx, int dtype, const float* vec, const float* cs,
+                   float* out, int raw, const Dims& d, hipStream_t st) {
+  const unsigned grid = (unsigned)(d.N * d.C);
+  if (dtype == EMA_BF16)
+    hipLaunchKernelGGL((row_dot_kernel<bf16_t, MODE>), dim3(grid), dim3(256), 0, st,
+                       (const bf16_t*)x, sx, vec, cs, out, (int)d.nh, (int)d.L, (int)d.T, (int)d.Q,
+                       (int)d.C, raw);
+  else
+    hipLaunchKernelGGL((row_dot_kernel<float, MODE>), dim3(grid), dim3(256), 0, st, (const float*)x,
+                       sx, vec, cs, out, (int)d.nh, (int)d.L, (int)d.T, (int)d.Q, (int)d.C, raw);
+  return launched();
+}
+
+int launch_da(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, int dtype,
+              const float* cs, float* ddA_intra, float* part, float* rowsum, const Dims& d,
+              hipStream_t st) {
+  const int MT = (int)((d.Q + kBM - 1) / kBM);
+  const int64_t grid = d.N * d.C * MT;
+  if (grid > 0x7fffffff) return EMA_ERR_SHAPE;
+  if (dtype == EMA_BF16)
+    hipLaunchKernelGGL((da_gemm_kernel<bf16_t>), dim3((unsigned)grid), dim3(256), 0, st,
+                       (const bf16_t*)x, sx, (const bf16_t*)dy, sd, cs, part, rowsum, (int)d.nh,
+                       (int)d.L, (int)d.T, (int)d.Q, (int)d.C, MT);
+  else
+    hipLaunchKernelGGL((da_gemm_kernel<float>), dim3((unsigned)grid), dim3(256), 0, st,
+                       (const float*)x, sx, (const float*)dy, sd, cs, part, rowsum, (int)d.nh,
+                       (int)d.L, (int)d.T, (int)d.Q, (int)d.C, MT);
+  EMA_TRY(launched());
+  const int64_t total = d.N * d.C;
+  hipLaunchKernelGGL(da_finish_kernel, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, st, part,
+                     rowsum, ddA_intra, (int)d.Q, MT, total);
+  return launched();
+}
+
+size_t da_part_floats(const Dims& d) {
+  const int64_t MT = (d.Q + kBM - 1) / kBM;
+  return (size_t)(d.N * d.C * MT * d.Q);
+}
+
+// Workspace carving for ema_bwd.
+struct BwdWs {
+  float *cs, *states, *prev, *ds, *g, *sp_part, *ddA_chunk, *da_part, *rowsum, *intra, *next, *sraw;
+  size_t bytes;
+};
+
+BwdWs carve_bwd(void* base, const Dims& d) {
+  BwdWs w;
+  size_t off = 0;
+  char* p = static_cast<char*>(base);
+  auto take = [&](size_t floats) {
+    float* r = reinterpret_cast<float*>(p + off);
+    off += align_up(floats * sizeof(float), 256);
+    return r;
+  };
+  const size_t ncq = (size_t)(d.N * d.C * d.Q), nct = (size_t)(d.N * d.C * d.T);
+  w.cs = take(ncq);
+  w.states = take(nct);
+  w.prev = take(nct);
+  w.ds = take(nct);
+  w.g = take(nct);
+  w.sp_part = take((size_t)(d.N * d.C * ((d.T + 63) / 64)));
+  w.ddA_chunk = take((size_t)(d.N * d.C));
+  w.da_part = take(da_part_floats(d));
+  w.rowsum = take(ncq);
+  w.intra = take(ncq);
+  w.next = take(ncq);
+  w.sraw = take(ncq);
+  w.bytes = off;
+  return w;
+}
+
+}  // namespace
+
+// ====================================================================================
+
+extern "C" {
+
+const char* ema_version(void) { return "ema_hip 0.1 (gfx950)"; }
+
+const char* ema_status_string(int status) {
+  switch (status) {
+    case EMA_OK: return "ok";
+    case EMA_ERR_NULL: return "null pointer";
+    case EMA_ERR_SHAPE: return "bad shape";
+    case EMA_ERR_ALIGN: return "dim, stride or pointer not 16-byte aligned";
+    case EMA_ERR_DTYPE: return "unknown dtype";
+    case EMA_ERR_UNSUPPORTED: return "unsupported";
+    case EMA_ERR_LAUNCH: return "kernel launch failed";
+    default: return "unknown status";
+  }
+}
+
+int ema_chunk_cumsum_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, float* cs,
+                         int64_t batch, int64_t nheads, int64_t seqlen, int64_t chunk,
+                         void* stream) {
+  Dims d;
+  EMA_TRY(check_dims(batch, nheads, seqlen, 1, chunk, false, &d));
+  if (!A || !cs) return EMA_ERR_NULL;
+  return launch_cumsum(A, SeqStrides{a_sb, a_sl, a_sh}, cs, d, as_stream(stream));
+}
+
+int ema_chunk_state_fwd(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype,
+                        const float* cs, float* states, int64_t batch, int64_t nheads,
+                        int64_t seqlen, int64_t dim, int64_t chunk, void* stream) {
+  Dims d;
+  EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
+  EMA_TRY(check_dtype(dtype));
+  EMA_TRY(check_seq(x, x_sb, x_sl, x_sh, dtype, dim));
+  if (!cs || !states) return EMA_ERR_NULL;
+  return launch_chunk_reduce<0>(x, SeqStrides{x_sb, x_sl, x_sh}, dtype, cs, states, d,
+                                as_stream(stream));
+}
+
+int ema_state_passing_fwd(const float* states, const float* cs_last, int64_t cl_sn, int64_t cl_sc,
+                          float* prev, float* final_state, int64_t nseq, int64_t nchunks,
+                          int64_t dim, void* stream) {
+  if (nseq <= 0 || nchunks <= 0 || dim <= 0) return EMA_ERR_SHAPE;
+  if (nseq * ((dim + 255) / 256) > 0x7fffffff) return EMA_ERR_SHAPE;
+  if (!states || !cs_last || !prev || !final_state) return EMA_ERR_NULL;
+  return launch_state_passing_fwd(states, cs_last, cl_sn, cl_sc, prev, final_state, nseq, nchunks,
+                                  dim, as_stream(stream));
+}
+
+int ema_scan_fwd(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype,
+                 const float* cs, const float* prev, void* y, int64_t y_sb, int64_t y_sl,
+                 int64_t y_sh, int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
+                 int64_t chunk, void* stream) {
+  Dims d;
+  EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
+  EMA_TRY(check_dtype(dtype));
+  EMA_TRY(check_seq(x, x_sb, x_sl, x_sh, dtype, dim));
+  EMA_TRY(check_seq(y, y_sb, y_sl, y_sh, dtype, dim));
+  if (!cs || !prev) return EMA_ERR_NULL;
+  return launch_chunk_gemm<false>(x, SeqStrides{x_sb, x_sl, x_sh}, dtype, cs, prev, y,
+                                  SeqStrides{y_sb, y_sl, y_sh}, d, as_stream(stream));
+}
+
+size_t ema_fwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
+                               int64_t chunk) {
+  Dims d;
+  if (check_dims(batch, nheads, seqlen, dim, chunk, true, &d) != EMA_OK) return 0;
+  return align_up((size_t)(d.N * d.C * d.T) * sizeof(float), 256);
+}
+
+int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void* x, int64_t x_sb,
+            int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb, int64_t y_sl,
+            int64_t y_sh, float* cs, float* prev, float* final_state, void* workspace,
+            size_t workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
+            int64_t chunk, void* stream) {
+  Dims d;
+  EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
+  EMA_TRY(check_dtype(dtype));
+  EMA_TRY(check_seq(x, x_sb, x_sl, x_sh, dtype, dim));
+  EMA_TRY(check_seq(y, y_sb, y_sl, y_sh, dtype, dim));
+  if (!A || !cs || !prev || !final_state) return EMA_ERR_NULL;
+  EMA_TRY(check_f32(workspace));
+  if (workspace_bytes < ema_fwd_workspace_bytes(batch, nheads, seqlen, dim, chunk))
+    return EMA_ERR_SHAPE;
+  hipStream_t st = as_stream(stream);
+  float* states = static_cast<float*>(workspace);
+  const SeqStrides sx{x_sb, x_sl, x_sh}, sy{y_sb, y_sl, y_sh};
+  EMA_TRY(launch_cumsum(A, SeqStrides{a_sb, a_sl, a_sh}, cs, d, st));
+  EMA_TRY(launch_chunk_reduce<0>(x, sx, dtype, cs, states, d, st));
+  EMA_TRY(launch_state_passing_fwd(states, cs + (d.Q - 1), d.C * d.Q, d.Q, prev, final_state, d.N,
+                                   d.C, d.T, st));
+  return launch_chunk_gemm<false>(x, sx, dtype, cs, prev, y, sy, d, st);
+}
+
+int ema_chunk_scan_bwd_dstates(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh,
+                               int dtype, const float* cs, float* ds, int64_t batch, int64_t nheads,
+                               int64_t seqlen, int64_t dim, int64_t chunk, void* stream) {
+  Dims d;
+  EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
+  EMA_TRY(check_dtype(dtype));
+  EMA_TRY(check_seq(dy, dy_sb, dy_sl, dy_sh, dtype, dim));
+  if (!cs || !ds) return EMA_ERR_NULL;
+  return launch_chunk_reduce<1>(dy, SeqStrides{dy_sb, dy_sl, dy_sh}, dtype, cs, ds, d,
+                                as_stream(stream));
+}
+
+size_t ema_state_passing_bwd_workspace_bytes(int64_t nseq, int64_t nchunks, int64_t dim) {
+  if (nseq <= 0 || nchunks <= 0 || dim <= 0) return 0;
+  return align_up((size_t)(nseq * nchunks * ((dim + 63) / 64)) * sizeof(float), 256);
+}
+
+int ema_state_passing_bwd(const float* prev, const float* cs_last, int64_t cl_sn, int64_t cl_sc,
+                          const float* ds, float* g, float* ddA_chunk, void* workspace,
+                          size_t workspace_bytes, int64_t nseq, int64_t nchunks, int64_t dim,
+                          void* stream) {
+  if (nseq <= 0 || nchunks <= 0 || dim <= 0) return EMA_ERR_SHAPE;
+  if (nseq * ((dim + 255) / 256) > 0x7fffffff) return EMA_ERR_SHAPE;
+  if (!prev || !cs_last || !ds || !g || !ddA_chunk || !workspace) return EMA_ERR_NULL;
+  if (workspace_bytes < ema_state_passing_bwd_workspace_bytes(nseq, nchunks, dim))
+    return EMA_ERR_SHAPE;
+  return launch_state_passing_bwd(prev, cs_last, cl_sn, cl_sc, ds, g, ddA_chunk,
+                                  static_cast<float*>(workspace), nseq, nchunks, dim,
+                                  as_stream(stream));
+}
+
+int ema_chunk_scan_chunk_state_bwd_dx(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh,
+                                      int dtype, const float* cs, const float* g, void* dx,
+                                      int64_t dx_sb, int64_t dx_sl, int64_t dx_sh, int64_t batch,
+                                      int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk,
+                                      void* stream) {
+  Dims d;
+  EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
+  EMA_TRY(check_dtype(dtype));
+  EMA_TRY(check_seq(dy, dy_sb, dy_sl, dy_sh, dtype, dim));
+  EMA_TRY(check_seq(dx, dx_sb, dx_sl, dx_sh, dtype, dim));
+  if (!cs || !g) return EMA_ERR_NULL;
+  return launch_chunk_gemm<true>(dy, SeqStrides{dy_sb, dy_sl, dy_sh}, dtype, cs, g, dx,
+                                 SeqStrides{dx_sb, dx_sl, dx_sh}, d, as_stream(stream));
+}
+
+int ema_chunk_state_bwd_db(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype,
+                           const float* cs, const float* g, float* ddA_next, int raw, int64_t batch,
+                           int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk,
+                           void* stream) {
+  Dims d;
+  EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
+  EMA_TRY(check_dtype(dtype));
+  EMA_TRY(check_seq(x, x_sb, x_sl, x_sh, dtype, dim));
+  if (!cs || !ddA_next) return EMA_ERR_NULL;
+  EMA_TRY(check_f32(g));
+  if (dim % 4) return EMA_ERR_ALIGN;
+  return launch_row_dot<0>(x, SeqStrides{x_sb, x_sl, x_sh}, dtype, g, cs, ddA_next, raw, d,
+                           as_stream(stream));
+}
+
+int ema_chunk_scan_bwd_dc(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, int dtype,
+                          const float* prev, const float* cs, float* ddA_prev, int64_t batch,
+                          int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk,
+                          void* stream) {
+  Dims d;
+  EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
+  EMA_TRY(check_dtype(dtype));
+  EMA_TRY(check_seq(dy, dy_sb, dy_sl, dy_sh, dtype, dim));
+  if (!cs || !ddA_prev) return EMA_ERR_NULL;
+  EMA_TRY(check_f32(prev));
+  return launch_row_dot<1>(dy, SeqStrides{dy_sb, dy_sl, dy_sh}, dtype, prev, cs, ddA_prev, 0, d,
+                           as_stream(stream));
+}
+
+size_t ema_chunk_scan_bwd_ddAcs_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen,
+                                                int64_t chunk) {
+  Dims d;
+  if (check_dims(batch, nheads, seqlen, 1, chunk, false, &d) != EMA_OK) return 0;
+  return align_up(da_part_floats(d) * sizeof(float), 256) +
+         align_up((size_t)(d.N * d.C * d.Q) * sizeof(float), 256);
+}
+
+int ema_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
+                             const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, int dtype,
+                             const float* cs, float* ddA_intra, void* workspace,
+                             size_t workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen,
+                             int64_t dim, int64_t chunk, void* stream) {
+  Dims d;
+  EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
+  EMA_TRY(check_dtype(dtype));
+  EMA_TRY(check_seq(x, x_sb, x_sl, x_sh, dtype, dim));
+  EMA_TRY(check_seq(dy, dy_sb, dy_sl, dy_sh, dtype, dim));
+  if (!cs || !ddA_intra) return EMA_ERR_NULL;
+  EMA_TRY(check_f32(workspace));
+  if (workspace_bytes < ema_chunk_scan_bwd_ddAcs_workspace_bytes(batch, nheads, seqlen, chunk))
+    return EMA_ERR_SHAPE;
+  float* part = static_cast<float*>(workspace);
+  float* rowsum = reinterpret_cast<float*>(static_cast<char*>(workspace) +
+                                           align_up(da_part_floats(d) * sizeof(float), 256));
+  return launch_da(x, SeqStrides{x_sb, x_sl, x_sh}, dy, SeqStrides{dy_sb, dy_sl, dy_sh}, dtype, cs,
+                   ddA_intra, part, rowsum, d, as_stream(stream));
+}
+
+size_t ema_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
+                               int64_t chunk) {
+  Dims d;
+  if (check_dims(batch, nheads, seqlen, dim, chunk, true, &d) != EMA_OK) return 0;
+  return carve_bwd(nullptr, d).bytes;
+}
+
+int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const void* x,
+            int64_t x_sb, int64_t x_sl, int64_t x_sh, const float* A, int64_t a_sb, int64_t a_sl,
+            int64_t a_sh, int dtype, void* dx, int64_t dx_sb, int64_t dx_sl, int64_t dx_sh,
+            float* ddA, void* y, int64_t y_sb, int64_t y_sl, int64_t y_sh, void* workspace,
+            size_t workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
+            int64_t chunk, void* stream) {
+  Dims d;
+  EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
+  EMA_TRY(check_dtype(dtype));
+  EMA_TRY(check_seq(dy, dy_sb, dy_sl, dy_sh, dtype, dim));
+  EMA_TRY(check_seq(x, x_sb, x_sl, x_sh, dtype, dim));
+  EMA_TRY(check_seq(dx, dx_sb, dx_sl, dx_sh, dtype, dim));
+  if (y) EMA_TRY(check_seq(y, y_sb, y_sl, y_sh, dtype, dim));
+  if (!A || !ddA) return EMA_ERR_NULL;
+  EMA_TRY(check_f32(workspace));
+  if (workspace_bytes < ema_bwd_workspace_bytes(batch, nheads, seqlen, dim, chunk))
+    return EMA_ERR_SHAPE;
+  hipStream_t st = as_stream(stream);
+  const BwdWs w = carve_bwd(workspace, d);
+  const SeqStrides sx{x_sb, x_sl, x_sh}, sd{dy_sb, dy_sl, dy_sh}, sdx{dx_sb, dx_sl, dx_sh};
+  const float* cs_last = w.cs + (d.Q - 1);
+  const int64_t cl_sn = d.C * d.Q, cl_sc = d.Q;
+
+  // recompute the forward intermediates
+  EMA_TRY(launch_cumsum(A, SeqStrides{a_sb, a_sl, a_sh}, w.cs, d, st));
+  EMA_TRY(launch_chunk_reduce<0>(x, sx, dtype, w.cs, w.states, d, st));
+  // final state is not needed; ds is free until B1 runs, use its first N*T floats
+  EMA_TRY(launch_state_passing_fwd(w.states, cs_last, cl_sn, cl_sc, w.prev, w.ds, d.N, d.C, d.T,
+                                   st));
+  if (y)
+    EMA_TRY(launch_chunk_gemm<false>(x, sx, dtype, w.cs, w.prev, y, SeqStrides{y_sb, y_sl, y_sh}, d,
+                                     st));
+  // backward proper
+  EMA_TRY(launch_chunk_reduce<1>(dy, sd, dtype, w.cs, w.ds, d, st));
+  EMA_TRY(launch_state_passing_bwd(w.prev, cs_last, cl_sn, cl_sc, w.ds, w.g, w.ddA_chunk,
+                                   w.sp_part, d.N, d.C, d.T, st));
+  EMA_TRY(launch_chunk_gemm<true>(dy, sd, dtype, w.cs, w.g, dx, sdx, d, st));
+  EMA_TRY(launch_row_dot<0>(x, sx, dtype, w.g, w.cs, w.next, 0, d, st));
+  EMA_TRY(launch_row_dot<1>(dy, sd, dtype, w.prev, w.cs, w.sraw, 0, d, st));
+  EMA_TRY(launch_da(x, sx, dy, sd, dtype, w.cs, w.intra, w.da_part, w.rowsum, d, st));
+  const int64_t total = d.N * d.C;
+  hipLaunchKernelGGL(combine_dA_kernel, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, st, w.intra,
+                     w.next, w.sraw, w.ddA_chunk, ddA, (int)d.Q, total);
+  return launched();
+}
+
+}  // extern "C"

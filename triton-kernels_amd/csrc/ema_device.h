@@ -1,0 +1,115 @@
+// Device-side helpers shared by the EMA kernels (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ema {
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+#define EMA_MAX_CHUNK_DEV 1024
+
+// One descriptor per sequence tensor: element strides of (batch, position, head); the
+// feature axis has unit stride.
+struct SeqStrides {
+  int64_t sb, sl, sh;
+};
+
+// ------------------------------------------------------------------ wave primitives
+
+// v of the lane selected by a DPP control, or 0 where the control has no source lane or
+// the row is masked out.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_or_zero(float v) {
+  return __int_as_float(
+      __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+
+// Inclusive prefix sum over the 64 lanes of a wave with DPP row shifts and row broadcasts
+// (no LDS traffic).
+__device__ __forceinline__ float wave_inclusive_scan(float v) {
+  v += dpp_or_zero<0x111, 0xf>(v);  // row_shr:1
+  v += dpp_or_zero<0x112, 0xf>(v);  // row_shr:2
+  v += dpp_or_zero<0x114, 0xf>(v);  // row_shr:4
+  v += dpp_or_zero<0x118, 0xf>(v);  // row_shr:8
+  v += dpp_or_zero<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+  v += dpp_or_zero<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
+// Sum over the 64 lanes, returned in every lane.
+__device__ __forceinline__ float wave_sum(float v) {
+  v = wave_inclusive_scan(v);
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
+// ------------------------------------------------------------------ 16-byte vectors
+
+template <typename T>
+struct Vec16;  // 16 bytes of T
+template <>
+struct Vec16<float> {
+  static constexpr int N = 4;
+  float4 raw;
+  __device__ __forceinline__ float get(int i) const {
+    return i == 0 ? raw.x : i == 1 ? raw.y : i == 2 ? raw.z : raw.w;
+  }
+  __device__ __forceinline__ void set(int i, float f) {
+    if (i == 0) raw.x = f;
+    else if (i == 1) raw.y = f;
+    else if (i == 2) raw.z = f;
+    else raw.w = f;
+  }
+  __device__ __forceinline__ void put(int i, float f) { set(i, f); }
+  __device__ __forceinline__ void zero() { raw = make_float4(0.f, 0.f, 0.f, 0.f); }
+};
+template <>
+struct Vec16<bf16_t> {
+  static constexpr int N = 8;
+  bf16x8 raw;
+  __device__ __forceinline__ float get(int i) const { return (float)raw[i]; }
+  __device__ __forceinline__ void set(int i, float f) { raw[i] = (bf16_t)f; }
+  __device__ __forceinline__ void put(int i, bf16_t f) { raw[i] = f; }
+  __device__ __forceinline__ void zero() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) raw[i] = (bf16_t)0.0f;
+  }
+};
+
+template <typename T>
+__device__ __forceinline__ Vec16<T> load16(const T* p) {
+  Vec16<T> v;
+  v.raw = *reinterpret_cast<const decltype(v.raw)*>(p);
+  return v;
+}
+template <typename T>
+__device__ __forceinline__ void store16(T* p, const Vec16<T>& v) {
+  *reinterpret_cast<decltype(v.raw)*>(p) = v.raw;
+}
+
+// ------------------------------------------------------------------ MFMA groups
+// One "group" multiplies a 32 x KG tile by a KG x 32 tile, KG = 2 * Vec16<T>::N.  A lane
+// holds Vec16<T>::N consecutive k of row (lane % 32), starting at k = N * (lane / 32),
+// for both operands; the accumulator of lane l, register v, is element
+// (8 * (v / 4) + 4 * (l / 32) + v % 4,  l % 32) of the 32 x 32 result.
+__device__ __forceinline__ void mma_group(const Vec16<bf16_t>& a, const Vec16<bf16_t>& b,
+                                          floatx16& acc) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.raw, b.raw, acc, 0, 0, 0);
+}
+__device__ __forceinline__ void mma_group(const Vec16<float>& a, const Vec16<float>& b,
+                                          floatx16& acc) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.raw.x, b.raw.x, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.raw.y, b.raw.y, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.raw.z, b.raw.z, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.raw.w, b.raw.w, acc, 0, 0, 0);
+}
+
+__device__ __forceinline__ int acc_row(int v, int lane) {
+  return 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+}
+
+}  // namespace ema

@@ -1,0 +1,299 @@
+// MFMA kernels of the EMA chunked scan: the intra-chunk contraction with the segsum-decay
+// matrix (forward y, backward dx) and the dy . x^T contraction over the feature axis for
+// the intra-chunk log-decay gradient.  bf16 operands use v_mfma_f32_32x32x16_bf16, f32
+// operands v_mfma_f32_32x32x2_f32; accumulation is f32 in both.
+#pragma once
+#include "ema_device.h"
+
+namespace ema {
+
+constexpr int kBM = 128;  // rows of a chunk handled by one workgroup (4 waves x 32)
+constexpr int kBN = 64;   // feature columns handled by one workgroup of chunk_gemm_kernel
+
+// ------------------------------------------------------------------------------------
+// F4 (REVERSE = false):
+//   out[m,t] = exp(min(cs[m],0)) * vec[t] + sum_{k<=m} exp(min(cs[m]-cs[k],0)) * in[k,t]
+// B3 (REVERSE = true):
+//   out[m,t] = exp(min(cs[Q-1]-cs[m],0)) * vec[t] + sum_{k>=m} exp(min(cs[k]-cs[m],0)) * in[k,t]
+// per chunk.  One workgroup per (n, c, 128-row tile, 64-column tile).  The input rows are
+// staged through LDS in tiles of 128 rows; wave w owns rows 32w..32w+31 of the row tile,
+// builds its slice of the decay matrix in registers (one exp per element, in the operand
+// layout of the MFMA) and reuses it for both 32-column blocks.
+// ------------------------------------------------------------------------------------
+template <typename T, bool REVERSE>
+__global__ __launch_bounds__(256) void chunk_gemm_kernel(
+    const T* __restrict__ in, SeqStrides si, const float* __restrict__ cs,
+    const float* __restrict__ vec, T* __restrict__ out, SeqStrides so, int nh, int L,
+    int Tdim, int Q, int C, int MT, int ntiles) {
+  constexpr int EPL = Vec16<T>::N;  // operand elements per lane and MFMA group
+  constexpr int KG = 2 * EPL;       // k extent of one MFMA group
+  constexpr int ROW = kBN + EPL;    // LDS row pitch in elements (16 bytes of padding)
+  __shared__ __attribute__((aligned(16))) T xs[kBM * ROW];
+  __shared__ float cs_s[EMA_MAX_CHUNK_DEV];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+
+  int64_t blk = blockIdx.x;
+  const int tile = (int)(blk % ntiles);
+  blk /= ntiles;
+  const int mt = (int)(blk % MT);
+  const int64_t chunk_id = blk / MT;
+  const int64_t n = chunk_id / C;
+  const int c = (int)(chunk_id - n * C);
+  const int64_t b = n / nh;
+  const int h = (int)(n - b * nh);
+  const int limit = min(Q, L - c * Q);
+  const int mt_base = mt * kBM;
+  const int col0 = tile * kBN;
+
+  const float* csp = cs + chunk_id * Q;
+  const int q_pad = (Q + kBM - 1) / kBM * kBM;
+  for (int i = tid; i < q_pad; i += 256) cs_s[i] = i < Q ? csp[i] : 0.f;
+  __syncthreads();
+  const float cs_last = cs_s[Q - 1];
+
+  const int m_lane = mt_base + wave * 32 + l32;  // row of this lane's decay-matrix slice
+  const float cs_m = cs_s[min(m_lane, q_pad - 1)];
+
+  // accumulators start from the carried-state term
+  floatx16 acc[kBN / 32];
+  const float* vp = vec + chunk_id * Tdim;
+#pragma unroll
+  for (int db = 0; db < kBN / 32; ++db) {
+    const int col = col0 + db * 32 + l32;
+    const float pv = col < Tdim ? vp[col] : 0.f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = mt_base + wave * 32 + acc_row(v, lane);
+      const float a = cs_s[min(row, q_pad - 1)];
+      const float sc = REVERSE ? __expf(fminf(cs_last - a, 0.f)) : __expf(fminf(a, 0.f));
+      acc[db][v] = sc * pv;
+    }
+  }
+
+  const int k_lo = REVERSE ? mt_base : 0;
+  const int k_hi = REVERSE ? limit : min(mt_base + kBM, limit);
+  const int wave_lo = mt_base + wave * 32;       // lowest row of this wave
+  const int wave_hi = wave_lo + 32;              // one past its highest row
+  const T* ip = in + b * si.sb + h * si.sh + (int64_t)c * Q * si.sl;
+
+  constexpr int VPR = kBN / EPL;        // 16-byte vectors per LDS row
+  constexpr int RPP = 256 / VPR;        // rows filled per pass
+  for (int kt0 = k_lo; kt0 < k_hi; kt0 += kBM) {
+    __syncthreads();
+    {
+      const int vcol = (tid % VPR) * EPL;
+      for (int r = tid / VPR; r < kBM; r += RPP) {
+        const int k = kt0 + r;
+        Vec16<T> v;
+        if (k < limit && col0 + vcol < Tdim) v = load16(ip + (int64_t)k * si.sl + col0 + vcol);
+        else v.zero();
+        store16(&xs[r * ROW + vcol], v);
+      }
+    }
+    __syncthreads();
+    const int kg_lo = REVERSE ? max(0, (wave_lo - kt0) / KG * KG) : 0;
+    const int kg_hi = REVERSE ? min(kBM, k_hi - kt0) : min(kBM, min(wave_hi, k_hi) - kt0);
+    for (int kg = kg_lo; kg < kg_hi; kg += KG) {
+      Vec16<T> a;
+      const int kl = kg + EPL * half;  // first k of this lane inside the tile
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) {
+        const int k = kt0 + kl + e;
+        const float d = REVERSE ? cs_s[k] - cs_m : cs_m - cs_s[k];
+        const bool keep = REVERSE ? (k >= m_lane) : (k <= m_lane);
+        a.set(e, keep ? __expf(fminf(d, 0.f)) : 0.f);
+      }
+#pragma unroll
+      for (int db = 0; db < kBN / 32; ++db) {
+        Vec16<T> bfrag;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) bfrag.put(e, xs[(kl + e) * ROW + db * 32 + l32]);
+        mma_group(a, bfrag, acc[db]);
+      }
+    }
+  }
+
+  T* op = out + b * so.sb + h * so.sh + (int64_t)c * Q * so.sl;
+#pragma unroll
+  for (int db = 0; db < kBN / 32; ++db) {
+    const int col = col0 + db * 32 + l32;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = mt_base + wave * 32 + acc_row(v, lane);
+      if (row < limit && col < Tdim) op[(int64_t)row * so.sl + col] = (T)acc[db][v];
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// B6, first part.  For the chunk (n, c) and the row tile mt (rows m of dy), for every
+// column tile kt <= mt (rows k of x):
+//   G[m,k] = <dy[m,:], x[k,:]>  (MFMA over the feature axis, operands read row-major)
+//   W[m,k] = G[m,k] * exp(min(cs[m]-cs[k],0)) for k < m, else 0
+//   part[(chunk*MT + mt)*Q + k] = sum_m W[m,k]      (column sums of this row tile)
+//   rowsum[chunk*Q + m]         = sum_k W[m,k]      (complete: all k < m are visited)
+// da_finish_kernel turns these into ddA_intra.
+// ------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void da_gemm_kernel(const T* __restrict__ x, SeqStrides sx,
+                                                      const T* __restrict__ dy, SeqStrides sd,
+                                                      const float* __restrict__ cs,
+                                                      float* __restrict__ part,
+                                                      float* __restrict__ rowsum, int nh, int L,
+                                                      int Tdim, int Q, int C, int MT) {
+  constexpr int EPL = Vec16<T>::N;
+  constexpr int KG = 2 * EPL;
+  constexpr int DK = 4 * KG;        // feature columns per LDS stage (128 bytes per row)
+  constexpr int ROW = DK + EPL;     // row pitch in elements (16 bytes of padding)
+  constexpr int TILE = kBM * ROW;   // elements per staged tile
+  // staging tiles, later reused for the row-sum exchange (256 x 17 floats = 17408 bytes)
+  __shared__ __attribute__((aligned(16))) T stage[2 * TILE];
+  __shared__ float cs_s[EMA_MAX_CHUNK_DEV];
+  __shared__ float colpart[4 * 2 * kBM];
+  static_assert(2 * TILE * sizeof(T) >= 256 * 17 * sizeof(float), "row exchange must fit");
+  T* dys = stage;
+  T* xs = stage + TILE;
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int mt = (int)(blockIdx.x % MT);
+  const int64_t chunk_id = blockIdx.x / MT;
+  const int64_t n = chunk_id / C;
+  const int c = (int)(chunk_id - n * C);
+  const int64_t b = n / nh;
+  const int h = (int)(n - b * nh);
+  const int limit = min(Q, L - c * Q);
+  const int mt_base = mt * kBM;
+
+  const float* csp = cs + chunk_id * Q;
+  const int q_pad = (Q + kBM - 1) / kBM * kBM;
+  for (int i = tid; i < q_pad; i += 256) cs_s[i] = i < Q ? csp[i] : 0.f;
+
+  const T* xp = x + b * sx.sb + h * sx.sh + (int64_t)c * Q * sx.sl;
+  const T* dp = dy + b * sd.sb + h * sd.sh + (int64_t)c * Q * sd.sl;
+
+  float rowacc[16];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) rowacc[v] = 0.f;
+
+  constexpr int VPR = DK / EPL;   // 8 vectors per row
+  constexpr int RPP = 256 / VPR;  // 32 rows per pass
+  for (int kt = 0; kt <= mt; ++kt) {
+    const int kt_base = kt * kBM;
+    const int ncb = kt == mt ? wave + 1 : 4;  // column blocks at or below the diagonal
+    floatx16 acc[4];
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[cb][v] = 0.f;
+
+    for (int d0 = 0; d0 < Tdim; d0 += DK) {
+      __syncthreads();
+      {
+        const int vcol = (tid % VPR) * EPL;
+        const bool cok = d0 + vcol < Tdim;
+        for (int r = tid / VPR; r < kBM; r += RPP) {
+          Vec16<T> v;
+          const int m = mt_base + r;
+          if (m < limit && cok) v = load16(dp + (int64_t)m * sd.sl + d0 + vcol);
+          else v.zero();
+          store16(&dys[r * ROW + vcol], v);
+          const int k = kt_base + r;
+          if (k < limit && cok) v = load16(xp + (int64_t)k * sx.sl + d0 + vcol);
+          else v.zero();
+          store16(&xs[r * ROW + vcol], v);
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int doff = g * KG + EPL * half;
+        const Vec16<T> a = load16(&dys[(wave * 32 + l32) * ROW + doff]);
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb) {
+          if (cb < ncb) {
+            const Vec16<T> bf = load16(&xs[(cb * 32 + l32) * ROW + doff]);
+            mma_group(a, bf, acc[cb]);
+          }
+        }
+      }
+    }
+
+    // scale, mask, and reduce this (mt, kt) tile
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) {
+      float colacc = 0.f;
+      if (cb < ncb) {
+        const int k = kt_base + cb * 32 + l32;
+        const float cs_k = cs_s[k];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int m = mt_base + wave * 32 + acc_row(v, lane);
+          float w = 0.f;
+          if (k < m && m < limit) w = acc[cb][v] * __expf(fminf(cs_s[m] - cs_k, 0.f));
+          rowacc[v] += w;
+          colacc += w;
+        }
+      }
+      colpart[(wave * 2 + half) * kBM + cb * 32 + l32] = colacc;
+    }
+    __syncthreads();
+    if (tid < kBM) {
+      float s = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s += colpart[i * kBM + tid];
+      const int k = kt_base + tid;
+      if (k < Q) part[(chunk_id * MT + mt) * (int64_t)Q + k] = s;
+    }
+  }
+
+  __syncthreads();
+  float* rowbuf = reinterpret_cast<float*>(stage);
+#pragma unroll
+  for (int v = 0; v < 16; ++v) rowbuf[tid * 17 + v] = rowacc[v];
+  __syncthreads();
+  if (tid < kBM) {
+    const int w = tid >> 5, rr = tid & 31;
+    const int v = 4 * (rr >> 3) + (rr & 3);
+    const int hf = (rr >> 2) & 1;
+    float s = 0.f;
+    for (int l = 0; l < 32; ++l) s += rowbuf[(w * 64 + hf * 32 + l) * 17 + v];
+    const int m = mt_base + tid;
+    if (m < Q) rowsum[chunk_id * Q + m] = s;
+  }
+}
+
+// B6, second part: ddA_intra[j] = sum_{i<j} (colsum[i] - rowsum[i]) with
+// colsum[i] = sum over the row tiles mt >= i / 128 of part[mt][i].  One wave per (n, c).
+__global__ __launch_bounds__(256) void da_finish_kernel(const float* __restrict__ part,
+                                                        const float* __restrict__ rowsum,
+                                                        float* __restrict__ ddA_intra, int Q,
+                                                        int MT, int64_t total_chunks) {
+  const int lane = threadIdx.x & 63;
+  const int64_t chunk_id = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (chunk_id >= total_chunks) return;
+  const int per = (Q + 63) >> 6;
+  const int q0 = lane * per;
+  auto val = [&](int q) {
+    float s = -rowsum[chunk_id * Q + q];
+    for (int mt = q / kBM; mt < MT; ++mt) s += part[(chunk_id * MT + mt) * (int64_t)Q + q];
+    return s;
+  };
+  float local = 0.f;
+  for (int i = 0; i < per; ++i)
+    if (q0 + i < Q) local += val(q0 + i);
+  float run = wave_inclusive_scan(local) - local;
+  for (int i = 0; i < per; ++i) {
+    const int q = q0 + i;
+    if (q < Q) {
+      ddA_intra[chunk_id * Q + q] = run;
+      run += val(q);
+    }
+  }
+}
+
+}  // namespace ema

@@ -1,0 +1,334 @@
+// HBM-bound kernels of the EMA chunked scan: cumsum, decay-weighted chunk reductions,
+// inter-chunk recurrences (forward and reverse), row dots for the log-decay gradient and
+// the final combination.  Device code only; launched from ema_abi.hip.
+#pragma once
+#include "ema_device.h"
+
+namespace ema {
+
+// ------------------------------------------------------------------------------------
+// F1: per-chunk inclusive cumsum of the log-decay.  One wave per (n, c); lane l owns the
+// `per` consecutive positions starting at l * per, sums them serially, and the lane totals
+// are scanned across the wave with DPP.
+// ------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void cumsum_kernel(const float* __restrict__ A,
+                                                     SeqStrides sa, float* __restrict__ cs,
+                                                     int nh, int L, int Q, int C,
+                                                     int64_t total_chunks) {
+  const int lane = threadIdx.x & 63;
+  const int64_t chunk_id = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (chunk_id >= total_chunks) return;
+  const int64_t n = chunk_id / C;
+  const int c = (int)(chunk_id - n * C);
+  const int64_t b = n / nh;
+  const int h = (int)(n - b * nh);
+  const int per = (Q + 63) >> 6;
+  const int q0 = lane * per;
+  const int limit = min(Q, L - c * Q);
+  const float* a = A + b * sa.sb + h * sa.sh + (int64_t)c * Q * sa.sl;
+
+  float local = 0.f;
+  for (int i = 0; i < per; ++i) {
+    const int q = q0 + i;
+    if (q < limit) local += a[(int64_t)q * sa.sl];
+  }
+  float run = wave_inclusive_scan(local) - local;  // exclusive prefix of the lane totals
+  float* out = cs + chunk_id * Q;
+  for (int i = 0; i < per; ++i) {
+    const int q = q0 + i;
+    if (q < limit) run += a[(int64_t)q * sa.sl];
+    if (q < Q) out[q] = run;
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// F2 / B1: out[n,c,t] = sum_q w[q] * x[n, cQ+q, t] with
+//   MODE 0 (chunk state):  w[q] = exp(min(cs[Q-1] - cs[q], 0))
+//   MODE 1 (dstates):      w[q] = exp(cs[q])
+// One workgroup per (n, c, column tile).  Threads are laid out as cg column groups (one
+// 16-byte vector each) by 256/cg row lanes; every row lane strides over the chunk's rows
+// with 16-byte coalesced loads, and the row lanes are then summed through LDS.
+// ------------------------------------------------------------------------------------
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void chunk_reduce_kernel(
+    const T* __restrict__ x, SeqStrides sx, const float* __restrict__ cs,
+    float* __restrict__ out, int nh, int L, int Tdim, int Q, int C, int cg_log2, int ntiles) {
+  constexpr int VEC = Vec16<T>::N;
+  __shared__ float red[256 * VEC];
+  const int tid = threadIdx.x;
+  const int cg = 1 << cg_log2;
+  const int col_group = tid & (cg - 1);
+  const int row_lane = tid >> cg_log2;
+  const int rows_par = 256 >> cg_log2;
+
+  const int64_t blk = blockIdx.x;
+  const int tile = (int)(blk % ntiles);
+  const int64_t chunk_id = blk / ntiles;
+  const int64_t n = chunk_id / C;
+  const int c = (int)(chunk_id - n * C);
+  const int64_t b = n / nh;
+  const int h = (int)(n - b * nh);
+  const int limit = min(Q, L - c * Q);
+  const int col = (tile * cg + col_group) * VEC;
+  const bool col_ok = col < Tdim;
+
+  const float* csp = cs + chunk_id * Q;
+  const float cs_last = csp[Q - 1];
+  const T* xp = x + b * sx.sb + h * sx.sh + (int64_t)c * Q * sx.sl + col;
+
+  float acc[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+
+  constexpr int U = 4;
+  for (int q0 = row_lane; q0 < limit; q0 += rows_par * U) {
+    Vec16<T> v[U];
+    float w[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int q = q0 + u * rows_par;
+      if (q < limit && col_ok) {
+        v[u] = load16(xp + (int64_t)q * sx.sl);
+        const float a = csp[q];
+        w[u] = MODE == 0 ? __expf(fminf(cs_last - a, 0.f)) : __expf(a);
+      } else {
+        v[u].zero();
+        w[u] = 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) acc[i] = fmaf(w[u], v[u].get(i), acc[i]);
+  }
+
+  // red[row_lane][col_group][i]
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) red[(row_lane * cg + col_group) * VEC + i] = acc[i];
+  __syncthreads();
+  // thread tid sums column (tid) of the tile over the row lanes, then a second pass for
+  // the remaining columns (cg * VEC may exceed 256).
+  for (int j = tid; j < cg * VEC; j += 256) {
+    float s = 0.f;
+    for (int r = 0; r < rows_par; ++r) s += red[r * cg * VEC + j];
+    const int ocol = tile * cg * VEC + j;
+    if (ocol < Tdim) out[chunk_id * Tdim + ocol] = s;
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// F3: forward inter-chunk recurrence.  One thread per (n, t); the running state stays in
+// a register, chunk-local states are fetched U chunks ahead of the dependent FMAs.
+// ------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void state_passing_fwd_kernel(
+    const float* __restrict__ states, const float* __restrict__ cs_last, int64_t cl_sn,
+    int64_t cl_sc, float* __restrict__ prev, float* __restrict__ final_state, int C,
+    int Tdim, int tiles_per_seq) {
+  const int64_t n = blockIdx.x / tiles_per_seq;
+  const int t = (int)(blockIdx.x % tiles_per_seq) * 256 + threadIdx.x;
+  if (t >= Tdim) return;
+  const float* st = states + n * (int64_t)C * Tdim + t;
+  float* pv = prev + n * (int64_t)C * Tdim + t;
+  const float* cl = cs_last + n * cl_sn;
+  float S = 0.f;
+  constexpr int U = 8;
+  for (int c0 = 0; c0 < C; c0 += U) {
+    float s[U], a[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = c0 + u;
+      s[u] = c < C ? st[(int64_t)c * Tdim] : 0.f;
+      a[u] = c < C ? cl[(int64_t)c * cl_sc] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = c0 + u;
+      if (c < C) {
+        pv[(int64_t)c * Tdim] = S;
+        S = fmaf(__expf(a[u]), S, s[u]);
+      }
+    }
+  }
+  final_state[n * Tdim + t] = S;
+}
+
+// ------------------------------------------------------------------------------------
+// B2: reverse inter-chunk recurrence.  One thread per (n, t).  Besides g, every wave
+// writes its partial of <prev[n,c], g[n,c]> to part[(n*C + c) * nw + wave_of_t]; the
+// partials are summed (and scaled by exp(cs_last)) by state_passing_bwd_finish_kernel.
+// ------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void state_passing_bwd_kernel(
+    const float* __restrict__ prev, const float* __restrict__ cs_last, int64_t cl_sn,
+    int64_t cl_sc, const float* __restrict__ ds, float* __restrict__ g,
+    float* __restrict__ part, int C, int Tdim, int tiles_per_seq, int nw) {
+  const int64_t n = blockIdx.x / tiles_per_seq;
+  const int tile = (int)(blockIdx.x % tiles_per_seq);
+  const int t = tile * 256 + threadIdx.x;
+  const bool ok = t < Tdim;
+  const int wave_id = tile * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int64_t base = n * (int64_t)C * Tdim + (ok ? t : 0);
+  const float* cl = cs_last + n * cl_sn;
+  float cur = 0.f;
+  constexpr int U = 8;
+  for (int c1 = C - 1; c1 >= 0; c1 -= U) {
+    float d[U], p[U], a[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = c1 - u;
+      const bool in = c >= 0;
+      d[u] = (in && ok) ? ds[base + (int64_t)c * Tdim] : 0.f;
+      p[u] = (in && ok) ? prev[base + (int64_t)c * Tdim] : 0.f;
+      a[u] = in ? cl[(int64_t)c * cl_sc] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = c1 - u;
+      if (c >= 0) {  // uniform across the wave
+        if (ok) g[base + (int64_t)c * Tdim] = cur;
+        const float dot = wave_sum(p[u] * cur);
+        if (lane == 0 && wave_id < nw) part[(n * C + c) * (int64_t)nw + wave_id] = dot;
+        cur = fmaf(__expf(a[u]), cur, d[u]);
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void state_passing_bwd_finish_kernel(
+    const float* __restrict__ part, const float* __restrict__ cs_last, int64_t cl_sn,
+    int64_t cl_sc, float* __restrict__ ddA_chunk, int C, int nw, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int64_t n = i / C;
+  const int c = (int)(i - n * C);
+  float s = 0.f;
+  for (int w = 0; w < nw; ++w) s += part[i * nw + w];
+  ddA_chunk[i] = c == 0 ? 0.f : __expf(cs_last[n * cl_sn + (int64_t)c * cl_sc]) * s;
+}
+
+// ------------------------------------------------------------------------------------
+// B4 / B5: per-row dot products against a per-chunk vector.
+//   MODE 0 (db): r[m] = exp(min(cs[Q-1]-cs[m],0)) * <g[n,c], x[n,cQ+m]>, rows past the
+//                chunk limit give 0; out[0] = 0, out[j] = r[j-1] (raw) or
+//                out[j] = sum_{m<j} r[m] (cumulative).
+//   MODE 1 (dc): out[m] = exp(cs[m]) * <dy[n,cQ+m], prev[n,c]>, 0 past the limit.
+// One workgroup per (n, c); wave w takes rows 4*w + 16*i + {0..3}; a wave covers the
+// feature axis with 16-byte loads per lane and reduces with DPP.
+// ------------------------------------------------------------------------------------
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void row_dot_kernel(const T* __restrict__ x, SeqStrides sx,
+                                                      const float* __restrict__ vec,
+                                                      const float* __restrict__ cs,
+                                                      float* __restrict__ out, int nh, int L,
+                                                      int Tdim, int Q, int C, int raw) {
+  constexpr int VEC = Vec16<T>::N;
+  __shared__ float rbuf[EMA_MAX_CHUNK_DEV];
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int64_t chunk_id = blockIdx.x;
+  const int64_t n = chunk_id / C;
+  const int c = (int)(chunk_id - n * C);
+  const int64_t b = n / nh;
+  const int h = (int)(n - b * nh);
+  const int limit = min(Q, L - c * Q);
+  const float* csp = cs + chunk_id * Q;
+  const float cs_last = csp[Q - 1];
+  const float* vp = vec + chunk_id * Tdim;
+  const T* xp = x + b * sx.sb + h * sx.sh + (int64_t)c * Q * sx.sl;
+
+  constexpr int R = 4;
+  for (int m0 = wave * R; m0 < Q; m0 += 4 * R) {
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+    for (int col = lane * VEC; col < Tdim; col += 64 * VEC) {
+      float gv[VEC];
+#pragma unroll
+      for (int i = 0; i < VEC; i += 4) {
+        const float4 t4 = *reinterpret_cast<const float4*>(vp + col + i);
+        gv[i] = t4.x; gv[i + 1] = t4.y; gv[i + 2] = t4.z; gv[i + 3] = t4.w;
+      }
+      Vec16<T> v[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        if (m0 + r < limit) v[r] = load16(xp + (int64_t)(m0 + r) * sx.sl + col);
+        else v[r].zero();
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[r] = fmaf(gv[i], v[r].get(i), acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float s = wave_sum(acc[r]);
+      const int m = m0 + r;
+      if (lane == 0 && m < Q) {
+        float w = 0.f;
+        if (m < limit) w = MODE == 0 ? __expf(fminf(cs_last - csp[m], 0.f)) : __expf(csp[m]);
+        rbuf[m] = w * s;
+      }
+    }
+  }
+  __syncthreads();
+  float* op = out + chunk_id * Q;
+  if (MODE == 1) {
+    for (int m = tid; m < Q; m += 256) op[m] = rbuf[m];
+  } else if (raw) {
+    for (int m = tid; m < Q; m += 256) op[m] = m == 0 ? 0.f : rbuf[m - 1];
+  } else if (wave == 0) {
+    // out[j] = sum_{m<j} r[m]: exclusive scan, lane l owns positions l*per .. l*per+per-1
+    const int per = (Q + 63) >> 6;
+    const int q0 = lane * per;
+    float local = 0.f;
+    for (int i = 0; i < per; ++i)
+      if (q0 + i < Q) local += rbuf[q0 + i];
+    float run = wave_inclusive_scan(local) - local;
+    for (int i = 0; i < per; ++i) {
+      const int q = q0 + i;
+      if (q < Q) {
+        op[q] = run;
+        run += rbuf[q];
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// Final sum of the log-decay gradient, one wave per (n, c):
+//   ddA[j] = intra[j] + next[j] + sum_{m>=j} (s[m] + [m == Q-1] * ddA_chunk)
+// (the reverse cumsum and the three-way add of the reference's combined backward).
+// ------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void combine_dA_kernel(const float* __restrict__ intra,
+                                                         const float* __restrict__ next,
+                                                         const float* __restrict__ sraw,
+                                                         const float* __restrict__ ddA_chunk,
+                                                         float* __restrict__ ddA, int Q,
+                                                         int64_t total_chunks) {
+  const int lane = threadIdx.x & 63;
+  const int64_t chunk_id = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (chunk_id >= total_chunks) return;
+  // Lane l owns the positions Q-1-p for p = l*per .. l*per+per-1, so a forward scan over
+  // the lanes accumulates from the end of the chunk.
+  const int per = (Q + 63) >> 6;
+  const int p0 = lane * per;
+  const float* sp = sraw + chunk_id * Q;
+  const float extra = ddA_chunk[chunk_id];
+  float local = 0.f;
+  for (int i = 0; i < per; ++i) {
+    const int p = p0 + i;
+    if (p < Q) local += sp[Q - 1 - p] + (p == 0 ? extra : 0.f);
+  }
+  float run = wave_inclusive_scan(local) - local;
+  for (int i = 0; i < per; ++i) {
+    const int p = p0 + i;
+    if (p < Q) {
+      const int q = Q - 1 - p;
+      run += sp[q] + (p == 0 ? extra : 0.f);
+      const int64_t o = chunk_id * Q + q;
+      ddA[o] = intra[o] + next[o] + run;
+    }
+  }
+}
+
+}  // namespace ema

@@ -1,0 +1,135 @@
+"""ctypes binding of libema_hip.so (the C ABI declared in include/ema_hip.h).
+
+The library is the only implementation: if it is missing, or no GPU is present, the
+operators raise.  There is no CPU or PyTorch fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libema_hip.so")
+
+EMA_F32, EMA_BF16 = 0, 1
+EMA_MAX_CHUNK = 1024
+
+_I = c_int64
+_P = c_void_p
+_SEQ = [_P, _I, _I, _I]  # pointer + (batch, position, head) strides
+
+_SIGNATURES = {
+    "ema_version": (c_char_p, []),
+    "ema_status_string": (c_char_p, [c_int]),
+    "ema_chunk_cumsum_fwd": (c_int, _SEQ + [_P, _I, _I, _I, _I, _P]),
+    "ema_chunk_state_fwd": (c_int, _SEQ + [c_int, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "ema_state_passing_fwd": (c_int, [_P, _P, _I, _I, _P, _P, _I, _I, _I, _P]),
+    "ema_scan_fwd": (c_int, _SEQ + [c_int, _P, _P] + _SEQ + [_I, _I, _I, _I, _I, _P]),
+    "ema_fwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I]),
+    "ema_fwd": (c_int, _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _P]),
+    "ema_chunk_scan_bwd_dstates": (c_int, _SEQ + [c_int, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "ema_state_passing_bwd_workspace_bytes": (c_size_t, [_I, _I, _I]),
+    "ema_state_passing_bwd": (c_int, [_P, _P, _I, _I, _P, _P, _P, _P, c_size_t, _I, _I, _I, _P]),
+    "ema_chunk_scan_chunk_state_bwd_dx": (c_int, _SEQ + [c_int, _P, _P] + _SEQ + [_I, _I, _I, _I, _I, _P]),
+    "ema_chunk_state_bwd_db": (c_int, _SEQ + [c_int, _P, _P, _P, c_int, _I, _I, _I, _I, _I, _P]),
+    "ema_chunk_scan_bwd_dc": (c_int, _SEQ + [c_int, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "ema_chunk_scan_bwd_ddAcs_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
+    "ema_chunk_scan_bwd_ddAcs": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _P]),
+    "ema_bwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I]),
+    "ema_bwd": (c_int, _SEQ + _SEQ + _SEQ + [c_int] + _SEQ + [_P] + _SEQ + [_P, c_size_t, _I, _I, _I, _I, _I, _P]),
+}
+
+_lib = None
+
+
+def exported_symbols():
+    """Names every build of the library must export (one per declaration in ema_hip.h)."""
+    return sorted(_SIGNATURES)
+
+
+def lib():
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python triton-kernels_amd/build.py` "
+                "(the EMA operators have no fallback implementation)"
+            )
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+_ERRORS = {
+    -1: (ValueError, "null pointer"),
+    -2: (AssertionError, "bad shape"),
+    -3: (AssertionError, "dim, stride or pointer not 16-byte aligned"),
+    -4: (TypeError, "unsupported dtype"),
+    -5: (NotImplementedError, "unsupported"),
+    -6: (RuntimeError, "kernel launch failed"),
+}
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        exc, msg = _ERRORS.get(status, (RuntimeError, f"status {status}"))
+        raise exc(f"{what}: {msg}")
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return EMA_F32
+    if t.dtype == torch.bfloat16:
+        return EMA_BF16
+    raise TypeError(f"EMA kernels take float32 or bfloat16 sequences, got {t.dtype}")
+
+
+def require_gpu(*tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    if dev.type != "cuda":
+        raise RuntimeError("EMA kernels run on the GPU only (tensor is on %s)" % dev)
+    for t in tensors:
+        if t is not None and t.device != dev:
+            raise AssertionError("all tensors must be on the same device")
+    return dev
+
+
+def stream_ptr(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def seq_view(x: torch.Tensor):
+    """(tensor with unit feature stride, [ptr, sb, sl, sh], batch, nheads, L, T) of a flat
+    (B, L, T) or headed (b, L, nh, d) sequence tensor."""
+    assert x.dim() in (3, 4), "expected (B, L, T) or (b, L, nh, d)"
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    if x.dim() == 3:
+        B, L, T = x.shape
+        return x, [x.data_ptr(), x.stride(0), x.stride(1), 0], B, 1, L, T
+    b, L, nh, d = x.shape
+    return x, [x.data_ptr(), x.stride(0), x.stride(1), x.stride(2)], b, nh, L, d
+
+
+def decay_view(A: torch.Tensor):
+    """([ptr, sb, sl, sh], batch, nheads, L) of a flat (B, L) or headed (b, L, nh) log-decay."""
+    assert A.dim() in (2, 3), "expected (B, L) or (b, L, nh)"
+    assert A.dtype == torch.float32, "log-decay must be float32"
+    if A.dim() == 2:
+        return [A.data_ptr(), A.stride(0), A.stride(1), 0], A.shape[0], 1, A.shape[1]
+    return [A.data_ptr(), A.stride(0), A.stride(1), A.stride(2)], A.shape[0], A.shape[2], A.shape[1]
+
+
+def f32c(t: torch.Tensor) -> torch.Tensor:
+    """Dense float32 view/copy of a chunked intermediate."""
+    if t.dtype != torch.float32:
+        t = t.float()
+    return t.contiguous()
