@@ -1,0 +1,266 @@
+#!/usr/bin/env python3
+"""Benchmark of the EMA chunked scan, forward + backward, on one MI355X.
+
+One step = one forward (cumsum, chunk states, state passing, chunk scan) and one backward
+(recompute + dstates, reverse state passing, dx, the three log-decay gradient terms) of
+BASELINE configuration 3 at chunk size 128: b16 nh2 d1024 L4096, bf16 x / dy, fp32
+log-decay and accumulation.  Inputs are synthetic and resident in HBM before the timed
+region; the step rotates over several input sets so that no step finds its inputs in the
+256 MB last-level cache.
+
+Prints ONE JSON line.  `roofline` describes the kernel with the largest share of the step,
+timed live with HIP events on the launch stream; `cpu_baseline` is the sequential CPU
+oracle timed on a bounded sample and scaled to the full workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "triton-kernels_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--chunk", type=int, default=128)
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--nheads", type=int, default=2)
+    ap.add_argument("--seqlen", type=int, default=4096)
+    ap.add_argument("--dim", type=int, default=1024)
+    ap.add_argument("--sets", type=int, default=3, help="input sets the steps rotate over")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel timing pass")
+    return ap.parse_args()
+
+
+def algorithmic_bytes(N, L, T, Q, esize):
+    """Compulsory HBM bytes per launch of each stage (every input read once, every output
+    written once), and of the whole forward / backward."""
+    C = -(-L // Q)
+    x = N * L * T * esize
+    a = N * L * 4
+    st = N * C * T * 4
+    return {
+        "cumsum": 2 * a,
+        "chunk_state": x + a + st,
+        "state_passing_fwd": 2 * st + N * C * 4 + N * T * 4,
+        "chunk_scan": 2 * x + a + st,
+        "bwd_dstates": x + a + st,
+        "state_passing_bwd": 3 * st + 2 * N * C * 4,
+        "bwd_dx": 2 * x + a + st,
+        "bwd_db": x + st + 2 * a,
+        "bwd_dc": x + st + 2 * a,
+        "bwd_da_intra": 2 * x + 2 * a,
+        "fwd": 2 * x + a,
+        "bwd": 3 * x + 2 * a,
+    }
+
+
+def time_region(fn, iters, torch):
+    """Average milliseconds of fn() over `iters` calls, HIP events on the current stream."""
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for i in range(iters):
+        fn(i)
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / iters
+
+
+def cpu_baseline(args, torch):
+    """Sequential CPU oracle (forward + closed-form reverse recurrence) on a sample of the
+    workload's sequences, scaled linearly to all of them."""
+    from oracle import ema_oracle as O
+
+    threads = torch.get_num_threads()
+    nseq_total = args.batch * args.nheads
+    sample_b = 1
+    x, A, dy = O.make_inputs(sample_b, args.nheads, args.seqlen, args.dim, seed=1, dtype=torch.bfloat16)
+    xf, Af = O.to_flat(x.float(), A)
+    dyf, _ = O.to_flat(dy.float(), A)
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        O.ema_loop(xf, Af)
+        O.ema_loop_bwd(dyf, xf, Af)
+        reps += 1
+        if time.perf_counter() - t0 > 10.0 or reps >= 20:
+            break
+    per = (time.perf_counter() - t0) / reps
+    scale = nseq_total / (sample_b * args.nheads)
+    return {
+        "value": per * scale * 1e3,
+        "unit": "ms",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{sample_b * args.nheads} of {nseq_total} sequences (L={args.seqlen}, d={args.dim}), "
+        f"fwd + bwd sequential recurrence in fp32 torch, {reps} repetitions, scaled x{scale:g}",
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU only: the EMA scan has no multi-GPU path in this build "
+              "(run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from kernels.ema_kernels.ema_combined_fwd import _ema_matmul_scan_combined_fwd
+    from kernels.ema_kernels_bwd.ema_combined_bwd import _ema_chunk_scan_combined_bwd
+    from oracle import ema_oracle as O
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    b, nh, L, T, Q = args.batch, args.nheads, args.seqlen, args.dim, args.chunk
+    N = b * nh
+    sets = []
+    for s in range(args.sets):
+        x, A, dy = O.make_inputs(b, nh, L, T, seed=1000 + Q + s, dtype=torch.bfloat16)
+        sets.append((x.to(dev), A.to(dev), dy.to(dev)))
+    del x, A, dy
+
+    def step(i):
+        x, A, dy = sets[i % len(sets)]
+        _ema_matmul_scan_combined_fwd(A, x, Q)
+        _ema_chunk_scan_combined_bwd(dy, x, A, Q)
+
+    def fwd_only(i):
+        x, A, dy = sets[i % len(sets)]
+        _ema_matmul_scan_combined_fwd(A, x, Q)
+
+    def bwd_only(i):
+        x, A, dy = sets[i % len(sets)]
+        _ema_chunk_scan_combined_bwd(dy, x, A, Q)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ms_step_events = time_region(step, args.steps, torch)
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_step = max(ms_step_events, wall_ms)
+
+    ab = algorithmic_bytes(N, L, T, Q, 2)
+    ms_fwd = time_region(fwd_only, args.steps, torch)
+    ms_bwd = time_region(bwd_only, args.steps, torch)
+
+    kernels = {}
+    if not args.no_kernels:
+        kernels = time_kernels(sets, Q, args.steps, ab, torch)
+
+    out = {
+        "metric": "EMA scan fwd+bwd ms @ b16 nh2 d1024 L4096 c128",
+        "value": ms_step,
+        "unit": "ms",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"EMA chunked scan fwd+bwd, b{b} nh{nh} d{T} L{L} chunk{Q}, bf16 x/dy, fp32 log-decay",
+            "batch": b, "nheads": nh, "seqlen": L, "dim": T, "chunk": Q,
+        },
+        "fwd_ms": ms_fwd,
+        "bwd_ms": ms_bwd,
+        "hbm_algorithmic_GBps": {
+            "fwd": ab["fwd"] / ms_fwd / 1e6,
+            "bwd": ab["bwd"] / ms_bwd / 1e6,
+            "fwd+bwd": (ab["fwd"] + ab["bwd"]) / ms_step / 1e6,
+        },
+        "hbm_frac_of_peak_fwd+bwd": (ab["fwd"] + ab["bwd"]) / ms_step / 1e6 / HBM_PEAK_GBS,
+        "kernels": kernels,
+    }
+    if kernels:
+        dom = max(kernels, key=lambda k: kernels[k]["ms"])
+        out["roofline"] = {
+            "kernel": dom,
+            "bound": "hbm",
+            "achieved": kernels[dom]["GBps"],
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": kernels[dom]["GBps"] / HBM_PEAK_GBS,
+            "traffic": None,
+        }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args, torch)
+    print(json.dumps(out))
+
+
+def time_kernels(sets, Q, iters, ab, torch):
+    """Per-stage timing through the per-stage launchers (one kernel each, plus at most one
+    tiny finishing kernel), HIP events on the launch stream."""
+    from kernels.ema_kernels.ema_cumsum import ema_chunk_cumsum_fwd
+    from kernels.ema_kernels.ema_scan_fwd import _ema_scan_fwd
+    from kernels.ema_kernels.ema_state_fwd import _ema_chunk_state_fwd
+    from kernels.ema_kernels.ema_state_pass import _ema_state_passing_fwd
+    from kernels.ema_kernels_bwd.ema_chunk_scan_bwd_dc import _ema_chunk_scan_bwd_dC
+    from kernels.ema_kernels_bwd.ema_chunk_scan_chunk_state_bwd_dx import _chunk_scan_chunk_state_bwd_dx
+    from kernels.ema_kernels_bwd.ema_chunk_state_bwd_db import _ema_chunk_state_bwd_db
+    from kernels.ema_kernels_bwd.ema_scan_bwd import _ema_chunk_scan_bwd_dstates
+    from kernels.ema_kernels_bwd.ema_scan_da import _ema_chunk_scan_bwd_ddAcs_stable
+    from kernels.ema_kernels_bwd.ema_state_passing_bwd_dstates import _ema_state_passing_bwd
+
+    inter = []
+    for x, A, dy in sets:
+        cs = ema_chunk_cumsum_fwd(A, Q)
+        states = _ema_chunk_state_fwd(x, cs)
+        prev, _ = _ema_state_passing_fwd(states, cs[..., -1], out_dtype=torch.float32)
+        ds = _ema_chunk_scan_bwd_dstates(cs, dy)
+        g, _, _ = _ema_state_passing_bwd(prev, cs[..., -1], ds)
+        inter.append((cs, states, prev, ds, g))
+
+    def pick(i):
+        k = i % len(sets)
+        return sets[k] + inter[k]
+
+    stages = {
+        "cumsum": lambda i: ema_chunk_cumsum_fwd(pick(i)[1], Q),
+        "chunk_state": lambda i: _ema_chunk_state_fwd(pick(i)[0], pick(i)[3]),
+        "state_passing_fwd": lambda i: _ema_state_passing_fwd(pick(i)[4], pick(i)[3][..., -1]),
+        "chunk_scan": lambda i: _ema_scan_fwd(pick(i)[0], pick(i)[3], pick(i)[5]),
+        "bwd_dstates": lambda i: _ema_chunk_scan_bwd_dstates(pick(i)[3], pick(i)[2]),
+        "state_passing_bwd": lambda i: _ema_state_passing_bwd(pick(i)[5], pick(i)[3][..., -1], pick(i)[6]),
+        "bwd_dx": lambda i: _chunk_scan_chunk_state_bwd_dx(pick(i)[0], pick(i)[3], pick(i)[2], pick(i)[7]),
+        "bwd_db": lambda i: _ema_chunk_state_bwd_db(pick(i)[0], pick(i)[3], pick(i)[7]),
+        "bwd_dc": lambda i: _ema_chunk_scan_bwd_dC(pick(i)[5], pick(i)[3], pick(i)[2]),
+        "bwd_da_intra": lambda i: _ema_chunk_scan_bwd_ddAcs_stable(pick(i)[0], pick(i)[3], pick(i)[2]),
+    }
+    res = {}
+    for name, fn in stages.items():
+        for i in range(3):
+            fn(i)
+        ms = time_region(fn, iters, torch)
+        gbps = ab[name] / ms / 1e6
+        res[name] = {"ms": ms, "GBps": gbps, "hbm_frac": gbps / HBM_PEAK_GBS, "bytes": ab[name]}
+    x = sets[0][0]
+    N, L, T = x.shape[0] * x.shape[2], x.shape[1], x.shape[3]
+    flops = 2.0 * Q * L * T * N
+    for name in ("chunk_scan", "bwd_dx", "bwd_da_intra"):
+        tf = flops / res[name]["ms"] / 1e9
+        res[name]["dense_TFLOPs"] = tf
+        res[name]["mfma_frac_dense"] = tf / MFMA_BF16_PEAK_TFLOPS
+    return res
+
+
+if __name__ == "__main__":
+    main()

@@ -108,6 +108,26 @@ __device__ __forceinline__ void mma_group(const Vec16<float>& a, const Vec16<flo
   acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.raw.w, b.raw.w, acc, 0, 0, 0);
 }
 
+// B operand of a bf16 MFMA group from a row-major LDS tile t[k][col] (pitch in elements):
+// lane l receives t[k0 + 8*(l/32) + e][col0 + l%32], e = 0..7, through two transposing
+// 64-bit LDS reads.  In each group of 16 lanes, lane i supplies the address of four
+// consecutive columns of row i/4 and receives, for column i of the 16-column strip, the
+// four rows of the group.
+typedef bf16_t bf16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ Vec16<bf16_t> lds_read_kmajor(const bf16_t* t, int pitch, int k0,
+                                                         int col0, int lane) {
+  const int i = lane & 15;
+  const int row = k0 + 8 * (lane >> 5) + (i >> 2);
+  const int col = col0 + 16 * ((lane >> 4) & 1) + 4 * (i & 3);
+  const bf16_t* p = t + row * pitch + col;
+  typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
+  const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)p);
+  const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(p + 4 * pitch));
+  Vec16<bf16_t> r;
+  r.raw = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return r;
+}
+
 __device__ __forceinline__ int acc_row(int v, int lane) {
   return 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
 }

@@ -97,21 +97,41 @@ __global__ __launch_bounds__(256) void chunk_gemm_kernel(
     const int kg_lo = REVERSE ? max(0, (wave_lo - kt0) / KG * KG) : 0;
     const int kg_hi = REVERSE ? min(kBM, k_hi - kt0) : min(kBM, min(wave_hi, k_hi) - kt0);
     for (int kg = kg_lo; kg < kg_hi; kg += KG) {
-      Vec16<T> a;
       const int kl = kg + EPL * half;  // first k of this lane inside the tile
+      float m[EPL];
 #pragma unroll
       for (int e = 0; e < EPL; ++e) {
         const int k = kt0 + kl + e;
         const float d = REVERSE ? cs_s[k] - cs_m : cs_m - cs_s[k];
         const bool keep = REVERSE ? (k >= m_lane) : (k <= m_lane);
-        a.set(e, keep ? __expf(fminf(d, 0.f)) : 0.f);
+        m[e] = keep ? __expf(fminf(d, 0.f)) : 0.f;
       }
+      if constexpr (sizeof(T) == 2) {
+        // bf16: the decay factors go in as hi + lo (two bf16 terms, ~16 significant bits)
+        // so that the product with the exact bf16 inputs keeps f32-grade accuracy.
+        Vec16<T> a_hi, a_lo;
 #pragma unroll
-      for (int db = 0; db < kBN / 32; ++db) {
-        Vec16<T> bfrag;
+        for (int e = 0; e < EPL; ++e) {
+          a_hi.set(e, m[e]);
+          a_lo.set(e, m[e] - a_hi.get(e));
+        }
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) bfrag.put(e, xs[(kl + e) * ROW + db * 32 + l32]);
-        mma_group(a, bfrag, acc[db]);
+        for (int db = 0; db < kBN / 32; ++db) {
+          const Vec16<T> bfrag = lds_read_kmajor(xs, ROW, kg, db * 32, lane);
+          mma_group(a_hi, bfrag, acc[db]);
+          mma_group(a_lo, bfrag, acc[db]);
+        }
+      } else {
+        Vec16<T> a;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) a.set(e, m[e]);
+#pragma unroll
+        for (int db = 0; db < kBN / 32; ++db) {
+          Vec16<T> bfrag;
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) bfrag.put(e, xs[(kl + e) * ROW + db * 32 + l32]);
+          mma_group(a, bfrag, acc[db]);
+        }
       }
     }
   }
