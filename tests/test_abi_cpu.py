@@ -43,6 +43,7 @@ def test_workspace_sizes():
     assert handle.ema_state_passing_bwd_workspace_bytes(32, 32, 1024) == 32 * 32 * 16 * 4
     assert handle.ema_chunk_scan_bwd_ddAcs_workspace_bytes(16, 2, 4096, 128) == 2 * 32 * 32 * 128 * 4
     assert handle.ema_bwd_workspace_bytes(16, 2, 4096, 1024, 128) > 4 * 32 * 32 * 1024 * 4
+    assert handle.ema_bwd_workspace_bytes(16, 2, 4096, 1024, 512) == handle.ema_bwd_workspace_bytes(16, 2, 4096, 1024, 128)
     # refused shapes report 0 bytes
     assert handle.ema_fwd_workspace_bytes(0, 2, 4096, 1024, 128) == 0
     assert handle.ema_bwd_workspace_bytes(16, 2, 4096, 1024, _lib.EMA_MAX_CHUNK + 1) == 0

@@ -47,10 +47,48 @@ def test_combined_vs_sequential(N, L, T, Q, kind, dtype, device):
     assert ddA.shape == (N, -(-L // Q), Q) and ddA.dtype == F32
     check_close("dA", ddA.reshape(N, -1)[:, :L], dA_ref, dtype)
     C = cs.shape[1]
-    for c in range(1, C):
-        pass
     ref_prev = torch.stack([y_ref[:, c * Q - 1] if c else torch.zeros(N, T) for c in range(C)], 1)
     check_close("prev", prev, ref_prev, F32 if dtype == F32 else BF16)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("N,L,T,Q", [(2, 1024, 256, 128), (2, 900, 64, 256), (1, 512, 128, 64)])
+def test_staged_backward_composition(N, L, T, Q, dtype, device):
+    """The stage launchers, glued as in kernels/ema_kernels_bwd/ema_combined_bwd.py:32-83 of
+    the reference, give the same gradients as the single-call backward and the oracle."""
+    from kernels.ema_kernels.ema_cumsum import ema_chunk_cumsum_fwd
+    from kernels.ema_kernels.ema_state_fwd import _ema_chunk_state_fwd
+    from kernels.ema_kernels.ema_state_pass import _ema_state_passing_fwd
+    from kernels.ema_kernels_bwd.ema_chunk_scan_bwd_dc import _ema_chunk_scan_bwd_dC
+    from kernels.ema_kernels_bwd.ema_chunk_scan_chunk_state_bwd_dx import _chunk_scan_chunk_state_bwd_dx
+    from kernels.ema_kernels_bwd.ema_chunk_state_bwd_db import _ema_chunk_state_bwd_db
+    from kernels.ema_kernels_bwd.ema_combined_bwd import _ema_chunk_scan_combined_bwd
+    from kernels.ema_kernels_bwd.ema_scan_bwd import _ema_chunk_scan_bwd_dstates
+    from kernels.ema_kernels_bwd.ema_scan_da import _ema_chunk_scan_bwd_ddAcs_stable
+    from kernels.ema_kernels_bwd.ema_state_passing_bwd_dstates import _ema_state_passing_bwd
+
+    announce(f"staged backward N{N} L{L} T{T} Q{Q} {dtype}")
+    A, X, dy = flat_case(N, L, T, seed=300 + L, dtype=dtype)
+    Ad, Xd, dyd = A.to(device), X.to(device), dy.to(device)
+    cs = ema_chunk_cumsum_fwd(Ad, Q)
+    states = _ema_chunk_state_fwd(Xd, cs)
+    prev, _ = _ema_state_passing_fwd(states, cs[..., -1], out_dtype=torch.float32)
+    ds = _ema_chunk_scan_bwd_dstates(cs, dyd)
+    g, ddA_chunk, _ = _ema_state_passing_bwd(prev, cs[..., -1], ds, chunk_size=Q)
+    dx = _chunk_scan_chunk_state_bwd_dx(Xd, cs, dyd, g)
+    ddA_next = _ema_chunk_state_bwd_db(Xd, cs, g)
+    ddA_prev = _ema_chunk_scan_bwd_dC(prev, cs, dyd)
+    ddA_prev[..., -1] += ddA_chunk
+    ddA_prev = ddA_prev.flip([-1]).cumsum(dim=-1).flip([-1])
+    ddA = _ema_chunk_scan_bwd_ddAcs_stable(Xd, cs, dyd) + ddA_next + ddA_prev
+    dx_ref, dA_ref = O.ema_loop_bwd(dy.float(), X.float(), A)
+    check_close("dx staged", dx, dx_ref, dtype)
+    check_close("dA staged", ddA.reshape(N, -1)[:, :L], dA_ref, dtype)
+    dx1, ddA1 = _ema_chunk_scan_combined_bwd(dyd, Xd, Ad, Q)
+    check_close("dx single call", dx1, dx_ref, dtype)
+    check_close("dA single call", ddA1.reshape(N, -1)[:, :L], dA_ref, dtype)
+    # slots past the end of the sequence are defined as zero by the single-call backward
+    assert float(ddA1.reshape(N, -1)[:, L:].abs().sum()) == 0.0
 
 
 def _headed_reference(x, A, dy):

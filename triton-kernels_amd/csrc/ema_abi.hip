@@ -7,6 +7,7 @@
 #include "ema_device.h"
 #include "ema_gemm_kernels.h"
 #include "ema_stream_kernels.h"
+#include "ema_walk_kernels.h"
 
 using namespace ema;
 
@@ -109,8 +110,13 @@ int launch_state_passing_bwd(const float* prev, const float* cs_last, int64_t cl
                              float* part, int64_t N, int64_t C, int64_t T, hipStream_t st) {
   const int tiles = (int)((T + 255) / 256);
   const int nw = (int)((T + 63) / 64);
-  hipLaunchKernelGGL(state_passing_bwd_kernel, dim3((unsigned)(N * tiles)), dim3(256), 0, st, prev,
-                     cs_last, cl_sn, cl_sc, ds, g, part, (int)C, (int)T, tiles, nw);
+  if (!ddA_chunk) {  // only the recurrence; no <prev, g> products
+    hipLaunchKernelGGL(state_passing_bwd_kernel<false>, dim3((unsigned)(N * tiles)), dim3(256), 0,
+                       st, prev, cs_last, cl_sn, cl_sc, ds, g, part, (int)C, (int)T, tiles, nw);
+    return launched();
+  }
+  hipLaunchKernelGGL(state_passing_bwd_kernel<true>, dim3((unsigned)(N * tiles)), dim3(256), 0, st,
+                     prev, cs_last, cl_sn, cl_sc, ds, g, part, (int)C, (int)T, tiles, nw);
   EMA_TRY(launched());
   const int64_t total = N * C;
   hipLaunchKernelGGL(state_passing_bwd_finish_kernel, dim3((unsigned)((total + 255) / 256)),
@@ -118,21 +124,62 @@ int launch_state_passing_bwd(const float* prev, const float* cs_last, int64_t cl
   return launched();
 }
 
+// Kernels that ask for more dynamic LDS than the default limit must opt in once.
+template <typename K>
+int allow_smem(K kernel, int bytes) {
+  if (bytes <= 48 * 1024) return EMA_OK;
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess
+             ? EMA_OK
+             : EMA_ERR_LAUNCH;
+}
+
+constexpr int kWalkBnBf16 = 128;  // column tile of the intra-chunk kernels, bf16
+constexpr int kWalkBnF32 = 64;    // and f32 (both are 256 bytes per row)
+
+template <typename T, int BN, bool REVERSE>
+int launch_chunk_scan_t(const void* in, SeqStrides si, const float* cs, const float* vec, void* out,
+                        SeqStrides so, const Dims& d, hipStream_t st) {
+  const int ntiles = (int)((d.T + BN - 1) / BN);
+  const int64_t grid = d.N * d.C * ntiles;
+  if (grid > 0x7fffffff) return EMA_ERR_SHAPE;
+  const int smem = WalkCfg<T, BN>::smem_bytes(1);
+  auto kernel = chunk_scan_walk_kernel<T, BN, REVERSE>;
+  EMA_TRY(allow_smem(kernel, smem));
+  hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), smem, st, (const T*)in, si, cs, vec,
+                     (T*)out, so, (int)d.nh, (int)d.L, (int)d.T, (int)d.Q, (int)d.C, ntiles);
+  return launched();
+}
+
 template <bool REVERSE>
 int launch_chunk_gemm(const void* in, SeqStrides si, int dtype, const float* cs, const float* vec,
                       void* out, SeqStrides so, const Dims& d, hipStream_t st) {
-  const int MT = (int)((d.Q + kBM - 1) / kBM);
-  const int ntiles = (int)((d.T + kBN - 1) / kBN);
-  const int64_t grid = d.N * d.C * MT * ntiles;
-  if (grid > 0x7fffffff) return EMA_ERR_SHAPE;
   if (dtype == EMA_BF16)
-    hipLaunchKernelGGL((chunk_gemm_kernel<bf16_t, REVERSE>), dim3((unsigned)grid), dim3(256), 0, st,
-                       (const bf16_t*)in, si, cs, vec, (bf16_t*)out, so, (int)d.nh, (int)d.L,
-                       (int)d.T, (int)d.Q, (int)d.C, MT, ntiles);
-  else
-    hipLaunchKernelGGL((chunk_gemm_kernel<float, REVERSE>), dim3((unsigned)grid), dim3(256), 0, st,
-                       (const float*)in, si, cs, vec, (float*)out, so, (int)d.nh, (int)d.L,
-                       (int)d.T, (int)d.Q, (int)d.C, MT, ntiles);
+    return launch_chunk_scan_t<bf16_t, kWalkBnBf16, REVERSE>(in, si, cs, vec, out, so, d, st);
+  return launch_chunk_scan_t<float, kWalkBnF32, REVERSE>(in, si, cs, vec, out, so, d, st);
+}
+
+template <typename T, int BN>
+int launch_bwd_fused_t(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* cs,
+                       const float* prev, const float* g, void* dx, SeqStrides sdx, void* y,
+                       SeqStrides sy, float* part, const Dims& di, hipStream_t st) {
+  const int ntiles = (int)((di.T + BN - 1) / BN);
+  const int64_t grid = di.N * di.C * ntiles;
+  if (grid > 0x7fffffff) return EMA_ERR_SHAPE;
+  const int smem = WalkCfg<T, BN>::smem_bytes(2);
+  if (y) {
+    auto kernel = bwd_fused_kernel<T, BN, true>;
+    EMA_TRY(allow_smem(kernel, smem));
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), smem, st, (const T*)x, sx,
+                       (const T*)dy, sd, cs, prev, g, (T*)dx, sdx, (T*)y, sy, part, (int)di.nh,
+                       (int)di.L, (int)di.T, (int)di.C, ntiles);
+  } else {
+    auto kernel = bwd_fused_kernel<T, BN, false>;
+    EMA_TRY(allow_smem(kernel, smem));
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), smem, st, (const T*)x, sx,
+                       (const T*)dy, sd, cs, prev, g, (T*)dx, sdx, (T*)nullptr, sy, part, (int)di.nh,
+                       (int)di.L, (int)di.T, (int)di.C, ntiles);
+  }
   return launched();
 }
 
@@ -176,13 +223,26 @@ size_t da_part_floats(const Dims& d) {
   return (size_t)(d.N * d.C * MT * d.Q);
 }
 
-// Workspace carving for ema_bwd.
+// Workspace carving for ema_bwd.  The backward chunks the sequence by 128 internally,
+// whatever the chunk size of the interface: di describes that chunking.
 struct BwdWs {
-  float *cs, *states, *prev, *ds, *g, *sp_part, *ddA_chunk, *da_part, *rowsum, *intra, *next, *sraw;
+  float *cs, *states, *prev, *ds, *g, *part;
   size_t bytes;
 };
 
-BwdWs carve_bwd(void* base, const Dims& d) {
+Dims internal_dims(const Dims& d) {
+  Dims di = d;
+  di.Q = kTileRows;
+  di.C = (d.L + kTileRows - 1) / kTileRows;
+  return di;
+}
+
+int bwd_col_tiles(const Dims& d, int dtype) {
+  const int bn = dtype == EMA_BF16 ? kWalkBnBf16 : kWalkBnF32;
+  return (int)((d.T + bn - 1) / bn);
+}
+
+BwdWs carve_bwd(void* base, const Dims& di, int dtype) {
   BwdWs w;
   size_t off = 0;
   char* p = static_cast<char*>(base);
@@ -191,19 +251,13 @@ BwdWs carve_bwd(void* base, const Dims& d) {
     off += align_up(floats * sizeof(float), 256);
     return r;
   };
-  const size_t ncq = (size_t)(d.N * d.C * d.Q), nct = (size_t)(d.N * d.C * d.T);
+  const size_t ncq = (size_t)(di.N * di.C * di.Q), nct = (size_t)(di.N * di.C * di.T);
   w.cs = take(ncq);
   w.states = take(nct);
   w.prev = take(nct);
   w.ds = take(nct);
   w.g = take(nct);
-  w.sp_part = take((size_t)(d.N * d.C * ((d.T + 63) / 64)));
-  w.ddA_chunk = take((size_t)(d.N * d.C));
-  w.da_part = take(da_part_floats(d));
-  w.rowsum = take(ncq);
-  w.intra = take(ncq);
-  w.next = take(ncq);
-  w.sraw = take(ncq);
+  w.part = take(ncq * (size_t)bwd_col_tiles(di, dtype));
   w.bytes = off;
   return w;
 }
@@ -413,7 +467,8 @@ size_t ema_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, in
                                int64_t chunk) {
   Dims d;
   if (check_dims(batch, nheads, seqlen, dim, chunk, true, &d) != EMA_OK) return 0;
-  return carve_bwd(nullptr, d).bytes;
+  // sized for the wider of the two column tilings so that it does not depend on the dtype
+  return carve_bwd(nullptr, internal_dims(d), EMA_F32).bytes;
 }
 
 int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const void* x,
@@ -434,31 +489,38 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
   if (workspace_bytes < ema_bwd_workspace_bytes(batch, nheads, seqlen, dim, chunk))
     return EMA_ERR_SHAPE;
   hipStream_t st = as_stream(stream);
-  const BwdWs w = carve_bwd(workspace, d);
+  // The gradients do not depend on how the sequence is chunked, so the backward always
+  // works on 128-row chunks (one tile of the fused kernel); `chunk` only fixes the
+  // (N, C, Q) layout in which ddA is returned.
+  const Dims di = internal_dims(d);
+  const BwdWs w = carve_bwd(workspace, di, dtype);
   const SeqStrides sx{x_sb, x_sl, x_sh}, sd{dy_sb, dy_sl, dy_sh}, sdx{dx_sb, dx_sl, dx_sh};
-  const float* cs_last = w.cs + (d.Q - 1);
-  const int64_t cl_sn = d.C * d.Q, cl_sc = d.Q;
+  const SeqStrides sy{y_sb, y_sl, y_sh};
+  const float* cs_last = w.cs + (di.Q - 1);
+  const int64_t cl_sn = di.C * di.Q, cl_sc = di.Q;
 
-  // recompute the forward intermediates
-  EMA_TRY(launch_cumsum(A, SeqStrides{a_sb, a_sl, a_sh}, w.cs, d, st));
-  EMA_TRY(launch_chunk_reduce<0>(x, sx, dtype, w.cs, w.states, d, st));
-  // final state is not needed; ds is free until B1 runs, use its first N*T floats
-  EMA_TRY(launch_state_passing_fwd(w.states, cs_last, cl_sn, cl_sc, w.prev, w.ds, d.N, d.C, d.T,
+  // forward intermediates: cumsum, chunk states, states entering each chunk
+  EMA_TRY(launch_cumsum(A, SeqStrides{a_sb, a_sl, a_sh}, w.cs, di, st));
+  EMA_TRY(launch_chunk_reduce<0>(x, sx, dtype, w.cs, w.states, di, st));
+  // the final state is not needed; ds is free until B1 runs, its first N*T floats take it
+  EMA_TRY(launch_state_passing_fwd(w.states, cs_last, cl_sn, cl_sc, w.prev, w.ds, di.N, di.C, di.T,
                                    st));
-  if (y)
-    EMA_TRY(launch_chunk_gemm<false>(x, sx, dtype, w.cs, w.prev, y, SeqStrides{y_sb, y_sl, y_sh}, d,
-                                     st));
-  // backward proper
-  EMA_TRY(launch_chunk_reduce<1>(dy, sd, dtype, w.cs, w.ds, d, st));
-  EMA_TRY(launch_state_passing_bwd(w.prev, cs_last, cl_sn, cl_sc, w.ds, w.g, w.ddA_chunk,
-                                   w.sp_part, d.N, d.C, d.T, st));
-  EMA_TRY(launch_chunk_gemm<true>(dy, sd, dtype, w.cs, w.g, dx, sdx, d, st));
-  EMA_TRY(launch_row_dot<0>(x, sx, dtype, w.g, w.cs, w.next, 0, d, st));
-  EMA_TRY(launch_row_dot<1>(dy, sd, dtype, w.prev, w.cs, w.sraw, 0, d, st));
-  EMA_TRY(launch_da(x, sx, dy, sd, dtype, w.cs, w.intra, w.da_part, w.rowsum, d, st));
-  const int64_t total = d.N * d.C;
-  hipLaunchKernelGGL(combine_dA_kernel, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, st, w.intra,
-                     w.next, w.sraw, w.ddA_chunk, ddA, (int)d.Q, total);
+  // gradient of the states: B1, then the reverse recurrence B2 (without its <prev, g>
+  // products, which the fused kernel does not need)
+  EMA_TRY(launch_chunk_reduce<1>(dy, sd, dtype, w.cs, w.ds, di, st));
+  EMA_TRY(launch_state_passing_bwd(w.prev, cs_last, cl_sn, cl_sc, w.ds, w.g, nullptr, nullptr, di.N,
+                                   di.C, di.T, st));
+  // dx, the recomputed y and the per-column-tile partials of dA in one pass over x and dy
+  if (dtype == EMA_BF16)
+    EMA_TRY((launch_bwd_fused_t<bf16_t, kWalkBnBf16>(x, sx, dy, sd, w.cs, w.prev, w.g, dx, sdx, y, sy,
+                                                     w.part, di, st)));
+  else
+    EMA_TRY((launch_bwd_fused_t<float, kWalkBnF32>(x, sx, dy, sd, w.cs, w.prev, w.g, dx, sdx, y, sy,
+                                                   w.part, di, st)));
+  const int64_t total = d.N * d.C * d.Q;
+  hipLaunchKernelGGL(dA_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                     w.part, ddA, (int)d.L, (int)d.Q, (int)d.C, (int)di.C, bwd_col_tiles(di, dtype),
+                     total);
   return launched();
 }
 

@@ -1,152 +1,12 @@
-// MFMA kernels of the EMA chunked scan: the intra-chunk contraction with the segsum-decay
-// matrix (forward y, backward dx) and the dy . x^T contraction over the feature axis for
-// the intra-chunk log-decay gradient.  bf16 operands use v_mfma_f32_32x32x16_bf16, f32
-// operands v_mfma_f32_32x32x2_f32; accumulation is f32 in both.
+// The dy . x^T contraction over the feature axis for the intra-chunk log-decay gradient
+// (stage B6 on its own).  bf16 operands use v_mfma_f32_32x32x16_bf16, f32 operands
+// v_mfma_f32_32x32x2_f32; accumulation is f32 in both.
 #pragma once
 #include "ema_device.h"
 
 namespace ema {
 
 constexpr int kBM = 128;  // rows of a chunk handled by one workgroup (4 waves x 32)
-constexpr int kBN = 64;   // feature columns handled by one workgroup of chunk_gemm_kernel
-
-// ------------------------------------------------------------------------------------
-// F4 (REVERSE = false):
-//   out[m,t] = exp(min(cs[m],0)) * vec[t] + sum_{k<=m} exp(min(cs[m]-cs[k],0)) * in[k,t]
-// B3 (REVERSE = true):
-//   out[m,t] = exp(min(cs[Q-1]-cs[m],0)) * vec[t] + sum_{k>=m} exp(min(cs[k]-cs[m],0)) * in[k,t]
-// per chunk.  One workgroup per (n, c, 128-row tile, 64-column tile).  The input rows are
-// staged through LDS in tiles of 128 rows; wave w owns rows 32w..32w+31 of the row tile,
-// builds its slice of the decay matrix in registers (one exp per element, in the operand
-// layout of the MFMA) and reuses it for both 32-column blocks.
-// ------------------------------------------------------------------------------------
-template <typename T, bool REVERSE>
-__global__ __launch_bounds__(256) void chunk_gemm_kernel(
-    const T* __restrict__ in, SeqStrides si, const float* __restrict__ cs,
-    const float* __restrict__ vec, T* __restrict__ out, SeqStrides so, int nh, int L,
-    int Tdim, int Q, int C, int MT, int ntiles) {
-  constexpr int EPL = Vec16<T>::N;  // operand elements per lane and MFMA group
-  constexpr int KG = 2 * EPL;       // k extent of one MFMA group
-  constexpr int ROW = kBN + EPL;    // LDS row pitch in elements (16 bytes of padding)
-  __shared__ __attribute__((aligned(16))) T xs[kBM * ROW];
-  __shared__ float cs_s[EMA_MAX_CHUNK_DEV];
-
-  const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63;
-  const int l32 = lane & 31, half = lane >> 5;
-
-  int64_t blk = blockIdx.x;
-  const int tile = (int)(blk % ntiles);
-  blk /= ntiles;
-  const int mt = (int)(blk % MT);
-  const int64_t chunk_id = blk / MT;
-  const int64_t n = chunk_id / C;
-  const int c = (int)(chunk_id - n * C);
-  const int64_t b = n / nh;
-  const int h = (int)(n - b * nh);
-  const int limit = min(Q, L - c * Q);
-  const int mt_base = mt * kBM;
-  const int col0 = tile * kBN;
-
-  const float* csp = cs + chunk_id * Q;
-  const int q_pad = (Q + kBM - 1) / kBM * kBM;
-  for (int i = tid; i < q_pad; i += 256) cs_s[i] = i < Q ? csp[i] : 0.f;
-  __syncthreads();
-  const float cs_last = cs_s[Q - 1];
-
-  const int m_lane = mt_base + wave * 32 + l32;  // row of this lane's decay-matrix slice
-  const float cs_m = cs_s[min(m_lane, q_pad - 1)];
-
-  // accumulators start from the carried-state term
-  floatx16 acc[kBN / 32];
-  const float* vp = vec + chunk_id * Tdim;
-#pragma unroll
-  for (int db = 0; db < kBN / 32; ++db) {
-    const int col = col0 + db * 32 + l32;
-    const float pv = col < Tdim ? vp[col] : 0.f;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int row = mt_base + wave * 32 + acc_row(v, lane);
-      const float a = cs_s[min(row, q_pad - 1)];
-      const float sc = REVERSE ? __expf(fminf(cs_last - a, 0.f)) : __expf(fminf(a, 0.f));
-      acc[db][v] = sc * pv;
-    }
-  }
-
-  const int k_lo = REVERSE ? mt_base : 0;
-  const int k_hi = REVERSE ? limit : min(mt_base + kBM, limit);
-  const int wave_lo = mt_base + wave * 32;       // lowest row of this wave
-  const int wave_hi = wave_lo + 32;              // one past its highest row
-  const T* ip = in + b * si.sb + h * si.sh + (int64_t)c * Q * si.sl;
-
-  constexpr int VPR = kBN / EPL;        // 16-byte vectors per LDS row
-  constexpr int RPP = 256 / VPR;        // rows filled per pass
-  for (int kt0 = k_lo; kt0 < k_hi; kt0 += kBM) {
-    __syncthreads();
-    {
-      const int vcol = (tid % VPR) * EPL;
-      for (int r = tid / VPR; r < kBM; r += RPP) {
-        const int k = kt0 + r;
-        Vec16<T> v;
-        if (k < limit && col0 + vcol < Tdim) v = load16(ip + (int64_t)k * si.sl + col0 + vcol);
-        else v.zero();
-        store16(&xs[r * ROW + vcol], v);
-      }
-    }
-    __syncthreads();
-    const int kg_lo = REVERSE ? max(0, (wave_lo - kt0) / KG * KG) : 0;
-    const int kg_hi = REVERSE ? min(kBM, k_hi - kt0) : min(kBM, min(wave_hi, k_hi) - kt0);
-    for (int kg = kg_lo; kg < kg_hi; kg += KG) {
-      const int kl = kg + EPL * half;  // first k of this lane inside the tile
-      float m[EPL];
-#pragma unroll
-      for (int e = 0; e < EPL; ++e) {
-        const int k = kt0 + kl + e;
-        const float d = REVERSE ? cs_s[k] - cs_m : cs_m - cs_s[k];
-        const bool keep = REVERSE ? (k >= m_lane) : (k <= m_lane);
-        m[e] = keep ? __expf(fminf(d, 0.f)) : 0.f;
-      }
-      if constexpr (sizeof(T) == 2) {
-        // bf16: the decay factors go in as hi + lo (two bf16 terms, ~16 significant bits)
-        // so that the product with the exact bf16 inputs keeps f32-grade accuracy.
-        Vec16<T> a_hi, a_lo;
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) {
-          a_hi.set(e, m[e]);
-          a_lo.set(e, m[e] - a_hi.get(e));
-        }
-#pragma unroll
-        for (int db = 0; db < kBN / 32; ++db) {
-          const Vec16<T> bfrag = lds_read_kmajor(xs, ROW, kg, db * 32, lane);
-          mma_group(a_hi, bfrag, acc[db]);
-          mma_group(a_lo, bfrag, acc[db]);
-        }
-      } else {
-        Vec16<T> a;
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) a.set(e, m[e]);
-#pragma unroll
-        for (int db = 0; db < kBN / 32; ++db) {
-          Vec16<T> bfrag;
-#pragma unroll
-          for (int e = 0; e < EPL; ++e) bfrag.put(e, xs[(kl + e) * ROW + db * 32 + l32]);
-          mma_group(a, bfrag, acc[db]);
-        }
-      }
-    }
-  }
-
-  T* op = out + b * so.sb + h * so.sh + (int64_t)c * Q * so.sl;
-#pragma unroll
-  for (int db = 0; db < kBN / 32; ++db) {
-    const int col = col0 + db * 32 + l32;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int row = mt_base + wave * 32 + acc_row(v, lane);
-      if (row < limit && col < Tdim) op[(int64_t)row * so.sl + col] = (T)acc[db][v];
-    }
-  }
-}
 
 // ------------------------------------------------------------------------------------
 // B6, first part.  For the chunk (n, c) and the row tile mt (rows m of dy), for every

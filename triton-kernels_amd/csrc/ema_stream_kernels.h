@@ -153,10 +153,11 @@ __global__ __launch_bounds__(256) void state_passing_fwd_kernel(
 }
 
 // ------------------------------------------------------------------------------------
-// B2: reverse inter-chunk recurrence.  One thread per (n, t).  Besides g, every wave
-// writes its partial of <prev[n,c], g[n,c]> to part[(n*C + c) * nw + wave_of_t]; the
+// B2: reverse inter-chunk recurrence.  One thread per (n, t).  With DOTS, besides g, every
+// wave writes its partial of <prev[n,c], g[n,c]> to part[(n*C + c) * nw + wave_of_t]; the
 // partials are summed (and scaled by exp(cs_last)) by state_passing_bwd_finish_kernel.
 // ------------------------------------------------------------------------------------
+template <bool DOTS>
 __global__ __launch_bounds__(256) void state_passing_bwd_kernel(
     const float* __restrict__ prev, const float* __restrict__ cs_last, int64_t cl_sn,
     int64_t cl_sc, const float* __restrict__ ds, float* __restrict__ g,
@@ -178,7 +179,7 @@ __global__ __launch_bounds__(256) void state_passing_bwd_kernel(
       const int c = c1 - u;
       const bool in = c >= 0;
       d[u] = (in && ok) ? ds[base + (int64_t)c * Tdim] : 0.f;
-      p[u] = (in && ok) ? prev[base + (int64_t)c * Tdim] : 0.f;
+      p[u] = (DOTS && in && ok) ? prev[base + (int64_t)c * Tdim] : 0.f;
       a[u] = in ? cl[(int64_t)c * cl_sc] : 0.f;
     }
 #pragma unroll
@@ -186,8 +187,10 @@ __global__ __launch_bounds__(256) void state_passing_bwd_kernel(
       const int c = c1 - u;
       if (c >= 0) {  // uniform across the wave
         if (ok) g[base + (int64_t)c * Tdim] = cur;
-        const float dot = wave_sum(p[u] * cur);
-        if (lane == 0 && wave_id < nw) part[(n * C + c) * (int64_t)nw + wave_id] = dot;
+        if (DOTS) {
+          const float dot = wave_sum(p[u] * cur);
+          if (lane == 0 && wave_id < nw) part[(n * C + c) * (int64_t)nw + wave_id] = dot;
+        }
         cur = fmaf(__expf(a[u]), cur, d[u]);
       }
     }
