@@ -40,6 +40,9 @@ def parse():
     ap.add_argument("--sets", type=int, default=3, help="input sets the steps rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel timing pass")
+    ap.add_argument("--stage", default=None,
+                    help="time only this stage (a name from the `kernels` table, or fwd, bwd, copy) "
+                    "and print a short JSON line; used for counter collection")
     return ap.parse_args()
 
 
@@ -61,6 +64,7 @@ def algorithmic_bytes(N, L, T, Q, esize):
         "bwd_db": x + st + 2 * a,
         "bwd_dc": x + st + 2 * a,
         "bwd_da_intra": 2 * x + 2 * a,
+        "bwd_fused_dx_dA": 3 * x + 2 * a + 2 * st,
         "fwd": 2 * x + a,
         "bwd": 3 * x + 2 * a,
     }
@@ -147,6 +151,16 @@ def main():
         x, A, dy = sets[i % len(sets)]
         _ema_chunk_scan_combined_bwd(dy, x, A, Q)
 
+    if args.stage:
+        stages = make_stages(sets, Q, torch)
+        stages.update({"fwd": fwd_only, "bwd": bwd_only, "step": step})
+        fn = stages[args.stage]
+        for i in range(args.warmup):
+            fn(i)
+        ms = time_region(fn, args.steps, torch)
+        print(json.dumps({"stage": args.stage, "ms": ms, "steps": args.steps}))
+        return
+
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -191,7 +205,10 @@ def main():
         "kernels": kernels,
     }
     if kernels:
-        dom = max(kernels, key=lambda k: kernels[k]["ms"])
+        # kernels the timed step actually launches (the other rows are the per-stage launchers)
+        on_path = ("cumsum", "chunk_state", "state_passing_fwd", "chunk_scan", "bwd_dstates",
+                   "bwd_fused_dx_dA")
+        dom = max(on_path, key=lambda k: kernels[k]["ms"])
         out["roofline"] = {
             "kernel": dom,
             "bound": "hbm",
@@ -206,9 +223,10 @@ def main():
     print(json.dumps(out))
 
 
-def time_kernels(sets, Q, iters, ab, torch):
-    """Per-stage timing through the per-stage launchers (one kernel each, plus at most one
-    tiny finishing kernel), HIP events on the launch stream."""
+def make_stages(sets, Q, torch):
+    """name -> callable(i) launching one stage through its per-stage launcher (one kernel each,
+    plus at most one tiny finishing kernel) on input set i; `copy` is a plain device copy of
+    one x-sized tensor, the practical ceiling of a read-once write-once kernel."""
     from kernels.ema_kernels.ema_cumsum import ema_chunk_cumsum_fwd
     from kernels.ema_kernels.ema_scan_fwd import _ema_scan_fwd
     from kernels.ema_kernels.ema_state_fwd import _ema_chunk_state_fwd
@@ -216,6 +234,7 @@ def time_kernels(sets, Q, iters, ab, torch):
     from kernels.ema_kernels_bwd.ema_chunk_scan_bwd_dc import _ema_chunk_scan_bwd_dC
     from kernels.ema_kernels_bwd.ema_chunk_scan_chunk_state_bwd_dx import _chunk_scan_chunk_state_bwd_dx
     from kernels.ema_kernels_bwd.ema_chunk_state_bwd_db import _ema_chunk_state_bwd_db
+    from kernels.ema_kernels_bwd.ema_combined_bwd import _ema_bwd_dx_dA_fused
     from kernels.ema_kernels_bwd.ema_scan_bwd import _ema_chunk_scan_bwd_dstates
     from kernels.ema_kernels_bwd.ema_scan_da import _ema_chunk_scan_bwd_ddAcs_stable
     from kernels.ema_kernels_bwd.ema_state_passing_bwd_dstates import _ema_state_passing_bwd
@@ -227,7 +246,14 @@ def time_kernels(sets, Q, iters, ab, torch):
         prev, _ = _ema_state_passing_fwd(states, cs[..., -1], out_dtype=torch.float32)
         ds = _ema_chunk_scan_bwd_dstates(cs, dy)
         g, _, _ = _ema_state_passing_bwd(prev, cs[..., -1], ds)
-        inter.append((cs, states, prev, ds, g))
+        if Q == 128:
+            fused_in = (cs, prev, g)
+        else:  # the fused backward kernel always works on 128-row chunks
+            cs1 = ema_chunk_cumsum_fwd(A, 128)
+            prev1, _ = _ema_state_passing_fwd(_ema_chunk_state_fwd(x, cs1), cs1[..., -1], out_dtype=torch.float32)
+            g1, _, _ = _ema_state_passing_bwd(prev1, cs1[..., -1], _ema_chunk_scan_bwd_dstates(cs1, dy))
+            fused_in = (cs1, prev1, g1)
+        inter.append((cs, states, prev, ds, g, fused_in))
 
     def pick(i):
         k = i % len(sets)
@@ -244,7 +270,19 @@ def time_kernels(sets, Q, iters, ab, torch):
         "bwd_db": lambda i: _ema_chunk_state_bwd_db(pick(i)[0], pick(i)[3], pick(i)[7]),
         "bwd_dc": lambda i: _ema_chunk_scan_bwd_dC(pick(i)[5], pick(i)[3], pick(i)[2]),
         "bwd_da_intra": lambda i: _ema_chunk_scan_bwd_ddAcs_stable(pick(i)[0], pick(i)[3], pick(i)[2]),
+        "bwd_fused_dx_dA": lambda i: _ema_bwd_dx_dA_fused(
+            pick(i)[0], pick(i)[8][0], pick(i)[2], pick(i)[8][1], pick(i)[8][2]),
     }
+    outs = [torch.empty_like(s[0]) for s in sets]
+    stages["copy"] = lambda i: outs[i % len(sets)].copy_(sets[i % len(sets)][0])
+    return stages
+
+
+def time_kernels(sets, Q, iters, ab, torch):
+    """Per-stage timing with HIP events on the launch stream."""
+    stages = make_stages(sets, Q, torch)
+    x = sets[0][0]
+    ab = dict(ab, copy=2 * x.numel() * x.element_size())
     res = {}
     for name, fn in stages.items():
         for i in range(3):
@@ -252,10 +290,9 @@ def time_kernels(sets, Q, iters, ab, torch):
         ms = time_region(fn, iters, torch)
         gbps = ab[name] / ms / 1e6
         res[name] = {"ms": ms, "GBps": gbps, "hbm_frac": gbps / HBM_PEAK_GBS, "bytes": ab[name]}
-    x = sets[0][0]
     N, L, T = x.shape[0] * x.shape[2], x.shape[1], x.shape[3]
     flops = 2.0 * Q * L * T * N
-    for name in ("chunk_scan", "bwd_dx", "bwd_da_intra"):
+    for name in ("chunk_scan", "bwd_dx", "bwd_da_intra"):  # dense-equivalent count, Q*Q per chunk
         tf = flops / res[name]["ms"] / 1e9
         res[name]["dense_TFLOPs"] = tf
         res[name]["mfma_frac_dense"] = tf / MFMA_BF16_PEAK_TFLOPS

@@ -86,17 +86,23 @@ int ema_scan_fwd(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dt
                  int64_t y_sh, int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
                  int64_t chunk, void* stream);
 
-/* Bytes of workspace ema_fwd needs (the chunk-local states). */
+/* Bytes of workspace ema_fwd needs. */
 size_t ema_fwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
                                int64_t chunk);
 
-/* F1..F4 in sequence.  Outputs y, cs (N,C,Q), prev (N,C,T), final (N,T).
+/* Whole forward.  Outputs y, cs (N,C,Q), prev (N,C,T) (state entering each chunk) and
+ * final (N,T).  When chunk is a multiple of 128 x is read ONCE: the scan runs on 128-row
+ * chunks and the inter-chunk state is handed from tile to tile inside the kernel (chained
+ * scan with look-back) instead of by separate F2 / F3 passes; prev128, if not NULL,
+ * receives the states entering each 128-row chunk, (N, ceil(seqlen/128), T), which
+ * ema_bwd accepts to skip their recomputation.  For other chunk sizes F1..F4 run in
+ * sequence and prev128 must be NULL.
  * Replaces _ema_matmul_scan_combined_fwd, kernels/ema_kernels/ema_combined_fwd.py:12-45. */
 int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void* x,
             int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb,
             int64_t y_sl, int64_t y_sh, float* cs, float* prev, float* final_state,
-            void* workspace, size_t workspace_bytes, int64_t batch, int64_t nheads,
-            int64_t seqlen, int64_t dim, int64_t chunk, void* stream);
+            float* prev128, void* workspace, size_t workspace_bytes, int64_t batch,
+            int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk, void* stream);
 
 /* --------------------------------------------------------------- backward stages ---- */
 
@@ -162,21 +168,48 @@ int ema_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t 
                              size_t workspace_bytes, int64_t batch, int64_t nheads,
                              int64_t seqlen, int64_t dim, int64_t chunk, void* stream);
 
+/* Bytes of workspace ema_bwd_dx_dA_fused needs (per-column-tile partials of ddA). */
+size_t ema_bwd_dx_dA_fused_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen,
+                                           int64_t dim);
+
+/* B3..B6 and their sum in ONE pass over x and dy, for a chunk size of exactly 128
+ * (cs, prev, g are (N, C, 128) / (N, C, T) with C = ceil(seqlen / 128)):
+ *   dx[m]  as in B3;
+ *   ddA[n,c,m] = exp(A[m]) * <dx[m], y[m-1]>  with y the forward output (y[-1] = prev),
+ * which equals ddA_intra + ddA_next + reverse-cumsum(ddA_prev, + ddA_chunk at the last
+ * slot): dx[m] is the gradient of the scan state at row m and y[m-1] is the state that
+ * exp(A[m]) multiplies.  When y is not NULL the forward output is written there too.
+ * Replaces the four launchers _chunk_scan_chunk_state_bwd_dx, _ema_chunk_state_bwd_db,
+ * _ema_chunk_scan_bwd_dC, _ema_chunk_scan_bwd_ddAcs_stable and the torch glue around them,
+ * kernels/ema_kernels_bwd/ema_combined_bwd.py:70-79. */
+int ema_bwd_dx_dA_fused(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, const void* dy,
+                        int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, int dtype, const float* cs,
+                        const float* prev, const float* g, void* dx, int64_t dx_sb, int64_t dx_sl,
+                        int64_t dx_sh, float* ddA, void* y, int64_t y_sb, int64_t y_sl,
+                        int64_t y_sh, void* workspace, size_t workspace_bytes, int64_t batch,
+                        int64_t nheads, int64_t seqlen, int64_t dim, void* stream);
+
 /* Bytes of workspace ema_bwd needs (cs, states, prev, ds, g and the partial sums). */
 size_t ema_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
                                int64_t chunk);
 
-/* Whole backward: recomputes F1..F3, then B1..B6 and their sum.  Outputs dx (layout of x)
- * and ddA (N,C,Q) float32 with ddA[n,c,q] = dL/dA[n, c*Q+q]; when y is not NULL the
- * forward output is recomputed into it (the reference's recompute_output=True).
+/* Whole backward.  The gradients do not depend on how the sequence is chunked, so the
+ * work is done on 128-row chunks in one pass over x and dy: dx, the recomputed forward
+ * state and ddA[m] = exp(A[m]) * <dx[m], y[m-1]> per tile, with the reverse inter-chunk
+ * state handed from tile to tile inside the kernel (chained scan, last chunk first).
+ * `chunk` only fixes the layout of the result.  prev128 (may be NULL) is the output of the
+ * same name of ema_fwd; without it the states entering each chunk are recomputed with one
+ * more pass over x (F1..F3).  Outputs dx (layout of x) and ddA (N,C,Q) float32 with
+ * ddA[n,c,q] = dL/dA[n, c*Q+q] (0 in the slots past seqlen); when y is not NULL the forward
+ * output is recomputed into it (the reference's recompute_output=True).
  * Replaces _ema_chunk_scan_combined_bwd,
  * kernels/ema_kernels_bwd/ema_combined_bwd.py:13-83. */
 int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const void* x,
             int64_t x_sb, int64_t x_sl, int64_t x_sh, const float* A, int64_t a_sb,
-            int64_t a_sl, int64_t a_sh, int dtype, void* dx, int64_t dx_sb, int64_t dx_sl,
-            int64_t dx_sh, float* ddA, void* y, int64_t y_sb, int64_t y_sl, int64_t y_sh,
-            void* workspace, size_t workspace_bytes, int64_t batch, int64_t nheads,
-            int64_t seqlen, int64_t dim, int64_t chunk, void* stream);
+            int64_t a_sl, int64_t a_sh, const float* prev128, int dtype, void* dx,
+            int64_t dx_sb, int64_t dx_sl, int64_t dx_sh, float* ddA, void* y, int64_t y_sb,
+            int64_t y_sl, int64_t y_sh, void* workspace, size_t workspace_bytes, int64_t batch,
+            int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk, void* stream);
 
 #ifdef __cplusplus
 }

@@ -39,7 +39,8 @@ def test_status_strings():
 def test_workspace_sizes():
     handle = _lib.lib()
     # config 2: N=32, C=32, T=1024, Q=128
-    assert handle.ema_fwd_workspace_bytes(16, 2, 4096, 1024, 128) == 32 * 32 * 1024 * 4
+    assert handle.ema_fwd_workspace_bytes(16, 2, 4096, 1024, 64) == 32 * 64 * 1024 * 4
+    assert handle.ema_fwd_workspace_bytes(16, 2, 4096, 1024, 128) > 32 * 32 * 1024 * 8
     assert handle.ema_state_passing_bwd_workspace_bytes(32, 32, 1024) == 32 * 32 * 16 * 4
     assert handle.ema_chunk_scan_bwd_ddAcs_workspace_bytes(16, 2, 4096, 128) == 2 * 32 * 32 * 128 * 4
     assert handle.ema_bwd_workspace_bytes(16, 2, 4096, 1024, 128) > 4 * 32 * 32 * 1024 * 4
@@ -67,7 +68,7 @@ def test_validation_happens_before_any_launch():
     # workspace too small
     assert (
         handle.ema_fwd(fake, 8, 1, 0, fake, 64, 8, 0, _lib.EMA_F32, fake, 64, 8, 0, fake, fake, fake,
-                       fake, 16, 1, 1, 8, 8, 4, None)
+                       None, fake, 16, 1, 1, 8, 8, 4, None)
         == -2
     )
 

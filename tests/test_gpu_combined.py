@@ -91,6 +91,26 @@ def test_staged_backward_composition(N, L, T, Q, dtype, device):
     assert float(ddA1.reshape(N, -1)[:, L:].abs().sum()) == 0.0
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("N,L,T", [(2, 1024, 256), (2, 300, 64), (1, 128, 1024)])
+def test_fused_dx_dA_stage(N, L, T, dtype, device):
+    """The fused backward launcher on the oracle's chunk-128 intermediates."""
+    from kernels.ema_kernels_bwd.ema_combined_bwd import _ema_bwd_dx_dA_fused
+    from parity_util import oracle_intermediates
+
+    announce(f"fused dx/dA stage N{N} L{L} T{T} {dtype}")
+    A, X, dy = flat_case(N, L, T, seed=500 + L, dtype=dtype)
+    it = oracle_intermediates(A, X, dy, 128)
+    dx, ddA, y = _ema_bwd_dx_dA_fused(
+        X.to(device), it["cs"].to(device), dy.to(device), it["prev"].to(device), it["g"].to(device),
+        recompute_output=True,
+    )
+    dx_ref, dA_ref = O.ema_loop_bwd(dy.float(), X.float(), A)
+    check_close("dx", dx, dx_ref, dtype)
+    check_close("dA", ddA.reshape(N, -1)[:, :L], dA_ref, dtype)
+    check_close("y", y, O.ema_loop(X.float(), A), dtype)
+
+
 def _headed_reference(x, A, dy):
     b, L, nh, d = x.shape
     xf, Af = O.to_flat(x.float(), A)

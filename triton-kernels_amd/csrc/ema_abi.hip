@@ -8,6 +8,7 @@
 #include "ema_gemm_kernels.h"
 #include "ema_stream_kernels.h"
 #include "ema_walk_kernels.h"
+#include "ema_chain_kernels.h"
 
 using namespace ema;
 
@@ -223,13 +224,8 @@ size_t da_part_floats(const Dims& d) {
   return (size_t)(d.N * d.C * MT * d.Q);
 }
 
-// Workspace carving for ema_bwd.  The backward chunks the sequence by 128 internally,
-// whatever the chunk size of the interface: di describes that chunking.
-struct BwdWs {
-  float *cs, *states, *prev, *ds, *g, *part;
-  size_t bytes;
-};
-
+// The backward chunks the sequence by 128 internally, whatever the chunk size of the
+// interface: internal_dims describes that chunking.
 Dims internal_dims(const Dims& d) {
   Dims di = d;
   di.Q = kTileRows;
@@ -242,24 +238,111 @@ int bwd_col_tiles(const Dims& d, int dtype) {
   return (int)((d.T + bn - 1) / bn);
 }
 
-BwdWs carve_bwd(void* base, const Dims& di, int dtype) {
-  BwdWs w;
-  size_t off = 0;
-  char* p = static_cast<char*>(base);
-  auto take = [&](size_t floats) {
-    float* r = reinterpret_cast<float*>(p + off);
-    off += align_up(floats * sizeof(float), 256);
-    return r;
-  };
-  const size_t ncq = (size_t)(di.N * di.C * di.Q), nct = (size_t)(di.N * di.C * di.T);
-  w.cs = take(ncq);
-  w.states = take(nct);
-  w.prev = take(nct);
-  w.ds = take(nct);
-  w.g = take(nct);
-  w.part = take(ncq * (size_t)bwd_col_tiles(di, dtype));
-  w.bytes = off;
+// ---------------------------------------------------------------- chained single-pass kernels
+
+// Workgroups of a persistent kernel that can be resident at once on the current device.
+template <typename K>
+int resident_blocks(K kernel, int smem) {
+  int dev = 0, ncu = 0, per_cu = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  if (hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) ncu = 256;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel), 256,
+                                                   smem) != hipSuccess || per_cu < 1)
+    per_cu = 1;
+  return ncu * per_cu;
+}
+
+inline int64_t padded_dim(int64_t T) { return (T + 127) / 128 * 128; }
+
+// status words + counters of one chained kernel
+struct ChainWs {
+  u64* status;
+  unsigned* counters;
+};
+inline size_t chain_ws_bytes(const Dims& di) {
+  return align_up((size_t)(di.N * di.C * padded_dim(di.T)) * sizeof(u64), 256) + 256;
+}
+inline ChainWs chain_carve(void* base, const Dims& di) {
+  ChainWs w;
+  w.status = static_cast<u64*>(base);
+  w.counters = reinterpret_cast<unsigned*>(
+      static_cast<char*>(base) + align_up((size_t)(di.N * di.C * padded_dim(di.T)) * sizeof(u64), 256));
   return w;
+}
+
+int launch_chain_init(const ChainWs& w, int64_t words, hipStream_t st) {
+  const int64_t n16 = (words * (int64_t)sizeof(u64) + 15) / 16;
+  const int64_t threads = n16 > 4 ? n16 : 4;
+  hipLaunchKernelGGL(chain_init_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st,
+                     reinterpret_cast<uint4*>(w.status), n16, w.counters);
+  return launched();
+}
+
+template <typename T, int BN>
+int launch_fwd_chained_t(const void* x, SeqStrides sx, const float* cs128, void* y, SeqStrides sy,
+                         float* prev128, float* prev_coarse, int ratio, float* fin, const ChainWs& w,
+                         const Dims& di, hipStream_t st) {
+  const int ntiles = (int)((di.T + BN - 1) / BN);
+  const int64_t cols = di.N * ntiles, total = cols * di.C;
+  if (total > 0x7fffffff) return EMA_ERR_SHAPE;
+  EMA_TRY(launch_chain_init(w, total * BN, st));
+  const int smem = WalkCfg<T, BN>::smem_bytes(1);
+  auto kernel = fwd_chained_kernel<T, BN, true>;
+  EMA_TRY(allow_smem(kernel, smem));
+  const int64_t cap = resident_blocks(kernel, smem);
+  const unsigned grid = (unsigned)(total < cap ? total : cap);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), smem, st, (const T*)x, sx, cs128, (T*)y, sy, prev128,
+                     prev_coarse, ratio, fin, w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T,
+                     (int)di.C, ntiles, (int)cols, (int)total);
+  return launched();
+}
+
+template <typename T, int BN>
+int launch_bwd_chained_t(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* cs128,
+                         const float* prev128, void* dx, SeqStrides sdx, void* y, SeqStrides sy,
+                         float* part, const ChainWs& w, const Dims& di, hipStream_t st) {
+  const int ntiles = (int)((di.T + BN - 1) / BN);
+  const int64_t cols = di.N * ntiles, total = cols * di.C;
+  if (total > 0x7fffffff) return EMA_ERR_SHAPE;
+  EMA_TRY(launch_chain_init(w, total * BN, st));
+  const int smem = WalkCfg<T, BN>::smem_bytes(2);
+  if (y) {
+    auto kernel = bwd_chained_kernel<T, BN, true>;
+    EMA_TRY(allow_smem(kernel, smem));
+    const int64_t cap = resident_blocks(kernel, smem);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(256), smem, st,
+                       (const T*)x, sx, (const T*)dy, sd, cs128, prev128, (T*)dx, sdx, (T*)y, sy, part,
+                       w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles,
+                       (int)cols, (int)total);
+  } else {
+    auto kernel = bwd_chained_kernel<T, BN, false>;
+    EMA_TRY(allow_smem(kernel, smem));
+    const int64_t cap = resident_blocks(kernel, smem);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(256), smem, st,
+                       (const T*)x, sx, (const T*)dy, sd, cs128, prev128, (T*)dx, sdx, (T*)nullptr, sy,
+                       part, w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles,
+                       (int)cols, (int)total);
+  }
+  return launched();
+}
+
+// dx, optionally the recomputed y, and the log-decay gradient in one pass over x and dy.
+// di is the 128-row chunking the kernel works on (cs, prev, g follow it); d fixes the
+// (N, C, Q) layout of ddA.
+int run_bwd_fused(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, int dtype,
+                  const float* cs, const float* prev, const float* g, void* dx, SeqStrides sdx,
+                  void* y, SeqStrides sy, float* ddA, float* part, const Dims& d, const Dims& di,
+                  hipStream_t st) {
+  if (dtype == EMA_BF16)
+    EMA_TRY((launch_bwd_fused_t<bf16_t, kWalkBnBf16>(x, sx, dy, sd, cs, prev, g, dx, sdx, y, sy, part,
+                                                     di, st)));
+  else
+    EMA_TRY((launch_bwd_fused_t<float, kWalkBnF32>(x, sx, dy, sd, cs, prev, g, dx, sdx, y, sy, part,
+                                                   di, st)));
+  const int64_t total = d.N * d.C * d.Q;
+  hipLaunchKernelGGL(dA_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, part,
+                     ddA, (int)d.L, (int)d.Q, (int)d.C, (int)di.C, bwd_col_tiles(di, dtype), total);
+  return launched();
 }
 
 }  // namespace
@@ -328,18 +411,41 @@ int ema_scan_fwd(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dt
                                   SeqStrides{y_sb, y_sl, y_sh}, d, as_stream(stream));
 }
 
+// Workspace of the single-pass forward (chunk size a multiple of 128).
+struct FwdWs {
+  float *cs128, *prev128;
+  ChainWs chain;
+  size_t bytes;
+};
+static FwdWs carve_fwd(void* base, const Dims& di) {
+  FwdWs w;
+  size_t off = 0;
+  char* p = static_cast<char*>(base);
+  w.cs128 = reinterpret_cast<float*>(p + off);
+  off += align_up((size_t)(di.N * di.C * di.Q) * sizeof(float), 256);
+  w.prev128 = reinterpret_cast<float*>(p + off);
+  off += align_up((size_t)(di.N * di.C * di.T) * sizeof(float), 256);
+  w.chain = chain_carve(p + off, di);
+  off += chain_ws_bytes(di);
+  w.bytes = off;
+  return w;
+}
+
 size_t ema_fwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
                                int64_t chunk) {
   Dims d;
   if (check_dims(batch, nheads, seqlen, dim, chunk, true, &d) != EMA_OK) return 0;
-  return align_up((size_t)(d.N * d.C * d.T) * sizeof(float), 256);
+  const size_t staged = align_up((size_t)(d.N * d.C * d.T) * sizeof(float), 256);
+  if (chunk % kTileRows) return staged;
+  const size_t chained = carve_fwd(nullptr, internal_dims(d)).bytes;
+  return chained > staged ? chained : staged;
 }
 
 int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void* x, int64_t x_sb,
             int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb, int64_t y_sl,
-            int64_t y_sh, float* cs, float* prev, float* final_state, void* workspace,
-            size_t workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
-            int64_t chunk, void* stream) {
+            int64_t y_sh, float* cs, float* prev, float* final_state, float* prev128,
+            void* workspace, size_t workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen,
+            int64_t dim, int64_t chunk, void* stream) {
   Dims d;
   EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
   EMA_TRY(check_dtype(dtype));
@@ -350,9 +456,30 @@ int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void
   if (workspace_bytes < ema_fwd_workspace_bytes(batch, nheads, seqlen, dim, chunk))
     return EMA_ERR_SHAPE;
   hipStream_t st = as_stream(stream);
+  const SeqStrides sx{x_sb, x_sl, x_sh}, sy{y_sb, y_sl, y_sh}, sa{a_sb, a_sl, a_sh};
+  EMA_TRY(launch_cumsum(A, sa, cs, d, st));
+  if (chunk % kTileRows == 0) {
+    // Single pass over x: the scan is computed on 128-row chunks with the inter-chunk state
+    // handed over inside the kernel; the states at the caller's chunk boundaries are every
+    // (chunk/128)-th of them.
+    const Dims di = internal_dims(d);
+    const FwdWs w = carve_fwd(workspace, di);
+    const int ratio = (int)(chunk / kTileRows);
+    const float* cs128 = cs;
+    if (ratio != 1) {
+      EMA_TRY(launch_cumsum(A, sa, w.cs128, di, st));
+      cs128 = w.cs128;
+    }
+    float* p128 = prev128 ? prev128 : (ratio == 1 ? prev : w.prev128);
+    float* coarse = p128 == prev ? nullptr : prev;
+    if (dtype == EMA_BF16)
+      return launch_fwd_chained_t<bf16_t, kWalkBnBf16>(x, sx, cs128, y, sy, p128, coarse, ratio,
+                                                       final_state, w.chain, di, st);
+    return launch_fwd_chained_t<float, kWalkBnF32>(x, sx, cs128, y, sy, p128, coarse, ratio,
+                                                   final_state, w.chain, di, st);
+  }
+  if (prev128) return EMA_ERR_UNSUPPORTED;  // only produced when chunk is a multiple of 128
   float* states = static_cast<float*>(workspace);
-  const SeqStrides sx{x_sb, x_sl, x_sh}, sy{y_sb, y_sl, y_sh};
-  EMA_TRY(launch_cumsum(A, SeqStrides{a_sb, a_sl, a_sh}, cs, d, st));
   EMA_TRY(launch_chunk_reduce<0>(x, sx, dtype, cs, states, d, st));
   EMA_TRY(launch_state_passing_fwd(states, cs + (d.Q - 1), d.C * d.Q, d.Q, prev, final_state, d.N,
                                    d.C, d.T, st));
@@ -463,20 +590,45 @@ int ema_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t 
                    ddA_intra, part, rowsum, d, as_stream(stream));
 }
 
+// Workspace of ema_bwd.
+struct BwdWs {
+  float *cs, *states, *prev, *part;
+  ChainWs chain;
+  size_t bytes;
+};
+static BwdWs carve_bwd(void* base, const Dims& di) {
+  BwdWs w;
+  size_t off = 0;
+  char* p = static_cast<char*>(base);
+  auto take = [&](size_t floats) {
+    float* r = reinterpret_cast<float*>(p + off);
+    off += align_up(floats * sizeof(float), 256);
+    return r;
+  };
+  const size_t ncq = (size_t)(di.N * di.C * di.Q), nct = (size_t)(di.N * di.C * di.T);
+  w.cs = take(ncq);
+  w.states = take(nct);
+  w.prev = take(nct);
+  w.part = take(ncq * (size_t)bwd_col_tiles(di, EMA_F32));  // the wider of the two tilings
+  w.chain = chain_carve(p + off, di);
+  off += chain_ws_bytes(di);
+  w.bytes = off;
+  return w;
+}
+
 size_t ema_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
                                int64_t chunk) {
   Dims d;
   if (check_dims(batch, nheads, seqlen, dim, chunk, true, &d) != EMA_OK) return 0;
-  // sized for the wider of the two column tilings so that it does not depend on the dtype
-  return carve_bwd(nullptr, internal_dims(d), EMA_F32).bytes;
+  return carve_bwd(nullptr, internal_dims(d)).bytes;
 }
 
 int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const void* x,
             int64_t x_sb, int64_t x_sl, int64_t x_sh, const float* A, int64_t a_sb, int64_t a_sl,
-            int64_t a_sh, int dtype, void* dx, int64_t dx_sb, int64_t dx_sl, int64_t dx_sh,
-            float* ddA, void* y, int64_t y_sb, int64_t y_sl, int64_t y_sh, void* workspace,
-            size_t workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
-            int64_t chunk, void* stream) {
+            int64_t a_sh, const float* prev128, int dtype, void* dx, int64_t dx_sb, int64_t dx_sl,
+            int64_t dx_sh, float* ddA, void* y, int64_t y_sb, int64_t y_sl, int64_t y_sh,
+            void* workspace, size_t workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen,
+            int64_t dim, int64_t chunk, void* stream) {
   Dims d;
   EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
   EMA_TRY(check_dtype(dtype));
@@ -490,38 +642,65 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
     return EMA_ERR_SHAPE;
   hipStream_t st = as_stream(stream);
   // The gradients do not depend on how the sequence is chunked, so the backward always
-  // works on 128-row chunks (one tile of the fused kernel); `chunk` only fixes the
-  // (N, C, Q) layout in which ddA is returned.
+  // works on 128-row chunks (one tile of the kernel); `chunk` only fixes the (N, C, Q)
+  // layout in which ddA is returned.
   const Dims di = internal_dims(d);
-  const BwdWs w = carve_bwd(workspace, di, dtype);
+  const BwdWs w = carve_bwd(workspace, di);
   const SeqStrides sx{x_sb, x_sl, x_sh}, sd{dy_sb, dy_sl, dy_sh}, sdx{dx_sb, dx_sl, dx_sh};
   const SeqStrides sy{y_sb, y_sl, y_sh};
-  const float* cs_last = w.cs + (di.Q - 1);
-  const int64_t cl_sn = di.C * di.Q, cl_sc = di.Q;
 
-  // forward intermediates: cumsum, chunk states, states entering each chunk
   EMA_TRY(launch_cumsum(A, SeqStrides{a_sb, a_sl, a_sh}, w.cs, di, st));
-  EMA_TRY(launch_chunk_reduce<0>(x, sx, dtype, w.cs, w.states, di, st));
-  // the final state is not needed; ds is free until B1 runs, its first N*T floats take it
-  EMA_TRY(launch_state_passing_fwd(w.states, cs_last, cl_sn, cl_sc, w.prev, w.ds, di.N, di.C, di.T,
-                                   st));
-  // gradient of the states: B1, then the reverse recurrence B2 (without its <prev, g>
-  // products, which the fused kernel does not need)
-  EMA_TRY(launch_chunk_reduce<1>(dy, sd, dtype, w.cs, w.ds, di, st));
-  EMA_TRY(launch_state_passing_bwd(w.prev, cs_last, cl_sn, cl_sc, w.ds, w.g, nullptr, nullptr, di.N,
-                                   di.C, di.T, st));
-  // dx, the recomputed y and the per-column-tile partials of dA in one pass over x and dy
+  if (!prev128) {
+    // states entering each chunk, recomputed: chunk states, then the inter-chunk recurrence
+    // (its final state is not needed and lands in `part`, which is free until the main kernel)
+    EMA_TRY(launch_chunk_reduce<0>(x, sx, dtype, w.cs, w.states, di, st));
+    EMA_TRY(launch_state_passing_fwd(w.states, w.cs + (di.Q - 1), di.C * di.Q, di.Q, w.prev,
+                                     w.part, di.N, di.C, di.T, st));
+    prev128 = w.prev;
+  }
+  // dx, the recomputed y and the per-column-tile partials of dA in one pass over x and dy;
+  // the reverse inter-chunk state is handed over inside the kernel
   if (dtype == EMA_BF16)
-    EMA_TRY((launch_bwd_fused_t<bf16_t, kWalkBnBf16>(x, sx, dy, sd, w.cs, w.prev, w.g, dx, sdx, y, sy,
-                                                     w.part, di, st)));
+    EMA_TRY((launch_bwd_chained_t<bf16_t, kWalkBnBf16>(x, sx, dy, sd, w.cs, prev128, dx, sdx, y, sy,
+                                                       w.part, w.chain, di, st)));
   else
-    EMA_TRY((launch_bwd_fused_t<float, kWalkBnF32>(x, sx, dy, sd, w.cs, w.prev, w.g, dx, sdx, y, sy,
-                                                   w.part, di, st)));
+    EMA_TRY((launch_bwd_chained_t<float, kWalkBnF32>(x, sx, dy, sd, w.cs, prev128, dx, sdx, y, sy,
+                                                     w.part, w.chain, di, st)));
   const int64_t total = d.N * d.C * d.Q;
-  hipLaunchKernelGGL(dA_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
-                     w.part, ddA, (int)d.L, (int)d.Q, (int)d.C, (int)di.C, bwd_col_tiles(di, dtype),
-                     total);
+  hipLaunchKernelGGL(dA_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w.part,
+                     ddA, (int)d.L, (int)d.Q, (int)d.C, (int)di.C, bwd_col_tiles(di, dtype), total);
   return launched();
+}
+
+size_t ema_bwd_dx_dA_fused_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen,
+                                           int64_t dim) {
+  Dims d;
+  if (check_dims(batch, nheads, seqlen, dim, kTileRows, true, &d) != EMA_OK) return 0;
+  return align_up((size_t)(d.N * d.C * d.Q) * bwd_col_tiles(d, EMA_F32) * sizeof(float), 256);
+}
+
+int ema_bwd_dx_dA_fused(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, const void* dy,
+                        int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, int dtype, const float* cs,
+                        const float* prev, const float* g, void* dx, int64_t dx_sb, int64_t dx_sl,
+                        int64_t dx_sh, float* ddA, void* y, int64_t y_sb, int64_t y_sl, int64_t y_sh,
+                        void* workspace, size_t workspace_bytes, int64_t batch, int64_t nheads,
+                        int64_t seqlen, int64_t dim, void* stream) {
+  Dims d;
+  EMA_TRY(check_dims(batch, nheads, seqlen, dim, kTileRows, true, &d));
+  EMA_TRY(check_dtype(dtype));
+  EMA_TRY(check_seq(x, x_sb, x_sl, x_sh, dtype, dim));
+  EMA_TRY(check_seq(dy, dy_sb, dy_sl, dy_sh, dtype, dim));
+  EMA_TRY(check_seq(dx, dx_sb, dx_sl, dx_sh, dtype, dim));
+  if (y) EMA_TRY(check_seq(y, y_sb, y_sl, y_sh, dtype, dim));
+  if (!cs || !ddA) return EMA_ERR_NULL;
+  EMA_TRY(check_f32(prev));
+  EMA_TRY(check_f32(g));
+  EMA_TRY(check_f32(workspace));
+  if (workspace_bytes < ema_bwd_dx_dA_fused_workspace_bytes(batch, nheads, seqlen, dim))
+    return EMA_ERR_SHAPE;
+  return run_bwd_fused(x, SeqStrides{x_sb, x_sl, x_sh}, dy, SeqStrides{dy_sb, dy_sl, dy_sh}, dtype, cs,
+                       prev, g, dx, SeqStrides{dx_sb, dx_sl, dx_sh}, y, SeqStrides{y_sb, y_sl, y_sh},
+                       ddA, static_cast<float*>(workspace), d, d, as_stream(stream));
 }
 
 }  // extern "C"

@@ -29,7 +29,7 @@ _SIGNATURES = {
     "ema_state_passing_fwd": (c_int, [_P, _P, _I, _I, _P, _P, _I, _I, _I, _P]),
     "ema_scan_fwd": (c_int, _SEQ + [c_int, _P, _P] + _SEQ + [_I, _I, _I, _I, _I, _P]),
     "ema_fwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I]),
-    "ema_fwd": (c_int, _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _P]),
+    "ema_fwd": (c_int, _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _P]),
     "ema_chunk_scan_bwd_dstates": (c_int, _SEQ + [c_int, _P, _P, _I, _I, _I, _I, _I, _P]),
     "ema_state_passing_bwd_workspace_bytes": (c_size_t, [_I, _I, _I]),
     "ema_state_passing_bwd": (c_int, [_P, _P, _I, _I, _P, _P, _P, _P, c_size_t, _I, _I, _I, _P]),
@@ -38,8 +38,10 @@ _SIGNATURES = {
     "ema_chunk_scan_bwd_dc": (c_int, _SEQ + [c_int, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "ema_chunk_scan_bwd_ddAcs_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "ema_chunk_scan_bwd_ddAcs": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _P]),
+    "ema_bwd_dx_dA_fused_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
+    "ema_bwd_dx_dA_fused": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P] + _SEQ + [_P] + _SEQ + [_P, c_size_t, _I, _I, _I, _I, _P]),
     "ema_bwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I]),
-    "ema_bwd": (c_int, _SEQ + _SEQ + _SEQ + [c_int] + _SEQ + [_P] + _SEQ + [_P, c_size_t, _I, _I, _I, _I, _I, _P]),
+    "ema_bwd": (c_int, _SEQ + _SEQ + _SEQ + [_P, c_int] + _SEQ + [_P] + _SEQ + [_P, c_size_t, _I, _I, _I, _I, _I, _P]),
 }
 
 _lib = None

@@ -10,11 +10,14 @@ import torch
 from kernels import _lib
 
 
-def _ema_matmul_scan_combined_fwd(A_ema, X_ema, chunk_size, dtype=torch.float32):
+def _ema_matmul_scan_combined_fwd(A_ema, X_ema, chunk_size, dtype=torch.float32, return_prev128=False):
     """A_ema: (B, L) or (b, L, nh) float32 log-decay; X_ema: (B, L, T) or (b, L, nh, d).
 
     Returns (out, dA_cumsum (N, C, Q), states entering each chunk (N, C, T), final (N, T)).
-    `dtype` is the dtype of the returned chunk states (computed in float32)."""
+    `dtype` is the dtype of the returned chunk states (computed in float32).  With
+    return_prev128 a fifth value follows: the states entering each 128-row chunk, which the
+    backward accepts to skip their recomputation (None when chunk_size is not a multiple
+    of 128)."""
     dev = _lib.require_gpu(A_ema, X_ema)
     x, x_args, batch, nh, seqlen, token_dim = _lib.seq_view(X_ema)
     a_args, a_batch, a_nh, a_len = _lib.decay_view(A_ema)
@@ -26,6 +29,10 @@ def _ema_matmul_scan_combined_fwd(A_ema, X_ema, chunk_size, dtype=torch.float32)
     cs = torch.empty(N, nchunks, chunk_size, device=dev, dtype=torch.float32)
     prev = torch.empty(N, nchunks, token_dim, device=dev, dtype=torch.float32)
     final = torch.empty(N, token_dim, device=dev, dtype=torch.float32)
+    prev128 = None
+    if return_prev128 and chunk_size % 128 == 0:
+        prev128 = prev if chunk_size == 128 else torch.empty(
+            N, math.ceil(seqlen / 128), token_dim, device=dev, dtype=torch.float32)
     L = _lib.lib()
     ws_bytes = L.ema_fwd_workspace_bytes(batch, nh, seqlen, token_dim, chunk_size)
     assert ws_bytes > 0, "unsupported shape"
@@ -33,12 +40,14 @@ def _ema_matmul_scan_combined_fwd(A_ema, X_ema, chunk_size, dtype=torch.float32)
     with torch.cuda.device(dev):
         st = L.ema_fwd(
             *a_args, *x_args, _lib.dtype_code(x), *y_args, cs.data_ptr(), prev.data_ptr(),
-            final.data_ptr(), ws.data_ptr(), ws_bytes, batch, nh, seqlen, token_dim, chunk_size,
-            _lib.stream_ptr(dev),
+            final.data_ptr(), None if prev128 is None or prev128 is prev else prev128.data_ptr(),
+            ws.data_ptr(), ws_bytes, batch, nh, seqlen, token_dim, chunk_size, _lib.stream_ptr(dev),
         )
     _lib.check(st, "_ema_matmul_scan_combined_fwd")
     if dtype != torch.float32:
         prev = prev.to(dtype)
+    if return_prev128:
+        return out, cs, prev, final, prev128
     return out, cs, prev, final
 
 
@@ -55,10 +64,11 @@ def _unchunk_dA(ddA, A_like, seqlen):
 class EMAMatmulCombinedFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, A_ema, X_ema, chunk_size):
-        out, dA_cumsum, states, final_states = _ema_matmul_scan_combined_fwd(
-            A_ema, X_ema, chunk_size=chunk_size
+        out, dA_cumsum, states, final_states, prev128 = _ema_matmul_scan_combined_fwd(
+            A_ema, X_ema, chunk_size=chunk_size, return_prev128=True
         )
         ctx.save_for_backward(out, dA_cumsum, states, final_states, A_ema, X_ema)
+        ctx.prev128 = prev128  # a small float32 tensor the backward reuses; not an input or output
         ctx.chunk_size = chunk_size
         return out
 
@@ -67,7 +77,7 @@ class EMAMatmulCombinedFn(torch.autograd.Function):
         from kernels.ema_kernels_bwd.ema_combined_bwd import _ema_chunk_scan_combined_bwd
 
         out, dA_cumsum, states, final_states, A_ema, X_ema = ctx.saved_tensors
-        dx, ddA = _ema_chunk_scan_combined_bwd(dout, X_ema, A_ema, ctx.chunk_size)
+        dx, ddA = _ema_chunk_scan_combined_bwd(dout, X_ema, A_ema, ctx.chunk_size, prev128=ctx.prev128)
         dA = _unchunk_dA(ddA, A_ema, X_ema.shape[1])
         return dA, dx, None
 
