@@ -144,7 +144,7 @@ int launch_chunk_scan_t(const void* in, SeqStrides si, const float* cs, const fl
   const int ntiles = (int)((d.T + BN - 1) / BN);
   const int64_t grid = d.N * d.C * ntiles;
   if (grid > 0x7fffffff) return EMA_ERR_SHAPE;
-  const int smem = WalkCfg<T, BN>::smem_bytes(1);
+  const int smem = WalkCfg<T, BN>::smem_bytes(1, 1);
   auto kernel = chunk_scan_walk_kernel<T, BN, REVERSE>;
   EMA_TRY(allow_smem(kernel, smem));
   hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), smem, st, (const T*)in, si, cs, vec,
@@ -167,7 +167,7 @@ int launch_bwd_fused_t(const void* x, SeqStrides sx, const void* dy, SeqStrides 
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t grid = di.N * di.C * ntiles;
   if (grid > 0x7fffffff) return EMA_ERR_SHAPE;
-  const int smem = WalkCfg<T, BN>::smem_bytes(2);
+  const int smem = WalkCfg<T, BN>::smem_bytes(2, 2);
   if (y) {
     auto kernel = bwd_fused_kernel<T, BN, true>;
     EMA_TRY(allow_smem(kernel, smem));
@@ -286,7 +286,7 @@ int launch_fwd_chained_t(const void* x, SeqStrides sx, const float* cs128, void*
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
   EMA_TRY(launch_chain_init(w, total * BN, st));
-  const int smem = WalkCfg<T, BN>::smem_bytes(1);
+  const int smem = WalkCfg<T, BN>::smem_bytes(1, 1);
   auto kernel = fwd_chained_kernel<T, BN, true>;
   EMA_TRY(allow_smem(kernel, smem));
   const int64_t cap = resident_blocks(kernel, smem);
@@ -305,7 +305,7 @@ int launch_bwd_chained_t(const void* x, SeqStrides sx, const void* dy, SeqStride
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
   EMA_TRY(launch_chain_init(w, total * BN, st));
-  const int smem = WalkCfg<T, BN>::smem_bytes(2);
+  const int smem = WalkCfg<T, BN>::smem_bytes(2, 2);
   if (y) {
     auto kernel = bwd_chained_kernel<T, BN, true>;
     EMA_TRY(allow_smem(kernel, smem));
@@ -702,5 +702,12 @@ int ema_bwd_dx_dA_fused(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
                        prev, g, dx, SeqStrides{dx_sb, dx_sl, dx_sh}, y, SeqStrides{y_sb, y_sl, y_sh},
                        ddA, static_cast<float*>(workspace), d, d, as_stream(stream));
 }
+
+#ifdef EMA_TIMING
+// Development aid, only in builds with -DEMA_TIMING: installs the per-tile timestamp buffer.
+int ema_debug_set_timing(void* buf) {
+  return hipMemcpyToSymbol(HIP_SYMBOL(ema::g_ema_timing), &buf, sizeof(buf)) == hipSuccess ? 0 : -6;
+}
+#endif
 
 }  // extern "C"

@@ -26,6 +26,19 @@ namespace ema {
 
 typedef unsigned long long u64;
 
+#ifdef EMA_TIMING
+// Development aid: per-tile phase timestamps into a global buffer (never built into the library).
+__device__ long long* g_ema_timing = nullptr;
+#define EMA_STAMP(slot)                                                          \
+  do {                                                                           \
+    if (threadIdx.x == 0 && g_ema_timing) g_ema_timing[(int64_t)cur * 8 + (slot)] = wall_clock64(); \
+  } while (0)
+#else
+#define EMA_STAMP(slot) \
+  do {                  \
+  } while (0)
+#endif
+
 constexpr unsigned kFlagAggregate = 1u;
 constexpr unsigned kFlagPrefix = 2u;
 constexpr int kSpinLimit = 1 << 20;
@@ -61,23 +74,22 @@ __global__ __launch_bounds__(256) void chain_init_kernel(uint4* __restrict__ wor
 }
 
 struct ChainTile {
-  int c, ctile, limit, col0;
-  int64_t n, b, chunk_id, col_id;  // col_id = n * ntiles + ctile
-  int h;
+  int c, ctile, limit, col0, n, b, h, chunk_id, col_id;  // col_id = n * ntiles + ctile
 };
 
-// Ticket -> tile, chunk-major; REV runs the chunks from last to first.
+// Ticket -> tile, chunk-major; REV runs the chunks from last to first.  All quantities fit
+// 32 bits (the host checks N * C * ntiles < 2^31).
 template <bool REV, int BN>
 __device__ __forceinline__ ChainTile chain_decode(int ticket, int cols, int ntiles, int C, int nh,
                                                   int L) {
   ChainTile t;
-  const int cc = ticket / cols;
-  t.c = REV ? C - 1 - cc : cc;
-  t.col_id = ticket - cc * cols;
-  t.n = t.col_id / ntiles;
-  t.ctile = (int)(t.col_id - t.n * ntiles);
-  t.b = t.n / nh;
-  t.h = (int)(t.n - t.b * nh);
+  const unsigned cc = (unsigned)ticket / (unsigned)cols;
+  t.c = REV ? C - 1 - (int)cc : (int)cc;
+  t.col_id = ticket - (int)cc * cols;
+  t.n = (int)((unsigned)t.col_id / (unsigned)ntiles);
+  t.ctile = t.col_id - t.n * ntiles;
+  t.b = (int)((unsigned)t.n / (unsigned)nh);
+  t.h = t.n - t.b * nh;
   t.chunk_id = t.n * C + t.c;
   t.limit = min(kTileRows, L - t.c * kTileRows);
   t.col0 = t.ctile * BN;
@@ -89,7 +101,7 @@ __device__ __forceinline__ void chain_issue_loads(Vec16<T>* pre, const T* __rest
                                                   SeqStrides s, const ChainTile& t, int Tdim,
                                                   int tid) {
   using C = WalkCfg<T, BN>;
-  const T* g = base + t.b * s.sb + t.h * s.sh + (int64_t)t.c * kTileRows * s.sl;
+  const T* g = base + (int64_t)t.b * s.sb + (int64_t)t.h * s.sh + (int64_t)t.c * kTileRows * s.sl;
   const int vcol = (tid % C::VPR) * C::EPL;
   const bool cok = t.col0 + vcol < Tdim;
 #pragma unroll
@@ -159,7 +171,7 @@ __device__ __forceinline__ float chain_look(const u64* status, const float* __re
 // status: N*ntiles*C*BN words (zeroed); counters[0] ticket, counters[3] error word.
 // ------------------------------------------------------------------------------------
 template <typename T, int BN, bool WRITE_Y>
-__global__ __launch_bounds__(256) void fwd_chained_kernel(
+__global__ __launch_bounds__(256, 4) void fwd_chained_kernel(
     const T* __restrict__ x, SeqStrides sx, const float* __restrict__ cs, T* __restrict__ y,
     SeqStrides sy, float* __restrict__ prev, float* __restrict__ prev_coarse, int ratio,
     float* __restrict__ final_state, u64* __restrict__ status, unsigned* __restrict__ counters,
@@ -167,7 +179,7 @@ __global__ __launch_bounds__(256) void fwd_chained_kernel(
   using Cfg = WalkCfg<T, BN>;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* tile = reinterpret_cast<T*>(smem);
-  const WalkScratch s = walk_scratch<T, BN>(smem, 1);
+  const WalkScratch s = walk_scratch<T, BN, 1>(smem, 1);
   __shared__ int s_ticket[2];
 
   const int tid = threadIdx.x;
@@ -179,41 +191,41 @@ __global__ __launch_bounds__(256) void fwd_chained_kernel(
   int cur = s_ticket[0];
   int slot = 1;
   Vec16<T> pre[kTileRows / Cfg::RPP];
-  if (cur < total) {
-    const ChainTile t = chain_decode<false, BN>(cur, cols, ntiles, C, nh, L);
-    chain_issue_loads<T, BN>(pre, x, sx, t, Tdim, tid);
-  }
+  ChainTile t = chain_decode<false, BN>(cur < total ? cur : 0, cols, ntiles, C, nh, L);
+  if (cur < total) chain_issue_loads<T, BN>(pre, x, sx, t, Tdim, tid);
   while (cur < total) {
-    const ChainTile t = chain_decode<false, BN>(cur, cols, ntiles, C, nh, L);
+    EMA_STAMP(0);
     chain_commit_loads<T, BN>(tile, pre, tid);
-    walk_load_cs(s, cs + t.chunk_id * kTileRows, 0, kTileRows, tid);
+    walk_load_cs<true, false>(s, cs + (int64_t)t.chunk_id * kTileRows, 0, kTileRows, tid);
     if (tid == 0) s_ticket[slot] = (int)atomicAdd(counters, 1u);
     __syncthreads();
+    EMA_STAMP(1);
     const int nxt = s_ticket[slot];
     slot ^= 1;
-    if (nxt < total) {
-      const ChainTile tn = chain_decode<false, BN>(nxt, cols, ntiles, C, nh, L);
-      chain_issue_loads<T, BN>(pre, x, sx, tn, Tdim, tid);
-    }
+    const ChainTile tn = chain_decode<false, BN>(nxt < total ? nxt : 0, cols, ntiles, C, nh, L);
+    if (nxt < total) chain_issue_loads<T, BN>(pre, x, sx, tn, Tdim, tid);
     walk_block_state<T, BN>(tile, s.wf, s.sj, wave, lane);
     __syncthreads();
+    EMA_STAMP(2);
     if (tid < BN) {
       float loc, dec;
       chain_local_fwd<BN>(s, tid, &loc, &dec);
-      u64* st = status + t.col_id * (int64_t)C * BN;
+      u64* st = status + (int64_t)t.col_id * C * BN;
       chain_publish(st + (int64_t)t.c * BN + tid, kFlagAggregate, loc);
-      const float p_in = chain_look<false, BN>(st, cs + t.n * (int64_t)C * kTileRows, t.c, C, tid, err);
+      const float p_in = chain_look<false, BN>(st, cs + (int64_t)t.n * C * kTileRows, t.c, C, tid, err);
       const float p_out = fmaf(dec, p_in, loc);
       chain_publish(st + (int64_t)t.c * BN + tid, kFlagPrefix, p_out);
       if (t.col0 + tid < Tdim) {
-        prev[t.chunk_id * Tdim + t.col0 + tid] = p_in;
+        prev[(int64_t)t.chunk_id * Tdim + t.col0 + tid] = p_in;
         if (prev_coarse && t.c % ratio == 0)
-          prev_coarse[(t.n * ((C + ratio - 1) / ratio) + t.c / ratio) * (int64_t)Tdim + t.col0 + tid] = p_in;
-        if (t.c == C - 1) final_state[t.n * Tdim + t.col0 + tid] = p_out;
+          prev_coarse[((int64_t)t.n * ((C + ratio - 1) / ratio) + t.c / ratio) * Tdim + t.col0 + tid] = p_in;
+        if (t.c == C - 1) final_state[(int64_t)t.n * Tdim + t.col0 + tid] = p_out;
       }
       walk_chain_fwd<BN>(s, p_in, tid);
     }
+    EMA_STAMP(3);
     __syncthreads();
+    EMA_STAMP(4);
     if (WRITE_Y) {
       Vec16<T> hi[Cfg::NG], lo[Cfg::NG];
       walk_decay_frags<T, false>(s.csT, wave, lane, hi, lo);
@@ -224,11 +236,14 @@ __global__ __launch_bounds__(256) void fwd_chained_kernel(
         const floatx16 acc = walk_block_mma<T, BN>(tile, hi, lo, s.Pj + wave * BN, u, wave, db, lane);
         walk_pack_block<T, BN>(tile, acc, wave, db, lane);
       }
-      walk_store_rows<T, BN>(tile, y + t.b * sy.sb + t.h * sy.sh + (int64_t)t.c * kTileRows * sy.sl,
+      walk_store_rows<T, BN>(tile, y + (int64_t)t.b * sy.sb + (int64_t)t.h * sy.sh + (int64_t)t.c * kTileRows * sy.sl,
                              sy.sl, 0, t.limit, t.col0, Tdim, wave, lane);
     }
+    EMA_STAMP(5);
     __syncthreads();
+    EMA_STAMP(6);
     cur = nxt;
+    t = tn;
   }
 }
 
@@ -249,7 +264,7 @@ __global__ __launch_bounds__(256, 2) void bwd_chained_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* xt = reinterpret_cast<T*>(smem);
   T* dt = xt + Cfg::TILE;
-  const WalkScratch s = walk_scratch<T, BN>(smem, 2);
+  const WalkScratch s = walk_scratch<T, BN, 2>(smem, 2);
   __shared__ int s_ticket[2];
 
   const int tid = threadIdx.x;
@@ -263,43 +278,47 @@ __global__ __launch_bounds__(256, 2) void bwd_chained_kernel(
   int slot = 1;
   Vec16<T> pre_x[kTileRows / Cfg::RPP], pre_d[kTileRows / Cfg::RPP];
   float p_pre = 0.f;
+  ChainTile t = chain_decode<true, BN>(cur < total ? cur : 0, cols, ntiles, C, nh, L);
   if (cur < total) {
-    const ChainTile t = chain_decode<true, BN>(cur, cols, ntiles, C, nh, L);
     chain_issue_loads<T, BN>(pre_d, dy, sd, t, Tdim, tid);
     chain_issue_loads<T, BN>(pre_x, x, sx, t, Tdim, tid);
-    if (tid < BN && t.col0 + tid < Tdim) p_pre = prev[t.chunk_id * Tdim + t.col0 + tid];
+    if (tid < BN && t.col0 + tid < Tdim) p_pre = prev[(int64_t)t.chunk_id * Tdim + t.col0 + tid];
   }
   while (cur < total) {
-    const ChainTile t = chain_decode<true, BN>(cur, cols, ntiles, C, nh, L);
+    EMA_STAMP(0);
     chain_commit_loads<T, BN>(dt, pre_d, tid);
     chain_commit_loads<T, BN>(xt, pre_x, tid);
     const float p_in = p_pre;
-    walk_load_cs(s, cs + t.chunk_id * kTileRows, 0, kTileRows, tid);
+    walk_load_cs<true, true>(s, cs + (int64_t)t.chunk_id * kTileRows, 0, kTileRows, tid);
     if (tid == 0) s_ticket[slot] = (int)atomicAdd(counters + 1, 1u);
     __syncthreads();
+    EMA_STAMP(1);
     const int nxt = s_ticket[slot];
     slot ^= 1;
     p_pre = 0.f;
+    const ChainTile tn = chain_decode<true, BN>(nxt < total ? nxt : 0, cols, ntiles, C, nh, L);
     if (nxt < total) {
-      const ChainTile tn = chain_decode<true, BN>(nxt, cols, ntiles, C, nh, L);
       chain_issue_loads<T, BN>(pre_d, dy, sd, tn, Tdim, tid);
       chain_issue_loads<T, BN>(pre_x, x, sx, tn, Tdim, tid);
-      if (tid < BN && tn.col0 + tid < Tdim) p_pre = prev[tn.chunk_id * Tdim + tn.col0 + tid];
+      if (tid < BN && tn.col0 + tid < Tdim) p_pre = prev[(int64_t)tn.chunk_id * Tdim + tn.col0 + tid];
     }
     walk_block_state<T, BN>(dt, s.wr, s.rj, wave, lane);
     walk_block_state<T, BN>(xt, s.wf, s.sj, wave, lane);
     __syncthreads();
+    EMA_STAMP(2);
     if (tid < BN) {
       float loc, dec;
       chain_local_rev<BN>(s, tid, &loc, &dec);
-      u64* st = status + t.col_id * (int64_t)C * BN;
+      u64* st = status + (int64_t)t.col_id * C * BN;
       chain_publish(st + (int64_t)t.c * BN + tid, kFlagAggregate, loc);
-      const float h_in = chain_look<true, BN>(st, cs + t.n * (int64_t)C * kTileRows, t.c, C, tid, err);
+      const float h_in = chain_look<true, BN>(st, cs + (int64_t)t.n * C * kTileRows, t.c, C, tid, err);
       chain_publish(st + (int64_t)t.c * BN + tid, kFlagPrefix, fmaf(dec, h_in, loc));
       walk_chain_rev<BN>(s, h_in, tid);
       walk_chain_fwd<BN>(s, p_in, tid);
     }
+    EMA_STAMP(3);
     __syncthreads();
+    EMA_STAMP(4);
 
     const float cm = s.csT[32 * wave + l32 + 1];
     Vec16<T> fhi[Cfg::NG], flo[Cfg::NG], rhi[Cfg::NG], rlo[Cfg::NG];
@@ -326,16 +345,19 @@ __global__ __launch_bounds__(256, 2) void bwd_chained_kernel(
     dot += __shfl_xor(dot, 32);
     if (lane < 32) {
       const int m = 32 * wave + lane;
-      part[(t.chunk_id * ntiles + t.ctile) * (int64_t)kTileRows + m] =
+      part[((int64_t)t.chunk_id * ntiles + t.ctile) * kTileRows + m] =
           m < t.limit ? __expf(cm - s.csT[m]) * dot : 0.f;
     }
-    walk_store_rows<T, BN>(dt, dx + t.b * sdx.sb + t.h * sdx.sh + (int64_t)t.c * kTileRows * sdx.sl,
+    walk_store_rows<T, BN>(dt, dx + (int64_t)t.b * sdx.sb + (int64_t)t.h * sdx.sh + (int64_t)t.c * kTileRows * sdx.sl,
                            sdx.sl, 0, t.limit, t.col0, Tdim, wave, lane);
     if (WRITE_Y)
-      walk_store_rows<T, BN>(xt, y + t.b * sy.sb + t.h * sy.sh + (int64_t)t.c * kTileRows * sy.sl,
+      walk_store_rows<T, BN>(xt, y + (int64_t)t.b * sy.sb + (int64_t)t.h * sy.sh + (int64_t)t.c * kTileRows * sy.sl,
                              sy.sl, 0, t.limit, t.col0, Tdim, wave, lane);
+    EMA_STAMP(5);
     __syncthreads();
+    EMA_STAMP(6);
     cur = nxt;
+    t = tn;
   }
 }
 

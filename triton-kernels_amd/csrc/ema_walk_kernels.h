@@ -36,10 +36,12 @@ struct WalkCfg {
   static constexpr int VPR = BN / EPL;           // 16-byte vectors per row
   static constexpr int RPP = 256 / VPR;          // rows staged per pass of the workgroup
   static constexpr int TILE_BYTES = TILE * (int)sizeof(T);
-  // f32 scratch after the tiles: csT[132] wf[128] wr[128] sj[4*BN] rj[4*BN] Pj[5*BN] Hj[5*BN]
-  static constexpr int SCRATCH_FLOATS = 132 + 128 + 128 + 4 * BN + 4 * BN + 5 * BN + 5 * BN;
-  static constexpr int smem_bytes(int ntiles) {
-    return ntiles * TILE_BYTES + SCRATCH_FLOATS * (int)sizeof(float);
+  // f32 scratch after the tiles.  Kernels that scan in both directions (DIRS = 2) keep
+  // csT[132] wf[128] wr[128] sj[4*BN] rj[4*BN] Pj[5*BN] Hj[5*BN]; one-directional kernels
+  // (DIRS = 1) keep csT[132] w[128] s[4*BN] P[5*BN] and the two names of each pair alias.
+  static constexpr int scratch_floats(int dirs) { return 132 + dirs * (128 + 4 * BN + 5 * BN); }
+  static constexpr int smem_bytes(int ntiles, int dirs) {
+    return ntiles * TILE_BYTES + scratch_floats(dirs) * (int)sizeof(float);
   }
 };
 
@@ -47,17 +49,17 @@ struct WalkScratch {
   float *csT, *wf, *wr, *sj, *rj, *Pj, *Hj;
 };
 
-template <typename T, int BN>
+template <typename T, int BN, int DIRS>
 __device__ __forceinline__ WalkScratch walk_scratch(unsigned char* smem, int ntiles) {
   float* f = reinterpret_cast<float*>(smem + ntiles * WalkCfg<T, BN>::TILE_BYTES);
   WalkScratch s;
   s.csT = f;
   s.wf = f + 132;
-  s.wr = s.wf + 128;
+  s.wr = DIRS == 2 ? s.wf + 128 : s.wf;
   s.sj = s.wr + 128;
-  s.rj = s.sj + 4 * BN;
+  s.rj = DIRS == 2 ? s.sj + 4 * BN : s.sj;
   s.Pj = s.rj + 4 * BN;
-  s.Hj = s.Pj + 5 * BN;
+  s.Hj = DIRS == 2 ? s.Pj + 5 * BN : s.Pj;
   return s;
 }
 
@@ -87,6 +89,7 @@ __device__ __forceinline__ void walk_load_tile(T* tile, const T* __restrict__ g,
 // wf[t] = exp(cs[e_j] - cs[t]), wr[t] = exp(cs[t] - cs[e_{j-1}]) for row t of block j = t/32
 // (e_j = last row of block j).  Thread t < 128 reads what it needs straight from global
 // memory so that no barrier is needed between this and the tile load.
+template <bool FWD, bool REV>
 __device__ __forceinline__ void walk_load_cs(const WalkScratch& s, const float* __restrict__ csp,
                                              int tb, int Q, int tid) {
   auto at = [&](int q) { return q < 0 ? 0.f : csp[min(q, Q - 1)]; };
@@ -95,8 +98,8 @@ __device__ __forceinline__ void walk_load_cs(const WalkScratch& s, const float* 
     const float c_t = at(tb + tid);
     s.csT[tid + 1] = c_t;
     if (tid == 0) s.csT[0] = at(tb - 1);
-    s.wf[tid] = __expf(fminf(at(tb + 32 * j + 31) - c_t, 0.f));
-    s.wr[tid] = __expf(fminf(c_t - at(tb + 32 * j - 1), 0.f));
+    if (FWD) s.wf[tid] = __expf(fminf(at(tb + 32 * j + 31) - c_t, 0.f));
+    if (REV) s.wr[tid] = __expf(fminf(c_t - at(tb + 32 * j - 1), 0.f));
   }
 }
 
@@ -273,7 +276,7 @@ __global__ __launch_bounds__(256) void chunk_scan_walk_kernel(
   using Cfg = WalkCfg<T, BN>;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* tile = reinterpret_cast<T*>(smem);
-  const WalkScratch s = walk_scratch<T, BN>(smem, 1);
+  const WalkScratch s = walk_scratch<T, BN, 1>(smem, 1);
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
@@ -296,7 +299,7 @@ __global__ __launch_bounds__(256) void chunk_scan_walk_kernel(
   for (int it = 0; it < nrt; ++it) {
     const int tb = (REV ? nrt - 1 - it : it) * kTileRows;
     if (it) __syncthreads();
-    walk_load_cs(s, csp, tb, Q, tid);
+    walk_load_cs<!REV, REV>(s, csp, tb, Q, tid);
     walk_load_tile<T, BN>(tile, ip, si.sl, tb, limit, col0, Tdim, tid);
     __syncthreads();
     walk_block_state<T, BN>(tile, REV ? s.wr : s.wf, REV ? s.rj : s.sj, wave, lane);
@@ -350,7 +353,7 @@ __global__ __launch_bounds__(256) void bwd_fused_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* xt = reinterpret_cast<T*>(smem);
   T* dt = xt + Cfg::TILE;
-  const WalkScratch s = walk_scratch<T, BN>(smem, 2);
+  const WalkScratch s = walk_scratch<T, BN, 2>(smem, 2);
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
@@ -370,7 +373,7 @@ __global__ __launch_bounds__(256) void bwd_fused_kernel(
     p_in = prev[chunk_id * Tdim + col0 + tid];
     h_in = g[chunk_id * Tdim + col0 + tid];
   }
-  walk_load_cs(s, csp, 0, Q, tid);
+  walk_load_cs<true, true>(s, csp, 0, Q, tid);
   walk_load_tile<T, BN>(xt, x + b * sx.sb + h * sx.sh + (int64_t)c * Q * sx.sl, sx.sl, 0, limit, col0,
                         Tdim, tid);
   walk_load_tile<T, BN>(dt, dy + b * sd.sb + h * sd.sh + (int64_t)c * Q * sd.sl, sd.sl, 0, limit,
