@@ -135,8 +135,17 @@ int allow_smem(K kernel, int bytes) {
              : EMA_ERR_LAUNCH;
 }
 
-constexpr int kWalkBnBf16 = 128;  // column tile of the intra-chunk kernels, bf16
+constexpr int kWalkBnBf16 = 128;  // column tile of the per-stage intra-chunk kernels, bf16
 constexpr int kWalkBnF32 = 64;    // and f32 (both are 256 bytes per row)
+
+// Shape of the chained single-pass kernels: column tile, threads, minimum waves per SIMD the
+// register allocation must allow.
+struct ChainBf16 {
+  static constexpr int BN = 128, NT = 256, FWD_MINW = 3, BWD_MINW = 2;
+};
+struct ChainF32 {
+  static constexpr int BN = 64, NT = 512, FWD_MINW = 4, BWD_MINW = 2;
+};
 
 template <typename T, int BN, bool REVERSE>
 int launch_chunk_scan_t(const void* in, SeqStrides si, const float* cs, const float* vec, void* out,
@@ -242,12 +251,12 @@ int bwd_col_tiles(const Dims& d, int dtype) {
 
 // Workgroups of a persistent kernel that can be resident at once on the current device.
 template <typename K>
-int resident_blocks(K kernel, int smem) {
+int resident_blocks(K kernel, int threads, int smem) {
   int dev = 0, ncu = 0, per_cu = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 256;
   if (hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) ncu = 256;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel), 256,
-                                                   smem) != hipSuccess || per_cu < 1)
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel),
+                                                   threads, smem) != hipSuccess || per_cu < 1)
     per_cu = 1;
   return ncu * per_cu;
 }
@@ -278,52 +287,60 @@ int launch_chain_init(const ChainWs& w, int64_t words, hipStream_t st) {
   return launched();
 }
 
-template <typename T, int BN>
+template <typename T, typename S>
 int launch_fwd_chained_t(const void* x, SeqStrides sx, const float* cs128, void* y, SeqStrides sy,
                          float* prev128, float* prev_coarse, int ratio, float* fin, const ChainWs& w,
                          const Dims& di, hipStream_t st) {
+  constexpr int BN = S::BN, NT = S::NT;
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
   EMA_TRY(launch_chain_init(w, total * BN, st));
   const int smem = WalkCfg<T, BN>::smem_bytes(1, 1);
-  auto kernel = fwd_chained_kernel<T, BN, true>;
+  auto kernel = fwd_chained_kernel<T, BN, NT, S::FWD_MINW, true>;
   EMA_TRY(allow_smem(kernel, smem));
-  const int64_t cap = resident_blocks(kernel, smem);
+  const int64_t cap = resident_blocks(kernel, NT, smem);
   const unsigned grid = (unsigned)(total < cap ? total : cap);
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), smem, st, (const T*)x, sx, cs128, (T*)y, sy, prev128,
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), smem, st, (const T*)x, sx, cs128, (T*)y, sy, prev128,
                      prev_coarse, ratio, fin, w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T,
                      (int)di.C, ntiles, (int)cols, (int)total);
   return launched();
 }
 
-template <typename T, int BN>
+template <typename T, typename S>
 int launch_bwd_chained_t(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* cs128,
                          const float* prev128, void* dx, SeqStrides sdx, void* y, SeqStrides sy,
                          float* part, const ChainWs& w, const Dims& di, hipStream_t st) {
+  constexpr int BN = S::BN, NT = S::NT;
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
   EMA_TRY(launch_chain_init(w, total * BN, st));
   const int smem = WalkCfg<T, BN>::smem_bytes(2, 2);
   if (y) {
-    auto kernel = bwd_chained_kernel<T, BN, true>;
+    auto kernel = bwd_chained_kernel<T, BN, NT, S::BWD_MINW, true>;
     EMA_TRY(allow_smem(kernel, smem));
-    const int64_t cap = resident_blocks(kernel, smem);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(256), smem, st,
+    const int64_t cap = resident_blocks(kernel, NT, smem);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), smem, st,
                        (const T*)x, sx, (const T*)dy, sd, cs128, prev128, (T*)dx, sdx, (T*)y, sy, part,
                        w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles,
                        (int)cols, (int)total);
   } else {
-    auto kernel = bwd_chained_kernel<T, BN, false>;
+    auto kernel = bwd_chained_kernel<T, BN, NT, S::BWD_MINW, false>;
     EMA_TRY(allow_smem(kernel, smem));
-    const int64_t cap = resident_blocks(kernel, smem);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(256), smem, st,
+    const int64_t cap = resident_blocks(kernel, NT, smem);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), smem, st,
                        (const T*)x, sx, (const T*)dy, sd, cs128, prev128, (T*)dx, sdx, (T*)nullptr, sy,
                        part, w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles,
                        (int)cols, (int)total);
   }
   return launched();
+}
+
+// Column partials of ddA that the chained backward writes per (n, chunk, row).
+template <typename S>
+constexpr int chain_parts_per_dim(int64_t T) {
+  return (int)((T + S::BN - 1) / S::BN) * (S::NT / 256);
 }
 
 // dx, optionally the recomputed y, and the log-decay gradient in one pass over x and dy.
@@ -472,10 +489,11 @@ int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void
     }
     float* p128 = prev128 ? prev128 : (ratio == 1 ? prev : w.prev128);
     float* coarse = p128 == prev ? nullptr : prev;
-    if (dtype == EMA_BF16)
-      return launch_fwd_chained_t<bf16_t, kWalkBnBf16>(x, sx, cs128, y, sy, p128, coarse, ratio,
+    if (dtype == EMA_BF16) {
+      return launch_fwd_chained_t<bf16_t, ChainBf16>(x, sx, cs128, y, sy, p128, coarse, ratio,
                                                        final_state, w.chain, di, st);
-    return launch_fwd_chained_t<float, kWalkBnF32>(x, sx, cs128, y, sy, p128, coarse, ratio,
+    }
+    return launch_fwd_chained_t<float, ChainF32>(x, sx, cs128, y, sy, p128, coarse, ratio,
                                                    final_state, w.chain, di, st);
   }
   if (prev128) return EMA_ERR_UNSUPPORTED;  // only produced when chunk is a multiple of 128
@@ -609,7 +627,8 @@ static BwdWs carve_bwd(void* base, const Dims& di) {
   w.cs = take(ncq);
   w.states = take(nct);
   w.prev = take(nct);
-  w.part = take(ncq * (size_t)bwd_col_tiles(di, EMA_F32));  // the wider of the two tilings
+  const int parts_bf16 = chain_parts_per_dim<ChainBf16>(di.T), parts_f32 = chain_parts_per_dim<ChainF32>(di.T);
+  w.part = take(ncq * (size_t)(parts_bf16 > parts_f32 ? parts_bf16 : parts_f32));
   w.chain = chain_carve(p + off, di);
   off += chain_ws_bytes(di);
   w.bytes = off;
@@ -660,15 +679,16 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
   }
   // dx, the recomputed y and the per-column-tile partials of dA in one pass over x and dy;
   // the reverse inter-chunk state is handed over inside the kernel
-  if (dtype == EMA_BF16)
-    EMA_TRY((launch_bwd_chained_t<bf16_t, kWalkBnBf16>(x, sx, dy, sd, w.cs, prev128, dx, sdx, y, sy,
-                                                       w.part, w.chain, di, st)));
-  else
-    EMA_TRY((launch_bwd_chained_t<float, kWalkBnF32>(x, sx, dy, sd, w.cs, prev128, dx, sdx, y, sy,
+  int parts = dtype == EMA_BF16 ? chain_parts_per_dim<ChainBf16>(di.T) : chain_parts_per_dim<ChainF32>(di.T);
+  if (dtype == EMA_BF16) {
+    EMA_TRY((launch_bwd_chained_t<bf16_t, ChainBf16>(x, sx, dy, sd, w.cs, prev128, dx, sdx, y, sy, w.part,
+                                                     w.chain, di, st)));
+  } else
+    EMA_TRY((launch_bwd_chained_t<float, ChainF32>(x, sx, dy, sd, w.cs, prev128, dx, sdx, y, sy,
                                                      w.part, w.chain, di, st)));
   const int64_t total = d.N * d.C * d.Q;
   hipLaunchKernelGGL(dA_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w.part,
-                     ddA, (int)d.L, (int)d.Q, (int)d.C, (int)di.C, bwd_col_tiles(di, dtype), total);
+                     ddA, (int)d.L, (int)d.Q, (int)d.C, (int)di.C, parts, total);
   return launched();
 }
 

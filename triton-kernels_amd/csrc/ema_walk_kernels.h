@@ -175,7 +175,8 @@ __device__ __forceinline__ void walk_decay_frags(const float* csT, int wave, int
       const int k = 32 * wave + g * KG + EPL * (lane >> 5) + e;
       const float ck = csT[k + 1];
       const bool keep = REV ? (k >= rm) : (k <= rm);
-      const float val = keep ? __expf(fminf(REV ? ck - cm : cm - ck, 0.f)) : 0.f;
+      // branch-free: a masked element gets exp(-huge) = 0
+      const float val = __expf(keep ? fminf(REV ? ck - cm : cm - ck, 0.f) : -1.0e30f);
       hi[g].set(e, val);
       if (sizeof(T) == 2) lo[g].set(e, val - hi[g].get(e));
     }
