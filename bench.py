@@ -1,15 +1,16 @@
 #!/usr/bin/env python3
 """Benchmark of the EMA chunked scan, forward + backward, on one MI355X.
 
-One step = one forward (cumsum, chunk states, state passing, chunk scan) and one backward
-(recompute + dstates, reverse state passing, dx, the three log-decay gradient terms) of
-BASELINE configuration 3 at chunk size 128: b16 nh2 d1024 L4096, bf16 x / dy, fp32
-log-decay and accumulation.  Inputs are synthetic and resident in HBM before the timed
+One step = one forward and one backward through the autograd entry point
+(ema_matmul_scan_combined(...).backward(dy)) of BASELINE configuration 3 at chunk size 128:
+b16 nh2 d1024 L4096, bf16 x / dy, fp32 log-decay and accumulation.  The forward is one pass
+over x (cumsum + single-pass chained scan), the backward one pass over x and dy.  Inputs are synthetic and resident in HBM before the timed
 region; the step rotates over several input sets so that no step finds its inputs in the
 256 MB last-level cache.
 
 Prints ONE JSON line.  `roofline` describes the kernel with the largest share of the step,
-timed live with HIP events on the launch stream; `cpu_baseline` is the sequential CPU
+timed live with HIP events that the library records on the launch stream right around it;
+`stage_launchers` times every per-stage launcher of the reference's interface on its own; `cpu_baseline` is the sequential CPU
 oracle timed on a bounded sample and scaled to the full workload.
 """
 import argparse
@@ -22,6 +23,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 for p in (ROOT, os.path.join(ROOT, "triton-kernels_amd")):
     if p not in sys.path:
         sys.path.insert(0, p)
+
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), scaled by
+# what the same counters read for a plain 268 435 456-byte device copy (FETCH_SIZE reads
+# 131 085 KiB for it, factor 1.99982; WRITE_SIZE reads 262 144 KiB, factor 1).
+TRAFFIC_BYTES = {"fwd_single_pass": 573696315, "bwd_single_pass": 875648256}
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
@@ -193,6 +199,31 @@ def main():
     bwd_saved(0)
     ms_bwd_saved = time_region(bwd_saved, args.steps, torch)
 
+    # the two kernels that carry the step, timed alone with HIP events recorded by the library
+    # on the launch stream right around them
+    def kernel_ms(call):
+        pairs = []
+        for i in range(args.steps):
+            ev = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+            ev[0].record(); ev[1].record()  # materialise the handles
+            call(i, ev)
+            pairs.append(ev)
+        torch.cuda.synchronize()
+        return sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
+
+    x_bytes = N * L * T * 2
+    small = N * (-(-L // 128)) * (128 * 4 + T * 4)  # cs + chunk-entry states at 128-row chunking
+    main = {}
+    ms = kernel_ms(lambda i, ev: _ema_matmul_scan_combined_fwd(
+        sets[i % len(sets)][1].detach(), sets[i % len(sets)][0].detach(), Q, kernel_events=ev))
+    b = 2 * x_bytes + small
+    main["fwd_single_pass"] = {"ms": ms, "bytes": b, "GBps": b / ms / 1e6, "hbm_frac": b / ms / 1e6 / HBM_PEAK_GBS}
+    ms = kernel_ms(lambda i, ev: _ema_chunk_scan_combined_bwd(
+        sets[i % len(sets)][2], sets[i % len(sets)][0].detach(), sets[i % len(sets)][1].detach(), Q,
+        prev128=saved[i % len(sets)], kernel_events=ev))
+    b = 3 * x_bytes + small + N * (-(-L // 128)) * 128 * 4 * (T // 128)
+    main["bwd_single_pass"] = {"ms": ms, "bytes": b, "GBps": b / ms / 1e6, "hbm_frac": b / ms / 1e6 / HBM_PEAK_GBS}
+
     kernels = {}
     if not args.no_kernels:
         kernels = time_kernels([tuple(t.detach() for t in st) for st in sets], Q, args.steps, ab, torch)
@@ -223,22 +254,19 @@ def main():
             "fwd+bwd": (ab["fwd"] + ab["bwd"]) / ms_step / 1e6,
         },
         "hbm_frac_of_peak_fwd+bwd": (ab["fwd"] + ab["bwd"]) / ms_step / 1e6 / HBM_PEAK_GBS,
-        "kernels": kernels,
+        "step_kernels": main,
+        "stage_launchers": kernels,
     }
-    if kernels:
-        # kernels the timed step actually launches (the other rows are the per-stage launchers)
-        on_path = ("cumsum", "chunk_state", "state_passing_fwd", "chunk_scan", "bwd_dstates",
-                   "bwd_fused_dx_dA")
-        dom = max(on_path, key=lambda k: kernels[k]["ms"])
-        out["roofline"] = {
-            "kernel": dom,
-            "bound": "hbm",
-            "achieved": kernels[dom]["GBps"],
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": kernels[dom]["GBps"] / HBM_PEAK_GBS,
-            "traffic": None,
-        }
+    dom = max(main, key=lambda k: main[k]["ms"])
+    out["roofline"] = {
+        "kernel": dom,
+        "bound": "hbm",
+        "achieved": main[dom]["GBps"],
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": main[dom]["GBps"] / HBM_PEAK_GBS,
+        "traffic": TRAFFIC_BYTES.get(dom),
+    }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args, torch)
     print(json.dumps(out))

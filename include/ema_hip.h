@@ -96,13 +96,16 @@ size_t ema_fwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, in
  * scan with look-back) instead of by separate F2 / F3 passes; prev128, if not NULL,
  * receives the states entering each 128-row chunk, (N, ceil(seqlen/128), T), which
  * ema_bwd accepts to skip their recomputation.  For other chunk sizes F1..F4 run in
- * sequence and prev128 must be NULL.
+ * sequence and prev128 must be NULL.  ev_start / ev_stop (hipEvent_t, may be NULL) are
+ * recorded on the stream right before and after the kernel(s) that read x, so that a
+ * caller can time them apart from the small set-up kernels.
  * Replaces _ema_matmul_scan_combined_fwd, kernels/ema_kernels/ema_combined_fwd.py:12-45. */
 int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void* x,
             int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb,
             int64_t y_sl, int64_t y_sh, float* cs, float* prev, float* final_state,
             float* prev128, void* workspace, size_t workspace_bytes, int64_t batch,
-            int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk, void* stream);
+            int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk, void* stream,
+            void* ev_start, void* ev_stop);
 
 /* --------------------------------------------------------------- backward stages ---- */
 
@@ -201,7 +204,8 @@ size_t ema_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, in
  * same name of ema_fwd; without it the states entering each chunk are recomputed with one
  * more pass over x (F1..F3).  Outputs dx (layout of x) and ddA (N,C,Q) float32 with
  * ddA[n,c,q] = dL/dA[n, c*Q+q] (0 in the slots past seqlen); when y is not NULL the forward
- * output is recomputed into it (the reference's recompute_output=True).
+ * output is recomputed into it (the reference's recompute_output=True).  ev_start / ev_stop
+ * (hipEvent_t, may be NULL) are recorded right before and after the single-pass kernel.
  * Replaces _ema_chunk_scan_combined_bwd,
  * kernels/ema_kernels_bwd/ema_combined_bwd.py:13-83. */
 int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const void* x,
@@ -209,7 +213,8 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
             int64_t a_sl, int64_t a_sh, const float* prev128, int dtype, void* dx,
             int64_t dx_sb, int64_t dx_sl, int64_t dx_sh, float* ddA, void* y, int64_t y_sb,
             int64_t y_sl, int64_t y_sh, void* workspace, size_t workspace_bytes, int64_t batch,
-            int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk, void* stream);
+            int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk, void* stream,
+            void* ev_start, void* ev_stop);
 
 #ifdef __cplusplus
 }

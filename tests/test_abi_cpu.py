@@ -68,7 +68,7 @@ def test_validation_happens_before_any_launch():
     # workspace too small
     assert (
         handle.ema_fwd(fake, 8, 1, 0, fake, 64, 8, 0, _lib.EMA_F32, fake, 64, 8, 0, fake, fake, fake,
-                       None, fake, 16, 1, 1, 8, 8, 4, None)
+                       None, fake, 16, 1, 1, 8, 8, 4, None, None, None)
         == -2
     )
 

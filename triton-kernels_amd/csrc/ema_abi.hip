@@ -249,6 +249,12 @@ int bwd_col_tiles(const Dims& d, int dtype) {
 
 // ---------------------------------------------------------------- chained single-pass kernels
 
+// Records an optional hipEvent_t (NULL = nothing) on the launch stream.
+inline int record_event(void* ev, hipStream_t st) {
+  if (!ev) return EMA_OK;
+  return hipEventRecord(reinterpret_cast<hipEvent_t>(ev), st) == hipSuccess ? EMA_OK : EMA_ERR_LAUNCH;
+}
+
 // Workgroups of a persistent kernel that can be resident at once on the current device.
 template <typename K>
 int resident_blocks(K kernel, int threads, int smem) {
@@ -290,7 +296,7 @@ int launch_chain_init(const ChainWs& w, int64_t words, hipStream_t st) {
 template <typename T, typename S>
 int launch_fwd_chained_t(const void* x, SeqStrides sx, const float* cs128, void* y, SeqStrides sy,
                          float* prev128, float* prev_coarse, int ratio, float* fin, const ChainWs& w,
-                         const Dims& di, hipStream_t st) {
+                         const Dims& di, hipStream_t st, void* ev0, void* ev1) {
   constexpr int BN = S::BN, NT = S::NT;
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
@@ -301,22 +307,26 @@ int launch_fwd_chained_t(const void* x, SeqStrides sx, const float* cs128, void*
   EMA_TRY(allow_smem(kernel, smem));
   const int64_t cap = resident_blocks(kernel, NT, smem);
   const unsigned grid = (unsigned)(total < cap ? total : cap);
+  EMA_TRY(record_event(ev0, st));
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), smem, st, (const T*)x, sx, cs128, (T*)y, sy, prev128,
                      prev_coarse, ratio, fin, w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T,
                      (int)di.C, ntiles, (int)cols, (int)total);
-  return launched();
+  EMA_TRY(launched());
+  return record_event(ev1, st);
 }
 
 template <typename T, typename S>
 int launch_bwd_chained_t(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* cs128,
                          const float* prev128, void* dx, SeqStrides sdx, void* y, SeqStrides sy,
-                         float* part, const ChainWs& w, const Dims& di, hipStream_t st) {
+                         float* part, const ChainWs& w, const Dims& di, hipStream_t st, void* ev0,
+                         void* ev1) {
   constexpr int BN = S::BN, NT = S::NT;
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
   EMA_TRY(launch_chain_init(w, total * BN, st));
   const int smem = WalkCfg<T, BN>::smem_bytes(2, 2);
+  EMA_TRY(record_event(ev0, st));
   if (y) {
     auto kernel = bwd_chained_kernel<T, BN, NT, S::BWD_MINW, true>;
     EMA_TRY(allow_smem(kernel, smem));
@@ -334,7 +344,8 @@ int launch_bwd_chained_t(const void* x, SeqStrides sx, const void* dy, SeqStride
                        part, w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles,
                        (int)cols, (int)total);
   }
-  return launched();
+  EMA_TRY(launched());
+  return record_event(ev1, st);
 }
 
 // Column partials of ddA that the chained backward writes per (n, chunk, row).
@@ -462,7 +473,7 @@ int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void
             int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb, int64_t y_sl,
             int64_t y_sh, float* cs, float* prev, float* final_state, float* prev128,
             void* workspace, size_t workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen,
-            int64_t dim, int64_t chunk, void* stream) {
+            int64_t dim, int64_t chunk, void* stream, void* ev_start, void* ev_stop) {
   Dims d;
   EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
   EMA_TRY(check_dtype(dtype));
@@ -491,17 +502,19 @@ int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void
     float* coarse = p128 == prev ? nullptr : prev;
     if (dtype == EMA_BF16) {
       return launch_fwd_chained_t<bf16_t, ChainBf16>(x, sx, cs128, y, sy, p128, coarse, ratio,
-                                                       final_state, w.chain, di, st);
+                                                     final_state, w.chain, di, st, ev_start, ev_stop);
     }
     return launch_fwd_chained_t<float, ChainF32>(x, sx, cs128, y, sy, p128, coarse, ratio,
-                                                   final_state, w.chain, di, st);
+                                                 final_state, w.chain, di, st, ev_start, ev_stop);
   }
   if (prev128) return EMA_ERR_UNSUPPORTED;  // only produced when chunk is a multiple of 128
   float* states = static_cast<float*>(workspace);
+  EMA_TRY(record_event(ev_start, st));
   EMA_TRY(launch_chunk_reduce<0>(x, sx, dtype, cs, states, d, st));
   EMA_TRY(launch_state_passing_fwd(states, cs + (d.Q - 1), d.C * d.Q, d.Q, prev, final_state, d.N,
                                    d.C, d.T, st));
-  return launch_chunk_gemm<false>(x, sx, dtype, cs, prev, y, sy, d, st);
+  EMA_TRY(launch_chunk_gemm<false>(x, sx, dtype, cs, prev, y, sy, d, st));
+  return record_event(ev_stop, st);
 }
 
 int ema_chunk_scan_bwd_dstates(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh,
@@ -647,7 +660,7 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
             int64_t a_sh, const float* prev128, int dtype, void* dx, int64_t dx_sb, int64_t dx_sl,
             int64_t dx_sh, float* ddA, void* y, int64_t y_sb, int64_t y_sl, int64_t y_sh,
             void* workspace, size_t workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen,
-            int64_t dim, int64_t chunk, void* stream) {
+            int64_t dim, int64_t chunk, void* stream, void* ev_start, void* ev_stop) {
   Dims d;
   EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
   EMA_TRY(check_dtype(dtype));
@@ -682,10 +695,10 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
   int parts = dtype == EMA_BF16 ? chain_parts_per_dim<ChainBf16>(di.T) : chain_parts_per_dim<ChainF32>(di.T);
   if (dtype == EMA_BF16) {
     EMA_TRY((launch_bwd_chained_t<bf16_t, ChainBf16>(x, sx, dy, sd, w.cs, prev128, dx, sdx, y, sy, w.part,
-                                                     w.chain, di, st)));
+                                                     w.chain, di, st, ev_start, ev_stop)));
   } else
-    EMA_TRY((launch_bwd_chained_t<float, ChainF32>(x, sx, dy, sd, w.cs, prev128, dx, sdx, y, sy,
-                                                     w.part, w.chain, di, st)));
+    EMA_TRY((launch_bwd_chained_t<float, ChainF32>(x, sx, dy, sd, w.cs, prev128, dx, sdx, y, sy, w.part,
+                                                   w.chain, di, st, ev_start, ev_stop)));
   const int64_t total = d.N * d.C * d.Q;
   hipLaunchKernelGGL(dA_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w.part,
                      ddA, (int)d.L, (int)d.Q, (int)d.C, (int)di.C, parts, total);

@@ -29,7 +29,7 @@ _SIGNATURES = {
     "ema_state_passing_fwd": (c_int, [_P, _P, _I, _I, _P, _P, _I, _I, _I, _P]),
     "ema_scan_fwd": (c_int, _SEQ + [c_int, _P, _P] + _SEQ + [_I, _I, _I, _I, _I, _P]),
     "ema_fwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I]),
-    "ema_fwd": (c_int, _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _P]),
+    "ema_fwd": (c_int, _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _P, _P, _P]),
     "ema_chunk_scan_bwd_dstates": (c_int, _SEQ + [c_int, _P, _P, _I, _I, _I, _I, _I, _P]),
     "ema_state_passing_bwd_workspace_bytes": (c_size_t, [_I, _I, _I]),
     "ema_state_passing_bwd": (c_int, [_P, _P, _I, _I, _P, _P, _P, _P, c_size_t, _I, _I, _I, _P]),
@@ -41,7 +41,7 @@ _SIGNATURES = {
     "ema_bwd_dx_dA_fused_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "ema_bwd_dx_dA_fused": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P] + _SEQ + [_P] + _SEQ + [_P, c_size_t, _I, _I, _I, _I, _P]),
     "ema_bwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I]),
-    "ema_bwd": (c_int, _SEQ + _SEQ + _SEQ + [_P, c_int] + _SEQ + [_P] + _SEQ + [_P, c_size_t, _I, _I, _I, _I, _I, _P]),
+    "ema_bwd": (c_int, _SEQ + _SEQ + _SEQ + [_P, c_int] + _SEQ + [_P] + _SEQ + [_P, c_size_t, _I, _I, _I, _I, _I, _P, _P, _P]),
 }
 
 _lib = None
@@ -128,6 +128,14 @@ def decay_view(A: torch.Tensor):
     if A.dim() == 2:
         return [A.data_ptr(), A.stride(0), A.stride(1), 0], A.shape[0], 1, A.shape[1]
     return [A.data_ptr(), A.stride(0), A.stride(1), A.stride(2)], A.shape[0], A.shape[2], A.shape[1]
+
+
+def event_ptrs(events):
+    """(start, stop) raw hipEvent_t handles of a pair of torch.cuda.Event (timing enabled), or
+    (None, None).  The events must have been recorded once so that their handles exist."""
+    if events is None:
+        return None, None
+    return events[0].cuda_event, events[1].cuda_event
 
 
 def f32c(t: torch.Tensor) -> torch.Tensor:

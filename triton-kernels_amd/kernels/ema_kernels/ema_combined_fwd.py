@@ -10,14 +10,16 @@ import torch
 from kernels import _lib
 
 
-def _ema_matmul_scan_combined_fwd(A_ema, X_ema, chunk_size, dtype=torch.float32, return_prev128=False):
+def _ema_matmul_scan_combined_fwd(A_ema, X_ema, chunk_size, dtype=torch.float32, return_prev128=False,
+                                  kernel_events=None):
     """A_ema: (B, L) or (b, L, nh) float32 log-decay; X_ema: (B, L, T) or (b, L, nh, d).
 
     Returns (out, dA_cumsum (N, C, Q), states entering each chunk (N, C, T), final (N, T)).
     `dtype` is the dtype of the returned chunk states (computed in float32).  With
     return_prev128 a fifth value follows: the states entering each 128-row chunk, which the
     backward accepts to skip their recomputation (None when chunk_size is not a multiple
-    of 128)."""
+    of 128).  kernel_events: optional (start, stop) torch.cuda.Event pair recorded around the
+    kernel that reads x."""
     dev = _lib.require_gpu(A_ema, X_ema)
     x, x_args, batch, nh, seqlen, token_dim = _lib.seq_view(X_ema)
     a_args, a_batch, a_nh, a_len = _lib.decay_view(A_ema)
@@ -42,6 +44,7 @@ def _ema_matmul_scan_combined_fwd(A_ema, X_ema, chunk_size, dtype=torch.float32,
             *a_args, *x_args, _lib.dtype_code(x), *y_args, cs.data_ptr(), prev.data_ptr(),
             final.data_ptr(), None if prev128 is None or prev128 is prev else prev128.data_ptr(),
             ws.data_ptr(), ws_bytes, batch, nh, seqlen, token_dim, chunk_size, _lib.stream_ptr(dev),
+            *_lib.event_ptrs(kernel_events),
         )
     _lib.check(st, "_ema_matmul_scan_combined_fwd")
     if dtype != torch.float32:

@@ -9,10 +9,12 @@ from kernels import _lib
 
 
 def _ema_chunk_scan_combined_bwd(dout, x, A, chunk_size, dt_limit=(0.0, float("inf")), recompute_output=False,
-                                 prev128=None):
+                                 prev128=None, kernel_events=None):
     """dout, x: (B, L, T) or (b, L, nh, d); A: (B, L) or (b, L, nh) float32.  prev128
     (optional) is the fifth return value of _ema_matmul_scan_combined_fwd(...,
     return_prev128=True); with it the backward does not re-read x to rebuild it.
+    kernel_events: optional (start, stop) torch.cuda.Event pair recorded around the
+    single-pass kernel.
 
     Returns (dx, ddA) with ddA (N, nchunks, chunk_size) float32, ddA[n, c, q] = dL/dA at
     position c * chunk_size + q of sequence n; with recompute_output also the forward
@@ -47,6 +49,7 @@ def _ema_chunk_scan_combined_bwd(dout, x, A, chunk_size, dt_limit=(0.0, float("i
             *d_args, *x_args, *a_args, None if prev128 is None else prev128.data_ptr(),
             _lib.dtype_code(x), *dx_args, ddA.data_ptr(), *y_args,
             ws.data_ptr(), ws_bytes, batch, nh, seqlen, token_dim, chunk_size, _lib.stream_ptr(dev),
+            *_lib.event_ptrs(kernel_events),
         )
     _lib.check(st, "_ema_chunk_scan_combined_bwd")
     return (dx, ddA) if not recompute_output else (dx, ddA, y)
