@@ -241,3 +241,52 @@ def test_error_behaviour(device):
         _ema_chunk_state_fwd(torch.zeros(2, 24, 8, device=device), torch.zeros(2, 2, 8, device=device))
     with pytest.raises(AssertionError):  # feature size must allow 16-byte rows
         _ema_chunk_state_fwd(torch.zeros(2, 16, 6, device=device), torch.zeros(2, 2, 8, device=device))
+
+
+def test_legacy_probability_entry_point(device):
+    """ema_scan_combined(x, p) against z_t = (1-p) z_{t-1} + p x_t (main.py:120-131 of the reference)."""
+    from kernels.ema import ema_scan_combined
+
+    announce("ema_scan_combined(x, p)")
+    g = torch.Generator().manual_seed(3)
+    X = torch.randn(2, 300, 64, generator=g)
+    P = torch.rand(2, 300, 1, generator=g) * 0.98 + 0.01
+    ref = torch.empty_like(X)
+    zprev = torch.zeros(2, 64)
+    for t in range(300):
+        zprev = (1 - P[:, t]) * zprev + P[:, t] * X[:, t]
+        ref[:, t] = zprev
+    got = ema_scan_combined(X.to(device), P.to(device))
+    check_close("z", got, ref, F32)
+
+
+def test_legacy_mamba_encoded_entry_point(device):
+    """ema_chunk_scan_combined with the encoding of main.py:92-98 of the reference
+    (dt = -log(1-p), B = p, C = 1, x / dt) reproduces the EMA loop."""
+    from kernels.ema_combined import ema_chunk_scan_combined
+
+    announce("ema_chunk_scan_combined(x, dt, A, B, C)")
+    g = torch.Generator().manual_seed(4)
+    b, L, nh, hd = 2, 260, 2, 32
+    X = torch.randn(b, L, nh * hd, generator=g)
+    P = torch.rand(b, L, 1, generator=g) * 0.9 + 0.05
+    ref = torch.empty_like(X)
+    zprev = torch.zeros(b, nh * hd)
+    for t in range(L):
+        zprev = (1 - P[:, t]) * zprev + P[:, t] * X[:, t]
+        ref[:, t] = zprev
+    dt = -torch.log(1 - P).squeeze(-1)
+    X_m = (X / dt[..., None]).reshape(b, L, nh, hd)
+    dt_h = dt[..., None].expand(b, L, nh).contiguous()
+    A = -torch.ones(nh)
+    B_m = P.reshape(b, L, 1, 1)
+    C_m = torch.ones_like(B_m)
+    out, final = ema_chunk_scan_combined(
+        X_m.to(device), dt_h.to(device), A.to(device), B_m.to(device), C_m.to(device), 64,
+        return_final_states=True,
+    )
+    check_close("out", out.reshape(b, L, nh * hd), ref, F32)
+    check_close("final", final.reshape(b, nh * hd), ref[:, -1], F32)
+    with pytest.raises(NotImplementedError):
+        ema_chunk_scan_combined(X_m.to(device), dt_h.to(device), A.to(device),
+                                torch.ones(b, L, 1, 4, device=device), torch.ones(b, L, 1, 4, device=device), 64)
