@@ -27,7 +27,7 @@ for p in (ROOT, os.path.join(ROOT, "triton-kernels_amd")):
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), scaled by
 # what the same counters read for a plain 268 435 456-byte device copy (FETCH_SIZE reads
 # 131 085 KiB for it, factor 1.99982; WRITE_SIZE reads 262 144 KiB, factor 1).
-TRAFFIC_BYTES = {"fwd_single_pass": 573696315, "bwd_single_pass": 875648256}
+TRAFFIC_BYTES = {"fwd_single_pass": 573698918, "bwd_single_pass": 875653612}
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
