@@ -9,6 +9,7 @@
 #include "ema_stream_kernels.h"
 #include "ema_walk_kernels.h"
 #include "ema_chain_kernels.h"
+#include "ema_wave_kernels.h"
 
 using namespace ema;
 
@@ -348,6 +349,72 @@ int launch_bwd_chained_t(const void* x, SeqStrides sx, const void* dy, SeqStride
   return record_event(ev1, st);
 }
 
+// Shape of the register-tile single-pass kernels: columns per lane (a wave tile is 128 rows
+// by 16 times that many columns), waves per workgroup, waves per SIMD the register
+// allocation must allow.
+struct WaveBf16 {
+  static constexpr int FWD_CPL = 4, FWD_MINW = 4, BWD_CPL = 4, BWD_MINW = 2, NWAVES = 4;
+};
+struct WaveF32 {
+  static constexpr int FWD_CPL = 4, FWD_MINW = 3, BWD_CPL = 2, BWD_MINW = 2, NWAVES = 4;
+};
+
+template <typename T, typename S>
+int launch_fwd_wave_t(const void* x, SeqStrides sx, const float* A, SeqStrides sa, const float* cs128,
+                      void* y, SeqStrides sy, float* prev128, float* prev_coarse, int ratio, float* fin,
+                      const ChainWs& w, const Dims& di, hipStream_t st, void* ev0, void* ev1) {
+  constexpr int CPL = S::FWD_CPL, BN = 16 * CPL, NT = 64 * S::NWAVES;
+  const int ntiles = (int)((di.T + BN - 1) / BN);
+  const int64_t cols = di.N * ntiles, total = cols * di.C;
+  if (total > 0x7fffffff) return EMA_ERR_SHAPE;
+  EMA_TRY(launch_chain_init(w, total * BN, st));
+  auto kernel = fwd_wave_kernel<T, CPL, S::NWAVES, S::FWD_MINW>;
+  const int64_t cap = resident_blocks(kernel, NT, 0);
+  const int64_t want = (total + S::NWAVES - 1) / S::NWAVES;
+  EMA_TRY(record_event(ev0, st));
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(NT), 0, st, (const T*)x, sx, A,
+                     sa, cs128, (T*)y, sy, prev128, prev_coarse, ratio, fin, w.status, w.counters,
+                     (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total);
+  EMA_TRY(launched());
+  return record_event(ev1, st);
+}
+
+template <typename T, typename S>
+int launch_bwd_wave_t(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* A,
+                      SeqStrides sa, const float* cs128, const float* prev128, void* dx, SeqStrides sdx,
+                      void* y, SeqStrides sy, float* part, const ChainWs& w, const Dims& di,
+                      hipStream_t st, void* ev0, void* ev1) {
+  constexpr int CPL = S::BWD_CPL, BN = 16 * CPL, NT = 64 * S::NWAVES;
+  const int ntiles = (int)((di.T + BN - 1) / BN);
+  const int64_t cols = di.N * ntiles, total = cols * di.C;
+  if (total > 0x7fffffff) return EMA_ERR_SHAPE;
+  EMA_TRY(launch_chain_init(w, total * BN, st));
+  const int64_t want = (total + S::NWAVES - 1) / S::NWAVES;
+  EMA_TRY(record_event(ev0, st));
+  if (y) {
+    auto kernel = bwd_wave_kernel<T, CPL, S::NWAVES, S::BWD_MINW, true>;
+    const int64_t cap = resident_blocks(kernel, NT, 0);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(NT), 0, st, (const T*)x, sx,
+                       (const T*)dy, sd, A, sa, cs128, prev128, (T*)dx, sdx, (T*)y, sy, part, w.status,
+                       w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols,
+                       (int)total);
+  } else {
+    auto kernel = bwd_wave_kernel<T, CPL, S::NWAVES, S::BWD_MINW, false>;
+    const int64_t cap = resident_blocks(kernel, NT, 0);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(NT), 0, st, (const T*)x, sx,
+                       (const T*)dy, sd, A, sa, cs128, prev128, (T*)dx, sdx, (T*)nullptr, sy, part,
+                       w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles,
+                       (int)cols, (int)total);
+  }
+  EMA_TRY(launched());
+  return record_event(ev1, st);
+}
+
+template <typename S>
+constexpr int wave_parts_per_dim(int64_t T) {
+  return (int)((T + 16 * S::BWD_CPL - 1) / (16 * S::BWD_CPL));
+}
+
 // Column partials of ddA that the chained backward writes per (n, chunk, row).
 template <typename S>
 constexpr int chain_parts_per_dim(int64_t T) {
@@ -501,11 +568,11 @@ int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void
     float* p128 = prev128 ? prev128 : (ratio == 1 ? prev : w.prev128);
     float* coarse = p128 == prev ? nullptr : prev;
     if (dtype == EMA_BF16) {
-      return launch_fwd_chained_t<bf16_t, ChainBf16>(x, sx, cs128, y, sy, p128, coarse, ratio,
-                                                     final_state, w.chain, di, st, ev_start, ev_stop);
-    }
-    return launch_fwd_chained_t<float, ChainF32>(x, sx, cs128, y, sy, p128, coarse, ratio,
+      return launch_fwd_wave_t<bf16_t, WaveBf16>(x, sx, A, sa, cs128, y, sy, p128, coarse, ratio,
                                                  final_state, w.chain, di, st, ev_start, ev_stop);
+    }
+    return launch_fwd_wave_t<float, WaveF32>(x, sx, A, sa, cs128, y, sy, p128, coarse, ratio,
+                                             final_state, w.chain, di, st, ev_start, ev_stop);
   }
   if (prev128) return EMA_ERR_UNSUPPORTED;  // only produced when chunk is a multiple of 128
   float* states = static_cast<float*>(workspace);
@@ -640,7 +707,7 @@ static BwdWs carve_bwd(void* base, const Dims& di) {
   w.cs = take(ncq);
   w.states = take(nct);
   w.prev = take(nct);
-  const int parts_bf16 = chain_parts_per_dim<ChainBf16>(di.T), parts_f32 = chain_parts_per_dim<ChainF32>(di.T);
+  const int parts_bf16 = wave_parts_per_dim<WaveBf16>(di.T), parts_f32 = wave_parts_per_dim<WaveF32>(di.T);
   w.part = take(ncq * (size_t)(parts_bf16 > parts_f32 ? parts_bf16 : parts_f32));
   w.chain = chain_carve(p + off, di);
   off += chain_ws_bytes(di);
@@ -681,7 +748,8 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
   const SeqStrides sx{x_sb, x_sl, x_sh}, sd{dy_sb, dy_sl, dy_sh}, sdx{dx_sb, dx_sl, dx_sh};
   const SeqStrides sy{y_sb, y_sl, y_sh};
 
-  EMA_TRY(launch_cumsum(A, SeqStrides{a_sb, a_sl, a_sh}, w.cs, di, st));
+  const SeqStrides sa{a_sb, a_sl, a_sh};
+  EMA_TRY(launch_cumsum(A, sa, w.cs, di, st));
   if (!prev128) {
     // states entering each chunk, recomputed: chunk states, then the inter-chunk recurrence
     // (its final state is not needed and lands in `part`, which is free until the main kernel)
@@ -692,13 +760,13 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
   }
   // dx, the recomputed y and the per-column-tile partials of dA in one pass over x and dy;
   // the reverse inter-chunk state is handed over inside the kernel
-  int parts = dtype == EMA_BF16 ? chain_parts_per_dim<ChainBf16>(di.T) : chain_parts_per_dim<ChainF32>(di.T);
+  int parts = dtype == EMA_BF16 ? wave_parts_per_dim<WaveBf16>(di.T) : wave_parts_per_dim<WaveF32>(di.T);
   if (dtype == EMA_BF16) {
-    EMA_TRY((launch_bwd_chained_t<bf16_t, ChainBf16>(x, sx, dy, sd, w.cs, prev128, dx, sdx, y, sy, w.part,
-                                                     w.chain, di, st, ev_start, ev_stop)));
+    EMA_TRY((launch_bwd_wave_t<bf16_t, WaveBf16>(x, sx, dy, sd, A, sa, w.cs, prev128, dx, sdx, y, sy, w.part,
+                                                 w.chain, di, st, ev_start, ev_stop)));
   } else
-    EMA_TRY((launch_bwd_chained_t<float, ChainF32>(x, sx, dy, sd, w.cs, prev128, dx, sdx, y, sy, w.part,
-                                                   w.chain, di, st, ev_start, ev_stop)));
+    EMA_TRY((launch_bwd_wave_t<float, WaveF32>(x, sx, dy, sd, A, sa, w.cs, prev128, dx, sdx, y, sy, w.part,
+                                               w.chain, di, st, ev_start, ev_stop)));
   const int64_t total = d.N * d.C * d.Q;
   hipLaunchKernelGGL(dA_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w.part,
                      ddA, (int)d.L, (int)d.Q, (int)d.C, (int)di.C, parts, total);
