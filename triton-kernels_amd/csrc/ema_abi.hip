@@ -9,7 +9,7 @@
 #include "ema_stream_kernels.h"
 #include "ema_walk_kernels.h"
 #include "ema_chain_kernels.h"
-#include "ema_wave_kernels.h"
+#include "ema_tile_kernels.h"
 
 using namespace ema;
 
@@ -268,7 +268,7 @@ int resident_blocks(K kernel, int threads, int smem) {
   return ncu * per_cu;
 }
 
-inline int64_t padded_dim(int64_t T) { return (T + 127) / 128 * 128; }
+inline int64_t padded_dim(int64_t T) { return (T + 255) / 256 * 256; }
 
 // status words + counters of one chained kernel
 struct ChainWs {
@@ -349,30 +349,30 @@ int launch_bwd_chained_t(const void* x, SeqStrides sx, const void* dy, SeqStride
   return record_event(ev1, st);
 }
 
-// Shape of the register-tile single-pass kernels: columns per lane (a wave tile is 128 rows
-// by 16 times that many columns), waves per workgroup, waves per SIMD the register
-// allocation must allow.
-struct WaveBf16 {
-  static constexpr int FWD_CPL = 4, FWD_MINW = 4, BWD_CPL = 4, BWD_MINW = 2, NWAVES = 4;
+// Shape of the register-tile single-pass kernels: columns per lane (a tile is 128 rows by
+// 64 times that many columns), rows per lane (128 / RPL waves per workgroup), waves per SIMD
+// the register allocation must allow.
+struct TileBf16 {
+  static constexpr int FWD_CPL = 4, BWD_CPL = 4, RPL = 8, FWD_MINW = 8, BWD_MINW = 4;
 };
-struct WaveF32 {
-  static constexpr int FWD_CPL = 4, FWD_MINW = 3, BWD_CPL = 2, BWD_MINW = 2, NWAVES = 4;
+struct TileF32 {
+  static constexpr int FWD_CPL = 2, BWD_CPL = 2, RPL = 8, FWD_MINW = 8, BWD_MINW = 4;
 };
 
 template <typename T, typename S>
-int launch_fwd_wave_t(const void* x, SeqStrides sx, const float* A, SeqStrides sa, const float* cs128,
+int launch_fwd_tile_t(const void* x, SeqStrides sx, const float* A, SeqStrides sa, const float* cs128,
                       void* y, SeqStrides sy, float* prev128, float* prev_coarse, int ratio, float* fin,
                       const ChainWs& w, const Dims& di, hipStream_t st, void* ev0, void* ev1) {
-  constexpr int CPL = S::FWD_CPL, BN = 16 * CPL, NT = 64 * S::NWAVES;
+  using Cfg = TileCfg<T, S::FWD_CPL, S::RPL>;
+  constexpr int BN = Cfg::BN, NT = Cfg::NT;
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
   EMA_TRY(launch_chain_init(w, total * BN, st));
-  auto kernel = fwd_wave_kernel<T, CPL, S::NWAVES, S::FWD_MINW>;
+  auto kernel = fwd_tile_kernel<T, S::FWD_CPL, S::RPL, S::FWD_MINW>;
   const int64_t cap = resident_blocks(kernel, NT, 0);
-  const int64_t want = (total + S::NWAVES - 1) / S::NWAVES;
   EMA_TRY(record_event(ev0, st));
-  hipLaunchKernelGGL(kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(NT), 0, st, (const T*)x, sx, A,
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), 0, st, (const T*)x, sx, A,
                      sa, cs128, (T*)y, sy, prev128, prev_coarse, ratio, fin, w.status, w.counters,
                      (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total);
   EMA_TRY(launched());
@@ -380,28 +380,28 @@ int launch_fwd_wave_t(const void* x, SeqStrides sx, const float* A, SeqStrides s
 }
 
 template <typename T, typename S>
-int launch_bwd_wave_t(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* A,
+int launch_bwd_tile_t(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* A,
                       SeqStrides sa, const float* cs128, const float* prev128, void* dx, SeqStrides sdx,
                       void* y, SeqStrides sy, float* part, const ChainWs& w, const Dims& di,
                       hipStream_t st, void* ev0, void* ev1) {
-  constexpr int CPL = S::BWD_CPL, BN = 16 * CPL, NT = 64 * S::NWAVES;
+  using Cfg = TileCfg<T, S::BWD_CPL, S::RPL>;
+  constexpr int BN = Cfg::BN, NT = Cfg::NT;
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
   EMA_TRY(launch_chain_init(w, total * BN, st));
-  const int64_t want = (total + S::NWAVES - 1) / S::NWAVES;
   EMA_TRY(record_event(ev0, st));
   if (y) {
-    auto kernel = bwd_wave_kernel<T, CPL, S::NWAVES, S::BWD_MINW, true>;
+    auto kernel = bwd_tile_kernel<T, S::BWD_CPL, S::RPL, S::BWD_MINW, true>;
     const int64_t cap = resident_blocks(kernel, NT, 0);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(NT), 0, st, (const T*)x, sx,
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), 0, st, (const T*)x, sx,
                        (const T*)dy, sd, A, sa, cs128, prev128, (T*)dx, sdx, (T*)y, sy, part, w.status,
                        w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols,
                        (int)total);
   } else {
-    auto kernel = bwd_wave_kernel<T, CPL, S::NWAVES, S::BWD_MINW, false>;
+    auto kernel = bwd_tile_kernel<T, S::BWD_CPL, S::RPL, S::BWD_MINW, false>;
     const int64_t cap = resident_blocks(kernel, NT, 0);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(NT), 0, st, (const T*)x, sx,
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), 0, st, (const T*)x, sx,
                        (const T*)dy, sd, A, sa, cs128, prev128, (T*)dx, sdx, (T*)nullptr, sy, part,
                        w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles,
                        (int)cols, (int)total);
@@ -411,8 +411,8 @@ int launch_bwd_wave_t(const void* x, SeqStrides sx, const void* dy, SeqStrides s
 }
 
 template <typename S>
-constexpr int wave_parts_per_dim(int64_t T) {
-  return (int)((T + 16 * S::BWD_CPL - 1) / (16 * S::BWD_CPL));
+constexpr int tile_parts_per_dim(int64_t T) {
+  return (int)((T + 64 * S::BWD_CPL - 1) / (64 * S::BWD_CPL));
 }
 
 // Column partials of ddA that the chained backward writes per (n, chunk, row).
@@ -568,10 +568,10 @@ int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void
     float* p128 = prev128 ? prev128 : (ratio == 1 ? prev : w.prev128);
     float* coarse = p128 == prev ? nullptr : prev;
     if (dtype == EMA_BF16) {
-      return launch_fwd_wave_t<bf16_t, WaveBf16>(x, sx, A, sa, cs128, y, sy, p128, coarse, ratio,
+      return launch_fwd_tile_t<bf16_t, TileBf16>(x, sx, A, sa, cs128, y, sy, p128, coarse, ratio,
                                                  final_state, w.chain, di, st, ev_start, ev_stop);
     }
-    return launch_fwd_wave_t<float, WaveF32>(x, sx, A, sa, cs128, y, sy, p128, coarse, ratio,
+    return launch_fwd_tile_t<float, TileF32>(x, sx, A, sa, cs128, y, sy, p128, coarse, ratio,
                                              final_state, w.chain, di, st, ev_start, ev_stop);
   }
   if (prev128) return EMA_ERR_UNSUPPORTED;  // only produced when chunk is a multiple of 128
@@ -707,7 +707,7 @@ static BwdWs carve_bwd(void* base, const Dims& di) {
   w.cs = take(ncq);
   w.states = take(nct);
   w.prev = take(nct);
-  const int parts_bf16 = wave_parts_per_dim<WaveBf16>(di.T), parts_f32 = wave_parts_per_dim<WaveF32>(di.T);
+  const int parts_bf16 = tile_parts_per_dim<TileBf16>(di.T), parts_f32 = tile_parts_per_dim<TileF32>(di.T);
   w.part = take(ncq * (size_t)(parts_bf16 > parts_f32 ? parts_bf16 : parts_f32));
   w.chain = chain_carve(p + off, di);
   off += chain_ws_bytes(di);
@@ -760,12 +760,12 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
   }
   // dx, the recomputed y and the per-column-tile partials of dA in one pass over x and dy;
   // the reverse inter-chunk state is handed over inside the kernel
-  int parts = dtype == EMA_BF16 ? wave_parts_per_dim<WaveBf16>(di.T) : wave_parts_per_dim<WaveF32>(di.T);
+  int parts = dtype == EMA_BF16 ? tile_parts_per_dim<TileBf16>(di.T) : tile_parts_per_dim<TileF32>(di.T);
   if (dtype == EMA_BF16) {
-    EMA_TRY((launch_bwd_wave_t<bf16_t, WaveBf16>(x, sx, dy, sd, A, sa, w.cs, prev128, dx, sdx, y, sy, w.part,
+    EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16>(x, sx, dy, sd, A, sa, w.cs, prev128, dx, sdx, y, sy, w.part,
                                                  w.chain, di, st, ev_start, ev_stop)));
   } else
-    EMA_TRY((launch_bwd_wave_t<float, WaveF32>(x, sx, dy, sd, A, sa, w.cs, prev128, dx, sdx, y, sy, w.part,
+    EMA_TRY((launch_bwd_tile_t<float, TileF32>(x, sx, dy, sd, A, sa, w.cs, prev128, dx, sdx, y, sy, w.part,
                                                w.chain, di, st, ev_start, ev_stop)));
   const int64_t total = d.N * d.C * d.Q;
   hipLaunchKernelGGL(dA_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w.part,

@@ -1,0 +1,434 @@
+// Single-pass forward and backward of the EMA scan with the tile held in registers.
+//
+// The scan is HBM-bound and needs one multiply-add per element, so the single-pass kernels
+// form no decay matrices: a workgroup owns a tile of 128 rows x BN columns; wave g owns the
+// RPL consecutive rows RPL*g .. of it and lane l the CPL adjacent columns CPL*l .., so every
+// load or store instruction of a wave moves one contiguous row segment of 64*CPL elements
+// and a lane has only RPL short loads in flight (the shape that measured closest to a plain
+// device copy on this part).  Each lane runs the recurrence y = a*y + x down its rows:
+//
+//   1. local pass from a zero state; the value after the last row is what the row group
+//      contributes;
+//   2. the row groups of the tile are combined per column through LDS, which gives the
+//      tile's aggregate; it is published and the state entering the tile is obtained from
+//      the earlier tiles of the same columns by the chained scan with look-back (see
+//      ema_chain_kernels.h: 64-bit {flag, value} words, ticket order);
+//   3. final pass: the recurrence again from the true state entering the row group, stored
+//      from registers.  The values are those of the sequential recurrence in float32,
+//      whatever the chunking.
+//
+// The backward does the same from the last row to the first for dx = dy + a[next]*dx[next],
+// keeps the forward values y (float32, from the states the forward pass saved) in registers
+// and forms dA[m] = a[m] * <dx[m], y[m-1]> on the way.
+#pragma once
+#include "ema_chain_kernels.h"
+
+namespace ema {
+
+#ifdef EMA_TIMING
+#define EMA_TSTAMP(slot)                                                                            \
+  do {                                                                                              \
+    if (threadIdx.x == 0 && g_ema_timing) g_ema_timing[(int64_t)cur * 8 + (slot)] = wall_clock64(); \
+  } while (0)
+#else
+#define EMA_TSTAMP(slot) \
+  do {                   \
+  } while (0)
+#endif
+
+template <typename T, int CPL, int RPL>
+struct TileCfg {
+  static constexpr int NG = kTileRows / RPL;            // row groups = waves of the workgroup
+  static constexpr int NT = 64 * NG;                    // threads
+  static constexpr int BN = 64 * CPL;                   // columns of a tile
+  static constexpr int NW = CPL * (int)sizeof(T) / 4;   // 32-bit words of one lane's row
+  static_assert(NW == 2 || NW == 4, "a lane's row is 8 or 16 bytes");
+  static_assert(NG * RPL == kTileRows && NG <= 16 && BN <= NT, "tile shape");
+};
+
+template <int NW>
+struct RowWords {
+  unsigned w[NW];
+};
+
+template <int NW>
+__device__ __forceinline__ RowWords<NW> row_load(const void* p) {
+  RowWords<NW> r;
+  if constexpr (NW == 4) {
+    const uint4 v = *reinterpret_cast<const uint4*>(p);
+    r.w[0] = v.x, r.w[1] = v.y, r.w[2] = v.z, r.w[3] = v.w;
+  } else {
+    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    r.w[0] = v.x, r.w[1] = v.y;
+  }
+  return r;
+}
+template <int NW>
+__device__ __forceinline__ void row_store(void* p, const RowWords<NW>& r) {
+  if constexpr (NW == 4) *reinterpret_cast<uint4*>(p) = make_uint4(r.w[0], r.w[1], r.w[2], r.w[3]);
+  else *reinterpret_cast<uint2*>(p) = make_uint2(r.w[0], r.w[1]);
+}
+template <int NW>
+__device__ __forceinline__ RowWords<NW> row_zero() {
+  RowWords<NW> r;
+#pragma unroll
+  for (int i = 0; i < NW; ++i) r.w[i] = 0u;
+  return r;
+}
+
+// element e of a row as float
+template <typename T, int NW>
+__device__ __forceinline__ float row_get(const RowWords<NW>& r, int e) {
+  if constexpr (sizeof(T) == 4) return __uint_as_float(r.w[e]);
+  else return __uint_as_float((e & 1) ? (r.w[e >> 1] & 0xffff0000u) : (r.w[e >> 1] << 16));
+}
+
+typedef bf16_t bf16x2 __attribute__((ext_vector_type(2)));
+// CPL floats -> a row (round to nearest even for bf16)
+template <typename T, int CPL, int NW>
+__device__ __forceinline__ RowWords<NW> row_pack(const float* v) {
+  RowWords<NW> r;
+  if constexpr (sizeof(T) == 4) {
+#pragma unroll
+    for (int e = 0; e < NW; ++e) r.w[e] = __float_as_uint(v[e]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < NW; ++e) {
+      bf16x2 p;
+      p[0] = (bf16_t)v[2 * e];
+      p[1] = (bf16_t)v[2 * e + 1];
+      r.w[e] = __builtin_bit_cast(unsigned, p);
+    }
+  }
+  return r;
+}
+
+// Makes the registers of a tile opaque to the optimiser, so that values derived from them in
+// one pass (the float32 conversions) are formed again in the next pass instead of being kept.
+template <int NW, int RPL>
+__device__ __forceinline__ void rows_opaque(RowWords<NW>* rows) {
+#pragma unroll
+  for (int i = 0; i < RPL; ++i)
+#pragma unroll
+    for (int k = 0; k < NW; ++k) asm volatile("" : "+v"(rows[i].w[k]));
+}
+
+// The RPL rows of this lane.  g points at (first row of the wave, first column of the tile);
+// rows at or past `nrows` and columns past the end read as 0.
+template <typename T, int CPL, int RPL>
+__device__ __forceinline__ void tile_load_rows(RowWords<TileCfg<T, CPL, RPL>::NW>* rows,
+                                               const T* __restrict__ g, int64_t sl, int nrows, bool cok,
+                                               int lane) {
+  constexpr int NW = TileCfg<T, CPL, RPL>::NW;
+  const unsigned off = (unsigned)lane * CPL;
+  if (nrows >= RPL && __all(cok)) {
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) rows[i] = row_load<NW>(g + (int64_t)i * sl + off);
+  } else {
+#pragma unroll
+    for (int i = 0; i < RPL; ++i)
+      rows[i] = (i < nrows && cok) ? row_load<NW>(g + (int64_t)i * sl + off) : row_zero<NW>();
+  }
+}
+
+// a[i] = exp(min(A[row], 0)) of the wave's rows (1 past the end of the sequence); the
+// addresses are uniform over the wave.
+template <int RPL>
+__device__ __forceinline__ void tile_decays(float* a, const float* __restrict__ A, int64_t a_sl, int nrows) {
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) a[i] = i < nrows ? __expf(fminf(A[(int64_t)i * a_sl], 0.f)) : 1.f;
+}
+
+// Inclusive state entering chunk c for one column, as chain_look, with the first word
+// requested before the loop so that a published predecessor costs one round trip.
+template <bool REV, int BN>
+__device__ __forceinline__ float tile_look(const u64* status, const float* __restrict__ cs_n, int c,
+                                           int C, int k, unsigned* err) {
+  return chain_look<REV, BN>(status, cs_n, c, C, k, err);
+}
+
+// ------------------------------------------------------------------------------------
+// Forward.  Writes y, prev[n,c,:] (state entering each 128-row chunk), optionally a copy at
+// a coarser chunking and the final state.  status: N*ntiles*C*BN zeroed words; counters[0]
+// ticket, counters[3] error word.  One ticket = one tile; the next ticket is fetched while
+// the tile is processed.
+// ------------------------------------------------------------------------------------
+template <typename T, int CPL, int RPL, int MINW>
+__global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
+    const T* __restrict__ x, SeqStrides sx, const float* __restrict__ A, SeqStrides sa,
+    const float* __restrict__ cs, T* __restrict__ y, SeqStrides sy, float* __restrict__ prev,
+    float* __restrict__ prev_coarse, int ratio, float* __restrict__ final_state,
+    u64* __restrict__ status, unsigned* __restrict__ counters, int nh, int L, int Tdim, int C,
+    int ntiles, int cols, int total) {
+  using W = TileCfg<T, CPL, RPL>;
+  constexpr int BN = W::BN, NW = W::NW, NG = W::NG;
+  __shared__ __attribute__((aligned(16))) float sS[2][NG][BN];  // group states, double-buffered by tile
+  __shared__ float sD[2][NG];                                   // total decay of each row group
+  __shared__ int s_ticket[2];
+  const int lane = threadIdx.x & 63;
+  const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  unsigned* err = counters + 3;
+
+  if (threadIdx.x == 0) s_ticket[0] = (int)atomicAdd(counters, 1u);
+  __syncthreads();
+  int cur = s_ticket[0], buf = 0, slot = 1;
+  while (cur < total) {
+    int future = 0;
+    if (threadIdx.x == 0) future = (int)atomicAdd(counters, 1u);
+    const ChainTile t = chain_decode<false, BN>(cur, cols, ntiles, C, nh, L);
+    const bool cok = t.col0 + lane * CPL < Tdim;
+    const int nrows = t.limit - RPL * grp;  // valid rows of this wave (may be <= 0)
+    EMA_TSTAMP(0);
+    RowWords<NW> rows[RPL];
+    tile_load_rows<T, CPL, RPL>(rows, x + (int64_t)t.b * sx.sb + (int64_t)t.h * sx.sh +
+                                          ((int64_t)t.c * kTileRows + RPL * grp) * sx.sl + t.col0,
+                                sx.sl, nrows, cok, lane);
+    float a[RPL];
+    tile_decays<RPL>(a, A + (int64_t)t.b * sa.sb + (int64_t)t.h * sa.sh +
+                            ((int64_t)t.c * kTileRows + RPL * grp) * sa.sl,
+                     sa.sl, nrows);
+    // 1. local pass
+    float s[CPL];
+    float D = 1.f;
+#pragma unroll
+    for (int e = 0; e < CPL; ++e) s[e] = 0.f;
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+      D *= a[i];
+#pragma unroll
+      for (int e = 0; e < CPL; ++e) s[e] = fmaf(a[i], s[e], row_get<T, NW>(rows[i], e));
+    }
+#pragma unroll
+    for (int e = 0; e < CPL; ++e) sS[buf][grp][lane * CPL + e] = s[e];
+    if (lane == 0) sD[buf][grp] = D;
+    rows_opaque<NW, RPL>(rows);
+    __syncthreads();
+    EMA_TSTAMP(1);
+
+    // 2. tile aggregate, look-back, states entering the row groups (one thread per column)
+    if (threadIdx.x < BN) {
+      const int k = threadIdx.x;
+      u64* st = status + (int64_t)t.col_id * C * BN;
+      float loc = 0.f, dec = 1.f;
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const float d = sD[buf][g];
+        loc = fmaf(d, loc, sS[buf][g][k]);
+        dec *= d;
+      }
+      float p_in = 0.f;
+      if (t.c > 0) {
+        chain_publish(st + (int64_t)t.c * BN + k, kFlagAggregate, loc);
+        p_in = tile_look<false, BN>(st, cs + (int64_t)t.n * C * kTileRows, t.c, C, k, err);
+      }
+      const float p_out = fmaf(dec, p_in, loc);
+      chain_publish(st + (int64_t)t.c * BN + k, kFlagPrefix, p_out);
+      if (t.col0 + k < Tdim) {
+        prev[(int64_t)t.chunk_id * Tdim + t.col0 + k] = p_in;
+        if (prev_coarse && t.c % ratio == 0)
+          prev_coarse[((int64_t)t.n * ((C + ratio - 1) / ratio) + t.c / ratio) * Tdim + t.col0 + k] = p_in;
+        if (t.c == C - 1) final_state[(int64_t)t.n * Tdim + t.col0 + k] = p_out;
+      }
+      float E = p_in;
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const float sg = sS[buf][g][k];
+        sS[buf][g][k] = E;
+        E = fmaf(sD[buf][g], E, sg);
+      }
+    }
+    if (threadIdx.x == 0) s_ticket[slot] = future;
+    __syncthreads();
+    EMA_TSTAMP(2);
+
+    // 3. final pass from the true state
+#pragma unroll
+    for (int e = 0; e < CPL; ++e) s[e] = sS[buf][grp][lane * CPL + e];
+    {
+      T* g = y + (int64_t)t.b * sy.sb + (int64_t)t.h * sy.sh +
+             ((int64_t)t.c * kTileRows + RPL * grp) * sy.sl + t.col0;
+      const unsigned off = (unsigned)lane * CPL;
+#pragma unroll
+      for (int i = 0; i < RPL; ++i) {
+#pragma unroll
+        for (int e = 0; e < CPL; ++e) s[e] = fmaf(a[i], s[e], row_get<T, NW>(rows[i], e));
+        if (i < nrows && cok) row_store<NW>(g + (int64_t)i * sy.sl + off, row_pack<T, CPL, NW>(s));
+      }
+    }
+    EMA_TSTAMP(3);
+    cur = s_ticket[slot];
+    slot ^= 1;
+    buf ^= 1;
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// Backward.  prev[n,c,:] (states entering each 128-row chunk, from the forward) is an input;
+// the reverse state entering each tile from the rows after it, H = a[next row] * dx[next row],
+// comes from the chained scan over dy, last chunk first.  Writes dx, optionally y, and the
+// column partials part[(chunk*ntiles + ctile)*128 + m] = a[m] * <dx[m], y[m-1]> over the
+// tile's columns.  counters[1] ticket, counters[3] error word.
+// ------------------------------------------------------------------------------------
+template <typename T, int CPL, int RPL, int MINW, bool WRITE_Y>
+__global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
+    const T* __restrict__ x, SeqStrides sx, const T* __restrict__ dy, SeqStrides sd,
+    const float* __restrict__ A, SeqStrides sa, const float* __restrict__ cs,
+    const float* __restrict__ prev, T* __restrict__ dx, SeqStrides sdx, T* __restrict__ y,
+    SeqStrides sy, float* __restrict__ part, u64* __restrict__ status,
+    unsigned* __restrict__ counters, int nh, int L, int Tdim, int C, int ntiles, int cols, int total) {
+  using W = TileCfg<T, CPL, RPL>;
+  constexpr int BN = W::BN, NW = W::NW, NG = W::NG;
+  __shared__ __attribute__((aligned(16))) float sS[2][NG][BN];  // forward group states
+  __shared__ __attribute__((aligned(16))) float sR[2][NG][BN];  // reverse group states
+  __shared__ float sD[2][NG];
+  __shared__ int s_ticket[2];
+  const int lane = threadIdx.x & 63;
+  const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  unsigned* err = counters + 3;
+
+  if (threadIdx.x == 0) s_ticket[0] = (int)atomicAdd(counters + 1, 1u);
+  __syncthreads();
+  int cur = s_ticket[0], buf = 0, slot = 1;
+  while (cur < total) {
+    int future = 0;
+    if (threadIdx.x == 0) future = (int)atomicAdd(counters + 1, 1u);
+    const ChainTile t = chain_decode<true, BN>(cur, cols, ntiles, C, nh, L);
+    const bool cok = t.col0 + lane * CPL < Tdim;
+    const int nrows = t.limit - RPL * grp;
+    EMA_TSTAMP(0);
+    RowWords<NW> dr[RPL], xr[RPL];
+    const int64_t row0 = (int64_t)t.c * kTileRows + RPL * grp;
+    tile_load_rows<T, CPL, RPL>(dr, dy + (int64_t)t.b * sd.sb + (int64_t)t.h * sd.sh + row0 * sd.sl + t.col0,
+                                sd.sl, nrows, cok, lane);
+    tile_load_rows<T, CPL, RPL>(xr, x + (int64_t)t.b * sx.sb + (int64_t)t.h * sx.sh + row0 * sx.sl + t.col0,
+                                sx.sl, nrows, cok, lane);
+    float p_in = 0.f;
+    if (threadIdx.x < BN && t.col0 + (int)threadIdx.x < Tdim)
+      p_in = prev[(int64_t)t.chunk_id * Tdim + t.col0 + threadIdx.x];
+    float a[RPL];
+    tile_decays<RPL>(a, A + (int64_t)t.b * sa.sb + (int64_t)t.h * sa.sh + row0 * sa.sl, sa.sl, nrows);
+
+    // 1a. local reverse pass over dy, r = a[i] * dx_local[i]; at the end the state that the
+    // group hands to the rows before it
+    float r[CPL], s[CPL];
+    float D = 1.f;
+#pragma unroll
+    for (int e = 0; e < CPL; ++e) r[e] = 0.f, s[e] = 0.f;
+#pragma unroll
+    for (int i = RPL - 1; i >= 0; --i) {
+      D *= a[i];
+#pragma unroll
+      for (int e = 0; e < CPL; ++e) r[e] = a[i] * (row_get<T, NW>(dr[i], e) + r[e]);
+    }
+    // 1b. local forward pass over x
+#pragma unroll
+    for (int i = 0; i < RPL; ++i)
+#pragma unroll
+      for (int e = 0; e < CPL; ++e) s[e] = fmaf(a[i], s[e], row_get<T, NW>(xr[i], e));
+#pragma unroll
+    for (int e = 0; e < CPL; ++e) {
+      sR[buf][grp][lane * CPL + e] = r[e];
+      sS[buf][grp][lane * CPL + e] = s[e];
+    }
+    if (lane == 0) sD[buf][grp] = D;
+    rows_opaque<NW, RPL>(dr);
+    rows_opaque<NW, RPL>(xr);
+    __syncthreads();
+    EMA_TSTAMP(1);
+
+    // 2a. publish the reverse aggregate; forward states entering the row groups
+    u64* st = status + (int64_t)t.col_id * C * BN;
+    float loc = 0.f, dec = 1.f;
+    if (threadIdx.x < BN) {
+      const int k = threadIdx.x;
+#pragma unroll
+      for (int g = NG - 1; g >= 0; --g) {
+        const float d = sD[buf][g];
+        loc = fmaf(d, loc, sR[buf][g][k]);
+        dec *= d;
+      }
+      if (t.c < C - 1) chain_publish(st + (int64_t)t.c * BN + k, kFlagAggregate, loc);
+      float E = p_in;
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const float sg = sS[buf][g][k];
+        sS[buf][g][k] = E;
+        E = fmaf(sD[buf][g], E, sg);
+      }
+    }
+    __syncthreads();
+    EMA_TSTAMP(2);
+
+    // 2b. look-back for the reverse state (the waves that own no column go straight on)
+    if (threadIdx.x < BN) {
+      const int k = threadIdx.x;
+      float h_in = 0.f;
+      if (t.c < C - 1) h_in = tile_look<true, BN>(st, cs + (int64_t)t.n * C * kTileRows, t.c, C, k, err);
+      chain_publish(st + (int64_t)t.c * BN + k, kFlagPrefix, fmaf(dec, h_in, loc));
+      float G = h_in;
+#pragma unroll
+      for (int g = NG - 1; g >= 0; --g) {
+        const float rg = sR[buf][g][k];
+        sR[buf][g][k] = G;
+        G = fmaf(sD[buf][g], G, rg);
+      }
+    }
+
+    // 1c. forward values y from the true state (kept in float32 for the dots)
+    float E[CPL];
+#pragma unroll
+    for (int e = 0; e < CPL; ++e) E[e] = sS[buf][grp][lane * CPL + e];
+    float yv[RPL][CPL];
+    {
+      T* g = WRITE_Y ? y + (int64_t)t.b * sy.sb + (int64_t)t.h * sy.sh + row0 * sy.sl + t.col0 : nullptr;
+      const unsigned off = (unsigned)lane * CPL;
+#pragma unroll
+      for (int e = 0; e < CPL; ++e) s[e] = E[e];
+#pragma unroll
+      for (int i = 0; i < RPL; ++i) {
+#pragma unroll
+        for (int e = 0; e < CPL; ++e) {
+          s[e] = fmaf(a[i], s[e], row_get<T, NW>(xr[i], e));
+          yv[i][e] = s[e];
+        }
+        if (WRITE_Y && i < nrows && cok) row_store<NW>(g + (int64_t)i * sy.sl + off, row_pack<T, CPL, NW>(s));
+      }
+    }
+    if (threadIdx.x == 0) s_ticket[slot] = future;
+    __syncthreads();
+    EMA_TSTAMP(3);
+
+    // 3. final reverse pass: dx, and the dots with the row before
+    {
+      T* g = dx + (int64_t)t.b * sdx.sb + (int64_t)t.h * sdx.sh + row0 * sdx.sl + t.col0;
+      const unsigned off = (unsigned)lane * CPL;
+      float dA = 0.f;  // lane i reports row i of the wave
+#pragma unroll
+      for (int e = 0; e < CPL; ++e) r[e] = sR[buf][grp][lane * CPL + e];
+#pragma unroll
+      for (int i = RPL - 1; i >= 0; --i) {
+        float dot = 0.f;
+#pragma unroll
+        for (int e = 0; e < CPL; ++e) {
+          // r holds a[i+1] * dx[i+1] on entry (the carried state for the last row)
+          const float d = row_get<T, NW>(dr[i], e) + r[e];
+          dot = fmaf(d, i > 0 ? yv[i - 1][e] : E[e], dot);
+          r[e] = d;
+        }
+        if (i < nrows && cok) row_store<NW>(g + (int64_t)i * sdx.sl + off, row_pack<T, CPL, NW>(r));
+#pragma unroll
+        for (int e = 0; e < CPL; ++e) r[e] *= a[i];
+        dot = a[i] * wave_sum(dot);
+        if (lane == i) dA = dot;
+      }
+      if (lane < RPL)
+        part[((int64_t)t.chunk_id * ntiles + t.ctile) * kTileRows + RPL * grp + lane] = lane < nrows ? dA : 0.f;
+    }
+    EMA_TSTAMP(4);
+    cur = s_ticket[slot];
+    slot ^= 1;
+    buf ^= 1;
+  }
+}
+
+}  // namespace ema
