@@ -27,7 +27,7 @@ for p in (ROOT, os.path.join(ROOT, "triton-kernels_amd")):
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), scaled by
 # what the same counters read for a plain 268 435 456-byte device copy (FETCH_SIZE reads
 # 131 085 KiB for it, factor 1.99982; WRITE_SIZE reads 262 144 KiB, factor 1).
-TRAFFIC_BYTES = {"fwd_single_pass": 573698918, "bwd_single_pass": 875653612}
+TRAFFIC_BYTES = {"fwd_single_pass": 591160982, "bwd_single_pass": 841346755}
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
@@ -216,13 +216,15 @@ def main():
     main = {}
     ms = kernel_ms(lambda i, ev: _ema_matmul_scan_combined_fwd(
         sets[i % len(sets)][1].detach(), sets[i % len(sets)][0].detach(), Q, kernel_events=ev))
-    b = 2 * x_bytes + small
-    main["fwd_single_pass"] = {"ms": ms, "bytes": b, "GBps": b / ms / 1e6, "hbm_frac": b / ms / 1e6 / HBM_PEAK_GBS}
+    nbytes = 2 * x_bytes + small
+    main["fwd_single_pass"] = {"ms": ms, "bytes": nbytes, "GBps": nbytes / ms / 1e6,
+                               "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBS}
     ms = kernel_ms(lambda i, ev: _ema_chunk_scan_combined_bwd(
         sets[i % len(sets)][2], sets[i % len(sets)][0].detach(), sets[i % len(sets)][1].detach(), Q,
         prev128=saved[i % len(sets)], kernel_events=ev))
-    b = 3 * x_bytes + small + N * (-(-L // 128)) * 128 * 4 * (T // 128)
-    main["bwd_single_pass"] = {"ms": ms, "bytes": b, "GBps": b / ms / 1e6, "hbm_frac": b / ms / 1e6 / HBM_PEAK_GBS}
+    nbytes = 3 * x_bytes + small + N * L * 4  # x, dy, dx, cs, chunk-entry states, dA
+    main["bwd_single_pass"] = {"ms": ms, "bytes": nbytes, "GBps": nbytes / ms / 1e6,
+                               "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBS}
 
     kernels = {}
     if not args.no_kernels:

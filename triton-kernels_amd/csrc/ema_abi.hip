@@ -2,6 +2,7 @@
 // reference launcher each entry point replaces are in include/ema_hip.h.
 #include "../../include/ema_hip.h"
 
+#include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 
 #include "ema_device.h"
@@ -256,6 +257,19 @@ inline int record_event(void* ev, hipStream_t st) {
   return hipEventRecord(reinterpret_cast<hipEvent_t>(ev), st) == hipSuccess ? EMA_OK : EMA_ERR_LAUNCH;
 }
 
+// Launches a kernel that uses no dynamic LDS.  With events (hipEvent_t, either may be NULL) the
+// runtime stamps them with the start and the end of this very dispatch, so their difference is
+// the kernel's own duration, free of the gaps around it.
+template <typename... Args>
+void launch_timed(void (*kernel)(Args...), dim3 grid, dim3 block, hipStream_t st, void* ev0, void* ev1,
+                  Args... args) {
+  if (ev0 || ev1)
+    hipExtLaunchKernelGGL(kernel, grid, block, 0, st, reinterpret_cast<hipEvent_t>(ev0),
+                          reinterpret_cast<hipEvent_t>(ev1), 0, args...);
+  else
+    hipLaunchKernelGGL(kernel, grid, block, 0, st, args...);
+}
+
 // Workgroups of a persistent kernel that can be resident at once on the current device.
 template <typename K>
 int resident_blocks(K kernel, int threads, int smem) {
@@ -371,12 +385,10 @@ int launch_fwd_tile_t(const void* x, SeqStrides sx, const float* A, SeqStrides s
   EMA_TRY(launch_chain_init(w, total * BN, st));
   auto kernel = fwd_tile_kernel<T, S::FWD_CPL, S::RPL, S::FWD_MINW>;
   const int64_t cap = resident_blocks(kernel, NT, 0);
-  EMA_TRY(record_event(ev0, st));
-  hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), 0, st, (const T*)x, sx, A,
-                     sa, cs128, (T*)y, sy, prev128, prev_coarse, ratio, fin, w.status, w.counters,
-                     (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total);
-  EMA_TRY(launched());
-  return record_event(ev1, st);
+  launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx, A,
+               sa, cs128, (T*)y, sy, prev128, prev_coarse, ratio, fin, w.status, w.counters,
+               (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total);
+  return launched();
 }
 
 template <typename T, typename S>
@@ -390,24 +402,20 @@ int launch_bwd_tile_t(const void* x, SeqStrides sx, const void* dy, SeqStrides s
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
   EMA_TRY(launch_chain_init(w, total * BN, st));
-  EMA_TRY(record_event(ev0, st));
   if (y) {
     auto kernel = bwd_tile_kernel<T, S::BWD_CPL, S::RPL, S::BWD_MINW, true>;
     const int64_t cap = resident_blocks(kernel, NT, 0);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), 0, st, (const T*)x, sx,
-                       (const T*)dy, sd, A, sa, cs128, prev128, (T*)dx, sdx, (T*)y, sy, part, w.status,
-                       w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols,
-                       (int)total);
+    launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx,
+                 (const T*)dy, sd, A, sa, cs128, prev128, (T*)dx, sdx, (T*)y, sy, part, w.status,
+                 w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total);
   } else {
     auto kernel = bwd_tile_kernel<T, S::BWD_CPL, S::RPL, S::BWD_MINW, false>;
     const int64_t cap = resident_blocks(kernel, NT, 0);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), 0, st, (const T*)x, sx,
-                       (const T*)dy, sd, A, sa, cs128, prev128, (T*)dx, sdx, (T*)nullptr, sy, part,
-                       w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles,
-                       (int)cols, (int)total);
+    launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx,
+                 (const T*)dy, sd, A, sa, cs128, prev128, (T*)dx, sdx, (T*)nullptr, sy, part, w.status,
+                 w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total);
   }
-  EMA_TRY(launched());
-  return record_event(ev1, st);
+  return launched();
 }
 
 template <typename S>
