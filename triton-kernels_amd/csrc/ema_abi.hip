@@ -140,15 +140,6 @@ int allow_smem(K kernel, int bytes) {
 constexpr int kWalkBnBf16 = 128;  // column tile of the per-stage intra-chunk kernels, bf16
 constexpr int kWalkBnF32 = 64;    // and f32 (both are 256 bytes per row)
 
-// Shape of the chained single-pass kernels: column tile, threads, minimum waves per SIMD the
-// register allocation must allow.
-struct ChainBf16 {
-  static constexpr int BN = 128, NT = 256, FWD_MINW = 3, BWD_MINW = 2;
-};
-struct ChainF32 {
-  static constexpr int BN = 64, NT = 512, FWD_MINW = 4, BWD_MINW = 2;
-};
-
 template <typename T, int BN, bool REVERSE>
 int launch_chunk_scan_t(const void* in, SeqStrides si, const float* cs, const float* vec, void* out,
                         SeqStrides so, const Dims& d, hipStream_t st) {
@@ -308,61 +299,6 @@ int launch_chain_init(const ChainWs& w, int64_t words, hipStream_t st) {
   return launched();
 }
 
-template <typename T, typename S>
-int launch_fwd_chained_t(const void* x, SeqStrides sx, const float* cs128, void* y, SeqStrides sy,
-                         float* prev128, float* prev_coarse, int ratio, float* fin, const ChainWs& w,
-                         const Dims& di, hipStream_t st, void* ev0, void* ev1) {
-  constexpr int BN = S::BN, NT = S::NT;
-  const int ntiles = (int)((di.T + BN - 1) / BN);
-  const int64_t cols = di.N * ntiles, total = cols * di.C;
-  if (total > 0x7fffffff) return EMA_ERR_SHAPE;
-  EMA_TRY(launch_chain_init(w, total * BN, st));
-  const int smem = WalkCfg<T, BN>::smem_bytes(1, 1);
-  auto kernel = fwd_chained_kernel<T, BN, NT, S::FWD_MINW, true>;
-  EMA_TRY(allow_smem(kernel, smem));
-  const int64_t cap = resident_blocks(kernel, NT, smem);
-  const unsigned grid = (unsigned)(total < cap ? total : cap);
-  EMA_TRY(record_event(ev0, st));
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), smem, st, (const T*)x, sx, cs128, (T*)y, sy, prev128,
-                     prev_coarse, ratio, fin, w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T,
-                     (int)di.C, ntiles, (int)cols, (int)total);
-  EMA_TRY(launched());
-  return record_event(ev1, st);
-}
-
-template <typename T, typename S>
-int launch_bwd_chained_t(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* cs128,
-                         const float* prev128, void* dx, SeqStrides sdx, void* y, SeqStrides sy,
-                         float* part, const ChainWs& w, const Dims& di, hipStream_t st, void* ev0,
-                         void* ev1) {
-  constexpr int BN = S::BN, NT = S::NT;
-  const int ntiles = (int)((di.T + BN - 1) / BN);
-  const int64_t cols = di.N * ntiles, total = cols * di.C;
-  if (total > 0x7fffffff) return EMA_ERR_SHAPE;
-  EMA_TRY(launch_chain_init(w, total * BN, st));
-  const int smem = WalkCfg<T, BN>::smem_bytes(2, 2);
-  EMA_TRY(record_event(ev0, st));
-  if (y) {
-    auto kernel = bwd_chained_kernel<T, BN, NT, S::BWD_MINW, true>;
-    EMA_TRY(allow_smem(kernel, smem));
-    const int64_t cap = resident_blocks(kernel, NT, smem);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), smem, st,
-                       (const T*)x, sx, (const T*)dy, sd, cs128, prev128, (T*)dx, sdx, (T*)y, sy, part,
-                       w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles,
-                       (int)cols, (int)total);
-  } else {
-    auto kernel = bwd_chained_kernel<T, BN, NT, S::BWD_MINW, false>;
-    EMA_TRY(allow_smem(kernel, smem));
-    const int64_t cap = resident_blocks(kernel, NT, smem);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), smem, st,
-                       (const T*)x, sx, (const T*)dy, sd, cs128, prev128, (T*)dx, sdx, (T*)nullptr, sy,
-                       part, w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles,
-                       (int)cols, (int)total);
-  }
-  EMA_TRY(launched());
-  return record_event(ev1, st);
-}
-
 // Shape of the register-tile single-pass kernels: columns per lane (a tile is 128 rows by
 // 64 times that many columns), rows per lane (128 / RPL waves per workgroup), waves per SIMD
 // the register allocation must allow.
@@ -421,12 +357,6 @@ int launch_bwd_tile_t(const void* x, SeqStrides sx, const void* dy, SeqStrides s
 template <typename S>
 constexpr int tile_parts_per_dim(int64_t T) {
   return (int)((T + 64 * S::BWD_CPL - 1) / (64 * S::BWD_CPL));
-}
-
-// Column partials of ddA that the chained backward writes per (n, chunk, row).
-template <typename S>
-constexpr int chain_parts_per_dim(int64_t T) {
-  return (int)((T + S::BN - 1) / S::BN) * (S::NT / 256);
 }
 
 // dx, optionally the recomputed y, and the log-decay gradient in one pass over x and dy.
