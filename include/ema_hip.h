@@ -50,6 +50,12 @@ typedef enum {
 
 typedef enum { EMA_F32 = 0, EMA_BF16 = 1 } ema_dtype;
 
+/* How the per-position coefficient of the sequence-level entry points is given. */
+typedef enum {
+  EMA_FORM_LOG_DECAY = 0,  /* A:  y[t] = exp(min(A[t], 0)) * y[t-1] + x[t]           */
+  EMA_FORM_PROBABILITY = 1 /* p:  y[t] = (1 - p[t]) * y[t-1] + p[t] * x[t]           */
+} ema_form;
+
 /* Largest chunk size accepted by every entry point. */
 #define EMA_MAX_CHUNK 1024
 
@@ -215,6 +221,50 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
             int64_t y_sl, int64_t y_sh, void* workspace, size_t workspace_bytes, int64_t batch,
             int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk, void* stream,
             void* ev_start, void* ev_stop);
+
+/* ------------------------------------------------- sequence-level entry points ---- */
+
+/* Bytes of workspace ema_seq_fwd / ema_seq_bwd need. */
+size_t ema_seq_fwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim);
+size_t ema_seq_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim);
+
+/* The whole scan in one pass over x, on the caller's raw tensors, with the elementwise steps
+ * that the reference's callers run as separate passes folded into the loads and stores:
+ *   form = EMA_FORM_LOG_DECAY:   coef = A,  y[t] = exp(min(A[t],0)) * y[t-1] + x[t]
+ *   form = EMA_FORM_PROBABILITY: coef = p,  y[t] = (1-p[t]) * y[t-1] + p[t] * x[t]
+ *     (the reference forms A = log(1-p) and X = p*x in torch first,
+ *      kernels/benchmarks/ema_bench.py:135-136, or runs the three kernels of
+ *      ema_scan_combined, kernels/ema.py:370-375)
+ * coef is float32, addressed like A above.  init (N,T) float32, may be NULL = zero: the state
+ * before the first position, which the reference's launchers reject
+ * (kernels/ema_kernels/ema_state_pass.py:129-130).  final_state (N,T), may be NULL: the state
+ * after the last position.  prev128 (N, ceil(seqlen/128), T) float32, required: the state
+ * entering each 128-row chunk, which ema_seq_bwd takes.  Chunking is internal; there is no
+ * chunk argument.  ev_start / ev_stop as for ema_fwd. */
+int ema_seq_fwd(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t c_sh,
+                const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y,
+                int64_t y_sb, int64_t y_sl, int64_t y_sh, const float* init, float* final_state,
+                float* prev128, void* workspace, size_t workspace_bytes, int64_t batch,
+                int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
+                void* ev_stop);
+
+/* Backward of ema_seq_fwd in one pass over x and dy.  With r the reverse scan of dy,
+ * r[t] = dy[t] + a[t+1] * r[t+1], started from dfinal (N,T) float32 (may be NULL = zero), the
+ * gradient reaching final_state:
+ *   EMA_FORM_LOG_DECAY:   dx[t] = r[t],        dcoef[t] = a[t] * <r[t], y[t-1]>
+ *   EMA_FORM_PROBABILITY: dx[t] = p[t] * r[t], dcoef[t] = <r[t], x[t] - y[t-1]>
+ * (the reference leaves dP = -dA * exp(A) commented out, kernels/tests/ema_bwd/_ema_full_bwd.py:128-130,
+ * and rearranges dA from (b,c,q) to (b,l) in torch, :71).  dcoef is float32 in the layout of
+ * coef, given by its own strides; dinit (N,T) float32, may be NULL, receives a[0] * r[0], the
+ * gradient of init.  prev128 is the forward's output of that name. */
+int ema_seq_bwd(int form, const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh,
+                const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, const float* coef,
+                int64_t c_sb, int64_t c_sl, int64_t c_sh, const float* prev128,
+                const float* dfinal, int dtype, void* dx, int64_t dx_sb, int64_t dx_sl,
+                int64_t dx_sh, float* dcoef, int64_t dc_sb, int64_t dc_sl, int64_t dc_sh,
+                float* dinit, void* workspace, size_t workspace_bytes, int64_t batch,
+                int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
+                void* ev_stop);
 
 #ifdef __cplusplus
 }

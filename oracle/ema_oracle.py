@@ -26,7 +26,10 @@ mathematics fixes: closed forms (constant decay -> geometric sum, A == 0 ->
 cumulative sum), a brute-force pure-Python evaluation on tiny inputs,
 chunk-size invariance, equality of the chunked composition with the sequential
 recurrence, torch.autograd through the sequential loop, and float64 central
-finite differences.  No function is left "parity unpinned".
+finite differences.  The sequence-level forms (probability coefficient, boundary states)
+are pinned the same way: equivalence with the log-decay form under A = log(1 - p),
+X = p * x, closed forms, and float64 autograd / finite differences.  No function is left
+"parity unpinned".
 """
 from __future__ import annotations
 
@@ -113,6 +116,65 @@ def ema_loop_bwd(dy: torch.Tensor, X: torch.Tensor, A: torch.Tensor):
         if t > 0:
             dA[:, t] = a[:, t] * (g * y[:, t - 1]).sum(-1)
     return dX, dA
+
+
+# --------------------------------------------------------------------------------------
+# sequence-level forms: probability coefficient, boundary states
+# --------------------------------------------------------------------------------------
+
+
+def ema_seq_loop(X: torch.Tensor, coef: torch.Tensor, form: str = "log_decay", init=None):
+    """Sequential recurrence from an optional initial state, in either form:
+
+        log_decay:    z_t = exp(min(A_t, 0)) * z_{t-1} + X_t
+                      (clamp as in kernels/ema_kernels/ema_scan_fwd.py:141)
+        probability:  z_t = (1 - p_t) * z_{t-1} + p_t * X_t
+                      (main.py:120-131, kernels/benchmarks/ema_bench.py:53-64)
+
+    X:(N,L,T), coef:(N,L), init:(N,T) or None.  Returns (y:(N,L,T), final:(N,T))."""
+    N, L, T = X.shape
+    if form == "probability":
+        keep, gain = 1.0 - coef, coef
+    else:
+        keep, gain = torch.exp(torch.clamp(coef, max=0.0)), None
+    y = torch.empty_like(X)
+    z = X.new_zeros(N, T) if init is None else init.to(X.dtype).clone()
+    for t in range(L):
+        xin = X[:, t] if gain is None else gain[:, t, None] * X[:, t]
+        z = keep[:, t, None] * z + xin
+        y[:, t] = z
+    return y, z
+
+
+def ema_seq_loop_bwd(dy, X, coef, form="log_decay", init=None, dfinal=None):
+    """Gradients of sum(y * dy) + sum(final * dfinal) for (y, final) = ema_seq_loop(...), by the
+    reverse recurrence r_t = dy_t + keep_{t+1} * r_{t+1} (r_{L-1} = dy_{L-1} + dfinal):
+
+        log_decay:    dX_t = r_t,        dA_t = keep_t * <r_t, y_{t-1}>   (0 where A_t > 0)
+        probability:  dX_t = p_t * r_t,  dp_t = <r_t, X_t - y_{t-1}>
+        dinit = keep_0 * r_0,            y_{-1} = init.
+
+    Returns (dX, dcoef, dinit); tests check it against torch.autograd through ema_seq_loop."""
+    N, L, T = X.shape
+    prob = form == "probability"
+    keep = 1.0 - coef if prob else torch.exp(torch.clamp(coef, max=0.0))
+    y, _ = ema_seq_loop(X, coef, form, init)
+    y_before = X.new_zeros(N, T) if init is None else init.to(X.dtype)
+    dX = torch.empty_like(X)
+    dcoef = coef.new_zeros(N, L)
+    r = X.new_zeros(N, T) if dfinal is None else dfinal.to(X.dtype).clone()
+    for t in range(L - 1, -1, -1):
+        r = dy[:, t] + r  # r now holds keep_{t+1} * r_{t+1} (or dfinal) from the step before
+        yp = y[:, t - 1] if t > 0 else y_before
+        if prob:
+            dX[:, t] = coef[:, t, None] * r
+            dcoef[:, t] = (r * (X[:, t] - yp)).sum(-1)
+        else:
+            dX[:, t] = r
+            dcoef[:, t] = torch.where(coef[:, t] > 0, torch.zeros_like(coef[:, t]),
+                                      keep[:, t] * (r * yp).sum(-1))
+        r = keep[:, t, None] * r
+    return dX, dcoef, r
 
 
 # --------------------------------------------------------------------------------------

@@ -1,0 +1,152 @@
+"""GPU parity of the sequence-level entry points (ema_seq_fwd / ema_seq_bwd through the C ABI)
+against the sequential CPU oracle: both forms of the coefficient, boundary states, flat and
+headed layouts, ragged lengths, and the bench shape through size-independent properties."""
+import pytest
+import torch
+
+from oracle import ema_oracle as O
+from parity_util import announce, check_close
+
+pytestmark = pytest.mark.gpu
+
+F32, BF16 = torch.float32, torch.bfloat16
+
+
+def _case(N, L, T, seed, dtype, form):
+    g = torch.Generator().manual_seed(seed)
+    X = torch.randn(N, L, T, generator=g).to(dtype)
+    u = torch.randn(N, L, generator=g) + 2.0
+    coef = torch.sigmoid(-u) if form == "probability" else torch.nn.functional.logsigmoid(u)
+    init = torch.randn(N, T, generator=g)
+    dy = torch.randn(N, L, T, generator=g).to(dtype)
+    dfinal = torch.randn(N, T, generator=g)
+    return X, coef, init, dy, dfinal
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("form", ["log_decay", "probability"])
+@pytest.mark.parametrize("states", [False, True], ids=["zero_init", "with_states"])
+@pytest.mark.parametrize("N,L,T", [(3, 1000, 264), (2, 128, 8), (2, 129, 512), (1, 1, 16), (4, 2048, 1024)])
+def test_seq_fwd_bwd_vs_oracle(N, L, T, states, form, dtype, device):
+    from kernels.ema_seq import ema_seq_bwd, ema_seq_fwd
+
+    announce(f"seq N{N} L{L} T{T} {form} states={states} {dtype}")
+    X, coef, init, dy, dfinal = _case(N, L, T, 11 + L + T, dtype, form)
+    y, fin, prev128 = ema_seq_fwd(coef.to(device), X.to(device), form, init.to(device) if states else None)
+    dx, dc, dinit = ema_seq_bwd(dy.to(device), X.to(device), coef.to(device), prev128, form,
+                                dfinal_states=dfinal.to(device) if states else None, want_dinit=states)
+    torch.cuda.synchronize()
+    y_ref, fin_ref = O.ema_seq_loop(X.float(), coef, form, init if states else None)
+    dx_ref, dc_ref, dinit_ref = O.ema_seq_loop_bwd(dy.float(), X.float(), coef, form,
+                                                   init if states else None, dfinal if states else None)
+    small = F32 if dtype == F32 else BF16
+    check_close("y", y, y_ref, dtype)
+    check_close("final", fin, fin_ref, small)
+    check_close("dx", dx, dx_ref, dtype)
+    check_close("dcoef", dc, dc_ref, dtype)
+    if states:
+        check_close("dinit", dinit, dinit_ref, small)
+    C = -(-L // 128)
+    y0 = init if states else torch.zeros(N, T)
+    ref_prev = torch.stack([y_ref[:, c * 128 - 1] if c else y0 for c in range(C)], 1)
+    check_close("prev128", prev128, ref_prev, small)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("form", ["log_decay", "probability"])
+def test_seq_autograd_headed(form, dtype, device):
+    """Headed (b, L, nh, d) tensors through the autograd function, with gradients flowing
+    through the final states and into the initial states."""
+    from kernels.ema_seq import ema_seq_scan
+
+    b, nh, L, d = 2, 3, 700, 64
+    announce(f"seq autograd headed b{b} nh{nh} L{L} d{d} {form} {dtype}")
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(b, L, nh, d, generator=g).to(dtype)
+    u = torch.randn(b, L, nh, generator=g) + 2.0
+    coef = torch.sigmoid(-u) if form == "probability" else torch.nn.functional.logsigmoid(u)
+    init = torch.randn(b, nh, d, generator=g)
+    dy = torch.randn(b, L, nh, d, generator=g).to(dtype)
+    dfin = torch.randn(b, nh, d, generator=g)
+    xg, cg, ig = (t.to(device).requires_grad_() for t in (x, coef, init))
+    y, fin = ema_seq_scan(cg, xg, form, initial_states=ig, return_final_states=True)
+    ((y.float() * dy.to(device).float()).sum() + (fin * dfin.to(device)).sum()).backward()
+    torch.cuda.synchronize()
+    xf, cf = O.to_flat(x.float(), coef)
+    dyf, _ = O.to_flat(dy.float(), coef)
+    i2, df2 = init.reshape(b * nh, d), dfin.reshape(b * nh, d)
+    y_ref, fin_ref = O.ema_seq_loop(xf, cf, form, i2)
+    dx_ref, dc_ref, di_ref = O.ema_seq_loop_bwd(dyf, xf, cf, form, i2, df2)
+    small = F32 if dtype == F32 else BF16
+    check_close("y", y, O.from_flat(y_ref, b, nh), dtype)
+    check_close("final", fin, fin_ref.reshape(b, nh, d), small)
+    check_close("dx", xg.grad, O.from_flat(dx_ref, b, nh), dtype)
+    check_close("dcoef", cg.grad, dc_ref.reshape(b, nh, L).permute(0, 2, 1), dtype)
+    check_close("dinit", ig.grad, di_ref.reshape(b, nh, d), small)
+
+
+def test_ema_scan_combined_xp_entry(device):
+    """The (x, p) entry point of the reference's first implementation (kernels/ema.py:370),
+    now one pass and differentiable."""
+    from kernels.ema import ema_scan_combined
+
+    B, L, D = 3, 777, 96
+    announce(f"ema_scan_combined(x, p) B{B} L{L} D{D}")
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(B, L, D, generator=g)
+    p = torch.sigmoid(torch.randn(B, L, 1, generator=g) - 2.0)
+    dy = torch.randn(B, L, D, generator=g)
+    xg, pg = x.to(device).requires_grad_(), p.to(device).requires_grad_()
+    z = ema_scan_combined(xg, pg)
+    z.backward(dy.to(device))
+    torch.cuda.synchronize()
+    z_ref, _ = O.ema_seq_loop(x, p.squeeze(-1), "probability")
+    dx_ref, dp_ref, _ = O.ema_seq_loop_bwd(dy, x, p.squeeze(-1), "probability")
+    check_close("z", z, z_ref, F32)
+    check_close("dx", xg.grad, dx_ref, F32)
+    check_close("dp", pg.grad, dp_ref[..., None], F32)
+
+
+def test_seq_probability_extremes(device):
+    """p = 0 keeps the state, p = 1 replaces it (log(1 - p) = -inf inside the chained scan)."""
+    from kernels.ema_seq import ema_seq_fwd
+
+    N, L, T = 2, 400, 64
+    g = torch.Generator().manual_seed(2)
+    X = torch.randn(N, L, T, generator=g)
+    p = torch.sigmoid(torch.randn(N, L, generator=g))
+    p[:, 100:140] = 0.0
+    p[:, 200] = 1.0
+    p[:, 255:257] = 1.0
+    y, fin, _ = ema_seq_fwd(p.to(device), X.to(device), "probability")
+    torch.cuda.synchronize()
+    y_ref, fin_ref = O.ema_seq_loop(X, p, "probability")
+    check_close("y", y, y_ref, F32)
+    # (equal up to the rounding of the group and tile combination, not bit for bit)
+    assert torch.allclose(y[:, 139].cpu(), y[:, 99].cpu(), rtol=1e-5, atol=1e-6)
+    assert torch.allclose(y[:, 200].cpu(), X[:, 200], rtol=1e-6, atol=1e-6)
+
+
+def test_seq_bench_shape_properties(device):
+    """b16 nh2 d1024 L4096 bf16: the two forms agree under A = log(1 - p), X = p * x, the final
+    state is the last output row, and a split scan (first half, then second half from the first
+    half's final state) equals the whole scan."""
+    from kernels.ema_seq import ema_seq_fwd
+
+    b, nh, L, d = 16, 2, 4096, 1024
+    announce("seq bench shape properties")
+    g = torch.Generator(device="cpu").manual_seed(1128)
+    x = torch.randn(b, L, nh, d, generator=g).to(BF16).to(device)
+    p = torch.sigmoid(-(torch.randn(b, L, nh, generator=g) + 2.0)).to(device)
+    y_p, fin_p, _ = ema_seq_fwd(p, x, "probability")
+    # (p * x) rounded to bf16 costs up to 2^-9 relative per term: compare at the bf16 bar
+    y_a, fin_a, _ = ema_seq_fwd(torch.log1p(-p), (p[..., None] * x.float()).to(BF16), "log_decay")
+    check_close("probability form vs log-decay form", y_p, y_a.float(), BF16)
+    check_close("final is last row", fin_p, y_p[:, -1].float(), BF16)
+    h = 2048 + 128 * 3
+    y1, f1, _ = ema_seq_fwd(p[:, :h], x[:, :h], "probability")
+    y2, f2, _ = ema_seq_fwd(p[:, h:], x[:, h:], "probability", initial_states=f1)
+    torch.cuda.synchronize()
+    check_close("split scan, first part", y1, y_p[:, :h].float(), BF16)
+    check_close("split scan, second part", y2, y_p[:, h:].float(), BF16)
+    check_close("split scan, final", f2, fin_p, BF16)

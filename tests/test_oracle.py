@@ -315,3 +315,104 @@ def test_fp32_oracle_close_to_fp64():
     dx64, dA64 = O.ema_loop_bwd(dyf.double(), xf.double(), Af.double())
     assert torch.allclose(dx32.double(), dx64, rtol=1e-4, atol=1e-5)
     assert torch.allclose(dA32.reshape(2, -1).double(), dA64, rtol=1e-4, atol=1e-4)
+
+
+# ---------------------------------------------------------------- sequence-level forms
+
+
+def _seq_inputs(N=3, L=37, T=5, seed=0, dtype=torch.float64):
+    gen = torch.Generator().manual_seed(seed)
+    X = torch.randn(N, L, T, generator=gen, dtype=dtype)
+    p = torch.sigmoid(torch.randn(N, L, generator=gen, dtype=dtype) - 1.0)
+    init = torch.randn(N, T, generator=gen, dtype=dtype)
+    dy = torch.randn(N, L, T, generator=gen, dtype=dtype)
+    dfinal = torch.randn(N, T, generator=gen, dtype=dtype)
+    return X, p, init, dy, dfinal
+
+
+def test_seq_probability_form_is_log_decay_form_of_scaled_input():
+    # the change of variables the reference's bench applies (ema_bench.py:135-136)
+    X, p, *_ = _seq_inputs()
+    y_p, fin_p = O.ema_seq_loop(X, p, "probability")
+    y_a = O.ema_loop(p[..., None] * X, torch.log1p(-p))
+    assert torch.allclose(y_p, y_a, rtol=1e-12, atol=1e-12)
+    assert torch.allclose(fin_p, y_a[:, -1], rtol=1e-12, atol=1e-12)
+
+
+def test_seq_constant_probability_closed_form():
+    # z_t = sum_k p (1-p)^(t-k) x_k + (1-p)^(t+1) init
+    N, L, T, p0 = 2, 20, 3, 0.3
+    gen = torch.Generator().manual_seed(3)
+    X = torch.randn(N, L, T, generator=gen, dtype=torch.float64)
+    init = torch.randn(N, T, generator=gen, dtype=torch.float64)
+    y, fin = O.ema_seq_loop(X, torch.full((N, L), p0, dtype=torch.float64), "probability", init)
+    for t in (0, 7, L - 1):
+        want = sum(p0 * (1 - p0) ** (t - k) * X[:, k] for k in range(t + 1)) + (1 - p0) ** (t + 1) * init
+        assert torch.allclose(y[:, t], want, rtol=1e-12, atol=1e-12)
+    assert torch.equal(fin, y[:, -1])
+
+
+def test_seq_initial_state_is_an_extra_first_row():
+    # a scan from state s equals the scan of [s, x_0, x_1, ...] from zero, first output dropped
+    X, p, init, *_ = _seq_inputs()
+    A = torch.log1p(-p)
+    y, _ = O.ema_seq_loop(X, A, "log_decay", init)
+    Xe = torch.cat([init[:, None], X], 1)
+    Ae = torch.cat([torch.zeros_like(A[:, :1]), A], 1)
+    assert torch.allclose(y, O.ema_loop(Xe, Ae)[:, 1:], rtol=1e-12, atol=1e-12)
+
+
+def test_seq_log_decay_clamps_positive_values():
+    X, p, *_ = _seq_inputs()
+    A = torch.log1p(-p)
+    A[:, 5] = 0.7
+    y, _ = O.ema_seq_loop(X, A, "log_decay")
+    A0 = A.clone()
+    A0[:, 5] = 0.0
+    assert torch.equal(y, O.ema_seq_loop(X, A0, "log_decay")[0])
+
+
+@pytest.mark.parametrize("form", ["log_decay", "probability"])
+@pytest.mark.parametrize("with_states", [False, True])
+def test_seq_bwd_matches_autograd(form, with_states):
+    X, p, init, dy, dfinal = _seq_inputs()
+    coef = p if form == "probability" else torch.log1p(-p)
+    Xr, cr = X.clone().requires_grad_(), coef.clone().requires_grad_()
+    ir = init.clone().requires_grad_() if with_states else None
+    y, fin = O.ema_seq_loop(Xr, cr, form, ir)
+    loss = (y * dy).sum() + ((fin * dfinal).sum() if with_states else 0.0)
+    loss.backward()
+    dX, dc, dinit = O.ema_seq_loop_bwd(dy, X, coef, form, init if with_states else None,
+                                       dfinal if with_states else None)
+    assert torch.allclose(dX, Xr.grad, rtol=1e-10, atol=1e-10)
+    assert torch.allclose(dc, cr.grad, rtol=1e-10, atol=1e-10)
+    if with_states:
+        assert torch.allclose(dinit, ir.grad, rtol=1e-10, atol=1e-10)
+
+
+def test_seq_bwd_finite_differences_probability():
+    X, p, init, dy, dfinal = _seq_inputs(N=1, L=9, T=2)
+    _, dp, dinit = O.ema_seq_loop_bwd(dy, X, p, "probability", init, dfinal)
+
+    def loss(pp, ii):
+        y, fin = O.ema_seq_loop(X, pp, "probability", ii)
+        return float((y * dy).sum() + (fin * dfinal).sum())
+
+    eps = 1e-6
+    for t in (0, 4, 8):
+        d = torch.zeros_like(p)
+        d[0, t] = eps
+        assert math.isclose((loss(p + d, init) - loss(p - d, init)) / (2 * eps), float(dp[0, t]), rel_tol=1e-6, abs_tol=1e-8)
+    d = torch.zeros_like(init)
+    d[0, 1] = eps
+    assert math.isclose((loss(p, init + d) - loss(p, init - d)) / (2 * eps), float(dinit[0, 1]), rel_tol=1e-6, abs_tol=1e-8)
+
+
+def test_seq_probability_gradient_is_chain_rule_of_log_decay_gradient():
+    # dp = <dX_scaled, x> - dA / (1 - p): the relation the reference leaves commented out
+    # (kernels/tests/ema_bwd/_ema_full_bwd.py:128-130) plus the input-scaling term
+    X, p, _, dy, _ = _seq_inputs()
+    dXs, dA = O.ema_loop_bwd(dy, p[..., None] * X, torch.log1p(-p))
+    _, dp, _ = O.ema_seq_loop_bwd(dy, X, p, "probability")
+    want = (dXs * X).sum(-1) - dA / (1 - p)
+    assert torch.allclose(dp, want, rtol=1e-10, atol=1e-10)

@@ -69,11 +69,12 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
 
 // ---------------------------------------------------------------- launch helpers
 
-int launch_cumsum(const float* A, SeqStrides sa, float* cs, const Dims& d, hipStream_t st) {
+// prob = 1: the input holds probabilities p and the sums are of log(1 - p).
+int launch_cumsum(const float* A, SeqStrides sa, float* cs, const Dims& d, hipStream_t st, int prob = 0) {
   const int64_t total = d.N * d.C;
   const unsigned grid = (unsigned)((total + 3) / 4);
   hipLaunchKernelGGL(cumsum_kernel, dim3(grid), dim3(256), 0, st, A, sa, cs, (int)d.nh, (int)d.L,
-                     (int)d.Q, (int)d.C, total);
+                     (int)d.Q, (int)d.C, total, prob);
   return launched();
 }
 
@@ -275,27 +276,31 @@ int resident_blocks(K kernel, int threads, int smem) {
 
 inline int64_t padded_dim(int64_t T) { return (T + 255) / 256 * 256; }
 
-// status words + counters of one chained kernel
+// status words + counters of one chained kernel: C tile slots and one virtual slot per column
 struct ChainWs {
   u64* status;
   unsigned* counters;
 };
-inline size_t chain_ws_bytes(const Dims& di) {
-  return align_up((size_t)(di.N * di.C * padded_dim(di.T)) * sizeof(u64), 256) + 256;
+inline size_t chain_status_bytes(const Dims& di) {
+  return align_up((size_t)(di.N * (di.C + 1) * padded_dim(di.T)) * sizeof(u64), 256);
 }
+inline size_t chain_ws_bytes(const Dims& di) { return chain_status_bytes(di) + 256; }
 inline ChainWs chain_carve(void* base, const Dims& di) {
   ChainWs w;
   w.status = static_cast<u64*>(base);
-  w.counters = reinterpret_cast<unsigned*>(
-      static_cast<char*>(base) + align_up((size_t)(di.N * di.C * padded_dim(di.T)) * sizeof(u64), 256));
+  w.counters = reinterpret_cast<unsigned*>(static_cast<char*>(base) + chain_status_bytes(di));
   return w;
 }
 
-int launch_chain_init(const ChainWs& w, int64_t words, hipStream_t st) {
-  const int64_t n16 = (words * (int64_t)sizeof(u64) + 15) / 16;
-  const int64_t threads = n16 > 4 ? n16 : 4;
+// Clears the words of cols column sets of BN columns; the virtual slot (0 forward, C reverse)
+// carries `seed` (N, T), or 0.
+int launch_chain_init(const ChainWs& w, int64_t cols, int BN, const Dims& di, bool reverse,
+                      const float* seed, int ntiles, hipStream_t st) {
+  const int64_t pairs = cols * (di.C + 1) * BN / 2;
+  const int64_t threads = pairs > 4 ? pairs : 4;
   hipLaunchKernelGGL(chain_init_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st,
-                     reinterpret_cast<uint4*>(w.status), n16, w.counters);
+                     reinterpret_cast<uint4*>(w.status), pairs, w.counters, BN, (int)di.C + 1,
+                     reverse ? (int)di.C : 0, ntiles, (int)di.T, seed);
   return launched();
 }
 
@@ -309,49 +314,55 @@ struct TileF32 {
   static constexpr int FWD_CPL = 2, BWD_CPL = 2, RPL = 8, FWD_MINW = 8, BWD_MINW = 4;
 };
 
-template <typename T, typename S>
+template <typename T, typename S, bool XP>
 int launch_fwd_tile_t(const void* x, SeqStrides sx, const float* A, SeqStrides sa, const float* cs128,
                       void* y, SeqStrides sy, float* prev128, float* prev_coarse, int ratio, float* fin,
-                      const ChainWs& w, const Dims& di, hipStream_t st, void* ev0, void* ev1) {
+                      const float* init, const ChainWs& w, const Dims& di, hipStream_t st, void* ev0,
+                      void* ev1) {
   using Cfg = TileCfg<T, S::FWD_CPL, S::RPL>;
   constexpr int BN = Cfg::BN, NT = Cfg::NT;
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
-  EMA_TRY(launch_chain_init(w, total * BN, st));
-  auto kernel = fwd_tile_kernel<T, S::FWD_CPL, S::RPL, S::FWD_MINW>;
+  EMA_TRY(launch_chain_init(w, cols, BN, di, false, init, ntiles, st));
+  auto kernel = fwd_tile_kernel<T, S::FWD_CPL, S::RPL, S::FWD_MINW, XP>;
   const int64_t cap = resident_blocks(kernel, NT, 0);
   launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx, A,
-               sa, cs128, (T*)y, sy, prev128, prev_coarse, ratio, fin, w.status, w.counters,
+               sa, cs128, (T*)y, sy, prev128, prev_coarse, ratio, fin, init ? 1 : 0, w.status, w.counters,
                (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total);
   return launched();
 }
 
-template <typename T, typename S>
-int launch_bwd_tile_t(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* A,
+template <typename T, typename S, bool WRITE_Y, bool XP>
+int launch_bwd_tile_k(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* A,
                       SeqStrides sa, const float* cs128, const float* prev128, void* dx, SeqStrides sdx,
-                      void* y, SeqStrides sy, float* part, const ChainWs& w, const Dims& di,
-                      hipStream_t st, void* ev0, void* ev1) {
+                      void* y, SeqStrides sy, float* part, const float* dfinal, float* dinit,
+                      const ChainWs& w, const Dims& di, hipStream_t st, void* ev0, void* ev1) {
   using Cfg = TileCfg<T, S::BWD_CPL, S::RPL>;
   constexpr int BN = Cfg::BN, NT = Cfg::NT;
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
-  EMA_TRY(launch_chain_init(w, total * BN, st));
-  if (y) {
-    auto kernel = bwd_tile_kernel<T, S::BWD_CPL, S::RPL, S::BWD_MINW, true>;
-    const int64_t cap = resident_blocks(kernel, NT, 0);
-    launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx,
-                 (const T*)dy, sd, A, sa, cs128, prev128, (T*)dx, sdx, (T*)y, sy, part, w.status,
-                 w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total);
-  } else {
-    auto kernel = bwd_tile_kernel<T, S::BWD_CPL, S::RPL, S::BWD_MINW, false>;
-    const int64_t cap = resident_blocks(kernel, NT, 0);
-    launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx,
-                 (const T*)dy, sd, A, sa, cs128, prev128, (T*)dx, sdx, (T*)nullptr, sy, part, w.status,
-                 w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total);
-  }
+  EMA_TRY(launch_chain_init(w, cols, BN, di, true, dfinal, ntiles, st));
+  auto kernel = bwd_tile_kernel<T, S::BWD_CPL, S::RPL, S::BWD_MINW, WRITE_Y, XP>;
+  const int64_t cap = resident_blocks(kernel, NT, 0);
+  launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx,
+               (const T*)dy, sd, A, sa, cs128, prev128, (T*)dx, sdx, (T*)y, sy, part, dfinal ? 1 : 0, dinit,
+               w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols,
+               (int)total);
   return launched();
+}
+
+template <typename T, typename S, bool XP>
+int launch_bwd_tile_t(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* A,
+                      SeqStrides sa, const float* cs128, const float* prev128, void* dx, SeqStrides sdx,
+                      void* y, SeqStrides sy, float* part, const float* dfinal, float* dinit,
+                      const ChainWs& w, const Dims& di, hipStream_t st, void* ev0, void* ev1) {
+  if (y)
+    return launch_bwd_tile_k<T, S, true, XP>(x, sx, dy, sd, A, sa, cs128, prev128, dx, sdx, y, sy, part,
+                                             dfinal, dinit, w, di, st, ev0, ev1);
+  return launch_bwd_tile_k<T, S, false, XP>(x, sx, dy, sd, A, sa, cs128, prev128, dx, sdx, nullptr, sy, part,
+                                            dfinal, dinit, w, di, st, ev0, ev1);
 }
 
 template <typename S>
@@ -506,11 +517,12 @@ int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void
     float* p128 = prev128 ? prev128 : (ratio == 1 ? prev : w.prev128);
     float* coarse = p128 == prev ? nullptr : prev;
     if (dtype == EMA_BF16) {
-      return launch_fwd_tile_t<bf16_t, TileBf16>(x, sx, A, sa, cs128, y, sy, p128, coarse, ratio,
-                                                 final_state, w.chain, di, st, ev_start, ev_stop);
+      return launch_fwd_tile_t<bf16_t, TileBf16, false>(x, sx, A, sa, cs128, y, sy, p128, coarse, ratio,
+                                                        final_state, nullptr, w.chain, di, st, ev_start,
+                                                        ev_stop);
     }
-    return launch_fwd_tile_t<float, TileF32>(x, sx, A, sa, cs128, y, sy, p128, coarse, ratio,
-                                             final_state, w.chain, di, st, ev_start, ev_stop);
+    return launch_fwd_tile_t<float, TileF32, false>(x, sx, A, sa, cs128, y, sy, p128, coarse, ratio,
+                                                    final_state, nullptr, w.chain, di, st, ev_start, ev_stop);
   }
   if (prev128) return EMA_ERR_UNSUPPORTED;  // only produced when chunk is a multiple of 128
   float* states = static_cast<float*>(workspace);
@@ -700,11 +712,13 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
   // the reverse inter-chunk state is handed over inside the kernel
   int parts = dtype == EMA_BF16 ? tile_parts_per_dim<TileBf16>(di.T) : tile_parts_per_dim<TileF32>(di.T);
   if (dtype == EMA_BF16) {
-    EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16>(x, sx, dy, sd, A, sa, w.cs, prev128, dx, sdx, y, sy, w.part,
-                                                 w.chain, di, st, ev_start, ev_stop)));
+    EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, false>(x, sx, dy, sd, A, sa, w.cs, prev128, dx, sdx, y, sy,
+                                                        w.part, nullptr, nullptr, w.chain, di, st, ev_start,
+                                                        ev_stop)));
   } else
-    EMA_TRY((launch_bwd_tile_t<float, TileF32>(x, sx, dy, sd, A, sa, w.cs, prev128, dx, sdx, y, sy, w.part,
-                                               w.chain, di, st, ev_start, ev_stop)));
+    EMA_TRY((launch_bwd_tile_t<float, TileF32, false>(x, sx, dy, sd, A, sa, w.cs, prev128, dx, sdx, y, sy,
+                                                      w.part, nullptr, nullptr, w.chain, di, st, ev_start,
+                                                      ev_stop)));
   const int64_t total = d.N * d.C * d.Q;
   hipLaunchKernelGGL(dA_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w.part,
                      ddA, (int)d.L, (int)d.Q, (int)d.C, (int)di.C, parts, total);
@@ -740,6 +754,135 @@ int ema_bwd_dx_dA_fused(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
   return run_bwd_fused(x, SeqStrides{x_sb, x_sl, x_sh}, dy, SeqStrides{dy_sb, dy_sl, dy_sh}, dtype, cs,
                        prev, g, dx, SeqStrides{dx_sb, dx_sl, dx_sh}, y, SeqStrides{y_sb, y_sl, y_sh},
                        ddA, static_cast<float*>(workspace), d, d, as_stream(stream));
+}
+
+// ---- sequence-level entry points: either form of the recurrence, optional boundary states
+
+struct SeqWs {
+  float *cs, *part;
+  ChainWs chain;
+  size_t bytes;
+};
+static SeqWs carve_seq(void* base, const Dims& di, bool backward) {
+  SeqWs w;
+  size_t off = 0;
+  char* p = static_cast<char*>(base);
+  auto take = [&](size_t floats) {
+    float* r = reinterpret_cast<float*>(p + off);
+    off += align_up(floats * sizeof(float), 256);
+    return r;
+  };
+  const size_t ncq = (size_t)(di.N * di.C * di.Q);
+  w.cs = take(ncq);
+  w.part = nullptr;
+  if (backward) {
+    const int pb = tile_parts_per_dim<TileBf16>(di.T), pf = tile_parts_per_dim<TileF32>(di.T);
+    w.part = take(ncq * (size_t)(pb > pf ? pb : pf));
+  }
+  w.chain = chain_carve(p + off, di);
+  off += chain_ws_bytes(di);
+  w.bytes = off;
+  return w;
+}
+
+static int check_form(int form) {
+  return (form == EMA_FORM_LOG_DECAY || form == EMA_FORM_PROBABILITY) ? EMA_OK : EMA_ERR_UNSUPPORTED;
+}
+
+size_t ema_seq_fwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim) {
+  Dims d;
+  if (check_dims(batch, nheads, seqlen, dim, kTileRows, true, &d) != EMA_OK) return 0;
+  return carve_seq(nullptr, d, false).bytes;
+}
+
+int ema_seq_fwd(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t c_sh, const void* x,
+                int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb,
+                int64_t y_sl, int64_t y_sh, const float* init, float* final_state, float* prev128,
+                void* workspace, size_t workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen,
+                int64_t dim, void* stream, void* ev_start, void* ev_stop) {
+  Dims d;
+  EMA_TRY(check_form(form));
+  EMA_TRY(check_dims(batch, nheads, seqlen, dim, kTileRows, true, &d));
+  EMA_TRY(check_dtype(dtype));
+  EMA_TRY(check_seq(x, x_sb, x_sl, x_sh, dtype, dim));
+  EMA_TRY(check_seq(y, y_sb, y_sl, y_sh, dtype, dim));
+  if (!coef || !prev128) return EMA_ERR_NULL;
+  EMA_TRY(check_f32(workspace));
+  if (workspace_bytes < ema_seq_fwd_workspace_bytes(batch, nheads, seqlen, dim)) return EMA_ERR_SHAPE;
+  hipStream_t st = as_stream(stream);
+  const SeqWs w = carve_seq(workspace, d, false);
+  const SeqStrides sx{x_sb, x_sl, x_sh}, sy{y_sb, y_sl, y_sh}, sc{c_sb, c_sl, c_sh};
+  const bool xp = form == EMA_FORM_PROBABILITY;
+  EMA_TRY(launch_cumsum(coef, sc, w.cs, d, st, xp ? 1 : 0));
+  if (dtype == EMA_BF16) {
+    if (xp)
+      return launch_fwd_tile_t<bf16_t, TileBf16, true>(x, sx, coef, sc, w.cs, y, sy, prev128, nullptr, 1,
+                                                       final_state, init, w.chain, d, st, ev_start, ev_stop);
+    return launch_fwd_tile_t<bf16_t, TileBf16, false>(x, sx, coef, sc, w.cs, y, sy, prev128, nullptr, 1,
+                                                      final_state, init, w.chain, d, st, ev_start, ev_stop);
+  }
+  if (xp)
+    return launch_fwd_tile_t<float, TileF32, true>(x, sx, coef, sc, w.cs, y, sy, prev128, nullptr, 1,
+                                                   final_state, init, w.chain, d, st, ev_start, ev_stop);
+  return launch_fwd_tile_t<float, TileF32, false>(x, sx, coef, sc, w.cs, y, sy, prev128, nullptr, 1,
+                                                  final_state, init, w.chain, d, st, ev_start, ev_stop);
+}
+
+size_t ema_seq_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim) {
+  Dims d;
+  if (check_dims(batch, nheads, seqlen, dim, kTileRows, true, &d) != EMA_OK) return 0;
+  return carve_seq(nullptr, d, true).bytes;
+}
+
+int ema_seq_bwd(int form, const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const void* x,
+                int64_t x_sb, int64_t x_sl, int64_t x_sh, const float* coef, int64_t c_sb, int64_t c_sl,
+                int64_t c_sh, const float* prev128, const float* dfinal, int dtype, void* dx,
+                int64_t dx_sb, int64_t dx_sl, int64_t dx_sh, float* dcoef, int64_t dc_sb, int64_t dc_sl,
+                int64_t dc_sh, float* dinit, void* workspace, size_t workspace_bytes, int64_t batch,
+                int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
+                void* ev_stop) {
+  Dims d;
+  EMA_TRY(check_form(form));
+  EMA_TRY(check_dims(batch, nheads, seqlen, dim, kTileRows, true, &d));
+  EMA_TRY(check_dtype(dtype));
+  EMA_TRY(check_seq(dy, dy_sb, dy_sl, dy_sh, dtype, dim));
+  EMA_TRY(check_seq(x, x_sb, x_sl, x_sh, dtype, dim));
+  EMA_TRY(check_seq(dx, dx_sb, dx_sl, dx_sh, dtype, dim));
+  if (!coef || !prev128 || !dcoef) return EMA_ERR_NULL;
+  EMA_TRY(check_f32(workspace));
+  if (workspace_bytes < ema_seq_bwd_workspace_bytes(batch, nheads, seqlen, dim)) return EMA_ERR_SHAPE;
+  hipStream_t st = as_stream(stream);
+  const SeqWs w = carve_seq(workspace, d, true);
+  const SeqStrides sx{x_sb, x_sl, x_sh}, sd{dy_sb, dy_sl, dy_sh}, sdx{dx_sb, dx_sl, dx_sh};
+  const SeqStrides sc{c_sb, c_sl, c_sh}, none{0, 0, 0};
+  const bool xp = form == EMA_FORM_PROBABILITY;
+  EMA_TRY(launch_cumsum(coef, sc, w.cs, d, st, xp ? 1 : 0));
+  int parts;
+  if (dtype == EMA_BF16) {
+    parts = tile_parts_per_dim<TileBf16>(d.T);
+    if (xp)
+      EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, true>(x, sx, dy, sd, coef, sc, w.cs, prev128, dx, sdx, nullptr,
+                                                         none, w.part, dfinal, dinit, w.chain, d, st, ev_start,
+                                                         ev_stop)));
+    else
+      EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, false>(x, sx, dy, sd, coef, sc, w.cs, prev128, dx, sdx,
+                                                          nullptr, none, w.part, dfinal, dinit, w.chain, d, st,
+                                                          ev_start, ev_stop)));
+  } else {
+    parts = tile_parts_per_dim<TileF32>(d.T);
+    if (xp)
+      EMA_TRY((launch_bwd_tile_t<float, TileF32, true>(x, sx, dy, sd, coef, sc, w.cs, prev128, dx, sdx, nullptr,
+                                                       none, w.part, dfinal, dinit, w.chain, d, st, ev_start,
+                                                       ev_stop)));
+    else
+      EMA_TRY((launch_bwd_tile_t<float, TileF32, false>(x, sx, dy, sd, coef, sc, w.cs, prev128, dx, sdx, nullptr,
+                                                        none, w.part, dfinal, dinit, w.chain, d, st, ev_start,
+                                                        ev_stop)));
+  }
+  const int64_t total = d.N * d.L;
+  hipLaunchKernelGGL(dcoef_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w.part,
+                     dcoef, SeqStrides{dc_sb, dc_sl, dc_sh}, (int)d.nh, (int)d.L, (int)d.C, parts, total);
+  return launched();
 }
 
 #ifdef EMA_TIMING

@@ -54,12 +54,36 @@ __device__ __forceinline__ unsigned chain_wait(const u64* p, float* v, unsigned*
   return kFlagPrefix;
 }
 
-// Zeroes the status words, the ticket counters and the error word before a chained kernel.
-__global__ __launch_bounds__(256) void chain_init_kernel(uint4* __restrict__ words, int64_t n16,
-                                                         unsigned* __restrict__ counters) {
+// Prepares the status words, the ticket counters and the error word before a chained kernel.
+// The words of one column set are laid out [slot][BN] with C + 1 slots: C tiles and one
+// virtual neighbour before the first tile (forward: slot 0, tiles at slot c + 1) or after the
+// last (reverse: slot C, tiles at slot c).  Tile slots are zeroed; the virtual slot carries
+// PREFIX with the state that enters the scan from outside, seed[n, column] or 0.  Each thread
+// writes two adjacent words (BN is even, so both lie in one slot).
+__global__ __launch_bounds__(256) void chain_init_kernel(uint4* __restrict__ words, int64_t n_pairs,
+                                                         unsigned* __restrict__ counters, int BN,
+                                                         int slots, int virt_slot, int ntiles, int Tdim,
+                                                         const float* __restrict__ seed) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < n16) words[i] = make_uint4(0u, 0u, 0u, 0u);
   if (i < 4) counters[i] = 0u;
+  if (i >= n_pairs) return;
+  const int64_t w = 2 * i;
+  const int64_t row = w / BN;  // (column set, slot)
+  const int k = (int)(w - row * BN);
+  const int64_t col_id = row / slots;
+  const int slot = (int)(row - col_id * slots);
+  uint4 v = make_uint4(0u, 0u, 0u, 0u);
+  if (slot == virt_slot) {
+    float s0 = 0.f, s1 = 0.f;
+    if (seed) {
+      const int64_t n = col_id / ntiles;
+      const int col = (int)(col_id - n * ntiles) * BN + k;
+      if (col < Tdim) s0 = seed[n * Tdim + col];
+      if (col + 1 < Tdim) s1 = seed[n * Tdim + col + 1];
+    }
+    v = make_uint4(__float_as_uint(s0), kFlagPrefix, __float_as_uint(s1), kFlagPrefix);
+  }
+  words[i] = v;
 }
 
 struct ChainTile {
@@ -87,20 +111,27 @@ __device__ __forceinline__ ChainTile chain_decode(int ticket, int cols, int ntil
 
 
 // Inclusive state entering chunk c for one column: walks the published words of the chunks
-// before (forward) or after (reverse) c.  status points at the words of this column set,
-// laid out [chunk][BN]; cs_last(j) is the total log-decay of chunk j.
+// before (forward) or after (reverse) c, ending at the virtual neighbour at the latest.
+// status points at the words of this column set, laid out [slot][BN] as chain_init_kernel
+// describes; cs_n[j * 128 + 127] is the total log-decay of chunk j.
 template <bool REV, int BN>
 __device__ __forceinline__ float chain_look(const u64* status, const float* __restrict__ cs_n,
                                             int c, int C, int t, unsigned* err) {
   float carry = 0.f, scale = 1.f;
-  for (int j = REV ? c + 1 : c - 1; REV ? j < C : j >= 0; j += REV ? 1 : -1) {
+  for (int j = REV ? c + 1 : c - 1; REV ? j <= C : j >= -1; j += REV ? 1 : -1) {
     float v;
-    const unsigned f = chain_wait(status + (int64_t)j * BN + t, &v, err);
+    const unsigned f = chain_wait(status + (int64_t)(REV ? j : j + 1) * BN + t, &v, err);
     carry = fmaf(scale, v, carry);
-    if (f == kFlagPrefix) break;
+    if (f == kFlagPrefix) break;  // always so at the virtual neighbour
     scale *= __expf(fminf(cs_n[(int64_t)j * kTileRows + kTileRows - 1], 0.f));
   }
   return carry;
+}
+
+// Slot of tile c of a column set.
+template <bool REV>
+__device__ __forceinline__ int chain_slot(int c) {
+  return REV ? c : c + 1;
 }
 
 }  // namespace ema

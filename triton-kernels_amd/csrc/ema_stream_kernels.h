@@ -9,12 +9,15 @@ namespace ema {
 // ------------------------------------------------------------------------------------
 // F1: per-chunk inclusive cumsum of the log-decay.  One wave per (n, c); lane l owns the
 // `per` consecutive positions starting at l * per, sums them serially, and the lane totals
-// are scanned across the wave with DPP.
+// are scanned across the wave with DPP.  With prob != 0 the input holds probabilities p and
+// the log-decay is log(1 - p).
 // ------------------------------------------------------------------------------------
+__device__ __forceinline__ float cumsum_term(float v, int prob) { return prob ? log1pf(-v) : v; }
+
 __global__ __launch_bounds__(256) void cumsum_kernel(const float* __restrict__ A,
                                                      SeqStrides sa, float* __restrict__ cs,
                                                      int nh, int L, int Q, int C,
-                                                     int64_t total_chunks) {
+                                                     int64_t total_chunks, int prob) {
   const int lane = threadIdx.x & 63;
   const int64_t chunk_id = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (chunk_id >= total_chunks) return;
@@ -30,13 +33,13 @@ __global__ __launch_bounds__(256) void cumsum_kernel(const float* __restrict__ A
   float local = 0.f;
   for (int i = 0; i < per; ++i) {
     const int q = q0 + i;
-    if (q < limit) local += a[(int64_t)q * sa.sl];
+    if (q < limit) local += cumsum_term(a[(int64_t)q * sa.sl], prob);
   }
   float run = wave_inclusive_scan(local) - local;  // exclusive prefix of the lane totals
   float* out = cs + chunk_id * Q;
   for (int i = 0; i < per; ++i) {
     const int q = q0 + i;
-    if (q < limit) run += a[(int64_t)q * sa.sl];
+    if (q < limit) run += cumsum_term(a[(int64_t)q * sa.sl], prob);
     if (q < Q) out[q] = run;
   }
 }

@@ -20,6 +20,13 @@
 // The backward does the same from the last row to the first for dx = dy + a[next]*dx[next],
 // keeps the forward values y (float32, from the states the forward pass saved) in registers
 // and forms dA[m] = a[m] * <dx[m], y[m-1]> on the way.
+//
+// Two forms of the recurrence (template flag XP):
+//   log-decay form   y = a*y + x,        a = exp(min(A, 0));   gradients dx = r, dA = a*<r, y_prev>
+//   probability form y = (1-p)*y + p*x,  evaluated as y + p*(x - y);  dx = p*r, dp = <r, x - y_prev>
+// with r the reverse scan of dy.  The state before the first row may be given (init) and the
+// gradient reaching the state after the last row (dfinal); the backward then also returns the
+// gradient of the initial state, a[0]*r[0].
 #pragma once
 #include "ema_chain_kernels.h"
 
@@ -131,16 +138,28 @@ __device__ __forceinline__ void tile_load_rows(RowWords<TileCfg<T, CPL, RPL>::NW
   }
 }
 
-// a[i] = exp(min(A[row], 0)) of the wave's rows (1 past the end of the sequence); the
-// addresses are uniform over the wave.
-template <int RPL>
+// Row coefficients of the wave's rows; the addresses are uniform over the wave.  Log-decay
+// form: a[i] = exp(min(A[row], 0)), 1 past the end of the sequence.  Probability form:
+// a[i] = p[row], 0 past the end.
+template <int RPL, bool XP>
 __device__ __forceinline__ void tile_decays(float* a, const float* __restrict__ A, int64_t a_sl, int nrows) {
 #pragma unroll
-  for (int i = 0; i < RPL; ++i) a[i] = i < nrows ? __expf(fminf(A[(int64_t)i * a_sl], 0.f)) : 1.f;
+  for (int i = 0; i < RPL; ++i) {
+    if (XP) a[i] = i < nrows ? A[(int64_t)i * a_sl] : 0.f;
+    else a[i] = i < nrows ? __expf(fminf(A[(int64_t)i * a_sl], 0.f)) : 1.f;
+  }
 }
 
-// Inclusive state entering chunk c for one column, as chain_look, with the first word
-// requested before the loop so that a published predecessor costs one round trip.
+// One step of the forward recurrence, and the factor by which the step scales the state.
+template <bool XP>
+__device__ __forceinline__ float tile_step(float coef, float s, float x) {
+  return XP ? fmaf(coef, x - s, s) : fmaf(coef, s, x);
+}
+template <bool XP>
+__device__ __forceinline__ float tile_keep(float coef) {
+  return XP ? 1.f - coef : coef;
+}
+
 template <bool REV, int BN>
 __device__ __forceinline__ float tile_look(const u64* status, const float* __restrict__ cs_n, int c,
                                            int C, int k, unsigned* err) {
@@ -149,16 +168,17 @@ __device__ __forceinline__ float tile_look(const u64* status, const float* __res
 
 // ------------------------------------------------------------------------------------
 // Forward.  Writes y, prev[n,c,:] (state entering each 128-row chunk), optionally a copy at
-// a coarser chunking and the final state.  status: N*ntiles*C*BN zeroed words; counters[0]
+// a coarser chunking and the final state.  With has_init the state before the first row is
+// what the virtual slot of the status words carries.  status: N*ntiles*C*BN zeroed words; counters[0]
 // ticket, counters[3] error word.  One ticket = one tile; the next ticket is fetched while
 // the tile is processed.
 // ------------------------------------------------------------------------------------
-template <typename T, int CPL, int RPL, int MINW>
+template <typename T, int CPL, int RPL, int MINW, bool XP>
 __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
     const T* __restrict__ x, SeqStrides sx, const float* __restrict__ A, SeqStrides sa,
     const float* __restrict__ cs, T* __restrict__ y, SeqStrides sy, float* __restrict__ prev,
     float* __restrict__ prev_coarse, int ratio, float* __restrict__ final_state,
-    u64* __restrict__ status, unsigned* __restrict__ counters, int nh, int L, int Tdim, int C,
+    int has_init, u64* __restrict__ status, unsigned* __restrict__ counters, int nh, int L, int Tdim, int C,
     int ntiles, int cols, int total) {
   using W = TileCfg<T, CPL, RPL>;
   constexpr int BN = W::BN, NW = W::NW, NG = W::NG;
@@ -184,9 +204,9 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
                                           ((int64_t)t.c * kTileRows + RPL * grp) * sx.sl + t.col0,
                                 sx.sl, nrows, cok, lane);
     float a[RPL];
-    tile_decays<RPL>(a, A + (int64_t)t.b * sa.sb + (int64_t)t.h * sa.sh +
-                            ((int64_t)t.c * kTileRows + RPL * grp) * sa.sl,
-                     sa.sl, nrows);
+    tile_decays<RPL, XP>(a, A + (int64_t)t.b * sa.sb + (int64_t)t.h * sa.sh +
+                                ((int64_t)t.c * kTileRows + RPL * grp) * sa.sl,
+                         sa.sl, nrows);
     // 1. local pass
     float s[CPL];
     float D = 1.f;
@@ -194,9 +214,9 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
     for (int e = 0; e < CPL; ++e) s[e] = 0.f;
 #pragma unroll
     for (int i = 0; i < RPL; ++i) {
-      D *= a[i];
+      D *= tile_keep<XP>(a[i]);
 #pragma unroll
-      for (int e = 0; e < CPL; ++e) s[e] = fmaf(a[i], s[e], row_get<T, NW>(rows[i], e));
+      for (int e = 0; e < CPL; ++e) s[e] = tile_step<XP>(a[i], s[e], row_get<T, NW>(rows[i], e));
     }
 #pragma unroll
     for (int e = 0; e < CPL; ++e) sS[buf][grp][lane * CPL + e] = s[e];
@@ -208,7 +228,8 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
     // 2. tile aggregate, look-back, states entering the row groups (one thread per column)
     if (threadIdx.x < BN) {
       const int k = threadIdx.x;
-      u64* st = status + (int64_t)t.col_id * C * BN;
+      u64* st = status + (int64_t)t.col_id * (C + 1) * BN;
+      u64* mine = st + (int64_t)chain_slot<false>(t.c) * BN + k;
       float loc = 0.f, dec = 1.f;
 #pragma unroll
       for (int g = 0; g < NG; ++g) {
@@ -217,17 +238,17 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
         dec *= d;
       }
       float p_in = 0.f;
-      if (t.c > 0) {
-        chain_publish(st + (int64_t)t.c * BN + k, kFlagAggregate, loc);
+      if (t.c > 0 || has_init) {  // the first tile's only neighbour is the virtual one
+        chain_publish(mine, kFlagAggregate, loc);
         p_in = tile_look<false, BN>(st, cs + (int64_t)t.n * C * kTileRows, t.c, C, k, err);
       }
       const float p_out = fmaf(dec, p_in, loc);
-      chain_publish(st + (int64_t)t.c * BN + k, kFlagPrefix, p_out);
+      chain_publish(mine, kFlagPrefix, p_out);
       if (t.col0 + k < Tdim) {
         prev[(int64_t)t.chunk_id * Tdim + t.col0 + k] = p_in;
         if (prev_coarse && t.c % ratio == 0)
           prev_coarse[((int64_t)t.n * ((C + ratio - 1) / ratio) + t.c / ratio) * Tdim + t.col0 + k] = p_in;
-        if (t.c == C - 1) final_state[(int64_t)t.n * Tdim + t.col0 + k] = p_out;
+        if (final_state && t.c == C - 1) final_state[(int64_t)t.n * Tdim + t.col0 + k] = p_out;
       }
       float E = p_in;
 #pragma unroll
@@ -251,7 +272,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
 #pragma unroll
       for (int i = 0; i < RPL; ++i) {
 #pragma unroll
-        for (int e = 0; e < CPL; ++e) s[e] = fmaf(a[i], s[e], row_get<T, NW>(rows[i], e));
+        for (int e = 0; e < CPL; ++e) s[e] = tile_step<XP>(a[i], s[e], row_get<T, NW>(rows[i], e));
         if (i < nrows && cok) row_store<NW>(g + (int64_t)i * sy.sl + off, row_pack<T, CPL, NW>(s));
       }
     }
@@ -267,15 +288,17 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
 // the reverse state entering each tile from the rows after it, H = a[next row] * dx[next row],
 // comes from the chained scan over dy, last chunk first.  Writes dx, optionally y, and the
 // column partials part[(chunk*ntiles + ctile)*128 + m] = a[m] * <dx[m], y[m-1]> over the
-// tile's columns.  counters[1] ticket, counters[3] error word.
+// tile's columns (probability form: <r[m], x[m] - y[m-1]>).  With has_dfinal the virtual slot
+// of the status words carries the gradient reaching the state after the last row; dinit (may
+// be null) receives the gradient of the state before the first.  counters[1] ticket, counters[3] error word.
 // ------------------------------------------------------------------------------------
-template <typename T, int CPL, int RPL, int MINW, bool WRITE_Y>
+template <typename T, int CPL, int RPL, int MINW, bool WRITE_Y, bool XP>
 __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     const T* __restrict__ x, SeqStrides sx, const T* __restrict__ dy, SeqStrides sd,
     const float* __restrict__ A, SeqStrides sa, const float* __restrict__ cs,
     const float* __restrict__ prev, T* __restrict__ dx, SeqStrides sdx, T* __restrict__ y,
-    SeqStrides sy, float* __restrict__ part, u64* __restrict__ status,
-    unsigned* __restrict__ counters, int nh, int L, int Tdim, int C, int ntiles, int cols, int total) {
+    SeqStrides sy, float* __restrict__ part, int has_dfinal,
+    float* __restrict__ dinit, u64* __restrict__ status, unsigned* __restrict__ counters, int nh, int L, int Tdim, int C, int ntiles, int cols, int total) {
   using W = TileCfg<T, CPL, RPL>;
   constexpr int BN = W::BN, NW = W::NW, NG = W::NG;
   __shared__ __attribute__((aligned(16))) float sS[2][NG][BN];  // forward group states
@@ -305,8 +328,11 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     float p_in = 0.f;
     if (threadIdx.x < BN && t.col0 + (int)threadIdx.x < Tdim)
       p_in = prev[(int64_t)t.chunk_id * Tdim + t.col0 + threadIdx.x];
-    float a[RPL];
-    tile_decays<RPL>(a, A + (int64_t)t.b * sa.sb + (int64_t)t.h * sa.sh + row0 * sa.sl, sa.sl, nrows);
+    // a: factor of the state per row; pc: the row's coefficient as tile_step takes it
+    float a[RPL], pc[RPL];
+    tile_decays<RPL, XP>(pc, A + (int64_t)t.b * sa.sb + (int64_t)t.h * sa.sh + row0 * sa.sl, sa.sl, nrows);
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) a[i] = tile_keep<XP>(pc[i]);
 
     // 1a. local reverse pass over dy, r = a[i] * dx_local[i]; at the end the state that the
     // group hands to the rows before it
@@ -324,7 +350,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
 #pragma unroll
     for (int i = 0; i < RPL; ++i)
 #pragma unroll
-      for (int e = 0; e < CPL; ++e) s[e] = fmaf(a[i], s[e], row_get<T, NW>(xr[i], e));
+      for (int e = 0; e < CPL; ++e) s[e] = tile_step<XP>(pc[i], s[e], row_get<T, NW>(xr[i], e));
 #pragma unroll
     for (int e = 0; e < CPL; ++e) {
       sR[buf][grp][lane * CPL + e] = r[e];
@@ -337,7 +363,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     EMA_TSTAMP(1);
 
     // 2a. publish the reverse aggregate; forward states entering the row groups
-    u64* st = status + (int64_t)t.col_id * C * BN;
+    u64* st = status + (int64_t)t.col_id * (C + 1) * BN;
     float loc = 0.f, dec = 1.f;
     if (threadIdx.x < BN) {
       const int k = threadIdx.x;
@@ -347,7 +373,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
         loc = fmaf(d, loc, sR[buf][g][k]);
         dec *= d;
       }
-      if (t.c < C - 1) chain_publish(st + (int64_t)t.c * BN + k, kFlagAggregate, loc);
+      if (t.c < C - 1 || has_dfinal) chain_publish(st + (int64_t)t.c * BN + k, kFlagAggregate, loc);
       float E = p_in;
 #pragma unroll
       for (int g = 0; g < NG; ++g) {
@@ -363,8 +389,11 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     if (threadIdx.x < BN) {
       const int k = threadIdx.x;
       float h_in = 0.f;
-      if (t.c < C - 1) h_in = tile_look<true, BN>(st, cs + (int64_t)t.n * C * kTileRows, t.c, C, k, err);
-      chain_publish(st + (int64_t)t.c * BN + k, kFlagPrefix, fmaf(dec, h_in, loc));
+      if (t.c < C - 1 || has_dfinal)
+        h_in = tile_look<true, BN>(st, cs + (int64_t)t.n * C * kTileRows, t.c, C, k, err);
+      const float h_out = fmaf(dec, h_in, loc);
+      chain_publish(st + (int64_t)t.c * BN + k, kFlagPrefix, h_out);
+      if (dinit && t.c == 0 && t.col0 + k < Tdim) dinit[(int64_t)t.n * Tdim + t.col0 + k] = h_out;
       float G = h_in;
 #pragma unroll
       for (int g = NG - 1; g >= 0; --g) {
@@ -388,7 +417,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
       for (int i = 0; i < RPL; ++i) {
 #pragma unroll
         for (int e = 0; e < CPL; ++e) {
-          s[e] = fmaf(a[i], s[e], row_get<T, NW>(xr[i], e));
+          s[e] = tile_step<XP>(pc[i], s[e], row_get<T, NW>(xr[i], e));
           yv[i][e] = s[e];
         }
         if (WRITE_Y && i < nrows && cok) row_store<NW>(g + (int64_t)i * sy.sl + off, row_pack<T, CPL, NW>(s));
@@ -412,13 +441,22 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
         for (int e = 0; e < CPL; ++e) {
           // r holds a[i+1] * dx[i+1] on entry (the carried state for the last row)
           const float d = row_get<T, NW>(dr[i], e) + r[e];
-          dot = fmaf(d, i > 0 ? yv[i - 1][e] : E[e], dot);
+          const float yp = i > 0 ? yv[i - 1][e] : E[e];
+          dot = fmaf(d, XP ? row_get<T, NW>(xr[i], e) - yp : yp, dot);
           r[e] = d;
         }
-        if (i < nrows && cok) row_store<NW>(g + (int64_t)i * sdx.sl + off, row_pack<T, CPL, NW>(r));
+        if (XP) {
+          float o[CPL];
+#pragma unroll
+          for (int e = 0; e < CPL; ++e) o[e] = pc[i] * r[e];
+          if (i < nrows && cok) row_store<NW>(g + (int64_t)i * sdx.sl + off, row_pack<T, CPL, NW>(o));
+        } else {
+          if (i < nrows && cok) row_store<NW>(g + (int64_t)i * sdx.sl + off, row_pack<T, CPL, NW>(r));
+        }
 #pragma unroll
         for (int e = 0; e < CPL; ++e) r[e] *= a[i];
-        dot = a[i] * wave_sum(dot);
+        dot = wave_sum(dot);
+        if (!XP) dot *= a[i];
         if (lane == i) dA = dot;
       }
       if (lane < RPL)
@@ -429,6 +467,25 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     slot ^= 1;
     buf ^= 1;
   }
+}
+
+// out[b, p, h] = sum over the column tiles of part[n, p / 128, tile, p % 128]: the gradient of
+// the per-position coefficient in the layout of the coefficient itself.  One thread per (n, p).
+__global__ __launch_bounds__(256) void dcoef_reduce_kernel(const float* __restrict__ part,
+                                                           float* __restrict__ out, SeqStrides so, int nh,
+                                                           int L, int Ci, int ntiles, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int64_t n = i / L;
+  const int64_t p = i - n * L;
+  const int64_t ci = p / kTileRows;
+  const int q = (int)(p - ci * kTileRows);
+  const float* pp = part + ((n * Ci + ci) * ntiles) * (int64_t)kTileRows + q;
+  float s = 0.f;
+  for (int t = 0; t < ntiles; ++t) s += pp[(int64_t)t * kTileRows];
+  const int64_t b = n / nh;
+  const int64_t h = n - b * nh;
+  out[b * so.sb + p * so.sl + h * so.sh] = s;
 }
 
 }  // namespace ema

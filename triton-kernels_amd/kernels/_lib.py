@@ -15,6 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libema_hip.so")
 
 EMA_F32, EMA_BF16 = 0, 1
+EMA_FORM_LOG_DECAY, EMA_FORM_PROBABILITY = 0, 1
 EMA_MAX_CHUNK = 1024
 
 _I = c_int64
@@ -42,6 +43,10 @@ _SIGNATURES = {
     "ema_bwd_dx_dA_fused": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P] + _SEQ + [_P] + _SEQ + [_P, c_size_t, _I, _I, _I, _I, _P]),
     "ema_bwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I]),
     "ema_bwd": (c_int, _SEQ + _SEQ + _SEQ + [_P, c_int] + _SEQ + [_P] + _SEQ + [_P, c_size_t, _I, _I, _I, _I, _I, _P, _P, _P]),
+    "ema_seq_fwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
+    "ema_seq_bwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
+    "ema_seq_fwd": (c_int, [c_int] + _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _P, _P, _P]),
+    "ema_seq_bwd": (c_int, [c_int] + _SEQ + _SEQ + _SEQ + [_P, _P, c_int] + _SEQ + _SEQ + [_P, _P, c_size_t, _I, _I, _I, _I, _P, _P, _P]),
 }
 
 _lib = None
