@@ -1,0 +1,213 @@
+"""CPU oracle for the Mamba-2 SSD chunked scan (forward).
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the product path may import this module: only tests/,
+__graft_entry__.smoke() and the cpu_baseline leg of bench.py use it, and only as the checker.
+
+It restates, in plain PyTorch on the CPU, the arithmetic of the reference repository
+kartiksrinivas007/triton-kernels (paths relative to its root):
+
+* the sequential definition (the state-space recurrence)
+      h_t = exp(dt_t * A) * h_{t-1} + dt_t * x_t (outer) B_t,   y_t = C_t . h_t + D * x_t,
+  optionally gated y_t * z_t * sigmoid(z_t): ssd_step_ref,
+  kernels/mamba_3_kernels/mamba_ssd_fwd.py:795-860, without its trapezoid / rotary / bias
+  options and with the natural exponential that kernels/mamba_kernels/ uses (that file's
+  own kernels use exp2);
+* the five stages of the chunked forward in kernels/mamba_kernels/:
+      chunk_cumsum   mamba_cumsum.py:32-128      (dt bias / softplus / clamp, dA = dt * A, cumsum)
+      chunk_state    mamba_state_fwd.py:54-169   (B^T x weighted by exp(dA_last - dA_k) * dt_k)
+      state_passing  mamba_state_pass.py:20-115  (inter-chunk recurrence, optional initial state)
+      bmm_chunk      mamba_bmm.py                (C B^T per chunk and group)
+      chunk_scan     mamba_scan_fwd.py:30-210    (C.prev * exp(dA_m) + causal (CB o decay o dt) x
+                                                  + D x, z gate)
+
+Layouts as in the reference: x (b, L, nh, hdim); dt (b, L, nh); A (nh,); B, C (b, L, g, dstate);
+chunked dt / dA_cumsum (b, nh, C, Q); states (b, C, nh, hdim, dstate); CB (b, C, g, Q, Q).
+
+Pinning status (tests/test_ssd_oracle.py): the reference holds no golden vectors for this path
+and its comparison provider (mamba_ssm) is not installed, so the functions here are pinned by
+what the mathematics fixes: a pure-Python brute force of the closed form on tiny inputs, the
+composition of the five stages against the sequential recurrence for several chunk sizes
+(chunk-size invariance), the reduction to the EMA scan for dstate = 1, B = C = 1, dt = 1 (whose
+oracle is pinned separately), the segsum form of ssd_fwd_ref, and linearity in x.  No function
+is left "parity unpinned".
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+
+def _up(t):
+    """float32 arithmetic as in the kernels; float64 inputs (used to pin the oracle) stay float64."""
+    return t if t.dtype == torch.float64 else t.float()
+
+
+def process_dt(dt, dt_bias=None, dt_softplus=False, dt_limit=(0.0, float("inf"))):
+    """dt (b, L, nh) -> float32 after bias, softplus (identity above 20) and clamp;
+    mamba_cumsum.py:72-80."""
+    dt = _up(dt)
+    if dt_bias is not None:
+        dt = dt + _up(dt_bias)
+    if dt_softplus:
+        dt = torch.where(dt <= 20.0, F.softplus(dt), dt)
+    return torch.clamp(dt, dt_limit[0], dt_limit[1])
+
+
+def ssd_loop(x, dt, A, B, C, D=None, z=None, initial_states=None):
+    """Sequential recurrence; dt is already processed (float32).  x (b,L,nh,p), dt (b,L,nh),
+    A (nh,), B/C (b,L,g,n), D (nh,) or (nh,p), z like x, initial_states (b,nh,p,n).
+    Returns (y (b,L,nh,p), final_states (b,nh,p,n)) in x's dtype / float32 arithmetic of x."""
+    b, L, nh, p = x.shape
+    g, n = B.shape[2], B.shape[3]
+    rep = nh // g
+    Bh = B.repeat_interleave(rep, dim=2)
+    Ch = C.repeat_interleave(rep, dim=2)
+    h = x.new_zeros(b, nh, p, n) if initial_states is None else initial_states.to(x.dtype).clone()
+    y = torch.empty_like(x)
+    for t in range(L):
+        a = torch.exp(dt[:, t] * A)  # (b, nh)
+        h = a[..., None, None] * h + (dt[:, t, :, None] * x[:, t])[..., None] * Bh[:, t, :, None, :]
+        out = (h * Ch[:, t, :, None, :]).sum(-1)
+        if D is not None:
+            out = out + (D[None, :, None] if D.dim() == 1 else D[None]) * x[:, t]
+        if z is not None:
+            out = out * z[:, t] * torch.sigmoid(z[:, t])
+        y[:, t] = out
+    return y, h
+
+
+# ------------------------------------------------------------------ the five stages
+
+
+def _pad_seq(t, Q):
+    pad = (-t.shape[1]) % Q
+    if pad == 0:
+        return t
+    return torch.cat([t, t.new_zeros(t.shape[0], pad, *t.shape[2:])], 1)
+
+
+def chunk_cumsum(dt, A, Q, dt_bias=None, dt_softplus=False, dt_limit=(0.0, float("inf"))):
+    """-> (dA_cumsum, dt_out), both (b, nh, C, Q) float32; positions past L hold dt = 0."""
+    b, L, nh = dt.shape
+    d = _pad_seq(process_dt(dt, dt_bias, dt_softplus, dt_limit), Q)
+    valid = _pad_seq(torch.ones(b, L, nh, dtype=d.dtype), Q)
+    d = d * valid
+    C = d.shape[1] // Q
+    d = d.reshape(b, C, Q, nh).permute(0, 3, 1, 2).contiguous()
+    dA = d * _up(A)[None, :, None, None]
+    return torch.cumsum(dA, -1), d
+
+
+def chunk_state(B, x, dt, dA_cumsum):
+    """states[b,c,h,p,n] = sum_k x[k,p] * B[k,n] * exp(min(dA_last - dA_k, 0)) * dt_k."""
+    b, L, nh, p = x.shape
+    _, _, C, Q = dt.shape
+    g, n = B.shape[2], B.shape[3]
+    xc = _pad_seq(_up(x), Q).reshape(b, C, Q, nh, p)
+    Bc = _pad_seq(_up(B), Q).reshape(b, C, Q, g, n).repeat_interleave(nh // g, dim=3)
+    w = torch.exp(torch.clamp(dA_cumsum[..., -1:] - dA_cumsum, max=0.0)) * dt  # (b, nh, C, Q)
+    w = w.permute(0, 2, 3, 1)  # (b, C, Q, nh)
+    return torch.einsum("bcqhp,bcqhn,bcqh->bchpn", xc, Bc, w)
+
+
+def state_passing(states, dA_chunk_cumsum, initial_states=None):
+    """states (b, C, nh, dim), dA_chunk_cumsum (b, nh, C) -> (out (b, C, nh, dim) = state
+    entering each chunk, final (b, nh, dim))."""
+    b, C, nh, dim = states.shape
+    out = torch.empty_like(states)
+    s = states.new_zeros(b, nh, dim) if initial_states is None else _up(initial_states).clone()
+    for c in range(C):
+        out[:, c] = s
+        s = torch.exp(dA_chunk_cumsum[:, :, c])[..., None] * s + states[:, c]
+    return out, s
+
+
+def bmm_chunk(a, bm, Q):
+    """out[b,c,g,m,k] = sum_n a[b,cQ+m,g,n] * bm[b,cQ+k,g,n]  (a = C, bm = B)."""
+    b, L, g, n = a.shape
+    ac = _pad_seq(_up(a), Q).reshape(b, -1, Q, g, n)
+    bc = _pad_seq(_up(bm), Q).reshape(b, -1, Q, g, n)
+    return torch.einsum("bcmgn,bckgn->bcgmk", ac, bc)
+
+
+def chunk_scan(cb, x, dt, dA_cumsum, C, states, D=None, z=None):
+    """out[m,p] = exp(dA_m) * sum_n C[m,n] prev[p,n]
+                 + sum_{k<=m} cb[m,k] exp(min(dA_m - dA_k, 0)) dt_k x[k,p]  + D x,  then the z gate.
+    Returns (out, out_x) with out_x the value before gating (None without z)."""
+    b, L, nh, p = x.shape
+    _, _, nc, Q = dt.shape
+    g, n = C.shape[2], C.shape[3]
+    rep = nh // g
+    xc = _pad_seq(_up(x), Q).reshape(b, nc, Q, nh, p)
+    Cc = _pad_seq(_up(C), Q).reshape(b, nc, Q, g, n).repeat_interleave(rep, dim=3)
+    cbh = _up(cb).repeat_interleave(rep, dim=2)  # (b, nc, nh, Q, Q)
+    dA = dA_cumsum.permute(0, 2, 1, 3)  # (b, nc, nh, Q)
+    dtc = dt.permute(0, 2, 1, 3)
+    decay = torch.exp(torch.clamp(dA[..., :, None] - dA[..., None, :], max=0.0))
+    mask = torch.tril(torch.ones(Q, Q, dtype=torch.bool))
+    w = cbh * decay * dtc[..., None, :]
+    w = torch.where(mask, w, w.new_zeros(()))
+    out = torch.einsum("bchmk,bckhp->bcmhp", w, xc)
+    out = out + torch.einsum("bcmhn,bchpn,bchm->bcmhp", Cc, _up(states), torch.exp(dA))
+    out = out.reshape(b, nc * Q, nh, p)[:, :L]
+    if D is not None:
+        out = out + (_up(D)[None, None, :, None] if D.dim() == 1 else _up(D)[None, None]) * _up(x)
+    out_x = None
+    if z is not None:
+        out_x = out
+        out = out * _up(z) * torch.sigmoid(_up(z))
+    return out, out_x
+
+
+def combined_fwd(x, dt, A, B, C, Q, D=None, z=None, dt_bias=None, initial_states=None,
+                 dt_softplus=False, dt_limit=(0.0, float("inf"))):
+    """The five stages in the order of mamba_ssm's combined forward, which the reference's
+    kernels/mamba_kernels/ files were taken from.  Returns (out, final_states)."""
+    b, L, nh, p = x.shape
+    n = B.shape[-1]
+    dA_cs, dt_out = chunk_cumsum(dt, A, Q, dt_bias, dt_softplus, dt_limit)
+    states = chunk_state(B, x, dt_out, dA_cs)
+    init = None if initial_states is None else initial_states.reshape(b, nh, p * n)
+    prev, final = state_passing(states.reshape(b, -1, nh, p * n), dA_cs[..., -1], init)
+    prev = prev.reshape(b, -1, nh, p, n)
+    cb = bmm_chunk(C, B, Q)
+    out, _ = chunk_scan(cb, x, dt_out, dA_cs, C, prev, D, z)
+    return out, final.reshape(b, nh, p, n)
+
+
+# ------------------------------------------------------------------ inputs and brute force
+
+
+def make_inputs(b, L, nh, p, g, n, seed, dtype=torch.float32, with_z=False):
+    """BASELINE configuration 5's distributions: x, B, C ~ N(0,1); dt = softplus(N(-2, 0.5));
+    A = -exp(U(log 1, log 16)) per head; D = 0 is the configuration's choice (a non-zero D is
+    returned for the tests that want one); z ~ N(0,1)."""
+    gen = torch.Generator().manual_seed(seed)
+    x = torch.randn(b, L, nh, p, generator=gen).to(dtype)
+    Bm = torch.randn(b, L, g, n, generator=gen).to(dtype)
+    Cm = torch.randn(b, L, g, n, generator=gen).to(dtype)
+    dt = F.softplus(torch.randn(b, L, nh, generator=gen) * 0.5 - 2.0)
+    A = -torch.exp(torch.rand(nh, generator=gen) * math.log(16.0))
+    D = torch.randn(nh, generator=gen)
+    z = torch.randn(b, L, nh, p, generator=gen).to(dtype) if with_z else None
+    return x, dt, A, Bm, Cm, D, z
+
+
+def brute_force(x, dt, A, B, C):
+    """Pure-Python O(L^2) evaluation of y_t = sum_{s<=t} (C_t . B_s) exp(A sum_{j=s+1..t} dt_j) dt_s x_s
+    (one group), tiny inputs only; shares no code with anything above."""
+    b, L, nh, p = x.shape
+    n = B.shape[-1]
+    out = torch.zeros(b, L, nh, p, dtype=torch.float64)
+    for bi in range(b):
+        for h in range(nh):
+            for t in range(L):
+                for s in range(t + 1):
+                    cbv = sum(float(C[bi, t, 0, k]) * float(B[bi, s, 0, k]) for k in range(n))
+                    dec = math.exp(float(A[h]) * sum(float(dt[bi, j, h]) for j in range(s + 1, t + 1)))
+                    wgt = cbv * dec * float(dt[bi, s, h])
+                    for f in range(p):
+                        out[bi, t, h, f] += wgt * float(x[bi, s, h, f])
+    return out

@@ -1,0 +1,119 @@
+"""Pins the SSD oracle (oracle/ssd_oracle.py) by what the mathematics fixes.  CPU only.
+
+The reference holds no golden vectors for the Mamba-2 path and its comparison provider
+(mamba_ssm) is not installed, so nothing here compares with reference outputs."""
+import math
+
+import pytest
+import torch
+
+from oracle import ema_oracle as E
+from oracle import ssd_oracle as S
+
+D64 = torch.float64
+
+
+def _f64(*ts):
+    return [None if t is None else t.to(D64) for t in ts]
+
+
+def test_loop_matches_brute_force():
+    x, dt, A, B, C, _, _ = _f64(*S.make_inputs(1, 7, 2, 3, 1, 4, seed=0))
+    y, _ = S.ssd_loop(x, dt, A, B, C)
+    assert torch.allclose(y, S.brute_force(x, dt, A, B, C), rtol=1e-12, atol=1e-12)
+
+
+def test_loop_reduces_to_ema_scan():
+    # dstate = 1, B = C = 1, dt = 1: h_t = exp(A) h_{t-1} + x_t per head, the EMA recurrence
+    b, L, nh, p = 2, 33, 3, 5
+    gen = torch.Generator().manual_seed(1)
+    x = torch.randn(b, L, nh, p, generator=gen, dtype=D64)
+    A = -torch.rand(nh, generator=gen, dtype=D64)
+    ones = torch.ones(b, L, 1, 1, dtype=D64)
+    y, fin = S.ssd_loop(x, torch.ones(b, L, nh, dtype=D64), A, ones, ones)
+    xf, Af = E.to_flat(x, A.expand(b, L, nh).contiguous())
+    y_ema = E.from_flat(E.ema_loop(xf, Af), b, nh)
+    assert torch.allclose(y, y_ema, rtol=1e-12, atol=1e-12)
+    assert torch.allclose(fin[..., 0], y[:, -1], rtol=1e-12, atol=1e-12)
+
+
+def test_loop_matches_segsum_matrix_form():
+    # the quadratic form of ssd_fwd_ref (mamba_ssd_fwd.py:772-777) with natural exp
+    x, dt, A, B, C, D, z = _f64(*S.make_inputs(2, 19, 4, 3, 2, 5, seed=2, with_z=True))
+    y, _ = S.ssd_loop(x, dt, A, B, C, D, z)
+    dA = (dt * A).permute(0, 2, 1)  # (b, h, s)
+    cs = torch.cumsum(dA, -1)
+    seg = cs[..., :, None] - cs[..., None, :]
+    L = x.shape[1]
+    mask = torch.tril(torch.ones(L, L, dtype=torch.bool))
+    Bh = B.repeat_interleave(2, dim=2) * dt[..., None]
+    Ch = C.repeat_interleave(2, dim=2)
+    cb = torch.einsum("bthd,bshd->bhts", Ch, Bh)
+    w = torch.where(mask, cb * torch.exp(torch.where(mask, seg, torch.zeros((), dtype=D64))), torch.zeros((), dtype=D64))
+    out = torch.einsum("bhts,bshd->bthd", w, x) + D[None, None, :, None] * x
+    out = out * z * torch.sigmoid(z)
+    assert torch.allclose(y, out, rtol=1e-11, atol=1e-11)
+
+
+@pytest.mark.parametrize("L,Q", [(64, 16), (50, 16), (37, 64), (96, 32), (5, 8)])
+@pytest.mark.parametrize("g", [1, 2])
+def test_chunked_stages_equal_loop(L, Q, g):
+    x, dt, A, B, C, D, z = _f64(*S.make_inputs(2, L, 4, 6, g, 5, seed=L + Q, with_z=True))
+    gen = torch.Generator().manual_seed(9)
+    init = torch.randn(2, 4, 6, 5, generator=gen, dtype=D64)
+    y_ref, fin_ref = S.ssd_loop(x, dt, A, B, C, D, z, init)
+    y, fin = S.combined_fwd(x, dt, A, B, C, Q, D=D, z=z, initial_states=init)
+    assert torch.allclose(y, y_ref, rtol=1e-10, atol=1e-10)
+    assert torch.allclose(fin, fin_ref, rtol=1e-10, atol=1e-10)
+
+
+def test_chunk_size_invariance_f32():
+    x, dt, A, B, C, D, _ = S.make_inputs(1, 200, 2, 8, 1, 16, seed=4)
+    outs = [S.combined_fwd(x, dt, A, B, C, Q, D=D)[0] for Q in (16, 64, 256)]
+    for o in outs[1:]:
+        assert torch.allclose(o, outs[0], rtol=1e-4, atol=1e-4)
+
+
+def test_process_dt_bias_softplus_clamp():
+    dt = torch.tensor([[[-3.0, 0.5, 25.0]]])
+    bias = torch.tensor([0.5, -0.5, 0.0])
+    out = S.process_dt(dt, bias, True, (0.1, 10.0))
+    want = [max(0.1, math.log1p(math.exp(-2.5))), math.log1p(math.exp(0.0)), 10.0]
+    assert torch.allclose(out.flatten(), torch.tensor(want), rtol=1e-6)
+
+
+def test_chunk_cumsum_restarts_and_pads():
+    dt = torch.rand(1, 10, 2)
+    A = torch.tensor([-1.0, -2.0])
+    dA_cs, dt_out = S.chunk_cumsum(dt, A, 4)
+    assert dA_cs.shape == (1, 2, 3, 4) and dt_out.shape == (1, 2, 3, 4)
+    assert torch.allclose(dA_cs[0, 1, 1], torch.cumsum(dt[0, 4:8, 1] * -2.0, 0))
+    assert torch.equal(dt_out[0, :, 2, 2:], torch.zeros(2, 2))  # past L
+    assert torch.allclose(dA_cs[0, 0, 2, 3], dA_cs[0, 0, 2, 1])
+
+
+def test_chunk_state_is_final_state_of_local_scan():
+    x, dt, A, B, C, _, _ = _f64(*S.make_inputs(1, 24, 2, 3, 1, 4, seed=6))
+    dA_cs, dt_out = S.chunk_cumsum(dt, A, 8)
+    st = S.chunk_state(B, x, dt_out.to(D64), dA_cs.to(D64))
+    for c in range(3):
+        sl = slice(8 * c, 8 * c + 8)
+        _, fin = S.ssd_loop(x[:, sl], dt[:, sl], A, B[:, sl], C[:, sl])
+        assert torch.allclose(st[:, c], fin, rtol=1e-6, atol=1e-7)  # dA_cs went through float32
+
+
+def test_linearity_in_x():
+    x, dt, A, B, C, D, _ = _f64(*S.make_inputs(1, 40, 2, 4, 1, 4, seed=7))
+    x2 = torch.randn_like(x)
+    f = lambda v: S.combined_fwd(v, dt, A, B, C, 16, D=D)[0]
+    assert torch.allclose(f(2.0 * x - 3.0 * x2), 2.0 * f(x) - 3.0 * f(x2), rtol=1e-10, atol=1e-10)
+
+
+def test_bmm_chunk_matches_einsum_per_chunk():
+    gen = torch.Generator().manual_seed(8)
+    Cm = torch.randn(2, 21, 2, 6, generator=gen)
+    Bm = torch.randn(2, 21, 2, 6, generator=gen)
+    cb = S.bmm_chunk(Cm, Bm, 8)
+    assert cb.shape == (2, 3, 2, 8, 8)
+    assert torch.allclose(cb[1, 1, 0], Cm[1, 8:16, 0] @ Bm[1, 8:16, 0].T, rtol=1e-5, atol=1e-5)
+    assert torch.equal(cb[0, 2, 1, 5:], torch.zeros(3, 8))  # rows past L
