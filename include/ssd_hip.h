@@ -1,0 +1,99 @@
+/*
+ * ssd_hip.h -- C ABI of the Mamba-2 SSD chunked-scan forward in libema_hip.so: hand-written
+ * HIP kernels for gfx950 (MI355X).
+ *
+ * Every entry point replaces one launcher of the reference repository
+ * kartiksrinivas007/triton-kernels under kernels/mamba_kernels/ (a Python function that
+ * allocates its output and starts one Triton kernel); the citation on each declaration is that
+ * launcher, with paths relative to the reference root.
+ *
+ * Conventions (as for ema_hip.h)
+ *   - All pointers are DEVICE pointers; the caller allocates inputs and outputs; the library
+ *     never allocates, frees or keeps a pointer, and only enqueues work on `stream`.
+ *   - x, z, out are (batch, seqlen, nheads, hdim); B, C are (batch, seqlen, ngroups, dstate);
+ *     dt is (batch, seqlen, nheads).  Each is addressed as ptr[b*s_b + l*s_l + h*s_h + i] with
+ *     strides in ELEMENTS and a unit stride along the last axis.
+ *   - Chunked intermediates are dense float32: dt_out and dA_cumsum (batch, nheads, C, Q),
+ *     states (batch, C, nheads, hdim, dstate), cb (batch, C, ngroups, Q, Q); C = ceil(seqlen/Q).
+ *   - `dtype` (ssd_dtype, same codes as ema_dtype) is the element type of x, z, B, C and out;
+ *     accumulation is float32.
+ *   - Supported shapes: hdim in {64, 128}, dstate in {64, 128}, nheads a multiple of ngroups,
+ *     chunk a multiple of 4 up to 1024; anything else returns SSD_ERR_UNSUPPORTED.
+ *   - Return value: 0 or a negative ssd_status (same values as ema_status).
+ */
+#ifndef SSD_HIP_H
+#define SSD_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  SSD_OK = 0,
+  SSD_ERR_NULL = -1,
+  SSD_ERR_SHAPE = -2,
+  SSD_ERR_ALIGN = -3,
+  SSD_ERR_DTYPE = -4,
+  SSD_ERR_UNSUPPORTED = -5,
+  SSD_ERR_LAUNCH = -6
+} ssd_status;
+
+typedef enum { SSD_F32 = 0, SSD_BF16 = 1 } ssd_dtype;
+
+/* dt_out = clamp(softplus?(dt + dt_bias), dt_min, dt_max) (softplus is the identity above 20),
+ * 0 past seqlen; dA_cumsum = per-chunk inclusive cumsum of dt_out * A[h].  dt may be float32
+ * or bfloat16 (dt_dtype); A and dt_bias (may be NULL) are float32 (nheads).
+ * Replaces _chunk_cumsum_fwd, kernels/mamba_kernels/mamba_cumsum.py:103-128. */
+int ssd_chunk_cumsum_fwd(const void* dt, int dt_dtype, int64_t dt_sb, int64_t dt_sl, int64_t dt_sh,
+                         const float* A, const float* dt_bias, float* dA_cumsum, float* dt_out,
+                         int64_t batch, int64_t seqlen, int64_t nheads, int64_t chunk, int dt_softplus,
+                         float dt_min, float dt_max, void* stream);
+
+/* states[b,c,h,p,n] = sum_k x[k,p] * B[k,n] * exp(min(dA_last - dA_k, 0)) * dt_k over the
+ * positions k of chunk c (the weighted B is rounded to `dtype` before the product, as the
+ * reference does).  Replaces _chunk_state_fwd, kernels/mamba_kernels/mamba_state_fwd.py:138-169
+ * (seq_idx is not supported). */
+int ssd_chunk_state_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64_t b_sg, const void* x,
+                        int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, const float* dt,
+                        const float* dA_cumsum, float* states, int64_t batch, int64_t seqlen,
+                        int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
+                        void* stream);
+
+/* out[b,c] = state entering chunk c; state <- exp(dA_chunk[b,h,c]) * state + states[b,c];
+ * final = the state after the last chunk.  states / out (batch, C, nheads, dim) float32,
+ * dA_chunk addressed by (batch, head, chunk) strides (it is dA_cumsum[..., -1]); initial
+ * (batch, nheads, dim) float32 may be NULL.  dim must be a multiple of 4.
+ * Replaces _state_passing_fwd, kernels/mamba_kernels/mamba_state_pass.py:84-115. */
+int ssd_state_passing_fwd(const float* states, const float* dA_chunk, int64_t da_sb, int64_t da_sh,
+                          int64_t da_sc, const float* initial, float* out, float* final_states,
+                          int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, void* stream);
+
+/* out[b,c,g,m,k] = sum_n a[b,cQ+m,g,n] * bm[b,cQ+k,g,n]; rows past seqlen are zero.  out is
+ * float32 or `dtype` (out_dtype).  Replaces _bmm_chunk_fwd, kernels/mamba_kernels/mamba_bmm.py:88-126
+ * (the whole Q x Q block is written, also with causal = True). */
+int ssd_bmm_chunk_fwd(const void* a, int64_t a_sb, int64_t a_sl, int64_t a_sg, const void* bm,
+                      int64_t b_sb, int64_t b_sl, int64_t b_sg, int dtype, void* out, int out_dtype,
+                      int64_t batch, int64_t seqlen, int64_t ngroups, int64_t k, int64_t chunk,
+                      void* stream);
+
+/* out[m,p] = exp(dA_m) * sum_n C[m,n] * prev[p,n]
+ *          + sum_{k<=m} cb[m,k] * exp(min(dA_m - dA_k, 0)) * dt_k * x[k,p]  +  D * x[m,p],
+ * then, with z: out_x = out (if out_x is not NULL) and out *= z * sigmoid(z).
+ * cb float32 (batch, C, ngroups, Q, Q); prev float32 (batch, C, nheads, hdim, dstate); D float32
+ * (nheads) or (nheads, hdim) (d_has_hdim), may be NULL; z may be NULL; out_x shares out's strides.
+ * Replaces _chunk_scan_fwd, kernels/mamba_kernels/mamba_scan_fwd.py:162-210. */
+int ssd_chunk_scan_fwd(const float* cb, const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
+                       const void* z, int64_t z_sb, int64_t z_sl, int64_t z_sh, int dtype,
+                       const float* dt, const float* dA_cumsum, const void* C, int64_t c_sb, int64_t c_sl,
+                       int64_t c_sg, const float* prev_states, const float* D, int d_has_hdim, void* out,
+                       int64_t o_sb, int64_t o_sl, int64_t o_sh, void* out_x, int64_t batch,
+                       int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate,
+                       int64_t chunk, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SSD_HIP_H */

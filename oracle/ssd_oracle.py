@@ -100,8 +100,15 @@ def chunk_cumsum(dt, A, Q, dt_bias=None, dt_softplus=False, dt_limit=(0.0, float
     return torch.cumsum(dA, -1), d
 
 
-def chunk_state(B, x, dt, dA_cumsum):
-    """states[b,c,h,p,n] = sum_k x[k,p] * B[k,n] * exp(min(dA_last - dA_k, 0)) * dt_k."""
+def _round(t, dtype):
+    """The reference rounds some operands to the input type before its tl.dot; `dtype` None
+    keeps full precision."""
+    return t if dtype is None else t.to(dtype).to(t.dtype)
+
+
+def chunk_state(B, x, dt, dA_cumsum, round_to=None):
+    """states[b,c,h,p,n] = sum_k x[k,p] * B[k,n] * exp(min(dA_last - dA_k, 0)) * dt_k.
+    With round_to the weighted B is rounded to that type first (mamba_state_fwd.py:118-119)."""
     b, L, nh, p = x.shape
     _, _, C, Q = dt.shape
     g, n = B.shape[2], B.shape[3]
@@ -109,7 +116,7 @@ def chunk_state(B, x, dt, dA_cumsum):
     Bc = _pad_seq(_up(B), Q).reshape(b, C, Q, g, n).repeat_interleave(nh // g, dim=3)
     w = torch.exp(torch.clamp(dA_cumsum[..., -1:] - dA_cumsum, max=0.0)) * dt  # (b, nh, C, Q)
     w = w.permute(0, 2, 3, 1)  # (b, C, Q, nh)
-    return torch.einsum("bcqhp,bcqhn,bcqh->bchpn", xc, Bc, w)
+    return torch.einsum("bcqhp,bcqhn->bchpn", xc, _round(Bc * w[..., None], round_to))
 
 
 def state_passing(states, dA_chunk_cumsum, initial_states=None):
@@ -132,10 +139,11 @@ def bmm_chunk(a, bm, Q):
     return torch.einsum("bcmgn,bckgn->bcgmk", ac, bc)
 
 
-def chunk_scan(cb, x, dt, dA_cumsum, C, states, D=None, z=None):
+def chunk_scan(cb, x, dt, dA_cumsum, C, states, D=None, z=None, round_to=None):
     """out[m,p] = exp(dA_m) * sum_n C[m,n] prev[p,n]
                  + sum_{k<=m} cb[m,k] exp(min(dA_m - dA_k, 0)) dt_k x[k,p]  + D x,  then the z gate.
-    Returns (out, out_x) with out_x the value before gating (None without z)."""
+    Returns (out, out_x) with out_x the value before gating (None without z).  With round_to the
+    weighted cb and prev are rounded to that type first (mamba_scan_fwd.py:97,137)."""
     b, L, nh, p = x.shape
     _, _, nc, Q = dt.shape
     g, n = C.shape[2], C.shape[3]
@@ -148,9 +156,9 @@ def chunk_scan(cb, x, dt, dA_cumsum, C, states, D=None, z=None):
     decay = torch.exp(torch.clamp(dA[..., :, None] - dA[..., None, :], max=0.0))
     mask = torch.tril(torch.ones(Q, Q, dtype=torch.bool))
     w = cbh * decay * dtc[..., None, :]
-    w = torch.where(mask, w, w.new_zeros(()))
+    w = _round(torch.where(mask, w, w.new_zeros(())), round_to)
     out = torch.einsum("bchmk,bckhp->bcmhp", w, xc)
-    out = out + torch.einsum("bcmhn,bchpn,bchm->bcmhp", Cc, _up(states), torch.exp(dA))
+    out = out + torch.einsum("bcmhn,bchpn,bchm->bcmhp", Cc, _round(_up(states), round_to), torch.exp(dA))
     out = out.reshape(b, nc * Q, nh, p)[:, :L]
     if D is not None:
         out = out + (_up(D)[None, None, :, None] if D.dim() == 1 else _up(D)[None, None]) * _up(x)
@@ -162,18 +170,18 @@ def chunk_scan(cb, x, dt, dA_cumsum, C, states, D=None, z=None):
 
 
 def combined_fwd(x, dt, A, B, C, Q, D=None, z=None, dt_bias=None, initial_states=None,
-                 dt_softplus=False, dt_limit=(0.0, float("inf"))):
+                 dt_softplus=False, dt_limit=(0.0, float("inf")), round_to=None):
     """The five stages in the order of mamba_ssm's combined forward, which the reference's
     kernels/mamba_kernels/ files were taken from.  Returns (out, final_states)."""
     b, L, nh, p = x.shape
     n = B.shape[-1]
     dA_cs, dt_out = chunk_cumsum(dt, A, Q, dt_bias, dt_softplus, dt_limit)
-    states = chunk_state(B, x, dt_out, dA_cs)
+    states = chunk_state(B, x, dt_out, dA_cs, round_to)
     init = None if initial_states is None else initial_states.reshape(b, nh, p * n)
     prev, final = state_passing(states.reshape(b, -1, nh, p * n), dA_cs[..., -1], init)
     prev = prev.reshape(b, -1, nh, p, n)
     cb = bmm_chunk(C, B, Q)
-    out, _ = chunk_scan(cb, x, dt_out, dA_cs, C, prev, D, z)
+    out, _ = chunk_scan(cb, x, dt_out, dA_cs, C, prev, D, z, round_to)
     return out, final.reshape(b, nh, p, n)
 
 

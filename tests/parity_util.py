@@ -21,8 +21,11 @@ def announce(msg):
     sys.stdout.flush()
 
 
-def check_close(name, got, ref, dtype):
-    """Asserts got ~= ref under the bar for `dtype` and prints the measured error."""
+def check_close(name, got, ref, dtype, loose=False):
+    """Asserts got ~= ref under the bar for `dtype` and prints the measured error.  With
+    loose the absolute term of the bfloat16 bar becomes 1 % of the largest reference magnitude:
+    for comparisons with a reference that skips roundings the checked arithmetic is required
+    to make (the tight comparison is then the one with a reference that makes them too)."""
     got = got.detach().float().cpu()
     ref = ref.detach().float().cpu()
     assert got.shape == ref.shape, (name, got.shape, ref.shape)
@@ -32,6 +35,8 @@ def check_close(name, got, ref, dtype):
         atol, rtol = F32_ATOL_REL * scale, F32_RTOL
     else:
         atol, rtol = BF16_ATOL, BF16_RTOL
+        if loose:
+            atol = max(atol, 1e-2 * scale)
     err = (got - ref).abs()
     bound = atol + rtol * ref.abs()
     worst = float((err / bound).max())

@@ -1,0 +1,136 @@
+"""GPU parity of the Mamba-2 SSD forward stages (through the C ABI) against the CPU oracle:
+each stage against its restatement on the same inputs, the five stages together against the
+sequential state-space recurrence, and BASELINE configuration 5 at full size through one
+sequence checked against the recurrence plus chunk-size invariance for the rest."""
+import pytest
+import torch
+
+from oracle import ssd_oracle as S
+from parity_util import announce, check_close
+
+pytestmark = pytest.mark.gpu
+
+F32, BF16 = torch.float32, torch.bfloat16
+
+
+def _dev(device, *ts):
+    return [None if t is None else t.to(device) for t in ts]
+
+
+CASES = [
+    # b, L, nh, P, g, N, Q
+    (2, 300, 4, 64, 1, 64, 64),
+    (1, 256, 2, 64, 2, 128, 128),
+    (2, 200, 4, 64, 1, 128, 256),   # one ragged chunk
+    (1, 520, 2, 128, 1, 64, 128),
+    (1, 130, 2, 128, 2, 128, 64),
+]
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("b,L,nh,P,g,N,Q", CASES)
+def test_stages_vs_oracle(b, L, nh, P, g, N, Q, dtype, device):
+    from kernels.mamba_kernels.mamba_bmm import _bmm_chunk_fwd
+    from kernels.mamba_kernels.mamba_cumsum import _chunk_cumsum_fwd
+    from kernels.mamba_kernels.mamba_scan_fwd import _chunk_scan_fwd
+    from kernels.mamba_kernels.mamba_state_fwd import _chunk_state_fwd
+    from kernels.mamba_kernels.mamba_state_pass import _state_passing_fwd
+
+    announce(f"ssd stages b{b} L{L} nh{nh} P{P} g{g} N{N} Q{Q} {dtype}")
+    x, dt_raw, A, B, C, D, z = S.make_inputs(b, L, nh, P, g, N, seed=L + N + Q, dtype=dtype, with_z=True)
+    gen = torch.Generator().manual_seed(3)
+    bias = torch.randn(nh, generator=gen) * 0.1
+    init = torch.randn(b, nh, P * N, generator=gen)
+    xd, dtd, Ad, Bd, Cd, Dd, zd, biasd, initd = _dev(device, x, dt_raw, A, B, C, D, z, bias, init)
+    small = F32 if dtype == F32 else BF16
+
+    # stage 1 (dt given before softplus so that the option is exercised)
+    pre = torch.log(torch.expm1(dt_raw)) - bias
+    dA_ref, dt_ref = S.chunk_cumsum(pre, A, Q, bias, True, (1e-3, 0.5))
+    dA_cs, dt_out = _chunk_cumsum_fwd(pre.to(device), Ad, Q, dt_bias=biasd, dt_softplus=True, dt_limit=(1e-3, 0.5))
+    check_close("dt_out", dt_out, dt_ref, F32)
+    check_close("dA_cumsum", dA_cs, dA_ref, F32)
+
+    # the later stages take the oracle's intermediates, so each is checked on its own
+    dA_d, dt_d = dA_ref.to(device), dt_ref.to(device)
+    rt = None if dtype == F32 else dtype  # the roundings the reference applies before its dots
+    st_ref = S.chunk_state(B, x, dt_ref, dA_ref, round_to=rt)
+    st = _chunk_state_fwd(Bd, xd, dt_d, dA_d)
+    check_close("states", st, st_ref, small)
+
+    prev_ref, fin_ref = S.state_passing(st_ref.reshape(b, -1, nh, P * N), dA_ref[..., -1], init)
+    prev, fin = _state_passing_fwd(st_ref.reshape(b, -1, nh, P * N).to(device), dA_d[..., -1], initial_states=initd)
+    check_close("prev states", prev, prev_ref, F32)
+    check_close("final states", fin, fin_ref, F32)
+
+    cb_ref = S.bmm_chunk(C, B, Q)
+    cb = _bmm_chunk_fwd(Cd, Bd, Q, output_dtype=torch.float32)
+    check_close("CB", cb, cb_ref, small)
+    if dtype == BF16:
+        check_close("CB (bf16 out)", _bmm_chunk_fwd(Cd, Bd, Q), cb_ref, BF16)
+
+    prev5 = prev_ref.reshape(b, -1, nh, P, N)
+    out_ref, outx_ref = S.chunk_scan(cb_ref, x, dt_ref, dA_ref, C, prev5, D, z, round_to=rt)
+    out, out_x = _chunk_scan_fwd(cb_ref.to(device), xd, dt_d, dA_d, Cd, prev5.to(device), D=Dd, z=zd)
+    check_close("out_x", out_x, outx_ref, dtype)
+    check_close("out", out, out_ref, dtype)
+    D2 = torch.randn(nh, P, generator=gen)
+    out_ref2, _ = S.chunk_scan(cb_ref, x, dt_ref, dA_ref, C, prev5, D2, None, round_to=rt)
+    out2, none = _chunk_scan_fwd(cb_ref.to(device), xd, dt_d, dA_d, Cd, prev5.to(device), D=D2.to(device))
+    assert none is None
+    check_close("out (D per feature, no gate)", out2, out_ref2, dtype)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("b,L,nh,P,g,N,Q", CASES)
+def test_combined_vs_recurrence(b, L, nh, P, g, N, Q, dtype, device):
+    from kernels.mamba_kernels.mamba_combined_fwd import mamba_chunk_scan_combined_fwd
+
+    announce(f"ssd combined b{b} L{L} nh{nh} P{P} g{g} N{N} Q{Q} {dtype}")
+    x, dt, A, B, C, D, z = S.make_inputs(b, L, nh, P, g, N, seed=7 + L + Q, dtype=dtype, with_z=True)
+    init = torch.randn(b, nh, P, N, generator=torch.Generator().manual_seed(4))
+    y_ref, fin_ref = S.ssd_loop(x.float(), dt, A, B.float(), C.float(), D, z.float(), init)
+    xd, dtd, Ad, Bd, Cd, Dd, zd, initd = _dev(device, x, dt, A, B, C, D, z, init)
+    y, fin = mamba_chunk_scan_combined_fwd(xd, dtd, Ad, Bd, Cd, Q, D=Dd, z=zd, initial_states=initd,
+                                           return_final_states=True)
+    torch.cuda.synchronize()
+    # The kernels round the weighted B, the weighted CB and the carried states to bf16 before the
+    # products, as the reference does; the recurrence rounds nothing, so it gets the loose bar and
+    # the chunked oracle that makes the same roundings gets the tight one.
+    if dtype == BF16:
+        y_rnd, fin_rnd = S.combined_fwd(x, dt, A, B, C, Q, D=D, z=z, initial_states=init, round_to=BF16)
+        check_close("y vs chunked oracle with the reference's roundings", y, y_rnd, BF16)
+        check_close("final states, same", fin, fin_rnd, BF16)
+    check_close("y", y, y_ref, dtype, loose=True)
+    check_close("final states", fin, fin_ref, F32 if dtype == F32 else BF16, loose=True)
+
+
+def test_unsupported_shapes_are_refused(device):
+    from kernels.mamba_kernels.mamba_state_fwd import _chunk_state_fwd
+
+    x = torch.zeros(1, 64, 2, 48, device=device)
+    B = torch.zeros(1, 64, 1, 64, device=device)
+    dt = torch.zeros(1, 2, 1, 64, device=device)
+    with pytest.raises(NotImplementedError):
+        _chunk_state_fwd(B, x, dt, dt)
+    with pytest.raises(NotImplementedError):
+        _chunk_state_fwd(B, torch.zeros(1, 64, 2, 64, device=device), dt, dt, seq_idx=torch.zeros(1, 64))
+
+
+def test_config5_full_size(device):
+    """b8 nh32 hdim64 dstate128 g1 L8192 Q256 bf16, D = 0: batch element 0 against the sequential
+    recurrence, every element against the same computation at chunk size 128."""
+    from kernels.mamba_kernels.mamba_combined_fwd import mamba_chunk_scan_combined_fwd
+
+    announce("ssd config 5 full size")
+    b, L, nh, P, g, N = 8, 8192, 32, 64, 1, 128
+    x, dt, A, B, C, _, _ = S.make_inputs(b, L, nh, P, g, N, seed=5, dtype=BF16)
+    xd, dtd, Ad, Bd, Cd = _dev(device, x, dt, A, B, C)
+    y256, fin256 = mamba_chunk_scan_combined_fwd(xd, dtd, Ad, Bd, Cd, 256, return_final_states=True)
+    y128, fin128 = mamba_chunk_scan_combined_fwd(xd, dtd, Ad, Bd, Cd, 128, return_final_states=True)
+    torch.cuda.synchronize()
+    check_close("chunk 256 vs chunk 128", y256, y128.float(), BF16, loose=True)
+    check_close("final states 256 vs 128", fin256, fin128, BF16, loose=True)
+    y_ref, fin_ref = S.ssd_loop(x[:1].float(), dt[:1], A, B[:1].float(), C[:1].float())
+    check_close("y[0] vs recurrence", y256[:1], y_ref, BF16, loose=True)
+    check_close("final[0] vs recurrence", fin256[:1], fin_ref, BF16, loose=True)

@@ -1,10 +1,11 @@
-"""Builds lib/libema_hip.so (gfx950) from csrc/ with hipcc.  Usage: python build.py"""
+"""Builds lib/libema_hip.so (gfx950) from csrc/ with hipcc: the EMA scan (ema_abi.hip) and the
+SSD forward stages (ssd_abi.hip).  Usage: python build.py"""
 import os
 import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SRC = os.path.join(HERE, "csrc", "ema_abi.hip")
+SRC = [os.path.join(HERE, "csrc", "ema_abi.hip"), os.path.join(HERE, "csrc", "ssd_abi.hip")]
 OUT = os.path.join(HERE, "lib", "libema_hip.so")
 
 FLAGS = [
@@ -21,7 +22,7 @@ FLAGS = [
 def build(verbose: bool = True) -> str:
     os.makedirs(os.path.dirname(OUT), exist_ok=True)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + FLAGS + ["-o", OUT, SRC]
+    cmd = [hipcc] + FLAGS + ["-o", OUT] + SRC
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)

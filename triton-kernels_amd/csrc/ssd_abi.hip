@@ -1,0 +1,244 @@
+// C ABI of the SSD forward stages: argument validation and kernel launches.  Declarations and
+// the reference launcher each entry point replaces are in include/ssd_hip.h.
+#include "../../include/ssd_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include "ssd_kernels.h"
+
+using namespace ssd;
+
+namespace {
+
+#define SSD_TRY(expr)            \
+  do {                           \
+    int _s = (expr);             \
+    if (_s != SSD_OK) return _s; \
+  } while (0)
+
+inline int launched() { return hipGetLastError() == hipSuccess ? SSD_OK : SSD_ERR_LAUNCH; }
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+inline int esize(int dtype) { return dtype == SSD_BF16 ? 2 : 4; }
+inline int check_dtype(int dtype) { return (dtype == SSD_F32 || dtype == SSD_BF16) ? SSD_OK : SSD_ERR_DTYPE; }
+
+// A tensor read or written in 16-byte pieces along its dense last axis of `inner` elements.
+int check_vec(const void* p, int64_t sb, int64_t sl, int64_t sh, int dtype, int64_t inner) {
+  if (!p) return SSD_ERR_NULL;
+  const int epl = 16 / esize(dtype);
+  if (inner % epl || sb % epl || sl % epl || sh % epl) return SSD_ERR_ALIGN;
+  if (reinterpret_cast<uintptr_t>(p) % 16) return SSD_ERR_ALIGN;
+  return SSD_OK;
+}
+int check_f32(const void* p) {
+  if (!p) return SSD_ERR_NULL;
+  return reinterpret_cast<uintptr_t>(p) % 16 ? SSD_ERR_ALIGN : SSD_OK;
+}
+
+struct Dims {
+  int64_t batch, L, nh, g, P, N, Q, C;
+};
+int check_dims(int64_t batch, int64_t L, int64_t nh, int64_t g, int64_t P, int64_t N, int64_t Q, Dims* d) {
+  if (batch <= 0 || L <= 0 || nh <= 0 || g <= 0 || Q <= 0) return SSD_ERR_SHAPE;
+  if (nh % g) return SSD_ERR_SHAPE;
+  if (Q > 1024 || Q % 4) return SSD_ERR_UNSUPPORTED;
+  if (batch > (1 << 20) || nh > (1 << 16) || L > ((int64_t)1 << 30)) return SSD_ERR_SHAPE;
+  *d = Dims{batch, L, nh, g, P, N, Q, (L + Q - 1) / Q};
+  if (batch * nh * d->C > ((int64_t)1 << 28)) return SSD_ERR_SHAPE;
+  return SSD_OK;
+}
+inline bool dim_ok(int64_t v) { return v == 64 || v == 128; }
+
+template <typename K>
+int allow_smem(K kernel, int bytes) {
+  if (bytes <= 64 * 1024) return SSD_OK;
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                             bytes) == hipSuccess
+             ? SSD_OK
+             : SSD_ERR_LAUNCH;
+}
+
+// Calls f.template run<T, P, N>() for the runtime (dtype, hdim, dstate).
+template <typename F>
+int dispatch_tpn(int dtype, int64_t P, int64_t N, F f) {
+  if (dtype == SSD_BF16) {
+    if (P == 64 && N == 64) return f.template run<bf16_t, 64, 64>();
+    if (P == 64 && N == 128) return f.template run<bf16_t, 64, 128>();
+    if (P == 128 && N == 64) return f.template run<bf16_t, 128, 64>();
+    return f.template run<bf16_t, 128, 128>();
+  }
+  if (P == 64 && N == 64) return f.template run<float, 64, 64>();
+  if (P == 64 && N == 128) return f.template run<float, 64, 128>();
+  if (P == 128 && N == 64) return f.template run<float, 128, 64>();
+  return f.template run<float, 128, 128>();
+}
+
+struct StateLaunch {
+  const void *x, *B;
+  Strides3 sx, sB;
+  const float *dt, *dA;
+  float* states;
+  Dims d;
+  hipStream_t st;
+  template <typename T, int P, int N>
+  int run() const {
+    auto kernel = ssd_chunk_state_kernel<T, P, N>;
+    constexpr int smem = StateSmem<T, P, N>::kBytes;
+    SSD_TRY(allow_smem(kernel, smem));
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh)), dim3(256), smem, st, (const T*)x, sx,
+                       (const T*)B, sB, dt, dA, states, (int)d.nh, (int)(d.nh / d.g), (int)d.L, (int)d.Q,
+                       (int)d.C);
+    return launched();
+  }
+};
+
+struct ScanLaunch {
+  const float* cb;
+  const void *x, *z, *C;
+  Strides3 sx, sz, sC, so;
+  const float *dt, *dA, *prev, *D;
+  int d_has_hdim;
+  void *out, *out_x;
+  Dims d;
+  hipStream_t st;
+  template <typename T, int P, int N>
+  int run() const {
+    auto kernel = ssd_chunk_scan_kernel<T, P, N>;
+    constexpr int smem = ScanSmem<T, P, N>::kBytes;
+    SSD_TRY(allow_smem(kernel, smem));
+    const int mtiles = (int)((d.Q + 63) / 64);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh * mtiles)), dim3(256), smem, st, cb,
+                       (const T*)x, sx, (const T*)z, sz, dt, dA, (const T*)C, sC, prev, D, d_has_hdim, (T*)out, so,
+                       (T*)out_x, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C, mtiles);
+    return launched();
+  }
+};
+
+template <typename T, typename TO, int K>
+int launch_bmm(const void* a, Strides3 sa, const void* bm, Strides3 sb, void* out, const Dims& d, hipStream_t st) {
+  auto kernel = ssd_bmm_kernel<T, TO, K>;
+  constexpr int smem = bmm_smem_bytes<T, K>();
+  SSD_TRY(allow_smem(kernel, smem));
+  const int tiles = (int)((d.Q + 63) / 64);
+  const int64_t grid = d.batch * d.C * d.g * tiles * tiles;
+  if (grid > 0x7fffffff) return SSD_ERR_SHAPE;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), smem, st, (const T*)a, sa, (const T*)bm, sb, (TO*)out,
+                     (int)d.g, (int)d.L, (int)d.Q, (int)d.C, tiles);
+  return launched();
+}
+
+}  // namespace
+
+extern "C" {
+
+int ssd_chunk_cumsum_fwd(const void* dt, int dt_dtype, int64_t dt_sb, int64_t dt_sl, int64_t dt_sh,
+                         const float* A, const float* dt_bias, float* dA_cumsum, float* dt_out,
+                         int64_t batch, int64_t seqlen, int64_t nheads, int64_t chunk, int dt_softplus,
+                         float dt_min, float dt_max, void* stream) {
+  Dims d;
+  SSD_TRY(check_dims(batch, seqlen, nheads, 1, 0, 0, chunk, &d));
+  SSD_TRY(check_dtype(dt_dtype));
+  if (!dt || !A || !dA_cumsum || !dt_out) return SSD_ERR_NULL;
+  const int64_t total = batch * nheads * d.C;
+  const Strides3 sd{dt_sb, dt_sl, dt_sh};
+  const unsigned grid = (unsigned)((total + 3) / 4);
+  if (dt_dtype == SSD_BF16)
+    hipLaunchKernelGGL(ssd_cumsum_kernel<bf16_t>, dim3(grid), dim3(256), 0, as_stream(stream), (const bf16_t*)dt,
+                       sd, A, dt_bias, dA_cumsum, dt_out, (int)nheads, (int)seqlen, (int)chunk, (int)d.C,
+                       dt_softplus, dt_min, dt_max, total);
+  else
+    hipLaunchKernelGGL(ssd_cumsum_kernel<float>, dim3(grid), dim3(256), 0, as_stream(stream), (const float*)dt, sd,
+                       A, dt_bias, dA_cumsum, dt_out, (int)nheads, (int)seqlen, (int)chunk, (int)d.C, dt_softplus,
+                       dt_min, dt_max, total);
+  return launched();
+}
+
+int ssd_chunk_state_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64_t b_sg, const void* x,
+                        int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, const float* dt,
+                        const float* dA_cumsum, float* states, int64_t batch, int64_t seqlen,
+                        int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
+                        void* stream) {
+  Dims d;
+  SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
+  SSD_TRY(check_dtype(dtype));
+  if (!dim_ok(hdim) || !dim_ok(dstate)) return SSD_ERR_UNSUPPORTED;
+  SSD_TRY(check_vec(x, x_sb, x_sl, x_sh, dtype, hdim));
+  SSD_TRY(check_vec(B, b_sb, b_sl, b_sg, dtype, dstate));
+  if (!dt || !dA_cumsum) return SSD_ERR_NULL;
+  SSD_TRY(check_f32(states));
+  return dispatch_tpn(dtype, hdim, dstate,
+                      StateLaunch{x, B, Strides3{x_sb, x_sl, x_sh}, Strides3{b_sb, b_sl, b_sg}, dt, dA_cumsum,
+                                  states, d, as_stream(stream)});
+}
+
+int ssd_state_passing_fwd(const float* states, const float* dA_chunk, int64_t da_sb, int64_t da_sh,
+                          int64_t da_sc, const float* initial, float* out, float* final_states,
+                          int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, void* stream) {
+  if (batch <= 0 || nchunks <= 0 || nheads <= 0 || dim <= 0) return SSD_ERR_SHAPE;
+  if (dim % 4) return SSD_ERR_ALIGN;
+  if (!dA_chunk) return SSD_ERR_NULL;
+  SSD_TRY(check_f32(states));
+  SSD_TRY(check_f32(out));
+  SSD_TRY(check_f32(final_states));
+  if (initial) SSD_TRY(check_f32(initial));
+  const int tiles = (int)((dim + 1023) / 1024);
+  const int64_t grid = batch * nheads * tiles;
+  if (grid > 0x7fffffff || dim > (1 << 24)) return SSD_ERR_SHAPE;
+  hipLaunchKernelGGL(ssd_state_passing_kernel, dim3((unsigned)grid), dim3(256), 0, as_stream(stream), states,
+                     dA_chunk, da_sb, da_sh, da_sc, initial, out, final_states, (int)nheads, (int)nchunks, (int)dim,
+                     tiles);
+  return launched();
+}
+
+int ssd_bmm_chunk_fwd(const void* a, int64_t a_sb, int64_t a_sl, int64_t a_sg, const void* bm,
+                      int64_t b_sb, int64_t b_sl, int64_t b_sg, int dtype, void* out, int out_dtype,
+                      int64_t batch, int64_t seqlen, int64_t ngroups, int64_t k, int64_t chunk,
+                      void* stream) {
+  Dims d;
+  SSD_TRY(check_dims(batch, seqlen, ngroups, ngroups, 0, k, chunk, &d));
+  SSD_TRY(check_dtype(dtype));
+  SSD_TRY(check_dtype(out_dtype));
+  if (!dim_ok(k)) return SSD_ERR_UNSUPPORTED;
+  if (out_dtype != SSD_F32 && out_dtype != dtype) return SSD_ERR_DTYPE;
+  SSD_TRY(check_vec(a, a_sb, a_sl, a_sg, dtype, k));
+  SSD_TRY(check_vec(bm, b_sb, b_sl, b_sg, dtype, k));
+  if (!out) return SSD_ERR_NULL;
+  const Strides3 sa{a_sb, a_sl, a_sg}, sb{b_sb, b_sl, b_sg};
+  hipStream_t st = as_stream(stream);
+  if (dtype == SSD_BF16) {
+    if (out_dtype == SSD_F32)
+      return k == 64 ? launch_bmm<bf16_t, float, 64>(a, sa, bm, sb, out, d, st)
+                     : launch_bmm<bf16_t, float, 128>(a, sa, bm, sb, out, d, st);
+    return k == 64 ? launch_bmm<bf16_t, bf16_t, 64>(a, sa, bm, sb, out, d, st)
+                   : launch_bmm<bf16_t, bf16_t, 128>(a, sa, bm, sb, out, d, st);
+  }
+  return k == 64 ? launch_bmm<float, float, 64>(a, sa, bm, sb, out, d, st)
+                 : launch_bmm<float, float, 128>(a, sa, bm, sb, out, d, st);
+}
+
+int ssd_chunk_scan_fwd(const float* cb, const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
+                       const void* z, int64_t z_sb, int64_t z_sl, int64_t z_sh, int dtype,
+                       const float* dt, const float* dA_cumsum, const void* C, int64_t c_sb, int64_t c_sl,
+                       int64_t c_sg, const float* prev_states, const float* D, int d_has_hdim, void* out,
+                       int64_t o_sb, int64_t o_sl, int64_t o_sh, void* out_x, int64_t batch,
+                       int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate,
+                       int64_t chunk, void* stream) {
+  Dims d;
+  SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
+  SSD_TRY(check_dtype(dtype));
+  if (!dim_ok(hdim) || !dim_ok(dstate)) return SSD_ERR_UNSUPPORTED;
+  SSD_TRY(check_vec(x, x_sb, x_sl, x_sh, dtype, hdim));
+  SSD_TRY(check_vec(out, o_sb, o_sl, o_sh, dtype, hdim));
+  SSD_TRY(check_vec(C, c_sb, c_sl, c_sg, dtype, dstate));
+  if (z) SSD_TRY(check_vec(z, z_sb, z_sl, z_sh, dtype, hdim));
+  if (out_x && reinterpret_cast<uintptr_t>(out_x) % 16) return SSD_ERR_ALIGN;
+  if (!dt || !dA_cumsum) return SSD_ERR_NULL;
+  SSD_TRY(check_f32(cb));
+  SSD_TRY(check_f32(prev_states));
+  if (batch * d.C * nheads * ((chunk + 63) / 64) > 0x7fffffff) return SSD_ERR_SHAPE;
+  return dispatch_tpn(dtype, hdim, dstate,
+                      ScanLaunch{cb, x, z, C, Strides3{x_sb, x_sl, x_sh}, Strides3{z_sb, z_sl, z_sh},
+                                 Strides3{c_sb, c_sl, c_sg}, Strides3{o_sb, o_sl, o_sh}, dt, dA_cumsum,
+                                 prev_states, D, d_has_hdim, out, out_x, d, as_stream(stream)});
+}
+
+}  // extern "C"

@@ -1,0 +1,484 @@
+// Forward kernels of the Mamba-2 SSD chunked scan (gfx950, wave64).
+//
+// Five stages, one kernel each, with the tensor layouts of the reference's launchers in
+// kernels/mamba_kernels/:
+//   chunk_cumsum   dt -> processed dt and the per-chunk cumsum of dt * A        (DPP scan)
+//   chunk_state    states[p][n] = sum_k x[k][p] * (B[k][n] * w_k)               (MFMA)
+//   state_passing  the inter-chunk recurrence over (hdim x dstate) states       (HBM stream)
+//   bmm_chunk      CB[m][k] = sum_n C[m][n] * B[k][n]                           (MFMA)
+//   chunk_scan     out = exp(dA_m) * C.prev + (CB o decay o dt, causal) x + D x (MFMA)
+//
+// MFMA operands are staged in LDS.  A tile that is contracted along its rows (x[k][p],
+// B[k][n]) is read with the transposing LDS read for bf16 (four scalar reads for f32); a tile
+// contracted along its columns (C[m][n], prev[p][n], the weighted CB[m][k]) is read with one
+// 16-byte LDS read per lane.  Accumulation is float32 throughout; operands that the reference
+// rounds to the input type before its dot (the weighted B, the weighted CB, prev) are rounded
+// the same way here.
+#pragma once
+#include <type_traits>
+
+#include "ema_device.h"
+
+namespace ssd {
+
+using ema::acc_row;
+using ema::bf16_t;
+using ema::floatx16;
+using ema::load16;
+using ema::mma_group;
+using ema::store16;
+using ema::Vec16;
+using ema::wave_inclusive_scan;
+
+// Element strides of a (batch, position, head-or-group) tensor whose last axis is dense.
+struct Strides3 {
+  int64_t sb, sl, sh;
+};
+
+// ------------------------------------------------------------------ operand fragments
+// Both return, for lane l, EPL = Vec16<T>::N consecutive contraction indices starting at
+// k0 + EPL * (l / 32), for row or column (l % 32) of the 32-wide block: the register layout
+// mma_group expects for either operand.
+
+// tile[row][k], contracted along k (row-major)
+template <typename T>
+__device__ __forceinline__ Vec16<T> frag_rows(const T* tile, int pitch, int row0, int k0, int lane) {
+  return load16(tile + (row0 + (lane & 31)) * pitch + k0 + Vec16<T>::N * (lane >> 5));
+}
+
+// tile[k][col], contracted along k (k-major)
+__device__ __forceinline__ Vec16<bf16_t> frag_cols(const bf16_t* tile, int pitch, int k0, int col0,
+                                                   int lane) {
+  return ema::lds_read_kmajor(tile, pitch, k0, col0, lane);
+}
+__device__ __forceinline__ Vec16<float> frag_cols(const float* tile, int pitch, int k0, int col0,
+                                                  int lane) {
+  const float* p = tile + (k0 + 4 * (lane >> 5)) * pitch + col0 + (lane & 31);
+  Vec16<float> r;
+  r.raw = make_float4(p[0], p[pitch], p[2 * pitch], p[3 * pitch]);
+  return r;
+}
+
+template <typename T>
+struct Tile {
+  static constexpr int EPL = Vec16<T>::N;
+  static constexpr int KG = 2 * EPL;  // contraction extent of one mma_group
+  // LDS pitch (elements) of a tile with `cols` dense columns: 16 bytes of padding
+  static constexpr int pitch(int cols) { return cols + EPL; }
+};
+
+__device__ __forceinline__ void zero_acc(floatx16& a) {
+#pragma unroll
+  for (int v = 0; v < 16; ++v) a[v] = 0.f;
+}
+
+// Rows [row0, row0 + ROWS) x COLS dense columns of a global tensor into an LDS tile, 16 bytes
+// per thread and step; rows at or past `limit` read as zero.  A `scale` other than NoScale
+// multiplies row r by scale(r) in float32 before the value is rounded to T.
+struct NoScale {
+  __device__ __forceinline__ float operator()(int) const { return 1.f; }
+};
+
+template <typename T, int ROWS, int COLS, typename F>
+__device__ __forceinline__ void stage_rows(T* tile, const T* __restrict__ g, int64_t row_stride, int row0,
+                                           int limit, int tid, F scale) {
+  constexpr int EPL = Vec16<T>::N, VPR = COLS / EPL, P = Tile<T>::pitch(COLS);
+  static_assert((ROWS * VPR) % 256 == 0, "tile must split evenly over 256 threads");
+#pragma unroll
+  for (int i = 0; i < ROWS * VPR / 256; ++i) {
+    const int idx = tid + 256 * i;
+    const int r = idx / VPR, cv = (idx % VPR) * EPL;
+    Vec16<T> v;
+    if (row0 + r < limit) {
+      v = load16(g + (int64_t)(row0 + r) * row_stride + cv);
+      if constexpr (!std::is_same<F, NoScale>::value) {
+        const float s = scale(row0 + r);
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) v.set(e, v.get(e) * s);
+      }
+    } else {
+      v.zero();
+    }
+    store16(tile + r * P + cv, v);
+  }
+}
+// ------------------------------------------------------------------------------------
+// chunk_cumsum.  One wave per (b, c, h).  dt is processed (bias, softplus with the identity
+// above 20, clamp), positions past the sequence give 0; dA = dt * A[h] is scanned across the
+// chunk with DPP.  Outputs are (b, nh, C, Q) float32.
+// ------------------------------------------------------------------------------------
+template <typename TD>
+__global__ __launch_bounds__(256) void ssd_cumsum_kernel(const TD* __restrict__ dt, Strides3 sd,
+                                                         const float* __restrict__ A,
+                                                         const float* __restrict__ dt_bias,
+                                                         float* __restrict__ dA_cs, float* __restrict__ dt_out,
+                                                         int nh, int L, int Q, int C, int softplus,
+                                                         float dt_min, float dt_max, int64_t total) {
+  const int lane = threadIdx.x & 63;
+  const int64_t id = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // ((b * nh) + h) * C + c
+  if (id >= total) return;
+  const int c = (int)(id % C);
+  const int64_t bh = id / C;
+  const int h = (int)(bh % nh);
+  const int64_t b = bh / nh;
+  const int per = (Q + 63) >> 6;
+  const int q0 = lane * per;
+  const int limit = min(Q, L - c * Q);
+  const TD* src = dt + b * sd.sb + h * sd.sh + (int64_t)c * Q * sd.sl;
+  const float a = A[h];
+  const float bias = dt_bias ? dt_bias[h] : 0.f;
+  auto value = [&](int q) {
+    if (q >= limit) return 0.f;
+    float v = (float)src[(int64_t)q * sd.sl] + bias;
+    if (softplus && v <= 20.f) v = log1pf(__expf(v));
+    return fminf(fmaxf(v, dt_min), dt_max);
+  };
+  float local = 0.f;
+  for (int i = 0; i < per; ++i) local += value(q0 + i) * a;
+  float run = wave_inclusive_scan(local) - local;
+  float* o_cs = dA_cs + id * Q;
+  float* o_dt = dt_out + id * Q;
+  for (int i = 0; i < per; ++i) {
+    const int q = q0 + i;
+    if (q < Q) {
+      const float v = value(q);
+      run += v * a;
+      o_dt[q] = v;
+      o_cs[q] = run;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// chunk_state.  One workgroup (4 waves) per (b, c, h):
+//   states[p][n] = sum_k x[k][p] * round_T(B[k][n] * exp(min(dA_last - dA_k, 0)) * dt_k).
+// The chunk is walked in stages of 64 rows; both operands are contracted along their rows.
+// The (P/32) x (N/32) output blocks are dealt to the waves round-robin.
+// ------------------------------------------------------------------------------------
+template <typename T, int P, int N>
+struct StateSmem {
+  static constexpr int KT = 64, PX = Tile<T>::pitch(P), PB = Tile<T>::pitch(N);
+  static constexpr int kBytes = KT * (PX + PB) * (int)sizeof(T);
+};
+
+template <typename T, int P, int N>
+__global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
+    const T* __restrict__ x, Strides3 sx, const T* __restrict__ B, Strides3 sB,
+    const float* __restrict__ dt, const float* __restrict__ dA_cs, float* __restrict__ states, int nh,
+    int heads_per_group, int L, int Q, int C) {
+  using S = StateSmem<T, P, N>;
+  constexpr int KT = S::KT, PX = S::PX, PB = S::PB, KG = Tile<T>::KG;
+  constexpr int MB = P / 32, NB = N / 32, BPW = MB * NB / 4;
+  static_assert(MB * NB % 4 == 0, "output blocks must split over 4 waves");
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T* xs = reinterpret_cast<T*>(smem);
+  T* bs = xs + KT * PX;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int h = blockIdx.x % nh;
+  const int c = (blockIdx.x / nh) % C;
+  const int64_t b = blockIdx.x / (nh * C);
+  const int limit = min(Q, L - c * Q);
+  const float* dAp = dA_cs + ((b * nh + h) * C + c) * (int64_t)Q;
+  const float* dtp = dt + ((b * nh + h) * C + c) * (int64_t)Q;
+  const float dA_last = dAp[Q - 1];
+  const T* xg = x + b * sx.sb + (int64_t)c * Q * sx.sl + h * sx.sh;
+  const T* Bg = B + b * sB.sb + (int64_t)c * Q * sB.sl + (h / heads_per_group) * sB.sh;
+
+  floatx16 acc[BPW];
+#pragma unroll
+  for (int i = 0; i < BPW; ++i) zero_acc(acc[i]);
+
+  for (int k0 = 0; k0 < limit; k0 += KT) {
+    stage_rows<T, KT, P>(xs, xg, sx.sl, k0, limit, tid, NoScale());
+    stage_rows<T, KT, N>(bs, Bg, sB.sl, k0, limit, tid, [&](int k) {
+      return __expf(fminf(dA_last - dAp[k], 0.f)) * dtp[k];
+    });
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < KT; kk += KG) {
+#pragma unroll
+      for (int i = 0; i < BPW; ++i) {
+        const int j = wave + 4 * i, mi = j % MB, ni = j / MB;
+        mma_group(frag_cols(xs, PX, kk, 32 * mi, lane), frag_cols(bs, PB, kk, 32 * ni, lane), acc[i]);
+      }
+    }
+    __syncthreads();
+  }
+  float* out = states + (((b * C + c) * nh + h) * (int64_t)P) * N;
+#pragma unroll
+  for (int i = 0; i < BPW; ++i) {
+    const int j = wave + 4 * i, mi = j % MB, ni = j / MB;
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+      out[(int64_t)(32 * mi + acc_row(v, lane)) * N + 32 * ni + (lane & 31)] = acc[i][v];
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// state_passing.  out[b, c] = state entering chunk c, state <- exp(dA_chunk[c]) * state +
+// states[b, c]; the value after the last chunk goes to final.  One thread per four adjacent
+// state elements, the running state in registers, chunks fetched four ahead.
+// states / out are (b, C, nh, dim) dense float32; dA_chunk is addressed by strides (it is the
+// last column of dA_cumsum).
+// ------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void ssd_state_passing_kernel(
+    const float* __restrict__ states, const float* __restrict__ dA_chunk, int64_t da_sb, int64_t da_sh,
+    int64_t da_sc, const float* __restrict__ initial, float* __restrict__ out, float* __restrict__ final_states,
+    int nh, int C, int dim, int tiles) {
+  const int tile = blockIdx.x % tiles;
+  const int h = (blockIdx.x / tiles) % nh;
+  const int64_t b = blockIdx.x / (tiles * nh);
+  const int e = (tile * 256 + threadIdx.x) * 4;
+  if (e >= dim) return;
+  const int64_t chunk_stride = (int64_t)nh * dim;
+  const float* src = states + (b * C * nh + h) * (int64_t)dim + e;
+  float* dst = out + (b * C * nh + h) * (int64_t)dim + e;
+  const float* da = dA_chunk + b * da_sb + h * da_sh;
+  float4 s = initial ? *reinterpret_cast<const float4*>(initial + (b * nh + h) * (int64_t)dim + e)
+                     : make_float4(0.f, 0.f, 0.f, 0.f);
+  constexpr int U = 4;
+  for (int c0 = 0; c0 < C; c0 += U) {
+    float4 nv[U];
+    float a[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = c0 + u;
+      nv[u] = c < C ? *reinterpret_cast<const float4*>(src + c * chunk_stride) : make_float4(0.f, 0.f, 0.f, 0.f);
+      a[u] = c < C ? __expf(da[(int64_t)c * da_sc]) : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = c0 + u;
+      if (c < C) {
+        *reinterpret_cast<float4*>(dst + c * chunk_stride) = s;
+        s.x = fmaf(a[u], s.x, nv[u].x);
+        s.y = fmaf(a[u], s.y, nv[u].y);
+        s.z = fmaf(a[u], s.z, nv[u].z);
+        s.w = fmaf(a[u], s.w, nv[u].w);
+      }
+    }
+  }
+  *reinterpret_cast<float4*>(final_states + (b * nh + h) * (int64_t)dim + e) = s;
+}
+
+// ------------------------------------------------------------------------------------
+// bmm_chunk.  out[b, c, g, m, k] = sum_n a[b, cQ+m, g, n] * bm[b, cQ+k, g, n]; one workgroup
+// per 64 x 64 output tile, one 32 x 32 block per wave; rows past the sequence are zero.
+// ------------------------------------------------------------------------------------
+template <typename T, int K>
+constexpr int bmm_smem_bytes() {
+  return 2 * 64 * Tile<T>::pitch(K) * (int)sizeof(T);
+}
+
+template <typename T, typename TO, int K>
+__global__ __launch_bounds__(256) void ssd_bmm_kernel(const T* __restrict__ a, Strides3 sa,
+                                                      const T* __restrict__ bm, Strides3 sb_,
+                                                      TO* __restrict__ out, int ngroups, int L, int Q, int C,
+                                                      int tiles) {
+  constexpr int PK = Tile<T>::pitch(K), KG = Tile<T>::KG;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T* as = reinterpret_cast<T*>(smem);
+  T* bs = as + 64 * PK;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tn = blockIdx.x % tiles;
+  const int tm = (blockIdx.x / tiles) % tiles;
+  const int64_t bcg = blockIdx.x / (tiles * tiles);
+  const int g = (int)(bcg % ngroups);
+  const int c = (int)((bcg / ngroups) % C);
+  const int64_t b = bcg / ((int64_t)ngroups * C);
+  const int limit = min(Q, L - c * Q);
+  stage_rows<T, 64, K>(as, a + b * sa.sb + (int64_t)c * Q * sa.sl + g * sa.sh, sa.sl, 64 * tm, limit, tid, NoScale());
+  stage_rows<T, 64, K>(bs, bm + b * sb_.sb + (int64_t)c * Q * sb_.sl + g * sb_.sh, sb_.sl, 64 * tn, limit, tid,
+                       NoScale());
+  __syncthreads();
+  const int wm = wave >> 1, wn = wave & 1;
+  floatx16 acc;
+  zero_acc(acc);
+#pragma unroll
+  for (int kk = 0; kk < K; kk += KG)
+    mma_group(frag_rows(as, PK, 32 * wm, kk, lane), frag_rows(bs, PK, 32 * wn, kk, lane), acc);
+  TO* o = out + bcg * (int64_t)Q * Q;
+  const int col = 64 * tn + 32 * wn + (lane & 31);
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int row = 64 * tm + 32 * wm + acc_row(v, lane);
+    if (row < Q && col < Q) o[(int64_t)row * Q + col] = (TO)acc[v];
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// chunk_scan.  One workgroup per (b, c, h, tile of 64 rows m):
+//   out[m][p] = exp(dA_m) * sum_n C[m][n] * round_T(prev[p][n])
+//             + sum_{k <= m} round_T(cb[m][k] * exp(min(dA_m - dA_k, 0)) * dt_k) * x[k][p]
+//             + D * x[m][p],            then out_x = out (if asked) and out *= z * sigmoid(z).
+// The causal sum walks the 64-row tiles k up to the diagonal one; the result leaves through an
+// LDS tile so that z, out and out_x move in 16-byte pieces.
+// cb is float32 (b, C, g, Q, Q); prev is float32 (b, C, nh, P, N).
+// ------------------------------------------------------------------------------------
+template <typename T, int P, int N>
+struct ScanSmem {
+  static constexpr int PC = Tile<T>::pitch(N), PX = Tile<T>::pitch(P), PW = Tile<T>::pitch(64), PO = P + 4;
+  static constexpr int kPhaseA = (64 + P) * PC * (int)sizeof(T);                 // C tile, prev tile
+  static constexpr int kPhaseB = (64 * PX + 64 * PW) * (int)sizeof(T);           // x tile, weights
+  static constexpr int kPhaseC = 64 * PO * (int)sizeof(float);                   // output staging
+  static constexpr int kMax1 = kPhaseA > kPhaseB ? kPhaseA : kPhaseB;
+  static constexpr int kBytes = (kMax1 > kPhaseC ? kMax1 : kPhaseC) + 64 * (int)sizeof(float);
+};
+
+template <typename T, int P, int N>
+__global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(
+    const float* __restrict__ cb, const T* __restrict__ x, Strides3 sx, const T* __restrict__ z, Strides3 sz,
+    const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Cm, Strides3 sC,
+    const float* __restrict__ prev, const float* __restrict__ D, int d_has_hdim, T* __restrict__ out,
+    Strides3 so, T* __restrict__ out_x, int nh, int heads_per_group, int ngroups, int L, int Q, int C,
+    int mtiles) {
+  using S = ScanSmem<T, P, N>;
+  constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, PB = P / 32, BPW = 2 * PB / 4;
+  static_assert(PB == 2 || PB == 4, "hdim 64 or 128");
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T* Cs = reinterpret_cast<T*>(smem);
+  T* Ps = Cs + 64 * S::PC;
+  T* Xs = reinterpret_cast<T*>(smem);
+  T* Ws = Xs + 64 * S::PX;
+  float* Os = reinterpret_cast<float*>(smem);
+  float* sm = reinterpret_cast<float*>(smem + S::kBytes - 64 * sizeof(float));  // exp(dA_m)
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int mt = blockIdx.x % mtiles;
+  const int h = (blockIdx.x / mtiles) % nh;
+  const int c = (blockIdx.x / (mtiles * nh)) % C;
+  const int64_t b = blockIdx.x / ((int64_t)mtiles * nh * C);
+  const int limit = min(Q, L - c * Q);
+  const int m0 = 64 * mt;
+  if (m0 >= limit) return;
+  const int g = h / heads_per_group;
+  const int64_t chunk = (b * nh + h) * C + c;
+  const float* dAp = dA_cs + chunk * Q;
+  const float* dtp = dt + chunk * Q;
+  const T* xg = x + b * sx.sb + (int64_t)c * Q * sx.sl + h * sx.sh;
+  const T* Cg = Cm + b * sC.sb + (int64_t)c * Q * sC.sl + g * sC.sh;
+  const float* pg = prev + (((b * C + c) * nh + h) * (int64_t)P) * N;
+  const float* cbg = cb + (((b * C + c) * ngroups + g) * (int64_t)Q) * Q;
+
+  // wave -> output blocks: rows 32*mi.., columns 32*(pi0 + 2*i)..
+  const int mi = wave & 1, pi0 = wave >> 1;
+  floatx16 acc[BPW];
+#pragma unroll
+  for (int i = 0; i < BPW; ++i) zero_acc(acc[i]);
+
+  // ---- phase A: C . prev, scaled by exp(dA_m)
+  stage_rows<T, 64, N>(Cs, Cg, sC.sl, m0, limit, tid, NoScale());
+  {
+    constexpr int VPR = N / 4;  // float4 per row of prev
+#pragma unroll
+    for (int i = 0; i < P * VPR / 256; ++i) {
+      const int idx = tid + 256 * i;
+      const int r = idx / VPR, cv = (idx % VPR) * 4;
+      const float4 v = *reinterpret_cast<const float4*>(pg + (int64_t)r * N + cv);
+      T* d = Ps + r * S::PC + cv;
+      d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
+    }
+  }
+  if (tid < 64) sm[tid] = m0 + tid < Q ? __expf(dAp[m0 + tid]) : 0.f;
+  __syncthreads();
+#pragma unroll
+  for (int kk = 0; kk < N; kk += KG) {
+    const Vec16<T> a = frag_rows(Cs, S::PC, 32 * mi, kk, lane);
+#pragma unroll
+    for (int i = 0; i < BPW; ++i) mma_group(a, frag_rows(Ps, S::PC, 32 * (pi0 + 2 * i), kk, lane), acc[i]);
+  }
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const float s = sm[32 * mi + acc_row(v, lane)];
+#pragma unroll
+    for (int i = 0; i < BPW; ++i) acc[i][v] *= s;
+  }
+  __syncthreads();
+
+  // ---- phase B: causal sum over the k tiles up to the diagonal one
+  for (int kt = 0; kt <= mt; ++kt) {
+    const int k0 = 64 * kt;
+    stage_rows<T, 64, P>(Xs, xg, sx.sl, k0, limit, tid, NoScale());
+    {
+      // weights: 64 x 64 float32 of cb -> scaled, masked, rounded to T; 16 float4 per row
+#pragma unroll
+      for (int i = 0; i < 64 * 16 / 256; ++i) {
+        const int idx = tid + 256 * i;
+        const int r = idx >> 4, cv = (idx & 15) * 4;
+        const int m = m0 + r;
+        T* d = Ws + r * S::PW + cv;
+        if (m < Q && k0 + cv < Q) {  // Q is a multiple of 4 (checked on the host)
+          const float4 w4 = *reinterpret_cast<const float4*>(cbg + (int64_t)m * Q + k0 + cv);
+          const float4 a4 = *reinterpret_cast<const float4*>(dAp + k0 + cv);
+          const float4 t4 = *reinterpret_cast<const float4*>(dtp + k0 + cv);
+          const float am = dAp[m];
+          const float w[4] = {w4.x, w4.y, w4.z, w4.w}, ak[4] = {a4.x, a4.y, a4.z, a4.w},
+                      tk[4] = {t4.x, t4.y, t4.z, t4.w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            d[e] = (T)(k0 + cv + e <= m ? w[e] * __expf(fminf(am - ak[e], 0.f)) * tk[e] : 0.f);
+        } else {
+          d[0] = d[1] = d[2] = d[3] = (T)0.f;
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 64; kk += KG) {
+      const Vec16<T> a = frag_rows(Ws, S::PW, 32 * mi, kk, lane);
+#pragma unroll
+      for (int i = 0; i < BPW; ++i) mma_group(a, frag_cols(Xs, S::PX, kk, 32 * (pi0 + 2 * i), lane), acc[i]);
+    }
+    if (kt == mt && D) {  // the diagonal tile holds rows m0.. of x: the skip term
+#pragma unroll
+      for (int i = 0; i < BPW; ++i) {
+        const int col = 32 * (pi0 + 2 * i) + (lane & 31);
+        const float dv = d_has_hdim ? D[h * P + col] : D[h];
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          acc[i][v] = fmaf(dv, (float)Xs[(32 * mi + acc_row(v, lane)) * S::PX + col], acc[i][v]);
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- phase C: through LDS to global memory, gate on the way
+#pragma unroll
+  for (int i = 0; i < BPW; ++i) {
+    const int col = 32 * (pi0 + 2 * i) + (lane & 31);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) Os[(32 * mi + acc_row(v, lane)) * S::PO + col] = acc[i][v];
+  }
+  __syncthreads();
+  constexpr int VPR = P / EPL;
+#pragma unroll
+  for (int i = 0; i < 64 * VPR / 256; ++i) {
+    const int idx = tid + 256 * i;
+    const int r = idx / VPR, cv = (idx % VPR) * EPL;
+    const int m = m0 + r;
+    if (m >= limit) continue;
+    const int64_t pos = (int64_t)c * Q + m;
+    float v[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) v[e] = Os[r * S::PO + cv + e];
+    Vec16<T> o;
+    if (z) {
+      if (out_x) {
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) o.set(e, v[e]);
+        store16(out_x + b * so.sb + pos * so.sl + h * so.sh + cv, o);
+      }
+      const Vec16<T> zv = load16(z + b * sz.sb + pos * sz.sl + h * sz.sh + cv);
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) {
+        const float zf = zv.get(e);
+        v[e] *= zf / (1.f + __expf(-zf));
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) o.set(e, v[e]);
+    store16(out + b * so.sb + pos * so.sl + h * so.sh + cv, o);
+  }
+}
+
+}  // namespace ssd

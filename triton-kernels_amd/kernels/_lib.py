@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 import torch
 
@@ -47,6 +47,12 @@ _SIGNATURES = {
     "ema_seq_bwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "ema_seq_fwd": (c_int, [c_int] + _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _P, _P, _P]),
     "ema_seq_bwd": (c_int, [c_int] + _SEQ + _SEQ + _SEQ + [_P, _P, c_int] + _SEQ + _SEQ + [_P, _P, c_size_t, _I, _I, _I, _I, _P, _P, _P]),
+    # SSD forward stages (include/ssd_hip.h)
+    "ssd_chunk_cumsum_fwd": (c_int, [_P, c_int, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, c_int, c_float, c_float, _P]),
+    "ssd_chunk_state_fwd": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "ssd_state_passing_fwd": (c_int, [_P, _P, _I, _I, _I, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "ssd_bmm_chunk_fwd": (c_int, _SEQ + _SEQ + [c_int, _P, c_int, _I, _I, _I, _I, _I, _P]),
+    "ssd_chunk_scan_fwd": (c_int, [_P] + _SEQ + _SEQ + [c_int, _P, _P] + _SEQ + [_P, _P, c_int] + _SEQ + [_P, _I, _I, _I, _I, _I, _I, _I, _P]),
 }
 
 _lib = None
@@ -141,6 +147,14 @@ def event_ptrs(events):
     if events is None:
         return None, None
     return events[0].cuda_event, events[1].cuda_event
+
+
+def strided4(t: torch.Tensor):
+    """(tensor with unit last stride, [ptr, s0, s1, s2]) of a 4-d tensor (b, l, h, inner)."""
+    assert t.dim() == 4
+    if t.stride(-1) != 1:
+        t = t.contiguous()
+    return t, [t.data_ptr(), t.stride(0), t.stride(1), t.stride(2)]
 
 
 def f32c(t: torch.Tensor) -> torch.Tensor:

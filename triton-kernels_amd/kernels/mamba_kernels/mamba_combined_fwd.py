@@ -1,0 +1,47 @@
+"""The five SSD forward stages in sequence.
+
+The reference ships the stage launchers of kernels/mamba_kernels/ without a wrapper that runs
+them together (its benchmarks call mamba_ssm's mamba_chunk_scan_combined instead, e.g.
+kernels/benchmarks/ema_bench.py:9); this function is that wrapper, with the argument names of
+the headed entry point in kernels/ema_combined.py:100-119."""
+import torch
+
+from kernels.mamba_kernels.mamba_bmm import _bmm_chunk_fwd
+from kernels.mamba_kernels.mamba_cumsum import _chunk_cumsum_fwd
+from kernels.mamba_kernels.mamba_scan_fwd import _chunk_scan_fwd
+from kernels.mamba_kernels.mamba_state_fwd import _chunk_state_fwd
+from kernels.mamba_kernels.mamba_state_pass import _state_passing_fwd
+
+
+def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
+                                   initial_states=None, seq_idx=None, dt_softplus=False,
+                                   dt_limit=(0.0, float("inf"))):
+    """Returns (out, out_x, dt_out, dA_cumsum, states, final_states)."""
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, ngroups, dstate = B.shape
+    assert nheads % ngroups == 0
+    assert B.shape == (batch, seqlen, ngroups, dstate) and C.shape == B.shape
+    assert dt.shape == (batch, seqlen, nheads) and A.shape == (nheads,)
+    if initial_states is not None:
+        assert initial_states.shape == (batch, nheads, headdim, dstate)
+    dA_cumsum, dt_out = _chunk_cumsum_fwd(dt, A, chunk_size, dt_bias=dt_bias, dt_softplus=dt_softplus,
+                                          dt_limit=dt_limit)
+    states = _chunk_state_fwd(B, x, dt_out, dA_cumsum, seq_idx=seq_idx, states_in_fp32=True)
+    init = None if initial_states is None else initial_states.reshape(batch, nheads, headdim * dstate)
+    states, final_states = _state_passing_fwd(states.reshape(batch, -1, nheads, headdim * dstate),
+                                              dA_cumsum[:, :, :, -1], initial_states=init, seq_idx=seq_idx,
+                                              chunk_size=chunk_size, out_dtype=torch.float32)
+    states = states.reshape(batch, -1, nheads, headdim, dstate)
+    final_states = final_states.reshape(batch, nheads, headdim, dstate)
+    CB = _bmm_chunk_fwd(C, B, chunk_size, seq_idx=seq_idx, output_dtype=torch.float32)
+    out, out_x = _chunk_scan_fwd(CB, x, dt_out, dA_cumsum, C, states, D=D, z=z, seq_idx=seq_idx)
+    return out, out_x, dt_out, dA_cumsum, states, final_states
+
+
+def mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
+                                  initial_states=None, dt_softplus=False, dt_limit=(0.0, float("inf")),
+                                  return_final_states=False):
+    out, _, _, _, _, final_states = _mamba_chunk_scan_combined_fwd(
+        x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, initial_states=initial_states,
+        dt_softplus=dt_softplus, dt_limit=dt_limit)
+    return (out, final_states) if return_final_states else out

@@ -1,0 +1,46 @@
+"""SSD stage 5: the chunk scan (carried state, causal intra-chunk sum, skip term, gate).
+
+Mirrors _chunk_scan_fwd, kernels/mamba_kernels/mamba_scan_fwd.py:162-210 of the reference;
+returns (out, out_x) like it."""
+import torch
+
+from kernels import _lib
+
+
+def _chunk_scan_fwd(cb, x, dt, dA_cumsum, C, states, D=None, z=None, seq_idx=None):
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, nchunks, chunk_size = dt.shape
+    _, _, ngroups, dstate = C.shape
+    assert nheads % ngroups == 0
+    assert C.shape == (batch, seqlen, ngroups, dstate)
+    assert cb.shape == (batch, nchunks, ngroups, chunk_size, chunk_size)
+    if z is not None:
+        assert z.shape == x.shape
+    if D is not None:
+        assert D.shape == (nheads, headdim) or D.shape == (nheads,)
+    assert dt.shape == (batch, nheads, nchunks, chunk_size)
+    assert dA_cumsum.shape == (batch, nheads, nchunks, chunk_size)
+    assert states.shape == (batch, nchunks, nheads, headdim, dstate)
+    if seq_idx is not None:
+        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
+    dev = _lib.require_gpu(x, cb, dt, dA_cumsum, C, states)
+    x, xs = _lib.strided4(x)
+    if C.dtype != x.dtype:
+        C = C.to(x.dtype)
+    C, cs = _lib.strided4(C)
+    zs = [None, 0, 0, 0]
+    if z is not None:
+        z, zs = _lib.strided4(z.to(x.dtype))
+    out = torch.empty(batch, seqlen, nheads, headdim, device=dev, dtype=x.dtype)
+    out_x = torch.empty_like(out) if z is not None else None
+    Df = None if D is None else _lib.f32c(D)
+    with torch.cuda.device(dev):
+        _lib.check(
+            _lib.lib().ssd_chunk_scan_fwd(
+                _lib.f32c(cb).data_ptr(), *xs, *zs, _lib.dtype_code(x), _lib.f32c(dt).data_ptr(),
+                _lib.f32c(dA_cumsum).data_ptr(), *cs, _lib.f32c(states).data_ptr(),
+                None if Df is None else Df.data_ptr(), int(D is not None and D.dim() == 2), out.data_ptr(),
+                out.stride(0), out.stride(1), out.stride(2), None if out_x is None else out_x.data_ptr(), batch,
+                seqlen, nheads, ngroups, headdim, dstate, chunk_size, _lib.stream_ptr(dev)),
+            "ssd_chunk_scan_fwd")
+    return out, out_x

@@ -1,0 +1,35 @@
+"""SSD stage 2: chunk states B^T x, weighted by the decay to the end of the chunk and dt.
+
+Mirrors _chunk_state_fwd, kernels/mamba_kernels/mamba_state_fwd.py:138-169 of the reference."""
+import torch
+
+from kernels import _lib
+
+
+def _chunk_state_fwd(B, x, dt, dA_cumsum, seq_idx=None, states=None, states_in_fp32=True):
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, nchunks, chunk_size = dt.shape
+    _, _, ngroups, dstate = B.shape
+    assert nheads % ngroups == 0
+    assert B.shape == (batch, seqlen, ngroups, dstate)
+    assert dt.shape == (batch, nheads, nchunks, chunk_size)
+    assert dA_cumsum.shape == dt.shape
+    if seq_idx is not None:
+        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
+    dev = _lib.require_gpu(x, B, dt, dA_cumsum)
+    if B.dtype != x.dtype:
+        B = B.to(x.dtype)  # the reference rounds the weighted B to x's type before the product
+    x, xs = _lib.strided4(x)
+    B, bs = _lib.strided4(B)
+    out = torch.empty(batch, nchunks, nheads, headdim, dstate, device=dev, dtype=torch.float32)
+    with torch.cuda.device(dev):
+        _lib.check(
+            _lib.lib().ssd_chunk_state_fwd(*bs, *xs, _lib.dtype_code(x), _lib.f32c(dt).data_ptr(),
+                                           _lib.f32c(dA_cumsum).data_ptr(), out.data_ptr(), batch, seqlen, nheads,
+                                           ngroups, headdim, dstate, chunk_size, _lib.stream_ptr(dev)),
+            "ssd_chunk_state_fwd")
+    if states is not None:
+        assert states.shape == (batch, nchunks, nheads, headdim, dstate)
+        states.copy_(out)
+        return states
+    return out if states_in_fp32 else out.to(B.dtype)

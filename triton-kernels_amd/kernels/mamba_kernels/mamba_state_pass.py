@@ -1,0 +1,31 @@
+"""SSD stage 3: the inter-chunk recurrence over the flattened (hdim * dstate) states.
+
+Mirrors _state_passing_fwd, kernels/mamba_kernels/mamba_state_pass.py:84-115 of the reference."""
+import torch
+
+from kernels import _lib
+
+
+def _state_passing_fwd(states, dA_chunk_cumsum, initial_states=None, seq_idx=None, chunk_size=None,
+                       out_dtype=None):
+    batch, nchunks, nheads, dim = states.shape
+    assert dA_chunk_cumsum.shape == (batch, nheads, nchunks)
+    if initial_states is not None:
+        assert initial_states.shape == (batch, nheads, dim)
+    if seq_idx is not None:
+        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
+    dev = _lib.require_gpu(states, dA_chunk_cumsum)
+    out_dtype = states.dtype if out_dtype is None else out_dtype
+    st = _lib.f32c(states)
+    da = dA_chunk_cumsum if dA_chunk_cumsum.dtype == torch.float32 else dA_chunk_cumsum.float()
+    init = None if initial_states is None else _lib.f32c(initial_states)
+    out = torch.empty(batch, nchunks, nheads, dim, device=dev, dtype=torch.float32)
+    final_states = torch.empty(batch, nheads, dim, device=dev, dtype=torch.float32)
+    with torch.cuda.device(dev):
+        _lib.check(
+            _lib.lib().ssd_state_passing_fwd(st.data_ptr(), da.data_ptr(), da.stride(0), da.stride(1), da.stride(2),
+                                             None if init is None else init.data_ptr(), out.data_ptr(),
+                                             final_states.data_ptr(), batch, nchunks, nheads, dim,
+                                             _lib.stream_ptr(dev)),
+            "ssd_state_passing_fwd")
+    return (out if out_dtype == torch.float32 else out.to(out_dtype)), final_states
