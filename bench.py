@@ -46,6 +46,9 @@ def parse():
     ap.add_argument("--sets", type=int, default=3, help="input sets the steps rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel timing pass")
+    ap.add_argument("--workload", default="ema", choices=["ema", "ssd"],
+                    help="ema: the headline EMA scan step (default); ssd: the Mamba-2 SSD forward stages at "
+                    "BASELINE configuration 5 (b8 nh32 hdim64 dstate128 g1 L8192 chunk256, bf16)")
     ap.add_argument("--stage", default=None,
                     help="time only this stage (a name from the `kernels` table, or fwd, bwd, copy) "
                     "and print a short JSON line; used for counter collection")
@@ -120,8 +123,108 @@ def cpu_baseline(args, torch):
     }
 
 
+def ssd_main(args):
+    """Mamba-2 SSD forward at BASELINE configuration 5: the five stage launchers and their sum,
+    timed with events on the launch stream; per stage the algorithmic bytes (inputs read once,
+    outputs written once) against the HBM peak and, for the three MFMA stages, dense FLOPs
+    against the bf16 MFMA peak."""
+    import torch
+
+    from kernels.mamba_kernels.mamba_bmm import _bmm_chunk_fwd
+    from kernels.mamba_kernels.mamba_combined_fwd import _mamba_chunk_scan_combined_fwd
+    from kernels.mamba_kernels.mamba_cumsum import _chunk_cumsum_fwd
+    from kernels.mamba_kernels.mamba_scan_fwd import _chunk_scan_fwd
+    from kernels.mamba_kernels.mamba_state_fwd import _chunk_state_fwd
+    from kernels.mamba_kernels.mamba_state_pass import _state_passing_fwd
+    from oracle import ssd_oracle as S
+
+    dev = torch.device("cuda:0")
+    b, L, nh, P, g, N, Q = 8, 8192, 32, 64, 1, 128, 256
+    C = L // Q
+    sets = []
+    for s in range(2):
+        x, dt, A, B, Cm, _, _ = S.make_inputs(b, L, nh, P, g, N, seed=5 + s, dtype=torch.bfloat16)
+        sets.append(tuple(t.to(dev) for t in (x, dt, A, B, Cm)))
+    inter = []
+    for x, dt, A, B, Cm in sets:
+        out, _, dt_out, dA_cs, states, _ = _mamba_chunk_scan_combined_fwd(x, dt, A, B, Cm, Q)
+        st = _chunk_state_fwd(B, x, dt_out, dA_cs)
+        cb = _bmm_chunk_fwd(Cm, B, Q, output_dtype=torch.float32)
+        inter.append((dt_out, dA_cs, st, states, cb))
+    del out
+
+    def pick(i):
+        k = i % len(sets)
+        return sets[k] + inter[k]
+
+    stages = {
+        "chunk_cumsum": lambda i: _chunk_cumsum_fwd(pick(i)[1], pick(i)[2], Q),
+        "chunk_state": lambda i: _chunk_state_fwd(pick(i)[3], pick(i)[0], pick(i)[5], pick(i)[6]),
+        "state_passing": lambda i: _state_passing_fwd(pick(i)[7].view(b, C, nh, P * N), pick(i)[6][..., -1]),
+        "bmm_chunk": lambda i: _bmm_chunk_fwd(pick(i)[4], pick(i)[3], Q, output_dtype=torch.float32),
+        "chunk_scan": lambda i: _chunk_scan_fwd(pick(i)[9], pick(i)[0], pick(i)[5], pick(i)[6], pick(i)[4], pick(i)[8]),
+        "forward": lambda i: _mamba_chunk_scan_combined_fwd(*pick(i)[:5], Q),
+    }
+    xb = b * L * nh * P * 2
+    bc = b * L * g * N * 2
+    dtb = b * L * nh * 4
+    stb = b * C * nh * P * N * 4
+    cbb = b * C * g * Q * Q * 4
+    nbytes = {
+        "chunk_cumsum": 3 * dtb, "chunk_state": xb + bc + 2 * dtb + stb, "state_passing": 2 * stb + dtb // Q,
+        "bmm_chunk": 2 * bc + cbb, "chunk_scan": cbb + 2 * xb + bc + stb + 2 * dtb,
+        "forward": 2 * xb + 2 * bc + dtb,
+    }
+    units = b * C * nh
+    flops = {"chunk_state": 2 * Q * P * N * units, "bmm_chunk": 2 * Q * Q * N * b * C * g,
+             "chunk_scan": (2 * Q * Q * P + 2 * Q * N * P) * units}
+    res = {}
+    for name, fn in stages.items():
+        if args.stage and name != args.stage:
+            continue
+        for i in range(args.warmup):
+            fn(i)
+        ms = time_region(fn, args.steps, torch)
+        res[name] = {"ms": ms, "bytes": nbytes[name], "GBps": nbytes[name] / ms / 1e6,
+                     "hbm_frac": nbytes[name] / ms / 1e6 / HBM_PEAK_GBS}
+        if name in flops:
+            res[name]["dense_TFLOPs"] = flops[name] / ms / 1e9
+            res[name]["mfma_frac"] = flops[name] / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS
+    if args.stage:
+        print(json.dumps({"stage": args.stage, **res[args.stage], "steps": args.steps}))
+        return
+    dom = max((k for k in res if k != "forward"), key=lambda k: res[k]["ms"])
+    out = {
+        "metric": "Mamba-2 SSD fwd ms @ b8 nh32 hdim64 dstate128 g1 L8192 c256",
+        "value": res["forward"]["ms"], "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": res["forward"]["ms"], "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "Mamba-2 SSD chunked scan forward, five stages, b8 nh32 hdim64 dstate128 g1 L8192 "
+                   "chunk256, bf16 x/B/C, fp32 dt/A, D = 0, no gate"},
+        "stages": res,
+        "roofline": {"kernel": dom, "bound": "hbm", "achieved": res[dom]["GBps"], "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": res[dom]["hbm_frac"], "traffic": None},
+    }
+    if not args.no_cpu_baseline:
+        x, dt, A, B, Cm, _, _ = S.make_inputs(1, 512, nh, P, g, N, seed=5, dtype=torch.bfloat16)
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < 10.0 and reps < 20:
+            S.ssd_loop(x.float(), dt, A, B.float(), Cm.float())
+            reps += 1
+        per = (time.perf_counter() - t0) / reps
+        scale = b * L / 512
+        out["cpu_baseline"] = {"value": per * scale * 1e3, "unit": "ms", "cores": torch.get_num_threads(),
+                               "kind": "port",
+                               "sample": f"1 of {b} sequences, 512 of {L} positions, sequential recurrence in fp32 "
+                               f"torch, {reps} repetitions, scaled x{scale:g}"}
+    print(json.dumps(out))
+
+
 def main():
     args = parse()
+    if args.workload == "ssd" and args.gpus == 1:
+        return ssd_main(args)
     if args.gpus != 1:
         print("bench.py measures one GPU only: the EMA scan has no multi-GPU path in this build "
               "(run with --gpus 1)", file=sys.stderr)

@@ -1,5 +1,5 @@
 """CPU-side checks of the C ABI: the built library loads, exports every symbol that
-include/ema_hip.h declares, and validates its arguments before launching anything (so the
+include/ema_hip.h and include/ssd_hip.h declare, and validates its arguments before launching anything (so the
 refusals can be exercised without a GPU)."""
 import os
 import re
@@ -9,13 +9,16 @@ import pytest
 from kernels import _lib
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "ema_hip.h")
+HEADERS = [os.path.join(ROOT, "include", "ema_hip.h"), os.path.join(ROOT, "include", "ssd_hip.h")]
 
 
 def declared_functions():
-    src = open(HEADER).read()
-    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
-    return sorted(set(re.findall(r"\b(ema_[a-z_A-Z0-9]+)\s*\(", src)))
+    names = set()
+    for header in HEADERS:
+        src = open(header).read()
+        src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+        names |= set(re.findall(r"\b((?:ema|ssd)_[a-z_A-Z0-9]+)\s*\(", src))
+    return sorted(names)
 
 
 def test_header_and_binding_agree():
@@ -71,6 +74,22 @@ def test_validation_happens_before_any_launch():
                        None, fake, 16, 1, 1, 8, 8, 4, None, None, None)
         == -2
     )
+
+
+def test_ssd_validation_happens_before_any_launch():
+    handle = _lib.lib()
+    fake = 0x1000
+    seq = [fake, 64 * 2 * 64, 2 * 64, 64]
+    grp = [fake, 64 * 64, 64, 64]
+    # null pointer, bad shape, unsupported head size, misaligned strides, unknown dtype
+    assert handle.ssd_chunk_cumsum_fwd(None, 0, 2, 2, 1, fake, None, fake, fake, 1, 64, 2, 64, 0, 0.0, 1.0, None) == -1
+    assert handle.ssd_chunk_cumsum_fwd(fake, 0, 2, 2, 1, fake, None, fake, fake, 1, 0, 2, 64, 0, 0.0, 1.0, None) == -2
+    assert handle.ssd_chunk_state_fwd(*grp, *seq, 0, fake, fake, fake, 1, 64, 2, 1, 48, 64, 64, None) == -5
+    assert handle.ssd_chunk_state_fwd(*grp, fake, 8190, 130, 65, 1, fake, fake, fake, 1, 64, 2, 1, 64, 64, 64, None) == -3
+    assert handle.ssd_chunk_state_fwd(*grp, *seq, 9, fake, fake, fake, 1, 64, 2, 1, 64, 64, 64, None) == -4
+    assert handle.ssd_chunk_state_fwd(*grp, *seq, 0, fake, fake, fake, 1, 64, 3, 2, 64, 64, 64, None) == -2
+    assert handle.ssd_bmm_chunk_fwd(*grp, *grp, 0, fake, 1, 1, 64, 1, 64, 64, None) == -4  # bf16 out of f32 in
+    assert handle.ssd_state_passing_fwd(fake, fake, 2, 1, 1, None, fake, fake, 1, 1, 2, 6, None) == -3
 
 
 def test_error_mapping():

@@ -24,6 +24,8 @@ CASES = [
     (2, 200, 4, 64, 1, 128, 256),   # one ragged chunk
     (1, 520, 2, 128, 1, 64, 128),
     (1, 130, 2, 128, 2, 128, 64),
+    (1, 900, 2, 64, 1, 64, 512),    # two 256-row super-tiles per chunk, the last chunk ragged
+    (1, 512, 2, 128, 2, 128, 256),
 ]
 
 

@@ -47,6 +47,7 @@ int check_dims(int64_t batch, int64_t L, int64_t nh, int64_t g, int64_t P, int64
   return SSD_OK;
 }
 inline bool dim_ok(int64_t v) { return v == 64 || v == 128; }
+constexpr int kLdsBytes = 160 * 1024;  // LDS of one CU
 
 template <typename K>
 int allow_smem(K kernel, int bytes) {
@@ -102,6 +103,18 @@ struct ScanLaunch {
   hipStream_t st;
   template <typename T, int P, int N>
   int run() const {
+    constexpr int wide_smem = WideSmem<T, P, N>::kBytes;
+    if (d.Q % 256 == 0 && wide_smem <= kLdsBytes) {  // 256-row super-tiles, no barrier inside the k loop
+      auto kernel = ssd_chunk_scan_wide_kernel<T, P, N>;
+      constexpr int smem = wide_smem;
+      SSD_TRY(allow_smem(kernel, smem));
+      const int stiles = (int)(d.Q / 256);
+      hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh * stiles)), dim3(256), smem, st, cb,
+                         (const T*)x, sx, (const T*)z, sz, dt, dA, (const T*)C, sC, prev, D, d_has_hdim, (T*)out,
+                         so, (T*)out_x, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C,
+                         stiles);
+      return launched();
+    }
     auto kernel = ssd_chunk_scan_kernel<T, P, N>;
     constexpr int smem = ScanSmem<T, P, N>::kBytes;
     SSD_TRY(allow_smem(kernel, smem));

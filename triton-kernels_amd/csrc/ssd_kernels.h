@@ -481,4 +481,189 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------
+// chunk_scan for chunk sizes that are multiples of 256.  One workgroup per (b, c, h, 256-row
+// super-tile); wave w owns the 32-row blocks w and 7 - w of it, which balances the causal sum,
+// and all hdim / 32 column blocks.  The operands that differ from lane to lane are built in
+// registers straight from global memory (C rows; cb rows, weighted and masked on the way), so
+// the k loop has no barrier: LDS only holds what every wave shares, the 256-row tile of x, the
+// carried state and the chunk's dA / dt.  Results leave through a per-wave LDS staging area.
+// ------------------------------------------------------------------------------------
+template <typename T, int P, int N>
+struct WideSmem {
+  static constexpr int ST = 256;
+  static constexpr int PX = Tile<T>::pitch(P), PC = Tile<T>::pitch(N), PO = P + 4;
+  static constexpr int kX = ST * PX * (int)sizeof(T);
+  static constexpr int kPrev = P * PC * (int)sizeof(T);
+  static constexpr int kOut = 4 * 32 * PO * (int)sizeof(float);                  // one 32-row block per wave
+  static constexpr int kMain = (kX + kPrev) > kOut ? (kX + kPrev) : kOut;
+  static constexpr int kBytes = kMain + 3 * ST * (int)sizeof(float);            // + dA_k, dt_k, exp(dA_m)
+};
+
+template <typename T, int P, int N>
+__global__ __launch_bounds__(256) void ssd_chunk_scan_wide_kernel(
+    const float* __restrict__ cb, const T* __restrict__ x, Strides3 sx, const T* __restrict__ z, Strides3 sz,
+    const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Cm, Strides3 sC,
+    const float* __restrict__ prev, const float* __restrict__ D, int d_has_hdim, T* __restrict__ out,
+    Strides3 so, T* __restrict__ out_x, int nh, int heads_per_group, int ngroups, int L, int Q, int C,
+    int stiles) {
+  using S = WideSmem<T, P, N>;
+  constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, PB = P / 32, ST = S::ST;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T* Xs = reinterpret_cast<T*>(smem);
+  T* Pv = reinterpret_cast<T*>(smem + S::kX);
+  float* Os = reinterpret_cast<float*>(smem);
+  float* dAk = reinterpret_cast<float*>(smem + S::kMain);
+  float* dtk = dAk + ST;
+  float* sm = dtk + ST;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
+  const int st = blockIdx.x % stiles;
+  const int h = (blockIdx.x / stiles) % nh;
+  const int c = (blockIdx.x / (stiles * nh)) % C;
+  const int64_t b = blockIdx.x / ((int64_t)stiles * nh * C);
+  const int limit = min(Q, L - c * Q);
+  const int m0 = ST * st;
+  if (m0 >= limit) return;
+  const int g = h / heads_per_group;
+  const int64_t chunk = (b * nh + h) * C + c;
+  const float* dAp = dA_cs + chunk * Q;
+  const float* dtp = dt + chunk * Q;
+  const T* xg = x + b * sx.sb + (int64_t)c * Q * sx.sl + h * sx.sh;
+  const T* Cg = Cm + b * sC.sb + (int64_t)c * Q * sC.sl + g * sC.sh;
+  const float* pg = prev + (((b * C + c) * nh + h) * (int64_t)P) * N;
+  const float* cbg = cb + (((b * C + c) * ngroups + g) * (int64_t)Q) * Q;
+
+  int mrow[2];
+  mrow[0] = 32 * wave;
+  mrow[1] = 32 * (7 - wave);
+  floatx16 acc[2][PB];
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+    for (int pb = 0; pb < PB; ++pb) zero_acc(acc[mb][pb]);
+
+  // ---- phase A: C . prev, scaled by exp(dA_m)
+  {
+    constexpr int VPR = N / 4;
+#pragma unroll
+    for (int i = 0; i < P * VPR / 256; ++i) {
+      const int idx = tid + 256 * i;
+      const int r = idx / VPR, cv = (idx % VPR) * 4;
+      const float4 v = *reinterpret_cast<const float4*>(pg + (int64_t)r * N + cv);
+      T* d = Pv + r * S::PC + cv;
+      d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
+    }
+  }
+  sm[tid] = __expf(dAp[m0 + tid]);
+  __syncthreads();
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb) {
+    const int m = m0 + mrow[mb] + l32;
+    const T* crow = Cg + (int64_t)m * sC.sl + EPL * half;
+#pragma unroll
+    for (int kk = 0; kk < N; kk += KG) {
+      Vec16<T> a;
+      if (m < limit) a = load16(crow + kk);
+      else a.zero();
+#pragma unroll
+      for (int pb = 0; pb < PB; ++pb) mma_group(a, frag_rows(Pv, S::PC, 32 * pb, kk, lane), acc[mb][pb]);
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const float sc = sm[mrow[mb] + acc_row(v, lane)];
+#pragma unroll
+      for (int pb = 0; pb < PB; ++pb) acc[mb][pb][v] *= sc;
+    }
+  }
+
+  // ---- phase B: the k super-tiles up to the diagonal one
+  for (int kt = 0; kt <= st; ++kt) {
+    const int k0 = ST * kt;
+    stage_rows<T, ST, P>(Xs, xg, sx.sl, k0, limit, tid, NoScale());
+    dAk[tid] = dAp[k0 + tid];
+    dtk[tid] = dtp[k0 + tid];
+    __syncthreads();
+    const bool diag = kt == st;
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) {
+      const int mloc = mrow[mb] + l32;  // row inside the super-tile
+      const float am = dAp[m0 + mloc];
+      const float* cbrow = cbg + (int64_t)(m0 + mloc) * Q + k0 + EPL * half;
+      const int kend = diag ? mrow[mb] + 32 : ST;
+      for (int kk = 0; kk < kend; kk += KG) {
+        float w[EPL];
+#pragma unroll
+        for (int e = 0; e < EPL; e += 4) {
+          const float4 c4 = *reinterpret_cast<const float4*>(cbrow + kk + e);
+          w[e] = c4.x, w[e + 1] = c4.y, w[e + 2] = c4.z, w[e + 3] = c4.w;
+        }
+        const int kb = kk + EPL * half;
+        Vec16<T> a;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+          const float f = w[e] * __expf(fminf(am - dAk[kb + e], 0.f)) * dtk[kb + e];
+          a.set(e, (diag && kb + e > mloc) ? 0.f : f);
+        }
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) mma_group(a, frag_cols(Xs, S::PX, kk, 32 * pb, lane), acc[mb][pb]);
+      }
+      if (diag && D) {
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) {
+          const int col = 32 * pb + l32;
+          const float dv = d_has_hdim ? D[h * P + col] : D[h];
+#pragma unroll
+          for (int v = 0; v < 16; ++v)
+            acc[mb][pb][v] = fmaf(dv, (float)Xs[(mrow[mb] + acc_row(v, lane)) * S::PX + col], acc[mb][pb][v]);
+        }
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- phase C: each wave moves its two blocks through its own staging area
+  float* mine = Os + wave * 32 * S::PO;
+  constexpr int VPR = P / EPL;
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb) {
+#pragma unroll
+    for (int pb = 0; pb < PB; ++pb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) mine[acc_row(v, lane) * S::PO + 32 * pb + l32] = acc[mb][pb][v];
+    // the wave's own writes are visible to its own reads once the LDS counter has drained
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+#pragma unroll
+    for (int i = 0; i < 32 * VPR / 64; ++i) {
+      const int idx = lane + 64 * i;
+      const int r = idx / VPR, cv = (idx % VPR) * EPL;
+      const int m = m0 + mrow[mb] + r;
+      if (m < limit) {
+        const int64_t pos = (int64_t)c * Q + m;
+        float v[EPL];
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) v[e] = mine[r * S::PO + cv + e];
+        Vec16<T> o;
+        if (z) {
+          if (out_x) {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) o.set(e, v[e]);
+            store16(out_x + b * so.sb + pos * so.sl + h * so.sh + cv, o);
+          }
+          const Vec16<T> zv = load16(z + b * sz.sb + pos * sz.sl + h * sz.sh + cv);
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) {
+            const float zf = zv.get(e);
+            v[e] *= zf / (1.f + __expf(-zf));
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) o.set(e, v[e]);
+        store16(out + b * so.sb + pos * so.sl + h * so.sh + cv, o);
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+  }
+}
+
 }  // namespace ssd
