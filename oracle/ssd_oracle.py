@@ -219,3 +219,134 @@ def brute_force(x, dt, A, B, C):
                     for f in range(p):
                         out[bi, t, h, f] += wgt * float(x[bi, s, h, f])
     return out
+
+
+# ------------------------------------------------------------------ backward stages
+# Restatements of the six launchers in kernels/mamba_kernels_bwd/ (the reference ships no
+# combined backward and no gradient of CB, dt's cumsum or the gate).  Each is pinned in
+# tests/test_ssd_oracle.py by torch.autograd (float64) through the forward stage it differentiates.
+
+
+def bwd_dstates(C, dA_cumsum, dout, round_to=None):
+    """dprev[b,c,h,p,n] = sum_m round(dout[m,p] * exp(dA_m)) * C[m,n]: the gradient of chunk_scan
+    with respect to the carried states; mamba_scan_bwd.py:62-76."""
+    b, L, nh, p = dout.shape
+    _, _, nc, Q = dA_cumsum.shape
+    g, n = C.shape[2], C.shape[3]
+    dc = _pad_seq(_up(dout), Q).reshape(b, nc, Q, nh, p)
+    Cc = _pad_seq(_up(C), Q).reshape(b, nc, Q, g, n).repeat_interleave(nh // g, dim=3)
+    valid = _pad_seq(torch.ones(b, L, 1, dtype=dc.dtype), Q).reshape(b, nc, Q, 1)
+    w = torch.exp(dA_cumsum).permute(0, 2, 3, 1) * valid  # (b, nc, Q, nh)
+    return torch.einsum("bcqhp,bcqhn->bchpn", _round(dc * w[..., None], round_to), Cc)
+
+
+def state_passing_bwd(states, dA_chunk_cumsum, dout, dfinal_states=None, has_initial_states=False):
+    """states (b, C, nh, dim) = the states entering each chunk (index 0 the initial one), dout the
+    gradient with respect to them.  Returns (dstates, ddA_chunk_cumsum, dinitstates):
+    dstates[c] = gradient of the chunk-local state of chunk c, ddA[c] = <states[c], dstates[c]> *
+    exp(dA[c]) (0 for c = 0 without initial states); mamba_state_passing_bwd_dstates.py:66-112."""
+    b, nc, nh, dim = states.shape
+    dstates = torch.empty_like(dout)
+    ddA = dA_chunk_cumsum.new_zeros(b, nh, nc)
+    G = dout.new_zeros(b, nh, dim) if dfinal_states is None else _up(dfinal_states).clone()
+    for c in range(nc - 1, -1, -1):
+        dstates[:, c] = G
+        scale = torch.exp(dA_chunk_cumsum[:, :, c])
+        if c > 0 or has_initial_states:
+            ddA[:, :, c] = (states[:, c] * G).sum(-1) * scale
+        G = scale[..., None] * G + dout[:, c]
+    return dstates, ddA, (G if has_initial_states else None)
+
+
+def chunk_state_bwd_db(x, dt, dA_cumsum, dstates, B=None, ngroups=1, round_to=None):
+    """dB[b,l,g,n] = sum over the heads of group g of (sum_p x[m,p] * round(dstates[p,n])) *
+    exp(min(dA_last - dA_m, 0)) * dt_m.  With B also ddA_cumsum (b, nh, C, Q): the inclusive cumsum
+    along the chunk of r shifted by one slot, r[m] = sum_n db_h[m,n] * B[m,n]: the gradient of the
+    chunk states with respect to the per-position dA; mamba_chunk_state_bwd_db.py:91-125,172-180."""
+    b, L, nh, p = x.shape
+    _, _, nc, Q = dt.shape
+    n = dstates.shape[-1]
+    xc = _pad_seq(_up(x), Q).reshape(b, nc, Q, nh, p)
+    w = (torch.exp(torch.clamp(dA_cumsum[..., -1:] - dA_cumsum, max=0.0)) * dt).permute(0, 2, 3, 1)
+    dbh = torch.einsum("bcqhp,bchpn->bcqhn", xc, _round(_up(dstates), round_to)) * w[..., None]
+    dB = dbh.reshape(b, nc, Q, ngroups, nh // ngroups, n).sum(4).reshape(b, nc * Q, ngroups, n)[:, :L]
+    if B is None:
+        return dB
+    Bc = _pad_seq(_up(B), Q).reshape(b, nc, Q, ngroups, n).repeat_interleave(nh // ngroups, dim=3)
+    r = (dbh * Bc).sum(-1).permute(0, 3, 1, 2)  # (b, nh, nc, Q)
+    raw = torch.zeros_like(r)
+    raw[..., 1:] = r[..., :-1]
+    return dB, torch.cumsum(raw, -1)
+
+
+def chunk_scan_bwd_dC(prev_states, dA_cumsum, dout, C=None, ngroups=1, round_to=None):
+    """dC[b,l,g,n] = sum over the heads of group g of (sum_p dout[m,p] * round(prev[p,n])) * exp(dA_m):
+    the part of dC that comes through the carried state.  With C also ddA_cumsum_prev[m] =
+    sum_n dc_h[m,n] * C[m,n], the gradient with respect to dA_cumsum[m] of that term;
+    mamba_chunk_scan_bwd_dc.py:84-101."""
+    b, L, nh, p = dout.shape
+    _, _, nc, Q = dA_cumsum.shape
+    n = prev_states.shape[-1]
+    dc_ = _pad_seq(_up(dout), Q).reshape(b, nc, Q, nh, p)
+    w = torch.exp(dA_cumsum).permute(0, 2, 3, 1)
+    dch = torch.einsum("bcqhp,bchpn->bcqhn", dc_, _round(_up(prev_states), round_to)) * w[..., None]
+    dC = dch.reshape(b, nc, Q, ngroups, nh // ngroups, n).sum(4).reshape(b, nc * Q, ngroups, n)[:, :L]
+    if C is None:
+        return dC
+    Cc = _pad_seq(_up(C), Q).reshape(b, nc, Q, ngroups, n).repeat_interleave(nh // ngroups, dim=3)
+    return dC, (dch * Cc).sum(-1).permute(0, 3, 1, 2)
+
+
+def chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum, B, CB, dout, dstates, D=None, round_to=None):
+    """acc[m,p] = exp(min(dA_last - dA_m, 0)) * sum_n B[m,n] * round(dstates[p,n])
+                + sum_{k>=m} round(CB[k,m] * exp(min(dA_k - dA_m, 0))) * dout[k,p]
+    dx = acc * dt_m + D * dout,  ddt[m] = sum_p acc[m,p] * x[m,p],  dD = sum dout * x;
+    mamba_chunk_scan_chunk_state_bwd_dx.py:86-187.  Returns (dx, ddt (b,nh,C,Q), dD)."""
+    b, L, nh, p = x.shape
+    _, _, nc, Q = dt.shape
+    g, n = B.shape[2], B.shape[3]
+    rep = nh // g
+    xc = _pad_seq(_up(x), Q).reshape(b, nc, Q, nh, p)
+    dc_ = _pad_seq(_up(dout), Q).reshape(b, nc, Q, nh, p)
+    Bc = _pad_seq(_up(B), Q).reshape(b, nc, Q, g, n).repeat_interleave(rep, dim=3)
+    dA = dA_cumsum.permute(0, 2, 1, 3)  # (b, nc, nh, Q)
+    scale = torch.exp(torch.clamp(dA[..., -1:] - dA, max=0.0))  # (b, nc, nh, Q)
+    acc = torch.einsum("bcmhn,bchpn,bchm->bcmhp", Bc, _round(_up(dstates), round_to), scale)
+    cbh = _up(CB).repeat_interleave(rep, dim=2)  # (b, nc, nh, k, m)
+    decay = torch.exp(torch.clamp(dA[..., :, None] - dA[..., None, :], max=0.0))  # [k, m]
+    valid = _pad_seq(torch.ones(b, L, 1, dtype=xc.dtype), Q).reshape(b, nc, 1, Q, 1)  # k < limit
+    mask = torch.tril(torch.ones(Q, Q, dtype=torch.bool))  # k >= m
+    w = cbh * decay * valid
+    w = _round(torch.where(mask, w, w.new_zeros(())), round_to)
+    acc = acc + torch.einsum("bchkm,bckhp->bcmhp", w, dc_)
+    dtc = dt.permute(0, 2, 3, 1)  # (b, nc, Q, nh)
+    dx = acc * dtc[..., None]
+    ddt = (acc * xc).sum(-1).permute(0, 3, 1, 2)
+    dD = None
+    if D is not None:
+        Dv = _up(D)[None, None, None, :, None] if D.dim() == 1 else _up(D)[None, None, None]
+        dx = dx + dc_ * Dv
+        dD = (dc_ * xc).sum((0, 1, 2)) if D.dim() == 2 else (dc_ * xc).sum((0, 1, 2, 4))
+    return dx.reshape(b, nc * Q, nh, p)[:, :L], ddt, dD
+
+
+def chunk_scan_bwd_ddAcs_stable(x, dt, dA_cumsum, dout, cb):
+    """With G[m,n] = <dout[m], x[n]> * dt_n * cb[m,n] * exp(min(dA_m - dA_n, 0)) for n < m:
+    ddA_cumsum[j] = sum_{m>=j} sum_{n<j} G[m,n] (0 for j = 0): the gradient of the causal term of
+    chunk_scan with respect to the per-position dA; mamba_chunk_scan_bwd_da.py:62-103."""
+    b, L, nh, p = x.shape
+    _, _, nc, Q = dt.shape
+    rep = nh // cb.shape[2]
+    xc = _pad_seq(_up(x), Q).reshape(b, nc, Q, nh, p)
+    dc_ = _pad_seq(_up(dout), Q).reshape(b, nc, Q, nh, p)
+    dA = dA_cumsum.permute(0, 2, 1, 3)
+    dtc = dt.permute(0, 2, 1, 3)
+    G = torch.einsum("bcmhp,bcnhp->bchmn", dc_, xc) * dtc[..., None, :] * _up(cb).repeat_interleave(rep, dim=2)
+    G = G * torch.exp(torch.clamp(dA[..., :, None] - dA[..., None, :], max=0.0))
+    strict = torch.tril(torch.ones(Q, Q, dtype=torch.bool), diagonal=-1)
+    G = torch.where(strict, G, G.new_zeros(()))
+    cum = torch.cumsum(G, -1)                         # over n
+    cum = torch.where(strict, cum, cum.new_zeros(()))
+    out = torch.zeros_like(dA)
+    out[..., 1:] = cum.sum(-2)[..., :-1]              # over m, shifted by one slot
+    return out.permute(0, 2, 1, 3)

@@ -117,3 +117,105 @@ def test_bmm_chunk_matches_einsum_per_chunk():
     assert cb.shape == (2, 3, 2, 8, 8)
     assert torch.allclose(cb[1, 1, 0], Cm[1, 8:16, 0] @ Bm[1, 8:16, 0].T, rtol=1e-5, atol=1e-5)
     assert torch.equal(cb[0, 2, 1, 5:], torch.zeros(3, 8))  # rows past L
+
+
+# ---------------------------------------------------------------- backward stages vs autograd
+
+
+def _bwd_case(b=2, L=21, nh=4, p=3, g=2, n=5, Q=8, seed=11):
+    x, dt_raw, A, B, C, D, _ = _f64(*S.make_inputs(b, L, nh, p, g, n, seed=seed))
+    dA_cs, dt = S.chunk_cumsum(dt_raw, A, Q)
+    gen = torch.Generator().manual_seed(seed + 1)
+    dout = torch.randn(b, L, nh, p, generator=gen, dtype=D64)
+    nc = dt.shape[2]
+    prev = torch.randn(b, nc, nh, p, n, generator=gen, dtype=D64)
+    dstates = torch.randn(b, nc, nh, p, n, generator=gen, dtype=D64)
+    return x, dt, dA_cs, B, C, D, dout, prev, dstates, Q
+
+
+def _cumsum_of(dA):
+    return torch.cumsum(dA, -1)
+
+
+def _per_position(dA_cs):
+    d = dA_cs.clone()
+    d[..., 1:] = dA_cs[..., 1:] - dA_cs[..., :-1]
+    return d
+
+
+def test_bwd_dstates_is_grad_of_chunk_scan_wrt_prev():
+    x, dt, dA_cs, B, C, D, dout, prev, _, Q = _bwd_case()
+    pr = prev.clone().requires_grad_()
+    out, _ = S.chunk_scan(S.bmm_chunk(C, B, Q), x, dt, dA_cs, C, pr, D)
+    (out * dout).sum().backward()
+    assert torch.allclose(S.bwd_dstates(C, dA_cs, dout), pr.grad, rtol=1e-10, atol=1e-10)
+
+
+def test_state_passing_bwd_is_autograd_of_state_passing():
+    gen = torch.Generator().manual_seed(3)
+    b, nc, nh, dim = 2, 5, 3, 7
+    st = torch.randn(b, nc, nh, dim, generator=gen, dtype=D64).requires_grad_()
+    dA = (-torch.rand(b, nh, nc, generator=gen, dtype=D64)).requires_grad_()
+    init = torch.randn(b, nh, dim, generator=gen, dtype=D64).requires_grad_()
+    dprev = torch.randn(b, nc, nh, dim, generator=gen, dtype=D64)
+    dfin = torch.randn(b, nh, dim, generator=gen, dtype=D64)
+    for use_init in (True, False):
+        for t in (st, dA, init):
+            t.grad = None
+        prev, fin = S.state_passing(st, dA, init if use_init else None)
+        ((prev * dprev).sum() + (fin * dfin).sum()).backward()
+        dst, ddA, dinit = S.state_passing_bwd(prev.detach(), dA.detach(), dprev, dfin, has_initial_states=use_init)
+        assert torch.allclose(dst, st.grad, rtol=1e-10, atol=1e-10)
+        assert torch.allclose(ddA, dA.grad, rtol=1e-10, atol=1e-10)
+        if use_init:
+            assert torch.allclose(dinit, init.grad, rtol=1e-10, atol=1e-10)
+        else:
+            assert dinit is None and torch.equal(ddA[:, :, 0], torch.zeros(b, nh, dtype=D64))
+
+
+def test_chunk_state_bwd_db_is_grad_of_chunk_state():
+    x, dt, dA_cs, B, C, D, dout, prev, dstates, Q = _bwd_case()
+    Br = B.clone().requires_grad_()
+    dA = _per_position(dA_cs).requires_grad_()
+    st = S.chunk_state(Br, x, dt, _cumsum_of(dA))
+    (st * dstates).sum().backward()
+    dB, ddA = S.chunk_state_bwd_db(x, dt, dA_cs, dstates, B=B, ngroups=B.shape[2])
+    assert torch.allclose(dB, Br.grad, rtol=1e-10, atol=1e-10)
+    assert torch.allclose(ddA, dA.grad, rtol=1e-10, atol=1e-10)
+    assert torch.allclose(S.chunk_state_bwd_db(x, dt, dA_cs, dstates, ngroups=B.shape[2]), dB)
+
+
+def test_chunk_scan_bwd_dC_is_grad_of_the_carried_state_term():
+    x, dt, dA_cs, B, C, D, dout, prev, _, Q = _bwd_case()
+    Cr = C.clone().requires_grad_()
+    dAr = dA_cs.clone().requires_grad_()
+    zero_cb = torch.zeros(x.shape[0], dt.shape[2], C.shape[2], Q, Q, dtype=D64)  # leaves only C . prev
+    out, _ = S.chunk_scan(zero_cb, x, dt, dAr, Cr, prev)
+    (out * dout).sum().backward()
+    dC, ddA_prev = S.chunk_scan_bwd_dC(prev, dA_cs, dout, C=C, ngroups=C.shape[2])
+    assert torch.allclose(dC, Cr.grad, rtol=1e-10, atol=1e-10)
+    assert torch.allclose(ddA_prev, dAr.grad, rtol=1e-10, atol=1e-10)
+
+
+def test_bwd_dx_is_grad_wrt_x_and_explicit_dt():
+    x, dt, dA_cs, B, C, D, dout, prev, dstates, Q = _bwd_case()
+    cb = S.bmm_chunk(C, B, Q)
+    xr, dtr, Dr = x.clone().requires_grad_(), dt.clone().requires_grad_(), D.clone().requires_grad_()
+    zero_prev = torch.zeros_like(prev)
+    out, _ = S.chunk_scan(cb, xr, dtr, dA_cs, C, zero_prev, Dr)   # dA_cs held fixed: only the explicit dt
+    st = S.chunk_state(B, xr, dtr, dA_cs)
+    ((out * dout).sum() + (st * dstates).sum()).backward()
+    dx, ddt, dD = S.chunk_scan_chunk_state_bwd_dx(x, dt, dA_cs, B, cb, dout, dstates, D=D)
+    assert torch.allclose(dx, xr.grad, rtol=1e-10, atol=1e-10)
+    assert torch.allclose(ddt, dtr.grad, rtol=1e-10, atol=1e-10)
+    assert torch.allclose(dD, Dr.grad, rtol=1e-10, atol=1e-10)
+
+
+def test_ddAcs_stable_is_grad_of_the_causal_term_wrt_dA():
+    x, dt, dA_cs, B, C, D, dout, prev, _, Q = _bwd_case()
+    cb = S.bmm_chunk(C, B, Q)
+    dA = _per_position(dA_cs).requires_grad_()
+    out, _ = S.chunk_scan(cb, x, dt, _cumsum_of(dA), C, torch.zeros_like(prev))
+    (out * dout).sum().backward()
+    got = S.chunk_scan_bwd_ddAcs_stable(x, dt, dA_cs, dout, cb)
+    assert torch.allclose(got, dA.grad, rtol=1e-10, atol=1e-10)

@@ -501,7 +501,7 @@ struct WideSmem {
 };
 
 template <typename T, int P, int N>
-__global__ __launch_bounds__(256) void ssd_chunk_scan_wide_kernel(
+__global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
     const float* __restrict__ cb, const T* __restrict__ x, Strides3 sx, const T* __restrict__ z, Strides3 sz,
     const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Cm, Strides3 sC,
     const float* __restrict__ prev, const float* __restrict__ D, int d_has_hdim, T* __restrict__ out,
