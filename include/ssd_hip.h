@@ -93,6 +93,54 @@ int ssd_chunk_scan_fwd(const float* cb, const void* x, int64_t x_sb, int64_t x_s
                        int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate,
                        int64_t chunk, void* stream);
 
+/* ---------------------------------------------------------------- backward stages ---- */
+
+/* dprev_states[b,c,h,p,n] = sum_m round(dout[m,p] * exp(dA_m)) * C[m,n] (float32): the gradient of
+ * the chunk scan with respect to the carried states.  Replaces _chunk_scan_bwd_dstates,
+ * kernels/mamba_kernels_bwd/mamba_scan_bwd.py:91-116. */
+int ssd_chunk_scan_bwd_dstates(const void* C, int64_t c_sb, int64_t c_sl, int64_t c_sg, const void* dout,
+                               int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype, const float* dA_cumsum,
+                               float* dprev_states, int64_t batch, int64_t seqlen, int64_t nheads,
+                               int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk, void* stream);
+
+/* Bytes of workspace ssd_state_passing_bwd needs (per-wave partial dot products). */
+size_t ssd_state_passing_bwd_workspace_bytes(int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim);
+
+/* Reverse inter-chunk recurrence.  states (batch, C, nheads, dim) are the states ENTERING each
+ * chunk (index 0 the initial one), dout the gradient with respect to them, dfinal (may be NULL)
+ * the gradient of the final state.  With G the gradient of the state entering the next chunk:
+ * dstates[c] = G (the gradient of the chunk-local state), ddA_chunk[b,h,c] = exp(dA_chunk[c]) *
+ * <states[c], G> (0 for c = 0 unless dinit is given), G <- exp(dA_chunk[c]) * G + dout[c];
+ * dinit (batch, nheads, dim), may be NULL, receives the last G.  All float32.
+ * Replaces _state_passing_bwd, kernels/mamba_kernels_bwd/mamba_state_passing_bwd_dstates.py:116-172. */
+int ssd_state_passing_bwd(const float* states, const float* dA_chunk, int64_t da_sb, int64_t da_sh,
+                          int64_t da_sc, const float* dout, const float* dfinal, float* dstates,
+                          float* ddA_chunk, float* dinit, void* workspace, size_t workspace_bytes,
+                          int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, void* stream);
+
+/* dB[b,l,g,n] = sum over the heads h of group g of (sum_p x[m,p] * round(dstates[b,c,h,p,n])) *
+ * exp(min(dA_last - dA_m, 0)) * dt_m (float32, dense (batch, seqlen, ngroups, dstate)).  With B
+ * (may be NULL, then ddA_cumsum is not written): r_h[m] = sum_n db_h[m,n] * B[m,n] and
+ * ddA_cumsum[b,h,c,j] = sum_{m<j} r_h[m], the gradient of the chunk states with respect to the
+ * per-position dA.  Replaces _chunk_state_bwd_db,
+ * kernels/mamba_kernels_bwd/mamba_chunk_state_bwd_db.py:131-181 (one pass over all heads of a
+ * group, so there is no split axis to sum afterwards). */
+int ssd_chunk_state_bwd_db(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype,
+                           const float* dt, const float* dA_cumsum, const float* dstates, const void* B,
+                           int64_t b_sb, int64_t b_sl, int64_t b_sg, float* dB, float* ddA_cumsum,
+                           int64_t batch, int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim,
+                           int64_t dstate, int64_t chunk, void* stream);
+
+/* dC[b,l,g,n] = sum over the heads of group g of (sum_p dout[m,p] * round(prev[b,c,h,p,n])) *
+ * exp(dA_m): the part of dC that comes through the carried state.  With C (may be NULL):
+ * ddA_cumsum_prev[b,h,c,m] = sum_n dc_h[m,n] * C[m,n].  Replaces _chunk_scan_bwd_dC,
+ * kernels/mamba_kernels_bwd/mamba_chunk_scan_bwd_dc.py:118-160. */
+int ssd_chunk_scan_bwd_dc(const void* dout, int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype,
+                          const float* dA_cumsum, const float* prev_states, const void* C, int64_t c_sb,
+                          int64_t c_sl, int64_t c_sg, float* dC, float* ddA_cumsum_prev, int64_t batch,
+                          int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate,
+                          int64_t chunk, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

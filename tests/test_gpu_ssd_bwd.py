@@ -1,0 +1,86 @@
+"""GPU parity of the Mamba-2 SSD backward stages (through the C ABI) against the CPU oracle's
+restatements, which tests/test_ssd_oracle.py pins by autograd.  bfloat16 cases compare with the
+oracle making the roundings the reference makes before its dots."""
+import pytest
+import torch
+
+from oracle import ssd_oracle as S
+from parity_util import announce, check_close
+
+pytestmark = pytest.mark.gpu
+
+F32, BF16 = torch.float32, torch.bfloat16
+
+CASES = [
+    # b, L, nh, P, g, N, Q
+    (2, 300, 4, 64, 1, 64, 64),
+    (1, 256, 4, 64, 2, 128, 128),
+    (2, 200, 4, 64, 1, 128, 256),   # one ragged chunk
+    (1, 520, 2, 128, 1, 64, 128),
+    (1, 130, 2, 128, 2, 128, 64),
+    (1, 900, 2, 64, 1, 64, 512),
+]
+
+
+def _inputs(b, L, nh, P, g, N, Q, dtype):
+    x, dt_raw, A, B, C, D, _ = S.make_inputs(b, L, nh, P, g, N, seed=2 * L + N + Q, dtype=dtype)
+    dA_cs, dt = S.chunk_cumsum(dt_raw, A, Q)
+    gen = torch.Generator().manual_seed(L + Q)
+    dout = torch.randn(b, L, nh, P, generator=gen).to(dtype)
+    nc = dt.shape[2]
+    prev = torch.randn(b, nc, nh, P, N, generator=gen)
+    dstates = torch.randn(b, nc, nh, P, N, generator=gen)
+    return x, dt, dA_cs, B, C, D, dout, prev, dstates
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("b,L,nh,P,g,N,Q", CASES)
+def test_dstates_db_dc_vs_oracle(b, L, nh, P, g, N, Q, dtype, device):
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_bwd_dc import _chunk_scan_bwd_dC
+    from kernels.mamba_kernels_bwd.mamba_chunk_state_bwd_db import _chunk_state_bwd_db
+    from kernels.mamba_kernels_bwd.mamba_scan_bwd import _chunk_scan_bwd_dstates
+
+    announce(f"ssd bwd dstates/db/dc b{b} L{L} nh{nh} P{P} g{g} N{N} Q{Q} {dtype}")
+    x, dt, dA_cs, B, C, D, dout, prev, dstates = _inputs(b, L, nh, P, g, N, Q, dtype)
+    rt = None if dtype == F32 else dtype
+    d = lambda t: t.to(device)
+
+    got = _chunk_scan_bwd_dstates(d(C), d(dA_cs), d(dout), dtype=torch.float32)
+    check_close("dprev_states", got, S.bwd_dstates(C, dA_cs, dout, round_to=rt), dtype)
+
+    dB_ref, ddA_ref = S.chunk_state_bwd_db(x, dt, dA_cs, dstates, B=B, ngroups=g, round_to=rt)
+    dB, ddA = _chunk_state_bwd_db(d(x), d(dt), d(dA_cs), d(dstates), B=d(B), ngroups=g)
+    check_close("dB", dB, dB_ref, dtype)
+    check_close("ddA_cumsum (chunk state)", ddA, ddA_ref, dtype)
+    check_close("dB without B", _chunk_state_bwd_db(d(x), d(dt), d(dA_cs), d(dstates), ngroups=g), dB_ref, dtype)
+
+    dC_ref, ddAp_ref = S.chunk_scan_bwd_dC(prev, dA_cs, dout, C=C, ngroups=g, round_to=rt)
+    dC, ddAp = _chunk_scan_bwd_dC(d(prev), d(dA_cs), d(dout), C=d(C), ngroups=g)
+    check_close("dC", dC, dC_ref, dtype)
+    check_close("ddA_cumsum_prev", ddAp, ddAp_ref, dtype)
+
+
+@pytest.mark.parametrize("has_init", [False, True])
+@pytest.mark.parametrize("b,nc,nh,dim", [(2, 5, 3, 64 * 64), (1, 33, 2, 64 * 128), (1, 1, 1, 128 * 128), (2, 7, 2, 100)])
+def test_state_passing_bwd_vs_oracle(b, nc, nh, dim, has_init, device):
+    from kernels.mamba_kernels_bwd.mamba_state_passing_bwd_dstates import _state_passing_bwd
+
+    announce(f"ssd state passing bwd b{b} C{nc} nh{nh} dim{dim} init={has_init}")
+    gen = torch.Generator().manual_seed(dim + nc)
+    states = torch.randn(b, nc, nh, dim, generator=gen)
+    dA = -torch.rand(b, nh, nc, generator=gen)
+    dout = torch.randn(b, nc, nh, dim, generator=gen)
+    dfin = torch.randn(b, nh, dim, generator=gen)
+    ref = S.state_passing_bwd(states, dA, dout, dfin, has_initial_states=has_init)
+    dA_view = torch.empty(b, nh, nc, 4).copy_(dA[..., None])[..., -1]  # strided, like dA_cumsum[..., -1]
+    got = _state_passing_bwd(states.to(device), dA_view.to(device), dout.to(device), dfinal_states=dfin.to(device),
+                             has_initial_states=has_init)
+    check_close("dstates", got[0], ref[0], F32)
+    check_close("ddA_chunk_cumsum", got[1], ref[1], F32)
+    if has_init:
+        check_close("dinitstates", got[2], ref[2], F32)
+    else:
+        assert got[2] is None
+    got0 = _state_passing_bwd(states.to(device), dA.to(device), dout.to(device))
+    ref0 = S.state_passing_bwd(states, dA, dout)
+    check_close("dstates, no dfinal", got0[0], ref0[0], F32)

@@ -73,6 +73,7 @@ int dispatch_tpn(int dtype, int64_t P, int64_t N, F f) {
   return f.template run<float, 128, 128>();
 }
 
+template <int MODE>
 struct StateLaunch {
   const void *x, *B;
   Strides3 sx, sB;
@@ -82,7 +83,7 @@ struct StateLaunch {
   hipStream_t st;
   template <typename T, int P, int N>
   int run() const {
-    auto kernel = ssd_chunk_state_kernel<T, P, N>;
+    auto kernel = ssd_chunk_state_kernel<T, P, N, MODE>;
     constexpr int smem = StateSmem<T, P, N>::kBytes;
     SSD_TRY(allow_smem(kernel, smem));
     hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh)), dim3(256), smem, st, (const T*)x, sx,
@@ -125,6 +126,34 @@ struct ScanLaunch {
     return launched();
   }
 };
+
+template <int MODE>
+struct GroupLaunch {
+  const void* a;
+  Strides3 sa;
+  const float *s, *dt, *dA;
+  const void* bc;
+  Strides3 sbc;
+  float *out, *ddA;
+  Dims d;
+  hipStream_t st;
+  template <typename T, int P, int N>
+  int run() const {
+    auto kernel = ssd_group_grad_kernel<T, P, N, MODE>;
+    constexpr int smem = GroupSmem<T, P, N>::kBytes;
+    SSD_TRY(allow_smem(kernel, smem));
+    const int mtiles = (int)((d.Q + 63) / 64);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.g * mtiles)), dim3(256), smem, st, (const T*)a, sa,
+                       s, dt, dA, (const T*)bc, sbc, out, ddA, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L,
+                       (int)d.Q, (int)d.C, mtiles);
+    return launched();
+  }
+};
+
+int launch_row_cumsum(float* v, int64_t Q, int64_t rows, hipStream_t st) {
+  hipLaunchKernelGGL(ssd_row_cumsum_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, v, (int)Q, rows);
+  return launched();
+}
 
 template <typename T, typename TO, int K>
 int launch_bmm(const void* a, Strides3 sa, const void* bm, Strides3 sb, void* out, const Dims& d, hipStream_t st) {
@@ -179,8 +208,8 @@ int ssd_chunk_state_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64_t b_sg,
   if (!dt || !dA_cumsum) return SSD_ERR_NULL;
   SSD_TRY(check_f32(states));
   return dispatch_tpn(dtype, hdim, dstate,
-                      StateLaunch{x, B, Strides3{x_sb, x_sl, x_sh}, Strides3{b_sb, b_sl, b_sg}, dt, dA_cumsum,
-                                  states, d, as_stream(stream)});
+                      StateLaunch<0>{x, B, Strides3{x_sb, x_sl, x_sh}, Strides3{b_sb, b_sl, b_sg}, dt, dA_cumsum,
+                                     states, d, as_stream(stream)});
 }
 
 int ssd_state_passing_fwd(const float* states, const float* dA_chunk, int64_t da_sb, int64_t da_sh,
@@ -252,6 +281,99 @@ int ssd_chunk_scan_fwd(const float* cb, const void* x, int64_t x_sb, int64_t x_s
                       ScanLaunch{cb, x, z, C, Strides3{x_sb, x_sl, x_sh}, Strides3{z_sb, z_sl, z_sh},
                                  Strides3{c_sb, c_sl, c_sg}, Strides3{o_sb, o_sl, o_sh}, dt, dA_cumsum,
                                  prev_states, D, d_has_hdim, out, out_x, d, as_stream(stream)});
+}
+
+int ssd_chunk_scan_bwd_dstates(const void* C, int64_t c_sb, int64_t c_sl, int64_t c_sg, const void* dout,
+                               int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype, const float* dA_cumsum,
+                               float* dprev_states, int64_t batch, int64_t seqlen, int64_t nheads,
+                               int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk, void* stream) {
+  Dims d;
+  SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
+  SSD_TRY(check_dtype(dtype));
+  if (!dim_ok(hdim) || !dim_ok(dstate)) return SSD_ERR_UNSUPPORTED;
+  SSD_TRY(check_vec(dout, d_sb, d_sl, d_sh, dtype, hdim));
+  SSD_TRY(check_vec(C, c_sb, c_sl, c_sg, dtype, dstate));
+  if (!dA_cumsum) return SSD_ERR_NULL;
+  SSD_TRY(check_f32(dprev_states));
+  return dispatch_tpn(dtype, hdim, dstate,
+                      StateLaunch<1>{dout, C, Strides3{d_sb, d_sl, d_sh}, Strides3{c_sb, c_sl, c_sg}, dA_cumsum,
+                                     dA_cumsum, dprev_states, d, as_stream(stream)});
+}
+
+size_t ssd_state_passing_bwd_workspace_bytes(int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim) {
+  if (batch <= 0 || nchunks <= 0 || nheads <= 0 || dim <= 0) return 0;
+  const int64_t tiles = (dim + 1023) / 1024;
+  return (size_t)(batch * nheads * nchunks * tiles * 4) * sizeof(float);
+}
+
+int ssd_state_passing_bwd(const float* states, const float* dA_chunk, int64_t da_sb, int64_t da_sh,
+                          int64_t da_sc, const float* dout, const float* dfinal, float* dstates,
+                          float* ddA_chunk, float* dinit, void* workspace, size_t workspace_bytes,
+                          int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, void* stream) {
+  if (batch <= 0 || nchunks <= 0 || nheads <= 0 || dim <= 0) return SSD_ERR_SHAPE;
+  if (dim % 4) return SSD_ERR_ALIGN;
+  if (!dA_chunk || !ddA_chunk) return SSD_ERR_NULL;
+  SSD_TRY(check_f32(states));
+  SSD_TRY(check_f32(dout));
+  SSD_TRY(check_f32(dstates));
+  SSD_TRY(check_f32(workspace));
+  if (dfinal) SSD_TRY(check_f32(dfinal));
+  if (dinit) SSD_TRY(check_f32(dinit));
+  if (workspace_bytes < ssd_state_passing_bwd_workspace_bytes(batch, nchunks, nheads, dim)) return SSD_ERR_SHAPE;
+  const int tiles = (int)((dim + 1023) / 1024);
+  const int64_t grid = batch * nheads * tiles;
+  if (grid > 0x7fffffff || dim > (1 << 24)) return SSD_ERR_SHAPE;
+  hipStream_t st = as_stream(stream);
+  float* part = static_cast<float*>(workspace);
+  hipLaunchKernelGGL(ssd_state_passing_bwd_kernel, dim3((unsigned)grid), dim3(256), 0, st, states, dA_chunk, da_sb,
+                     da_sh, da_sc, dout, dfinal, dstates, part, dinit, (int)nheads, (int)nchunks, (int)dim, tiles);
+  SSD_TRY(launched());
+  const int64_t total = batch * nheads * nchunks;
+  hipLaunchKernelGGL(ssd_state_passing_bwd_finish_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                     part, dA_chunk, da_sb, da_sh, da_sc, ddA_chunk, (int)nheads, (int)nchunks, tiles * 4,
+                     dinit ? 1 : 0, total);
+  return launched();
+}
+
+int ssd_chunk_state_bwd_db(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype,
+                           const float* dt, const float* dA_cumsum, const float* dstates, const void* B,
+                           int64_t b_sb, int64_t b_sl, int64_t b_sg, float* dB, float* ddA_cumsum,
+                           int64_t batch, int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim,
+                           int64_t dstate, int64_t chunk, void* stream) {
+  Dims d;
+  SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
+  SSD_TRY(check_dtype(dtype));
+  if (!dim_ok(hdim) || !dim_ok(dstate)) return SSD_ERR_UNSUPPORTED;
+  SSD_TRY(check_vec(x, x_sb, x_sl, x_sh, dtype, hdim));
+  if (!dt || !dA_cumsum || !dB) return SSD_ERR_NULL;
+  SSD_TRY(check_f32(dstates));
+  if (B && !ddA_cumsum) return SSD_ERR_NULL;
+  if (B) SSD_TRY(check_vec(B, b_sb, b_sl, b_sg, dtype, dstate));
+  hipStream_t st = as_stream(stream);
+  SSD_TRY(dispatch_tpn(dtype, hdim, dstate,
+                       GroupLaunch<0>{x, Strides3{x_sb, x_sl, x_sh}, dstates, dt, dA_cumsum, B,
+                                      Strides3{b_sb, b_sl, b_sg}, dB, ddA_cumsum, d, st}));
+  if (!B) return SSD_OK;
+  return launch_row_cumsum(ddA_cumsum, chunk, batch * nheads * d.C, st);
+}
+
+int ssd_chunk_scan_bwd_dc(const void* dout, int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype,
+                          const float* dA_cumsum, const float* prev_states, const void* C, int64_t c_sb,
+                          int64_t c_sl, int64_t c_sg, float* dC, float* ddA_cumsum_prev, int64_t batch,
+                          int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate,
+                          int64_t chunk, void* stream) {
+  Dims d;
+  SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
+  SSD_TRY(check_dtype(dtype));
+  if (!dim_ok(hdim) || !dim_ok(dstate)) return SSD_ERR_UNSUPPORTED;
+  SSD_TRY(check_vec(dout, d_sb, d_sl, d_sh, dtype, hdim));
+  if (!dA_cumsum || !dC) return SSD_ERR_NULL;
+  SSD_TRY(check_f32(prev_states));
+  if (C && !ddA_cumsum_prev) return SSD_ERR_NULL;
+  if (C) SSD_TRY(check_vec(C, c_sb, c_sl, c_sg, dtype, dstate));
+  return dispatch_tpn(dtype, hdim, dstate,
+                      GroupLaunch<1>{dout, Strides3{d_sb, d_sl, d_sh}, prev_states, dA_cumsum, dA_cumsum, C,
+                                     Strides3{c_sb, c_sl, c_sg}, dC, ddA_cumsum_prev, d, as_stream(stream)});
 }
 
 }  // extern "C"

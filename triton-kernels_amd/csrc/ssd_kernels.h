@@ -150,10 +150,13 @@ __global__ __launch_bounds__(256) void ssd_cumsum_kernel(const TD* __restrict__ 
 }
 
 // ------------------------------------------------------------------------------------
-// chunk_state.  One workgroup (4 waves) per (b, c, h):
-//   states[p][n] = sum_k x[k][p] * round_T(B[k][n] * exp(min(dA_last - dA_k, 0)) * dt_k).
-// The chunk is walked in stages of 64 rows; both operands are contracted along their rows.
-// The (P/32) x (N/32) output blocks are dealt to the waves round-robin.
+// chunk_state (MODE 0) and its mirror image in the backward, dstates (MODE 1).  One workgroup
+// (4 waves) per (b, c, h):
+//   MODE 0  states[p][n] = sum_k x[k][p] * round_T(B[k][n] * exp(min(dA_last - dA_k, 0)) * dt_k)
+//   MODE 1  dprev[p][n]  = sum_k round_T(dout[k][p] * exp(dA_k)) * C[k][n]
+// (x / B stand for dout / C in MODE 1; dt is not read).  The chunk is walked in stages of 64
+// rows; both operands are contracted along their rows.  The (P/32) x (N/32) output blocks are
+// dealt to the waves round-robin.
 // ------------------------------------------------------------------------------------
 template <typename T, int P, int N>
 struct StateSmem {
@@ -161,7 +164,7 @@ struct StateSmem {
   static constexpr int kBytes = KT * (PX + PB) * (int)sizeof(T);
 };
 
-template <typename T, int P, int N>
+template <typename T, int P, int N, int MODE>
 __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
     const T* __restrict__ x, Strides3 sx, const T* __restrict__ B, Strides3 sB,
     const float* __restrict__ dt, const float* __restrict__ dA_cs, float* __restrict__ states, int nh,
@@ -189,10 +192,15 @@ __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
   for (int i = 0; i < BPW; ++i) zero_acc(acc[i]);
 
   for (int k0 = 0; k0 < limit; k0 += KT) {
-    stage_rows<T, KT, P>(xs, xg, sx.sl, k0, limit, tid, NoScale());
-    stage_rows<T, KT, N>(bs, Bg, sB.sl, k0, limit, tid, [&](int k) {
-      return __expf(fminf(dA_last - dAp[k], 0.f)) * dtp[k];
-    });
+    if (MODE == 0) {
+      stage_rows<T, KT, P>(xs, xg, sx.sl, k0, limit, tid, NoScale());
+      stage_rows<T, KT, N>(bs, Bg, sB.sl, k0, limit, tid, [&](int k) {
+        return __expf(fminf(dA_last - dAp[k], 0.f)) * dtp[k];
+      });
+    } else {
+      stage_rows<T, KT, P>(xs, xg, sx.sl, k0, limit, tid, [&](int k) { return __expf(dAp[k]); });
+      stage_rows<T, KT, N>(bs, Bg, sB.sl, k0, limit, tid, NoScale());
+    }
     __syncthreads();
 #pragma unroll
     for (int kk = 0; kk < KT; kk += KG) {
@@ -259,6 +267,255 @@ __global__ __launch_bounds__(256) void ssd_state_passing_kernel(
     }
   }
   *reinterpret_cast<float4*>(final_states + (b * nh + h) * (int64_t)dim + e) = s;
+}
+
+// Sum over the 32 lanes of each half of a wave (lanes 0..31 and 32..63 apart), left in lanes 31
+// and 63: the DPP prefix steps of wave_inclusive_scan without the last one.
+__device__ __forceinline__ float half_wave_sum(float v) {
+  v += ema::dpp_or_zero<0x111, 0xf>(v);
+  v += ema::dpp_or_zero<0x112, 0xf>(v);
+  v += ema::dpp_or_zero<0x114, 0xf>(v);
+  v += ema::dpp_or_zero<0x118, 0xf>(v);
+  v += ema::dpp_or_zero<0x142, 0xa>(v);
+  return v;
+}
+
+// ------------------------------------------------------------------------------------
+// state_passing backward.  With G the gradient of the state entering the next chunk (G starts
+// from dfinal or 0): dstates[c] = G, part[(b,h,c), wave] = <states[c], G> over the wave's
+// elements, G <- exp(dA_chunk[c]) * G + dout[c]; after chunk 0, G goes to dinit if asked.
+// The finish kernel sums the wave partials: ddA[b,h,c] = exp(dA_chunk[c]) * sum, and 0 for
+// c = 0 when there is no initial state.
+// ------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void ssd_state_passing_bwd_kernel(
+    const float* __restrict__ states, const float* __restrict__ dA_chunk, int64_t da_sb, int64_t da_sh,
+    int64_t da_sc, const float* __restrict__ dout, const float* __restrict__ dfinal,
+    float* __restrict__ dstates, float* __restrict__ part, float* __restrict__ dinit, int nh, int C, int dim,
+    int tiles) {
+  const int tile = blockIdx.x % tiles;
+  const int h = (blockIdx.x / tiles) % nh;
+  const int64_t b = blockIdx.x / (tiles * nh);
+  const int e = (tile * 256 + threadIdx.x) * 4;
+  const bool ok = e < dim;
+  const int lane = threadIdx.x & 63;
+  const int wave_id = tile * 4 + (threadIdx.x >> 6), nw = tiles * 4;
+  const int64_t chunk_stride = (int64_t)nh * dim;
+  const int64_t base = (b * C * nh + h) * (int64_t)dim + (ok ? e : 0);
+  const float* da = dA_chunk + b * da_sb + h * da_sh;
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 G = (dfinal && ok) ? *reinterpret_cast<const float4*>(dfinal + (b * nh + h) * (int64_t)dim + e) : zero4;
+  constexpr int U = 4;
+  for (int c1 = C - 1; c1 >= 0; c1 -= U) {
+    float4 sv[U], dv[U];
+    float a[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = c1 - u;
+      const bool in = c >= 0 && ok;
+      sv[u] = in ? *reinterpret_cast<const float4*>(states + base + c * chunk_stride) : zero4;
+      dv[u] = in ? *reinterpret_cast<const float4*>(dout + base + c * chunk_stride) : zero4;
+      a[u] = c >= 0 ? __expf(da[(int64_t)c * da_sc]) : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = c1 - u;
+      if (c >= 0) {  // uniform across the workgroup
+        if (ok) *reinterpret_cast<float4*>(dstates + base + c * chunk_stride) = G;
+        const float dot = ema::wave_sum(sv[u].x * G.x + sv[u].y * G.y + sv[u].z * G.z + sv[u].w * G.w);
+        if (lane == 0) part[((b * nh + h) * C + c) * (int64_t)nw + wave_id] = dot;
+        G.x = fmaf(a[u], G.x, dv[u].x);
+        G.y = fmaf(a[u], G.y, dv[u].y);
+        G.z = fmaf(a[u], G.z, dv[u].z);
+        G.w = fmaf(a[u], G.w, dv[u].w);
+      }
+    }
+  }
+  if (dinit && ok) *reinterpret_cast<float4*>(dinit + (b * nh + h) * (int64_t)dim + e) = G;
+}
+
+__global__ __launch_bounds__(256) void ssd_state_passing_bwd_finish_kernel(
+    const float* __restrict__ part, const float* __restrict__ dA_chunk, int64_t da_sb, int64_t da_sh,
+    int64_t da_sc, float* __restrict__ ddA, int nh, int C, int nw, int has_init, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // (b * nh + h) * C + c
+  if (i >= total) return;
+  const int c = (int)(i % C);
+  const int64_t bh = i / C;
+  const int h = (int)(bh % nh);
+  const int64_t b = bh / nh;
+  float s = 0.f;
+  for (int w = 0; w < nw; ++w) s += part[i * nw + w];
+  ddA[i] = (c == 0 && !has_init) ? 0.f : __expf(dA_chunk[b * da_sb + h * da_sh + (int64_t)c * da_sc]) * s;
+}
+
+// In-place inclusive cumsum along the last axis of a dense (rows, Q) float32 array; one wave
+// per row, lane l owns ceil(Q/64) consecutive positions.
+__global__ __launch_bounds__(256) void ssd_row_cumsum_kernel(float* __restrict__ v, int Q, int64_t rows) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int per = (Q + 63) >> 6;
+  float* p = v + row * Q;
+  float local = 0.f;
+  for (int i = 0; i < per; ++i) {
+    const int q = lane * per + i;
+    if (q < Q) local += p[q];
+  }
+  float run = wave_inclusive_scan(local) - local;
+  for (int i = 0; i < per; ++i) {
+    const int q = lane * per + i;
+    if (q < Q) {
+      run += p[q];
+      p[q] = run;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// Gradients that are summed over the heads of a group: dB (MODE 0) and the carried-state part
+// of dC (MODE 1).  One workgroup per (b, c, g, tile of 64 rows m), looping over the group's heads:
+//   per head   d_h[m][n] = (sum_p a[m][p] * round_T(s[p][n])) * w_m
+//     MODE 0:  a = x,    s = dstates, w_m = exp(min(dA_last - dA_m, 0)) * dt_m
+//     MODE 1:  a = dout, s = prev,    w_m = exp(dA_m)
+//   out[m][n] = sum_h d_h[m][n]                       (float32, (b, L, g, N))
+//   with bc (B for MODE 0, C for MODE 1): r_h[m] = sum_n d_h[m][n] * bc[m][n], written to
+//   ddA[b,h,c, m + 1] (MODE 0, slot 0 = 0; the caller then takes the cumsum) or ddA[b,h,c,m] (MODE 1).
+// a is read row-major straight from global memory; s is staged in LDS (rounded to T) and
+// contracted along its rows.
+// ------------------------------------------------------------------------------------
+template <typename T, int P, int N>
+struct GroupSmem {
+  static constexpr int PS = Tile<T>::pitch(N);
+  static constexpr int kBytes = P * PS * (int)sizeof(T) + 4 * 64 * (int)sizeof(float);
+};
+
+template <typename T, int P, int N, int MODE>
+__global__ __launch_bounds__(256) void ssd_group_grad_kernel(
+    const T* __restrict__ a, Strides3 sa, const float* __restrict__ s, const float* __restrict__ dt,
+    const float* __restrict__ dA_cs, const T* __restrict__ bc, Strides3 sbc, float* __restrict__ out,
+    float* __restrict__ ddA, int nh, int heads_per_group, int ngroups, int L, int Q, int C, int mtiles) {
+  using S = GroupSmem<T, P, N>;
+  constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, NB = N / 32, BPW = 2 * NB / 4;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T* St = reinterpret_cast<T*>(smem);
+  float* rs = reinterpret_cast<float*>(smem + P * S::PS * sizeof(T));  // [4 waves][64 rows]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
+  const int mt = blockIdx.x % mtiles;
+  const int g = (blockIdx.x / mtiles) % ngroups;
+  const int c = (blockIdx.x / (mtiles * ngroups)) % C;
+  const int64_t b = blockIdx.x / ((int64_t)mtiles * ngroups * C);
+  const int limit = min(Q, L - c * Q);
+  const int m0 = 64 * mt;
+
+  // block i of this wave: rows 32*mi.., columns 32*ni..
+  int mi[BPW], ni[BPW];
+#pragma unroll
+  for (int i = 0; i < BPW; ++i) {
+    const int j = wave + 4 * i;
+    mi[i] = j & 1;
+    ni[i] = j >> 1;
+  }
+  // bc in the accumulator layout (float), once per workgroup
+  float bcv[BPW][16];
+  const bool want_ddA = bc != nullptr;
+  if (want_ddA) {
+    const T* bcg = bc + b * sbc.sb + (int64_t)c * Q * sbc.sl + g * sbc.sh;
+#pragma unroll
+    for (int i = 0; i < BPW; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + 32 * mi[i] + acc_row(v, lane);
+        bcv[i][v] = m < limit ? (float)bcg[(int64_t)m * sbc.sl + 32 * ni[i] + l32] : 0.f;
+      }
+  }
+  floatx16 total[BPW];
+#pragma unroll
+  for (int i = 0; i < BPW; ++i) zero_acc(total[i]);
+
+  for (int hh = 0; hh < heads_per_group; ++hh) {
+    const int h = g * heads_per_group + hh;
+    const int64_t chunk = (b * nh + h) * C + c;
+    const float* dAp = dA_cs + chunk * Q;
+    const float* dtp = dt + chunk * Q;
+    const float* sg = s + (((b * C + c) * nh + h) * (int64_t)P) * N;
+    {
+      constexpr int VPR = N / 4;
+#pragma unroll
+      for (int i = 0; i < P * VPR / 256; ++i) {
+        const int idx = tid + 256 * i;
+        const int r = idx / VPR, cv = (idx % VPR) * 4;
+        const float4 v = *reinterpret_cast<const float4*>(sg + (int64_t)r * N + cv);
+        T* d = St + r * S::PS + cv;
+        d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
+      }
+    }
+    __syncthreads();
+    floatx16 acc[BPW];
+#pragma unroll
+    for (int i = 0; i < BPW; ++i) zero_acc(acc[i]);
+    const T* ag = a + b * sa.sb + (int64_t)c * Q * sa.sl + h * sa.sh;
+#pragma unroll
+    for (int kk = 0; kk < P; kk += KG) {
+#pragma unroll
+      for (int i = 0; i < BPW; ++i) {
+        const int m = m0 + 32 * mi[i] + l32;
+        Vec16<T> av;
+        if (m < limit) av = load16(ag + (int64_t)m * sa.sl + kk + EPL * half);
+        else av.zero();
+        mma_group(av, frag_cols(St, S::PS, kk, 32 * ni[i], lane), acc[i]);
+      }
+    }
+    const float dA_last = dAp[Q - 1];
+#pragma unroll
+    for (int i = 0; i < BPW; ++i) {
+      float r16[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + 32 * mi[i] + acc_row(v, lane);
+        float w = 0.f;
+        if (m < Q) w = MODE == 0 ? __expf(fminf(dA_last - dAp[m], 0.f)) * dtp[m] : __expf(dAp[m]);
+        const float d = acc[i][v] * w;
+        total[i][v] += d;
+        r16[v] = d * (want_ddA ? bcv[i][v] : 0.f);
+      }
+      if (want_ddA) {
+        // rows of this block over its 32 columns, then over the column blocks through LDS
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const float t = half_wave_sum(r16[v]);
+          if (l32 == 31) {
+            float* dst = rs + wave * 64 + 32 * mi[i] + acc_row(v, lane);
+            if (i == 0) *dst = t;
+            else *dst += t;  // the wave's second block covers the same rows
+          }
+        }
+      }
+    }
+    __syncthreads();
+    if (want_ddA && tid < 64) {
+      // row block tid / 32 belongs to the waves w0 = tid / 32 and w0 + 2 (a wave's blocks share
+      // their rows and differ in their columns)
+      const int w0 = tid >> 5;
+      const float r = rs[w0 * 64 + tid] + rs[(w0 + 2) * 64 + tid];
+      const int m = m0 + tid;
+      float* o = ddA + chunk * Q;
+      if (MODE == 0) {
+        if (m + 1 < Q) o[m + 1] = r;
+        if (m == 0) o[0] = 0.f;
+      } else if (m < Q) {
+        o[m] = r;
+      }
+    }
+    // the next head's staging overwrites St; rs is rewritten only after the next barrier
+  }
+  float* og = out + (b * L + (int64_t)c * Q) * ngroups * N + (int64_t)g * N;
+#pragma unroll
+  for (int i = 0; i < BPW; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int m = m0 + 32 * mi[i] + acc_row(v, lane);
+      if (m < limit) og[(int64_t)m * ngroups * N + 32 * ni[i] + l32] = total[i][v];
+    }
 }
 
 // ------------------------------------------------------------------------------------

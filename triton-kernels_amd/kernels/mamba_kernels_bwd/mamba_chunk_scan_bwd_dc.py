@@ -1,0 +1,36 @@
+"""SSD backward: the part of dC that comes through the carried state, and the matching gradient
+of dA_cumsum.
+
+Mirrors _chunk_scan_bwd_dC, kernels/mamba_kernels_bwd/mamba_chunk_scan_bwd_dc.py:118-160 of the
+reference (no split axis: one workgroup walks all heads of a group)."""
+import torch
+
+from kernels import _lib
+
+
+def _chunk_scan_bwd_dC(prev_states, dA_cumsum, dout, seq_idx=None, C=None, ngroups=1):
+    batch, nchunks, nheads, headdim, dstate = prev_states.shape
+    _, seqlen, _, _ = dout.shape
+    _, _, _, chunk_size = dA_cumsum.shape
+    assert prev_states.shape == (batch, nchunks, nheads, headdim, dstate)
+    assert dA_cumsum.shape == (batch, nheads, nchunks, chunk_size)
+    assert dout.shape == (batch, seqlen, nheads, headdim)
+    if seq_idx is not None:
+        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
+    dev = _lib.require_gpu(prev_states, dA_cumsum, dout)
+    dout, ds = _lib.strided4(dout)
+    cs = [None, 0, 0, 0]
+    ddA_prev = None
+    if C is not None:
+        assert C.shape == (batch, seqlen, ngroups, dstate)
+        C, cs = _lib.strided4(C.to(dout.dtype))
+        ddA_prev = torch.empty(batch, nheads, nchunks, chunk_size, device=dev, dtype=torch.float32)
+    dC = torch.empty(batch, seqlen, ngroups, dstate, device=dev, dtype=torch.float32)
+    with torch.cuda.device(dev):
+        _lib.check(
+            _lib.lib().ssd_chunk_scan_bwd_dc(*ds, _lib.dtype_code(dout), _lib.f32c(dA_cumsum).data_ptr(),
+                                             _lib.f32c(prev_states).data_ptr(), *cs, dC.data_ptr(),
+                                             None if ddA_prev is None else ddA_prev.data_ptr(), batch, seqlen,
+                                             nheads, ngroups, headdim, dstate, chunk_size, _lib.stream_ptr(dev)),
+            "ssd_chunk_scan_bwd_dc")
+    return dC if C is None else (dC, ddA_prev)

@@ -1,0 +1,32 @@
+"""SSD backward: gradient of the chunk scan with respect to the carried states.
+
+Mirrors _chunk_scan_bwd_dstates, kernels/mamba_kernels_bwd/mamba_scan_bwd.py:91-116 of the
+reference."""
+import torch
+
+from kernels import _lib
+
+
+def _chunk_scan_bwd_dstates(C, dA_cumsum, dout, seq_idx=None, dtype=None):
+    batch, seqlen, nheads, headdim = dout.shape
+    _, _, nchunks, chunk_size = dA_cumsum.shape
+    _, _, ngroups, dstate = C.shape
+    assert nheads % ngroups == 0
+    assert C.shape == (batch, seqlen, ngroups, dstate)
+    assert dA_cumsum.shape == (batch, nheads, nchunks, chunk_size)
+    if seq_idx is not None:
+        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
+    dev = _lib.require_gpu(C, dA_cumsum, dout)
+    dtype = C.dtype if dtype is None else dtype
+    dout, ds = _lib.strided4(dout)
+    if C.dtype != dout.dtype:
+        C = C.to(dout.dtype)
+    C, cs = _lib.strided4(C)
+    out = torch.empty(batch, nchunks, nheads, headdim, dstate, device=dev, dtype=torch.float32)
+    with torch.cuda.device(dev):
+        _lib.check(
+            _lib.lib().ssd_chunk_scan_bwd_dstates(*cs, *ds, _lib.dtype_code(dout), _lib.f32c(dA_cumsum).data_ptr(),
+                                                  out.data_ptr(), batch, seqlen, nheads, ngroups, headdim, dstate,
+                                                  chunk_size, _lib.stream_ptr(dev)),
+            "ssd_chunk_scan_bwd_dstates")
+    return out if dtype == torch.float32 else out.to(dtype)

@@ -1,0 +1,46 @@
+"""SSD backward: the reverse inter-chunk recurrence.
+
+Mirrors _state_passing_bwd, kernels/mamba_kernels_bwd/mamba_state_passing_bwd_dstates.py:116-172
+of the reference (same arguments, same tuple of results)."""
+import torch
+
+from kernels import _lib
+
+
+def _state_passing_bwd(states, dA_chunk_cumsum, dout, dfinal_states=None, seq_idx=None, has_initial_states=None,
+                       dstates_dtype=None, states_dtype=None, chunk_size=None):
+    """states holds the state entering each chunk (the initial state at index 0); the final state
+    is not part of it."""
+    batch, nchunks, nheads, dim = states.shape
+    assert dA_chunk_cumsum.shape == (batch, nheads, nchunks)
+    assert dout.shape == (batch, nchunks, nheads, dim)
+    if seq_idx is not None:
+        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
+    if dfinal_states is not None:
+        assert dfinal_states.shape == (batch, nheads, dim)
+    dev = _lib.require_gpu(states, dA_chunk_cumsum, dout)
+    lib = _lib.lib()
+    st, do = _lib.f32c(states), _lib.f32c(dout)
+    da = dA_chunk_cumsum if dA_chunk_cumsum.dtype == torch.float32 else dA_chunk_cumsum.float()
+    dfin = None if dfinal_states is None else _lib.f32c(dfinal_states)
+    dstates = torch.empty(batch, nchunks, nheads, dim, device=dev, dtype=torch.float32)
+    ddA = torch.empty(batch, nheads, nchunks, device=dev, dtype=torch.float32)
+    dinit = torch.empty(batch, nheads, dim, device=dev, dtype=torch.float32) if has_initial_states else None
+    nbytes = lib.ssd_state_passing_bwd_workspace_bytes(batch, nchunks, nheads, dim)
+    ws = torch.empty(max(nbytes, 16), device=dev, dtype=torch.uint8)
+    with torch.cuda.device(dev):
+        _lib.check(
+            lib.ssd_state_passing_bwd(st.data_ptr(), da.data_ptr(), da.stride(0), da.stride(1), da.stride(2),
+                                      do.data_ptr(), None if dfin is None else dfin.data_ptr(), dstates.data_ptr(),
+                                      ddA.data_ptr(), None if dinit is None else dinit.data_ptr(), ws.data_ptr(),
+                                      nbytes, batch, nchunks, nheads, dim, _lib.stream_ptr(dev)),
+            "ssd_state_passing_bwd")
+    out_dtype = dstates_dtype if dstates_dtype is not None else dout.dtype
+    if out_dtype != torch.float32:
+        dstates = dstates.to(out_dtype)
+        dinit = None if dinit is None else dinit.to(out_dtype)
+    ddA = ddA.to(dA_chunk_cumsum.dtype)
+    if states_dtype is None:
+        return dstates, ddA, dinit
+    states_converted = states if states_dtype == states.dtype else states.to(out_dtype)
+    return dstates, ddA, dinit, states_converted
