@@ -141,6 +141,22 @@ int ssd_chunk_scan_bwd_dc(const void* dout, int64_t d_sb, int64_t d_sl, int64_t 
                           int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate,
                           int64_t chunk, void* stream);
 
+/* acc[m,p] = exp(min(dA_last - dA_m, 0)) * sum_n B[m,n] * round(dstates[p,n])
+ *          + sum_{k>=m} round(cb[k,m] * exp(min(dA_k - dA_m, 0))) * dout[k,p];
+ * dx = acc * dt_m + D * dout (type `dtype`, dx's own strides), ddt[b,h,c,m] = sum_p acc[m,p] * x[m,p]
+ * (float32, 0 past seqlen).  cb float32 (batch, C, ngroups, Q, Q), dstates float32
+ * (batch, C, nheads, hdim, dstate), D as for ssd_chunk_scan_fwd (its gradient, sum dout * x, is
+ * left to the caller).  Replaces _chunk_scan_chunk_state_bwd_dx,
+ * kernels/mamba_kernels_bwd/mamba_chunk_scan_chunk_state_bwd_dx.py:189-248. */
+int ssd_chunk_scan_chunk_state_bwd_dx(const float* cb, const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
+                                      const void* dout, int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype,
+                                      const float* dt, const float* dA_cumsum, const void* B, int64_t b_sb,
+                                      int64_t b_sl, int64_t b_sg, const float* dstates, const float* D,
+                                      int d_has_hdim, void* dx, int64_t dx_sb, int64_t dx_sl, int64_t dx_sh,
+                                      float* ddt, int64_t batch, int64_t seqlen, int64_t nheads,
+                                      int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
+                                      void* stream);
+
 #ifdef __cplusplus
 }
 #endif

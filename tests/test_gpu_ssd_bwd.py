@@ -84,3 +84,29 @@ def test_state_passing_bwd_vs_oracle(b, nc, nh, dim, has_init, device):
     got0 = _state_passing_bwd(states.to(device), dA.to(device), dout.to(device))
     ref0 = S.state_passing_bwd(states, dA, dout)
     check_close("dstates, no dfinal", got0[0], ref0[0], F32)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("b,L,nh,P,g,N,Q", CASES)
+def test_dx_vs_oracle(b, L, nh, P, g, N, Q, dtype, device):
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_chunk_state_bwd_dx import _chunk_scan_chunk_state_bwd_dx
+
+    announce(f"ssd bwd dx b{b} L{L} nh{nh} P{P} g{g} N{N} Q{Q} {dtype}")
+    x, dt, dA_cs, B, C, D, dout, prev, dstates = _inputs(b, L, nh, P, g, N, Q, dtype)
+    rt = None if dtype == F32 else dtype
+    d = lambda t: t.to(device)
+    cb = S.bmm_chunk(C, B, Q)
+    dx_ref, ddt_ref, dD_ref = S.chunk_scan_chunk_state_bwd_dx(x, dt, dA_cs, B, cb, dout, dstates, D=D, round_to=rt)
+    dx, ddt, dD = _chunk_scan_chunk_state_bwd_dx(d(x), d(dt), d(dA_cs), d(B), d(cb), d(dout), d(dstates), D=d(D))
+    check_close("dx", dx, dx_ref, dtype)
+    check_close("ddt", ddt, ddt_ref, dtype, loose=dtype == BF16)
+    check_close("dD", dD, dD_ref, F32)
+    D2 = torch.randn(nh, P, generator=torch.Generator().manual_seed(1))
+    dx_ref2, _, dD_ref2 = S.chunk_scan_chunk_state_bwd_dx(x, dt, dA_cs, B, cb, dout, dstates, D=D2, round_to=rt)
+    dx2, _, dD2 = _chunk_scan_chunk_state_bwd_dx(d(x), d(dt), d(dA_cs), d(B), d(cb), d(dout), d(dstates), D=d(D2))
+    check_close("dx (D per feature)", dx2, dx_ref2, dtype)
+    check_close("dD per feature", dD2, dD_ref2, F32)
+    dx3, _, none = _chunk_scan_chunk_state_bwd_dx(d(x), d(dt), d(dA_cs), d(B), d(cb), d(dout), d(dstates))
+    assert none is None
+    check_close("dx (no D)", dx3, S.chunk_scan_chunk_state_bwd_dx(x, dt, dA_cs, B, cb, dout, dstates, round_to=rt)[0],
+                dtype)

@@ -127,6 +127,29 @@ struct ScanLaunch {
   }
 };
 
+struct DxLaunch {
+  const float* cb;
+  const void *x, *dout, *B;
+  Strides3 sx, sd, sB, sdx;
+  const float *dt, *dA, *dstates, *D;
+  int d_has_hdim;
+  void* dx;
+  float* ddt;
+  Dims d;
+  hipStream_t st;
+  template <typename T, int P, int N>
+  int run() const {
+    auto kernel = ssd_chunk_scan_bwd_dx_kernel<T, P, N>;
+    constexpr int smem = ScanSmem<T, P, N>::kBytes;
+    SSD_TRY(allow_smem(kernel, smem));
+    const int mtiles = (int)((d.Q + 63) / 64);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh * mtiles)), dim3(256), smem, st, cb,
+                       (const T*)x, sx, (const T*)dout, sd, dt, dA, (const T*)B, sB, dstates, D, d_has_hdim, (T*)dx,
+                       sdx, ddt, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C, mtiles);
+    return launched();
+  }
+};
+
 template <int MODE>
 struct GroupLaunch {
   const void* a;
@@ -374,6 +397,32 @@ int ssd_chunk_scan_bwd_dc(const void* dout, int64_t d_sb, int64_t d_sl, int64_t 
   return dispatch_tpn(dtype, hdim, dstate,
                       GroupLaunch<1>{dout, Strides3{d_sb, d_sl, d_sh}, prev_states, dA_cumsum, dA_cumsum, C,
                                      Strides3{c_sb, c_sl, c_sg}, dC, ddA_cumsum_prev, d, as_stream(stream)});
+}
+
+int ssd_chunk_scan_chunk_state_bwd_dx(const float* cb, const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
+                                      const void* dout, int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype,
+                                      const float* dt, const float* dA_cumsum, const void* B, int64_t b_sb,
+                                      int64_t b_sl, int64_t b_sg, const float* dstates, const float* D,
+                                      int d_has_hdim, void* dx, int64_t dx_sb, int64_t dx_sl, int64_t dx_sh,
+                                      float* ddt, int64_t batch, int64_t seqlen, int64_t nheads,
+                                      int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
+                                      void* stream) {
+  Dims d;
+  SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
+  SSD_TRY(check_dtype(dtype));
+  if (!dim_ok(hdim) || !dim_ok(dstate)) return SSD_ERR_UNSUPPORTED;
+  SSD_TRY(check_vec(x, x_sb, x_sl, x_sh, dtype, hdim));
+  SSD_TRY(check_vec(dout, d_sb, d_sl, d_sh, dtype, hdim));
+  SSD_TRY(check_vec(dx, dx_sb, dx_sl, dx_sh, dtype, hdim));
+  SSD_TRY(check_vec(B, b_sb, b_sl, b_sg, dtype, dstate));
+  if (!dt || !dA_cumsum || !ddt) return SSD_ERR_NULL;
+  SSD_TRY(check_f32(cb));
+  SSD_TRY(check_f32(dstates));
+  if (batch * d.C * nheads * ((chunk + 63) / 64) > 0x7fffffff) return SSD_ERR_SHAPE;
+  return dispatch_tpn(dtype, hdim, dstate,
+                      DxLaunch{cb, x, dout, B, Strides3{x_sb, x_sl, x_sh}, Strides3{d_sb, d_sl, d_sh},
+                               Strides3{b_sb, b_sl, b_sg}, Strides3{dx_sb, dx_sl, dx_sh}, dt, dA_cumsum, dstates, D,
+                               d_has_hdim, dx, ddt, d, as_stream(stream)});
 }
 
 }  // extern "C"

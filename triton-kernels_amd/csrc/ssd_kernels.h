@@ -923,4 +923,162 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------
+// Backward of chunk_scan and chunk_state with respect to x (and the explicit dt factors).
+// One workgroup per (b, c, h, tile of 64 rows m):
+//   acc[m][p] = exp(min(dA_last - dA_m, 0)) * sum_n B[m][n] * round_T(dstates[p][n])
+//             + sum_{k >= m, k < limit} round_T(cb[k][m] * exp(min(dA_k - dA_m, 0))) * dout[k][p]
+//   dx[m][p] = acc * dt_m + D * dout[m][p],    ddt[m] = sum_p acc[m][p] * x[m][p]
+// The mirror image of ssd_chunk_scan_kernel: the k tiles run from the diagonal one to the end
+// of the chunk, and the weights are staged transposed (k-major), so that cb is still read along
+// its rows.
+// ------------------------------------------------------------------------------------
+template <typename T, int P, int N>
+__global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
+    const float* __restrict__ cb, const T* __restrict__ x, Strides3 sx, const T* __restrict__ dout, Strides3 sd,
+    const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Bm, Strides3 sB,
+    const float* __restrict__ dstates, const float* __restrict__ D, int d_has_hdim, T* __restrict__ dx,
+    Strides3 sdx, float* __restrict__ ddt, int nh, int heads_per_group, int ngroups, int L, int Q, int C,
+    int mtiles) {
+  using S = ScanSmem<T, P, N>;
+  constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, PB = P / 32, BPW = 2 * PB / 4;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T* Bs = reinterpret_cast<T*>(smem);
+  T* Ps = Bs + 64 * S::PC;
+  T* Ds = reinterpret_cast<T*>(smem);
+  T* Wt = Ds + 64 * S::PX;  // [k][m]
+  float* Os = reinterpret_cast<float*>(smem);
+  float* sm = reinterpret_cast<float*>(smem + S::kBytes - 64 * sizeof(float));
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int mt = blockIdx.x % mtiles;
+  const int h = (blockIdx.x / mtiles) % nh;
+  const int c = (blockIdx.x / (mtiles * nh)) % C;
+  const int64_t b = blockIdx.x / ((int64_t)mtiles * nh * C);
+  const int limit = min(Q, L - c * Q);
+  const int m0 = 64 * mt;
+  const int64_t chunk = (b * nh + h) * C + c;
+  float* ddtp = ddt + chunk * Q;
+  if (m0 >= limit) {  // nothing of the sequence in this tile: its ddt slots are zero
+    if (tid < 64 && m0 + tid < Q) ddtp[m0 + tid] = 0.f;
+    return;
+  }
+  const int g = h / heads_per_group;
+  const float* dAp = dA_cs + chunk * Q;
+  const float* dtp = dt + chunk * Q;
+  const T* xg = x + b * sx.sb + (int64_t)c * Q * sx.sl + h * sx.sh;
+  const T* dg = dout + b * sd.sb + (int64_t)c * Q * sd.sl + h * sd.sh;
+  const T* Bg = Bm + b * sB.sb + (int64_t)c * Q * sB.sl + g * sB.sh;
+  const float* sg = dstates + (((b * C + c) * nh + h) * (int64_t)P) * N;
+  const float* cbg = cb + (((b * C + c) * ngroups + g) * (int64_t)Q) * Q;
+
+  const int mi = wave & 1, pi0 = wave >> 1;
+  floatx16 acc[BPW];
+#pragma unroll
+  for (int i = 0; i < BPW; ++i) zero_acc(acc[i]);
+
+  // ---- phase A: B . dstates, scaled by the decay to the end of the chunk
+  stage_rows<T, 64, N>(Bs, Bg, sB.sl, m0, limit, tid, NoScale());
+  {
+    constexpr int VPR = N / 4;
+#pragma unroll
+    for (int i = 0; i < P * VPR / 256; ++i) {
+      const int idx = tid + 256 * i;
+      const int r = idx / VPR, cv = (idx % VPR) * 4;
+      const float4 v = *reinterpret_cast<const float4*>(sg + (int64_t)r * N + cv);
+      T* d = Ps + r * S::PC + cv;
+      d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
+    }
+  }
+  if (tid < 64) sm[tid] = m0 + tid < Q ? __expf(fminf(dAp[Q - 1] - dAp[m0 + tid], 0.f)) : 0.f;
+  __syncthreads();
+#pragma unroll
+  for (int kk = 0; kk < N; kk += KG) {
+    const Vec16<T> a = frag_rows(Bs, S::PC, 32 * mi, kk, lane);
+#pragma unroll
+    for (int i = 0; i < BPW; ++i) mma_group(a, frag_rows(Ps, S::PC, 32 * (pi0 + 2 * i), kk, lane), acc[i]);
+  }
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const float sc = sm[32 * mi + acc_row(v, lane)];
+#pragma unroll
+    for (int i = 0; i < BPW; ++i) acc[i][v] *= sc;
+  }
+  __syncthreads();
+
+  // ---- phase B: the k tiles from the diagonal one to the end of the chunk
+  const int ktiles = (limit + 63) / 64;
+  for (int kt = mt; kt < ktiles; ++kt) {
+    const int k0 = 64 * kt;
+    stage_rows<T, 64, P>(Ds, dg, sd.sl, k0, limit, tid, NoScale());
+#pragma unroll
+    for (int i = 0; i < 64 * 16 / 256; ++i) {
+      const int idx = tid + 256 * i;
+      const int r = idx >> 4, cv = (idx & 15) * 4;  // row k0 + r of cb, columns m0 + cv ..
+      const int k = k0 + r;
+      T* d = Wt + r * S::PW + cv;
+      if (k < limit && m0 + cv < Q) {
+        const float4 w4 = *reinterpret_cast<const float4*>(cbg + (int64_t)k * Q + m0 + cv);
+        const float4 a4 = *reinterpret_cast<const float4*>(dAp + m0 + cv);
+        const float ak = dAp[k];
+        const float w[4] = {w4.x, w4.y, w4.z, w4.w}, am[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) d[e] = (T)(k >= m0 + cv + e ? w[e] * __expf(fminf(ak - am[e], 0.f)) : 0.f);
+      } else {
+        d[0] = d[1] = d[2] = d[3] = (T)0.f;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 64; kk += KG) {
+      const Vec16<T> a = frag_cols(Wt, S::PW, kk, 32 * mi, lane);
+#pragma unroll
+      for (int i = 0; i < BPW; ++i) mma_group(a, frag_cols(Ds, S::PX, kk, 32 * (pi0 + 2 * i), lane), acc[i]);
+    }
+    __syncthreads();
+  }
+
+  // ---- phase C: through LDS; dx = acc * dt + D * dout, ddt = <acc, x> per row
+#pragma unroll
+  for (int i = 0; i < BPW; ++i) {
+    const int col = 32 * (pi0 + 2 * i) + (lane & 31);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) Os[(32 * mi + acc_row(v, lane)) * S::PO + col] = acc[i][v];
+  }
+  __syncthreads();
+  constexpr int VPR = P / EPL;
+#pragma unroll
+  for (int i = 0; i < 64 * VPR / 256; ++i) {
+    const int idx = tid + 256 * i;
+    const int r = idx / VPR, cv = (idx % VPR) * EPL;
+    const int m = m0 + r;
+    float dot = 0.f;
+    if (m < limit) {
+      const int64_t pos = (int64_t)c * Q + m;
+      const Vec16<T> xv = load16(x + b * sx.sb + pos * sx.sl + h * sx.sh + cv);
+      const float dtm = dtp[m];
+      float v[EPL];
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) {
+        v[e] = Os[r * S::PO + cv + e];
+        dot = fmaf(v[e], xv.get(e), dot);
+        v[e] *= dtm;
+      }
+      if (D) {
+        const Vec16<T> dv = load16(dout + b * sd.sb + pos * sd.sl + h * sd.sh + cv);
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) v[e] = fmaf(d_has_hdim ? D[h * P + cv + e] : D[h], dv.get(e), v[e]);
+      }
+      Vec16<T> o;
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) o.set(e, v[e]);
+      store16(dx + b * sdx.sb + pos * sdx.sl + h * sdx.sh + cv, o);
+    }
+    // the VPR lanes of a row are adjacent: butterfly sum, then one of them writes
+#pragma unroll
+    for (int off = 1; off < VPR; off <<= 1) dot += __shfl_xor(dot, off);
+    if ((idx % VPR) == 0 && m < Q) ddtp[m] = dot;
+  }
+}
+
 }  // namespace ssd

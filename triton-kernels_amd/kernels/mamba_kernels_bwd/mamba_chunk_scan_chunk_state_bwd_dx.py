@@ -1,0 +1,49 @@
+"""SSD backward: dx, the explicit-dt gradient ddt and dD.
+
+Mirrors _chunk_scan_chunk_state_bwd_dx,
+kernels/mamba_kernels_bwd/mamba_chunk_scan_chunk_state_bwd_dx.py:189-248 of the reference (same
+arguments, returns (dx, ddt, dD)).  dD = sum dout * x is a plain reduction and is taken in torch."""
+import torch
+
+from kernels import _lib
+
+
+def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum, B, CB, dout, dstates, D=None, seq_idx=None, dx=None):
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, nchunks, chunk_size = dt.shape
+    _, _, ngroups, dstate = B.shape
+    assert nheads % ngroups == 0
+    assert B.shape == (batch, seqlen, ngroups, dstate)
+    assert CB.shape == (batch, nchunks, ngroups, chunk_size, chunk_size)
+    assert dt.shape == (batch, nheads, nchunks, chunk_size)
+    assert dA_cumsum.shape == dt.shape
+    assert dout.shape == x.shape
+    assert dstates.shape == (batch, nchunks, nheads, headdim, dstate)
+    if seq_idx is not None:
+        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
+    if D is not None:
+        assert D.shape == (nheads, headdim) or D.shape == (nheads,)
+    dev = _lib.require_gpu(x, dt, dA_cumsum, B, CB, dout, dstates)
+    x, xs = _lib.strided4(x)
+    dout, ds = _lib.strided4(dout.to(x.dtype))
+    B, bs = _lib.strided4(B.to(x.dtype))
+    if dx is None:
+        dx = torch.empty_like(x)
+    else:
+        assert dx.shape == x.shape and dx.dtype == x.dtype and dx.stride(-1) == 1
+    ddt = torch.empty(batch, nheads, nchunks, chunk_size, device=dev, dtype=torch.float32)
+    Df = None if D is None else _lib.f32c(D)
+    with torch.cuda.device(dev):
+        _lib.check(
+            _lib.lib().ssd_chunk_scan_chunk_state_bwd_dx(
+                _lib.f32c(CB).data_ptr(), *xs, *ds, _lib.dtype_code(x), _lib.f32c(dt).data_ptr(),
+                _lib.f32c(dA_cumsum).data_ptr(), *bs, _lib.f32c(dstates).data_ptr(),
+                None if Df is None else Df.data_ptr(), int(D is not None and D.dim() == 2), dx.data_ptr(),
+                dx.stride(0), dx.stride(1), dx.stride(2), ddt.data_ptr(), batch, seqlen, nheads, ngroups, headdim,
+                dstate, chunk_size, _lib.stream_ptr(dev)),
+            "ssd_chunk_scan_chunk_state_bwd_dx")
+    dD = None
+    if D is not None:
+        prod = dout.float() * x.float()
+        dD = (prod.sum((0, 1)) if D.dim() == 2 else prod.sum((0, 1, 3))).to(D.dtype)
+    return dx, ddt.to(dtype=dt.dtype), dD
