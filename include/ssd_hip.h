@@ -157,6 +157,21 @@ int ssd_chunk_scan_chunk_state_bwd_dx(const float* cb, const void* x, int64_t x_
                                       int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
                                       void* stream);
 
+/* Bytes of workspace ssd_chunk_scan_bwd_ddAcs needs (column sums per row tile, row sums). */
+size_t ssd_chunk_scan_bwd_ddAcs_workspace_bytes(int64_t batch, int64_t seqlen, int64_t nheads, int64_t chunk);
+
+/* With W[m,n] = <dout[m], x[n]> * dt_n * cb[m,n] * exp(min(dA_m - dA_n, 0)) for n < m:
+ * ddA_cumsum[b,h,c,j] = sum_{m>=j} sum_{n<j} W[m,n] (float32; 0 for j = 0): the gradient of the causal
+ * term of the chunk scan with respect to the per-position dA.  It is formed as the prefix sum of
+ * (column sum - row sum) of W, which is the same quantity as the reference's row-wise cumsum
+ * followed by column sums.  Replaces _chunk_scan_bwd_ddAcs_stable,
+ * kernels/mamba_kernels_bwd/mamba_chunk_scan_bwd_da.py:111-140 (and its torch sum over row blocks). */
+int ssd_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, const void* dout,
+                             int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype, const float* dt,
+                             const float* dA_cumsum, const float* cb, float* ddA_cumsum, void* workspace,
+                             size_t workspace_bytes, int64_t batch, int64_t seqlen, int64_t nheads,
+                             int64_t ngroups, int64_t hdim, int64_t chunk, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -110,3 +110,17 @@ def test_dx_vs_oracle(b, L, nh, P, g, N, Q, dtype, device):
     assert none is None
     check_close("dx (no D)", dx3, S.chunk_scan_chunk_state_bwd_dx(x, dt, dA_cs, B, cb, dout, dstates, round_to=rt)[0],
                 dtype)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("b,L,nh,P,g,N,Q", CASES)
+def test_ddAcs_vs_oracle(b, L, nh, P, g, N, Q, dtype, device):
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_bwd_da import _chunk_scan_bwd_ddAcs_stable
+
+    announce(f"ssd bwd ddAcs b{b} L{L} nh{nh} P{P} g{g} N{N} Q{Q} {dtype}")
+    x, dt, dA_cs, B, C, D, dout, prev, dstates = _inputs(b, L, nh, P, g, N, Q, dtype)
+    d = lambda t: t.to(device)
+    cb = S.bmm_chunk(C, B, Q)
+    ref = S.chunk_scan_bwd_ddAcs_stable(x, dt, dA_cs, dout, cb)
+    got = _chunk_scan_bwd_ddAcs_stable(d(x), d(dt), d(dA_cs), d(dout), d(cb))
+    check_close("ddA_cumsum (causal term)", got, ref, dtype, loose=dtype == BF16)

@@ -210,14 +210,14 @@ int launch_da(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, int d
   if (dtype == EMA_BF16)
     hipLaunchKernelGGL((da_gemm_kernel<bf16_t>), dim3((unsigned)grid), dim3(256), 0, st,
                        (const bf16_t*)x, sx, (const bf16_t*)dy, sd, cs, part, rowsum, (int)d.nh,
-                       (int)d.L, (int)d.T, (int)d.Q, (int)d.C, MT);
+                       (int)d.L, (int)d.T, (int)d.Q, (int)d.C, MT, nullptr, nullptr, 1, 1);
   else
     hipLaunchKernelGGL((da_gemm_kernel<float>), dim3((unsigned)grid), dim3(256), 0, st,
                        (const float*)x, sx, (const float*)dy, sd, cs, part, rowsum, (int)d.nh,
-                       (int)d.L, (int)d.T, (int)d.Q, (int)d.C, MT);
+                       (int)d.L, (int)d.T, (int)d.Q, (int)d.C, MT, nullptr, nullptr, 1, 1);
   EMA_TRY(launched());
   const int64_t total = d.N * d.C;
-  hipLaunchKernelGGL(da_finish_kernel, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, st, part,
+  hipLaunchKernelGGL(da_finish_kernel<kBM>, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, st, part,
                      rowsum, ddA_intra, (int)d.Q, MT, total);
   return launched();
 }

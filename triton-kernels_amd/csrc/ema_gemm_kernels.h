@@ -12,7 +12,10 @@ constexpr int kBM = 128;  // rows of a chunk handled by one workgroup (4 waves x
 // B6, first part.  For the chunk (n, c) and the row tile mt (rows m of dy), for every
 // column tile kt <= mt (rows k of x):
 //   G[m,k] = <dy[m,:], x[k,:]>  (MFMA over the feature axis, operands read row-major)
-//   W[m,k] = G[m,k] * exp(min(cs[m]-cs[k],0)) for k < m, else 0
+//   W[m,k] = G[m,k] * exp(min(cs[m]-cs[k],0)) for k < m, else 0; with wk (per-position
+//            weights, laid out like cs) and wmk (a (batch, C, ngroups, Q, Q) matrix per chunk
+//            and group of heads_per_group heads) also * wk[k] * wmk[m,k]: the form the SSD
+//            scan needs (wk = dt, wmk = C B^T); both are null for the EMA scan
 //   part[(chunk*MT + mt)*Q + k] = sum_m W[m,k]      (column sums of this row tile)
 //   rowsum[chunk*Q + m]         = sum_k W[m,k]      (complete: all k < m are visited)
 // da_finish_kernel turns these into ddA_intra.
@@ -23,7 +26,10 @@ __global__ __launch_bounds__(256) void da_gemm_kernel(const T* __restrict__ x, S
                                                       const float* __restrict__ cs,
                                                       float* __restrict__ part,
                                                       float* __restrict__ rowsum, int nh, int L,
-                                                      int Tdim, int Q, int C, int MT) {
+                                                      int Tdim, int Q, int C, int MT,
+                                                      const float* __restrict__ wk,
+                                                      const float* __restrict__ wmk,
+                                                      int heads_per_group, int ngroups) {
   constexpr int EPL = Vec16<T>::N;
   constexpr int KG = 2 * EPL;
   constexpr int DK = 4 * KG;        // feature columns per LDS stage (128 bytes per row)
@@ -50,6 +56,8 @@ __global__ __launch_bounds__(256) void da_gemm_kernel(const T* __restrict__ x, S
   const int mt_base = mt * kBM;
 
   const float* csp = cs + chunk_id * Q;
+  const float* wkp = wk ? wk + chunk_id * Q : nullptr;
+  const float* wmp = wmk ? wmk + (((b * C + c) * ngroups + h / heads_per_group) * (int64_t)Q) * Q : nullptr;
   const int q_pad = (Q + kBM - 1) / kBM * kBM;
   for (int i = tid; i < q_pad; i += 256) cs_s[i] = i < Q ? csp[i] : 0.f;
 
@@ -110,11 +118,15 @@ __global__ __launch_bounds__(256) void da_gemm_kernel(const T* __restrict__ x, S
       if (cb < ncb) {
         const int k = kt_base + cb * 32 + l32;
         const float cs_k = cs_s[k];
+        const float wk_k = (wkp && k < Q) ? wkp[k] : 1.f;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int m = mt_base + wave * 32 + acc_row(v, lane);
           float w = 0.f;
-          if (k < m && m < limit) w = acc[cb][v] * __expf(fminf(cs_s[m] - cs_k, 0.f));
+          if (k < m && m < limit) {
+            w = acc[cb][v] * __expf(fminf(cs_s[m] - cs_k, 0.f)) * wk_k;
+            if (wmp) w *= wmp[(int64_t)m * Q + k];
+          }
           rowacc[v] += w;
           colacc += w;
         }
@@ -149,6 +161,7 @@ __global__ __launch_bounds__(256) void da_gemm_kernel(const T* __restrict__ x, S
 
 // B6, second part: ddA_intra[j] = sum_{i<j} (colsum[i] - rowsum[i]) with
 // colsum[i] = sum over the row tiles mt >= i / 128 of part[mt][i].  One wave per (n, c).
+template <int BM>
 __global__ __launch_bounds__(256) void da_finish_kernel(const float* __restrict__ part,
                                                         const float* __restrict__ rowsum,
                                                         float* __restrict__ ddA_intra, int Q,
@@ -160,7 +173,7 @@ __global__ __launch_bounds__(256) void da_finish_kernel(const float* __restrict_
   const int q0 = lane * per;
   auto val = [&](int q) {
     float s = -rowsum[chunk_id * Q + q];
-    for (int mt = q / kBM; mt < MT; ++mt) s += part[(chunk_id * MT + mt) * (int64_t)Q + q];
+    for (int mt = q / BM; mt < MT; ++mt) s += part[(chunk_id * MT + mt) * (int64_t)Q + q];
     return s;
   };
   float local = 0.f;

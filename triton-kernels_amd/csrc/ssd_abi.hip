@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include "ema_gemm_kernels.h"
 #include "ssd_kernels.h"
 
 using namespace ssd;
@@ -423,6 +424,54 @@ int ssd_chunk_scan_chunk_state_bwd_dx(const float* cb, const void* x, int64_t x_
                       DxLaunch{cb, x, dout, B, Strides3{x_sb, x_sl, x_sh}, Strides3{d_sb, d_sl, d_sh},
                                Strides3{b_sb, b_sl, b_sg}, Strides3{dx_sb, dx_sl, dx_sh}, dt, dA_cumsum, dstates, D,
                                d_has_hdim, dx, ddt, d, as_stream(stream)});
+}
+
+static size_t ddAcs_part_floats(const Dims& d) {
+  const int64_t MT = (d.Q + ema::kBM - 1) / ema::kBM;
+  return (size_t)(d.batch * d.nh * d.C * MT * d.Q);
+}
+
+size_t ssd_chunk_scan_bwd_ddAcs_workspace_bytes(int64_t batch, int64_t seqlen, int64_t nheads, int64_t chunk) {
+  Dims d;
+  if (check_dims(batch, seqlen, nheads, 1, 0, 0, chunk, &d) != SSD_OK) return 0;
+  return (ddAcs_part_floats(d) + (size_t)(batch * nheads * d.C * chunk)) * sizeof(float);
+}
+
+int ssd_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, const void* dout,
+                             int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype, const float* dt,
+                             const float* dA_cumsum, const float* cb, float* ddA_cumsum, void* workspace,
+                             size_t workspace_bytes, int64_t batch, int64_t seqlen, int64_t nheads,
+                             int64_t ngroups, int64_t hdim, int64_t chunk, void* stream) {
+  Dims d;
+  SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, 0, chunk, &d));
+  SSD_TRY(check_dtype(dtype));
+  if (hdim <= 0 || hdim > (1 << 16)) return SSD_ERR_SHAPE;
+  SSD_TRY(check_vec(x, x_sb, x_sl, x_sh, dtype, hdim));
+  SSD_TRY(check_vec(dout, d_sb, d_sl, d_sh, dtype, hdim));
+  if (!dt || !dA_cumsum || !cb || !ddA_cumsum) return SSD_ERR_NULL;
+  SSD_TRY(check_f32(workspace));
+  if (workspace_bytes < ssd_chunk_scan_bwd_ddAcs_workspace_bytes(batch, seqlen, nheads, chunk)) return SSD_ERR_SHAPE;
+  hipStream_t st = as_stream(stream);
+  float* part = static_cast<float*>(workspace);
+  float* rowsum = part + ddAcs_part_floats(d);
+  const int MT = (int)((d.Q + ema::kBM - 1) / ema::kBM);
+  const int64_t grid = batch * nheads * d.C * MT;
+  if (grid > 0x7fffffff) return SSD_ERR_SHAPE;
+  const ema::SeqStrides sx{x_sb, x_sl, x_sh}, sd{d_sb, d_sl, d_sh};
+  const int hpg = (int)(nheads / ngroups);
+  if (dtype == SSD_BF16)
+    hipLaunchKernelGGL((ema::da_gemm_kernel<bf16_t>), dim3((unsigned)grid), dim3(256), 0, st, (const bf16_t*)x, sx,
+                       (const bf16_t*)dout, sd, dA_cumsum, part, rowsum, (int)nheads, (int)seqlen, (int)hdim,
+                       (int)chunk, (int)d.C, MT, dt, cb, hpg, (int)ngroups);
+  else
+    hipLaunchKernelGGL((ema::da_gemm_kernel<float>), dim3((unsigned)grid), dim3(256), 0, st, (const float*)x, sx,
+                       (const float*)dout, sd, dA_cumsum, part, rowsum, (int)nheads, (int)seqlen, (int)hdim,
+                       (int)chunk, (int)d.C, MT, dt, cb, hpg, (int)ngroups);
+  SSD_TRY(launched());
+  const int64_t total = batch * nheads * d.C;
+  hipLaunchKernelGGL(ema::da_finish_kernel<ema::kBM>, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, st, part,
+                     rowsum, ddA_cumsum, (int)chunk, MT, total);
+  return launched();
 }
 
 }  // extern "C"

@@ -60,6 +60,8 @@ _SIGNATURES = {
     "ssd_chunk_state_bwd_db": (c_int, _SEQ + [c_int, _P, _P, _P] + _SEQ + [_P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "ssd_chunk_scan_bwd_dc": (c_int, _SEQ + [c_int, _P, _P] + _SEQ + [_P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "ssd_chunk_scan_chunk_state_bwd_dx": (c_int, [_P] + _SEQ + _SEQ + [c_int, _P, _P] + _SEQ + [_P, _P, c_int] + _SEQ + [_P, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "ssd_chunk_scan_bwd_ddAcs_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
+    "ssd_chunk_scan_bwd_ddAcs": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _I, _P]),
 }
 
 _lib = None
