@@ -136,6 +136,12 @@ def ssd_main(args):
     from kernels.mamba_kernels.mamba_scan_fwd import _chunk_scan_fwd
     from kernels.mamba_kernels.mamba_state_fwd import _chunk_state_fwd
     from kernels.mamba_kernels.mamba_state_pass import _state_passing_fwd
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_bwd_da import _chunk_scan_bwd_ddAcs_stable
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_bwd_dc import _chunk_scan_bwd_dC
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_chunk_state_bwd_dx import _chunk_scan_chunk_state_bwd_dx
+    from kernels.mamba_kernels_bwd.mamba_chunk_state_bwd_db import _chunk_state_bwd_db
+    from kernels.mamba_kernels_bwd.mamba_scan_bwd import _chunk_scan_bwd_dstates
+    from kernels.mamba_kernels_bwd.mamba_state_passing_bwd_dstates import _state_passing_bwd
     from oracle import ssd_oracle as S
 
     dev = torch.device("cuda:0")
@@ -150,8 +156,11 @@ def ssd_main(args):
         out, _, dt_out, dA_cs, states, _ = _mamba_chunk_scan_combined_fwd(x, dt, A, B, Cm, Q)
         st = _chunk_state_fwd(B, x, dt_out, dA_cs)
         cb = _bmm_chunk_fwd(Cm, B, Q, output_dtype=torch.float32)
-        inter.append((dt_out, dA_cs, st, states, cb))
-    del out
+        dout = torch.randn_like(x)
+        dprev = _chunk_scan_bwd_dstates(Cm, dA_cs, dout, dtype=torch.float32)
+        dstates, _, _ = _state_passing_bwd(states.view(b, C, nh, P * N), dA_cs[..., -1], dprev.view(b, C, nh, P * N))
+        inter.append((dt_out, dA_cs, st, states, cb, dout, dprev, dstates.view(b, C, nh, P, N)))
+    del out, dprev, dstates
 
     def pick(i):
         k = i % len(sets)
@@ -164,6 +173,15 @@ def ssd_main(args):
         "bmm_chunk": lambda i: _bmm_chunk_fwd(pick(i)[4], pick(i)[3], Q, output_dtype=torch.float32),
         "chunk_scan": lambda i: _chunk_scan_fwd(pick(i)[9], pick(i)[0], pick(i)[5], pick(i)[6], pick(i)[4], pick(i)[8]),
         "forward": lambda i: _mamba_chunk_scan_combined_fwd(*pick(i)[:5], Q),
+        # backward stages (the reference has no combined backward): x dt A B C | dt_out dA st states cb dout dprev dstates
+        "bwd_dstates": lambda i: _chunk_scan_bwd_dstates(pick(i)[4], pick(i)[6], pick(i)[10], dtype=torch.float32),
+        "bwd_state_passing": lambda i: _state_passing_bwd(pick(i)[8].view(b, C, nh, P * N), pick(i)[6][..., -1],
+                                                          pick(i)[11].view(b, C, nh, P * N)),
+        "bwd_db": lambda i: _chunk_state_bwd_db(pick(i)[0], pick(i)[5], pick(i)[6], pick(i)[12], B=pick(i)[3], ngroups=g),
+        "bwd_dc": lambda i: _chunk_scan_bwd_dC(pick(i)[8], pick(i)[6], pick(i)[10], C=pick(i)[4], ngroups=g),
+        "bwd_dx": lambda i: _chunk_scan_chunk_state_bwd_dx(pick(i)[0], pick(i)[5], pick(i)[6], pick(i)[3], pick(i)[9],
+                                                           pick(i)[10], pick(i)[12]),
+        "bwd_ddAcs": lambda i: _chunk_scan_bwd_ddAcs_stable(pick(i)[0], pick(i)[5], pick(i)[6], pick(i)[10], pick(i)[9]),
     }
     xb = b * L * nh * P * 2
     bc = b * L * g * N * 2
@@ -174,10 +192,15 @@ def ssd_main(args):
         "chunk_cumsum": 3 * dtb, "chunk_state": xb + bc + 2 * dtb + stb, "state_passing": 2 * stb + dtb // Q,
         "bmm_chunk": 2 * bc + cbb, "chunk_scan": cbb + 2 * xb + bc + stb + 2 * dtb,
         "forward": 2 * xb + 2 * bc + dtb,
+        "bwd_dstates": xb + bc + dtb + stb, "bwd_state_passing": 3 * stb + 2 * dtb // Q,
+        "bwd_db": xb + stb + 2 * dtb + bc + 2 * bc + dtb, "bwd_dc": xb + stb + dtb + bc + 2 * bc + dtb,
+        "bwd_dx": cbb + 3 * xb + bc + stb + 3 * dtb, "bwd_ddAcs": 2 * xb + 3 * dtb + cbb,
     }
     units = b * C * nh
     flops = {"chunk_state": 2 * Q * P * N * units, "bmm_chunk": 2 * Q * Q * N * b * C * g,
-             "chunk_scan": (2 * Q * Q * P + 2 * Q * N * P) * units}
+             "chunk_scan": (2 * Q * Q * P + 2 * Q * N * P) * units, "bwd_dstates": 2 * Q * P * N * units,
+             "bwd_db": 2 * Q * P * N * units, "bwd_dc": 2 * Q * P * N * units,
+             "bwd_dx": (2 * Q * Q * P + 2 * Q * N * P) * units, "bwd_ddAcs": 2 * Q * Q * P * units}
     res = {}
     for name, fn in stages.items():
         if args.stage and name != args.stage:
@@ -193,7 +216,8 @@ def ssd_main(args):
     if args.stage:
         print(json.dumps({"stage": args.stage, **res[args.stage], "steps": args.steps}))
         return
-    dom = max((k for k in res if k != "forward"), key=lambda k: res[k]["ms"])
+    res["backward_stages_sum"] = {"ms": sum(v["ms"] for k, v in res.items() if k.startswith("bwd_"))}
+    dom = max((k for k in res if k not in ("forward", "backward_stages_sum")), key=lambda k: res[k]["ms"])
     out = {
         "metric": "Mamba-2 SSD fwd ms @ b8 nh32 hdim64 dstate128 g1 L8192 c256",
         "value": res["forward"]["ms"], "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -124,3 +124,68 @@ def test_ddAcs_vs_oracle(b, L, nh, P, g, N, Q, dtype, device):
     ref = S.chunk_scan_bwd_ddAcs_stable(x, dt, dA_cs, dout, cb)
     got = _chunk_scan_bwd_ddAcs_stable(d(x), d(dt), d(dA_cs), d(dout), d(cb))
     check_close("ddA_cumsum (causal term)", got, ref, dtype, loose=dtype == BF16)
+
+
+def test_config5_backward_stages_full_size(device):
+    """b8 nh32 hdim64 dstate128 g1 L8192 Q256 bf16: every backward launcher runs on the whole
+    workload; batch element 0 of each result is compared with the oracle."""
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_bwd_da import _chunk_scan_bwd_ddAcs_stable
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_bwd_dc import _chunk_scan_bwd_dC
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_chunk_state_bwd_dx import _chunk_scan_chunk_state_bwd_dx
+    from kernels.mamba_kernels_bwd.mamba_chunk_state_bwd_db import _chunk_state_bwd_db
+    from kernels.mamba_kernels_bwd.mamba_scan_bwd import _chunk_scan_bwd_dstates
+    from kernels.mamba_kernels_bwd.mamba_state_passing_bwd_dstates import _state_passing_bwd
+
+    announce("ssd config 5 backward stages, full size")
+    b, L, nh, P, g, N, Q = 8, 8192, 32, 64, 1, 128, 256
+    C_ = L // Q
+    x, dt_raw, A, B, C, _, _ = S.make_inputs(b, L, nh, P, g, N, seed=5, dtype=BF16)
+    dA_cs, dt = S.chunk_cumsum(dt_raw, A, Q)
+    gen = torch.Generator().manual_seed(55)
+    dout = torch.randn(b, L, nh, P, generator=gen).to(BF16)
+    d = lambda t: t.to(device)
+    xd, dtd, dAd, Bd, Cd, doutd = d(x), d(dt), d(dA_cs), d(B), d(C), d(dout)
+    one = lambda t: t[:1]
+
+    # forward intermediates of element 0 from the oracle (float32), the rest from the GPU
+    st0 = S.chunk_state(one(B), one(x), one(dt), one(dA_cs), round_to=BF16)
+    prev0, _ = S.state_passing(st0.reshape(1, C_, nh, P * N), one(dA_cs)[..., -1])
+    prev0 = prev0.reshape(1, C_, nh, P, N)
+    cb0 = S.bmm_chunk(one(C), one(B), Q)
+    from kernels.mamba_kernels.mamba_combined_fwd import _mamba_chunk_scan_combined_fwd
+    from kernels.mamba_kernels.mamba_bmm import _bmm_chunk_fwd
+    _, _, _, _, prevd, _ = _mamba_chunk_scan_combined_fwd(xd, d(dt_raw), d(A), Bd, Cd, Q)
+    cbd = _bmm_chunk_fwd(Cd, Bd, Q, output_dtype=torch.float32)
+    check_close("prev states[0] (forward)", prevd[:1], prev0, BF16)
+
+    dprev = _chunk_scan_bwd_dstates(Cd, dAd, doutd, dtype=torch.float32)
+    dprev0 = S.bwd_dstates(one(C), one(dA_cs), one(dout), round_to=BF16)
+    check_close("dprev_states[0]", dprev[:1], dprev0, BF16)
+
+    dstates, ddA_chunk, _ = _state_passing_bwd(prevd.view(b, C_, nh, P * N), dAd[..., -1], dprev.view(b, C_, nh, P * N))
+    ds0, ddAc0, _ = S.state_passing_bwd(prev0.reshape(1, C_, nh, P * N), one(dA_cs)[..., -1],
+                                        dprev0.reshape(1, C_, nh, P * N))
+    check_close("dstates[0]", dstates[:1], ds0, BF16, loose=True)
+    check_close("ddA_chunk[0]", ddA_chunk[:1], ddAc0, BF16, loose=True)
+    dstates5, ds05 = dstates.view(b, C_, nh, P, N), ds0.reshape(1, C_, nh, P, N)
+
+    dB, ddA_b = _chunk_state_bwd_db(xd, dtd, dAd, dstates5, B=Bd, ngroups=g)
+    dB0, ddAb0 = S.chunk_state_bwd_db(one(x), one(dt), one(dA_cs), ds05, B=one(B), ngroups=g, round_to=BF16)
+    check_close("dB[0]", dB[:1], dB0, BF16, loose=True)
+    check_close("ddA (chunk state)[0]", ddA_b[:1], ddAb0, BF16, loose=True)
+
+    dC, ddA_p = _chunk_scan_bwd_dC(prevd, dAd, doutd, C=Cd, ngroups=g)
+    dC0, ddAp0 = S.chunk_scan_bwd_dC(prev0, one(dA_cs), one(dout), C=one(C), ngroups=g, round_to=BF16)
+    check_close("dC[0]", dC[:1], dC0, BF16, loose=True)
+    check_close("ddA_prev[0]", ddA_p[:1], ddAp0, BF16, loose=True)
+
+    dx, ddt, _ = _chunk_scan_chunk_state_bwd_dx(xd, dtd, dAd, Bd, cbd, doutd, dstates5)
+    dx0, ddt0, _ = S.chunk_scan_chunk_state_bwd_dx(one(x), one(dt), one(dA_cs), one(B), cb0, one(dout), ds05, round_to=BF16)
+    check_close("dx[0]", dx[:1], dx0, BF16, loose=True)
+    check_close("ddt[0]", ddt[:1], ddt0, BF16, loose=True)
+
+    ddA_s = _chunk_scan_bwd_ddAcs_stable(xd, dtd, dAd, doutd, cbd)
+    check_close("ddA (causal term)[0]", ddA_s[:1], S.chunk_scan_bwd_ddAcs_stable(one(x), one(dt), one(dA_cs), one(dout), cb0),
+                BF16, loose=True)
+    for name, t in (("dprev", dprev), ("dstates", dstates), ("dB", dB), ("dC", dC), ("dx", dx), ("ddt", ddt), ("ddA", ddA_s)):
+        assert torch.isfinite(t.float()).all(), name
