@@ -122,11 +122,11 @@ __global__ __launch_bounds__(256) void da_gemm_kernel(const T* __restrict__ x, S
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int m = mt_base + wave * 32 + acc_row(v, lane);
-          float w = 0.f;
-          if (k < m && m < limit) {
-            w = acc[cb][v] * __expf(fminf(cs_s[m] - cs_k, 0.f)) * wk_k;
-            if (wmp) w *= wmp[(int64_t)m * Q + k];
-          }
+          float w = acc[cb][v] * __expf(fminf(cs_s[m] - cs_k, 0.f)) * wk_k;
+          // the load is unconditional (row and column clamped into the matrix) so that the
+          // sixteen of a block are in flight together
+          if (wmp) w *= wmp[(int64_t)min(m, Q - 1) * Q + min(k, Q - 1)];
+          w = (k < m && m < limit) ? w : 0.f;
           rowacc[v] += w;
           colacc += w;
         }

@@ -452,6 +452,31 @@ int ssd_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t 
   SSD_TRY(check_f32(workspace));
   if (workspace_bytes < ssd_chunk_scan_bwd_ddAcs_workspace_bytes(batch, seqlen, nheads, chunk)) return SSD_ERR_SHAPE;
   hipStream_t st = as_stream(stream);
+  if ((chunk == 64 || chunk == 128 || chunk == 256) && dim_ok(hdim)) {
+    // one workgroup per (b, c, h) does everything, prefix sum included
+    const int64_t wgs = batch * nheads * d.C;
+    if (wgs > 0x7fffffff) return SSD_ERR_SHAPE;
+    const Strides3 sx{x_sb, x_sl, x_sh}, sd{d_sb, d_sl, d_sh};
+    const int hpg = (int)(nheads / ngroups);
+#define SSD_DDA_LAUNCH(T, P)                                                                                    \
+  do {                                                                                                          \
+    auto kernel = ssd_ddA_causal_kernel<T, P>;                                                                  \
+    constexpr int smem = DdaSmem<T, P>::kBytes;                                                                 \
+    SSD_TRY(allow_smem(kernel, smem));                                                                          \
+    hipLaunchKernelGGL(kernel, dim3((unsigned)wgs), dim3(256), smem, st, (const T*)x, sx, (const T*)dout, sd,  \
+                       dt, dA_cumsum, cb, ddA_cumsum, (int)nheads, hpg, (int)ngroups, (int)seqlen, (int)chunk,  \
+                       (int)d.C);                                                                               \
+  } while (0)
+    if (dtype == SSD_BF16) {
+      if (hdim == 64) SSD_DDA_LAUNCH(bf16_t, 64);
+      else SSD_DDA_LAUNCH(bf16_t, 128);
+    } else {
+      if (hdim == 64) SSD_DDA_LAUNCH(float, 64);
+      else SSD_DDA_LAUNCH(float, 128);
+    }
+#undef SSD_DDA_LAUNCH
+    return launched();
+  }
   float* part = static_cast<float*>(workspace);
   float* rowsum = part + ddAcs_part_floats(d);
   const int MT = (int)((d.Q + ema::kBM - 1) / ema::kBM);

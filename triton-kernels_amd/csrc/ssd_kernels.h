@@ -88,17 +88,17 @@ __device__ __forceinline__ void stage_rows(T* tile, const T* __restrict__ g, int
   for (int i = 0; i < ROWS * VPR / 256; ++i) {
     const int idx = tid + 256 * i;
     const int r = idx / VPR, cv = (idx % VPR) * EPL;
-    Vec16<T> v;
-    if (row0 + r < limit) {
-      v = load16(g + (int64_t)(row0 + r) * row_stride + cv);
-      if constexpr (!std::is_same<F, NoScale>::value) {
-        const float s = scale(row0 + r);
+    // The load is unconditional, from a row clamped into the sequence (limit >= 1): a load inside
+    // a branch would have to complete before the next one is issued.
+    const bool in = row0 + r < limit;
+    const int row = in ? row0 + r : limit - 1;
+    Vec16<T> v = load16(g + (int64_t)row * row_stride + cv);
+    if constexpr (!std::is_same<F, NoScale>::value) {
+      const float s = scale(row);
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) v.set(e, v.get(e) * s);
-      }
-    } else {
-      v.zero();
+      for (int e = 0; e < EPL; ++e) v.set(e, v.get(e) * s);
     }
+    if (!in) v.zero();
     store16(tile + r * P + cv, v);
   }
 }
@@ -425,7 +425,8 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int m = m0 + 32 * mi[i] + acc_row(v, lane);
-        bcv[i][v] = m < limit ? (float)bcg[(int64_t)m * sbc.sl + 32 * ni[i] + l32] : 0.f;
+        const float t = (float)bcg[(int64_t)min(m, limit - 1) * sbc.sl + 32 * ni[i] + l32];
+        bcv[i][v] = m < limit ? t : 0.f;
       }
   }
   floatx16 total[BPW];
@@ -459,9 +460,8 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
 #pragma unroll
       for (int i = 0; i < BPW; ++i) {
         const int m = m0 + 32 * mi[i] + l32;
-        Vec16<T> av;
-        if (m < limit) av = load16(ag + (int64_t)m * sa.sl + kk + EPL * half);
-        else av.zero();
+        Vec16<T> av = load16(ag + (int64_t)min(m, limit - 1) * sa.sl + kk + EPL * half);
+        if (m >= limit) av.zero();
         mma_group(av, frag_cols(St, S::PS, kk, 32 * ni[i], lane), acc[i]);
       }
     }
@@ -472,8 +472,9 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int m = m0 + 32 * mi[i] + acc_row(v, lane);
-        float w = 0.f;
-        if (m < Q) w = MODE == 0 ? __expf(fminf(dA_last - dAp[m], 0.f)) * dtp[m] : __expf(dAp[m]);
+        const int mc = min(m, Q - 1);  // loads stay unconditional; rows past the chunk get weight 0
+        float w = MODE == 0 ? __expf(fminf(dA_last - dAp[mc], 0.f)) * dtp[mc] : __expf(dAp[mc]);
+        w = m < Q ? w : 0.f;
         const float d = acc[i][v] * w;
         total[i][v] += d;
         r16[v] = d * (want_ddA ? bcv[i][v] : 0.f);
@@ -664,19 +665,18 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(
         const int r = idx >> 4, cv = (idx & 15) * 4;
         const int m = m0 + r;
         T* d = Ws + r * S::PW + cv;
-        if (m < Q && k0 + cv < Q) {  // Q is a multiple of 4 (checked on the host)
-          const float4 w4 = *reinterpret_cast<const float4*>(cbg + (int64_t)m * Q + k0 + cv);
-          const float4 a4 = *reinterpret_cast<const float4*>(dAp + k0 + cv);
-          const float4 t4 = *reinterpret_cast<const float4*>(dtp + k0 + cv);
-          const float am = dAp[m];
-          const float w[4] = {w4.x, w4.y, w4.z, w4.w}, ak[4] = {a4.x, a4.y, a4.z, a4.w},
-                      tk[4] = {t4.x, t4.y, t4.z, t4.w};
+        // unconditional loads from indices clamped into the chunk (Q is a multiple of 4)
+        const bool in = m < Q && k0 + cv < Q;
+        const int mc = min(m, Q - 1), kc = min(k0 + cv, Q - 4);
+        const float4 w4 = *reinterpret_cast<const float4*>(cbg + (int64_t)mc * Q + kc);
+        const float4 a4 = *reinterpret_cast<const float4*>(dAp + kc);
+        const float4 t4 = *reinterpret_cast<const float4*>(dtp + kc);
+        const float am = dAp[mc];
+        const float w[4] = {w4.x, w4.y, w4.z, w4.w}, ak[4] = {a4.x, a4.y, a4.z, a4.w},
+                    tk[4] = {t4.x, t4.y, t4.z, t4.w};
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            d[e] = (T)(k0 + cv + e <= m ? w[e] * __expf(fminf(am - ak[e], 0.f)) * tk[e] : 0.f);
-        } else {
-          d[0] = d[1] = d[2] = d[3] = (T)0.f;
-        }
+        for (int e = 0; e < 4; ++e)
+          d[e] = (T)((in && k0 + cv + e <= m) ? w[e] * __expf(fminf(am - ak[e], 0.f)) * tk[e] : 0.f);
       }
     }
     __syncthreads();
@@ -817,12 +817,11 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {
     const int m = m0 + mrow[mb] + l32;
-    const T* crow = Cg + (int64_t)m * sC.sl + EPL * half;
+    const T* crow = Cg + (int64_t)min(m, limit - 1) * sC.sl + EPL * half;
 #pragma unroll
     for (int kk = 0; kk < N; kk += KG) {
-      Vec16<T> a;
-      if (m < limit) a = load16(crow + kk);
-      else a.zero();
+      Vec16<T> a = load16(crow + kk);  // row clamped into the sequence, zeroed if past it
+      if (m >= limit) a.zero();
 #pragma unroll
       for (int pb = 0; pb < PB; ++pb) mma_group(a, frag_rows(Pv, S::PC, 32 * pb, kk, lane), acc[mb][pb]);
     }
@@ -1017,16 +1016,16 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
       const int r = idx >> 4, cv = (idx & 15) * 4;  // row k0 + r of cb, columns m0 + cv ..
       const int k = k0 + r;
       T* d = Wt + r * S::PW + cv;
-      if (k < limit && m0 + cv < Q) {
-        const float4 w4 = *reinterpret_cast<const float4*>(cbg + (int64_t)k * Q + m0 + cv);
-        const float4 a4 = *reinterpret_cast<const float4*>(dAp + m0 + cv);
-        const float ak = dAp[k];
-        const float w[4] = {w4.x, w4.y, w4.z, w4.w}, am[4] = {a4.x, a4.y, a4.z, a4.w};
+      // unconditional loads from indices clamped into the chunk
+      const bool in = k < limit && m0 + cv < Q;
+      const int kc = min(k, limit - 1), mc = min(m0 + cv, Q - 4);
+      const float4 w4 = *reinterpret_cast<const float4*>(cbg + (int64_t)kc * Q + mc);
+      const float4 a4 = *reinterpret_cast<const float4*>(dAp + mc);
+      const float ak = dAp[kc];
+      const float w[4] = {w4.x, w4.y, w4.z, w4.w}, am[4] = {a4.x, a4.y, a4.z, a4.w};
 #pragma unroll
-        for (int e = 0; e < 4; ++e) d[e] = (T)(k >= m0 + cv + e ? w[e] * __expf(fminf(ak - am[e], 0.f)) : 0.f);
-      } else {
-        d[0] = d[1] = d[2] = d[3] = (T)0.f;
-      }
+      for (int e = 0; e < 4; ++e)
+        d[e] = (T)((in && k >= m0 + cv + e) ? w[e] * __expf(fminf(ak - am[e], 0.f)) : 0.f);
     }
     __syncthreads();
 #pragma unroll
@@ -1078,6 +1077,137 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
 #pragma unroll
     for (int off = 1; off < VPR; off <<= 1) dot += __shfl_xor(dot, off);
     if ((idx % VPR) == 0 && m < Q) ddtp[m] = dot;
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// Gradient of the causal term of the chunk scan with respect to the per-position dA, for chunk
+// sizes of 64, 128 or 256.  One workgroup per (b, c, h).  With
+//   W[m][n] = <dout[m], x[n]> * dt_n * cb[m][n] * exp(min(dA_m - dA_n, 0))   for n < m < limit,
+// ddA[j] = sum_{i < j} (colsum_i - rowsum_i).  Wave w owns the 32-row blocks w and MB-1-w (which
+// balances the triangle) and walks their column blocks up to the diagonal: <dout, x> on the MFMA
+// (dout rows straight from global memory, the chunk's x rows shared through LDS), the weights in
+// the accumulator layout, row sums kept per lane, column sums combined through LDS.  The prefix
+// sum over the chunk closes the kernel, so nothing else is launched and no workspace is needed.
+// ------------------------------------------------------------------------------------
+template <typename T, int P>
+struct DdaSmem {
+  static constexpr int PX = Tile<T>::pitch(P);
+  static constexpr int kBytes = 256 * PX * (int)sizeof(T) + (4 * 256 + 256 + 256 + 256) * (int)sizeof(float);
+};
+
+template <typename T, int P>
+__global__ __launch_bounds__(256) void ssd_ddA_causal_kernel(
+    const T* __restrict__ x, Strides3 sx, const T* __restrict__ dout, Strides3 sd, const float* __restrict__ dt,
+    const float* __restrict__ dA_cs, const float* __restrict__ cb, float* __restrict__ ddA, int nh,
+    int heads_per_group, int ngroups, int L, int Q, int C) {
+  using S = DdaSmem<T, P>;
+  constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, KS = P / KG;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T* Xs = reinterpret_cast<T*>(smem);
+  float* colpart = reinterpret_cast<float*>(smem + 256 * S::PX * sizeof(T));  // [4 waves][256]
+  float* rowsum = colpart + 4 * 256;
+  float* dAs = rowsum + 256;
+  float* dts = dAs + 256;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
+  const int h = blockIdx.x % nh;
+  const int c = (blockIdx.x / nh) % C;
+  const int64_t b = blockIdx.x / ((int64_t)nh * C);
+  const int limit = min(Q, L - c * Q);
+  const int MB = Q / 32;
+  const int64_t chunk = (b * nh + h) * C + c;
+  const float* cbg = cb + (((b * C + c) * ngroups + h / heads_per_group) * (int64_t)Q) * Q;
+  const T* xg = x + b * sx.sb + (int64_t)c * Q * sx.sl + h * sx.sh;
+  const T* dg = dout + b * sd.sb + (int64_t)c * Q * sd.sl + h * sd.sh;
+
+  // shared: the chunk's x rows (zero past the limit), dA, dt; cleared: the sums
+  {
+    constexpr int VPR = P / EPL;
+    for (int idx = tid; idx < Q * VPR; idx += 256) {
+      const int r = idx / VPR, cv = (idx % VPR) * EPL;
+      Vec16<T> v = load16(xg + (int64_t)min(r, limit - 1) * sx.sl + cv);
+      if (r >= limit) v.zero();
+      store16(Xs + r * S::PX + cv, v);
+    }
+  }
+  if (tid < Q) {
+    dAs[tid] = dA_cs[chunk * Q + tid];
+    dts[tid] = dt[chunk * Q + tid];
+  }
+  rowsum[tid] = 0.f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) colpart[w * 256 + tid] = 0.f;
+  __syncthreads();
+
+#pragma unroll
+  for (int slot = 0; slot < 2; ++slot) {
+    const int mb = slot == 0 ? wave : MB - 1 - wave;
+    if (2 * wave >= MB) continue;  // fewer than 8 row blocks: the upper waves have none
+    const int m_lane = 32 * mb + l32;  // row whose dout this lane feeds into the MFMA
+    Vec16<T> a[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      a[ks] = load16(dg + (int64_t)min(m_lane, limit - 1) * sd.sl + KG * ks + EPL * half);
+      if (m_lane >= limit) a[ks].zero();
+    }
+    float rowacc[16], dAm[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      rowacc[v] = 0.f;
+      dAm[v] = dAs[32 * mb + acc_row(v, lane)];
+    }
+    for (int nb = 0; nb <= mb; ++nb) {
+      floatx16 acc;
+      zero_acc(acc);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) mma_group(a[ks], frag_rows(Xs, S::PX, 32 * nb, KG * ks, lane), acc);
+      const int n = 32 * nb + l32;
+      const float dAn = dAs[n], wn = dts[n];
+      float col = 0.f;
+      // every load is issued before the first use: none of them sits inside a branch
+      float cbv[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) cbv[v] = cbg[(int64_t)(32 * mb + acc_row(v, lane)) * Q + n];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = 32 * mb + acc_row(v, lane);
+        const float f = acc[v] * cbv[v] * wn * __expf(fminf(dAm[v] - dAn, 0.f));
+        const float w = (n < m && m < limit) ? f : 0.f;
+        rowacc[v] += w;
+        col += w;
+      }
+      col += __shfl_xor(col, 32);  // the two halves of the wave hold different rows of one column
+      if (half == 0) colpart[wave * 256 + n] += col;
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const float t = half_wave_sum(rowacc[v]);
+      if (l32 == 31) rowsum[32 * mb + acc_row(v, lane)] = t;
+    }
+  }
+  __syncthreads();
+  // delta_i = colsum_i - rowsum_i; ddA[j] = sum_{i<j} delta_i: wave 0, four positions per lane
+  if (wave == 0) {
+    const int per = (Q + 63) >> 6;
+    float d[4], local = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int q = lane * per + i;
+      d[i] = 0.f;
+      if (i < per && q < Q)
+        d[i] = colpart[q] + colpart[256 + q] + colpart[512 + q] + colpart[768 + q] - rowsum[q];
+      local += d[i];
+    }
+    float run = wave_inclusive_scan(local) - local;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int q = lane * per + i;
+      if (i < per && q < Q) {
+        ddA[chunk * Q + q] = run;
+        run += d[i];
+      }
+    }
   }
 }
 
