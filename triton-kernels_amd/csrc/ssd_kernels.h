@@ -385,7 +385,7 @@ __global__ __launch_bounds__(256) void ssd_row_cumsum_kernel(float* __restrict__
 template <typename T, int P, int N>
 struct GroupSmem {
   static constexpr int PS = Tile<T>::pitch(N);
-  static constexpr int kBytes = P * PS * (int)sizeof(T) + 4 * 64 * (int)sizeof(float);
+  static constexpr int kBytes = P * PS * (int)sizeof(T) + (4 * 64 + 64) * (int)sizeof(float);
 };
 
 template <typename T, int P, int N, int MODE>
@@ -398,6 +398,7 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* St = reinterpret_cast<T*>(smem);
   float* rs = reinterpret_cast<float*>(smem + P * S::PS * sizeof(T));  // [4 waves][64 rows]
+  float* wrow = rs + 4 * 64;                                           // this head's row weights
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
   const int mt = blockIdx.x % mtiles;
@@ -439,43 +440,50 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
     const float* dAp = dA_cs + chunk * Q;
     const float* dtp = dt + chunk * Q;
     const float* sg = s + (((b * C + c) * nh + h) * (int64_t)P) * N;
-    {
-      constexpr int VPR = N / 4;
+    const T* ag = a + b * sa.sb + (int64_t)c * Q * sa.sl + h * sa.sh;
+    // every global load of this head goes out here, before the first wait: the state tile, the
+    // wave's rows of a (its blocks share them), the row weights
+    constexpr int VPR = N / 4, NLD = P * VPR / 256, KS = P / KG;
+    float4 sv[NLD];
 #pragma unroll
-      for (int i = 0; i < P * VPR / 256; ++i) {
-        const int idx = tid + 256 * i;
-        const int r = idx / VPR, cv = (idx % VPR) * 4;
-        const float4 v = *reinterpret_cast<const float4*>(sg + (int64_t)r * N + cv);
-        T* d = St + r * S::PS + cv;
-        d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
-      }
+    for (int i = 0; i < NLD; ++i) {
+      const int idx = tid + 256 * i;
+      sv[i] = *reinterpret_cast<const float4*>(sg + (int64_t)(idx / VPR) * N + (idx % VPR) * 4);
+    }
+    const int m_lane = m0 + 32 * mi[0] + l32;
+    Vec16<T> av[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      av[ks] = load16(ag + (int64_t)min(m_lane, limit - 1) * sa.sl + KG * ks + EPL * half);
+    float wv = 0.f;
+    if (tid < 64) {  // one weight per row, computed once instead of by every lane that holds the row
+      const int mc = min(m0 + tid, Q - 1);
+      wv = MODE == 0 ? __expf(fminf(dAp[Q - 1] - dAp[mc], 0.f)) * dtp[mc] : __expf(dAp[mc]);
+      wrow[tid] = m0 + tid < Q ? wv : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const int idx = tid + 256 * i;
+      T* d = St + (idx / VPR) * S::PS + (idx % VPR) * 4;
+      d[0] = (T)sv[i].x, d[1] = (T)sv[i].y, d[2] = (T)sv[i].z, d[3] = (T)sv[i].w;
     }
     __syncthreads();
     floatx16 acc[BPW];
 #pragma unroll
     for (int i = 0; i < BPW; ++i) zero_acc(acc[i]);
-    const T* ag = a + b * sa.sb + (int64_t)c * Q * sa.sl + h * sa.sh;
 #pragma unroll
-    for (int kk = 0; kk < P; kk += KG) {
+    for (int ks = 0; ks < KS; ++ks) {
+      if (m_lane >= limit) av[ks].zero();
 #pragma unroll
-      for (int i = 0; i < BPW; ++i) {
-        const int m = m0 + 32 * mi[i] + l32;
-        Vec16<T> av = load16(ag + (int64_t)min(m, limit - 1) * sa.sl + kk + EPL * half);
-        if (m >= limit) av.zero();
-        mma_group(av, frag_cols(St, S::PS, kk, 32 * ni[i], lane), acc[i]);
-      }
+      for (int i = 0; i < BPW; ++i)
+        mma_group(av[ks], frag_cols(St, S::PS, KG * ks, 32 * ni[i], lane), acc[i]);
     }
-    const float dA_last = dAp[Q - 1];
 #pragma unroll
     for (int i = 0; i < BPW; ++i) {
       float r16[16];
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int m = m0 + 32 * mi[i] + acc_row(v, lane);
-        const int mc = min(m, Q - 1);  // loads stay unconditional; rows past the chunk get weight 0
-        float w = MODE == 0 ? __expf(fminf(dA_last - dAp[mc], 0.f)) * dtp[mc] : __expf(dAp[mc]);
-        w = m < Q ? w : 0.f;
-        const float d = acc[i][v] * w;
+        const float d = acc[i][v] * wrow[32 * mi[i] + acc_row(v, lane)];
         total[i][v] += d;
         r16[v] = d * (want_ddA ? bcv[i][v] : 0.f);
       }
