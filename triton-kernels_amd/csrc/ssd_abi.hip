@@ -140,6 +140,17 @@ struct DxLaunch {
   hipStream_t st;
   template <typename T, int P, int N>
   int run() const {
+    constexpr int wide_smem = WideSmem<T, P, N>::kBytes;
+    if (d.Q % 256 == 0 && wide_smem <= kLdsBytes) {
+      auto kernel = ssd_chunk_scan_bwd_dx_wide_kernel<T, P, N>;
+      SSD_TRY(allow_smem(kernel, wide_smem));
+      const int stiles = (int)(d.Q / 256);
+      hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh * stiles)), dim3(256), wide_smem, st, cb,
+                         (const T*)x, sx, (const T*)dout, sd, dt, dA, (const T*)B, sB, dstates, D, d_has_hdim,
+                         (T*)dx, sdx, ddt, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C,
+                         stiles);
+      return launched();
+    }
     auto kernel = ssd_chunk_scan_bwd_dx_kernel<T, P, N>;
     constexpr int smem = ScanSmem<T, P, N>::kBytes;
     SSD_TRY(allow_smem(kernel, smem));

@@ -1219,4 +1219,166 @@ __global__ __launch_bounds__(256) void ssd_ddA_causal_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------
+// dx / ddt for chunk sizes that are multiples of 256: the mirror image of
+// ssd_chunk_scan_wide_kernel.  One workgroup per (b, c, h, 256-row super-tile); wave w owns the
+// 32-row blocks w and 7 - w.  The k super-tiles run from the diagonal one to the end of the
+// chunk; the weight fragment of a lane (row m, consecutive k) is a column piece of cb, read as
+// one 4-byte load per k that is contiguous across the 32 lanes of a half-wave.
+// ------------------------------------------------------------------------------------
+template <typename T, int P, int N>
+__global__ __launch_bounds__(256, 2) void ssd_chunk_scan_bwd_dx_wide_kernel(
+    const float* __restrict__ cb, const T* __restrict__ x, Strides3 sx, const T* __restrict__ dout, Strides3 sd,
+    const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Bm, Strides3 sB,
+    const float* __restrict__ dstates, const float* __restrict__ D, int d_has_hdim, T* __restrict__ dx,
+    Strides3 sdx, float* __restrict__ ddt, int nh, int heads_per_group, int ngroups, int L, int Q, int C,
+    int stiles) {
+  using S = WideSmem<T, P, N>;
+  constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, PB = P / 32, ST = S::ST;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T* Ds = reinterpret_cast<T*>(smem);
+  T* Pv = reinterpret_cast<T*>(smem + S::kX);
+  float* Os = reinterpret_cast<float*>(smem);
+  float* dAk = reinterpret_cast<float*>(smem + S::kMain);
+  float* sm = dAk + 2 * ST;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
+  const int st = blockIdx.x % stiles;
+  const int h = (blockIdx.x / stiles) % nh;
+  const int c = (blockIdx.x / (stiles * nh)) % C;
+  const int64_t b = blockIdx.x / ((int64_t)stiles * nh * C);
+  const int limit = min(Q, L - c * Q);
+  const int m0 = ST * st;
+  const int64_t chunk = (b * nh + h) * C + c;
+  float* ddtp = ddt + chunk * Q;
+  if (m0 >= limit) {
+    ddtp[m0 + tid] = 0.f;
+    return;
+  }
+  const int g = h / heads_per_group;
+  const float* dAp = dA_cs + chunk * Q;
+  const float* dtp = dt + chunk * Q;
+  const T* dg = dout + b * sd.sb + (int64_t)c * Q * sd.sl + h * sd.sh;
+  const T* Bg = Bm + b * sB.sb + (int64_t)c * Q * sB.sl + g * sB.sh;
+  const float* sg = dstates + (((b * C + c) * nh + h) * (int64_t)P) * N;
+  const float* cbg = cb + (((b * C + c) * ngroups + g) * (int64_t)Q) * Q;
+
+  int mrow[2];
+  mrow[0] = 32 * wave;
+  mrow[1] = 32 * (7 - wave);
+  floatx16 acc[2][PB];
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+    for (int pb = 0; pb < PB; ++pb) zero_acc(acc[mb][pb]);
+
+  // ---- phase A: B . dstates, scaled by the decay to the end of the chunk
+  {
+    constexpr int VPR = N / 4;
+#pragma unroll
+    for (int i = 0; i < P * VPR / 256; ++i) {
+      const int idx = tid + 256 * i;
+      const int r = idx / VPR, cv = (idx % VPR) * 4;
+      const float4 v = *reinterpret_cast<const float4*>(sg + (int64_t)r * N + cv);
+      T* d = Pv + r * S::PC + cv;
+      d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
+    }
+  }
+  sm[tid] = __expf(fminf(dAp[Q - 1] - dAp[m0 + tid], 0.f));
+  __syncthreads();
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb) {
+    const int m = m0 + mrow[mb] + l32;
+    const T* brow = Bg + (int64_t)min(m, limit - 1) * sB.sl + EPL * half;
+#pragma unroll
+    for (int kk = 0; kk < N; kk += KG) {
+      Vec16<T> a = load16(brow + kk);
+      if (m >= limit) a.zero();
+#pragma unroll
+      for (int pb = 0; pb < PB; ++pb) mma_group(a, frag_rows(Pv, S::PC, 32 * pb, kk, lane), acc[mb][pb]);
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const float sc = sm[mrow[mb] + acc_row(v, lane)];
+#pragma unroll
+      for (int pb = 0; pb < PB; ++pb) acc[mb][pb][v] *= sc;
+    }
+  }
+
+  // ---- phase B: the k super-tiles from the diagonal one to the end of the chunk
+  for (int kt = st; kt < stiles && ST * kt < limit; ++kt) {
+    const int k0 = ST * kt;
+    stage_rows<T, ST, P>(Ds, dg, sd.sl, k0, limit, tid, NoScale());
+    dAk[tid] = dAp[k0 + tid];
+    __syncthreads();
+    const bool diag = kt == st;
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) {
+      const int mloc = mrow[mb] + l32;
+      const float am = dAp[m0 + mloc];
+      const float* cbcol = cbg + (int64_t)k0 * Q + m0 + mloc;  // cb[k0 + k][m]: stride Q along k
+      for (int kk = diag ? mrow[mb] : 0; kk < ST; kk += KG) {
+        const int kb = kk + EPL * half;
+        float w[EPL];
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) w[e] = cbcol[(int64_t)(kb + e) * Q];
+        Vec16<T> a;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+          const int k = kb + e;
+          const float f = w[e] * __expf(fminf(dAk[k] - am, 0.f));
+          a.set(e, ((diag && k < mloc) || k0 + k >= limit) ? 0.f : f);
+        }
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) mma_group(a, frag_cols(Ds, S::PX, kk, 32 * pb, lane), acc[mb][pb]);
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- phase C: each wave moves its two blocks through its own staging area
+  float* mine = Os + wave * 32 * S::PO;
+  constexpr int VPR = P / EPL;
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb) {
+#pragma unroll
+    for (int pb = 0; pb < PB; ++pb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) mine[acc_row(v, lane) * S::PO + 32 * pb + l32] = acc[mb][pb][v];
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+#pragma unroll
+    for (int i = 0; i < 32 * VPR / 64; ++i) {
+      const int idx = lane + 64 * i;
+      const int r = idx / VPR, cv = (idx % VPR) * EPL;
+      const int m = m0 + mrow[mb] + r;
+      const int64_t pos = (int64_t)c * Q + min(m, limit - 1);
+      const Vec16<T> xv = load16(x + b * sx.sb + pos * sx.sl + h * sx.sh + cv);
+      const float dtm = dtp[m];
+      float dot = 0.f, v[EPL];
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) {
+        v[e] = mine[r * S::PO + cv + e];
+        dot = fmaf(v[e], xv.get(e), dot);
+        v[e] *= dtm;
+      }
+      if (m >= limit) dot = 0.f;
+      if (D) {
+        const Vec16<T> dv = load16(dout + b * sd.sb + pos * sd.sl + h * sd.sh + cv);
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) v[e] = fmaf(d_has_hdim ? D[h * P + cv + e] : D[h], dv.get(e), v[e]);
+      }
+      if (m < limit) {
+        Vec16<T> o;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) o.set(e, v[e]);
+        store16(dx + b * sdx.sb + pos * sdx.sl + h * sdx.sh + cv, o);
+      }
+#pragma unroll
+      for (int off = 1; off < VPR; off <<= 1) dot += __shfl_xor(dot, off);
+      if ((idx % VPR) == 0) ddtp[m] = dot;
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+  }
+}
+
 }  // namespace ssd
