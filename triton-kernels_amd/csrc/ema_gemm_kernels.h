@@ -84,16 +84,17 @@ __global__ __launch_bounds__(256) void da_gemm_kernel(const T* __restrict__ x, S
       {
         const int vcol = (tid % VPR) * EPL;
         const bool cok = d0 + vcol < Tdim;
+#pragma unroll
         for (int r = tid / VPR; r < kBM; r += RPP) {
-          Vec16<T> v;
-          const int m = mt_base + r;
-          if (m < limit && cok) v = load16(dp + (int64_t)m * sd.sl + d0 + vcol);
-          else v.zero();
-          store16(&dys[r * ROW + vcol], v);
-          const int k = kt_base + r;
-          if (k < limit && cok) v = load16(xp + (int64_t)k * sx.sl + d0 + vcol);
-          else v.zero();
-          store16(&xs[r * ROW + vcol], v);
+          // unconditional loads from indices clamped into the tensor, zeroed afterwards
+          const int m = mt_base + r, k = kt_base + r;
+          const int dcol = cok ? d0 + vcol : 0;
+          Vec16<T> vd = load16(dp + (int64_t)min(m, limit - 1) * sd.sl + dcol);
+          Vec16<T> vx = load16(xp + (int64_t)min(k, limit - 1) * sx.sl + dcol);
+          if (m >= limit || !cok) vd.zero();
+          if (k >= limit || !cok) vx.zero();
+          store16(&dys[r * ROW + vcol], vd);
+          store16(&xs[r * ROW + vcol], vx);
         }
       }
       __syncthreads();

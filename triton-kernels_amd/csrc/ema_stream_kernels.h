@@ -84,20 +84,21 @@ __global__ __launch_bounds__(256) void chunk_reduce_kernel(
   for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
 
   constexpr int U = 4;
+  const T* xq = col_ok ? xp : xp - col;  // a column tile past the end reads column 0 and is discarded
   for (int q0 = row_lane; q0 < limit; q0 += rows_par * U) {
     Vec16<T> v[U];
     float w[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
+      // unconditional loads from an index clamped into the chunk (a load inside a branch has to
+      // complete before the next one is issued); what lies outside gets weight 0
       const int q = q0 + u * rows_par;
-      if (q < limit && col_ok) {
-        v[u] = load16(xp + (int64_t)q * sx.sl);
-        const float a = csp[q];
-        w[u] = MODE == 0 ? __expf(fminf(cs_last - a, 0.f)) : __expf(a);
-      } else {
-        v[u].zero();
-        w[u] = 0.f;
-      }
+      const int qc = min(q, limit - 1);
+      v[u] = load16(xq + (int64_t)qc * sx.sl);
+      const float a = csp[qc];
+      const float wt = MODE == 0 ? __expf(fminf(cs_last - a, 0.f)) : __expf(a);
+      w[u] = (q < limit && col_ok) ? wt : 0.f;
+      if (!(q < limit && col_ok)) v[u].zero();
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -257,8 +258,8 @@ __global__ __launch_bounds__(256) void row_dot_kernel(const T* __restrict__ x, S
       Vec16<T> v[R];
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        if (m0 + r < limit) v[r] = load16(xp + (int64_t)(m0 + r) * sx.sl + col);
-        else v[r].zero();
+        v[r] = load16(xp + (int64_t)min(m0 + r, limit - 1) * sx.sl + col);
+        if (m0 + r >= limit) v[r].zero();
       }
 #pragma unroll
       for (int r = 0; r < R; ++r)

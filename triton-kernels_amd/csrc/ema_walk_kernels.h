@@ -75,8 +75,9 @@ __device__ __forceinline__ void walk_load_tile(T* tile, const T* __restrict__ g,
 #pragma unroll
   for (int p = 0; p < kTileRows / C::RPP; ++p) {
     const int r = tid / C::VPR + p * C::RPP;
-    if (tb + r < limit && cok) v[p] = load16(g + (int64_t)(tb + r) * sl + col0 + vcol);
-    else v[p].zero();
+    // unconditional load from a row and column clamped into the tensor, zeroed afterwards
+    v[p] = load16(g + (int64_t)min(tb + r, limit - 1) * sl + (cok ? col0 + vcol : 0));
+    if (tb + r >= limit || !cok) v[p].zero();
   }
 #pragma unroll
   for (int p = 0; p < kTileRows / C::RPP; ++p) {
