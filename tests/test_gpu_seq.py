@@ -150,3 +150,36 @@ def test_seq_bench_shape_properties(device):
     check_close("split scan, first part", y1, y_p[:, :h].float(), BF16)
     check_close("split scan, second part", y2, y_p[:, h:].float(), BF16)
     check_close("split scan, final", f2, fin_p, BF16)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+def test_seq_packed_sequences(dtype, device):
+    """seq_idx: sequences packed along the length axis scan as if each were alone, forward and
+    backward; boundaries fall inside tiles, on tile edges and inside 8-row groups."""
+    from kernels.ema_seq import ema_seq_scan
+
+    B, L, T = 2, 1000, 72
+    announce(f"seq packed sequences {dtype}")
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn(B, L, T, generator=g).to(dtype)
+    A = torch.nn.functional.logsigmoid(torch.randn(B, L, generator=g) + 2.0)
+    dy = torch.randn(B, L, T, generator=g).to(dtype)
+    cuts = [[0, 3, 128, 131, 640, 1000], [0, 255, 256, 257, 900, 1000]]
+    seq_idx = torch.zeros(B, L, dtype=torch.int32)
+    for bi, cs in enumerate(cuts):
+        for k in range(len(cs) - 1):
+            seq_idx[bi, cs[k]:cs[k + 1]] = k
+    xg, Ag = x.to(device).requires_grad_(), A.to(device).requires_grad_()
+    y = ema_seq_scan(Ag, xg, "log_decay", seq_idx=seq_idx.to(device))
+    y.backward(dy.to(device))
+    torch.cuda.synchronize()
+    y_ref, dx_ref, dA_ref = torch.zeros(B, L, T), torch.zeros(B, L, T), torch.zeros(B, L)
+    for bi, cs in enumerate(cuts):
+        for k in range(len(cs) - 1):
+            sl = slice(cs[k], cs[k + 1])
+            y_ref[bi, sl] = O.ema_loop(x[bi:bi + 1, sl].float(), A[bi:bi + 1, sl])[0]
+            dxs, dAs = O.ema_loop_bwd(dy[bi:bi + 1, sl].float(), x[bi:bi + 1, sl].float(), A[bi:bi + 1, sl])
+            dx_ref[bi, sl], dA_ref[bi, sl] = dxs[0], dAs[0]
+    check_close("y", y, y_ref, dtype)
+    check_close("dx", xg.grad, dx_ref, dtype)
+    check_close("dA", Ag.grad, dA_ref, dtype)

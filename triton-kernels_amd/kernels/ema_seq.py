@@ -115,7 +115,27 @@ class EMASeqFn(torch.autograd.Function):
         return dcoef, dx, dinit, None
 
 
-def ema_seq_scan(coef, x, form="log_decay", initial_states=None, return_final_states=False):
-    """Differentiable in coef, x and initial_states (and through the final states)."""
+def pack_log_decay(A, seq_idx):
+    """Log-decay of several sequences packed along the length axis: wherever seq_idx (batch, L)
+    changes, the state must not carry over, which is a decay of exp(-inf) = 0 at the first
+    position of the new sequence (what the reference's seq_idx arguments ask of its kernels, e.g.
+    kernels/ema_chunk_state.py:500-604: scale = where(seq_idx_k == seq_idx_last, exp(...), 0)).
+    A is (B, L) or (b, L, nh); returns a tensor of A's shape.  The gradient that reaches the
+    masked positions is zero."""
+    assert seq_idx.shape == A.shape[:2], "seq_idx must be (batch, seqlen)"
+    start = torch.zeros_like(seq_idx, dtype=torch.bool)
+    start[:, 1:] = seq_idx[:, 1:] != seq_idx[:, :-1]
+    if A.dim() == 3:
+        start = start[..., None]
+    return torch.where(start, torch.full_like(A, float("-inf")), A)
+
+
+def ema_seq_scan(coef, x, form="log_decay", initial_states=None, return_final_states=False, seq_idx=None):
+    """Differentiable in coef, x and initial_states (and through the final states).  seq_idx
+    (batch, L) marks packed sequences (log-decay form only): the state is reset where it changes."""
+    if seq_idx is not None:
+        if form != "log_decay":
+            raise NotImplementedError("seq_idx needs the log-decay form (a reset is a decay of 0)")
+        coef = pack_log_decay(coef, seq_idx)
     y, final = EMASeqFn.apply(coef, x, initial_states, form)
     return (y, final) if return_final_states else y
