@@ -761,7 +761,10 @@ struct WideSmem {
   static constexpr int kX = ST * PX * (int)sizeof(T);
   static constexpr int kPrev = P * PC * (int)sizeof(T);
   static constexpr int kOut = 4 * 32 * PO * (int)sizeof(float);                  // one 32-row block per wave
-  static constexpr int kMain = (kX + kPrev) > kOut ? (kX + kPrev) : kOut;
+  // the carried state is only read before the k loop, the x tile only inside it, the output
+  // staging only after it: the three share one region
+  static constexpr int kXP = kX > kPrev ? kX : kPrev;
+  static constexpr int kMain = kXP > kOut ? kXP : kOut;
   static constexpr int kBytes = kMain + 3 * ST * (int)sizeof(float);            // + dA_k, dt_k, exp(dA_m)
 };
 
@@ -776,7 +779,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
   constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, PB = P / 32, ST = S::ST;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* Xs = reinterpret_cast<T*>(smem);
-  T* Pv = reinterpret_cast<T*>(smem + S::kX);
+  T* Pv = reinterpret_cast<T*>(smem);
   float* Os = reinterpret_cast<float*>(smem);
   float* dAk = reinterpret_cast<float*>(smem + S::kMain);
   float* dtk = dAk + ST;
@@ -842,6 +845,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
   }
 
   // ---- phase B: the k super-tiles up to the diagonal one
+  __syncthreads();  // the x tile takes the place of the carried state
   for (int kt = 0; kt <= st; ++kt) {
     const int k0 = ST * kt;
     stage_rows<T, ST, P>(Xs, xg, sx.sl, k0, limit, tid, NoScale());
@@ -1227,7 +1231,7 @@ __global__ __launch_bounds__(256) void ssd_ddA_causal_kernel(
 // one 4-byte load per k that is contiguous across the 32 lanes of a half-wave.
 // ------------------------------------------------------------------------------------
 template <typename T, int P, int N>
-__global__ __launch_bounds__(256, 2) void ssd_chunk_scan_bwd_dx_wide_kernel(
+__global__ __launch_bounds__(256, 3) void ssd_chunk_scan_bwd_dx_wide_kernel(
     const float* __restrict__ cb, const T* __restrict__ x, Strides3 sx, const T* __restrict__ dout, Strides3 sd,
     const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Bm, Strides3 sB,
     const float* __restrict__ dstates, const float* __restrict__ D, int d_has_hdim, T* __restrict__ dx,
@@ -1237,7 +1241,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_bwd_dx_wide_kernel(
   constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, PB = P / 32, ST = S::ST;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* Ds = reinterpret_cast<T*>(smem);
-  T* Pv = reinterpret_cast<T*>(smem + S::kX);
+  T* Pv = reinterpret_cast<T*>(smem);
   float* Os = reinterpret_cast<float*>(smem);
   float* dAk = reinterpret_cast<float*>(smem + S::kMain);
   float* sm = dAk + 2 * ST;
@@ -1306,6 +1310,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_bwd_dx_wide_kernel(
   }
 
   // ---- phase B: the k super-tiles from the diagonal one to the end of the chunk
+  __syncthreads();  // the dout tile takes the place of dstates
   for (int kt = st; kt < stiles && ST * kt < limit; ++kt) {
     const int k0 = ST * kt;
     stage_rows<T, ST, P>(Ds, dg, sd.sl, k0, limit, tid, NoScale());
