@@ -17,6 +17,10 @@
  *     states (batch, C, nheads, hdim, dstate), cb (batch, C, ngroups, Q, Q); C = ceil(seqlen/Q).
  *   - `dtype` (ssd_dtype, same codes as ema_dtype) is the element type of x, z, B, C and out;
  *     accumulation is float32.
+ *   - seq_idx (may be NULL) marks a packed batch: int32 ids (batch, seqlen) addressed as
+ *     seq_idx[b*seq_sb + l*seq_sl]; positions with different ids belong to different sequences
+ *     and do not see each other's state.  Ids are expected to be non-negative and not to
+ *     decrease along a row; the carried state of a row starts with id 0.
  *   - Supported shapes: hdim in {64, 128}, dstate in {64, 128}, nheads a multiple of ngroups,
  *     chunk a multiple of 4 up to 1024; anything else returns SSD_ERR_UNSUPPORTED.
  *   - Return value: 0 or a negative ssd_status (same values as ema_status).
@@ -54,36 +58,45 @@ int ssd_chunk_cumsum_fwd(const void* dt, int dt_dtype, int64_t dt_sb, int64_t dt
 
 /* states[b,c,h,p,n] = sum_k x[k,p] * B[k,n] * exp(min(dA_last - dA_k, 0)) * dt_k over the
  * positions k of chunk c (the weighted B is rounded to `dtype` before the product, as the
- * reference does).  Replaces _chunk_state_fwd, kernels/mamba_kernels/mamba_state_fwd.py:138-169
- * (seq_idx is not supported). */
+ * reference does).  With seq_idx, position k only counts if its id equals the id of the chunk's
+ * last position, and none counts if that id is negative (mamba_state_fwd.py:113).
+ * Replaces _chunk_state_fwd, kernels/mamba_kernels/mamba_state_fwd.py:138-169. */
 int ssd_chunk_state_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64_t b_sg, const void* x,
                         int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, const float* dt,
                         const float* dA_cumsum, float* states, int64_t batch, int64_t seqlen,
                         int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
-                        void* stream);
+                        const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream);
 
 /* out[b,c] = state entering chunk c; state <- exp(dA_chunk[b,h,c]) * state + states[b,c];
  * final = the state after the last chunk.  states / out (batch, C, nheads, dim) float32,
  * dA_chunk addressed by (batch, head, chunk) strides (it is dA_cumsum[..., -1]); initial
- * (batch, nheads, dim) float32 may be NULL.  dim must be a multiple of 4.
+ * (batch, nheads, dim) float32 may be NULL.  dim must be a multiple of 4.  With seq_idx the
+ * state is dropped across a chunk whose last position has another id than the previous chunk's
+ * last position (id 0 before the first chunk; mamba_state_pass.py:68-71); seqlen and chunk
+ * locate those positions and are ignored without seq_idx.
  * Replaces _state_passing_fwd, kernels/mamba_kernels/mamba_state_pass.py:84-115. */
 int ssd_state_passing_fwd(const float* states, const float* dA_chunk, int64_t da_sb, int64_t da_sh,
                           int64_t da_sc, const float* initial, float* out, float* final_states,
-                          int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, void* stream);
+                          int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, const int32_t* seq_idx,
+                          int64_t seq_sb, int64_t seq_sl, int64_t seqlen, int64_t chunk, void* stream);
 
 /* out[b,c,g,m,k] = sum_n a[b,cQ+m,g,n] * bm[b,cQ+k,g,n]; rows past seqlen are zero.  out is
- * float32 or `dtype` (out_dtype).  Replaces _bmm_chunk_fwd, kernels/mamba_kernels/mamba_bmm.py:88-126
+ * float32 or `dtype` (out_dtype).  With seq_idx, out[m,k] = 0 where the ids of m and k differ
+ * (mamba_bmm.py:70-73).  Replaces _bmm_chunk_fwd, kernels/mamba_kernels/mamba_bmm.py:88-126
  * (the whole Q x Q block is written, also with causal = True). */
 int ssd_bmm_chunk_fwd(const void* a, int64_t a_sb, int64_t a_sl, int64_t a_sg, const void* bm,
                       int64_t b_sb, int64_t b_sl, int64_t b_sg, int dtype, void* out, int out_dtype,
                       int64_t batch, int64_t seqlen, int64_t ngroups, int64_t k, int64_t chunk,
-                      void* stream);
+                      const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream);
 
 /* out[m,p] = exp(dA_m) * sum_n C[m,n] * prev[p,n]
  *          + sum_{k<=m} cb[m,k] * exp(min(dA_m - dA_k, 0)) * dt_k * x[k,p]  +  D * x[m,p],
  * then, with z: out_x = out (if out_x is not NULL) and out *= z * sigmoid(z).
  * cb float32 (batch, C, ngroups, Q, Q); prev float32 (batch, C, nheads, hdim, dstate); D float32
  * (nheads) or (nheads, hdim) (d_has_hdim), may be NULL; z may be NULL; out_x shares out's strides.
+ * With seq_idx the first term only reaches the rows m whose id equals that of the previous
+ * chunk's last position (0 for the first chunk; mamba_scan_fwd.py:77-92); cb is expected to
+ * hold zeros between positions of different ids, as ssd_bmm_chunk_fwd leaves it.
  * Replaces _chunk_scan_fwd, kernels/mamba_kernels/mamba_scan_fwd.py:162-210. */
 int ssd_chunk_scan_fwd(const float* cb, const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
                        const void* z, int64_t z_sb, int64_t z_sl, int64_t z_sh, int dtype,
@@ -91,17 +104,20 @@ int ssd_chunk_scan_fwd(const float* cb, const void* x, int64_t x_sb, int64_t x_s
                        int64_t c_sg, const float* prev_states, const float* D, int d_has_hdim, void* out,
                        int64_t o_sb, int64_t o_sl, int64_t o_sh, void* out_x, int64_t batch,
                        int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate,
-                       int64_t chunk, void* stream);
+                       int64_t chunk, const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream);
 
 /* ---------------------------------------------------------------- backward stages ---- */
 
 /* dprev_states[b,c,h,p,n] = sum_m round(dout[m,p] * exp(dA_m)) * C[m,n] (float32): the gradient of
- * the chunk scan with respect to the carried states.  Replaces _chunk_scan_bwd_dstates,
+ * the chunk scan with respect to the carried states.  With seq_idx only the rows m whose id
+ * equals that of the previous chunk's last position count (mamba_scan_bwd.py:63-71).
+ * Replaces _chunk_scan_bwd_dstates,
  * kernels/mamba_kernels_bwd/mamba_scan_bwd.py:91-116. */
 int ssd_chunk_scan_bwd_dstates(const void* C, int64_t c_sb, int64_t c_sl, int64_t c_sg, const void* dout,
                                int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype, const float* dA_cumsum,
                                float* dprev_states, int64_t batch, int64_t seqlen, int64_t nheads,
-                               int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk, void* stream);
+                               int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
+                               const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream);
 
 /* Bytes of workspace ssd_state_passing_bwd needs (per-wave partial dot products). */
 size_t ssd_state_passing_bwd_workspace_bytes(int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim);
@@ -111,42 +127,51 @@ size_t ssd_state_passing_bwd_workspace_bytes(int64_t batch, int64_t nchunks, int
  * the gradient of the final state.  With G the gradient of the state entering the next chunk:
  * dstates[c] = G (the gradient of the chunk-local state), ddA_chunk[b,h,c] = exp(dA_chunk[c]) *
  * <states[c], G> (0 for c = 0 unless dinit is given), G <- exp(dA_chunk[c]) * G + dout[c];
- * dinit (batch, nheads, dim), may be NULL, receives the last G.  All float32.
+ * dinit (batch, nheads, dim), may be NULL, receives the last G.  All float32.  With seq_idx the
+ * factor exp(dA_chunk[c]) is 0 for the chunks across which ssd_state_passing_fwd drops the state
+ * (mamba_state_passing_bwd_dstates.py:72-80,105); seqlen and chunk as there.
  * Replaces _state_passing_bwd, kernels/mamba_kernels_bwd/mamba_state_passing_bwd_dstates.py:116-172. */
 int ssd_state_passing_bwd(const float* states, const float* dA_chunk, int64_t da_sb, int64_t da_sh,
                           int64_t da_sc, const float* dout, const float* dfinal, float* dstates,
                           float* ddA_chunk, float* dinit, void* workspace, size_t workspace_bytes,
-                          int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, void* stream);
+                          int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, const int32_t* seq_idx,
+                          int64_t seq_sb, int64_t seq_sl, int64_t seqlen, int64_t chunk, void* stream);
 
 /* dB[b,l,g,n] = sum over the heads h of group g of (sum_p x[m,p] * round(dstates[b,c,h,p,n])) *
  * exp(min(dA_last - dA_m, 0)) * dt_m (float32, dense (batch, seqlen, ngroups, dstate)).  With B
  * (may be NULL, then ddA_cumsum is not written): r_h[m] = sum_n db_h[m,n] * B[m,n] and
  * ddA_cumsum[b,h,c,j] = sum_{m<j} r_h[m], the gradient of the chunk states with respect to the
- * per-position dA.  Replaces _chunk_state_bwd_db,
+ * per-position dA.  With seq_idx the weight of row m is 0 unless its id equals that of the
+ * chunk's last position (mamba_chunk_state_bwd_db.py:88-104).  Replaces _chunk_state_bwd_db,
  * kernels/mamba_kernels_bwd/mamba_chunk_state_bwd_db.py:131-181 (one pass over all heads of a
  * group, so there is no split axis to sum afterwards). */
 int ssd_chunk_state_bwd_db(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype,
                            const float* dt, const float* dA_cumsum, const float* dstates, const void* B,
                            int64_t b_sb, int64_t b_sl, int64_t b_sg, float* dB, float* ddA_cumsum,
                            int64_t batch, int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim,
-                           int64_t dstate, int64_t chunk, void* stream);
+                           int64_t dstate, int64_t chunk, const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl,
+                           void* stream);
 
 /* dC[b,l,g,n] = sum over the heads of group g of (sum_p dout[m,p] * round(prev[b,c,h,p,n])) *
  * exp(dA_m): the part of dC that comes through the carried state.  With C (may be NULL):
- * ddA_cumsum_prev[b,h,c,m] = sum_n dc_h[m,n] * C[m,n].  Replaces _chunk_scan_bwd_dC,
+ * ddA_cumsum_prev[b,h,c,m] = sum_n dc_h[m,n] * C[m,n].  With seq_idx the weight of row m is 0
+ * unless its id equals that of the previous chunk's last position
+ * (mamba_chunk_scan_bwd_dc.py:84-96).  Replaces _chunk_scan_bwd_dC,
  * kernels/mamba_kernels_bwd/mamba_chunk_scan_bwd_dc.py:118-160. */
 int ssd_chunk_scan_bwd_dc(const void* dout, int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype,
                           const float* dA_cumsum, const float* prev_states, const void* C, int64_t c_sb,
                           int64_t c_sl, int64_t c_sg, float* dC, float* ddA_cumsum_prev, int64_t batch,
                           int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate,
-                          int64_t chunk, void* stream);
+                          int64_t chunk, const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream);
 
 /* acc[m,p] = exp(min(dA_last - dA_m, 0)) * sum_n B[m,n] * round(dstates[p,n])
  *          + sum_{k>=m} round(cb[k,m] * exp(min(dA_k - dA_m, 0))) * dout[k,p];
  * dx = acc * dt_m + D * dout (type `dtype`, dx's own strides), ddt[b,h,c,m] = sum_p acc[m,p] * x[m,p]
  * (float32, 0 past seqlen).  cb float32 (batch, C, ngroups, Q, Q), dstates float32
  * (batch, C, nheads, hdim, dstate), D as for ssd_chunk_scan_fwd (its gradient, sum dout * x, is
- * left to the caller).  Replaces _chunk_scan_chunk_state_bwd_dx,
+ * left to the caller).  With seq_idx the first term only reaches the rows m whose id equals that
+ * of the chunk's last position (mamba_chunk_scan_chunk_state_bwd_dx.py:93-96).
+ * Replaces _chunk_scan_chunk_state_bwd_dx,
  * kernels/mamba_kernels_bwd/mamba_chunk_scan_chunk_state_bwd_dx.py:189-248. */
 int ssd_chunk_scan_chunk_state_bwd_dx(const float* cb, const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
                                       const void* dout, int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype,
@@ -155,7 +180,7 @@ int ssd_chunk_scan_chunk_state_bwd_dx(const float* cb, const void* x, int64_t x_
                                       int d_has_hdim, void* dx, int64_t dx_sb, int64_t dx_sl, int64_t dx_sh,
                                       float* ddt, int64_t batch, int64_t seqlen, int64_t nheads,
                                       int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
-                                      void* stream);
+                                      const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream);
 
 /* Bytes of workspace ssd_chunk_scan_bwd_ddAcs needs (column sums per row tile, row sums). */
 size_t ssd_chunk_scan_bwd_ddAcs_workspace_bytes(int64_t batch, int64_t seqlen, int64_t nheads, int64_t chunk);
@@ -164,7 +189,8 @@ size_t ssd_chunk_scan_bwd_ddAcs_workspace_bytes(int64_t batch, int64_t seqlen, i
  * ddA_cumsum[b,h,c,j] = sum_{m>=j} sum_{n<j} W[m,n] (float32; 0 for j = 0): the gradient of the causal
  * term of the chunk scan with respect to the per-position dA.  It is formed as the prefix sum of
  * (column sum - row sum) of W, which is the same quantity as the reference's row-wise cumsum
- * followed by column sums.  Replaces _chunk_scan_bwd_ddAcs_stable,
+ * followed by column sums.  A packed batch needs nothing here: cb already holds zeros between
+ * positions of different ids (mamba_chunk_scan_bwd_da.py:86).  Replaces _chunk_scan_bwd_ddAcs_stable,
  * kernels/mamba_kernels_bwd/mamba_chunk_scan_bwd_da.py:111-140 (and its torch sum over row blocks). */
 int ssd_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, const void* dout,
                              int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype, const float* dt,

@@ -81,15 +81,18 @@ def test_ssd_validation_happens_before_any_launch():
     fake = 0x1000
     seq = [fake, 64 * 2 * 64, 2 * 64, 64]
     grp = [fake, 64 * 64, 64, 64]
+    ids = [None, 0, 0]  # not a packed batch
     # null pointer, bad shape, unsupported head size, misaligned strides, unknown dtype
     assert handle.ssd_chunk_cumsum_fwd(None, 0, 2, 2, 1, fake, None, fake, fake, 1, 64, 2, 64, 0, 0.0, 1.0, None) == -1
     assert handle.ssd_chunk_cumsum_fwd(fake, 0, 2, 2, 1, fake, None, fake, fake, 1, 0, 2, 64, 0, 0.0, 1.0, None) == -2
-    assert handle.ssd_chunk_state_fwd(*grp, *seq, 0, fake, fake, fake, 1, 64, 2, 1, 48, 64, 64, None) == -5
-    assert handle.ssd_chunk_state_fwd(*grp, fake, 8190, 130, 65, 1, fake, fake, fake, 1, 64, 2, 1, 64, 64, 64, None) == -3
-    assert handle.ssd_chunk_state_fwd(*grp, *seq, 9, fake, fake, fake, 1, 64, 2, 1, 64, 64, 64, None) == -4
-    assert handle.ssd_chunk_state_fwd(*grp, *seq, 0, fake, fake, fake, 1, 64, 3, 2, 64, 64, 64, None) == -2
-    assert handle.ssd_bmm_chunk_fwd(*grp, *grp, 0, fake, 1, 1, 64, 1, 64, 64, None) == -4  # bf16 out of f32 in
-    assert handle.ssd_state_passing_fwd(fake, fake, 2, 1, 1, None, fake, fake, 1, 1, 2, 6, None) == -3
+    assert handle.ssd_chunk_state_fwd(*grp, *seq, 0, fake, fake, fake, 1, 64, 2, 1, 48, 64, 64, *ids, None) == -5
+    assert handle.ssd_chunk_state_fwd(*grp, fake, 8190, 130, 65, 1, fake, fake, fake, 1, 64, 2, 1, 64, 64, 64, *ids, None) == -3
+    assert handle.ssd_chunk_state_fwd(*grp, *seq, 9, fake, fake, fake, 1, 64, 2, 1, 64, 64, 64, *ids, None) == -4
+    assert handle.ssd_chunk_state_fwd(*grp, *seq, 0, fake, fake, fake, 1, 64, 3, 2, 64, 64, 64, *ids, None) == -2
+    assert handle.ssd_bmm_chunk_fwd(*grp, *grp, 0, fake, 1, 1, 64, 1, 64, 64, *ids, None) == -4  # bf16 out of f32 in
+    assert handle.ssd_state_passing_fwd(fake, fake, 2, 1, 1, None, fake, fake, 1, 1, 2, 6, *ids, 0, 0, None) == -3
+    # a packed batch must come with the chunking that gives nchunks
+    assert handle.ssd_state_passing_fwd(fake, fake, 2, 1, 1, None, fake, fake, 1, 2, 2, 8, fake, 64, 1, 64, 16, None) == -2
 
 
 def test_error_mapping():

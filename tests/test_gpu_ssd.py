@@ -115,8 +115,8 @@ def test_unsupported_shapes_are_refused(device):
     dt = torch.zeros(1, 2, 1, 64, device=device)
     with pytest.raises(NotImplementedError):
         _chunk_state_fwd(B, x, dt, dt)
-    with pytest.raises(NotImplementedError):
-        _chunk_state_fwd(B, torch.zeros(1, 64, 2, 64, device=device), dt, dt, seq_idx=torch.zeros(1, 64))
+    with pytest.raises(AssertionError):  # ids must be (batch, seqlen)
+        _chunk_state_fwd(B, torch.zeros(1, 64, 2, 64, device=device), dt, dt, seq_idx=torch.zeros(1, 32, device=device))
 
 
 def test_config5_full_size(device):

@@ -48,6 +48,14 @@ int check_dims(int64_t batch, int64_t L, int64_t nh, int64_t g, int64_t P, int64
   return SSD_OK;
 }
 inline bool dim_ok(int64_t v) { return v == 64 || v == 128; }
+// The state-passing entries take the chunking only to locate the last position of each chunk of
+// a packed batch; without seq_idx both numbers are ignored.
+inline int check_seq_chunks(const int32_t* seq_idx, int64_t seqlen, int64_t chunk, int64_t nchunks) {
+  if (!seq_idx) return SSD_OK;
+  if (seqlen <= 0 || chunk <= 0 || seqlen > ((int64_t)1 << 30)) return SSD_ERR_SHAPE;
+  return (seqlen + chunk - 1) / chunk == nchunks ? SSD_OK : SSD_ERR_SHAPE;
+}
+inline SeqIdx as_seq(const int32_t* p, int64_t sb, int64_t sl) { return SeqIdx{p, sb, sl}; }
 constexpr int kLdsBytes = 160 * 1024;  // LDS of one CU
 
 template <typename K>
@@ -81,6 +89,7 @@ struct StateLaunch {
   const float *dt, *dA;
   float* states;
   Dims d;
+  SeqIdx seq;
   hipStream_t st;
   template <typename T, int P, int N>
   int run() const {
@@ -89,7 +98,7 @@ struct StateLaunch {
     SSD_TRY(allow_smem(kernel, smem));
     hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh)), dim3(256), smem, st, (const T*)x, sx,
                        (const T*)B, sB, dt, dA, states, (int)d.nh, (int)(d.nh / d.g), (int)d.L, (int)d.Q,
-                       (int)d.C);
+                       (int)d.C, seq);
     return launched();
   }
 };
@@ -102,6 +111,7 @@ struct ScanLaunch {
   int d_has_hdim;
   void *out, *out_x;
   Dims d;
+  SeqIdx seq;
   hipStream_t st;
   template <typename T, int P, int N>
   int run() const {
@@ -114,7 +124,7 @@ struct ScanLaunch {
       hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh * stiles)), dim3(256), smem, st, cb,
                          (const T*)x, sx, (const T*)z, sz, dt, dA, (const T*)C, sC, prev, D, d_has_hdim, (T*)out,
                          so, (T*)out_x, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C,
-                         stiles);
+                         stiles, seq);
       return launched();
     }
     auto kernel = ssd_chunk_scan_kernel<T, P, N>;
@@ -123,7 +133,8 @@ struct ScanLaunch {
     const int mtiles = (int)((d.Q + 63) / 64);
     hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh * mtiles)), dim3(256), smem, st, cb,
                        (const T*)x, sx, (const T*)z, sz, dt, dA, (const T*)C, sC, prev, D, d_has_hdim, (T*)out, so,
-                       (T*)out_x, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C, mtiles);
+                       (T*)out_x, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C, mtiles,
+                       seq);
     return launched();
   }
 };
@@ -137,6 +148,7 @@ struct DxLaunch {
   void* dx;
   float* ddt;
   Dims d;
+  SeqIdx seq;
   hipStream_t st;
   template <typename T, int P, int N>
   int run() const {
@@ -148,7 +160,7 @@ struct DxLaunch {
       hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh * stiles)), dim3(256), wide_smem, st, cb,
                          (const T*)x, sx, (const T*)dout, sd, dt, dA, (const T*)B, sB, dstates, D, d_has_hdim,
                          (T*)dx, sdx, ddt, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C,
-                         stiles);
+                         stiles, seq);
       return launched();
     }
     auto kernel = ssd_chunk_scan_bwd_dx_kernel<T, P, N>;
@@ -157,7 +169,8 @@ struct DxLaunch {
     const int mtiles = (int)((d.Q + 63) / 64);
     hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh * mtiles)), dim3(256), smem, st, cb,
                        (const T*)x, sx, (const T*)dout, sd, dt, dA, (const T*)B, sB, dstates, D, d_has_hdim, (T*)dx,
-                       sdx, ddt, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C, mtiles);
+                       sdx, ddt, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C, mtiles,
+                       seq);
     return launched();
   }
 };
@@ -171,6 +184,7 @@ struct GroupLaunch {
   Strides3 sbc;
   float *out, *ddA;
   Dims d;
+  SeqIdx seq;
   hipStream_t st;
   template <typename T, int P, int N>
   int run() const {
@@ -180,7 +194,7 @@ struct GroupLaunch {
     const int mtiles = (int)((d.Q + 63) / 64);
     hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.g * mtiles)), dim3(256), smem, st, (const T*)a, sa,
                        s, dt, dA, (const T*)bc, sbc, out, ddA, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L,
-                       (int)d.Q, (int)d.C, mtiles);
+                       (int)d.Q, (int)d.C, mtiles, seq);
     return launched();
   }
 };
@@ -191,7 +205,8 @@ int launch_row_cumsum(float* v, int64_t Q, int64_t rows, hipStream_t st) {
 }
 
 template <typename T, typename TO, int K>
-int launch_bmm(const void* a, Strides3 sa, const void* bm, Strides3 sb, void* out, const Dims& d, hipStream_t st) {
+int launch_bmm(const void* a, Strides3 sa, const void* bm, Strides3 sb, void* out, const Dims& d, SeqIdx seq,
+               hipStream_t st) {
   auto kernel = ssd_bmm_kernel<T, TO, K>;
   constexpr int smem = bmm_smem_bytes<T, K>();
   SSD_TRY(allow_smem(kernel, smem));
@@ -199,7 +214,7 @@ int launch_bmm(const void* a, Strides3 sa, const void* bm, Strides3 sb, void* ou
   const int64_t grid = d.batch * d.C * d.g * tiles * tiles;
   if (grid > 0x7fffffff) return SSD_ERR_SHAPE;
   hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), smem, st, (const T*)a, sa, (const T*)bm, sb, (TO*)out,
-                     (int)d.g, (int)d.L, (int)d.Q, (int)d.C, tiles);
+                     (int)d.g, (int)d.L, (int)d.Q, (int)d.C, tiles, seq);
   return launched();
 }
 
@@ -233,7 +248,7 @@ int ssd_chunk_state_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64_t b_sg,
                         int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, const float* dt,
                         const float* dA_cumsum, float* states, int64_t batch, int64_t seqlen,
                         int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
-                        void* stream) {
+                        const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream) {
   Dims d;
   SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
   SSD_TRY(check_dtype(dtype));
@@ -244,15 +259,17 @@ int ssd_chunk_state_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64_t b_sg,
   SSD_TRY(check_f32(states));
   return dispatch_tpn(dtype, hdim, dstate,
                       StateLaunch<0>{x, B, Strides3{x_sb, x_sl, x_sh}, Strides3{b_sb, b_sl, b_sg}, dt, dA_cumsum,
-                                     states, d, as_stream(stream)});
+                                     states, d, as_seq(seq_idx, seq_sb, seq_sl), as_stream(stream)});
 }
 
 int ssd_state_passing_fwd(const float* states, const float* dA_chunk, int64_t da_sb, int64_t da_sh,
                           int64_t da_sc, const float* initial, float* out, float* final_states,
-                          int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, void* stream) {
+                          int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, const int32_t* seq_idx,
+                          int64_t seq_sb, int64_t seq_sl, int64_t seqlen, int64_t chunk, void* stream) {
   if (batch <= 0 || nchunks <= 0 || nheads <= 0 || dim <= 0) return SSD_ERR_SHAPE;
   if (dim % 4) return SSD_ERR_ALIGN;
   if (!dA_chunk) return SSD_ERR_NULL;
+  SSD_TRY(check_seq_chunks(seq_idx, seqlen, chunk, nchunks));
   SSD_TRY(check_f32(states));
   SSD_TRY(check_f32(out));
   SSD_TRY(check_f32(final_states));
@@ -262,14 +279,14 @@ int ssd_state_passing_fwd(const float* states, const float* dA_chunk, int64_t da
   if (grid > 0x7fffffff || dim > (1 << 24)) return SSD_ERR_SHAPE;
   hipLaunchKernelGGL(ssd_state_passing_kernel, dim3((unsigned)grid), dim3(256), 0, as_stream(stream), states,
                      dA_chunk, da_sb, da_sh, da_sc, initial, out, final_states, (int)nheads, (int)nchunks, (int)dim,
-                     tiles);
+                     tiles, as_seq(seq_idx, seq_sb, seq_sl), (int)seqlen, (int)chunk);
   return launched();
 }
 
 int ssd_bmm_chunk_fwd(const void* a, int64_t a_sb, int64_t a_sl, int64_t a_sg, const void* bm,
                       int64_t b_sb, int64_t b_sl, int64_t b_sg, int dtype, void* out, int out_dtype,
                       int64_t batch, int64_t seqlen, int64_t ngroups, int64_t k, int64_t chunk,
-                      void* stream) {
+                      const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream) {
   Dims d;
   SSD_TRY(check_dims(batch, seqlen, ngroups, ngroups, 0, k, chunk, &d));
   SSD_TRY(check_dtype(dtype));
@@ -281,15 +298,16 @@ int ssd_bmm_chunk_fwd(const void* a, int64_t a_sb, int64_t a_sl, int64_t a_sg, c
   if (!out) return SSD_ERR_NULL;
   const Strides3 sa{a_sb, a_sl, a_sg}, sb{b_sb, b_sl, b_sg};
   hipStream_t st = as_stream(stream);
+  const SeqIdx seq = as_seq(seq_idx, seq_sb, seq_sl);
   if (dtype == SSD_BF16) {
     if (out_dtype == SSD_F32)
-      return k == 64 ? launch_bmm<bf16_t, float, 64>(a, sa, bm, sb, out, d, st)
-                     : launch_bmm<bf16_t, float, 128>(a, sa, bm, sb, out, d, st);
-    return k == 64 ? launch_bmm<bf16_t, bf16_t, 64>(a, sa, bm, sb, out, d, st)
-                   : launch_bmm<bf16_t, bf16_t, 128>(a, sa, bm, sb, out, d, st);
+      return k == 64 ? launch_bmm<bf16_t, float, 64>(a, sa, bm, sb, out, d, seq, st)
+                     : launch_bmm<bf16_t, float, 128>(a, sa, bm, sb, out, d, seq, st);
+    return k == 64 ? launch_bmm<bf16_t, bf16_t, 64>(a, sa, bm, sb, out, d, seq, st)
+                   : launch_bmm<bf16_t, bf16_t, 128>(a, sa, bm, sb, out, d, seq, st);
   }
-  return k == 64 ? launch_bmm<float, float, 64>(a, sa, bm, sb, out, d, st)
-                 : launch_bmm<float, float, 128>(a, sa, bm, sb, out, d, st);
+  return k == 64 ? launch_bmm<float, float, 64>(a, sa, bm, sb, out, d, seq, st)
+                 : launch_bmm<float, float, 128>(a, sa, bm, sb, out, d, seq, st);
 }
 
 int ssd_chunk_scan_fwd(const float* cb, const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
@@ -298,7 +316,7 @@ int ssd_chunk_scan_fwd(const float* cb, const void* x, int64_t x_sb, int64_t x_s
                        int64_t c_sg, const float* prev_states, const float* D, int d_has_hdim, void* out,
                        int64_t o_sb, int64_t o_sl, int64_t o_sh, void* out_x, int64_t batch,
                        int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate,
-                       int64_t chunk, void* stream) {
+                       int64_t chunk, const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream) {
   Dims d;
   SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
   SSD_TRY(check_dtype(dtype));
@@ -315,13 +333,15 @@ int ssd_chunk_scan_fwd(const float* cb, const void* x, int64_t x_sb, int64_t x_s
   return dispatch_tpn(dtype, hdim, dstate,
                       ScanLaunch{cb, x, z, C, Strides3{x_sb, x_sl, x_sh}, Strides3{z_sb, z_sl, z_sh},
                                  Strides3{c_sb, c_sl, c_sg}, Strides3{o_sb, o_sl, o_sh}, dt, dA_cumsum,
-                                 prev_states, D, d_has_hdim, out, out_x, d, as_stream(stream)});
+                                 prev_states, D, d_has_hdim, out, out_x, d, as_seq(seq_idx, seq_sb, seq_sl),
+                                 as_stream(stream)});
 }
 
 int ssd_chunk_scan_bwd_dstates(const void* C, int64_t c_sb, int64_t c_sl, int64_t c_sg, const void* dout,
                                int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype, const float* dA_cumsum,
                                float* dprev_states, int64_t batch, int64_t seqlen, int64_t nheads,
-                               int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk, void* stream) {
+                               int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
+                               const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream) {
   Dims d;
   SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
   SSD_TRY(check_dtype(dtype));
@@ -332,7 +352,8 @@ int ssd_chunk_scan_bwd_dstates(const void* C, int64_t c_sb, int64_t c_sl, int64_
   SSD_TRY(check_f32(dprev_states));
   return dispatch_tpn(dtype, hdim, dstate,
                       StateLaunch<1>{dout, C, Strides3{d_sb, d_sl, d_sh}, Strides3{c_sb, c_sl, c_sg}, dA_cumsum,
-                                     dA_cumsum, dprev_states, d, as_stream(stream)});
+                                     dA_cumsum, dprev_states, d, as_seq(seq_idx, seq_sb, seq_sl),
+                                     as_stream(stream)});
 }
 
 size_t ssd_state_passing_bwd_workspace_bytes(int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim) {
@@ -344,10 +365,13 @@ size_t ssd_state_passing_bwd_workspace_bytes(int64_t batch, int64_t nchunks, int
 int ssd_state_passing_bwd(const float* states, const float* dA_chunk, int64_t da_sb, int64_t da_sh,
                           int64_t da_sc, const float* dout, const float* dfinal, float* dstates,
                           float* ddA_chunk, float* dinit, void* workspace, size_t workspace_bytes,
-                          int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, void* stream) {
+                          int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, const int32_t* seq_idx,
+                          int64_t seq_sb, int64_t seq_sl, int64_t seqlen, int64_t chunk, void* stream) {
   if (batch <= 0 || nchunks <= 0 || nheads <= 0 || dim <= 0) return SSD_ERR_SHAPE;
   if (dim % 4) return SSD_ERR_ALIGN;
   if (!dA_chunk || !ddA_chunk) return SSD_ERR_NULL;
+  SSD_TRY(check_seq_chunks(seq_idx, seqlen, chunk, nchunks));
+  const SeqIdx seq = as_seq(seq_idx, seq_sb, seq_sl);
   SSD_TRY(check_f32(states));
   SSD_TRY(check_f32(dout));
   SSD_TRY(check_f32(dstates));
@@ -361,12 +385,13 @@ int ssd_state_passing_bwd(const float* states, const float* dA_chunk, int64_t da
   hipStream_t st = as_stream(stream);
   float* part = static_cast<float*>(workspace);
   hipLaunchKernelGGL(ssd_state_passing_bwd_kernel, dim3((unsigned)grid), dim3(256), 0, st, states, dA_chunk, da_sb,
-                     da_sh, da_sc, dout, dfinal, dstates, part, dinit, (int)nheads, (int)nchunks, (int)dim, tiles);
+                     da_sh, da_sc, dout, dfinal, dstates, part, dinit, (int)nheads, (int)nchunks, (int)dim, tiles, seq,
+                     (int)seqlen, (int)chunk);
   SSD_TRY(launched());
   const int64_t total = batch * nheads * nchunks;
   hipLaunchKernelGGL(ssd_state_passing_bwd_finish_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
                      part, dA_chunk, da_sb, da_sh, da_sc, ddA_chunk, (int)nheads, (int)nchunks, tiles * 4,
-                     dinit ? 1 : 0, total);
+                     dinit ? 1 : 0, total, seq, (int)seqlen, (int)chunk);
   return launched();
 }
 
@@ -374,7 +399,8 @@ int ssd_chunk_state_bwd_db(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_
                            const float* dt, const float* dA_cumsum, const float* dstates, const void* B,
                            int64_t b_sb, int64_t b_sl, int64_t b_sg, float* dB, float* ddA_cumsum,
                            int64_t batch, int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim,
-                           int64_t dstate, int64_t chunk, void* stream) {
+                           int64_t dstate, int64_t chunk, const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl,
+                           void* stream) {
   Dims d;
   SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
   SSD_TRY(check_dtype(dtype));
@@ -387,7 +413,8 @@ int ssd_chunk_state_bwd_db(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_
   hipStream_t st = as_stream(stream);
   SSD_TRY(dispatch_tpn(dtype, hdim, dstate,
                        GroupLaunch<0>{x, Strides3{x_sb, x_sl, x_sh}, dstates, dt, dA_cumsum, B,
-                                      Strides3{b_sb, b_sl, b_sg}, dB, ddA_cumsum, d, st}));
+                                      Strides3{b_sb, b_sl, b_sg}, dB, ddA_cumsum, d,
+                                      as_seq(seq_idx, seq_sb, seq_sl), st}));
   if (!B) return SSD_OK;
   return launch_row_cumsum(ddA_cumsum, chunk, batch * nheads * d.C, st);
 }
@@ -396,7 +423,7 @@ int ssd_chunk_scan_bwd_dc(const void* dout, int64_t d_sb, int64_t d_sl, int64_t 
                           const float* dA_cumsum, const float* prev_states, const void* C, int64_t c_sb,
                           int64_t c_sl, int64_t c_sg, float* dC, float* ddA_cumsum_prev, int64_t batch,
                           int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate,
-                          int64_t chunk, void* stream) {
+                          int64_t chunk, const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream) {
   Dims d;
   SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
   SSD_TRY(check_dtype(dtype));
@@ -408,7 +435,8 @@ int ssd_chunk_scan_bwd_dc(const void* dout, int64_t d_sb, int64_t d_sl, int64_t 
   if (C) SSD_TRY(check_vec(C, c_sb, c_sl, c_sg, dtype, dstate));
   return dispatch_tpn(dtype, hdim, dstate,
                       GroupLaunch<1>{dout, Strides3{d_sb, d_sl, d_sh}, prev_states, dA_cumsum, dA_cumsum, C,
-                                     Strides3{c_sb, c_sl, c_sg}, dC, ddA_cumsum_prev, d, as_stream(stream)});
+                                     Strides3{c_sb, c_sl, c_sg}, dC, ddA_cumsum_prev, d,
+                                     as_seq(seq_idx, seq_sb, seq_sl), as_stream(stream)});
 }
 
 int ssd_chunk_scan_chunk_state_bwd_dx(const float* cb, const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
@@ -418,7 +446,7 @@ int ssd_chunk_scan_chunk_state_bwd_dx(const float* cb, const void* x, int64_t x_
                                       int d_has_hdim, void* dx, int64_t dx_sb, int64_t dx_sl, int64_t dx_sh,
                                       float* ddt, int64_t batch, int64_t seqlen, int64_t nheads,
                                       int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
-                                      void* stream) {
+                                      const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream) {
   Dims d;
   SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
   SSD_TRY(check_dtype(dtype));
@@ -434,7 +462,7 @@ int ssd_chunk_scan_chunk_state_bwd_dx(const float* cb, const void* x, int64_t x_
   return dispatch_tpn(dtype, hdim, dstate,
                       DxLaunch{cb, x, dout, B, Strides3{x_sb, x_sl, x_sh}, Strides3{d_sb, d_sl, d_sh},
                                Strides3{b_sb, b_sl, b_sg}, Strides3{dx_sb, dx_sl, dx_sh}, dt, dA_cumsum, dstates, D,
-                               d_has_hdim, dx, ddt, d, as_stream(stream)});
+                               d_has_hdim, dx, ddt, d, as_seq(seq_idx, seq_sb, seq_sl), as_stream(stream)});
 }
 
 static size_t ddAcs_part_floats(const Dims& d) {

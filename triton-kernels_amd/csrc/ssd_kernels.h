@@ -35,6 +35,36 @@ struct Strides3 {
   int64_t sb, sl, sh;
 };
 
+// Sequence ids of a packed batch: (batch, seqlen) int32 addressed by element strides; p is null
+// when the batch is not packed.  Positions with different ids belong to different sequences and
+// do not see each other's state.
+struct SeqIdx {
+  const int* p;
+  int64_t sb, sl;
+};
+
+// The ids of one chunk.  at(-1) is the last position of the previous chunk.
+struct ChunkSeq {
+  const int* p;
+  int64_t sl;
+  __device__ __forceinline__ bool on() const { return p != nullptr; }
+  __device__ __forceinline__ int at(int k) const { return p[(int64_t)k * sl]; }
+  // id that the state entering chunk c carries: the reference starts from id 0
+  __device__ __forceinline__ int entering(int c) const { return c > 0 ? at(-1) : 0; }
+};
+__device__ __forceinline__ ChunkSeq chunk_seq(SeqIdx s, int64_t b, int c, int Q) {
+  return ChunkSeq{s.p ? s.p + b * s.sb + (int64_t)c * Q * s.sl : nullptr, s.sl};
+}
+// Whether the state survives chunk c: the id at the end of the chunk equals the id at the end of
+// the previous one (0 before the first chunk).
+__device__ __forceinline__ bool chunk_keeps_state(SeqIdx s, int64_t b, int c, int Q, int L) {
+  if (!s.p) return true;
+  const int* q = s.p + b * s.sb;
+  const int cur = q[(int64_t)(min((c + 1) * Q, L) - 1) * s.sl];
+  const int before = c > 0 ? q[(int64_t)(c * Q - 1) * s.sl] : 0;
+  return cur == before;
+}
+
 // ------------------------------------------------------------------ operand fragments
 // Both return, for lane l, EPL = Vec16<T>::N consecutive contraction indices starting at
 // k0 + EPL * (l / 32), for row or column (l % 32) of the 32-wide block: the register layout
@@ -154,7 +184,9 @@ __global__ __launch_bounds__(256) void ssd_cumsum_kernel(const TD* __restrict__ 
 // (4 waves) per (b, c, h):
 //   MODE 0  states[p][n] = sum_k x[k][p] * round_T(B[k][n] * exp(min(dA_last - dA_k, 0)) * dt_k)
 //   MODE 1  dprev[p][n]  = sum_k round_T(dout[k][p] * exp(dA_k)) * C[k][n]
-// (x / B stand for dout / C in MODE 1; dt is not read).  The chunk is walked in stages of 64
+// (x / B stand for dout / C in MODE 1; dt is not read).  In a packed batch position k only
+// counts if its id equals the id of the chunk's last position (MODE 0; none counts if that id is
+// negative) or of the previous chunk's last position (MODE 1).  The chunk is walked in stages of 64
 // rows; both operands are contracted along their rows.  The (P/32) x (N/32) output blocks are
 // dealt to the waves round-robin.
 // ------------------------------------------------------------------------------------
@@ -168,7 +200,7 @@ template <typename T, int P, int N, int MODE>
 __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
     const T* __restrict__ x, Strides3 sx, const T* __restrict__ B, Strides3 sB,
     const float* __restrict__ dt, const float* __restrict__ dA_cs, float* __restrict__ states, int nh,
-    int heads_per_group, int L, int Q, int C) {
+    int heads_per_group, int L, int Q, int C, SeqIdx seq) {
   using S = StateSmem<T, P, N>;
   constexpr int KT = S::KT, PX = S::PX, PB = S::PB, KG = Tile<T>::KG;
   constexpr int MB = P / 32, NB = N / 32, BPW = MB * NB / 4;
@@ -186,6 +218,9 @@ __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
   const float dA_last = dAp[Q - 1];
   const T* xg = x + b * sx.sb + (int64_t)c * Q * sx.sl + h * sx.sh;
   const T* Bg = B + b * sB.sb + (int64_t)c * Q * sB.sl + (h / heads_per_group) * sB.sh;
+  const ChunkSeq sq = chunk_seq(seq, b, c, Q);
+  const int seq_ref = !sq.on() ? 0 : (MODE == 0 ? sq.at(limit - 1) : sq.entering(c));
+  const bool seq_dead = MODE == 0 && seq_ref < 0;
 
   floatx16 acc[BPW];
 #pragma unroll
@@ -195,10 +230,14 @@ __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
     if (MODE == 0) {
       stage_rows<T, KT, P>(xs, xg, sx.sl, k0, limit, tid, NoScale());
       stage_rows<T, KT, N>(bs, Bg, sB.sl, k0, limit, tid, [&](int k) {
-        return __expf(fminf(dA_last - dAp[k], 0.f)) * dtp[k];
+        const float w = __expf(fminf(dA_last - dAp[k], 0.f)) * dtp[k];
+        return (sq.on() && (seq_dead || sq.at(k) != seq_ref)) ? 0.f : w;
       });
     } else {
-      stage_rows<T, KT, P>(xs, xg, sx.sl, k0, limit, tid, [&](int k) { return __expf(dAp[k]); });
+      stage_rows<T, KT, P>(xs, xg, sx.sl, k0, limit, tid, [&](int k) {
+        const float w = __expf(dAp[k]);
+        return (sq.on() && sq.at(k) != seq_ref) ? 0.f : w;
+      });
       stage_rows<T, KT, N>(bs, Bg, sB.sl, k0, limit, tid, NoScale());
     }
     __syncthreads();
@@ -227,12 +266,13 @@ __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
 // states[b, c]; the value after the last chunk goes to final.  One thread per four adjacent
 // state elements, the running state in registers, chunks fetched four ahead.
 // states / out are (b, C, nh, dim) dense float32; dA_chunk is addressed by strides (it is the
-// last column of dA_cumsum).
+// last column of dA_cumsum).  In a packed batch the state is dropped across a chunk whose last
+// position has another id than the previous chunk's last position.
 // ------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void ssd_state_passing_kernel(
     const float* __restrict__ states, const float* __restrict__ dA_chunk, int64_t da_sb, int64_t da_sh,
     int64_t da_sc, const float* __restrict__ initial, float* __restrict__ out, float* __restrict__ final_states,
-    int nh, int C, int dim, int tiles) {
+    int nh, int C, int dim, int tiles, SeqIdx seq, int L, int Q) {
   const int tile = blockIdx.x % tiles;
   const int h = (blockIdx.x / tiles) % nh;
   const int64_t b = blockIdx.x / (tiles * nh);
@@ -253,6 +293,7 @@ __global__ __launch_bounds__(256) void ssd_state_passing_kernel(
       const int c = c0 + u;
       nv[u] = c < C ? *reinterpret_cast<const float4*>(src + c * chunk_stride) : make_float4(0.f, 0.f, 0.f, 0.f);
       a[u] = c < C ? __expf(da[(int64_t)c * da_sc]) : 0.f;
+      if (c < C && !chunk_keeps_state(seq, b, c, Q, L)) a[u] = 0.f;
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -291,7 +332,7 @@ __global__ __launch_bounds__(256) void ssd_state_passing_bwd_kernel(
     const float* __restrict__ states, const float* __restrict__ dA_chunk, int64_t da_sb, int64_t da_sh,
     int64_t da_sc, const float* __restrict__ dout, const float* __restrict__ dfinal,
     float* __restrict__ dstates, float* __restrict__ part, float* __restrict__ dinit, int nh, int C, int dim,
-    int tiles) {
+    int tiles, SeqIdx seq, int L, int Q) {
   const int tile = blockIdx.x % tiles;
   const int h = (blockIdx.x / tiles) % nh;
   const int64_t b = blockIdx.x / (tiles * nh);
@@ -315,6 +356,7 @@ __global__ __launch_bounds__(256) void ssd_state_passing_bwd_kernel(
       sv[u] = in ? *reinterpret_cast<const float4*>(states + base + c * chunk_stride) : zero4;
       dv[u] = in ? *reinterpret_cast<const float4*>(dout + base + c * chunk_stride) : zero4;
       a[u] = c >= 0 ? __expf(da[(int64_t)c * da_sc]) : 0.f;
+      if (c >= 0 && !chunk_keeps_state(seq, b, c, Q, L)) a[u] = 0.f;
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -335,7 +377,8 @@ __global__ __launch_bounds__(256) void ssd_state_passing_bwd_kernel(
 
 __global__ __launch_bounds__(256) void ssd_state_passing_bwd_finish_kernel(
     const float* __restrict__ part, const float* __restrict__ dA_chunk, int64_t da_sb, int64_t da_sh,
-    int64_t da_sc, float* __restrict__ ddA, int nh, int C, int nw, int has_init, int64_t total) {
+    int64_t da_sc, float* __restrict__ ddA, int nh, int C, int nw, int has_init, int64_t total, SeqIdx seq,
+    int L, int Q) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // (b * nh + h) * C + c
   if (i >= total) return;
   const int c = (int)(i % C);
@@ -344,7 +387,8 @@ __global__ __launch_bounds__(256) void ssd_state_passing_bwd_finish_kernel(
   const int64_t b = bh / nh;
   float s = 0.f;
   for (int w = 0; w < nw; ++w) s += part[i * nw + w];
-  ddA[i] = (c == 0 && !has_init) ? 0.f : __expf(dA_chunk[b * da_sb + h * da_sh + (int64_t)c * da_sc]) * s;
+  const bool dropped = (c == 0 && !has_init) || !chunk_keeps_state(seq, b, c, Q, L);
+  ddA[i] = dropped ? 0.f : __expf(dA_chunk[b * da_sb + h * da_sh + (int64_t)c * da_sc]) * s;
 }
 
 // In-place inclusive cumsum along the last axis of a dense (rows, Q) float32 array; one wave
@@ -379,6 +423,8 @@ __global__ __launch_bounds__(256) void ssd_row_cumsum_kernel(float* __restrict__
 //   out[m][n] = sum_h d_h[m][n]                       (float32, (b, L, g, N))
 //   with bc (B for MODE 0, C for MODE 1): r_h[m] = sum_n d_h[m][n] * bc[m][n], written to
 //   ddA[b,h,c, m + 1] (MODE 0, slot 0 = 0; the caller then takes the cumsum) or ddA[b,h,c,m] (MODE 1).
+// In a packed batch w_m is 0 unless the id of m equals the id of the chunk's last position
+// (MODE 0) or of the previous chunk's last position (MODE 1).
 // a is read row-major straight from global memory; s is staged in LDS (rounded to T) and
 // contracted along its rows.
 // ------------------------------------------------------------------------------------
@@ -392,7 +438,8 @@ template <typename T, int P, int N, int MODE>
 __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
     const T* __restrict__ a, Strides3 sa, const float* __restrict__ s, const float* __restrict__ dt,
     const float* __restrict__ dA_cs, const T* __restrict__ bc, Strides3 sbc, float* __restrict__ out,
-    float* __restrict__ ddA, int nh, int heads_per_group, int ngroups, int L, int Q, int C, int mtiles) {
+    float* __restrict__ ddA, int nh, int heads_per_group, int ngroups, int L, int Q, int C, int mtiles,
+    SeqIdx seq) {
   using S = GroupSmem<T, P, N>;
   constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, NB = N / 32, BPW = 2 * NB / 4;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -408,6 +455,15 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
   const int limit = min(Q, L - c * Q);
   const int m0 = 64 * mt;
 
+  // packed batch: rows of another sequence than the reference position get no weight
+  bool row_live = true;
+  {
+    const ChunkSeq sq = chunk_seq(seq, b, c, Q);
+    if (sq.on() && tid < 64) {
+      const int ref = MODE == 0 ? sq.at(limit - 1) : sq.entering(c);
+      row_live = sq.at(min(m0 + tid, limit - 1)) == ref;
+    }
+  }
   // block i of this wave: rows 32*mi.., columns 32*ni..
   int mi[BPW], ni[BPW];
 #pragma unroll
@@ -459,7 +515,7 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
     if (tid < 64) {  // one weight per row, computed once instead of by every lane that holds the row
       const int mc = min(m0 + tid, Q - 1);
       wv = MODE == 0 ? __expf(fminf(dAp[Q - 1] - dAp[mc], 0.f)) * dtp[mc] : __expf(dAp[mc]);
-      wrow[tid] = m0 + tid < Q ? wv : 0.f;
+      wrow[tid] = (m0 + tid < Q && row_live) ? wv : 0.f;
     }
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
@@ -529,7 +585,8 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
 
 // ------------------------------------------------------------------------------------
 // bmm_chunk.  out[b, c, g, m, k] = sum_n a[b, cQ+m, g, n] * bm[b, cQ+k, g, n]; one workgroup
-// per 64 x 64 output tile, one 32 x 32 block per wave; rows past the sequence are zero.
+// per 64 x 64 output tile, one 32 x 32 block per wave; rows past the sequence are zero, and so
+// are, in a packed batch, the entries whose two positions carry different ids.
 // ------------------------------------------------------------------------------------
 template <typename T, int K>
 constexpr int bmm_smem_bytes() {
@@ -540,7 +597,7 @@ template <typename T, typename TO, int K>
 __global__ __launch_bounds__(256) void ssd_bmm_kernel(const T* __restrict__ a, Strides3 sa,
                                                       const T* __restrict__ bm, Strides3 sb_,
                                                       TO* __restrict__ out, int ngroups, int L, int Q, int C,
-                                                      int tiles) {
+                                                      int tiles, SeqIdx seq) {
   constexpr int PK = Tile<T>::pitch(K), KG = Tile<T>::KG;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* as = reinterpret_cast<T*>(smem);
@@ -565,10 +622,14 @@ __global__ __launch_bounds__(256) void ssd_bmm_kernel(const T* __restrict__ a, S
     mma_group(frag_rows(as, PK, 32 * wm, kk, lane), frag_rows(bs, PK, 32 * wn, kk, lane), acc);
   TO* o = out + bcg * (int64_t)Q * Q;
   const int col = 64 * tn + 32 * wn + (lane & 31);
+  const ChunkSeq sq = chunk_seq(seq, b, c, Q);
+  const int col_id = sq.on() ? sq.at(min(col, limit - 1)) : 0;
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
     const int row = 64 * tm + 32 * wm + acc_row(v, lane);
-    if (row < Q && col < Q) o[(int64_t)row * Q + col] = (TO)acc[v];
+    float val = acc[v];
+    if (sq.on() && sq.at(min(row, limit - 1)) != col_id) val = 0.f;
+    if (row < Q && col < Q) o[(int64_t)row * Q + col] = (TO)val;
   }
 }
 
@@ -578,7 +639,9 @@ __global__ __launch_bounds__(256) void ssd_bmm_kernel(const T* __restrict__ a, S
 //             + sum_{k <= m} round_T(cb[m][k] * exp(min(dA_m - dA_k, 0)) * dt_k) * x[k][p]
 //             + D * x[m][p],            then out_x = out (if asked) and out *= z * sigmoid(z).
 // The causal sum walks the 64-row tiles k up to the diagonal one; the result leaves through an
-// LDS tile so that z, out and out_x move in 16-byte pieces.
+// LDS tile so that z, out and out_x move in 16-byte pieces.  In a packed batch the carried state
+// only reaches the rows whose id equals that of the previous chunk's last position (cb already
+// holds zeros between positions of different ids).
 // cb is float32 (b, C, g, Q, Q); prev is float32 (b, C, nh, P, N).
 // ------------------------------------------------------------------------------------
 template <typename T, int P, int N>
@@ -597,7 +660,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(
     const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Cm, Strides3 sC,
     const float* __restrict__ prev, const float* __restrict__ D, int d_has_hdim, T* __restrict__ out,
     Strides3 so, T* __restrict__ out_x, int nh, int heads_per_group, int ngroups, int L, int Q, int C,
-    int mtiles) {
+    int mtiles, SeqIdx seq) {
   using S = ScanSmem<T, P, N>;
   constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, PB = P / 32, BPW = 2 * PB / 4;
   static_assert(PB == 2 || PB == 4, "hdim 64 or 128");
@@ -645,7 +708,11 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(
       d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
     }
   }
-  if (tid < 64) sm[tid] = m0 + tid < Q ? __expf(dAp[m0 + tid]) : 0.f;
+  if (tid < 64) {
+    const ChunkSeq sq = chunk_seq(seq, b, c, Q);
+    const bool live = !sq.on() || sq.at(min(m0 + tid, limit - 1)) == sq.entering(c);
+    sm[tid] = (m0 + tid < Q && live) ? __expf(dAp[m0 + tid]) : 0.f;
+  }
   __syncthreads();
 #pragma unroll
   for (int kk = 0; kk < N; kk += KG) {
@@ -774,7 +841,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
     const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Cm, Strides3 sC,
     const float* __restrict__ prev, const float* __restrict__ D, int d_has_hdim, T* __restrict__ out,
     Strides3 so, T* __restrict__ out_x, int nh, int heads_per_group, int ngroups, int L, int Q, int C,
-    int stiles) {
+    int stiles, SeqIdx seq) {
   using S = WideSmem<T, P, N>;
   constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, PB = P / 32, ST = S::ST;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -823,7 +890,11 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
       d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
     }
   }
-  sm[tid] = __expf(dAp[m0 + tid]);
+  {
+    const ChunkSeq sq = chunk_seq(seq, b, c, Q);
+    const bool live = !sq.on() || sq.at(min(m0 + tid, limit - 1)) == sq.entering(c);
+    sm[tid] = live ? __expf(dAp[m0 + tid]) : 0.f;
+  }
   __syncthreads();
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {
@@ -942,7 +1013,8 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
 //   dx[m][p] = acc * dt_m + D * dout[m][p],    ddt[m] = sum_p acc[m][p] * x[m][p]
 // The mirror image of ssd_chunk_scan_kernel: the k tiles run from the diagonal one to the end
 // of the chunk, and the weights are staged transposed (k-major), so that cb is still read along
-// its rows.
+// its rows.  In a packed batch the dstates term only reaches the rows whose id equals that of the
+// chunk's last position.
 // ------------------------------------------------------------------------------------
 template <typename T, int P, int N>
 __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
@@ -950,7 +1022,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
     const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Bm, Strides3 sB,
     const float* __restrict__ dstates, const float* __restrict__ D, int d_has_hdim, T* __restrict__ dx,
     Strides3 sdx, float* __restrict__ ddt, int nh, int heads_per_group, int ngroups, int L, int Q, int C,
-    int mtiles) {
+    int mtiles, SeqIdx seq) {
   using S = ScanSmem<T, P, N>;
   constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, PB = P / 32, BPW = 2 * PB / 4;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -1001,7 +1073,11 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
       d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
     }
   }
-  if (tid < 64) sm[tid] = m0 + tid < Q ? __expf(fminf(dAp[Q - 1] - dAp[m0 + tid], 0.f)) : 0.f;
+  if (tid < 64) {
+    const ChunkSeq sq = chunk_seq(seq, b, c, Q);
+    const bool live = !sq.on() || sq.at(min(m0 + tid, limit - 1)) == sq.at(limit - 1);
+    sm[tid] = (m0 + tid < Q && live) ? __expf(fminf(dAp[Q - 1] - dAp[m0 + tid], 0.f)) : 0.f;
+  }
   __syncthreads();
 #pragma unroll
   for (int kk = 0; kk < N; kk += KG) {
@@ -1236,7 +1312,7 @@ __global__ __launch_bounds__(256, 3) void ssd_chunk_scan_bwd_dx_wide_kernel(
     const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Bm, Strides3 sB,
     const float* __restrict__ dstates, const float* __restrict__ D, int d_has_hdim, T* __restrict__ dx,
     Strides3 sdx, float* __restrict__ ddt, int nh, int heads_per_group, int ngroups, int L, int Q, int C,
-    int stiles) {
+    int stiles, SeqIdx seq) {
   using S = WideSmem<T, P, N>;
   constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, PB = P / 32, ST = S::ST;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -1288,7 +1364,11 @@ __global__ __launch_bounds__(256, 3) void ssd_chunk_scan_bwd_dx_wide_kernel(
       d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
     }
   }
-  sm[tid] = __expf(fminf(dAp[Q - 1] - dAp[m0 + tid], 0.f));
+  {
+    const ChunkSeq sq = chunk_seq(seq, b, c, Q);
+    const bool live = !sq.on() || sq.at(min(m0 + tid, limit - 1)) == sq.at(limit - 1);
+    sm[tid] = live ? __expf(fminf(dAp[Q - 1] - dAp[m0 + tid], 0.f)) : 0.f;
+  }
   __syncthreads();
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {

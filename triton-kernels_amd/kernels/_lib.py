@@ -21,6 +21,7 @@ EMA_MAX_CHUNK = 1024
 _I = c_int64
 _P = c_void_p
 _SEQ = [_P, _I, _I, _I]  # pointer + (batch, position, head) strides
+_IDS = [_P, _I, _I]  # seq_idx pointer (may be null) + (batch, position) strides
 
 _SIGNATURES = {
     "ema_version": (c_char_p, []),
@@ -49,17 +50,17 @@ _SIGNATURES = {
     "ema_seq_bwd": (c_int, [c_int] + _SEQ + _SEQ + _SEQ + [_P, _P, c_int] + _SEQ + _SEQ + [_P, _P, c_size_t, _I, _I, _I, _I, _P, _P, _P]),
     # SSD forward stages (include/ssd_hip.h)
     "ssd_chunk_cumsum_fwd": (c_int, [_P, c_int, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, c_int, c_float, c_float, _P]),
-    "ssd_chunk_state_fwd": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
-    "ssd_state_passing_fwd": (c_int, [_P, _P, _I, _I, _I, _P, _P, _P, _I, _I, _I, _I, _P]),
-    "ssd_bmm_chunk_fwd": (c_int, _SEQ + _SEQ + [c_int, _P, c_int, _I, _I, _I, _I, _I, _P]),
-    "ssd_chunk_scan_fwd": (c_int, [_P] + _SEQ + _SEQ + [c_int, _P, _P] + _SEQ + [_P, _P, c_int] + _SEQ + [_P, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "ssd_chunk_state_fwd": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
+    "ssd_state_passing_fwd": (c_int, [_P, _P, _I, _I, _I, _P, _P, _P, _I, _I, _I, _I] + _IDS + [_I, _I, _P]),
+    "ssd_bmm_chunk_fwd": (c_int, _SEQ + _SEQ + [c_int, _P, c_int, _I, _I, _I, _I, _I] + _IDS + [_P]),
+    "ssd_chunk_scan_fwd": (c_int, [_P] + _SEQ + _SEQ + [c_int, _P, _P] + _SEQ + [_P, _P, c_int] + _SEQ + [_P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
     # SSD backward stages
-    "ssd_chunk_scan_bwd_dstates": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "ssd_chunk_scan_bwd_dstates": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
     "ssd_state_passing_bwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
-    "ssd_state_passing_bwd": (c_int, [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _P]),
-    "ssd_chunk_state_bwd_db": (c_int, _SEQ + [c_int, _P, _P, _P] + _SEQ + [_P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
-    "ssd_chunk_scan_bwd_dc": (c_int, _SEQ + [c_int, _P, _P] + _SEQ + [_P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
-    "ssd_chunk_scan_chunk_state_bwd_dx": (c_int, [_P] + _SEQ + _SEQ + [c_int, _P, _P] + _SEQ + [_P, _P, c_int] + _SEQ + [_P, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "ssd_state_passing_bwd": (c_int, [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I] + _IDS + [_I, _I, _P]),
+    "ssd_chunk_state_bwd_db": (c_int, _SEQ + [c_int, _P, _P, _P] + _SEQ + [_P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
+    "ssd_chunk_scan_bwd_dc": (c_int, _SEQ + [c_int, _P, _P] + _SEQ + [_P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
+    "ssd_chunk_scan_chunk_state_bwd_dx": (c_int, [_P] + _SEQ + _SEQ + [c_int, _P, _P] + _SEQ + [_P, _P, c_int] + _SEQ + [_P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
     "ssd_chunk_scan_bwd_ddAcs_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "ssd_chunk_scan_bwd_ddAcs": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _I, _P]),
 }
@@ -171,3 +172,15 @@ def f32c(t: torch.Tensor) -> torch.Tensor:
     if t.dtype != torch.float32:
         t = t.float()
     return t.contiguous()
+
+
+def seq_ids(seq_idx, batch: int, seqlen: int, dev: torch.device):
+    """(int32 tensor kept alive by the caller or None, [ptr, sb, sl]) of the ids of a packed batch."""
+    if seq_idx is None:
+        return None, [None, 0, 0]
+    assert seq_idx.shape == (batch, seqlen)
+    if seq_idx.device != dev:
+        raise AssertionError("all tensors must be on the same device")
+    if seq_idx.dtype != torch.int32:
+        seq_idx = seq_idx.to(torch.int32)
+    return seq_idx, [seq_idx.data_ptr(), seq_idx.stride(0), seq_idx.stride(1)]

@@ -20,9 +20,8 @@ def _bmm_chunk_fwd(a, b, chunk_size, seq_idx=None, causal=False, output_dtype=No
         batch, seqlen, ngroups, k = a.shape
         a4, b4 = a, b
     assert b.shape == a.shape
-    if seq_idx is not None:
-        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
     dev = _lib.require_gpu(a, b)
+    seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)
     if b4.dtype != a4.dtype:
         b4 = b4.to(a4.dtype)
     a4, sa = _lib.strided4(a4)
@@ -34,7 +33,7 @@ def _bmm_chunk_fwd(a, b, chunk_size, seq_idx=None, causal=False, output_dtype=No
     with torch.cuda.device(dev):
         _lib.check(
             _lib.lib().ssd_bmm_chunk_fwd(*sa, *sb, _lib.dtype_code(a4), out.data_ptr(), _lib.dtype_code(out), batch,
-                                         seqlen, ngroups, k, chunk_size, _lib.stream_ptr(dev)),
+                                         seqlen, ngroups, k, chunk_size, *ids, _lib.stream_ptr(dev)),
             "ssd_bmm_chunk_fwd")
     if out.dtype != out_dtype:
         out = out.to(out_dtype)

@@ -39,9 +39,9 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
 
 
 def mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
-                                  initial_states=None, dt_softplus=False, dt_limit=(0.0, float("inf")),
-                                  return_final_states=False):
+                                  initial_states=None, seq_idx=None, dt_softplus=False,
+                                  dt_limit=(0.0, float("inf")), return_final_states=False):
     out, _, _, _, _, final_states = _mamba_chunk_scan_combined_fwd(
         x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, initial_states=initial_states,
-        dt_softplus=dt_softplus, dt_limit=dt_limit)
+        seq_idx=seq_idx, dt_softplus=dt_softplus, dt_limit=dt_limit)
     return (out, final_states) if return_final_states else out

@@ -21,9 +21,8 @@ def _chunk_scan_fwd(cb, x, dt, dA_cumsum, C, states, D=None, z=None, seq_idx=Non
     assert dt.shape == (batch, nheads, nchunks, chunk_size)
     assert dA_cumsum.shape == (batch, nheads, nchunks, chunk_size)
     assert states.shape == (batch, nchunks, nheads, headdim, dstate)
-    if seq_idx is not None:
-        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
     dev = _lib.require_gpu(x, cb, dt, dA_cumsum, C, states)
+    seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)
     x, xs = _lib.strided4(x)
     if C.dtype != x.dtype:
         C = C.to(x.dtype)
@@ -41,6 +40,6 @@ def _chunk_scan_fwd(cb, x, dt, dA_cumsum, C, states, D=None, z=None, seq_idx=Non
                 _lib.f32c(dA_cumsum).data_ptr(), *cs, _lib.f32c(states).data_ptr(),
                 None if Df is None else Df.data_ptr(), int(D is not None and D.dim() == 2), out.data_ptr(),
                 out.stride(0), out.stride(1), out.stride(2), None if out_x is None else out_x.data_ptr(), batch,
-                seqlen, nheads, ngroups, headdim, dstate, chunk_size, _lib.stream_ptr(dev)),
+                seqlen, nheads, ngroups, headdim, dstate, chunk_size, *ids, _lib.stream_ptr(dev)),
             "ssd_chunk_scan_fwd")
     return out, out_x

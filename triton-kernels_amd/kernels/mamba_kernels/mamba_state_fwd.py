@@ -14,11 +14,10 @@ def _chunk_state_fwd(B, x, dt, dA_cumsum, seq_idx=None, states=None, states_in_f
     assert B.shape == (batch, seqlen, ngroups, dstate)
     assert dt.shape == (batch, nheads, nchunks, chunk_size)
     assert dA_cumsum.shape == dt.shape
-    if seq_idx is not None:
-        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
     dev = _lib.require_gpu(x, B, dt, dA_cumsum)
     if B.dtype != x.dtype:
         B = B.to(x.dtype)  # the reference rounds the weighted B to x's type before the product
+    seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)
     x, xs = _lib.strided4(x)
     B, bs = _lib.strided4(B)
     out = torch.empty(batch, nchunks, nheads, headdim, dstate, device=dev, dtype=torch.float32)
@@ -26,7 +25,7 @@ def _chunk_state_fwd(B, x, dt, dA_cumsum, seq_idx=None, states=None, states_in_f
         _lib.check(
             _lib.lib().ssd_chunk_state_fwd(*bs, *xs, _lib.dtype_code(x), _lib.f32c(dt).data_ptr(),
                                            _lib.f32c(dA_cumsum).data_ptr(), out.data_ptr(), batch, seqlen, nheads,
-                                           ngroups, headdim, dstate, chunk_size, _lib.stream_ptr(dev)),
+                                           ngroups, headdim, dstate, chunk_size, *ids, _lib.stream_ptr(dev)),
             "ssd_chunk_state_fwd")
     if states is not None:
         assert states.shape == (batch, nchunks, nheads, headdim, dstate)

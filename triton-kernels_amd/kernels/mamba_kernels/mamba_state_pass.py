@@ -12,9 +12,13 @@ def _state_passing_fwd(states, dA_chunk_cumsum, initial_states=None, seq_idx=Non
     assert dA_chunk_cumsum.shape == (batch, nheads, nchunks)
     if initial_states is not None:
         assert initial_states.shape == (batch, nheads, dim)
-    if seq_idx is not None:
-        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
     dev = _lib.require_gpu(states, dA_chunk_cumsum)
+    seqlen = 0
+    if seq_idx is not None:
+        assert chunk_size is not None
+        seqlen = seq_idx.shape[-1]
+        assert nchunks == (seqlen + chunk_size - 1) // chunk_size
+    seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)
     out_dtype = states.dtype if out_dtype is None else out_dtype
     st = _lib.f32c(states)
     da = dA_chunk_cumsum if dA_chunk_cumsum.dtype == torch.float32 else dA_chunk_cumsum.float()
@@ -25,7 +29,7 @@ def _state_passing_fwd(states, dA_chunk_cumsum, initial_states=None, seq_idx=Non
         _lib.check(
             _lib.lib().ssd_state_passing_fwd(st.data_ptr(), da.data_ptr(), da.stride(0), da.stride(1), da.stride(2),
                                              None if init is None else init.data_ptr(), out.data_ptr(),
-                                             final_states.data_ptr(), batch, nchunks, nheads, dim,
-                                             _lib.stream_ptr(dev)),
+                                             final_states.data_ptr(), batch, nchunks, nheads, dim, *ids, seqlen,
+                                             chunk_size or 0, _lib.stream_ptr(dev)),
             "ssd_state_passing_fwd")
     return (out if out_dtype == torch.float32 else out.to(out_dtype)), final_states

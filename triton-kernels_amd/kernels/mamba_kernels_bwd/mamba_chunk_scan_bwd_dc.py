@@ -15,9 +15,8 @@ def _chunk_scan_bwd_dC(prev_states, dA_cumsum, dout, seq_idx=None, C=None, ngrou
     assert prev_states.shape == (batch, nchunks, nheads, headdim, dstate)
     assert dA_cumsum.shape == (batch, nheads, nchunks, chunk_size)
     assert dout.shape == (batch, seqlen, nheads, headdim)
-    if seq_idx is not None:
-        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
     dev = _lib.require_gpu(prev_states, dA_cumsum, dout)
+    seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)
     dout, ds = _lib.strided4(dout)
     cs = [None, 0, 0, 0]
     ddA_prev = None
@@ -31,6 +30,7 @@ def _chunk_scan_bwd_dC(prev_states, dA_cumsum, dout, seq_idx=None, C=None, ngrou
             _lib.lib().ssd_chunk_scan_bwd_dc(*ds, _lib.dtype_code(dout), _lib.f32c(dA_cumsum).data_ptr(),
                                              _lib.f32c(prev_states).data_ptr(), *cs, dC.data_ptr(),
                                              None if ddA_prev is None else ddA_prev.data_ptr(), batch, seqlen,
-                                             nheads, ngroups, headdim, dstate, chunk_size, _lib.stream_ptr(dev)),
+                                             nheads, ngroups, headdim, dstate, chunk_size, *ids,
+                                             _lib.stream_ptr(dev)),
             "ssd_chunk_scan_bwd_dc")
     return dC if C is None else (dC, ddA_prev)

@@ -19,11 +19,10 @@ def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum, B, CB, dout, dstates, D=Non
     assert dA_cumsum.shape == dt.shape
     assert dout.shape == x.shape
     assert dstates.shape == (batch, nchunks, nheads, headdim, dstate)
-    if seq_idx is not None:
-        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
     if D is not None:
         assert D.shape == (nheads, headdim) or D.shape == (nheads,)
     dev = _lib.require_gpu(x, dt, dA_cumsum, B, CB, dout, dstates)
+    seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)
     x, xs = _lib.strided4(x)
     dout, ds = _lib.strided4(dout.to(x.dtype))
     B, bs = _lib.strided4(B.to(x.dtype))
@@ -40,7 +39,7 @@ def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum, B, CB, dout, dstates, D=Non
                 _lib.f32c(dA_cumsum).data_ptr(), *bs, _lib.f32c(dstates).data_ptr(),
                 None if Df is None else Df.data_ptr(), int(D is not None and D.dim() == 2), dx.data_ptr(),
                 dx.stride(0), dx.stride(1), dx.stride(2), ddt.data_ptr(), batch, seqlen, nheads, ngroups, headdim,
-                dstate, chunk_size, _lib.stream_ptr(dev)),
+                dstate, chunk_size, *ids, _lib.stream_ptr(dev)),
             "ssd_chunk_scan_chunk_state_bwd_dx")
     dD = None
     if D is not None:

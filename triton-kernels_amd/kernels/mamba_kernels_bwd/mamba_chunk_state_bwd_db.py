@@ -15,9 +15,8 @@ def _chunk_state_bwd_db(x, dt, dA_cumsum, dstates, seq_idx=None, B=None, ngroups
     assert dt.shape == (batch, nheads, nchunks, chunk_size)
     assert dA_cumsum.shape == dt.shape
     assert dstates.shape == (batch, nchunks, nheads, headdim, dstate)
-    if seq_idx is not None:
-        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
     dev = _lib.require_gpu(x, dt, dA_cumsum, dstates)
+    seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)
     x, xs = _lib.strided4(x)
     bs = [None, 0, 0, 0]
     ddA_cumsum = None
@@ -31,7 +30,7 @@ def _chunk_state_bwd_db(x, dt, dA_cumsum, dstates, seq_idx=None, B=None, ngroups
             _lib.lib().ssd_chunk_state_bwd_db(*xs, _lib.dtype_code(x), _lib.f32c(dt).data_ptr(),
                                               _lib.f32c(dA_cumsum).data_ptr(), _lib.f32c(dstates).data_ptr(), *bs,
                                               dB.data_ptr(), None if ddA_cumsum is None else ddA_cumsum.data_ptr(),
-                                              batch, seqlen, nheads, ngroups, headdim, dstate, chunk_size,
+                                              batch, seqlen, nheads, ngroups, headdim, dstate, chunk_size, *ids,
                                               _lib.stream_ptr(dev)),
             "ssd_chunk_state_bwd_db")
     return dB if B is None else (dB, ddA_cumsum)

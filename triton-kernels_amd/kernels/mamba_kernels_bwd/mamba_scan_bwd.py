@@ -14,10 +14,9 @@ def _chunk_scan_bwd_dstates(C, dA_cumsum, dout, seq_idx=None, dtype=None):
     assert nheads % ngroups == 0
     assert C.shape == (batch, seqlen, ngroups, dstate)
     assert dA_cumsum.shape == (batch, nheads, nchunks, chunk_size)
-    if seq_idx is not None:
-        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
     dev = _lib.require_gpu(C, dA_cumsum, dout)
     dtype = C.dtype if dtype is None else dtype
+    seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)
     dout, ds = _lib.strided4(dout)
     if C.dtype != dout.dtype:
         C = C.to(dout.dtype)
@@ -27,6 +26,6 @@ def _chunk_scan_bwd_dstates(C, dA_cumsum, dout, seq_idx=None, dtype=None):
         _lib.check(
             _lib.lib().ssd_chunk_scan_bwd_dstates(*cs, *ds, _lib.dtype_code(dout), _lib.f32c(dA_cumsum).data_ptr(),
                                                   out.data_ptr(), batch, seqlen, nheads, ngroups, headdim, dstate,
-                                                  chunk_size, _lib.stream_ptr(dev)),
+                                                  chunk_size, *ids, _lib.stream_ptr(dev)),
             "ssd_chunk_scan_bwd_dstates")
     return out if dtype == torch.float32 else out.to(dtype)

@@ -14,12 +14,16 @@ def _state_passing_bwd(states, dA_chunk_cumsum, dout, dfinal_states=None, seq_id
     batch, nchunks, nheads, dim = states.shape
     assert dA_chunk_cumsum.shape == (batch, nheads, nchunks)
     assert dout.shape == (batch, nchunks, nheads, dim)
-    if seq_idx is not None:
-        raise NotImplementedError("seq_idx is not supported by the HIP SSD kernels")
     if dfinal_states is not None:
         assert dfinal_states.shape == (batch, nheads, dim)
     dev = _lib.require_gpu(states, dA_chunk_cumsum, dout)
     lib = _lib.lib()
+    seqlen = 0
+    if seq_idx is not None:
+        assert chunk_size is not None
+        seqlen = seq_idx.shape[-1]
+        assert nchunks == (seqlen + chunk_size - 1) // chunk_size
+    seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)
     st, do = _lib.f32c(states), _lib.f32c(dout)
     da = dA_chunk_cumsum if dA_chunk_cumsum.dtype == torch.float32 else dA_chunk_cumsum.float()
     dfin = None if dfinal_states is None else _lib.f32c(dfinal_states)
@@ -33,7 +37,8 @@ def _state_passing_bwd(states, dA_chunk_cumsum, dout, dfinal_states=None, seq_id
             lib.ssd_state_passing_bwd(st.data_ptr(), da.data_ptr(), da.stride(0), da.stride(1), da.stride(2),
                                       do.data_ptr(), None if dfin is None else dfin.data_ptr(), dstates.data_ptr(),
                                       ddA.data_ptr(), None if dinit is None else dinit.data_ptr(), ws.data_ptr(),
-                                      nbytes, batch, nchunks, nheads, dim, _lib.stream_ptr(dev)),
+                                      nbytes, batch, nchunks, nheads, dim, *ids, seqlen, chunk_size or 0,
+                                      _lib.stream_ptr(dev)),
             "ssd_state_passing_bwd")
     out_dtype = dstates_dtype if dstates_dtype is not None else dout.dtype
     if out_dtype != torch.float32:
