@@ -235,6 +235,10 @@ size_t ema_seq_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen
  *     (the reference forms A = log(1-p) and X = p*x in torch first,
  *      kernels/benchmarks/ema_bench.py:135-136, or runs the three kernels of
  *      ema_scan_combined, kernels/ema.py:370-375)
+ * Packed sequences (what the reference's seq_idx arguments ask for, e.g.
+ * kernels/ema_chunk_state.py:500-604): the state is dropped at the first position t of a new
+ * sequence when A[t] = -inf (log-decay form) or when p[t] carries a set sign bit, i.e. is given
+ * as -p[t], -0.0 for p[t] = 0 (probability form; then y[t] = p[t] * x[t]).
  * coef is float32, addressed like A above.  init (N,T) float32, may be NULL = zero: the state
  * before the first position, which the reference's launchers reject
  * (kernels/ema_kernels/ema_state_pass.py:129-130).  final_state (N,T), may be NULL: the state
@@ -253,6 +257,8 @@ int ema_seq_fwd(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t
  * gradient reaching final_state:
  *   EMA_FORM_LOG_DECAY:   dx[t] = r[t],        dcoef[t] = a[t] * <r[t], y[t-1]>
  *   EMA_FORM_PROBABILITY: dx[t] = p[t] * r[t], dcoef[t] = <r[t], x[t] - y[t-1]>
+ * (at a position whose p carries the sign bit that marks a sequence start, y[t-1] counts as 0 and
+ * dcoef[t] is the derivative with respect to the stored value -p[t], i.e. -<r[t], x[t]>)
  * (the reference leaves dP = -dA * exp(A) commented out, kernels/tests/ema_bwd/_ema_full_bwd.py:128-130,
  * and rearranges dA from (b,c,q) to (b,l) in torch, :71).  dcoef is float32 in the layout of
  * coef, given by its own strides; dinit (N,T) float32, may be NULL, receives a[0] * r[0], the

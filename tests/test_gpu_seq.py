@@ -183,3 +183,55 @@ def test_seq_packed_sequences(dtype, device):
     check_close("y", y, y_ref, dtype)
     check_close("dx", xg.grad, dx_ref, dtype)
     check_close("dA", Ag.grad, dA_ref, dtype)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+def test_seq_packed_sequences_probability_form(dtype, device):
+    """seq_idx in the probability form (a set sign bit on p at sequence starts): forward, the
+    gradients of x and p, initial state (reaches the first sequence only), final state (the last
+    sequence's) and the gradients through both, against each sequence scanned alone.  One
+    sequence starts with p = 0 (encoded as -0.0) and one with p = 1."""
+    from kernels.ema_seq import ema_seq_scan
+
+    B, L, T = 2, 1000, 72
+    announce(f"seq packed sequences, probability form {dtype}")
+    g = torch.Generator().manual_seed(23)
+    x = torch.randn(B, L, T, generator=g).to(dtype)
+    p = torch.sigmoid(-(torch.randn(B, L, generator=g) + 2.0))
+    p[0, 128] = 0.0
+    p[1, 257] = 1.0
+    dy = torch.randn(B, L, T, generator=g).to(dtype)
+    init = torch.randn(B, T, generator=g)
+    dfin = torch.randn(B, T, generator=g)
+    cuts = [[0, 3, 128, 131, 640, 1000], [0, 255, 256, 257, 900, 1000]]
+    seq_idx = torch.zeros(B, L, dtype=torch.int32)
+    for bi, cs in enumerate(cuts):
+        for k in range(len(cs) - 1):
+            seq_idx[bi, cs[k]:cs[k + 1]] = k
+    xg, pg = x.to(device).requires_grad_(), p.to(device).requires_grad_()
+    ig = init.to(device).requires_grad_()
+    y, fin = ema_seq_scan(pg, xg, "probability", initial_states=ig, return_final_states=True,
+                          seq_idx=seq_idx.to(device))
+    ((y.float() * dy.to(device).float()).sum() + (fin * dfin.to(device)).sum()).backward()
+    torch.cuda.synchronize()
+    y_ref, dx_ref, dp_ref = torch.zeros(B, L, T), torch.zeros(B, L, T), torch.zeros(B, L)
+    fin_ref, dinit_ref = torch.zeros(B, T), torch.zeros(B, T)
+    for bi, cs in enumerate(cuts):
+        for k in range(len(cs) - 1):
+            sl = slice(cs[k], cs[k + 1])
+            first, last = k == 0, k == len(cs) - 2
+            one = lambda t: t[bi:bi + 1, sl].float()
+            i0 = init[bi:bi + 1] if first else None
+            df = dfin[bi:bi + 1] if last else None
+            ys, fs = O.ema_seq_loop(one(x), p[bi:bi + 1, sl], "probability", i0)
+            dxs, dps, dis = O.ema_seq_loop_bwd(one(dy), one(x), p[bi:bi + 1, sl], "probability", i0, df)
+            y_ref[bi, sl], dx_ref[bi, sl], dp_ref[bi, sl] = ys[0], dxs[0], dps[0]
+            if first:
+                dinit_ref[bi] = dis[0]
+            if last:
+                fin_ref[bi] = fs[0]
+    check_close("y", y, y_ref, dtype)
+    check_close("final state", fin, fin_ref, dtype)
+    check_close("dx", xg.grad, dx_ref, dtype)
+    check_close("dp", pg.grad, dp_ref, dtype)
+    check_close("dinit", ig.grad, dinit_ref, dtype)

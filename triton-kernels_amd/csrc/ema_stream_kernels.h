@@ -12,7 +12,12 @@ namespace ema {
 // are scanned across the wave with DPP.  With prob != 0 the input holds probabilities p and
 // the log-decay is log(1 - p).
 // ------------------------------------------------------------------------------------
-__device__ __forceinline__ float cumsum_term(float v, int prob) { return prob ? log1pf(-v) : v; }
+// A probability with its sign bit set marks the first position of a packed sequence: nothing
+// survives it, a log-decay of -inf.
+__device__ __forceinline__ float cumsum_term(float v, int prob) {
+  if (!prob) return v;
+  return (__float_as_uint(v) >> 31) ? -INFINITY : log1pf(-v);
+}
 
 __global__ __launch_bounds__(256) void cumsum_kernel(const float* __restrict__ A,
                                                      SeqStrides sa, float* __restrict__ cs,

@@ -24,7 +24,11 @@
 // Two forms of the recurrence (template flag XP):
 //   log-decay form   y = a*y + x,        a = exp(min(A, 0));   gradients dx = r, dA = a*<r, y_prev>
 //   probability form y = (1-p)*y + p*x,  evaluated as y + p*(x - y);  dx = p*r, dp = <r, x - y_prev>
-// with r the reverse scan of dy.  The state before the first row may be given (init) and the
+// with r the reverse scan of dy.  In the probability form a set sign bit on p (-p, or -0.0 for
+// p = 0) marks the first position of a packed sequence: the state is dropped there, y = p*x,
+// and the gradient returned for such a coefficient is that of the encoded value, -<r, x>.  (In
+// the log-decay form the same is a decay of exp(-inf) = 0 and needs no flag.)
+// The state before the first row may be given (init) and the
 // gradient reaching the state after the last row (dfinal); the backward then also returns the
 // gradient of the initial state, a[0]*r[0].
 #pragma once
@@ -150,14 +154,22 @@ __device__ __forceinline__ void tile_decays(float* a, const float* __restrict__ 
   }
 }
 
+// Probability form: the sign bit of a coefficient marks the first position of a packed sequence.
+__device__ __forceinline__ bool coef_resets(float coef) { return (__float_as_uint(coef) >> 31) != 0u; }
+
 // One step of the forward recurrence, and the factor by which the step scales the state.
 template <bool XP>
 __device__ __forceinline__ float tile_step(float coef, float s, float x) {
-  return XP ? fmaf(coef, x - s, s) : fmaf(coef, s, x);
+  if (XP) {
+    const float s0 = coef_resets(coef) ? 0.f : s;
+    return fmaf(fabsf(coef), x - s0, s0);
+  }
+  return fmaf(coef, s, x);
 }
 template <bool XP>
 __device__ __forceinline__ float tile_keep(float coef) {
-  return XP ? 1.f - coef : coef;
+  if (XP) return coef_resets(coef) ? 0.f : 1.f - coef;
+  return coef;
 }
 
 template <bool REV, int BN>
@@ -441,14 +453,15 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
         for (int e = 0; e < CPL; ++e) {
           // r holds a[i+1] * dx[i+1] on entry (the carried state for the last row)
           const float d = row_get<T, NW>(dr[i], e) + r[e];
-          const float yp = i > 0 ? yv[i - 1][e] : E[e];
+          float yp = i > 0 ? yv[i - 1][e] : E[e];
+          if (XP && coef_resets(pc[i])) yp = 0.f;
           dot = fmaf(d, XP ? row_get<T, NW>(xr[i], e) - yp : yp, dot);
           r[e] = d;
         }
         if (XP) {
           float o[CPL];
 #pragma unroll
-          for (int e = 0; e < CPL; ++e) o[e] = pc[i] * r[e];
+          for (int e = 0; e < CPL; ++e) o[e] = fabsf(pc[i]) * r[e];
           if (i < nrows && cok) row_store<NW>(g + (int64_t)i * sdx.sl + off, row_pack<T, CPL, NW>(o));
         } else {
           if (i < nrows && cok) row_store<NW>(g + (int64_t)i * sdx.sl + off, row_pack<T, CPL, NW>(r));
@@ -457,6 +470,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
         for (int e = 0; e < CPL; ++e) r[e] *= a[i];
         dot = wave_sum(dot);
         if (!XP) dot *= a[i];
+        else if (coef_resets(pc[i])) dot = -dot;  // derivative with respect to the encoded value -p
         if (lane == i) dA = dot;
       }
       if (lane < RPL)

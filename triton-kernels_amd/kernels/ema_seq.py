@@ -130,12 +130,23 @@ def pack_log_decay(A, seq_idx):
     return torch.where(start, torch.full_like(A, float("-inf")), A)
 
 
+def pack_probability(p, seq_idx):
+    """Probabilities of several sequences packed along the length axis: the kernels drop the
+    state at a position whose probability carries a set sign bit, so p is negated (0 becomes
+    -0.0) at the first position of each new sequence.  Autograd through the negation returns the
+    gradient with respect to p itself."""
+    assert seq_idx.shape == p.shape[:2], "seq_idx must be (batch, seqlen)"
+    start = torch.zeros_like(seq_idx, dtype=torch.bool)
+    start[:, 1:] = seq_idx[:, 1:] != seq_idx[:, :-1]
+    if p.dim() == 3:
+        start = start[..., None]
+    return torch.where(start, -p, p)
+
+
 def ema_seq_scan(coef, x, form="log_decay", initial_states=None, return_final_states=False, seq_idx=None):
     """Differentiable in coef, x and initial_states (and through the final states).  seq_idx
-    (batch, L) marks packed sequences (log-decay form only): the state is reset where it changes."""
+    (batch, L) marks packed sequences: the state is reset where it changes."""
     if seq_idx is not None:
-        if form != "log_decay":
-            raise NotImplementedError("seq_idx needs the log-decay form (a reset is a decay of 0)")
-        coef = pack_log_decay(coef, seq_idx)
+        coef = pack_log_decay(coef, seq_idx) if form == "log_decay" else pack_probability(coef, seq_idx)
     y, final = EMASeqFn.apply(coef, x, initial_states, form)
     return (y, final) if return_final_states else y
