@@ -65,6 +65,17 @@ __device__ __forceinline__ bool chunk_keeps_state(SeqIdx s, int64_t b, int c, in
   return cur == before;
 }
 
+// Workgroups are dealt to the 8 XCDs round-robin by their index, and each XCD has its own L2.
+// This maps the hardware index to a logical one whose consecutive values run on the same XCD,
+// so that workgroups which share operands (the heads of a group, the row tiles of a chunk) find
+// them in that L2 instead of fetching them once per XCD.  A bijection on [0, nblocks).
+__device__ __forceinline__ int xcd_local_index(int bid, int nblocks) {
+  constexpr int kXcds = 8;
+  const int per = nblocks / kXcds;
+  if (bid >= per * kXcds) return bid;  // the tail that does not fill a round keeps its place
+  return (bid % kXcds) * per + bid / kXcds;
+}
+
 // ------------------------------------------------------------------ operand fragments
 // Both return, for lane l, EPL = Vec16<T>::N consecutive contraction indices starting at
 // k0 + EPL * (l / 32), for row or column (l % 32) of the 32-wide block: the register layout
@@ -209,9 +220,10 @@ __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
   T* xs = reinterpret_cast<T*>(smem);
   T* bs = xs + KT * PX;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int h = blockIdx.x % nh;
-  const int c = (blockIdx.x / nh) % C;
-  const int64_t b = blockIdx.x / (nh * C);
+  const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
+  const int h = bid % nh;
+  const int c = (bid / nh) % C;
+  const int64_t b = bid / (nh * C);
   const int limit = min(Q, L - c * Q);
   const float* dAp = dA_cs + ((b * nh + h) * C + c) * (int64_t)Q;
   const float* dtp = dt + ((b * nh + h) * C + c) * (int64_t)Q;
@@ -426,7 +438,11 @@ __global__ __launch_bounds__(256) void ssd_row_cumsum_kernel(float* __restrict__
 // In a packed batch w_m is 0 unless the id of m equals the id of the chunk's last position
 // (MODE 0) or of the previous chunk's last position (MODE 1).
 // a is read row-major straight from global memory; s is staged in LDS (rounded to T) and
-// contracted along its rows.
+// contracted along its rows.  The products are formed transposed, d_h^T = s^T a^T, so that in
+// the accumulator a lane owns one row m and sixteen columns n: the row weight is one value per
+// lane and the sum over n for r_h is in-register adds, one exchange between the halves of the
+// wave and one between two waves through LDS (summing the untransposed accumulator across
+// lanes took as long as everything else in the kernel).
 // ------------------------------------------------------------------------------------
 template <typename T, int P, int N>
 struct GroupSmem {
@@ -448,10 +464,11 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
   float* wrow = rs + 4 * 64;                                           // this head's row weights
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
-  const int mt = blockIdx.x % mtiles;
-  const int g = (blockIdx.x / mtiles) % ngroups;
-  const int c = (blockIdx.x / (mtiles * ngroups)) % C;
-  const int64_t b = blockIdx.x / ((int64_t)mtiles * ngroups * C);
+  const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
+  const int mt = bid % mtiles;
+  const int g = (bid / mtiles) % ngroups;
+  const int c = (bid / (mtiles * ngroups)) % C;
+  const int64_t b = bid / ((int64_t)mtiles * ngroups * C);
   const int limit = min(Q, L - c * Q);
   const int m0 = 64 * mt;
 
@@ -472,17 +489,17 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
     mi[i] = j & 1;
     ni[i] = j >> 1;
   }
-  // bc in the accumulator layout (float), once per workgroup
+  // bc in the (transposed) accumulator layout: this lane's row m, columns n of each block
   float bcv[BPW][16];
   const bool want_ddA = bc != nullptr;
   if (want_ddA) {
     const T* bcg = bc + b * sbc.sb + (int64_t)c * Q * sbc.sl + g * sbc.sh;
+    const int m = m0 + 32 * mi[0] + l32;
 #pragma unroll
     for (int i = 0; i < BPW; ++i)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int m = m0 + 32 * mi[i] + acc_row(v, lane);
-        const float t = (float)bcg[(int64_t)min(m, limit - 1) * sbc.sl + 32 * ni[i] + l32];
+        const float t = (float)bcg[(int64_t)min(m, limit - 1) * sbc.sl + 32 * ni[i] + acc_row(v, lane)];
         bcv[i][v] = m < limit ? t : 0.f;
       }
   }
@@ -532,36 +549,29 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
       if (m_lane >= limit) av[ks].zero();
 #pragma unroll
       for (int i = 0; i < BPW; ++i)
-        mma_group(av[ks], frag_cols(St, S::PS, KG * ks, 32 * ni[i], lane), acc[i]);
+        mma_group(frag_cols(St, S::PS, KG * ks, 32 * ni[i], lane), av[ks], acc[i]);  // [n][m]
     }
+    {
+      const float w = wrow[32 * mi[0] + l32];  // the wave's blocks share their rows m
+      float part = 0.f;
 #pragma unroll
-    for (int i = 0; i < BPW; ++i) {
-      float r16[16];
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const float d = acc[i][v] * wrow[32 * mi[i] + acc_row(v, lane)];
-        total[i][v] += d;
-        r16[v] = d * (want_ddA ? bcv[i][v] : 0.f);
-      }
-      if (want_ddA) {
-        // rows of this block over its 32 columns, then over the column blocks through LDS
+      for (int i = 0; i < BPW; ++i)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const float t = half_wave_sum(r16[v]);
-          if (l32 == 31) {
-            float* dst = rs + wave * 64 + 32 * mi[i] + acc_row(v, lane);
-            if (i == 0) *dst = t;
-            else *dst += t;  // the wave's second block covers the same rows
-          }
+          total[i][v] = fmaf(acc[i][v], w, total[i][v]);
+          if (want_ddA) part = fmaf(acc[i][v], bcv[i][v], part);
         }
+      if (want_ddA) {
+        part += __shfl_xor(part, 32);  // the halves of the wave hold different columns n of row m
+        if (half == 0) rs[wave * 32 + l32] = part * w;
       }
     }
     __syncthreads();
     if (want_ddA && tid < 64) {
-      // row block tid / 32 belongs to the waves w0 = tid / 32 and w0 + 2 (a wave's blocks share
-      // their rows and differ in their columns)
+      // rows 32 * (tid / 32) .. belong to the waves w0 = tid / 32 and w0 + 2, which own different
+      // columns of them
       const int w0 = tid >> 5;
-      const float r = rs[w0 * 64 + tid] + rs[(w0 + 2) * 64 + tid];
+      const float r = rs[w0 * 32 + (tid & 31)] + rs[(w0 + 2) * 32 + (tid & 31)];
       const int m = m0 + tid;
       float* o = ddA + chunk * Q;
       if (MODE == 0) {
@@ -573,14 +583,17 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
     }
     // the next head's staging overwrites St; rs is rewritten only after the next barrier
   }
+  // total is [n][m] per block: a lane writes four adjacent n of its row m at a time
   float* og = out + (b * L + (int64_t)c * Q) * ngroups * N + (int64_t)g * N;
+  const int m = m0 + 32 * mi[0] + l32;
+  if (m < limit) {
 #pragma unroll
-  for (int i = 0; i < BPW; ++i)
+    for (int i = 0; i < BPW; ++i)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int m = m0 + 32 * mi[i] + acc_row(v, lane);
-      if (m < limit) og[(int64_t)m * ngroups * N + 32 * ni[i] + l32] = total[i][v];
-    }
+      for (int v = 0; v < 16; v += 4)
+        *reinterpret_cast<float4*>(og + (int64_t)m * ngroups * N + 32 * ni[i] + acc_row(v, lane)) =
+            make_float4(total[i][v], total[i][v + 1], total[i][v + 2], total[i][v + 3]);
+  }
 }
 
 // ------------------------------------------------------------------------------------
@@ -603,9 +616,10 @@ __global__ __launch_bounds__(256) void ssd_bmm_kernel(const T* __restrict__ a, S
   T* as = reinterpret_cast<T*>(smem);
   T* bs = as + 64 * PK;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int tn = blockIdx.x % tiles;
-  const int tm = (blockIdx.x / tiles) % tiles;
-  const int64_t bcg = blockIdx.x / (tiles * tiles);
+  const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
+  const int tn = bid % tiles;
+  const int tm = (bid / tiles) % tiles;
+  const int64_t bcg = bid / (tiles * tiles);
   const int g = (int)(bcg % ngroups);
   const int c = (int)((bcg / ngroups) % C);
   const int64_t b = bcg / ((int64_t)ngroups * C);
@@ -673,10 +687,11 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(
   float* sm = reinterpret_cast<float*>(smem + S::kBytes - 64 * sizeof(float));  // exp(dA_m)
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int mt = blockIdx.x % mtiles;
-  const int h = (blockIdx.x / mtiles) % nh;
-  const int c = (blockIdx.x / (mtiles * nh)) % C;
-  const int64_t b = blockIdx.x / ((int64_t)mtiles * nh * C);
+  const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
+  const int mt = bid % mtiles;
+  const int h = (bid / mtiles) % nh;
+  const int c = (bid / (mtiles * nh)) % C;
+  const int64_t b = bid / ((int64_t)mtiles * nh * C);
   const int limit = min(Q, L - c * Q);
   const int m0 = 64 * mt;
   if (m0 >= limit) return;
@@ -853,10 +868,11 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
   float* sm = dtk + ST;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
-  const int st = blockIdx.x % stiles;
-  const int h = (blockIdx.x / stiles) % nh;
-  const int c = (blockIdx.x / (stiles * nh)) % C;
-  const int64_t b = blockIdx.x / ((int64_t)stiles * nh * C);
+  const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
+  const int st = bid % stiles;
+  const int h = (bid / stiles) % nh;
+  const int c = (bid / (stiles * nh)) % C;
+  const int64_t b = bid / ((int64_t)stiles * nh * C);
   const int limit = min(Q, L - c * Q);
   const int m0 = ST * st;
   if (m0 >= limit) return;
@@ -1034,10 +1050,11 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
   float* sm = reinterpret_cast<float*>(smem + S::kBytes - 64 * sizeof(float));
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int mt = blockIdx.x % mtiles;
-  const int h = (blockIdx.x / mtiles) % nh;
-  const int c = (blockIdx.x / (mtiles * nh)) % C;
-  const int64_t b = blockIdx.x / ((int64_t)mtiles * nh * C);
+  const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
+  const int mt = bid % mtiles;
+  const int h = (bid / mtiles) % nh;
+  const int c = (bid / (mtiles * nh)) % C;
+  const int64_t b = bid / ((int64_t)mtiles * nh * C);
   const int limit = min(Q, L - c * Q);
   const int m0 = 64 * mt;
   const int64_t chunk = (b * nh + h) * C + c;
@@ -1199,9 +1216,10 @@ __global__ __launch_bounds__(256) void ssd_ddA_causal_kernel(
   float* dts = dAs + 256;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
-  const int h = blockIdx.x % nh;
-  const int c = (blockIdx.x / nh) % C;
-  const int64_t b = blockIdx.x / ((int64_t)nh * C);
+  const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
+  const int h = bid % nh;
+  const int c = (bid / nh) % C;
+  const int64_t b = bid / ((int64_t)nh * C);
   const int limit = min(Q, L - c * Q);
   const int MB = Q / 32;
   const int64_t chunk = (b * nh + h) * C + c;
@@ -1323,10 +1341,11 @@ __global__ __launch_bounds__(256, 3) void ssd_chunk_scan_bwd_dx_wide_kernel(
   float* sm = dAk + 2 * ST;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
-  const int st = blockIdx.x % stiles;
-  const int h = (blockIdx.x / stiles) % nh;
-  const int c = (blockIdx.x / (stiles * nh)) % C;
-  const int64_t b = blockIdx.x / ((int64_t)stiles * nh * C);
+  const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
+  const int st = bid % stiles;
+  const int h = (bid / stiles) % nh;
+  const int c = (bid / (stiles * nh)) % C;
+  const int64_t b = bid / ((int64_t)stiles * nh * C);
   const int limit = min(Q, L - c * Q);
   const int m0 = ST * st;
   const int64_t chunk = (b * nh + h) * C + c;
