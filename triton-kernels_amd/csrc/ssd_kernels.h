@@ -125,22 +125,36 @@ __device__ __forceinline__ void stage_rows(T* tile, const T* __restrict__ g, int
                                            int limit, int tid, F scale) {
   constexpr int EPL = Vec16<T>::N, VPR = COLS / EPL, P = Tile<T>::pitch(COLS);
   static_assert((ROWS * VPR) % 256 == 0, "tile must split evenly over 256 threads");
+  constexpr int CNT = ROWS * VPR / 256, GRP = CNT < 8 ? CNT : 8;
+  static_assert(CNT % GRP == 0, "load groups must divide the tile");
+  // Up to eight loads go out before the first LDS store of a group (the compiler otherwise tends
+  // to wait for each load in turn to save registers).  They are unconditional, from rows clamped
+  // into the sequence (limit >= 1): a load inside a branch would have to complete before the
+  // next one is issued.
 #pragma unroll
-  for (int i = 0; i < ROWS * VPR / 256; ++i) {
-    const int idx = tid + 256 * i;
-    const int r = idx / VPR, cv = (idx % VPR) * EPL;
-    // The load is unconditional, from a row clamped into the sequence (limit >= 1): a load inside
-    // a branch would have to complete before the next one is issued.
-    const bool in = row0 + r < limit;
-    const int row = in ? row0 + r : limit - 1;
-    Vec16<T> v = load16(g + (int64_t)row * row_stride + cv);
-    if constexpr (!std::is_same<F, NoScale>::value) {
-      const float s = scale(row);
+  for (int i0 = 0; i0 < CNT; i0 += GRP) {
+    Vec16<T> v[GRP];
 #pragma unroll
-      for (int e = 0; e < EPL; ++e) v.set(e, v.get(e) * s);
+    for (int i = 0; i < GRP; ++i) {
+      const int idx = tid + 256 * (i0 + i);
+      const int r = idx / VPR, cv = (idx % VPR) * EPL;
+      const int row = row0 + r < limit ? row0 + r : limit - 1;
+      v[i] = load16(g + (int64_t)row * row_stride + cv);
     }
-    if (!in) v.zero();
-    store16(tile + r * P + cv, v);
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < GRP; ++i) {
+      const int idx = tid + 256 * (i0 + i);
+      const int r = idx / VPR, cv = (idx % VPR) * EPL;
+      const bool in = row0 + r < limit;
+      if constexpr (!std::is_same<F, NoScale>::value) {
+        const float s = scale(in ? row0 + r : limit - 1);
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) v[i].set(e, v[i].get(e) * s);
+      }
+      if (!in) v[i].zero();
+      store16(tile + r * P + cv, v[i]);
+    }
   }
 }
 // ------------------------------------------------------------------------------------
@@ -946,22 +960,31 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
       const float am = dAp[m0 + mloc];
       const float* cbrow = cbg + (int64_t)(m0 + mloc) * Q + k0 + EPL * half;
       const int kend = diag ? mrow[mb] + 32 : ST;
-      for (int kk = 0; kk < kend; kk += KG) {
-        float w[EPL];
+      // NS steps at a time (the step count is even): their cb fragments are all requested before
+      // the first is used, so the wave waits for memory once per NS steps.  Only where the
+      // registers allow it without losing a wave per SIMD.
+      constexpr int NS = (P == 64 && sizeof(T) == 2) ? 2 : 1;
+      for (int kk0 = 0; kk0 < kend; kk0 += NS * KG) {
+        float w[NS][EPL];
 #pragma unroll
-        for (int e = 0; e < EPL; e += 4) {
-          const float4 c4 = *reinterpret_cast<const float4*>(cbrow + kk + e);
-          w[e] = c4.x, w[e + 1] = c4.y, w[e + 2] = c4.z, w[e + 3] = c4.w;
+        for (int u = 0; u < NS; ++u)
+#pragma unroll
+          for (int e = 0; e < EPL; e += 4) {
+            const float4 c4 = *reinterpret_cast<const float4*>(cbrow + kk0 + KG * u + e);
+            w[u][e] = c4.x, w[u][e + 1] = c4.y, w[u][e + 2] = c4.z, w[u][e + 3] = c4.w;
+          }
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+          const int kk = kk0 + KG * u, kb = kk + EPL * half;
+          Vec16<T> a;
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) {
+            const float f = w[u][e] * __expf(fminf(am - dAk[kb + e], 0.f)) * dtk[kb + e];
+            a.set(e, (diag && kb + e > mloc) ? 0.f : f);
+          }
+#pragma unroll
+          for (int pb = 0; pb < PB; ++pb) mma_group(a, frag_cols(Xs, S::PX, kk, 32 * pb, lane), acc[mb][pb]);
         }
-        const int kb = kk + EPL * half;
-        Vec16<T> a;
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) {
-          const float f = w[e] * __expf(fminf(am - dAk[kb + e], 0.f)) * dtk[kb + e];
-          a.set(e, (diag && kb + e > mloc) ? 0.f : f);
-        }
-#pragma unroll
-        for (int pb = 0; pb < PB; ++pb) mma_group(a, frag_cols(Xs, S::PX, kk, 32 * pb, lane), acc[mb][pb]);
       }
       if (diag && D) {
 #pragma unroll
@@ -1325,7 +1348,7 @@ __global__ __launch_bounds__(256) void ssd_ddA_causal_kernel(
 // one 4-byte load per k that is contiguous across the 32 lanes of a half-wave.
 // ------------------------------------------------------------------------------------
 template <typename T, int P, int N>
-__global__ __launch_bounds__(256, 3) void ssd_chunk_scan_bwd_dx_wide_kernel(
+__global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_wide_kernel(
     const float* __restrict__ cb, const T* __restrict__ x, Strides3 sx, const T* __restrict__ dout, Strides3 sd,
     const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Bm, Strides3 sB,
     const float* __restrict__ dstates, const float* __restrict__ D, int d_has_hdim, T* __restrict__ dx,
