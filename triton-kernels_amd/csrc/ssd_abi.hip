@@ -538,4 +538,11 @@ int ssd_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t 
   return launched();
 }
 
+#ifdef SSD_TIMING
+// Development aid, only in builds with -DSSD_TIMING: installs the per-workgroup timestamp buffer.
+int ssd_debug_set_timing(void* buf) {
+  return hipMemcpyToSymbol(HIP_SYMBOL(ssd::g_ssd_timing), &buf, sizeof(buf)) == hipSuccess ? 0 : -6;
+}
+#endif
+
 }  // extern "C"

@@ -30,6 +30,19 @@ using ema::store16;
 using ema::Vec16;
 using ema::wave_inclusive_scan;
 
+#ifdef SSD_TIMING
+// Development aid: per-workgroup phase timestamps into a global buffer (never built into the library).
+__device__ long long* g_ssd_timing = nullptr;
+#define SSD_TSTAMP(slot)                                                                              \
+  do {                                                                                                \
+    if (threadIdx.x == 0 && g_ssd_timing) g_ssd_timing[(int64_t)blockIdx.x * 8 + (slot)] = wall_clock64(); \
+  } while (0)
+#else
+#define SSD_TSTAMP(slot) \
+  do {                   \
+  } while (0)
+#endif
+
 // Element strides of a (batch, position, head-or-group) tensor whose last axis is dense.
 struct Strides3 {
   int64_t sb, sl, sh;
@@ -233,7 +246,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* xs = reinterpret_cast<T*>(smem);
   T* bs = xs + KT * PX;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
   const int h = bid % nh;
   const int c = (bid / nh) % C;
@@ -477,7 +490,7 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
   float* rs = reinterpret_cast<float*>(smem + P * S::PS * sizeof(T));  // [4 waves][64 rows]
   float* wrow = rs + 4 * 64;                                           // this head's row weights
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31, half = lane >> 5;
   const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
   const int mt = bid % mtiles;
   const int g = (bid / mtiles) % ngroups;
@@ -629,7 +642,7 @@ __global__ __launch_bounds__(256) void ssd_bmm_kernel(const T* __restrict__ a, S
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* as = reinterpret_cast<T*>(smem);
   T* bs = as + 64 * PK;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
   const int tn = bid % tiles;
   const int tm = (bid / tiles) % tiles;
@@ -700,7 +713,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(
   float* Os = reinterpret_cast<float*>(smem);
   float* sm = reinterpret_cast<float*>(smem + S::kBytes - 64 * sizeof(float));  // exp(dA_m)
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
   const int mt = bid % mtiles;
   const int h = (bid / mtiles) % nh;
@@ -879,9 +892,10 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
   float* Os = reinterpret_cast<float*>(smem);
   float* dAk = reinterpret_cast<float*>(smem + S::kMain);
   float* dtk = dAk + ST;
-  float* sm = dtk + ST;
+  float* sm = dtk + ST;  // exp(dA_m) of the carried-state term, then
+  float* fk = sm;        // the per-position factor of the causal term
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31, half = lane >> 5;
   const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
   const int st = bid % stiles;
   const int h = (bid / stiles) % nh;
@@ -908,6 +922,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
 #pragma unroll
     for (int pb = 0; pb < PB; ++pb) zero_acc(acc[mb][pb]);
 
+  SSD_TSTAMP(0);
   // ---- phase A: C . prev, scaled by exp(dA_m)
   {
     constexpr int VPR = N / 4;
@@ -926,6 +941,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
     sm[tid] = live ? __expf(dAp[m0 + tid]) : 0.f;
   }
   __syncthreads();
+  SSD_TSTAMP(1);
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {
     const int m = m0 + mrow[mb] + l32;
@@ -946,13 +962,25 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
   }
 
   // ---- phase B: the k super-tiles up to the diagonal one
+  SSD_TSTAMP(2);
   __syncthreads();  // the x tile takes the place of the carried state
+  SSD_TSTAMP(3);
   for (int kt = 0; kt <= st; ++kt) {
     const int k0 = ST * kt;
     stage_rows<T, ST, P>(Xs, xg, sx.sl, k0, limit, tid, NoScale());
-    dAk[tid] = dAp[k0 + tid];
-    dtk[tid] = dtp[k0 + tid];
+    {
+      // Below the diagonal the weight of (m, k) is split at the last position r of k's group of
+      // 32: exp(dA_m - dA_r) is one exponential per row and group, exp(dA_r - dA_k) * dt_k one
+      // per position k, shared by all rows.  Each exponent is clamped at 0 like the whole is in
+      // the reference; for a dA_cumsum that is monotone inside the chunk (A of one sign,
+      // dt >= 0) the product is the reference's clamped exponential.
+      const float ak = dAp[k0 + tid], ar = dAp[k0 + (tid | 31)], tk = dtp[k0 + tid];
+      dAk[tid] = ak;
+      dtk[tid] = tk;
+      fk[tid] = __expf(fminf(ar - ak, 0.f)) * tk;
+    }
     __syncthreads();
+    SSD_TSTAMP(4);
     const bool diag = kt == st;
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) {
@@ -973,14 +1001,23 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
             const float4 c4 = *reinterpret_cast<const float4*>(cbrow + kk0 + KG * u + e);
             w[u][e] = c4.x, w[u][e + 1] = c4.y, w[u][e + 2] = c4.z, w[u][e + 3] = c4.w;
           }
+        // the group of 32 positions that holds the diagonal takes the exact, masked form
+        const int grp_last = (kk0 & ~31) + 31;
+        const bool exact = diag && grp_last >= mrow[mb];
+        const float gm = __expf(fminf(am - dAk[grp_last], 0.f));
 #pragma unroll
         for (int u = 0; u < NS; ++u) {
           const int kk = kk0 + KG * u, kb = kk + EPL * half;
           Vec16<T> a;
+          if (exact) {
 #pragma unroll
-          for (int e = 0; e < EPL; ++e) {
-            const float f = w[u][e] * __expf(fminf(am - dAk[kb + e], 0.f)) * dtk[kb + e];
-            a.set(e, (diag && kb + e > mloc) ? 0.f : f);
+            for (int e = 0; e < EPL; ++e) {
+              const float f = w[u][e] * __expf(fminf(am - dAk[kb + e], 0.f)) * dtk[kb + e];
+              a.set(e, kb + e > mloc ? 0.f : f);
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) a.set(e, w[u][e] * fk[kb + e] * gm);
           }
 #pragma unroll
           for (int pb = 0; pb < PB; ++pb) mma_group(a, frag_cols(Xs, S::PX, kk, 32 * pb, lane), acc[mb][pb]);
@@ -997,8 +1034,10 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
         }
       }
     }
+    SSD_TSTAMP(5);
     __syncthreads();
   }
+  SSD_TSTAMP(6);
 
   // ---- phase C: each wave moves its two blocks through its own staging area
   float* mine = Os + wave * 32 * S::PO;
@@ -1042,6 +1081,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
+  SSD_TSTAMP(7);
 }
 
 // ------------------------------------------------------------------------------------
@@ -1072,7 +1112,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
   float* Os = reinterpret_cast<float*>(smem);
   float* sm = reinterpret_cast<float*>(smem + S::kBytes - 64 * sizeof(float));
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
   const int mt = bid % mtiles;
   const int h = (bid / mtiles) % nh;
@@ -1238,7 +1278,7 @@ __global__ __launch_bounds__(256) void ssd_ddA_causal_kernel(
   float* dAs = rowsum + 256;
   float* dts = dAs + 256;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31, half = lane >> 5;
   const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
   const int h = bid % nh;
   const int c = (bid / nh) % C;
@@ -1363,7 +1403,7 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
   float* dAk = reinterpret_cast<float*>(smem + S::kMain);
   float* sm = dAk + 2 * ST;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31, half = lane >> 5;
   const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
   const int st = bid % stiles;
   const int h = (bid / stiles) % nh;
