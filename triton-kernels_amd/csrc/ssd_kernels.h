@@ -170,6 +170,49 @@ __device__ __forceinline__ void stage_rows(T* tile, const T* __restrict__ g, int
     }
   }
 }
+// The two halves of stage_rows for tiles of at most eight 16-byte pieces per thread: the loads
+// (into registers) and, later, the scaling, masking and LDS stores.  A kernel that has the next
+// tile's loads in flight while it works on the current one calls them apart.  Up to two float32
+// values per row (aux0[row], aux1[row]; null = not wanted) travel with the pieces, so that a
+// row scale computed from them costs no load at store time.
+template <typename T, int ROWS, int COLS>
+struct RowPieces {
+  static constexpr int EPL = Vec16<T>::N, VPR = COLS / EPL, CNT = ROWS * VPR / 256;
+  static_assert((ROWS * VPR) % 256 == 0 && CNT <= 8, "tile must split evenly over 256 threads");
+  Vec16<T> v[CNT];
+  float a0[CNT], a1[CNT];
+  __device__ __forceinline__ void load(const T* __restrict__ g, int64_t row_stride, int row0, int limit, int tid,
+                                       const float* __restrict__ aux0 = nullptr,
+                                       const float* __restrict__ aux1 = nullptr) {
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) {
+      const int idx = tid + 256 * i;
+      const int row = min(row0 + idx / VPR, limit - 1);
+      v[i] = load16(g + (int64_t)row * row_stride + (idx % VPR) * EPL);
+      if (aux0) a0[i] = aux0[row];
+      if (aux1) a1[i] = aux1[row];
+    }
+  }
+  // scale(row, aux0[row], aux1[row]) multiplies the row; NoScale leaves it
+  template <typename F>
+  __device__ __forceinline__ void store(T* tile, int row0, int limit, int tid, F scale) {
+    constexpr int P = Tile<T>::pitch(COLS);
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) {
+      const int idx = tid + 256 * i;
+      const int r = idx / VPR, cv = (idx % VPR) * EPL;
+      const bool in = row0 + r < limit;
+      if constexpr (!std::is_same<F, NoScale>::value) {
+        const float s = scale(in ? row0 + r : limit - 1, a0[i], a1[i]);
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) v[i].set(e, v[i].get(e) * s);
+      }
+      if (!in) v[i].zero();
+      store16(tile + r * P + cv, v[i]);
+    }
+  }
+};
+
 // ------------------------------------------------------------------------------------
 // chunk_cumsum.  One wave per (b, c, h).  dt is processed (bias, softplus with the identity
 // above 20, clamp), positions past the sequence give 0; dA = dt * A[h] is scanned across the
@@ -231,7 +274,8 @@ __global__ __launch_bounds__(256) void ssd_cumsum_kernel(const TD* __restrict__ 
 template <typename T, int P, int N>
 struct StateSmem {
   static constexpr int KT = 64, PX = Tile<T>::pitch(P), PB = Tile<T>::pitch(N);
-  static constexpr int kBytes = KT * (PX + PB) * (int)sizeof(T);
+  static constexpr int kStage = KT * (PX + PB) * (int)sizeof(T);
+  static constexpr int kBytes = 2 * kStage;  // two stages: one being multiplied, one being filled
 };
 
 template <typename T, int P, int N, int MODE>
@@ -265,30 +309,44 @@ __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
 #pragma unroll
   for (int i = 0; i < BPW; ++i) zero_acc(acc[i]);
 
-  for (int k0 = 0; k0 < limit; k0 += KT) {
+  // Stage s + 1 is requested before the products of stage s and written to the other half of LDS
+  // after them: one barrier per stage, and the loads have the products to hide behind.
+  auto scale_b = [&](int k, float dA_k, float dt_k) {
+    const float w = __expf(fminf(dA_last - dA_k, 0.f)) * dt_k;
+    return (sq.on() && (seq_dead || sq.at(k) != seq_ref)) ? 0.f : w;
+  };
+  auto scale_x = [&](int k, float dA_k, float) {
+    const float w = __expf(dA_k);
+    return (sq.on() && sq.at(k) != seq_ref) ? 0.f : w;
+  };
+  RowPieces<T, KT, P> px;
+  RowPieces<T, KT, N> pb;
+  auto request = [&](int k0) {  // the pieces of a stage and the per-row values their scale needs
+    px.load(xg, sx.sl, k0, limit, tid, MODE == 1 ? dAp : nullptr);
+    pb.load(Bg, sB.sl, k0, limit, tid, MODE == 0 ? dAp : nullptr, MODE == 0 ? dtp : nullptr);
+  };
+  request(0);
+  int buf = 0;
+  for (int k0 = 0; k0 < limit; k0 += KT, buf ^= 1) {
+    T* xb = xs + buf * (S::kStage / (int)sizeof(T));
+    T* bb = bs + buf * (S::kStage / (int)sizeof(T));
     if (MODE == 0) {
-      stage_rows<T, KT, P>(xs, xg, sx.sl, k0, limit, tid, NoScale());
-      stage_rows<T, KT, N>(bs, Bg, sB.sl, k0, limit, tid, [&](int k) {
-        const float w = __expf(fminf(dA_last - dAp[k], 0.f)) * dtp[k];
-        return (sq.on() && (seq_dead || sq.at(k) != seq_ref)) ? 0.f : w;
-      });
+      px.store(xb, k0, limit, tid, NoScale());
+      pb.store(bb, k0, limit, tid, scale_b);
     } else {
-      stage_rows<T, KT, P>(xs, xg, sx.sl, k0, limit, tid, [&](int k) {
-        const float w = __expf(dAp[k]);
-        return (sq.on() && sq.at(k) != seq_ref) ? 0.f : w;
-      });
-      stage_rows<T, KT, N>(bs, Bg, sB.sl, k0, limit, tid, NoScale());
+      px.store(xb, k0, limit, tid, scale_x);
+      pb.store(bb, k0, limit, tid, NoScale());
     }
     __syncthreads();
+    if (k0 + KT < limit) request(k0 + KT);
 #pragma unroll
     for (int kk = 0; kk < KT; kk += KG) {
 #pragma unroll
       for (int i = 0; i < BPW; ++i) {
         const int j = wave + 4 * i, mi = j % MB, ni = j / MB;
-        mma_group(frag_cols(xs, PX, kk, 32 * mi, lane), frag_cols(bs, PB, kk, 32 * ni, lane), acc[i]);
+        mma_group(frag_cols(xb, PX, kk, 32 * mi, lane), frag_cols(bb, PB, kk, 32 * ni, lane), acc[i]);
       }
     }
-    __syncthreads();
   }
   float* out = states + (((b * C + c) * nh + h) * (int64_t)P) * N;
 #pragma unroll
