@@ -28,6 +28,12 @@ for p in (ROOT, os.path.join(ROOT, "triton-kernels_amd")):
 # what the same counters read for a plain 268 435 456-byte device copy (FETCH_SIZE reads
 # 131 085 KiB for it, factor 1.99982; WRITE_SIZE reads 262 144 KiB, factor 1).
 TRAFFIC_BYTES = {"fwd_single_pass": 591160982, "bwd_single_pass": 841346755}
+# the same for the SSD stage kernels at configuration 5 (finishing kernels added to their stage)
+SSD_TRAFFIC_BYTES = {
+    "chunk_cumsum": 25728185, "chunk_state": 571561815, "state_passing": 553727051, "bmm_chunk": 100777471,
+    "chunk_scan": 878544586, "bwd_dstates": 562102058, "bwd_state_passing": 827459644, "bwd_db": 630374066,
+    "bwd_dc": 604094138, "bwd_dx": 1156650141, "bwd_ddAcs": 599910406,
+}
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
@@ -227,7 +233,7 @@ def ssd_main(args):
                    "chunk256, bf16 x/B/C, fp32 dt/A, D = 0, no gate"},
         "stages": res,
         "roofline": {"kernel": dom, "bound": "hbm", "achieved": res[dom]["GBps"], "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": res[dom]["hbm_frac"], "traffic": None},
+                     "unit": "GB/s", "frac": res[dom]["hbm_frac"], "traffic": SSD_TRAFFIC_BYTES.get(dom)},
     }
     if not args.no_cpu_baseline:
         x, dt, A, B, Cm, _, _ = S.make_inputs(1, 512, nh, P, g, N, seed=5, dtype=torch.bfloat16)
