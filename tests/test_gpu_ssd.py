@@ -26,6 +26,9 @@ CASES = [
     (1, 130, 2, 128, 2, 128, 64),
     (1, 900, 2, 64, 1, 64, 512),    # two 256-row super-tiles per chunk, the last chunk ragged
     (1, 512, 2, 128, 2, 128, 256),
+    (1, 150, 2, 64, 1, 64, 48),     # chunk sizes that are no multiple of the 64-row tiles
+    (1, 333, 2, 64, 2, 64, 200),
+    (1, 1100, 2, 64, 1, 128, 1024),  # the largest chunk size, second chunk ragged
 ]
 
 

@@ -19,6 +19,9 @@ CASES = [
     (1, 520, 2, 128, 1, 64, 128),
     (1, 130, 2, 128, 2, 128, 64),
     (1, 900, 2, 64, 1, 64, 512),
+    (1, 150, 2, 64, 1, 64, 48),     # chunk sizes that are no multiple of the 64-row tiles
+    (1, 333, 2, 64, 2, 64, 200),
+    (1, 1100, 2, 64, 1, 128, 1024),  # the largest chunk size, second chunk ragged
 ]
 
 
