@@ -168,8 +168,12 @@ int ssd_chunk_scan_bwd_dc(const void* dout, int64_t d_sb, int64_t d_sl, int64_t 
  *          + sum_{k>=m} round(cb[k,m] * exp(min(dA_k - dA_m, 0))) * dout[k,p];
  * dx = acc * dt_m + D * dout (type `dtype`, dx's own strides), ddt[b,h,c,m] = sum_p acc[m,p] * x[m,p]
  * (float32, 0 past seqlen).  cb float32 (batch, C, ngroups, Q, Q), dstates float32
- * (batch, C, nheads, hdim, dstate), D as for ssd_chunk_scan_fwd (its gradient, sum dout * x, is
- * left to the caller).  With seq_idx the first term only reaches the rows m whose id equals that
+ * (batch, C, nheads, hdim, dstate), D as for ssd_chunk_scan_fwd.  dD_partial (may be NULL; needs D):
+ * float32 (batch, C, nheads, S, hdim) with S = ssd_chunk_scan_chunk_state_bwd_dx_dD_slots(...),
+ * every slot written: partial sums over positions of dout * x, whose sum over batch, C and S is
+ * the gradient of D (nheads, hdim), summed over hdim too for a D of shape (nheads) -- the
+ * reference writes such partials per block and sums them in torch
+ * (mamba_chunk_scan_chunk_state_bwd_dx.py:176-183,245-247).  With seq_idx the first term only reaches the rows m whose id equals that
  * of the chunk's last position (mamba_chunk_scan_chunk_state_bwd_dx.py:93-96).
  * Replaces _chunk_scan_chunk_state_bwd_dx,
  * kernels/mamba_kernels_bwd/mamba_chunk_scan_chunk_state_bwd_dx.py:189-248. */
@@ -180,7 +184,11 @@ int ssd_chunk_scan_chunk_state_bwd_dx(const float* cb, const void* x, int64_t x_
                                       int d_has_hdim, void* dx, int64_t dx_sb, int64_t dx_sl, int64_t dx_sh,
                                       float* ddt, int64_t batch, int64_t seqlen, int64_t nheads,
                                       int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
-                                      const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream);
+                                      const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, float* dD_partial,
+                                      void* stream);
+
+/* Slots per (batch, chunk, head) of dD_partial above for a shape; 0 for an unsupported one. */
+int64_t ssd_chunk_scan_chunk_state_bwd_dx_dD_slots(int dtype, int64_t hdim, int64_t dstate, int64_t chunk);
 
 /* Bytes of workspace ssd_chunk_scan_bwd_ddAcs needs (column sums per row tile, row sums). */
 size_t ssd_chunk_scan_bwd_ddAcs_workspace_bytes(int64_t batch, int64_t seqlen, int64_t nheads, int64_t chunk);

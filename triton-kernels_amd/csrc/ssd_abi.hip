@@ -149,18 +149,24 @@ struct DxLaunch {
   float* ddt;
   Dims d;
   SeqIdx seq;
+  float* dD_part;
   hipStream_t st;
+  // whether the 256-row kernel runs this shape (it must also fit the LDS of a CU)
+  template <typename T, int P, int N>
+  static bool wide(int64_t Q) {
+    return Q % 256 == 0 && WideSmem<T, P, N>::kBytes <= kLdsBytes;
+  }
   template <typename T, int P, int N>
   int run() const {
     constexpr int wide_smem = WideSmem<T, P, N>::kBytes;
-    if (d.Q % 256 == 0 && wide_smem <= kLdsBytes) {
+    if (wide<T, P, N>(d.Q)) {
       auto kernel = ssd_chunk_scan_bwd_dx_wide_kernel<T, P, N>;
       SSD_TRY(allow_smem(kernel, wide_smem));
       const int stiles = (int)(d.Q / 256);
       hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh * stiles)), dim3(256), wide_smem, st, cb,
                          (const T*)x, sx, (const T*)dout, sd, dt, dA, (const T*)B, sB, dstates, D, d_has_hdim,
                          (T*)dx, sdx, ddt, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C,
-                         stiles, seq);
+                         stiles, seq, dD_part);
       return launched();
     }
     auto kernel = ssd_chunk_scan_bwd_dx_kernel<T, P, N>;
@@ -170,8 +176,17 @@ struct DxLaunch {
     hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh * mtiles)), dim3(256), smem, st, cb,
                        (const T*)x, sx, (const T*)dout, sd, dt, dA, (const T*)B, sB, dstates, D, d_has_hdim, (T*)dx,
                        sdx, ddt, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C, mtiles,
-                       seq);
+                       seq, dD_part);
     return launched();
+  }
+};
+
+// Number of per-wave slots the dx kernel of a shape writes per (batch, chunk, head).
+struct DxSlots {
+  int64_t Q;
+  template <typename T, int P, int N>
+  int run() const {
+    return DxLaunch::wide<T, P, N>(Q) ? (int)(4 * (Q / 256)) : (int)(4 * ((Q + 63) / 64));
   }
 };
 
@@ -446,11 +461,14 @@ int ssd_chunk_scan_chunk_state_bwd_dx(const float* cb, const void* x, int64_t x_
                                       int d_has_hdim, void* dx, int64_t dx_sb, int64_t dx_sl, int64_t dx_sh,
                                       float* ddt, int64_t batch, int64_t seqlen, int64_t nheads,
                                       int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
-                                      const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream) {
+                                      const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, float* dD_partial,
+                                      void* stream) {
   Dims d;
   SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
   SSD_TRY(check_dtype(dtype));
   if (!dim_ok(hdim) || !dim_ok(dstate)) return SSD_ERR_UNSUPPORTED;
+  if (dD_partial && !D) return SSD_ERR_NULL;
+  if (dD_partial) SSD_TRY(check_f32(dD_partial));
   SSD_TRY(check_vec(x, x_sb, x_sl, x_sh, dtype, hdim));
   SSD_TRY(check_vec(dout, d_sb, d_sl, d_sh, dtype, hdim));
   SSD_TRY(check_vec(dx, dx_sb, dx_sl, dx_sh, dtype, hdim));
@@ -462,7 +480,14 @@ int ssd_chunk_scan_chunk_state_bwd_dx(const float* cb, const void* x, int64_t x_
   return dispatch_tpn(dtype, hdim, dstate,
                       DxLaunch{cb, x, dout, B, Strides3{x_sb, x_sl, x_sh}, Strides3{d_sb, d_sl, d_sh},
                                Strides3{b_sb, b_sl, b_sg}, Strides3{dx_sb, dx_sl, dx_sh}, dt, dA_cumsum, dstates, D,
-                               d_has_hdim, dx, ddt, d, as_seq(seq_idx, seq_sb, seq_sl), as_stream(stream)});
+                               d_has_hdim, dx, ddt, d, as_seq(seq_idx, seq_sb, seq_sl), dD_partial,
+                               as_stream(stream)});
+}
+
+int64_t ssd_chunk_scan_chunk_state_bwd_dx_dD_slots(int dtype, int64_t hdim, int64_t dstate, int64_t chunk) {
+  if (check_dtype(dtype) != SSD_OK || !dim_ok(hdim) || !dim_ok(dstate)) return 0;
+  if (chunk <= 0 || chunk > 1024 || chunk % 4) return 0;
+  return dispatch_tpn(dtype, hdim, dstate, DxSlots{chunk});
 }
 
 static size_t ddAcs_part_floats(const Dims& d) {

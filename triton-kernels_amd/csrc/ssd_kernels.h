@@ -1142,6 +1142,22 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
   SSD_TSTAMP(7);
 }
 
+// Partial sums for the gradient of the skip weight D: a lane holds, for its EPL adjacent features
+// cv .. (cv = EPL * (lane % VPR)), the sum of dout * x over the rows it handled; the lanes of a
+// wave that share cv are added up and the wave's hdim sums go to its slot.  The caller adds the
+// slots of all waves, chunks and batch elements.
+template <int EPL, int VPR>
+__device__ __forceinline__ void store_dD_partial(float* __restrict__ slot, float* dsum, int lane) {
+#pragma unroll
+  for (int off = VPR; off < 64; off <<= 1)
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) dsum[e] += __shfl_xor(dsum[e], off);
+  if (lane < VPR) {
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) slot[lane * EPL + e] = dsum[e];
+  }
+}
+
 // ------------------------------------------------------------------------------------
 // Backward of chunk_scan and chunk_state with respect to x (and the explicit dt factors).
 // One workgroup per (b, c, h, tile of 64 rows m):
@@ -1159,7 +1175,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
     const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Bm, Strides3 sB,
     const float* __restrict__ dstates, const float* __restrict__ D, int d_has_hdim, T* __restrict__ dx,
     Strides3 sdx, float* __restrict__ ddt, int nh, int heads_per_group, int ngroups, int L, int Q, int C,
-    int mtiles, SeqIdx seq) {
+    int mtiles, SeqIdx seq, float* __restrict__ dD_part) {
   using S = ScanSmem<T, P, N>;
   constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, PB = P / 32, BPW = 2 * PB / 4;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -1180,8 +1196,14 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
   const int m0 = 64 * mt;
   const int64_t chunk = (b * nh + h) * C + c;
   float* ddtp = ddt + chunk * Q;
-  if (m0 >= limit) {  // nothing of the sequence in this tile: its ddt slots are zero
+  // slot of this wave in dD_part (batch, C, nheads, 4 * mtiles, hdim)
+  float* dslot = dD_part ? dD_part + ((((b * C + c) * nh + h) * (int64_t)mtiles + mt) * 4 + wave) * P : nullptr;
+  if (m0 >= limit) {  // nothing of the sequence in this tile: its ddt and dD slots are zero
     if (tid < 64 && m0 + tid < Q) ddtp[m0 + tid] = 0.f;
+    if (dslot && lane < P / EPL) {
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) dslot[lane * EPL + e] = 0.f;
+    }
     return;
   }
   const int g = h / heads_per_group;
@@ -1272,6 +1294,9 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
   }
   __syncthreads();
   constexpr int VPR = P / EPL;
+  float dsum[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) dsum[e] = 0.f;
 #pragma unroll
   for (int i = 0; i < 64 * VPR / 256; ++i) {
     const int idx = tid + 256 * i;
@@ -1292,7 +1317,10 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
       if (D) {
         const Vec16<T> dv = load16(dout + b * sd.sb + pos * sd.sl + h * sd.sh + cv);
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) v[e] = fmaf(d_has_hdim ? D[h * P + cv + e] : D[h], dv.get(e), v[e]);
+        for (int e = 0; e < EPL; ++e) {
+          v[e] = fmaf(d_has_hdim ? D[h * P + cv + e] : D[h], dv.get(e), v[e]);
+          dsum[e] = fmaf(dv.get(e), xv.get(e), dsum[e]);
+        }
       }
       Vec16<T> o;
 #pragma unroll
@@ -1304,6 +1332,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
     for (int off = 1; off < VPR; off <<= 1) dot += __shfl_xor(dot, off);
     if ((idx % VPR) == 0 && m < Q) ddtp[m] = dot;
   }
+  if (dslot) store_dD_partial<EPL, VPR>(dslot, dsum, lane);
 }
 
 // ------------------------------------------------------------------------------------
@@ -1451,7 +1480,7 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
     const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Bm, Strides3 sB,
     const float* __restrict__ dstates, const float* __restrict__ D, int d_has_hdim, T* __restrict__ dx,
     Strides3 sdx, float* __restrict__ ddt, int nh, int heads_per_group, int ngroups, int L, int Q, int C,
-    int stiles, SeqIdx seq) {
+    int stiles, SeqIdx seq, float* __restrict__ dD_part) {
   using S = WideSmem<T, P, N>;
   constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, PB = P / 32, ST = S::ST;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -1471,8 +1500,14 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
   const int m0 = ST * st;
   const int64_t chunk = (b * nh + h) * C + c;
   float* ddtp = ddt + chunk * Q;
+  // slot of this wave in dD_part (batch, C, nheads, 4 * stiles, hdim)
+  float* dslot = dD_part ? dD_part + ((((b * C + c) * nh + h) * (int64_t)stiles + st) * 4 + wave) * P : nullptr;
   if (m0 >= limit) {
     ddtp[m0 + tid] = 0.f;
+    if (dslot && lane < P / EPL) {
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) dslot[lane * EPL + e] = 0.f;
+    }
     return;
   }
   const int g = h / heads_per_group;
@@ -1492,6 +1527,7 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
 #pragma unroll
     for (int pb = 0; pb < PB; ++pb) zero_acc(acc[mb][pb]);
 
+  SSD_TSTAMP(0);
   // ---- phase A: B . dstates, scaled by the decay to the end of the chunk
   {
     constexpr int VPR = N / 4;
@@ -1510,6 +1546,7 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
     sm[tid] = live ? __expf(fminf(dAp[Q - 1] - dAp[m0 + tid], 0.f)) : 0.f;
   }
   __syncthreads();
+  SSD_TSTAMP(1);
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {
     const int m = m0 + mrow[mb] + l32;
@@ -1530,12 +1567,15 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
   }
 
   // ---- phase B: the k super-tiles from the diagonal one to the end of the chunk
+  SSD_TSTAMP(2);
   __syncthreads();  // the dout tile takes the place of dstates
+  SSD_TSTAMP(3);
   for (int kt = st; kt < stiles && ST * kt < limit; ++kt) {
     const int k0 = ST * kt;
     stage_rows<T, ST, P>(Ds, dg, sd.sl, k0, limit, tid, NoScale());
     dAk[tid] = dAp[k0 + tid];
     __syncthreads();
+    SSD_TSTAMP(4);
     const bool diag = kt == st;
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) {
@@ -1558,39 +1598,71 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
         for (int pb = 0; pb < PB; ++pb) mma_group(a, frag_cols(Ds, S::PX, kk, 32 * pb, lane), acc[mb][pb]);
       }
     }
+    SSD_TSTAMP(5);
     __syncthreads();
   }
+  SSD_TSTAMP(6);
 
-  // ---- phase C: each wave moves its two blocks through its own staging area
+  // ---- phase C: each wave moves its two blocks through its own staging area.  The rows of x
+  // (and dout, dt) that the block's results meet are requested before the accumulators go to
+  // LDS, so that their latency hides behind the staging (where that takes at most four pieces
+  // per lane; otherwise they are fetched as they are needed).
   float* mine = Os + wave * 32 * S::PO;
-  constexpr int VPR = P / EPL;
+  constexpr int VPR = P / EPL, NI = 32 * VPR / 64;
+  constexpr bool kEarly = NI <= 4;
+  float dsum[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) dsum[e] = 0.f;
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {
+    Vec16<T> xv[kEarly ? NI : 1], dv[kEarly ? NI : 1];
+    float dtm[kEarly ? NI : 1];
+    if constexpr (kEarly) {
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int idx = lane + 64 * i;
+        const int r = idx / VPR, cv = (idx % VPR) * EPL;
+        const int m = m0 + mrow[mb] + r;
+        const int64_t pos = (int64_t)c * Q + min(m, limit - 1);
+        xv[i] = load16(x + b * sx.sb + pos * sx.sl + h * sx.sh + cv);
+        dtm[i] = dtp[m];
+        if (D) dv[i] = load16(dout + b * sd.sb + pos * sd.sl + h * sd.sh + cv);
+      }
+    }
 #pragma unroll
     for (int pb = 0; pb < PB; ++pb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) mine[acc_row(v, lane) * S::PO + 32 * pb + l32] = acc[mb][pb][v];
     __builtin_amdgcn_s_waitcnt(0xc07f);
 #pragma unroll
-    for (int i = 0; i < 32 * VPR / 64; ++i) {
+    for (int i = 0; i < NI; ++i) {
       const int idx = lane + 64 * i;
       const int r = idx / VPR, cv = (idx % VPR) * EPL;
       const int m = m0 + mrow[mb] + r;
       const int64_t pos = (int64_t)c * Q + min(m, limit - 1);
-      const Vec16<T> xv = load16(x + b * sx.sb + pos * sx.sl + h * sx.sh + cv);
-      const float dtm = dtp[m];
+      Vec16<T> xi, di;
+      float dti;
+      if constexpr (kEarly) {
+        xi = xv[i], di = dv[i], dti = dtm[i];
+      } else {
+        xi = load16(x + b * sx.sb + pos * sx.sl + h * sx.sh + cv);
+        dti = dtp[m];
+        if (D) di = load16(dout + b * sd.sb + pos * sd.sl + h * sd.sh + cv);
+      }
       float dot = 0.f, v[EPL];
 #pragma unroll
       for (int e = 0; e < EPL; ++e) {
         v[e] = mine[r * S::PO + cv + e];
-        dot = fmaf(v[e], xv.get(e), dot);
-        v[e] *= dtm;
+        dot = fmaf(v[e], xi.get(e), dot);
+        v[e] *= dti;
       }
       if (m >= limit) dot = 0.f;
       if (D) {
-        const Vec16<T> dv = load16(dout + b * sd.sb + pos * sd.sl + h * sd.sh + cv);
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) v[e] = fmaf(d_has_hdim ? D[h * P + cv + e] : D[h], dv.get(e), v[e]);
+        for (int e = 0; e < EPL; ++e) {
+          v[e] = fmaf(d_has_hdim ? D[h * P + cv + e] : D[h], di.get(e), v[e]);
+          if (m < limit) dsum[e] = fmaf(di.get(e), xi.get(e), dsum[e]);
+        }
       }
       if (m < limit) {
         Vec16<T> o;
@@ -1604,6 +1676,8 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
+  if (dslot) store_dD_partial<EPL, VPR>(dslot, dsum, lane);
+  SSD_TSTAMP(7);
 }
 
 }  // namespace ssd

@@ -60,7 +60,8 @@ _SIGNATURES = {
     "ssd_state_passing_bwd": (c_int, [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I] + _IDS + [_I, _I, _P]),
     "ssd_chunk_state_bwd_db": (c_int, _SEQ + [c_int, _P, _P, _P] + _SEQ + [_P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
     "ssd_chunk_scan_bwd_dc": (c_int, _SEQ + [c_int, _P, _P] + _SEQ + [_P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
-    "ssd_chunk_scan_chunk_state_bwd_dx": (c_int, [_P] + _SEQ + _SEQ + [c_int, _P, _P] + _SEQ + [_P, _P, c_int] + _SEQ + [_P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
+    "ssd_chunk_scan_chunk_state_bwd_dx": (c_int, [_P] + _SEQ + _SEQ + [c_int, _P, _P] + _SEQ + [_P, _P, c_int] + _SEQ + [_P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P, _P]),
+    "ssd_chunk_scan_chunk_state_bwd_dx_dD_slots": (c_int64, [c_int, _I, _I, _I]),
     "ssd_chunk_scan_bwd_ddAcs_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "ssd_chunk_scan_bwd_ddAcs": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _I, _P]),
 }

@@ -2,7 +2,8 @@
 
 Mirrors _chunk_scan_chunk_state_bwd_dx,
 kernels/mamba_kernels_bwd/mamba_chunk_scan_chunk_state_bwd_dx.py:189-248 of the reference (same
-arguments, returns (dx, ddt, dD)).  dD = sum dout * x is a plain reduction and is taken in torch."""
+arguments, returns (dx, ddt, dD)).  For dD = sum dout * x the kernel leaves one partial sum per wave
+and feature, which are added up here, as the reference adds its per-block partials (:245-247)."""
 import torch
 
 from kernels import _lib
@@ -32,6 +33,11 @@ def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum, B, CB, dout, dstates, D=Non
         assert dx.shape == x.shape and dx.dtype == x.dtype and dx.stride(-1) == 1
     ddt = torch.empty(batch, nheads, nchunks, chunk_size, device=dev, dtype=torch.float32)
     Df = None if D is None else _lib.f32c(D)
+    dD_part = None
+    if D is not None:  # per-wave partial sums of dout * x, summed below like the reference's per-block ones
+        slots = _lib.lib().ssd_chunk_scan_chunk_state_bwd_dx_dD_slots(_lib.dtype_code(x), headdim, dstate, chunk_size)
+        assert slots > 0, "unsupported shape"
+        dD_part = torch.empty(batch, nchunks, nheads, slots, headdim, device=dev, dtype=torch.float32)
     with torch.cuda.device(dev):
         _lib.check(
             _lib.lib().ssd_chunk_scan_chunk_state_bwd_dx(
@@ -39,10 +45,10 @@ def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum, B, CB, dout, dstates, D=Non
                 _lib.f32c(dA_cumsum).data_ptr(), *bs, _lib.f32c(dstates).data_ptr(),
                 None if Df is None else Df.data_ptr(), int(D is not None and D.dim() == 2), dx.data_ptr(),
                 dx.stride(0), dx.stride(1), dx.stride(2), ddt.data_ptr(), batch, seqlen, nheads, ngroups, headdim,
-                dstate, chunk_size, *ids, _lib.stream_ptr(dev)),
+                dstate, chunk_size, *ids, None if dD_part is None else dD_part.data_ptr(), _lib.stream_ptr(dev)),
             "ssd_chunk_scan_chunk_state_bwd_dx")
     dD = None
     if D is not None:
-        prod = dout.float() * x.float()
-        dD = (prod.sum((0, 1)) if D.dim() == 2 else prod.sum((0, 1, 3))).to(D.dtype)
+        dD = dD_part.sum((0, 1, 3))
+        dD = (dD if D.dim() == 2 else dD.sum(-1)).to(D.dtype)
     return dx, ddt.to(dtype=dt.dtype), dD
