@@ -1377,16 +1377,12 @@ __global__ __launch_bounds__(256) void ssd_ddA_causal_kernel(
   const T* xg = x + b * sx.sb + (int64_t)c * Q * sx.sl + h * sx.sh;
   const T* dg = dout + b * sd.sb + (int64_t)c * Q * sd.sl + h * sd.sh;
 
+  SSD_TSTAMP(0);
   // shared: the chunk's x rows (zero past the limit), dA, dt; cleared: the sums
-  {
-    constexpr int VPR = P / EPL;
-    for (int idx = tid; idx < Q * VPR; idx += 256) {
-      const int r = idx / VPR, cv = (idx % VPR) * EPL;
-      Vec16<T> v = load16(xg + (int64_t)min(r, limit - 1) * sx.sl + cv);
-      if (r >= limit) v.zero();
-      store16(Xs + r * S::PX + cv, v);
-    }
-  }
+  static_assert(S::PX == Tile<T>::pitch(P), "stage_rows writes rows at this pitch");
+  if (Q == 256) stage_rows<T, 256, P>(Xs, xg, sx.sl, 0, limit, tid, NoScale());
+  else if (Q == 128) stage_rows<T, 128, P>(Xs, xg, sx.sl, 0, limit, tid, NoScale());
+  else stage_rows<T, 64, P>(Xs, xg, sx.sl, 0, limit, tid, NoScale());
   if (tid < Q) {
     dAs[tid] = dA_cs[chunk * Q + tid];
     dts[tid] = dt[chunk * Q + tid];
@@ -1395,10 +1391,12 @@ __global__ __launch_bounds__(256) void ssd_ddA_causal_kernel(
 #pragma unroll
   for (int w = 0; w < 4; ++w) colpart[w * 256 + tid] = 0.f;
   __syncthreads();
+  SSD_TSTAMP(1);
 
 #pragma unroll
   for (int slot = 0; slot < 2; ++slot) {
     const int mb = slot == 0 ? wave : MB - 1 - wave;
+    if (slot == 1) SSD_TSTAMP(2);
     if (2 * wave >= MB) continue;  // fewer than 8 row blocks: the upper waves have none
     const int m_lane = 32 * mb + l32;  // row whose dout this lane feeds into the MFMA
     Vec16<T> a[KS];
@@ -1442,7 +1440,9 @@ __global__ __launch_bounds__(256) void ssd_ddA_causal_kernel(
       if (l32 == 31) rowsum[32 * mb + acc_row(v, lane)] = t;
     }
   }
+  SSD_TSTAMP(3);
   __syncthreads();
+  SSD_TSTAMP(4);
   // delta_i = colsum_i - rowsum_i; ddA[j] = sum_{i<j} delta_i: wave 0, four positions per lane
   if (wave == 0) {
     const int per = (Q + 63) >> 6;
@@ -1465,6 +1465,7 @@ __global__ __launch_bounds__(256) void ssd_ddA_causal_kernel(
       }
     }
   }
+  SSD_TSTAMP(5);
 }
 
 // ------------------------------------------------------------------------------------
