@@ -65,6 +65,7 @@ struct Vec16<float> {
     else raw.w = f;
   }
   __device__ __forceinline__ void put(int i, float f) { set(i, f); }
+  __device__ __forceinline__ void set_all(const float* f) { raw = make_float4(f[0], f[1], f[2], f[3]); }
   __device__ __forceinline__ void zero() { raw = make_float4(0.f, 0.f, 0.f, 0.f); }
 };
 template <>
@@ -74,6 +75,19 @@ struct Vec16<bf16_t> {
   __device__ __forceinline__ float get(int i) const { return (float)raw[i]; }
   __device__ __forceinline__ void set(int i, float f) { raw[i] = (bf16_t)f; }
   __device__ __forceinline__ void put(int i, bf16_t f) { raw[i] = f; }
+  // all eight elements from floats, converted two at a time (one packed conversion per pair
+  // instead of a conversion and a byte permute per element)
+  __device__ __forceinline__ void set_all(const float* f) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef bf16_t b16x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const f32x2 p = {f[2 * i], f[2 * i + 1]};
+      const b16x2 q = __builtin_convertvector(p, b16x2);
+      raw[2 * i] = q[0];
+      raw[2 * i + 1] = q[1];
+    }
+  }
   __device__ __forceinline__ void zero() {
 #pragma unroll
     for (int i = 0; i < 8; ++i) raw[i] = (bf16_t)0.0f;

@@ -207,6 +207,7 @@ struct GroupLaunch {
     constexpr int smem = GroupSmem<T, P, N>::kBytes;
     SSD_TRY(allow_smem(kernel, smem));
     const int mtiles = (int)((d.Q + 63) / 64);
+    if (d.batch * d.C * d.g * mtiles > 0x7fffffff) return SSD_ERR_SHAPE;
     hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.g * mtiles)), dim3(256), smem, st, (const T*)a, sa,
                        s, dt, dA, (const T*)bc, sbc, out, ddA, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L,
                        (int)d.Q, (int)d.C, mtiles, seq);

@@ -162,8 +162,10 @@ __device__ __forceinline__ void stage_rows(T* tile, const T* __restrict__ g, int
       const bool in = row0 + r < limit;
       if constexpr (!std::is_same<F, NoScale>::value) {
         const float s = scale(in ? row0 + r : limit - 1);
+        float t[EPL];
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) v[i].set(e, v[i].get(e) * s);
+        for (int e = 0; e < EPL; ++e) t[e] = v[i].get(e) * s;
+        v[i].set_all(t);
       }
       if (!in) v[i].zero();
       store16(tile + r * P + cv, v[i]);
@@ -204,8 +206,10 @@ struct RowPieces {
       const bool in = row0 + r < limit;
       if constexpr (!std::is_same<F, NoScale>::value) {
         const float s = scale(in ? row0 + r : limit - 1, a0[i], a1[i]);
+        float t[EPL];
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) v[i].set(e, v[i].get(e) * s);
+        for (int e = 0; e < EPL; ++e) t[e] = v[i].get(e) * s;
+        v[i].set_all(t);
       }
       if (!in) v[i].zero();
       store16(tile + r * P + cv, v[i]);
@@ -896,8 +900,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(
     Vec16<T> o;
     if (z) {
       if (out_x) {
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) o.set(e, v[e]);
+        o.set_all(v);
         store16(out_x + b * so.sb + pos * so.sl + h * so.sh + cv, o);
       }
       const Vec16<T> zv = load16(z + b * sz.sb + pos * sz.sl + h * sz.sh + cv);
@@ -907,8 +910,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(
         v[e] *= zf / (1.f + __expf(-zf));
       }
     }
-#pragma unroll
-    for (int e = 0; e < EPL; ++e) o.set(e, v[e]);
+    o.set_all(v);
     store16(out + b * so.sb + pos * so.sl + h * so.sh + cv, o);
   }
 }
@@ -1067,16 +1069,18 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
         for (int u = 0; u < NS; ++u) {
           const int kk = kk0 + KG * u, kb = kk + EPL * half;
           Vec16<T> a;
+          float wf[EPL];
           if (exact) {
 #pragma unroll
             for (int e = 0; e < EPL; ++e) {
               const float f = w[u][e] * __expf(fminf(am - dAk[kb + e], 0.f)) * dtk[kb + e];
-              a.set(e, kb + e > mloc ? 0.f : f);
+              wf[e] = kb + e > mloc ? 0.f : f;
             }
           } else {
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) a.set(e, w[u][e] * fk[kb + e] * gm);
+            for (int e = 0; e < EPL; ++e) wf[e] = w[u][e] * fk[kb + e] * gm;
           }
+          a.set_all(wf);
 #pragma unroll
           for (int pb = 0; pb < PB; ++pb) mma_group(a, frag_cols(Xs, S::PX, kk, 32 * pb, lane), acc[mb][pb]);
         }
@@ -1121,8 +1125,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
         Vec16<T> o;
         if (z) {
           if (out_x) {
-#pragma unroll
-            for (int e = 0; e < EPL; ++e) o.set(e, v[e]);
+            o.set_all(v);
             store16(out_x + b * so.sb + pos * so.sl + h * so.sh + cv, o);
           }
           const Vec16<T> zv = load16(z + b * sz.sb + pos * sz.sl + h * sz.sh + cv);
@@ -1132,8 +1135,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
             v[e] *= zf / (1.f + __expf(-zf));
           }
         }
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) o.set(e, v[e]);
+        o.set_all(v);
         store16(out + b * so.sb + pos * so.sl + h * so.sh + cv, o);
       }
     }
@@ -1323,8 +1325,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
         }
       }
       Vec16<T> o;
-#pragma unroll
-      for (int e = 0; e < EPL; ++e) o.set(e, v[e]);
+      o.set_all(v);
       store16(dx + b * sdx.sb + pos * sdx.sl + h * sdx.sh + cv, o);
     }
     // the VPR lanes of a row are adjacent: butterfly sum, then one of them writes
@@ -1589,12 +1590,14 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
 #pragma unroll
         for (int e = 0; e < EPL; ++e) w[e] = cbcol[(int64_t)(kb + e) * Q];
         Vec16<T> a;
+        float wf[EPL];
 #pragma unroll
         for (int e = 0; e < EPL; ++e) {
           const int k = kb + e;
           const float f = w[e] * __expf(fminf(dAk[k] - am, 0.f));
-          a.set(e, ((diag && k < mloc) || k0 + k >= limit) ? 0.f : f);
+          wf[e] = ((diag && k < mloc) || k0 + k >= limit) ? 0.f : f;
         }
+        a.set_all(wf);
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) mma_group(a, frag_cols(Ds, S::PX, kk, 32 * pb, lane), acc[mb][pb]);
       }
@@ -1667,8 +1670,7 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
       }
       if (m < limit) {
         Vec16<T> o;
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) o.set(e, v[e]);
+        o.set_all(v);
         store16(dx + b * sdx.sb + pos * sdx.sl + h * sdx.sh + cv, o);
       }
 #pragma unroll
