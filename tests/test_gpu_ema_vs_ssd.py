@@ -1,0 +1,86 @@
+"""The EMA kernels against the Mamba-2 SSD kernels on the same problem, both through the C ABI
+on the GPU: the reference's own EMA tests hold its EMA launchers against its Mamba launchers
+this way (kernels/tests/ema/test_ema_state_fwd.py:120-141,
+kernels/tests/ema_bwd/test_ema_scan_bwd_dstates.py:95-125): with dt = -log(1 - p), A = -1,
+B = p, C = 1 and x = X / dt per head, the SSD recurrence h = exp(dt A) h + dt B x, y = C h is the
+EMA y = (1 - p) y + p X.  The SSD kernels need a state size of 64, so B and C carry their value
+in component 0 and zeros elsewhere.  float32, where both families compute in full precision."""
+import pytest
+import torch
+
+from parity_util import announce, check_close
+
+pytestmark = pytest.mark.gpu
+
+F32 = torch.float32
+NSTATE = 64
+
+
+def _encode(b, L, nh, P, seed, device):
+    gen = torch.Generator().manual_seed(seed)
+    X = torch.randn(b, L, nh * P, generator=gen)
+    p = torch.sigmoid(torch.randn(b, L, generator=gen) - 1.0)
+    dt1 = -torch.log1p(-p)                                    # (b, L)
+    ema = dict(A=torch.log1p(-p), X=X * p[..., None])         # the EMA kernels' inputs
+    Bm = torch.zeros(b, L, 1, NSTATE)
+    Bm[..., 0, 0] = p
+    Cm = torch.zeros(b, L, 1, NSTATE)
+    Cm[..., 0, 0] = 1.0
+    ssd = dict(x=(X / dt1[..., None]).reshape(b, L, nh, P), dt=dt1[..., None].expand(b, L, nh).contiguous(),
+               A=-torch.ones(nh), B=Bm, C=Cm)
+    to = lambda d: {k: v.to(device) for k, v in d.items()}
+    return to(ema), to(ssd)
+
+
+CASES = [(2, 512, 2, 64, 128), (1, 700, 4, 64, 256), (2, 300, 2, 128, 64)]  # b, L, nh, P, Q
+
+
+@pytest.mark.parametrize("b,L,nh,P,Q", CASES)
+def test_forward_agrees(b, L, nh, P, Q, device):
+    from kernels.ema_kernels.ema_combined_fwd import _ema_matmul_scan_combined_fwd
+    from kernels.mamba_kernels.mamba_combined_fwd import _mamba_chunk_scan_combined_fwd
+
+    announce(f"ema vs ssd forward b{b} L{L} nh{nh} P{P} Q{Q}")
+    ema, ssd = _encode(b, L, nh, P, seed=L + Q, device=device)
+    y_e, cs_e, prev_e, fin_e = _ema_matmul_scan_combined_fwd(ema["A"], ema["X"], Q)
+    y_s, _, dt_out, dA_cs, prev_s, fin_s = _mamba_chunk_scan_combined_fwd(ssd["x"], ssd["dt"], ssd["A"], ssd["B"],
+                                                                          ssd["C"], Q)
+    torch.cuda.synchronize()
+    nc = cs_e.shape[1]
+    check_close("y", y_s.reshape(b, L, nh * P), y_e.cpu(), F32)
+    check_close("dA_cumsum", dA_cs[:, 0], cs_e.cpu(), F32)                      # the heads share one decay
+    check_close("states entering the chunks", prev_s[..., 0].reshape(b, nc, nh * P), prev_e.cpu(), F32)
+    check_close("final state", fin_s[..., 0].reshape(b, nh * P), fin_e.cpu(), F32)
+    assert float(prev_s[..., 1:].abs().max()) == 0.0 and float(fin_s[..., 1:].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("b,L,nh,P,Q", CASES)
+def test_backward_stages_agree(b, L, nh, P, Q, device):
+    from kernels.ema_kernels.ema_cumsum import ema_chunk_cumsum_fwd
+    from kernels.ema_kernels_bwd.ema_scan_bwd import _ema_chunk_scan_bwd_dstates
+    from kernels.ema_kernels_bwd.ema_state_passing_bwd_dstates import _ema_state_passing_bwd
+    from kernels.mamba_kernels.mamba_cumsum import _chunk_cumsum_fwd
+    from kernels.mamba_kernels_bwd.mamba_scan_bwd import _chunk_scan_bwd_dstates
+    from kernels.mamba_kernels_bwd.mamba_state_passing_bwd_dstates import _state_passing_bwd
+
+    announce(f"ema vs ssd backward stages b{b} L{L} nh{nh} P{P} Q{Q}")
+    ema, ssd = _encode(b, L, nh, P, seed=2 * L + Q, device=device)
+    gen = torch.Generator().manual_seed(L)
+    dout = torch.randn(b, L, nh * P, generator=gen).to(device)
+    cs_e = ema_chunk_cumsum_fwd(ema["A"], Q)
+    dA_cs, _ = _chunk_cumsum_fwd(ssd["dt"], ssd["A"], Q)
+    nc = cs_e.shape[1]
+
+    # gradient of the states entering the chunks: component 0 of the SSD result (C = e_0)
+    ds_e = _ema_chunk_scan_bwd_dstates(cs_e, dout)
+    ds_s = _chunk_scan_bwd_dstates(ssd["C"], dA_cs, dout.reshape(b, L, nh, P), dtype=F32)
+    check_close("dstates of the chunk scan", ds_s[..., 0].reshape(b, nc, nh * P), ds_e.cpu(), F32)
+    assert float(ds_s[..., 1:].abs().max()) == 0.0
+
+    # reverse inter-chunk recurrence on the same flattened states
+    states = torch.randn(b, nc, nh * P, generator=gen).to(device)
+    g_e, ddA_e, _ = _ema_state_passing_bwd(states, cs_e[:, :, -1], ds_e, chunk_size=Q)
+    st4 = states.reshape(b, nc, nh, P)
+    g_s, ddA_s, _ = _state_passing_bwd(st4, dA_cs[:, :, :, -1], ds_e.reshape(b, nc, nh, P), chunk_size=Q)
+    check_close("dstates of state passing", g_s.reshape(b, nc, nh * P), g_e.cpu(), F32)
+    check_close("ddA of the chunk decays (summed over heads)", ddA_s.sum(1), ddA_e.cpu(), F32)
