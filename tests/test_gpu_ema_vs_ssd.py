@@ -3,8 +3,9 @@ on the GPU: the reference's own EMA tests hold its EMA launchers against its Mam
 this way (kernels/tests/ema/test_ema_state_fwd.py:120-141,
 kernels/tests/ema_bwd/test_ema_scan_bwd_dstates.py:95-125): with dt = -log(1 - p), A = -1,
 B = p, C = 1 and x = X / dt per head, the SSD recurrence h = exp(dt A) h + dt B x, y = C h is the
-EMA y = (1 - p) y + p X.  The SSD kernels need a state size of 64, so B and C carry their value
-in component 0 and zeros elsewhere.  float32, where both families compute in full precision."""
+EMA y = (1 - p) y + p X.  The state size is 1, as in the reference's tests (head sizes 32 and
+512 there), or 64 with B and C carrying their value in component 0, which is the shape the SSD
+kernels take as it is.  float32, where both families compute in full precision."""
 import pytest
 import torch
 
@@ -13,18 +14,17 @@ from parity_util import announce, check_close
 pytestmark = pytest.mark.gpu
 
 F32 = torch.float32
-NSTATE = 64
 
 
-def _encode(b, L, nh, P, seed, device):
+def _encode(b, L, nh, P, nstate, seed, device):
     gen = torch.Generator().manual_seed(seed)
     X = torch.randn(b, L, nh * P, generator=gen)
     p = torch.sigmoid(torch.randn(b, L, generator=gen) - 1.0)
     dt1 = -torch.log1p(-p)                                    # (b, L)
     ema = dict(A=torch.log1p(-p), X=X * p[..., None])         # the EMA kernels' inputs
-    Bm = torch.zeros(b, L, 1, NSTATE)
+    Bm = torch.zeros(b, L, 1, nstate)
     Bm[..., 0, 0] = p
-    Cm = torch.zeros(b, L, 1, NSTATE)
+    Cm = torch.zeros(b, L, 1, nstate)
     Cm[..., 0, 0] = 1.0
     ssd = dict(x=(X / dt1[..., None]).reshape(b, L, nh, P), dt=dt1[..., None].expand(b, L, nh).contiguous(),
                A=-torch.ones(nh), B=Bm, C=Cm)
@@ -32,16 +32,20 @@ def _encode(b, L, nh, P, seed, device):
     return to(ema), to(ssd)
 
 
-CASES = [(2, 512, 2, 64, 128), (1, 700, 4, 64, 256), (2, 300, 2, 128, 64)]  # b, L, nh, P, Q
+CASES = [  # b, L, nh, P, Q, state size
+    (2, 512, 2, 64, 128, 64), (1, 700, 4, 64, 256, 64), (2, 300, 2, 128, 64, 64),
+    (2, 512, 16, 32, 128, 1),   # HEAD_DIM 512 as 16 heads of 32: kernels/tests/ema/test_ema_scan_fwd.py:73-74
+    (1, 640, 2, 512, 128, 1),   # 1024 features as 2 heads: kernels/benchmarks/ema/scan_fwd/scan_fwd_bench.py:20-42
+]
 
 
-@pytest.mark.parametrize("b,L,nh,P,Q", CASES)
-def test_forward_agrees(b, L, nh, P, Q, device):
+@pytest.mark.parametrize("b,L,nh,P,Q,nstate", CASES)
+def test_forward_agrees(b, L, nh, P, Q, nstate, device):
     from kernels.ema_kernels.ema_combined_fwd import _ema_matmul_scan_combined_fwd
     from kernels.mamba_kernels.mamba_combined_fwd import _mamba_chunk_scan_combined_fwd
 
     announce(f"ema vs ssd forward b{b} L{L} nh{nh} P{P} Q{Q}")
-    ema, ssd = _encode(b, L, nh, P, seed=L + Q, device=device)
+    ema, ssd = _encode(b, L, nh, P, nstate, seed=L + Q, device=device)
     y_e, cs_e, prev_e, fin_e = _ema_matmul_scan_combined_fwd(ema["A"], ema["X"], Q)
     y_s, _, dt_out, dA_cs, prev_s, fin_s = _mamba_chunk_scan_combined_fwd(ssd["x"], ssd["dt"], ssd["A"], ssd["B"],
                                                                           ssd["C"], Q)
@@ -51,11 +55,12 @@ def test_forward_agrees(b, L, nh, P, Q, device):
     check_close("dA_cumsum", dA_cs[:, 0], cs_e.cpu(), F32)                      # the heads share one decay
     check_close("states entering the chunks", prev_s[..., 0].reshape(b, nc, nh * P), prev_e.cpu(), F32)
     check_close("final state", fin_s[..., 0].reshape(b, nh * P), fin_e.cpu(), F32)
-    assert float(prev_s[..., 1:].abs().max()) == 0.0 and float(fin_s[..., 1:].abs().max()) == 0.0
+    if nstate > 1:
+        assert float(prev_s[..., 1:].abs().max()) == 0.0 and float(fin_s[..., 1:].abs().max()) == 0.0
 
 
-@pytest.mark.parametrize("b,L,nh,P,Q", CASES)
-def test_backward_stages_agree(b, L, nh, P, Q, device):
+@pytest.mark.parametrize("b,L,nh,P,Q,nstate", CASES)
+def test_backward_stages_agree(b, L, nh, P, Q, nstate, device):
     from kernels.ema_kernels.ema_cumsum import ema_chunk_cumsum_fwd
     from kernels.ema_kernels_bwd.ema_scan_bwd import _ema_chunk_scan_bwd_dstates
     from kernels.ema_kernels_bwd.ema_state_passing_bwd_dstates import _ema_state_passing_bwd
@@ -64,7 +69,7 @@ def test_backward_stages_agree(b, L, nh, P, Q, device):
     from kernels.mamba_kernels_bwd.mamba_state_passing_bwd_dstates import _state_passing_bwd
 
     announce(f"ema vs ssd backward stages b{b} L{L} nh{nh} P{P} Q{Q}")
-    ema, ssd = _encode(b, L, nh, P, seed=2 * L + Q, device=device)
+    ema, ssd = _encode(b, L, nh, P, nstate, seed=2 * L + Q, device=device)
     gen = torch.Generator().manual_seed(L)
     dout = torch.randn(b, L, nh * P, generator=gen).to(device)
     cs_e = ema_chunk_cumsum_fwd(ema["A"], Q)
@@ -75,7 +80,8 @@ def test_backward_stages_agree(b, L, nh, P, Q, device):
     ds_e = _ema_chunk_scan_bwd_dstates(cs_e, dout)
     ds_s = _chunk_scan_bwd_dstates(ssd["C"], dA_cs, dout.reshape(b, L, nh, P), dtype=F32)
     check_close("dstates of the chunk scan", ds_s[..., 0].reshape(b, nc, nh * P), ds_e.cpu(), F32)
-    assert float(ds_s[..., 1:].abs().max()) == 0.0
+    if nstate > 1:
+        assert float(ds_s[..., 1:].abs().max()) == 0.0
 
     # reverse inter-chunk recurrence on the same flattened states
     states = torch.randn(b, nc, nh * P, generator=gen).to(device)

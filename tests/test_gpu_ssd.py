@@ -29,6 +29,14 @@ CASES = [
     (1, 150, 2, 64, 1, 64, 48),     # chunk sizes that are no multiple of the 64-row tiles
     (1, 333, 2, 64, 2, 64, 200),
     (1, 1100, 2, 64, 1, 128, 1024),  # the largest chunk size, second chunk ragged
+    # head and state sizes the kernels do not take natively (split into sub-heads / zero-padded
+    # around them); the reference's EMA tests and benchmarks call its Mamba launchers with
+    # dstate = 1 and head sizes 8, 32 and 512
+    (1, 200, 2, 32, 1, 1, 64),
+    (1, 300, 2, 512, 1, 1, 128),
+    (2, 150, 4, 8, 2, 16, 64),
+    (1, 260, 2, 200, 1, 100, 256),
+    (1, 100, 2, 6, 1, 1, 32),
 ]
 
 
@@ -113,11 +121,13 @@ def test_combined_vs_recurrence(b, L, nh, P, g, N, Q, dtype, device):
 def test_unsupported_shapes_are_refused(device):
     from kernels.mamba_kernels.mamba_state_fwd import _chunk_state_fwd
 
-    x = torch.zeros(1, 64, 2, 48, device=device)
+    x = torch.zeros(1, 64, 2, 64, device=device)
     B = torch.zeros(1, 64, 1, 64, device=device)
     dt = torch.zeros(1, 2, 1, 64, device=device)
-    with pytest.raises(NotImplementedError):
-        _chunk_state_fwd(B, x, dt, dt)
+    with pytest.raises(NotImplementedError):  # a state larger than 128
+        _chunk_state_fwd(torch.zeros(1, 64, 1, 256, device=device), x, dt, dt)
+    with pytest.raises(NotImplementedError):  # a chunk size that is no multiple of 4
+        _chunk_state_fwd(B[:, :62], x[:, :62], dt[..., :62], dt[..., :62])
     with pytest.raises(AssertionError):  # ids must be (batch, seqlen)
         _chunk_state_fwd(B, torch.zeros(1, 64, 2, 64, device=device), dt, dt, seq_idx=torch.zeros(1, 32, device=device))
 

@@ -22,6 +22,14 @@ CASES = [
     (1, 150, 2, 64, 1, 64, 48),     # chunk sizes that are no multiple of the 64-row tiles
     (1, 333, 2, 64, 2, 64, 200),
     (1, 1100, 2, 64, 1, 128, 1024),  # the largest chunk size, second chunk ragged
+    # head and state sizes the kernels do not take natively (split into sub-heads / zero-padded
+    # around them); the reference's EMA tests and benchmarks call its Mamba launchers with
+    # dstate = 1 and head sizes 8, 32 and 512
+    (1, 200, 2, 32, 1, 1, 64),
+    (1, 300, 2, 512, 1, 1, 128),
+    (2, 150, 4, 8, 2, 16, 64),
+    (1, 260, 2, 200, 1, 100, 256),
+    (1, 100, 2, 6, 1, 1, 32),
 ]
 
 

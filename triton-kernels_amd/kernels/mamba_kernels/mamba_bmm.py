@@ -8,6 +8,7 @@ import math
 import torch
 
 from kernels import _lib
+from kernels.mamba_kernels._shapes import Plan
 
 
 def _bmm_chunk_fwd(a, b, chunk_size, seq_idx=None, causal=False, output_dtype=None):
@@ -20,6 +21,10 @@ def _bmm_chunk_fwd(a, b, chunk_size, seq_idx=None, causal=False, output_dtype=No
         batch, seqlen, ngroups, k = a.shape
         a4, b4 = a, b
     assert b.shape == a.shape
+    plan = Plan(64, k)
+    if plan.N != k:  # a short contraction axis is padded with zeros
+        return _bmm_chunk_fwd(plan.bc(a), plan.bc(b), chunk_size, seq_idx=seq_idx, causal=causal,
+                              output_dtype=a.dtype if output_dtype is None else output_dtype)
     dev = _lib.require_gpu(a, b)
     seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)
     if b4.dtype != a4.dtype:

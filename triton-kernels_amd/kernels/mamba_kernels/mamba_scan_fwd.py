@@ -5,6 +5,7 @@ returns (out, out_x) like it."""
 import torch
 
 from kernels import _lib
+from kernels.mamba_kernels._shapes import Plan
 
 
 def _chunk_scan_fwd(cb, x, dt, dA_cumsum, C, states, D=None, z=None, seq_idx=None):
@@ -21,6 +22,11 @@ def _chunk_scan_fwd(cb, x, dt, dA_cumsum, C, states, D=None, z=None, seq_idx=Non
     assert dt.shape == (batch, nheads, nchunks, chunk_size)
     assert dA_cumsum.shape == (batch, nheads, nchunks, chunk_size)
     assert states.shape == (batch, nchunks, nheads, headdim, dstate)
+    plan = Plan(headdim, dstate)
+    if not plan.native:
+        out, out_x = _chunk_scan_fwd(cb, plan.x(x), plan.per_head(dt), plan.per_head(dA_cumsum), plan.bc(C),
+                                     plan.states(states), D=plan.D(D), z=plan.x(z), seq_idx=seq_idx)
+        return plan.x_back(out), plan.x_back(out_x)
     dev = _lib.require_gpu(x, cb, dt, dA_cumsum, C, states)
     seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)
     x, xs = _lib.strided4(x)

@@ -4,6 +4,7 @@ Mirrors _chunk_state_fwd, kernels/mamba_kernels/mamba_state_fwd.py:138-169 of th
 import torch
 
 from kernels import _lib
+from kernels.mamba_kernels._shapes import Plan
 
 
 def _chunk_state_fwd(B, x, dt, dA_cumsum, seq_idx=None, states=None, states_in_fp32=True):
@@ -14,6 +15,12 @@ def _chunk_state_fwd(B, x, dt, dA_cumsum, seq_idx=None, states=None, states_in_f
     assert B.shape == (batch, seqlen, ngroups, dstate)
     assert dt.shape == (batch, nheads, nchunks, chunk_size)
     assert dA_cumsum.shape == dt.shape
+    plan = Plan(headdim, dstate)
+    if not plan.native:  # bring the shape to one the kernels take, run, cut the result back
+        assert states is None, "a preallocated result needs a native shape"
+        out = _chunk_state_fwd(plan.bc(B), plan.x(x), plan.per_head(dt), plan.per_head(dA_cumsum), seq_idx=seq_idx,
+                               states_in_fp32=states_in_fp32)
+        return plan.states_back(out)
     dev = _lib.require_gpu(x, B, dt, dA_cumsum)
     if B.dtype != x.dtype:
         B = B.to(x.dtype)  # the reference rounds the weighted B to x's type before the product

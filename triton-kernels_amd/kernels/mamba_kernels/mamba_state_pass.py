@@ -2,6 +2,7 @@
 
 Mirrors _state_passing_fwd, kernels/mamba_kernels/mamba_state_pass.py:84-115 of the reference."""
 import torch
+import torch.nn.functional as F
 
 from kernels import _lib
 
@@ -12,6 +13,12 @@ def _state_passing_fwd(states, dA_chunk_cumsum, initial_states=None, seq_idx=Non
     assert dA_chunk_cumsum.shape == (batch, nheads, nchunks)
     if initial_states is not None:
         assert initial_states.shape == (batch, nheads, dim)
+    if dim % 4:  # the kernel moves four state elements per thread: pad with zeros, cut off again
+        pad = (0, -dim % 4)
+        out, final = _state_passing_fwd(F.pad(states, pad), dA_chunk_cumsum,
+                                        None if initial_states is None else F.pad(initial_states, pad),
+                                        seq_idx=seq_idx, chunk_size=chunk_size, out_dtype=out_dtype)
+        return out[..., :dim], final[..., :dim]
     dev = _lib.require_gpu(states, dA_chunk_cumsum)
     seqlen = 0
     if seq_idx is not None:

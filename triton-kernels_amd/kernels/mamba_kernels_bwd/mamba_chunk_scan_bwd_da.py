@@ -4,6 +4,7 @@ Mirrors _chunk_scan_bwd_ddAcs_stable, kernels/mamba_kernels_bwd/mamba_chunk_scan
 of the reference; the sum over row blocks that the reference takes in torch is part of the
 library call."""
 import torch
+import torch.nn.functional as F
 
 from kernels import _lib
 
@@ -17,6 +18,9 @@ def _chunk_scan_bwd_ddAcs_stable(x, dt, dA_cumsum, dout, cb):
     ngroups = cb.shape[2]
     assert nheads % ngroups == 0
     assert cb.shape == (batch, nchunks, ngroups, chunk_size, chunk_size)
+    if headdim % 8:  # rows move in 16-byte pieces: zero features change no dot product
+        pad = (0, -headdim % 8)
+        return _chunk_scan_bwd_ddAcs_stable(F.pad(x, pad), dt, dA_cumsum, F.pad(dout, pad), cb)
     dev = _lib.require_gpu(x, dt, dA_cumsum, dout, cb)
     lib = _lib.lib()
     x, xs = _lib.strided4(x)

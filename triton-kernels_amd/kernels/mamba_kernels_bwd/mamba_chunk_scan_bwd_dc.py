@@ -6,6 +6,7 @@ reference (no split axis: one workgroup walks all heads of a group)."""
 import torch
 
 from kernels import _lib
+from kernels.mamba_kernels._shapes import Plan
 
 
 def _chunk_scan_bwd_dC(prev_states, dA_cumsum, dout, seq_idx=None, C=None, ngroups=1):
@@ -15,6 +16,13 @@ def _chunk_scan_bwd_dC(prev_states, dA_cumsum, dout, seq_idx=None, C=None, ngrou
     assert prev_states.shape == (batch, nchunks, nheads, headdim, dstate)
     assert dA_cumsum.shape == (batch, nheads, nchunks, chunk_size)
     assert dout.shape == (batch, seqlen, nheads, headdim)
+    plan = Plan(headdim, dstate)
+    if not plan.native:
+        res = _chunk_scan_bwd_dC(plan.states(prev_states), plan.per_head(dA_cumsum), plan.x(dout), seq_idx=seq_idx,
+                                 C=plan.bc(C), ngroups=ngroups)
+        if C is None:
+            return plan.bc_back(res)
+        return plan.bc_back(res[0]), plan.per_head_sum(res[1])
     dev = _lib.require_gpu(prev_states, dA_cumsum, dout)
     seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)
     dout, ds = _lib.strided4(dout)

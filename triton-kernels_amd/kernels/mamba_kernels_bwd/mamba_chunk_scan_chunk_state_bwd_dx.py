@@ -7,6 +7,7 @@ and feature, which are added up here, as the reference adds its per-block partia
 import torch
 
 from kernels import _lib
+from kernels.mamba_kernels._shapes import Plan
 
 
 def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum, B, CB, dout, dstates, D=None, seq_idx=None, dx=None):
@@ -20,6 +21,13 @@ def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum, B, CB, dout, dstates, D=Non
     assert dA_cumsum.shape == dt.shape
     assert dout.shape == x.shape
     assert dstates.shape == (batch, nchunks, nheads, headdim, dstate)
+    plan = Plan(headdim, dstate)
+    if not plan.native:
+        assert dx is None, "a preallocated result needs a native shape"
+        dxs, ddt, dD = _chunk_scan_chunk_state_bwd_dx(plan.x(x), plan.per_head(dt), plan.per_head(dA_cumsum),
+                                                      plan.bc(B), CB, plan.x(dout), plan.states(dstates),
+                                                      D=plan.D(D), seq_idx=seq_idx)
+        return plan.x_back(dxs), plan.per_head_sum(ddt), plan.dD_back(dD, D)
     if D is not None:
         assert D.shape == (nheads, headdim) or D.shape == (nheads,)
     dev = _lib.require_gpu(x, dt, dA_cumsum, B, CB, dout, dstates)

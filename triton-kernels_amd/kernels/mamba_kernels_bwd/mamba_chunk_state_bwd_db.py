@@ -6,6 +6,7 @@ torch sum over it are gone; the cumsum of ddA_cumsum is part of the library call
 import torch
 
 from kernels import _lib
+from kernels.mamba_kernels._shapes import Plan
 
 
 def _chunk_state_bwd_db(x, dt, dA_cumsum, dstates, seq_idx=None, B=None, ngroups=1):
@@ -15,6 +16,13 @@ def _chunk_state_bwd_db(x, dt, dA_cumsum, dstates, seq_idx=None, B=None, ngroups
     assert dt.shape == (batch, nheads, nchunks, chunk_size)
     assert dA_cumsum.shape == dt.shape
     assert dstates.shape == (batch, nchunks, nheads, headdim, dstate)
+    plan = Plan(headdim, dstate)
+    if not plan.native:
+        res = _chunk_state_bwd_db(plan.x(x), plan.per_head(dt), plan.per_head(dA_cumsum), plan.states(dstates),
+                                  seq_idx=seq_idx, B=plan.bc(B), ngroups=ngroups)
+        if B is None:
+            return plan.bc_back(res)
+        return plan.bc_back(res[0]), plan.per_head_sum(res[1])
     dev = _lib.require_gpu(x, dt, dA_cumsum, dstates)
     seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)
     x, xs = _lib.strided4(x)

@@ -5,6 +5,7 @@ reference."""
 import torch
 
 from kernels import _lib
+from kernels.mamba_kernels._shapes import Plan
 
 
 def _chunk_scan_bwd_dstates(C, dA_cumsum, dout, seq_idx=None, dtype=None):
@@ -14,6 +15,11 @@ def _chunk_scan_bwd_dstates(C, dA_cumsum, dout, seq_idx=None, dtype=None):
     assert nheads % ngroups == 0
     assert C.shape == (batch, seqlen, ngroups, dstate)
     assert dA_cumsum.shape == (batch, nheads, nchunks, chunk_size)
+    plan = Plan(headdim, dstate)
+    if not plan.native:
+        out = _chunk_scan_bwd_dstates(plan.bc(C), plan.per_head(dA_cumsum), plan.x(dout), seq_idx=seq_idx,
+                                      dtype=C.dtype if dtype is None else dtype)
+        return plan.states_back(out)
     dev = _lib.require_gpu(C, dA_cumsum, dout)
     dtype = C.dtype if dtype is None else dtype
     seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)

@@ -3,6 +3,7 @@
 Mirrors _state_passing_bwd, kernels/mamba_kernels_bwd/mamba_state_passing_bwd_dstates.py:116-172
 of the reference (same arguments, same tuple of results)."""
 import torch
+import torch.nn.functional as F
 
 from kernels import _lib
 
@@ -14,6 +15,14 @@ def _state_passing_bwd(states, dA_chunk_cumsum, dout, dfinal_states=None, seq_id
     batch, nchunks, nheads, dim = states.shape
     assert dA_chunk_cumsum.shape == (batch, nheads, nchunks)
     assert dout.shape == (batch, nchunks, nheads, dim)
+    if dim % 4:  # the kernel moves four state elements per thread: pad with zeros, cut off again
+        pad = (0, -dim % 4)
+        res = _state_passing_bwd(F.pad(states, pad), dA_chunk_cumsum, F.pad(dout, pad),
+                                 None if dfinal_states is None else F.pad(dfinal_states, pad), seq_idx=seq_idx,
+                                 has_initial_states=has_initial_states, dstates_dtype=dstates_dtype,
+                                 states_dtype=states_dtype, chunk_size=chunk_size)
+        cut = lambda t: None if t is None else t[..., :dim]
+        return (cut(res[0]), res[1], cut(res[2])) + tuple(cut(t) for t in res[3:])
     if dfinal_states is not None:
         assert dfinal_states.shape == (batch, nheads, dim)
     dev = _lib.require_gpu(states, dA_chunk_cumsum, dout)
