@@ -90,3 +90,35 @@ def test_backward_stages_agree(b, L, nh, P, Q, nstate, device):
     g_s, ddA_s, _ = _state_passing_bwd(st4, dA_cs[:, :, :, -1], ds_e.reshape(b, nc, nh, P), chunk_size=Q)
     check_close("dstates of state passing", g_s.reshape(b, nc, nh * P), g_e.cpu(), F32)
     check_close("ddA of the chunk decays (summed over heads)", ddA_s.sum(1), ddA_e.cpu(), F32)
+
+
+def test_main_script_flow(device):
+    """The three providers of the reference's main.py:77-143 on its own shapes (batch 2, length
+    512, 64 features as 2 heads of 32, chunk size 8): the (x, p) entry point, the Mamba-encoded
+    EMA entry point and the Mamba forward itself (main.py takes that one from mamba_ssm) against
+    the loop z = (1 - p) z + p x."""
+    from kernels.ema import ema_scan_combined
+    from kernels.ema_combined import ema_chunk_scan_combined
+    from kernels.mamba_kernels.mamba_combined_fwd import mamba_chunk_scan_combined_fwd
+
+    announce("main.py flow: ema_scan_combined, ema_chunk_scan_combined, mamba forward")
+    b, L, D, hd, nh, Q = 2, 512, 64, 32, 2, 8
+    gen = torch.Generator().manual_seed(42)
+    X = torch.randn(b, L, D, generator=gen)
+    P = torch.rand(b, L, 1, generator=gen) * 0.98 + 0.01
+    ref = torch.empty_like(X)
+    z = torch.zeros(b, D)
+    for t in range(L):
+        z = (1 - P[:, t]) * z + P[:, t] * X[:, t]
+        ref[:, t] = z
+    dt1 = -torch.log(1 - P).squeeze(-1)
+    X_m = (X / dt1[..., None]).reshape(b, L, nh, hd).to(device)
+    dt = dt1[..., None].expand(b, L, nh).contiguous().to(device)
+    A = -torch.ones(nh, device=device)
+    B_m = P.reshape(b, L, 1, 1).to(device)
+    C_m = torch.ones_like(B_m)
+    check_close("ema_scan_combined(X, P)", ema_scan_combined(X.to(device), P.to(device)), ref, F32)
+    got = ema_chunk_scan_combined(X_m, dt, A, B_m, C_m, chunk_size=Q, seq_idx=None)
+    check_close("ema_chunk_scan_combined", got.reshape(b, L, D), ref, F32)
+    got = mamba_chunk_scan_combined_fwd(X_m, dt, A, B_m, C_m, Q)
+    check_close("mamba forward", got.reshape(b, L, D), ref, F32)
