@@ -362,6 +362,17 @@ __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
   }
 }
 
+// Non-temporal 16-byte accesses for data that a kernel touches once.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 stream_load4(const float* p) {
+  const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
+  return make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void stream_store4(float* p, float4 v) {
+  const f32x4 w = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(w, reinterpret_cast<f32x4*>(p));
+}
+
 // ------------------------------------------------------------------------------------
 // state_passing.  out[b, c] = state entering chunk c, state <- exp(dA_chunk[c]) * state +
 // states[b, c]; the value after the last chunk goes to final.  One thread per four adjacent
@@ -392,7 +403,7 @@ __global__ __launch_bounds__(256) void ssd_state_passing_kernel(
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int c = c0 + u;
-      nv[u] = c < C ? *reinterpret_cast<const float4*>(src + c * chunk_stride) : make_float4(0.f, 0.f, 0.f, 0.f);
+      nv[u] = c < C ? stream_load4(src + c * chunk_stride) : make_float4(0.f, 0.f, 0.f, 0.f);
       a[u] = c < C ? __expf(da[(int64_t)c * da_sc]) : 0.f;
       if (c < C && !chunk_keeps_state(seq, b, c, Q, L)) a[u] = 0.f;
     }
@@ -400,7 +411,7 @@ __global__ __launch_bounds__(256) void ssd_state_passing_kernel(
     for (int u = 0; u < U; ++u) {
       const int c = c0 + u;
       if (c < C) {
-        *reinterpret_cast<float4*>(dst + c * chunk_stride) = s;
+        stream_store4(dst + c * chunk_stride, s);
         s.x = fmaf(a[u], s.x, nv[u].x);
         s.y = fmaf(a[u], s.y, nv[u].y);
         s.z = fmaf(a[u], s.z, nv[u].z);
@@ -454,8 +465,8 @@ __global__ __launch_bounds__(256) void ssd_state_passing_bwd_kernel(
     for (int u = 0; u < U; ++u) {
       const int c = c1 - u;
       const bool in = c >= 0 && ok;
-      sv[u] = in ? *reinterpret_cast<const float4*>(states + base + c * chunk_stride) : zero4;
-      dv[u] = in ? *reinterpret_cast<const float4*>(dout + base + c * chunk_stride) : zero4;
+      sv[u] = in ? stream_load4(states + base + c * chunk_stride) : zero4;
+      dv[u] = in ? stream_load4(dout + base + c * chunk_stride) : zero4;
       a[u] = c >= 0 ? __expf(da[(int64_t)c * da_sc]) : 0.f;
       if (c >= 0 && !chunk_keeps_state(seq, b, c, Q, L)) a[u] = 0.f;
     }
@@ -463,7 +474,7 @@ __global__ __launch_bounds__(256) void ssd_state_passing_bwd_kernel(
     for (int u = 0; u < U; ++u) {
       const int c = c1 - u;
       if (c >= 0) {  // uniform across the workgroup
-        if (ok) *reinterpret_cast<float4*>(dstates + base + c * chunk_stride) = G;
+        if (ok) stream_store4(dstates + base + c * chunk_stride, G);
         const float dot = ema::wave_sum(sv[u].x * G.x + sv[u].y * G.y + sv[u].z * G.z + sv[u].w * G.w);
         if (lane == 0) part[((b * nh + h) * C + c) * (int64_t)nw + wave_id] = dot;
         G.x = fmaf(a[u], G.x, dv[u].x);
