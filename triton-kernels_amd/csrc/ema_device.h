@@ -105,6 +105,28 @@ __device__ __forceinline__ void store16(T* p, const Vec16<T>& v) {
   *reinterpret_cast<decltype(v.raw)*>(p) = v.raw;
 }
 
+// The same with the non-temporal hint, for global data that the kernel touches once and no other
+// workgroup is about to read through the same L2.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ Vec16<float> load16_stream(const float* p) {
+  const f32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(p));
+  Vec16<float> v;
+  v.raw = make_float4(t[0], t[1], t[2], t[3]);
+  return v;
+}
+__device__ __forceinline__ Vec16<bf16_t> load16_stream(const bf16_t* p) {
+  Vec16<bf16_t> v;
+  v.raw = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(p));
+  return v;
+}
+__device__ __forceinline__ void store16_stream(float* p, const Vec16<float>& v) {
+  const f32x4_t t = {v.raw.x, v.raw.y, v.raw.z, v.raw.w};
+  __builtin_nontemporal_store(t, reinterpret_cast<f32x4_t*>(p));
+}
+__device__ __forceinline__ void store16_stream(bf16_t* p, const Vec16<bf16_t>& v) {
+  __builtin_nontemporal_store(v.raw, reinterpret_cast<bf16x8*>(p));
+}
+
 // ------------------------------------------------------------------ MFMA groups
 // One "group" multiplies a 32 x KG tile by a KG x 32 tile, KG = 2 * Vec16<T>::N.  A lane
 // holds Vec16<T>::N consecutive k of row (lane % 32), starting at k = N * (lane / 32),

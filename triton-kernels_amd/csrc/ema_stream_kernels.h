@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256) void chunk_reduce_kernel(
       // complete before the next one is issued); what lies outside gets weight 0
       const int q = q0 + u * rows_par;
       const int qc = min(q, limit - 1);
-      v[u] = load16(xq + (int64_t)qc * sx.sl);
+      v[u] = load16_stream(xq + (int64_t)qc * sx.sl);
       const float a = csp[qc];
       const float wt = MODE == 0 ? __expf(fminf(cs_last - a, 0.f)) : __expf(a);
       w[u] = (q < limit && col_ok) ? wt : 0.f;
@@ -263,7 +263,7 @@ __global__ __launch_bounds__(256) void row_dot_kernel(const T* __restrict__ x, S
       Vec16<T> v[R];
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        v[r] = load16(xp + (int64_t)min(m0 + r, limit - 1) * sx.sl + col);
+        v[r] = load16_stream(xp + (int64_t)min(m0 + r, limit - 1) * sx.sl + col);
         if (m0 + r >= limit) v[r].zero();
       }
 #pragma unroll

@@ -76,7 +76,7 @@ __device__ __forceinline__ void walk_load_tile(T* tile, const T* __restrict__ g,
   for (int p = 0; p < kTileRows / C::RPP; ++p) {
     const int r = tid / C::VPR + p * C::RPP;
     // unconditional load from a row and column clamped into the tensor, zeroed afterwards
-    v[p] = load16(g + (int64_t)min(tb + r, limit - 1) * sl + (cok ? col0 + vcol : 0));
+    v[p] = load16_stream(g + (int64_t)min(tb + r, limit - 1) * sl + (cok ? col0 + vcol : 0));
     if (tb + r >= limit || !cok) v[p].zero();
   }
 #pragma unroll
@@ -258,7 +258,7 @@ __device__ __forceinline__ void walk_store_rows(const T* tile, T* __restrict__ g
   for (int p = 0; p < 32 / RPW; ++p) {
     const int r = 32 * wave + p * RPW + lane / C::VPR;
     if (tb + r < limit)
-      store16(g + (int64_t)(tb + r) * sl + col0 + vcol, load16(&tile[r * C::ROW + vcol]));
+      store16_stream(g + (int64_t)(tb + r) * sl + col0 + vcol, load16(&tile[r * C::ROW + vcol]));
   }
 }
 

@@ -25,8 +25,10 @@ using ema::acc_row;
 using ema::bf16_t;
 using ema::floatx16;
 using ema::load16;
+using ema::load16_stream;
 using ema::mma_group;
 using ema::store16;
+using ema::store16_stream;
 using ema::Vec16;
 using ema::wave_inclusive_scan;
 
@@ -133,7 +135,9 @@ struct NoScale {
   __device__ __forceinline__ float operator()(int) const { return 1.f; }
 };
 
-template <typename T, int ROWS, int COLS, typename F>
+// STREAM: the rows are read with the non-temporal hint (data of one head that no other workgroup
+// is about to read through the same L2).
+template <typename T, int ROWS, int COLS, typename F, bool STREAM = false>
 __device__ __forceinline__ void stage_rows(T* tile, const T* __restrict__ g, int64_t row_stride, int row0,
                                            int limit, int tid, F scale) {
   constexpr int EPL = Vec16<T>::N, VPR = COLS / EPL, P = Tile<T>::pitch(COLS);
@@ -152,7 +156,7 @@ __device__ __forceinline__ void stage_rows(T* tile, const T* __restrict__ g, int
       const int idx = tid + 256 * (i0 + i);
       const int r = idx / VPR, cv = (idx % VPR) * EPL;
       const int row = row0 + r < limit ? row0 + r : limit - 1;
-      v[i] = load16(g + (int64_t)row * row_stride + cv);
+      v[i] = STREAM ? load16_stream(g + (int64_t)row * row_stride + cv) : load16(g + (int64_t)row * row_stride + cv);
     }
     asm volatile("" ::: "memory");
 #pragma unroll
@@ -183,6 +187,7 @@ struct RowPieces {
   static_assert((ROWS * VPR) % 256 == 0 && CNT <= 8, "tile must split evenly over 256 threads");
   Vec16<T> v[CNT];
   float a0[CNT], a1[CNT];
+  template <bool STREAM = false>
   __device__ __forceinline__ void load(const T* __restrict__ g, int64_t row_stride, int row0, int limit, int tid,
                                        const float* __restrict__ aux0 = nullptr,
                                        const float* __restrict__ aux1 = nullptr) {
@@ -190,7 +195,8 @@ struct RowPieces {
     for (int i = 0; i < CNT; ++i) {
       const int idx = tid + 256 * i;
       const int row = min(row0 + idx / VPR, limit - 1);
-      v[i] = load16(g + (int64_t)row * row_stride + (idx % VPR) * EPL);
+      const T* src = g + (int64_t)row * row_stride + (idx % VPR) * EPL;
+      v[i] = STREAM ? load16_stream(src) : load16(src);
       if (aux0) a0[i] = aux0[row];
       if (aux1) a1[i] = aux1[row];
     }
@@ -326,7 +332,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
   RowPieces<T, KT, P> px;
   RowPieces<T, KT, N> pb;
   auto request = [&](int k0) {  // the pieces of a stage and the per-row values their scale needs
-    px.load(xg, sx.sl, k0, limit, tid, MODE == 1 ? dAp : nullptr);
+    px.template load<true>(xg, sx.sl, k0, limit, tid, MODE == 1 ? dAp : nullptr);
     pb.load(Bg, sB.sl, k0, limit, tid, MODE == 0 ? dAp : nullptr, MODE == 0 ? dtp : nullptr);
   };
   request(0);
@@ -358,7 +364,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
     const int j = wave + 4 * i, mi = j % MB, ni = j / MB;
 #pragma unroll
     for (int v = 0; v < 16; ++v)
-      out[(int64_t)(32 * mi + acc_row(v, lane)) * N + 32 * ni + (lane & 31)] = acc[i][v];
+      __builtin_nontemporal_store(acc[i][v], out + (int64_t)(32 * mi + acc_row(v, lane)) * N + 32 * ni + (lane & 31));
   }
 }
 
@@ -1001,7 +1007,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
     for (int i = 0; i < P * VPR / 256; ++i) {
       const int idx = tid + 256 * i;
       const int r = idx / VPR, cv = (idx % VPR) * 4;
-      const float4 v = *reinterpret_cast<const float4*>(pg + (int64_t)r * N + cv);
+      const float4 v = stream_load4(pg + (int64_t)r * N + cv);
       T* d = Pv + r * S::PC + cv;
       d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
     }
@@ -1038,7 +1044,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
   SSD_TSTAMP(3);
   for (int kt = 0; kt <= st; ++kt) {
     const int k0 = ST * kt;
-    stage_rows<T, ST, P>(Xs, xg, sx.sl, k0, limit, tid, NoScale());
+    stage_rows<T, ST, P, NoScale, true>(Xs, xg, sx.sl, k0, limit, tid, NoScale());
     {
       // Below the diagonal the weight of (m, k) is split at the last position r of k's group of
       // 32: exp(dA_m - dA_r) is one exponential per row and group, exp(dA_r - dA_k) * dt_k one
@@ -1147,7 +1153,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
           }
         }
         o.set_all(v);
-        store16(out + b * so.sb + pos * so.sl + h * so.sh + cv, o);
+        store16_stream(out + b * so.sb + pos * so.sl + h * so.sh + cv, o);
       }
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
@@ -1392,9 +1398,9 @@ __global__ __launch_bounds__(256) void ssd_ddA_causal_kernel(
   SSD_TSTAMP(0);
   // shared: the chunk's x rows (zero past the limit), dA, dt; cleared: the sums
   static_assert(S::PX == Tile<T>::pitch(P), "stage_rows writes rows at this pitch");
-  if (Q == 256) stage_rows<T, 256, P>(Xs, xg, sx.sl, 0, limit, tid, NoScale());
-  else if (Q == 128) stage_rows<T, 128, P>(Xs, xg, sx.sl, 0, limit, tid, NoScale());
-  else stage_rows<T, 64, P>(Xs, xg, sx.sl, 0, limit, tid, NoScale());
+  if (Q == 256) stage_rows<T, 256, P, NoScale, true>(Xs, xg, sx.sl, 0, limit, tid, NoScale());
+  else if (Q == 128) stage_rows<T, 128, P, NoScale, true>(Xs, xg, sx.sl, 0, limit, tid, NoScale());
+  else stage_rows<T, 64, P, NoScale, true>(Xs, xg, sx.sl, 0, limit, tid, NoScale());
   if (tid < Q) {
     dAs[tid] = dA_cs[chunk * Q + tid];
     dts[tid] = dt[chunk * Q + tid];
@@ -1548,7 +1554,7 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
     for (int i = 0; i < P * VPR / 256; ++i) {
       const int idx = tid + 256 * i;
       const int r = idx / VPR, cv = (idx % VPR) * 4;
-      const float4 v = *reinterpret_cast<const float4*>(sg + (int64_t)r * N + cv);
+      const float4 v = stream_load4(sg + (int64_t)r * N + cv);
       T* d = Pv + r * S::PC + cv;
       d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
     }
@@ -1639,7 +1645,7 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
         const int r = idx / VPR, cv = (idx % VPR) * EPL;
         const int m = m0 + mrow[mb] + r;
         const int64_t pos = (int64_t)c * Q + min(m, limit - 1);
-        xv[i] = load16(x + b * sx.sb + pos * sx.sl + h * sx.sh + cv);
+        xv[i] = load16_stream(x + b * sx.sb + pos * sx.sl + h * sx.sh + cv);
         dtm[i] = dtp[m];
         if (D) dv[i] = load16(dout + b * sd.sb + pos * sd.sl + h * sd.sh + cv);
       }
@@ -1660,7 +1666,7 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
       if constexpr (kEarly) {
         xi = xv[i], di = dv[i], dti = dtm[i];
       } else {
-        xi = load16(x + b * sx.sb + pos * sx.sl + h * sx.sh + cv);
+        xi = load16_stream(x + b * sx.sb + pos * sx.sl + h * sx.sh + cv);
         dti = dtp[m];
         if (D) di = load16(dout + b * sd.sb + pos * sd.sl + h * sd.sh + cv);
       }
@@ -1682,7 +1688,7 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
       if (m < limit) {
         Vec16<T> o;
         o.set_all(v);
-        store16(dx + b * sdx.sb + pos * sdx.sl + h * sdx.sh + cv, o);
+        store16_stream(dx + b * sdx.sb + pos * sdx.sl + h * sdx.sh + cv, o);
       }
 #pragma unroll
       for (int off = 1; off < VPR; off <<= 1) dot += __shfl_xor(dot, off);
