@@ -27,7 +27,7 @@ for p in (ROOT, os.path.join(ROOT, "triton-kernels_amd")):
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), scaled by
 # what the same counters read for a plain 268 435 456-byte device copy (FETCH_SIZE reads
 # 131 085 KiB for it, factor 1.99982; WRITE_SIZE reads 262 144 KiB, factor 1).
-TRAFFIC_BYTES = {"fwd_single_pass": 591160982, "bwd_single_pass": 841346755}
+TRAFFIC_BYTES = {"fwd_single_pass": 589083033, "bwd_single_pass": 841025145}
 # the same for the SSD stage kernels at configuration 5 (finishing kernels added to their stage)
 SSD_TRAFFIC_BYTES = {
     "chunk_cumsum": 25728185, "chunk_state": 571561815, "state_passing": 553727051, "bmm_chunk": 100777471,
