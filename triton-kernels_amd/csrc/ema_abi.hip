@@ -293,14 +293,22 @@ inline ChainWs chain_carve(void* base, const Dims& di) {
 }
 
 // Clears the words of cols column sets of BN columns; the virtual slot (0 forward, C reverse)
-// carries `seed` (N, T), or 0.
+// carries `seed` (N, T), or 0.  With cs_out the same launch also computes the cumsum of the
+// coefficient over the 128-row tiles (prob = 1: the coefficient is a probability), which the
+// look-back of the kernel that follows reads: one launch and one gap less per pass.
 int launch_chain_init(const ChainWs& w, int64_t cols, int BN, const Dims& di, bool reverse,
-                      const float* seed, int ntiles, hipStream_t st) {
+                      const float* seed, int ntiles, hipStream_t st, const float* A = nullptr,
+                      SeqStrides sa = SeqStrides{0, 0, 0}, float* cs_out = nullptr, int prob = 0) {
   const int64_t pairs = cols * (di.C + 1) * BN / 2;
   const int64_t threads = pairs > 4 ? pairs : 4;
-  hipLaunchKernelGGL(chain_init_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st,
+  const int64_t init_blocks = (threads + 255) / 256;
+  const int64_t chunks = di.N * di.C;
+  const int64_t cumsum_blocks = cs_out ? (chunks + 3) / 4 : 0;
+  if (init_blocks + cumsum_blocks > 0x7fffffff) return EMA_ERR_SHAPE;
+  hipLaunchKernelGGL(chain_init_kernel, dim3((unsigned)(init_blocks + cumsum_blocks)), dim3(256), 0, st,
                      reinterpret_cast<uint4*>(w.status), pairs, w.counters, BN, (int)di.C + 1,
-                     reverse ? (int)di.C : 0, ntiles, (int)di.T, seed);
+                     reverse ? (int)di.C : 0, ntiles, (int)di.T, seed, (int)init_blocks, A, sa, cs_out,
+                     (int)di.nh, (int)di.L, (int)di.C, chunks, prob);
   return launched();
 }
 
@@ -314,8 +322,9 @@ struct TileF32 {
   static constexpr int FWD_CPL = 2, BWD_CPL = 2, RPL = 8, FWD_MINW = 8, BWD_MINW = 4;
 };
 
+// cs128 is computed by the set-up launch (the caller does not launch a cumsum for it).
 template <typename T, typename S, bool XP>
-int launch_fwd_tile_t(const void* x, SeqStrides sx, const float* A, SeqStrides sa, const float* cs128,
+int launch_fwd_tile_t(const void* x, SeqStrides sx, const float* A, SeqStrides sa, float* cs128,
                       void* y, SeqStrides sy, float* prev128, float* prev_coarse, int ratio, float* fin,
                       const float* init, const ChainWs& w, const Dims& di, hipStream_t st, void* ev0,
                       void* ev1) {
@@ -324,30 +333,32 @@ int launch_fwd_tile_t(const void* x, SeqStrides sx, const float* A, SeqStrides s
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
-  EMA_TRY(launch_chain_init(w, cols, BN, di, false, init, ntiles, st));
+  EMA_TRY(launch_chain_init(w, cols, BN, di, false, init, ntiles, st, A, sa, cs128, XP ? 1 : 0));
   auto kernel = fwd_tile_kernel<T, S::FWD_CPL, S::RPL, S::FWD_MINW, XP>;
   const int64_t cap = resident_blocks(kernel, NT, 0);
   launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx, A,
-               sa, cs128, (T*)y, sy, prev128, prev_coarse, ratio, fin, init ? 1 : 0, w.status, w.counters,
+               sa, (const float*)cs128, (T*)y, sy, prev128, prev_coarse, ratio, fin, init ? 1 : 0, w.status, w.counters,
                (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total);
   return launched();
 }
 
+// cumsum_here: cs128 is computed by the set-up launch; otherwise the caller has filled it.
 template <typename T, typename S, bool WRITE_Y, bool XP>
 int launch_bwd_tile_k(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* A,
-                      SeqStrides sa, const float* cs128, const float* prev128, void* dx, SeqStrides sdx,
-                      void* y, SeqStrides sy, float* part, const float* dfinal, float* dinit,
+                      SeqStrides sa, float* cs128, bool cumsum_here, const float* prev128, void* dx,
+                      SeqStrides sdx, void* y, SeqStrides sy, float* part, const float* dfinal, float* dinit,
                       const ChainWs& w, const Dims& di, hipStream_t st, void* ev0, void* ev1) {
   using Cfg = TileCfg<T, S::BWD_CPL, S::RPL>;
   constexpr int BN = Cfg::BN, NT = Cfg::NT;
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
-  EMA_TRY(launch_chain_init(w, cols, BN, di, true, dfinal, ntiles, st));
+  EMA_TRY(launch_chain_init(w, cols, BN, di, true, dfinal, ntiles, st, A, sa, cumsum_here ? cs128 : nullptr,
+                            XP ? 1 : 0));
   auto kernel = bwd_tile_kernel<T, S::BWD_CPL, S::RPL, S::BWD_MINW, WRITE_Y, XP>;
   const int64_t cap = resident_blocks(kernel, NT, 0);
   launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx,
-               (const T*)dy, sd, A, sa, cs128, prev128, (T*)dx, sdx, (T*)y, sy, part, dfinal ? 1 : 0, dinit,
+               (const T*)dy, sd, A, sa, (const float*)cs128, prev128, (T*)dx, sdx, (T*)y, sy, part, dfinal ? 1 : 0, dinit,
                w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols,
                (int)total);
   return launched();
@@ -355,14 +366,14 @@ int launch_bwd_tile_k(const void* x, SeqStrides sx, const void* dy, SeqStrides s
 
 template <typename T, typename S, bool XP>
 int launch_bwd_tile_t(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* A,
-                      SeqStrides sa, const float* cs128, const float* prev128, void* dx, SeqStrides sdx,
-                      void* y, SeqStrides sy, float* part, const float* dfinal, float* dinit,
+                      SeqStrides sa, float* cs128, bool cumsum_here, const float* prev128, void* dx,
+                      SeqStrides sdx, void* y, SeqStrides sy, float* part, const float* dfinal, float* dinit,
                       const ChainWs& w, const Dims& di, hipStream_t st, void* ev0, void* ev1) {
   if (y)
-    return launch_bwd_tile_k<T, S, true, XP>(x, sx, dy, sd, A, sa, cs128, prev128, dx, sdx, y, sy, part,
-                                             dfinal, dinit, w, di, st, ev0, ev1);
-  return launch_bwd_tile_k<T, S, false, XP>(x, sx, dy, sd, A, sa, cs128, prev128, dx, sdx, nullptr, sy, part,
-                                            dfinal, dinit, w, di, st, ev0, ev1);
+    return launch_bwd_tile_k<T, S, true, XP>(x, sx, dy, sd, A, sa, cs128, cumsum_here, prev128, dx, sdx, y, sy,
+                                             part, dfinal, dinit, w, di, st, ev0, ev1);
+  return launch_bwd_tile_k<T, S, false, XP>(x, sx, dy, sd, A, sa, cs128, cumsum_here, prev128, dx, sdx, nullptr,
+                                            sy, part, dfinal, dinit, w, di, st, ev0, ev1);
 }
 
 template <typename S>
@@ -501,19 +512,16 @@ int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void
     return EMA_ERR_SHAPE;
   hipStream_t st = as_stream(stream);
   const SeqStrides sx{x_sb, x_sl, x_sh}, sy{y_sb, y_sl, y_sh}, sa{a_sb, a_sl, a_sh};
-  EMA_TRY(launch_cumsum(A, sa, cs, d, st));
+  if (chunk != kTileRows) EMA_TRY(launch_cumsum(A, sa, cs, d, st));
   if (chunk % kTileRows == 0) {
     // Single pass over x: the scan is computed on 128-row chunks with the inter-chunk state
     // handed over inside the kernel; the states at the caller's chunk boundaries are every
-    // (chunk/128)-th of them.
+    // (chunk/128)-th of them.  The cumsum over the 128-row chunks is part of the kernel's set-up
+    // launch; for chunk = 128 it is the caller's cs.
     const Dims di = internal_dims(d);
     const FwdWs w = carve_fwd(workspace, di);
     const int ratio = (int)(chunk / kTileRows);
-    const float* cs128 = cs;
-    if (ratio != 1) {
-      EMA_TRY(launch_cumsum(A, sa, w.cs128, di, st));
-      cs128 = w.cs128;
-    }
+    float* cs128 = ratio == 1 ? cs : w.cs128;
     float* p128 = prev128 ? prev128 : (ratio == 1 ? prev : w.prev128);
     float* coarse = p128 == prev ? nullptr : prev;
     if (dtype == EMA_BF16) {
@@ -699,10 +707,11 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
   const SeqStrides sy{y_sb, y_sl, y_sh};
 
   const SeqStrides sa{a_sb, a_sl, a_sh};
-  EMA_TRY(launch_cumsum(A, sa, w.cs, di, st));
+  const bool cumsum_here = prev128 != nullptr;  // otherwise the recomputation below needs cs first
   if (!prev128) {
     // states entering each chunk, recomputed: chunk states, then the inter-chunk recurrence
     // (its final state is not needed and lands in `part`, which is free until the main kernel)
+    EMA_TRY(launch_cumsum(A, sa, w.cs, di, st));
     EMA_TRY(launch_chunk_reduce<0>(x, sx, dtype, w.cs, w.states, di, st));
     EMA_TRY(launch_state_passing_fwd(w.states, w.cs + (di.Q - 1), di.C * di.Q, di.Q, w.prev,
                                      w.part, di.N, di.C, di.T, st));
@@ -712,11 +721,11 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
   // the reverse inter-chunk state is handed over inside the kernel
   int parts = dtype == EMA_BF16 ? tile_parts_per_dim<TileBf16>(di.T) : tile_parts_per_dim<TileF32>(di.T);
   if (dtype == EMA_BF16) {
-    EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, false>(x, sx, dy, sd, A, sa, w.cs, prev128, dx, sdx, y, sy,
+    EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, false>(x, sx, dy, sd, A, sa, w.cs, cumsum_here, prev128, dx, sdx, y, sy,
                                                         w.part, nullptr, nullptr, w.chain, di, st, ev_start,
                                                         ev_stop)));
   } else
-    EMA_TRY((launch_bwd_tile_t<float, TileF32, false>(x, sx, dy, sd, A, sa, w.cs, prev128, dx, sdx, y, sy,
+    EMA_TRY((launch_bwd_tile_t<float, TileF32, false>(x, sx, dy, sd, A, sa, w.cs, cumsum_here, prev128, dx, sdx, y, sy,
                                                       w.part, nullptr, nullptr, w.chain, di, st, ev_start,
                                                       ev_stop)));
   const int64_t total = d.N * d.C * d.Q;
@@ -812,8 +821,7 @@ int ema_seq_fwd(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t
   hipStream_t st = as_stream(stream);
   const SeqWs w = carve_seq(workspace, d, false);
   const SeqStrides sx{x_sb, x_sl, x_sh}, sy{y_sb, y_sl, y_sh}, sc{c_sb, c_sl, c_sh};
-  const bool xp = form == EMA_FORM_PROBABILITY;
-  EMA_TRY(launch_cumsum(coef, sc, w.cs, d, st, xp ? 1 : 0));
+  const bool xp = form == EMA_FORM_PROBABILITY;  // the cumsum of the coefficient is part of the set-up launch
   if (dtype == EMA_BF16) {
     if (xp)
       return launch_fwd_tile_t<bf16_t, TileBf16, true>(x, sx, coef, sc, w.cs, y, sy, prev128, nullptr, 1,
@@ -855,27 +863,26 @@ int ema_seq_bwd(int form, const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t 
   const SeqWs w = carve_seq(workspace, d, true);
   const SeqStrides sx{x_sb, x_sl, x_sh}, sd{dy_sb, dy_sl, dy_sh}, sdx{dx_sb, dx_sl, dx_sh};
   const SeqStrides sc{c_sb, c_sl, c_sh}, none{0, 0, 0};
-  const bool xp = form == EMA_FORM_PROBABILITY;
-  EMA_TRY(launch_cumsum(coef, sc, w.cs, d, st, xp ? 1 : 0));
+  const bool xp = form == EMA_FORM_PROBABILITY;  // the cumsum of the coefficient is part of the set-up launch
   int parts;
   if (dtype == EMA_BF16) {
     parts = tile_parts_per_dim<TileBf16>(d.T);
     if (xp)
-      EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, true>(x, sx, dy, sd, coef, sc, w.cs, prev128, dx, sdx, nullptr,
+      EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, true>(x, sx, dy, sd, coef, sc, w.cs, true, prev128, dx, sdx, nullptr,
                                                          none, w.part, dfinal, dinit, w.chain, d, st, ev_start,
                                                          ev_stop)));
     else
-      EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, false>(x, sx, dy, sd, coef, sc, w.cs, prev128, dx, sdx,
+      EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, false>(x, sx, dy, sd, coef, sc, w.cs, true, prev128, dx, sdx,
                                                           nullptr, none, w.part, dfinal, dinit, w.chain, d, st,
                                                           ev_start, ev_stop)));
   } else {
     parts = tile_parts_per_dim<TileF32>(d.T);
     if (xp)
-      EMA_TRY((launch_bwd_tile_t<float, TileF32, true>(x, sx, dy, sd, coef, sc, w.cs, prev128, dx, sdx, nullptr,
+      EMA_TRY((launch_bwd_tile_t<float, TileF32, true>(x, sx, dy, sd, coef, sc, w.cs, true, prev128, dx, sdx, nullptr,
                                                        none, w.part, dfinal, dinit, w.chain, d, st, ev_start,
                                                        ev_stop)));
     else
-      EMA_TRY((launch_bwd_tile_t<float, TileF32, false>(x, sx, dy, sd, coef, sc, w.cs, prev128, dx, sdx, nullptr,
+      EMA_TRY((launch_bwd_tile_t<float, TileF32, false>(x, sx, dy, sd, coef, sc, w.cs, true, prev128, dx, sdx, nullptr,
                                                         none, w.part, dfinal, dinit, w.chain, d, st, ev_start,
                                                         ev_stop)));
   }

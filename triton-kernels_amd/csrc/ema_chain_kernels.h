@@ -60,10 +60,20 @@ __device__ __forceinline__ unsigned chain_wait(const u64* p, float* v, unsigned*
 // last (reverse: slot C, tiles at slot c).  Tile slots are zeroed; the virtual slot carries
 // PREFIX with the state that enters the scan from outside, seed[n, column] or 0.  Each thread
 // writes two adjacent words (BN is even, so both lie in one slot).
+// The set-up of a single-pass kernel in one launch: the first init_blocks workgroups clear the
+// status words (and seed the virtual slot), the rest, if any, compute the per-tile cumsum of the
+// log-decay that the look-back reads (cumsum_block; cs null = no such workgroups are launched).
 __global__ __launch_bounds__(256) void chain_init_kernel(uint4* __restrict__ words, int64_t n_pairs,
                                                          unsigned* __restrict__ counters, int BN,
                                                          int slots, int virt_slot, int ntiles, int Tdim,
-                                                         const float* __restrict__ seed) {
+                                                         const float* __restrict__ seed, int init_blocks,
+                                                         const float* __restrict__ A, SeqStrides sa,
+                                                         float* __restrict__ cs, int nh, int L, int C,
+                                                         int64_t total_chunks, int prob) {
+  if ((int)blockIdx.x >= init_blocks) {
+    cumsum_block((int64_t)blockIdx.x - init_blocks, A, sa, cs, nh, L, kTileRows, C, total_chunks, prob);
+    return;
+  }
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i < 4) counters[i] = 0u;
   if (i >= n_pairs) return;

@@ -19,12 +19,12 @@ __device__ __forceinline__ float cumsum_term(float v, int prob) {
   return (__float_as_uint(v) >> 31) ? -INFINITY : log1pf(-v);
 }
 
-__global__ __launch_bounds__(256) void cumsum_kernel(const float* __restrict__ A,
-                                                     SeqStrides sa, float* __restrict__ cs,
-                                                     int nh, int L, int Q, int C,
-                                                     int64_t total_chunks, int prob) {
+// The work of workgroup `block` (four chunks, one per wave).
+__device__ __forceinline__ void cumsum_block(int64_t block, const float* __restrict__ A, SeqStrides sa,
+                                             float* __restrict__ cs, int nh, int L, int Q, int C,
+                                             int64_t total_chunks, int prob) {
   const int lane = threadIdx.x & 63;
-  const int64_t chunk_id = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t chunk_id = block * 4 + (threadIdx.x >> 6);
   if (chunk_id >= total_chunks) return;
   const int64_t n = chunk_id / C;
   const int c = (int)(chunk_id - n * C);
@@ -47,6 +47,13 @@ __global__ __launch_bounds__(256) void cumsum_kernel(const float* __restrict__ A
     if (q < limit) run += cumsum_term(a[(int64_t)q * sa.sl], prob);
     if (q < Q) out[q] = run;
   }
+}
+
+__global__ __launch_bounds__(256) void cumsum_kernel(const float* __restrict__ A,
+                                                     SeqStrides sa, float* __restrict__ cs,
+                                                     int nh, int L, int Q, int C,
+                                                     int64_t total_chunks, int prob) {
+  cumsum_block(blockIdx.x, A, sa, cs, nh, L, Q, C, total_chunks, prob);
 }
 
 // ------------------------------------------------------------------------------------
