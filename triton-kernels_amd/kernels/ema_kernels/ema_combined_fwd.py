@@ -80,7 +80,14 @@ class EMAMatmulCombinedFn(torch.autograd.Function):
         from kernels.ema_kernels_bwd.ema_combined_bwd import _ema_chunk_scan_combined_bwd
 
         out, dA_cumsum, states, final_states, A_ema, X_ema = ctx.saved_tensors
-        dx, ddA = _ema_chunk_scan_combined_bwd(dout, X_ema, A_ema, ctx.chunk_size, prev128=ctx.prev128)
+        if ctx.prev128 is not None:
+            # the same single-pass kernel through the entry point that returns the gradient of the
+            # log-decay in the layout of A itself: nothing to rearrange afterwards
+            from kernels.ema_seq import ema_seq_bwd
+
+            dx, dA, _ = ema_seq_bwd(dout, X_ema, A_ema, ctx.prev128, form="log_decay")
+            return dA, dx, None
+        dx, ddA = _ema_chunk_scan_combined_bwd(dout, X_ema, A_ema, ctx.chunk_size)
         dA = _unchunk_dA(ddA, A_ema, X_ema.shape[1])
         return dA, dx, None
 
