@@ -287,6 +287,20 @@ def test_legacy_mamba_encoded_entry_point(device):
     )
     check_close("out", out.reshape(b, L, nh * hd), ref, F32)
     check_close("final", final.reshape(b, nh * hd), ref[:, -1], F32)
+    # anything but the EMA encoding (here a state of 4, D, z and an initial state) is the general
+    # recurrence with dA = -dt, whatever A holds (kernels/ema_chunk_state.py:95 of the reference)
+    from oracle import ssd_oracle as S
+
+    g2 = torch.Generator().manual_seed(5)
+    Bg, Cg = torch.randn(b, L, 1, 4, generator=g2), torch.randn(b, L, 1, 4, generator=g2)
+    D, z = torch.randn(nh, generator=g2), torch.randn(b, L, nh, hd, generator=g2)
+    init = torch.randn(b, nh, hd, 4, generator=g2)
+    y_ref, fin_ref = S.ssd_loop(X_m, dt_h, -torch.ones(nh), Bg, Cg, D, z, init)
+    out, final = ema_chunk_scan_combined(
+        X_m.to(device), dt_h.to(device), torch.full((nh,), -3.0, device=device), Bg.to(device), Cg.to(device), 64,
+        D=D.to(device), z=z.to(device), initial_states=init.to(device), return_final_states=True)
+    check_close("general case: out", out, y_ref, F32)
+    check_close("general case: final", final, fin_ref, F32)
     with pytest.raises(NotImplementedError):
-        ema_chunk_scan_combined(X_m.to(device), dt_h.to(device), A.to(device),
-                                torch.ones(b, L, 1, 4, device=device), torch.ones(b, L, 1, 4, device=device), 64)
+        ema_chunk_scan_combined(X_m.to(device), dt_h.to(device), A.to(device), B_m.to(device), C_m.to(device), 64,
+                                cu_seqlens=torch.tensor([0, L], device=device))

@@ -1,13 +1,14 @@
 """Headed, Mamba-encoded entry point of the reference's legacy EMA path.
 
 Mirrors the signature of ema_chunk_scan_combined, kernels/ema_combined.py:100-119 of the
-reference.  That path runs the Mamba-2 SSD kernels with a state dimension of 1 and the decay
-fixed to dA = -dt (kernels/ema_chunk_state.py:95 ignores A); with that encoding
+reference.  That path runs Mamba-2 SSD kernels with the decay fixed to dA = -dt
+(kernels/ema_chunk_state.py:95 ignores A):
 
-    state_t = exp(-dt_t) * state_{t-1} + dt_t * B_t * x_t,     out_t = C_t * state_t
+    state_t = exp(-dt_t) * state_{t-1} + dt_t * x_t (outer) B_t,     out_t = C_t . state_t + D x_t
 
-per (batch, head, feature), which is the EMA scan with log-decay -dt and input dt * B * x,
-scaled by C.  Only that encoding is supported."""
+The EMA encoding is the case of a state dimension of 1 with no D, z, bias or initial state:
+per (batch, head, feature) it is the EMA scan with log-decay -dt and input dt * B * x, scaled by
+C, and runs on the EMA kernels.  Every other case runs on the SSD stage kernels with A = -1."""
 import torch
 
 from kernels.ema_kernels.ema_combined_fwd import _ema_matmul_scan_combined_fwd, ema_matmul_scan_combined
@@ -17,8 +18,9 @@ def ema_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=
                             seq_idx=None, cu_seqlens=None, dt_softplus=False, dt_limit=(0.0, float("inf")),
                             return_final_states=False, return_varlen_states=False):
     """x: (batch, seqlen, nheads, headdim); dt: (batch, seqlen, nheads); A: (nheads,) (unused, as
-    in the reference); B, C: (batch, seqlen, ngroups, 1).  Returns out (batch, seqlen, nheads,
-    headdim), and the final states (batch, nheads, headdim, 1) if return_final_states."""
+    in the reference); B, C: (batch, seqlen, ngroups, dstate).  Returns out (batch, seqlen, nheads,
+    headdim), and the final states (batch, nheads, headdim, dstate) if return_final_states.
+    cu_seqlens / return_varlen_states are refused."""
     batch, seqlen, nheads, headdim = x.shape
     _, _, ngroups, dstate = B.shape
     assert nheads % ngroups == 0
@@ -26,14 +28,18 @@ def ema_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=
     assert dt.shape == (batch, seqlen, nheads)
     assert A.shape == (nheads,)
     assert C.shape == B.shape
-    if dstate != 1:
-        raise NotImplementedError("the EMA encoding has a state dimension of 1")
-    if D is not None or z is not None or dt_bias is not None or dt_softplus:
-        raise NotImplementedError("D, z, dt_bias and dt_softplus are not part of the EMA encoding")
-    if initial_states is not None or seq_idx is not None or cu_seqlens is not None or return_varlen_states:
-        raise NotImplementedError("initial_states, seq_idx and varlen states are not supported")
-    if tuple(dt_limit) != (0.0, float("inf")):
-        raise NotImplementedError("dt_limit is not supported")
+    if cu_seqlens is not None or return_varlen_states:
+        raise NotImplementedError("varlen states (cu_seqlens) are not supported")
+    ema_encoding = (dstate == 1 and D is None and z is None and dt_bias is None and not dt_softplus
+                    and initial_states is None and seq_idx is None and tuple(dt_limit) == (0.0, float("inf")))
+    if not ema_encoding:
+        from kernels.mamba_kernels.mamba_combined_fwd import _mamba_chunk_scan_combined_fwd
+
+        minus_one = -torch.ones(nheads, device=x.device, dtype=torch.float32)  # the path ignores A
+        out, _, _, _, _, final = _mamba_chunk_scan_combined_fwd(
+            x, dt, minus_one, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, initial_states=initial_states,
+            seq_idx=seq_idx, dt_softplus=dt_softplus, dt_limit=dt_limit)
+        return (out, final) if return_final_states else out
     rep = nheads // ngroups
     dtf = dt.float()
     Bh = B[..., 0].float().repeat_interleave(rep, dim=-1)  # (batch, seqlen, nheads)
