@@ -217,10 +217,39 @@ def chunk_scan(cb, x, dt, dA_cumsum, C, states, D=None, z=None, round_to=None, s
     return out, out_x
 
 
+def chunk_state_varlen(B, x, dt, dA_cumsum, cu_seqlens, chunk_states, round_to=None):
+    """State at the end of each sequence of a packed batch without batch dimension
+    (kernels/ema_chunk_state.py:500-604 of the reference).  B (L, g, n), x (L, nh, p), dt and
+    dA_cumsum (nh, C, Q), chunk_states (C, nh, p, n) = state entering each chunk, cu_seqlens
+    (nseq + 1).  For a sequence [start, end) with c the chunk of end - 1: the positions of the
+    sequence inside chunk c, weighted by exp(min(dA[end-1] - dA[k], 0)) * dt[k] (:551-555), plus
+    exp(dA[end-1]) * chunk_states[c] if the sequence began before chunk c (:563-568)."""
+    L, nh, p = x.shape
+    _, C, Q = dt.shape
+    g, n = B.shape[1], B.shape[2]
+    Bh = _up(B).repeat_interleave(nh // g, dim=1)  # (L, nh, n)
+    xs = _up(x)
+    out = []
+    for s in range(len(cu_seqlens) - 1):
+        start, end = int(cu_seqlens[s]), int(cu_seqlens[s + 1])
+        c = (end - 1) // Q
+        lo = max(start, c * Q)
+        k = torch.arange(lo, end)
+        dA_last = dA_cumsum[:, c, end - 1 - c * Q]  # (nh,)
+        w = torch.exp(torch.clamp(dA_last[:, None] - dA_cumsum[:, c, k - c * Q], max=0.0)) * dt[:, c, k - c * Q]
+        st = torch.einsum("khp,khn->hpn", xs[k], _round(Bh[k] * w.T[..., None], round_to))
+        if start < c * Q:
+            st = st + torch.exp(dA_last)[:, None, None] * chunk_states[c]
+        out.append(st)
+    return torch.stack(out)
+
+
 def combined_fwd(x, dt, A, B, C, Q, D=None, z=None, dt_bias=None, initial_states=None,
-                 dt_softplus=False, dt_limit=(0.0, float("inf")), round_to=None, seq_idx=None):
+                 dt_softplus=False, dt_limit=(0.0, float("inf")), round_to=None, seq_idx=None, cu_seqlens=None):
     """The five stages in the order of mamba_ssm's combined forward, which the reference's
-    kernels/mamba_kernels/ files were taken from.  Returns (out, final_states)."""
+    kernels/mamba_kernels/ files were taken from.  Returns (out, final_states), and the states at
+    the sequence ends as a third item when cu_seqlens is given (batch of 1,
+    kernels/ema_combined.py:56-62)."""
     b, L, nh, p = x.shape
     n = B.shape[-1]
     dA_cs, dt_out = chunk_cumsum(dt, A, Q, dt_bias, dt_softplus, dt_limit)
@@ -230,7 +259,11 @@ def combined_fwd(x, dt, A, B, C, Q, D=None, z=None, dt_bias=None, initial_states
     prev = prev.reshape(b, -1, nh, p, n)
     cb = bmm_chunk(C, B, Q, seq_idx)
     out, _ = chunk_scan(cb, x, dt_out, dA_cs, C, prev, D, z, round_to, seq_idx)
-    return out, final.reshape(b, nh, p, n)
+    if cu_seqlens is None:
+        return out, final.reshape(b, nh, p, n)
+    assert b == 1
+    varlen = chunk_state_varlen(B[0], x[0], dt_out[0], dA_cs[0], cu_seqlens, prev[0], round_to)
+    return out, final.reshape(b, nh, p, n), varlen
 
 
 # ------------------------------------------------------------------ inputs and brute force

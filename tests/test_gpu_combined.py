@@ -301,6 +301,17 @@ def test_legacy_mamba_encoded_entry_point(device):
         D=D.to(device), z=z.to(device), initial_states=init.to(device), return_final_states=True)
     check_close("general case: out", out, y_ref, F32)
     check_close("general case: final", final, fin_ref, F32)
-    with pytest.raises(NotImplementedError):
-        ema_chunk_scan_combined(X_m.to(device), dt_h.to(device), A.to(device), B_m.to(device), C_m.to(device), 64,
-                                cu_seqlens=torch.tensor([0, L], device=device))
+    # the state at the end of each packed sequence (a batch of 1): every sequence on its own
+    cu = torch.tensor([0, 70, 200, L], dtype=torch.int32)
+    seq = torch.repeat_interleave(torch.arange(3, dtype=torch.int32), cu.diff())[None]
+    one = lambda t: t[:1].to(device)
+    out, varlen = ema_chunk_scan_combined(one(X_m), one(dt_h), A.to(device), one(Bg), one(Cg), 64, seq_idx=seq.to(device),
+                                          cu_seqlens=cu.to(device), return_varlen_states=True)
+    assert varlen.shape == (3, nh, hd, 4)
+    for i in range(3):
+        sl = slice(int(cu[i]), int(cu[i + 1]))
+        y_i, fin_i = S.ssd_loop(X_m[:1, sl], dt_h[:1, sl], -torch.ones(nh), Bg[:1, sl], Cg[:1, sl])
+        check_close(f"packed sequence {i}: out", out[:, sl], y_i, F32)
+        check_close(f"packed sequence {i}: end state", varlen[i], fin_i[0], F32)
+    with pytest.raises(AssertionError):
+        ema_chunk_scan_combined(one(X_m), one(dt_h), A.to(device), one(Bg), one(Cg), 64, return_varlen_states=True)

@@ -207,3 +207,79 @@ def test_packed_state_passing_bwd_vs_oracle(b, nc, nh, dim, Q, L, has_init, devi
     if has_init:
         check_close("dinitstates", got[2], ref[2], F32)
         assert torch.equal(got[2][0].cpu(), dout[0, 0])  # nothing flows back across the dropped state
+
+
+VARLEN_CASES = [
+    # L, nh, P, g, N, Q
+    (300, 4, 64, 1, 64, 64),
+    (520, 2, 128, 2, 128, 128),
+    (200, 2, 64, 1, 128, 256),     # one ragged chunk that holds every sequence
+    (333, 2, 48, 1, 20, 64),       # head and state sizes off the tile sizes
+    (150, 2, 8, 1, 1, 32),
+]
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("L,nh,P,g,N,Q", VARLEN_CASES)
+def test_varlen_states(L, nh, P, g, N, Q, dtype, device):
+    """The state at the end of each packed sequence (cu_seqlens): the launcher against the oracle on
+    the oracle's intermediates, and the combined forward against each sequence run through the
+    recurrence on its own."""
+    from kernels.ema_chunk_state import chunk_state_varlen
+    from kernels.mamba_kernels.mamba_combined_fwd import mamba_chunk_scan_combined_fwd
+
+    announce(f"ssd varlen states L{L} nh{nh} P{P} g{g} N{N} Q{Q} {dtype}")
+    x, dt, A, B, C, _, _ = S.make_inputs(1, L, nh, P, g, N, seed=L + P, dtype=dtype)
+    A = slow(A)
+    seq = pack_ids(1, L, Q, seed=L)
+    starts = (torch.nonzero(seq[0, 1:] != seq[0, :-1])[:, 0] + 1).tolist()
+    cu = torch.tensor([0] + starts + [L], dtype=torch.int32)
+    init = torch.randn(1, nh, P, N, generator=torch.Generator().manual_seed(6))
+    rt = None if dtype == F32 else dtype
+    small = F32 if dtype == F32 else BF16
+
+    dA_cs, dt_out = S.chunk_cumsum(dt, A, Q)
+    states = S.chunk_state(B, x, dt_out, dA_cs, rt, seq)
+    prev, _ = S.state_passing(states.reshape(1, -1, nh, P * N), dA_cs[..., -1], init.reshape(1, nh, P * N), seq, Q)
+    prev = prev.reshape(-1, nh, P, N)
+    ref = S.chunk_state_varlen(B[0], x[0], dt_out[0], dA_cs[0], cu, prev, rt)
+    got = chunk_state_varlen(*_dev(device, B[0], x[0], dt_out[0], dA_cs[0], cu, prev))
+    assert got.shape == (len(cu) - 1, nh, P, N)
+    check_close("varlen states vs oracle", got, ref, small)
+
+    y, fin, varlen = mamba_chunk_scan_combined_fwd(
+        *_dev(device, x, dt, A, B, C), Q, initial_states=init.to(device), seq_idx=seq.to(device),
+        cu_seqlens=cu.to(device), return_final_states=True, return_varlen_states=True)
+    for i in range(len(cu) - 1):
+        sl = slice(int(cu[i]), int(cu[i + 1]))
+        # the first sequence continues the initial state only if it reaches past chunk 0
+        # (kernels/ema_chunk_state.py:563 of the reference)
+        first = init if i == 0 and int(cu[1]) > Q else None
+        _, fi = S.ssd_loop(x[:, sl].float(), dt[:, sl], A, B[:, sl].float(), C[:, sl].float(), initial_states=first)
+        check_close(f"sequence {i} alone", varlen[i], fi[0], small, loose=dtype == BF16)
+    check_close("last sequence = final state", varlen[-1], fin[0].float(), small)
+
+
+def test_varlen_states_edge_cases(device):
+    """A sequence of one position, an empty one, one that is the whole batch, and bounds that do
+    not fit (zeros, no fault)."""
+    from kernels.ema_chunk_state import chunk_state_varlen
+
+    L, nh, P, g, N, Q = 100, 2, 64, 1, 64, 32
+    x, dt, A, B, _, _, _ = S.make_inputs(1, L, nh, P, g, N, seed=1)
+    dA_cs, dt_out = S.chunk_cumsum(dt, slow(A), Q)
+    prev = torch.randn(4, nh, P, N, generator=torch.Generator().manual_seed(1))
+    args = lambda cu: _dev(device, B[0], x[0], dt_out[0], dA_cs[0], cu, prev)
+    cu = torch.tensor([0, 1, 1, 64, 100], dtype=torch.int32)
+    got = chunk_state_varlen(*args(cu)).cpu()
+    ref = S.chunk_state_varlen(B[0], x[0], dt_out[0], dA_cs[0], torch.tensor([0, 1]), prev)
+    check_close("one position", got[0], ref[0], F32)
+    assert torch.equal(got[1], torch.zeros(nh, P, N))  # empty
+    ref = S.chunk_state_varlen(B[0], x[0], dt_out[0], dA_cs[0], torch.tensor([1, 64, 100]), prev)
+    check_close("ends on a chunk edge / ragged last chunk", got[2:], ref, F32)
+    whole = chunk_state_varlen(*args(torch.tensor([0, L], dtype=torch.int32)))
+    check_close("whole batch", whole, S.chunk_state_varlen(B[0], x[0], dt_out[0], dA_cs[0], [0, L], prev), F32)
+    odd = chunk_state_varlen(*args(torch.tensor([-5, 10, 5, 400], dtype=torch.int32))).cpu()
+    assert torch.equal(odd[0], torch.zeros(nh, P, N)) and torch.equal(odd[1], torch.zeros(nh, P, N))
+    ref = S.chunk_state_varlen(B[0], x[0], dt_out[0], dA_cs[0], torch.tensor([5, 100]), prev)
+    check_close("end clamped to the length", odd[2], ref[0], F32)

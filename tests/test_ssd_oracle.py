@@ -179,6 +179,29 @@ def test_chunked_stages_equal_loop_packed(pack, Q):
     assert torch.allclose(fin, fin_ref, rtol=1e-10, atol=1e-10)
 
 
+@pytest.mark.parametrize("lengths", [[13, 8, 16], [16, 16, 5], [1, 35, 1], [3, 2, 4, 28], [37]])
+@pytest.mark.parametrize("Q", [8, 16, 64])
+def test_varlen_states_equal_each_sequence_alone(lengths, Q):
+    """The state at the end of every packed sequence is the final state of that sequence run
+    through the recurrence on its own.  The first one continues the initial state only if it reaches
+    past the first chunk: the reference adds the state entering the last chunk of a sequence only
+    for sequences that began before that chunk (kernels/ema_chunk_state.py:563), which leaves the
+    initial state out for a first sequence that ends inside chunk 0."""
+    L = sum(lengths)
+    x, dt, A, B, C, _, _ = _f64(*S.make_inputs(1, L, 4, 6, 2, 5, seed=Q + L))
+    init = torch.randn(1, 4, 6, 5, generator=torch.Generator().manual_seed(2), dtype=D64)
+    cu = torch.tensor([0] + list(torch.tensor(lengths).cumsum(0)), dtype=torch.int32)
+    _, fin, varlen = S.combined_fwd(x, dt, A, B, C, Q, initial_states=init, seq_idx=_ids([lengths]), cu_seqlens=cu)
+    assert varlen.shape == (len(lengths), 4, 6, 5)
+    for i in range(len(lengths)):
+        sl = slice(int(cu[i]), int(cu[i + 1]))
+        continues = i == 0 and int(cu[1]) > Q
+        _, fi = S.ssd_loop(x[:, sl], dt[:, sl], A, B[:, sl], C[:, sl], initial_states=init if continues else None)
+        assert torch.allclose(varlen[i], fi[0], rtol=1e-10, atol=1e-10)
+    if len(lengths) > 1 or L > Q:
+        assert torch.allclose(varlen[-1], fin[0], rtol=1e-10, atol=1e-10)
+
+
 def test_bmm_chunk_masks_pairs_of_different_sequences():
     gen = torch.Generator().manual_seed(8)
     Cm = torch.randn(1, 21, 1, 6, generator=gen)

@@ -1700,4 +1700,86 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
   SSD_TSTAMP(7);
 }
 
+// ------------------------------------------------------------------------------------
+// States at the end of each sequence of a packed batch: for sequence s ending at position e
+// (exclusive) in chunk c = (e - 1) / Q, the positions of s that lie in chunk c weighted by the decay
+// to e - 1 and dt, plus the state entering chunk c decayed to e - 1 when s began before that chunk
+// (_chunk_state_varlen_kernel, kernels/ema_chunk_state.py:500-575 of the reference).  A handful of
+// sequences per call: plain fp32 multiply-adds on 64 x 64 tiles of the state, 4 x 4 per thread.
+// Grid (P tiles * N tiles, sequences, heads).  The weighted B is rounded to T before the product,
+// as the reference does; an empty or out-of-range sequence gives zeros.
+// ------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void ssd_chunk_state_varlen_kernel(
+    const T* __restrict__ x, int64_t x_sl, int64_t x_sh, const T* __restrict__ Bm, int64_t b_sl, int64_t b_sg,
+    const float* __restrict__ dt, const float* __restrict__ dA_cs, const float* __restrict__ chunk_states,
+    const int32_t* __restrict__ cu_seqlens, float* __restrict__ out, int L, int nh, int hpg, int P, int N, int Q,
+    int C) {
+  constexpr int TP = 64, TN = 64, KB = 32;
+  __shared__ float sx[KB][TP];
+  __shared__ float sb[KB][TN];
+  __shared__ float ss[KB];
+  const int tid = threadIdx.x;
+  const int tiles_n = (N + TN - 1) / TN;
+  const int p0 = (blockIdx.x / tiles_n) * TP, n0 = (blockIdx.x % tiles_n) * TN;
+  const int s = blockIdx.y, h = blockIdx.z;
+  const int tp = (tid >> 4) * 4, tn = (tid & 15) * 4;
+  const int start = cu_seqlens[s];
+  const int end = min(cu_seqlens[s + 1], L);
+  float acc[4][4] = {};
+  const bool live = start >= 0 && end > start;  // uniform over the workgroup
+  const int c = live ? (end - 1) / Q : 0;
+  const int limit = end - c * Q;                // positions of chunk c up to the sequence's end
+  const int first = max(start - c * Q, 0);      // first position of chunk c that belongs to s
+  const int64_t row = ((int64_t)h * C + c) * Q;  // dt, dA_cumsum are (nheads, nchunks, Q)
+  const float dA_last = live ? dA_cs[row + limit - 1] : 0.f;
+  const T* xg = x + (int64_t)c * Q * x_sl + (int64_t)h * x_sh;
+  const T* bg = Bm + (int64_t)c * Q * b_sl + (int64_t)(h / hpg) * b_sg;
+  for (int k0 = live ? (first / KB) * KB : limit; k0 < limit; k0 += KB) {
+    if (tid < KB) {
+      const int k = k0 + tid;
+      const int kc = min(k, limit - 1);
+      const float w = __expf(fminf(dA_last - dA_cs[row + kc], 0.f)) * dt[row + kc];
+      ss[tid] = (k >= first && k < limit) ? w : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < KB * TP / 256; ++i) {
+      const int idx = tid + i * 256;
+      const int kk = idx / TP, col = idx % TP;
+      const int kc = min(k0 + kk, limit - 1);
+      const float w = ss[kk];
+      const float xv = (float)xg[(int64_t)kc * x_sl + min(p0 + col, P - 1)];
+      const float bv = (float)bg[(int64_t)kc * b_sl + min(n0 + col, N - 1)];
+      sx[kk][col] = (w != 0.f && p0 + col < P) ? xv : 0.f;
+      sb[kk][col] = (w != 0.f && n0 + col < N) ? (float)(T)(bv * w) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int kk = 0; kk < KB; ++kk) {
+      const float4 a = *reinterpret_cast<const float4*>(&sx[kk][tp]);
+      const float4 b = *reinterpret_cast<const float4*>(&sb[kk][tn]);
+      const float av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+  const bool carried = live && start < c * Q;  // the sequence began before chunk c
+  const float keep = carried ? __expf(dA_last) : 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int p = p0 + tp + i, n = n0 + tn + j;
+      if (p < P && n < N) {
+        float v = acc[i][j];
+        if (carried) v = fmaf(chunk_states[(((int64_t)c * nh + h) * P + p) * N + n], keep, v);
+        out[(((int64_t)s * nh + h) * P + p) * N + n] = v;
+      }
+    }
+}
+
 }  // namespace ssd

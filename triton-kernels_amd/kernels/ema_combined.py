@@ -19,8 +19,9 @@ def ema_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=
                             return_final_states=False, return_varlen_states=False):
     """x: (batch, seqlen, nheads, headdim); dt: (batch, seqlen, nheads); A: (nheads,) (unused, as
     in the reference); B, C: (batch, seqlen, ngroups, dstate).  Returns out (batch, seqlen, nheads,
-    headdim), and the final states (batch, nheads, headdim, dstate) if return_final_states.
-    cu_seqlens / return_varlen_states are refused."""
+    headdim), then the final states (batch, nheads, headdim, dstate) if return_final_states, then
+    the state at the end of each packed sequence (num_sequences, nheads, headdim, dstate) if
+    return_varlen_states (cu_seqlens (num_sequences + 1), batch of 1)."""
     batch, seqlen, nheads, headdim = x.shape
     _, _, ngroups, dstate = B.shape
     assert nheads % ngroups == 0
@@ -28,18 +29,19 @@ def ema_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=
     assert dt.shape == (batch, seqlen, nheads)
     assert A.shape == (nheads,)
     assert C.shape == B.shape
-    if cu_seqlens is not None or return_varlen_states:
-        raise NotImplementedError("varlen states (cu_seqlens) are not supported")
+    if return_varlen_states:
+        assert cu_seqlens is not None, "cu_seqlens must be provided if return_varlen_states is True"
     ema_encoding = (dstate == 1 and D is None and z is None and dt_bias is None and not dt_softplus
-                    and initial_states is None and seq_idx is None and tuple(dt_limit) == (0.0, float("inf")))
+                    and initial_states is None and seq_idx is None and not return_varlen_states
+                    and tuple(dt_limit) == (0.0, float("inf")))
     if not ema_encoding:
-        from kernels.mamba_kernels.mamba_combined_fwd import _mamba_chunk_scan_combined_fwd
+        from kernels.mamba_kernels.mamba_combined_fwd import mamba_chunk_scan_combined_fwd
 
         minus_one = -torch.ones(nheads, device=x.device, dtype=torch.float32)  # the path ignores A
-        out, _, _, _, _, final = _mamba_chunk_scan_combined_fwd(
+        return mamba_chunk_scan_combined_fwd(
             x, dt, minus_one, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, initial_states=initial_states,
-            seq_idx=seq_idx, dt_softplus=dt_softplus, dt_limit=dt_limit)
-        return (out, final) if return_final_states else out
+            seq_idx=seq_idx, cu_seqlens=cu_seqlens, dt_softplus=dt_softplus, dt_limit=dt_limit,
+            return_final_states=return_final_states, return_varlen_states=return_varlen_states)
     rep = nheads // ngroups
     dtf = dt.float()
     Bh = B[..., 0].float().repeat_interleave(rep, dim=-1)  # (batch, seqlen, nheads)

@@ -9,14 +9,16 @@ import torch
 from kernels.mamba_kernels.mamba_bmm import _bmm_chunk_fwd
 from kernels.mamba_kernels.mamba_cumsum import _chunk_cumsum_fwd
 from kernels.mamba_kernels.mamba_scan_fwd import _chunk_scan_fwd
-from kernels.mamba_kernels.mamba_state_fwd import _chunk_state_fwd
+from kernels.mamba_kernels.mamba_state_fwd import _chunk_state_fwd, chunk_state_varlen
 from kernels.mamba_kernels.mamba_state_pass import _state_passing_fwd
 
 
 def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
-                                   initial_states=None, seq_idx=None, dt_softplus=False,
+                                   initial_states=None, seq_idx=None, cu_seqlens=None, dt_softplus=False,
                                    dt_limit=(0.0, float("inf"))):
-    """Returns (out, out_x, dt_out, dA_cumsum, states, final_states)."""
+    """Returns (out, out_x, dt_out, dA_cumsum, states, final_states), and as a seventh item the state
+    at the end of each packed sequence when cu_seqlens is given (batch must be 1 then; the boundaries
+    are the ones seq_idx marks), as kernels/ema_combined.py:56-62 of the reference does."""
     batch, seqlen, nheads, headdim = x.shape
     _, _, ngroups, dstate = B.shape
     assert nheads % ngroups == 0
@@ -35,13 +37,26 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
     final_states = final_states.reshape(batch, nheads, headdim, dstate)
     CB = _bmm_chunk_fwd(C, B, chunk_size, seq_idx=seq_idx, output_dtype=torch.float32)
     out, out_x = _chunk_scan_fwd(CB, x, dt_out, dA_cumsum, C, states, D=D, z=z, seq_idx=seq_idx)
-    return out, out_x, dt_out, dA_cumsum, states, final_states
+    if cu_seqlens is None:
+        return out, out_x, dt_out, dA_cumsum, states, final_states
+    assert batch == 1, "passing cu_seqlens to get the varlen states is only supported if batch dimension is 1"
+    varlen_states = chunk_state_varlen(B.squeeze(0), x.squeeze(0), dt_out.squeeze(0), dA_cumsum.squeeze(0),
+                                       cu_seqlens, states.squeeze(0))
+    return out, out_x, dt_out, dA_cumsum, states, final_states, varlen_states
 
 
 def mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
-                                  initial_states=None, seq_idx=None, dt_softplus=False,
-                                  dt_limit=(0.0, float("inf")), return_final_states=False):
-    out, _, _, _, _, final_states = _mamba_chunk_scan_combined_fwd(
+                                  initial_states=None, seq_idx=None, cu_seqlens=None, dt_softplus=False,
+                                  dt_limit=(0.0, float("inf")), return_final_states=False,
+                                  return_varlen_states=False):
+    """out, then the final states and the per-sequence states as asked for, in that order
+    (kernels/ema_combined.py:83-87 of the reference)."""
+    if return_varlen_states:
+        assert cu_seqlens is not None, "cu_seqlens must be provided if return_varlen_states is True"
+    else:
+        cu_seqlens = None
+    out, _, _, _, _, final_states, *rest = _mamba_chunk_scan_combined_fwd(
         x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, initial_states=initial_states,
-        seq_idx=seq_idx, dt_softplus=dt_softplus, dt_limit=dt_limit)
-    return (out, final_states) if return_final_states else out
+        seq_idx=seq_idx, cu_seqlens=cu_seqlens, dt_softplus=dt_softplus, dt_limit=dt_limit)
+    res = (out,) + ((final_states,) if return_final_states else ()) + tuple(rest)
+    return res if len(res) > 1 else out

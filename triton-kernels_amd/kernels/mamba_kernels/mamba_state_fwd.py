@@ -1,6 +1,7 @@
 """SSD stage 2: chunk states B^T x, weighted by the decay to the end of the chunk and dt.
 
-Mirrors _chunk_state_fwd, kernels/mamba_kernels/mamba_state_fwd.py:138-169 of the reference."""
+Mirrors _chunk_state_fwd, kernels/mamba_kernels/mamba_state_fwd.py:138-169 of the reference, and
+chunk_state_varlen of its legacy stage file, kernels/ema_chunk_state.py:578-604."""
 import torch
 
 from kernels import _lib
@@ -39,3 +40,39 @@ def _chunk_state_fwd(B, x, dt, dA_cumsum, seq_idx=None, states=None, states_in_f
         states.copy_(out)
         return states
     return out if states_in_fp32 else out.to(B.dtype)
+
+
+def chunk_state_varlen(B, x, dt, dA_cumsum, cu_seqlens, chunk_states):
+    """States at the end of each sequence of a packed batch (no batch dimension: x is
+    (total_seqlen, nheads, headdim), B (total_seqlen, ngroups, dstate), dt and dA_cumsum
+    (nheads, nchunks, chunk_size), chunk_states (nchunks, nheads, headdim, dstate) the state
+    entering each chunk, cu_seqlens (num_sequences + 1) the sequence boundaries).  Returns
+    (num_sequences, nheads, headdim, dstate) in the dtype of chunk_states."""
+    total_seqlen, nheads, headdim = x.shape
+    _, nchunks, chunk_size = dt.shape
+    _, ngroups, dstate = B.shape
+    batch = cu_seqlens.shape[0] - 1
+    assert nheads % ngroups == 0
+    assert B.shape == (total_seqlen, ngroups, dstate)
+    assert dt.shape == (nheads, nchunks, chunk_size)
+    assert dA_cumsum.shape == dt.shape
+    assert chunk_states.shape == (nchunks, nheads, headdim, dstate)
+    assert batch >= 1 and nchunks == -(-total_seqlen // chunk_size)
+    dev = _lib.require_gpu(x, B, dt, dA_cumsum, chunk_states, cu_seqlens)
+    if B.dtype != x.dtype:
+        B = B.to(x.dtype)
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    if B.stride(-1) != 1:
+        B = B.contiguous()
+    cu = cu_seqlens.to(torch.int32).contiguous()
+    states = torch.empty(batch, nheads, headdim, dstate, device=dev, dtype=torch.float32)
+    with torch.cuda.device(dev):
+        _lib.check(
+            _lib.lib().ssd_chunk_state_varlen(B.data_ptr(), B.stride(0), B.stride(1), x.data_ptr(), x.stride(0),
+                                              x.stride(1), _lib.dtype_code(x), _lib.f32c(dt).data_ptr(),
+                                              _lib.f32c(dA_cumsum).data_ptr(), _lib.f32c(chunk_states).data_ptr(),
+                                              cu.data_ptr(), states.data_ptr(), batch, total_seqlen, nheads, ngroups,
+                                              headdim, dstate, chunk_size, _lib.stream_ptr(dev)),
+            "ssd_chunk_state_varlen")
+    return states.to(chunk_states.dtype)
