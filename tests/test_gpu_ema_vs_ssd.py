@@ -122,3 +122,31 @@ def test_main_script_flow(device):
     check_close("ema_chunk_scan_combined", got.reshape(b, L, D), ref, F32)
     got = mamba_chunk_scan_combined_fwd(X_m, dt, A, B_m, C_m, Q)
     check_close("mamba forward", got.reshape(b, L, D), ref, F32)
+
+
+def test_legacy_stage_modules(device):
+    """The stage launchers under the module paths of the reference's legacy headed path, run in the
+    order of kernels/ema_combined.py:43-55 with an A that must be ignored, against the same loop."""
+    from kernels.ema_bmm import _bmm_chunk_fwd
+    from kernels.ema_chunk_scan import _chunk_scan_fwd
+    from kernels.ema_chunk_state import _chunk_cumsum_fwd, _simplified_chunk_state_fwd
+    from kernels.ema_state_passing import _state_passing_fwd
+
+    announce("legacy stage modules: cumsum, simplified chunk state, state passing, bmm, chunk scan")
+    b, L, nh, P, Q = 2, 300, 2, 32, 64
+    ema, ssd = _encode(b, L, nh, P, 1, seed=3, device=device)
+    x, dt, Bm, Cm = ssd["x"], ssd["dt"], ssd["B"], ssd["C"]
+    dA_cs, dt_out = _chunk_cumsum_fwd(dt, torch.full((nh,), -7.0, device=device), Q)
+    states = _simplified_chunk_state_fwd(Bm, x, dt_out, dA_cs, states_in_fp32=True)
+    states, final = _state_passing_fwd(states.reshape(b, -1, nh, P), dA_cs[:, :, :, -1], chunk_size=Q,
+                                       out_dtype=torch.float32)
+    CB = _bmm_chunk_fwd(Cm, Bm, Q, output_dtype=torch.float32)
+    out, _ = _chunk_scan_fwd(CB, x, dt_out, dA_cs, Cm, states.reshape(b, -1, nh, P, 1))
+    ref = torch.empty(b, L, nh * P)
+    z = torch.zeros(b, nh * P)
+    Xc, Ac = ema["X"].cpu(), ema["A"].cpu()
+    for t in range(L):
+        z = torch.exp(Ac[:, t, None]) * z + Xc[:, t]
+        ref[:, t] = z
+    check_close("out", out.reshape(b, L, nh * P), ref, F32)
+    check_close("final", final.reshape(b, nh * P), ref[:, -1], F32)

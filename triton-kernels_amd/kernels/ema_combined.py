@@ -8,7 +8,9 @@ reference.  That path runs Mamba-2 SSD kernels with the decay fixed to dA = -dt
 
 The EMA encoding is the case of a state dimension of 1 with no D, z, bias or initial state:
 per (batch, head, feature) it is the EMA scan with log-decay -dt and input dt * B * x, scaled by
-C, and runs on the EMA kernels.  Every other case runs on the SSD stage kernels with A = -1."""
+C, and runs on the EMA kernels.  Every other case runs on the SSD stage kernels with A = -1,
+including state dimensions above 1, which the reference's path does not compute (its chunk-state
+kernel writes state column 0 only, kernels/ema_chunk_state.py:325-345)."""
 import torch
 
 from kernels.ema_kernels.ema_combined_fwd import _ema_matmul_scan_combined_fwd, ema_matmul_scan_combined
