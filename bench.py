@@ -163,7 +163,7 @@ def ssd_main(args):
         st = _chunk_state_fwd(B, x, dt_out, dA_cs)
         cb = _bmm_chunk_fwd(Cm, B, Q, output_dtype=torch.float32)
         dout = torch.randn_like(x)
-        dprev = _chunk_scan_bwd_dstates(Cm, dA_cs, dout, dtype=torch.float32)
+        dprev = _chunk_scan_bwd_dstates(Cm, dA_cs, dout)  # state-sized gradients travel in bf16 too
         dstates, _, _ = _state_passing_bwd(states.view(b, C, nh, P * N), dA_cs[..., -1], dprev.view(b, C, nh, P * N))
         inter.append((dt_out, dA_cs, st, states, cb, dout, dprev, dstates.view(b, C, nh, P, N)))
     del out, dprev, dstates
@@ -175,12 +175,13 @@ def ssd_main(args):
     stages = {
         "chunk_cumsum": lambda i: _chunk_cumsum_fwd(pick(i)[1], pick(i)[2], Q),
         "chunk_state": lambda i: _chunk_state_fwd(pick(i)[3], pick(i)[0], pick(i)[5], pick(i)[6]),
-        "state_passing": lambda i: _state_passing_fwd(pick(i)[7].view(b, C, nh, P * N), pick(i)[6][..., -1]),
+        "state_passing": lambda i: _state_passing_fwd(pick(i)[7].view(b, C, nh, P * N), pick(i)[6][..., -1],
+                                                      out_dtype=torch.bfloat16),
         "bmm_chunk": lambda i: _bmm_chunk_fwd(pick(i)[4], pick(i)[3], Q, output_dtype=torch.float32),
         "chunk_scan": lambda i: _chunk_scan_fwd(pick(i)[9], pick(i)[0], pick(i)[5], pick(i)[6], pick(i)[4], pick(i)[8]),
         "forward": lambda i: _mamba_chunk_scan_combined_fwd(*pick(i)[:5], Q),
         # backward stages (the reference has no combined backward): x dt A B C | dt_out dA st states cb dout dprev dstates
-        "bwd_dstates": lambda i: _chunk_scan_bwd_dstates(pick(i)[4], pick(i)[6], pick(i)[10], dtype=torch.float32),
+        "bwd_dstates": lambda i: _chunk_scan_bwd_dstates(pick(i)[4], pick(i)[6], pick(i)[10]),
         "bwd_state_passing": lambda i: _state_passing_bwd(pick(i)[8].view(b, C, nh, P * N), pick(i)[6][..., -1],
                                                           pick(i)[11].view(b, C, nh, P * N)),
         "bwd_db": lambda i: _chunk_state_bwd_db(pick(i)[0], pick(i)[5], pick(i)[6], pick(i)[12], B=pick(i)[3], ngroups=g),
@@ -194,13 +195,16 @@ def ssd_main(args):
     dtb = b * L * nh * 4
     stb = b * C * nh * P * N * 4
     cbb = b * C * g * Q * Q * 4
+    # the states entering the chunks travel in bf16, as in the reference's combined forward, and so
+    # do the state-sized gradients of the backward stages (their dtype / dstates_dtype arguments)
+    pvb = stb // 2
     nbytes = {
-        "chunk_cumsum": 3 * dtb, "chunk_state": xb + bc + 2 * dtb + stb, "state_passing": 2 * stb + dtb // Q,
-        "bmm_chunk": 2 * bc + cbb, "chunk_scan": cbb + 2 * xb + bc + stb + 2 * dtb,
+        "chunk_cumsum": 3 * dtb, "chunk_state": xb + bc + 2 * dtb + stb, "state_passing": stb + pvb + dtb // Q,
+        "bmm_chunk": 2 * bc + cbb, "chunk_scan": cbb + 2 * xb + bc + pvb + 2 * dtb,
         "forward": 2 * xb + 2 * bc + dtb,
-        "bwd_dstates": xb + bc + dtb + stb, "bwd_state_passing": 3 * stb + 2 * dtb // Q,
-        "bwd_db": xb + stb + 2 * dtb + bc + 2 * bc + dtb, "bwd_dc": xb + stb + dtb + bc + 2 * bc + dtb,
-        "bwd_dx": cbb + 3 * xb + bc + stb + 3 * dtb, "bwd_ddAcs": 2 * xb + 3 * dtb + cbb,
+        "bwd_dstates": xb + bc + dtb + pvb, "bwd_state_passing": 3 * pvb + 2 * dtb // Q,
+        "bwd_db": xb + pvb + 2 * dtb + bc + 2 * bc + dtb, "bwd_dc": xb + pvb + dtb + bc + 2 * bc + dtb,
+        "bwd_dx": cbb + 3 * xb + bc + pvb + 3 * dtb, "bwd_ddAcs": 2 * xb + 3 * dtb + cbb,
     }
     units = b * C * nh
     flops = {"chunk_state": 2 * Q * P * N * units, "bmm_chunk": 2 * Q * Q * N * b * C * g,

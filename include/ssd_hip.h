@@ -68,7 +68,9 @@ int ssd_chunk_state_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64_t b_sg,
                         const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream);
 
 /* out[b,c] = state entering chunk c; state <- exp(dA_chunk[b,h,c]) * state + states[b,c];
- * final = the state after the last chunk.  states / out (batch, C, nheads, dim) float32,
+ * final = the state after the last chunk.  states (batch, C, nheads, dim) float32; out the same
+ * shape in float32 or bfloat16 (out_dtype: the recurrence itself runs in float32 registers, only
+ * the stored copy is rounded, as with out_dtype in mamba_state_pass.py:95-96); final float32;
  * dA_chunk addressed by (batch, head, chunk) strides (it is dA_cumsum[..., -1]); initial
  * (batch, nheads, dim) float32 may be NULL.  dim must be a multiple of 4.  With seq_idx the
  * state is dropped across a chunk whose last position has another id than the previous chunk's
@@ -76,7 +78,7 @@ int ssd_chunk_state_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64_t b_sg,
  * locate those positions and are ignored without seq_idx.
  * Replaces _state_passing_fwd, kernels/mamba_kernels/mamba_state_pass.py:84-115. */
 int ssd_state_passing_fwd(const float* states, const float* dA_chunk, int64_t da_sb, int64_t da_sh,
-                          int64_t da_sc, const float* initial, float* out, float* final_states,
+                          int64_t da_sc, const float* initial, void* out, int out_dtype, float* final_states,
                           int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, const int32_t* seq_idx,
                           int64_t seq_sb, int64_t seq_sl, int64_t seqlen, int64_t chunk, void* stream);
 
@@ -92,7 +94,9 @@ int ssd_bmm_chunk_fwd(const void* a, int64_t a_sb, int64_t a_sl, int64_t a_sg, c
 /* out[m,p] = exp(dA_m) * sum_n C[m,n] * prev[p,n]
  *          + sum_{k<=m} cb[m,k] * exp(min(dA_m - dA_k, 0)) * dt_k * x[k,p]  +  D * x[m,p],
  * then, with z: out_x = out (if out_x is not NULL) and out *= z * sigmoid(z).
- * cb float32 (batch, C, ngroups, Q, Q); prev float32 (batch, C, nheads, hdim, dstate); D float32
+ * cb float32 (batch, C, ngroups, Q, Q); prev (batch, C, nheads, hdim, dstate) in float32 or in
+ * `dtype` (states_dtype; the product rounds it to `dtype` either way, so the result is the same and
+ * the bfloat16 form moves half the bytes); D float32
  * (nheads) or (nheads, hdim) (d_has_hdim), may be NULL; z may be NULL; out_x shares out's strides.
  * With seq_idx the first term only reaches the rows m whose id equals that of the previous
  * chunk's last position (0 for the first chunk; mamba_scan_fwd.py:77-92); cb is expected to
@@ -101,22 +105,23 @@ int ssd_bmm_chunk_fwd(const void* a, int64_t a_sb, int64_t a_sl, int64_t a_sg, c
 int ssd_chunk_scan_fwd(const float* cb, const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
                        const void* z, int64_t z_sb, int64_t z_sl, int64_t z_sh, int dtype,
                        const float* dt, const float* dA_cumsum, const void* C, int64_t c_sb, int64_t c_sl,
-                       int64_t c_sg, const float* prev_states, const float* D, int d_has_hdim, void* out,
-                       int64_t o_sb, int64_t o_sl, int64_t o_sh, void* out_x, int64_t batch,
+                       int64_t c_sg, const void* prev_states, int states_dtype, const float* D, int d_has_hdim,
+                       void* out, int64_t o_sb, int64_t o_sl, int64_t o_sh, void* out_x, int64_t batch,
                        int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate,
                        int64_t chunk, const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream);
 
 /* ---------------------------------------------------------------- backward stages ---- */
 
-/* dprev_states[b,c,h,p,n] = sum_m round(dout[m,p] * exp(dA_m)) * C[m,n] (float32): the gradient of
- * the chunk scan with respect to the carried states.  With seq_idx only the rows m whose id
+/* dprev_states[b,c,h,p,n] = sum_m round(dout[m,p] * exp(dA_m)) * C[m,n]: the gradient of the chunk
+ * scan with respect to the carried states, accumulated in float32 and stored in float32 or in
+ * `dtype` (states_dtype; the dtype argument of the reference's launcher).  With seq_idx only the rows m whose id
  * equals that of the previous chunk's last position count (mamba_scan_bwd.py:63-71).
  * Replaces _chunk_scan_bwd_dstates,
  * kernels/mamba_kernels_bwd/mamba_scan_bwd.py:91-116. */
 int ssd_chunk_scan_bwd_dstates(const void* C, int64_t c_sb, int64_t c_sl, int64_t c_sg, const void* dout,
                                int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype, const float* dA_cumsum,
-                               float* dprev_states, int64_t batch, int64_t seqlen, int64_t nheads,
-                               int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
+                               void* dprev_states, int states_dtype, int64_t batch, int64_t seqlen,
+                               int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
                                const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream);
 
 /* Bytes of workspace ssd_state_passing_bwd needs (per-wave partial dot products). */
@@ -127,12 +132,16 @@ size_t ssd_state_passing_bwd_workspace_bytes(int64_t batch, int64_t nchunks, int
  * the gradient of the final state.  With G the gradient of the state entering the next chunk:
  * dstates[c] = G (the gradient of the chunk-local state), ddA_chunk[b,h,c] = exp(dA_chunk[c]) *
  * <states[c], G> (0 for c = 0 unless dinit is given), G <- exp(dA_chunk[c]) * G + dout[c];
- * dinit (batch, nheads, dim), may be NULL, receives the last G.  All float32.  With seq_idx the
+ * dinit (batch, nheads, dim), may be NULL, receives the last G.  All float32, except that states,
+ * dout and dstates may each be bfloat16 (states_dtype, dout_dtype, dstates_dtype, as with
+ * dstates_dtype / states_dtype in the reference's launcher; G itself stays in float32 registers).
+ * With seq_idx the
  * factor exp(dA_chunk[c]) is 0 for the chunks across which ssd_state_passing_fwd drops the state
  * (mamba_state_passing_bwd_dstates.py:72-80,105); seqlen and chunk as there.
  * Replaces _state_passing_bwd, kernels/mamba_kernels_bwd/mamba_state_passing_bwd_dstates.py:116-172. */
-int ssd_state_passing_bwd(const float* states, const float* dA_chunk, int64_t da_sb, int64_t da_sh,
-                          int64_t da_sc, const float* dout, const float* dfinal, float* dstates,
+int ssd_state_passing_bwd(const void* states, int states_dtype, const float* dA_chunk, int64_t da_sb, int64_t da_sh,
+                          int64_t da_sc, const void* dout, int dout_dtype, const float* dfinal, void* dstates,
+                          int dstates_dtype,
                           float* ddA_chunk, float* dinit, void* workspace, size_t workspace_bytes,
                           int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, const int32_t* seq_idx,
                           int64_t seq_sb, int64_t seq_sl, int64_t seqlen, int64_t chunk, void* stream);
@@ -142,12 +151,13 @@ int ssd_state_passing_bwd(const float* states, const float* dA_chunk, int64_t da
  * (may be NULL, then ddA_cumsum is not written): r_h[m] = sum_n db_h[m,n] * B[m,n] and
  * ddA_cumsum[b,h,c,j] = sum_{m<j} r_h[m], the gradient of the chunk states with respect to the
  * per-position dA.  With seq_idx the weight of row m is 0 unless its id equals that of the
- * chunk's last position (mamba_chunk_state_bwd_db.py:88-104).  Replaces _chunk_state_bwd_db,
+ * chunk's last position (mamba_chunk_state_bwd_db.py:88-104).  dstates in float32 or in `dtype`
+ * (states_dtype).  Replaces _chunk_state_bwd_db,
  * kernels/mamba_kernels_bwd/mamba_chunk_state_bwd_db.py:131-181 (one pass over all heads of a
  * group, so there is no split axis to sum afterwards). */
 int ssd_chunk_state_bwd_db(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype,
-                           const float* dt, const float* dA_cumsum, const float* dstates, const void* B,
-                           int64_t b_sb, int64_t b_sl, int64_t b_sg, float* dB, float* ddA_cumsum,
+                           const float* dt, const float* dA_cumsum, const void* dstates, int states_dtype,
+                           const void* B, int64_t b_sb, int64_t b_sl, int64_t b_sg, float* dB, float* ddA_cumsum,
                            int64_t batch, int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim,
                            int64_t dstate, int64_t chunk, const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl,
                            void* stream);
@@ -156,19 +166,20 @@ int ssd_chunk_state_bwd_db(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_
  * exp(dA_m): the part of dC that comes through the carried state.  With C (may be NULL):
  * ddA_cumsum_prev[b,h,c,m] = sum_n dc_h[m,n] * C[m,n].  With seq_idx the weight of row m is 0
  * unless its id equals that of the previous chunk's last position
- * (mamba_chunk_scan_bwd_dc.py:84-96).  Replaces _chunk_scan_bwd_dC,
+ * (mamba_chunk_scan_bwd_dc.py:84-96).  prev_states in float32 or in `dtype` (states_dtype), as
+ * for ssd_chunk_scan_fwd.  Replaces _chunk_scan_bwd_dC,
  * kernels/mamba_kernels_bwd/mamba_chunk_scan_bwd_dc.py:118-160. */
 int ssd_chunk_scan_bwd_dc(const void* dout, int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype,
-                          const float* dA_cumsum, const float* prev_states, const void* C, int64_t c_sb,
-                          int64_t c_sl, int64_t c_sg, float* dC, float* ddA_cumsum_prev, int64_t batch,
+                          const float* dA_cumsum, const void* prev_states, int states_dtype, const void* C,
+                          int64_t c_sb, int64_t c_sl, int64_t c_sg, float* dC, float* ddA_cumsum_prev, int64_t batch,
                           int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate,
                           int64_t chunk, const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream);
 
 /* acc[m,p] = exp(min(dA_last - dA_m, 0)) * sum_n B[m,n] * round(dstates[p,n])
  *          + sum_{k>=m} round(cb[k,m] * exp(min(dA_k - dA_m, 0))) * dout[k,p];
  * dx = acc * dt_m + D * dout (type `dtype`, dx's own strides), ddt[b,h,c,m] = sum_p acc[m,p] * x[m,p]
- * (float32, 0 past seqlen).  cb float32 (batch, C, ngroups, Q, Q), dstates float32
- * (batch, C, nheads, hdim, dstate), D as for ssd_chunk_scan_fwd.  dD_partial (may be NULL; needs D):
+ * (float32, 0 past seqlen).  cb float32 (batch, C, ngroups, Q, Q), dstates float32 or `dtype`
+ * (states_dtype) (batch, C, nheads, hdim, dstate), D as for ssd_chunk_scan_fwd.  dD_partial (may be NULL; needs D):
  * float32 (batch, C, nheads, S, hdim) with S = ssd_chunk_scan_chunk_state_bwd_dx_dD_slots(...),
  * every slot written: partial sums over positions of dout * x, whose sum over batch, C and S is
  * the gradient of D (nheads, hdim), summed over hdim too for a D of shape (nheads) -- the
@@ -180,7 +191,7 @@ int ssd_chunk_scan_bwd_dc(const void* dout, int64_t d_sb, int64_t d_sl, int64_t 
 int ssd_chunk_scan_chunk_state_bwd_dx(const float* cb, const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
                                       const void* dout, int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype,
                                       const float* dt, const float* dA_cumsum, const void* B, int64_t b_sb,
-                                      int64_t b_sl, int64_t b_sg, const float* dstates, const float* D,
+                                      int64_t b_sl, int64_t b_sg, const void* dstates, int states_dtype, const float* D,
                                       int d_has_hdim, void* dx, int64_t dx_sb, int64_t dx_sl, int64_t dx_sh,
                                       float* ddt, int64_t batch, int64_t seqlen, int64_t nheads,
                                       int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,

@@ -90,9 +90,12 @@ def test_ssd_validation_happens_before_any_launch():
     assert handle.ssd_chunk_state_fwd(*grp, *seq, 9, fake, fake, fake, 1, 64, 2, 1, 64, 64, 64, *ids, None) == -4
     assert handle.ssd_chunk_state_fwd(*grp, *seq, 0, fake, fake, fake, 1, 64, 3, 2, 64, 64, 64, *ids, None) == -2
     assert handle.ssd_bmm_chunk_fwd(*grp, *grp, 0, fake, 1, 1, 64, 1, 64, 64, *ids, None) == -4  # bf16 out of f32 in
-    assert handle.ssd_state_passing_fwd(fake, fake, 2, 1, 1, None, fake, fake, 1, 1, 2, 6, *ids, 0, 0, None) == -3
+    assert handle.ssd_state_passing_fwd(fake, fake, 2, 1, 1, None, fake, 0, fake, 1, 1, 2, 6, *ids, 0, 0, None) == -3
+    assert handle.ssd_state_passing_fwd(fake, fake, 2, 1, 1, None, fake, 7, fake, 1, 1, 2, 8, *ids, 0, 0, None) == -4
+    # carried states are float32 or of the inputs' type: bfloat16 states with float32 inputs are refused
+    assert handle.ssd_chunk_scan_bwd_dc(*seq, 0, fake, fake, 1, *grp, fake, fake, 1, 64, 2, 1, 64, 64, 64, *ids, None) == -4
     # a packed batch must come with the chunking that gives nchunks
-    assert handle.ssd_state_passing_fwd(fake, fake, 2, 1, 1, None, fake, fake, 1, 2, 2, 8, fake, 64, 1, 64, 16, None) == -2
+    assert handle.ssd_state_passing_fwd(fake, fake, 2, 1, 1, None, fake, 0, fake, 1, 2, 2, 8, fake, 64, 1, 64, 16, None) == -2
 
 
 def test_error_mapping():

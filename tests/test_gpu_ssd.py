@@ -76,6 +76,11 @@ def test_stages_vs_oracle(b, L, nh, P, g, N, Q, dtype, device):
     check_close("prev states", prev, prev_ref, F32)
     check_close("final states", fin, fin_ref, F32)
 
+    if dtype == BF16:  # the carried states stored in the inputs' type, as the combined forward asks
+        prev16, fin16 = _state_passing_fwd(st_ref.reshape(b, -1, nh, P * N).to(device), dA_d[..., -1],
+                                           initial_states=initd, out_dtype=BF16)
+        assert prev16.dtype == BF16 and torch.equal(prev16, prev.to(BF16)) and torch.equal(fin16, fin)
+
     cb_ref = S.bmm_chunk(C, B, Q)
     cb = _bmm_chunk_fwd(Cd, Bd, Q, output_dtype=torch.float32)
     check_close("CB", cb, cb_ref, small)
@@ -87,6 +92,9 @@ def test_stages_vs_oracle(b, L, nh, P, g, N, Q, dtype, device):
     out, out_x = _chunk_scan_fwd(cb_ref.to(device), xd, dt_d, dA_d, Cd, prev5.to(device), D=Dd, z=zd)
     check_close("out_x", out_x, outx_ref, dtype)
     check_close("out", out, out_ref, dtype)
+    if dtype == BF16:  # the product rounds the carried states to bfloat16 either way
+        out16, _ = _chunk_scan_fwd(cb_ref.to(device), xd, dt_d, dA_d, Cd, prev5.to(device).to(BF16), D=Dd, z=zd)
+        assert torch.equal(out16, out)
     D2 = torch.randn(nh, P, generator=gen)
     out_ref2, _ = S.chunk_scan(cb_ref, x, dt_ref, dA_ref, C, prev5, D2, None, round_to=rt)
     out2, none = _chunk_scan_fwd(cb_ref.to(device), xd, dt_d, dA_d, Cd, prev5.to(device), D=D2.to(device))

@@ -58,17 +58,26 @@ def test_dstates_db_dc_vs_oracle(b, L, nh, P, g, N, Q, dtype, device):
 
     got = _chunk_scan_bwd_dstates(d(C), d(dA_cs), d(dout), dtype=torch.float32)
     check_close("dprev_states", got, S.bwd_dstates(C, dA_cs, dout, round_to=rt), dtype)
+    if dtype == BF16:  # stored in the inputs' type by the kernel: the rounded float32 result
+        got16 = _chunk_scan_bwd_dstates(d(C), d(dA_cs), d(dout))
+        assert got16.dtype == BF16 and torch.equal(got16, got.to(BF16))
 
     dB_ref, ddA_ref = S.chunk_state_bwd_db(x, dt, dA_cs, dstates, B=B, ngroups=g, round_to=rt)
     dB, ddA = _chunk_state_bwd_db(d(x), d(dt), d(dA_cs), d(dstates), B=d(B), ngroups=g)
     check_close("dB", dB, dB_ref, dtype)
     check_close("ddA_cumsum (chunk state)", ddA, ddA_ref, dtype)
     check_close("dB without B", _chunk_state_bwd_db(d(x), d(dt), d(dA_cs), d(dstates), ngroups=g), dB_ref, dtype)
+    if dtype == BF16:  # gradient states already in bfloat16: the product rounds them there either way
+        dB16, ddA16 = _chunk_state_bwd_db(d(x), d(dt), d(dA_cs), d(dstates).to(BF16), B=d(B), ngroups=g)
+        assert torch.equal(dB16, dB) and torch.equal(ddA16, ddA)
 
     dC_ref, ddAp_ref = S.chunk_scan_bwd_dC(prev, dA_cs, dout, C=C, ngroups=g, round_to=rt)
     dC, ddAp = _chunk_scan_bwd_dC(d(prev), d(dA_cs), d(dout), C=d(C), ngroups=g)
     check_close("dC", dC, dC_ref, dtype)
     check_close("ddA_cumsum_prev", ddAp, ddAp_ref, dtype)
+    if dtype == BF16:  # carried states already in bfloat16: the product rounds them there either way
+        dC16, ddAp16 = _chunk_scan_bwd_dC(d(prev).to(BF16), d(dA_cs), d(dout), C=d(C), ngroups=g)
+        assert torch.equal(dC16, dC) and torch.equal(ddAp16, ddAp)
 
 
 @pytest.mark.parametrize("has_init", [False, True])
@@ -95,6 +104,26 @@ def test_state_passing_bwd_vs_oracle(b, nc, nh, dim, has_init, device):
     got0 = _state_passing_bwd(states.to(device), dA.to(device), dout.to(device))
     ref0 = S.state_passing_bwd(states, dA, dout)
     check_close("dstates, no dfinal", got0[0], ref0[0], F32)
+    # states in bfloat16 (what the combined forward keeps): read as they are, same result as their
+    # float32 copy
+    s16 = states.to(BF16)
+    got16 = _state_passing_bwd(s16.to(device), dA.to(device), dout.to(device), dfinal_states=dfin.to(device))
+    ref16 = S.state_passing_bwd(s16.float(), dA, dout, dfin)
+    check_close("dstates, bfloat16 states", got16[0], ref16[0], F32)
+    check_close("ddA_chunk_cumsum, bfloat16 states", got16[1], ref16[1], F32)
+    # all three state-sized tensors in bfloat16 (dstates_dtype / states_dtype of the reference's
+    # launcher): the recurrence itself stays in float32, only what is stored is rounded
+    d16 = dout.to(BF16)
+    got16 = _state_passing_bwd(s16.to(device), dA.to(device), d16.to(device), dfinal_states=dfin.to(device),
+                               has_initial_states=has_init)
+    ref16 = S.state_passing_bwd(s16.float(), dA, d16.float(), dfin, has_initial_states=has_init)
+    assert got16[0].dtype == BF16
+    check_close("dstates, all bfloat16", got16[0], ref16[0], BF16)
+    check_close("ddA_chunk_cumsum, all bfloat16", got16[1], ref16[1], F32)
+    mixed = _state_passing_bwd(s16.to(device), dA.to(device), d16.to(device), dfinal_states=dfin.to(device),
+                               dstates_dtype=F32)
+    assert mixed[0].dtype == F32
+    check_close("dstates, float32 out of bfloat16 in", mixed[0], ref16[0], F32)
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
@@ -112,6 +141,10 @@ def test_dx_vs_oracle(b, L, nh, P, g, N, Q, dtype, device):
     check_close("dx", dx, dx_ref, dtype)
     check_close("ddt", ddt, ddt_ref, dtype, loose=dtype == BF16)
     check_close("dD", dD, dD_ref, F32)
+    if dtype == BF16:  # gradient states already in bfloat16
+        dx16, ddt16, _ = _chunk_scan_chunk_state_bwd_dx(d(x), d(dt), d(dA_cs), d(B), d(cb), d(dout), d(dstates).to(BF16),
+                                                        D=d(D))
+        assert torch.equal(dx16, dx) and torch.equal(ddt16, ddt)
     D2 = torch.randn(nh, P, generator=torch.Generator().manual_seed(1))
     dx_ref2, _, dD_ref2 = S.chunk_scan_chunk_state_bwd_dx(x, dt, dA_cs, B, cb, dout, dstates, D=D2, round_to=rt)
     dx2, _, dD2 = _chunk_scan_chunk_state_bwd_dx(d(x), d(dt), d(dA_cs), d(B), d(cb), d(dout), d(dstates), D=d(D2))

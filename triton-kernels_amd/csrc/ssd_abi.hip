@@ -4,6 +4,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "ema_gemm_kernels.h"
 #include "ssd_kernels.h"
 
@@ -33,6 +35,12 @@ int check_vec(const void* p, int64_t sb, int64_t sl, int64_t sh, int dtype, int6
 int check_f32(const void* p) {
   if (!p) return SSD_ERR_NULL;
   return reinterpret_cast<uintptr_t>(p) % 16 ? SSD_ERR_ALIGN : SSD_OK;
+}
+
+// A carried-state tensor is float32 or of the inputs' type (16-byte aligned either way).
+int check_state(const void* p, int state_dtype, int dtype) {
+  if (state_dtype != SSD_F32 && state_dtype != dtype) return SSD_ERR_DTYPE;
+  return check_f32(p);
 }
 
 struct Dims {
@@ -87,17 +95,24 @@ struct StateLaunch {
   const void *x, *B;
   Strides3 sx, sB;
   const float *dt, *dA;
-  float* states;
+  void* states;
+  int states_dtype;
   Dims d;
   SeqIdx seq;
   hipStream_t st;
   template <typename T, int P, int N>
   int run() const {
-    auto kernel = ssd_chunk_state_kernel<T, P, N, MODE>;
+    if constexpr (!std::is_same<T, float>::value)
+      if (states_dtype != SSD_F32) return run_as<T, P, N, T>();
+    return run_as<T, P, N, float>();
+  }
+  template <typename T, int P, int N, typename TO>
+  int run_as() const {
+    auto kernel = ssd_chunk_state_kernel<T, P, N, MODE, TO>;
     constexpr int smem = StateSmem<T, P, N>::kBytes;
     SSD_TRY(allow_smem(kernel, smem));
     hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh)), dim3(256), smem, st, (const T*)x, sx,
-                       (const T*)B, sB, dt, dA, states, (int)d.nh, (int)(d.nh / d.g), (int)d.L, (int)d.Q,
+                       (const T*)B, sB, dt, dA, (TO*)states, (int)d.nh, (int)(d.nh / d.g), (int)d.L, (int)d.Q,
                        (int)d.C, seq);
     return launched();
   }
@@ -107,7 +122,10 @@ struct ScanLaunch {
   const float* cb;
   const void *x, *z, *C;
   Strides3 sx, sz, sC, so;
-  const float *dt, *dA, *prev, *D;
+  const float *dt, *dA;
+  const void* prev;
+  int prev_dtype;
+  const float* D;
   int d_has_hdim;
   void *out, *out_x;
   Dims d;
@@ -115,25 +133,31 @@ struct ScanLaunch {
   hipStream_t st;
   template <typename T, int P, int N>
   int run() const {
+    if constexpr (!std::is_same<T, float>::value)
+      if (prev_dtype != SSD_F32) return run_as<T, P, N, T>();
+    return run_as<T, P, N, float>();
+  }
+  template <typename T, int P, int N, typename TS>
+  int run_as() const {
     constexpr int wide_smem = WideSmem<T, P, N>::kBytes;
     if (d.Q % 256 == 0 && wide_smem <= kLdsBytes) {  // 256-row super-tiles, no barrier inside the k loop
-      auto kernel = ssd_chunk_scan_wide_kernel<T, P, N>;
+      auto kernel = ssd_chunk_scan_wide_kernel<T, P, N, TS>;
       constexpr int smem = wide_smem;
       SSD_TRY(allow_smem(kernel, smem));
       const int stiles = (int)(d.Q / 256);
       hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh * stiles)), dim3(256), smem, st, cb,
-                         (const T*)x, sx, (const T*)z, sz, dt, dA, (const T*)C, sC, prev, D, d_has_hdim, (T*)out,
-                         so, (T*)out_x, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C,
+                         (const T*)x, sx, (const T*)z, sz, dt, dA, (const T*)C, sC, (const TS*)prev, D, d_has_hdim,
+                         (T*)out, so, (T*)out_x, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C,
                          stiles, seq);
       return launched();
     }
-    auto kernel = ssd_chunk_scan_kernel<T, P, N>;
+    auto kernel = ssd_chunk_scan_kernel<T, P, N, TS>;
     constexpr int smem = ScanSmem<T, P, N>::kBytes;
     SSD_TRY(allow_smem(kernel, smem));
     const int mtiles = (int)((d.Q + 63) / 64);
     hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh * mtiles)), dim3(256), smem, st, cb,
-                       (const T*)x, sx, (const T*)z, sz, dt, dA, (const T*)C, sC, prev, D, d_has_hdim, (T*)out, so,
-                       (T*)out_x, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C, mtiles,
+                       (const T*)x, sx, (const T*)z, sz, dt, dA, (const T*)C, sC, (const TS*)prev, D, d_has_hdim,
+                       (T*)out, so, (T*)out_x, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C, mtiles,
                        seq);
     return launched();
   }
@@ -143,7 +167,10 @@ struct DxLaunch {
   const float* cb;
   const void *x, *dout, *B;
   Strides3 sx, sd, sB, sdx;
-  const float *dt, *dA, *dstates, *D;
+  const float *dt, *dA;
+  const void* dstates;
+  int states_dtype;
+  const float* D;
   int d_has_hdim;
   void* dx;
   float* ddt;
@@ -158,24 +185,30 @@ struct DxLaunch {
   }
   template <typename T, int P, int N>
   int run() const {
+    if constexpr (!std::is_same<T, float>::value)
+      if (states_dtype != SSD_F32) return run_as<T, P, N, T>();
+    return run_as<T, P, N, float>();
+  }
+  template <typename T, int P, int N, typename TS>
+  int run_as() const {
     constexpr int wide_smem = WideSmem<T, P, N>::kBytes;
     if (wide<T, P, N>(d.Q)) {
-      auto kernel = ssd_chunk_scan_bwd_dx_wide_kernel<T, P, N>;
+      auto kernel = ssd_chunk_scan_bwd_dx_wide_kernel<T, P, N, TS>;
       SSD_TRY(allow_smem(kernel, wide_smem));
       const int stiles = (int)(d.Q / 256);
       hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh * stiles)), dim3(256), wide_smem, st, cb,
-                         (const T*)x, sx, (const T*)dout, sd, dt, dA, (const T*)B, sB, dstates, D, d_has_hdim,
-                         (T*)dx, sdx, ddt, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C,
-                         stiles, seq, dD_part);
+                         (const T*)x, sx, (const T*)dout, sd, dt, dA, (const T*)B, sB, (const TS*)dstates, D,
+                         d_has_hdim, (T*)dx, sdx, ddt, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q,
+                         (int)d.C, stiles, seq, dD_part);
       return launched();
     }
-    auto kernel = ssd_chunk_scan_bwd_dx_kernel<T, P, N>;
+    auto kernel = ssd_chunk_scan_bwd_dx_kernel<T, P, N, TS>;
     constexpr int smem = ScanSmem<T, P, N>::kBytes;
     SSD_TRY(allow_smem(kernel, smem));
     const int mtiles = (int)((d.Q + 63) / 64);
     hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh * mtiles)), dim3(256), smem, st, cb,
-                       (const T*)x, sx, (const T*)dout, sd, dt, dA, (const T*)B, sB, dstates, D, d_has_hdim, (T*)dx,
-                       sdx, ddt, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C, mtiles,
+                       (const T*)x, sx, (const T*)dout, sd, dt, dA, (const T*)B, sB, (const TS*)dstates, D, d_has_hdim,
+                       (T*)dx, sdx, ddt, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C, mtiles,
                        seq, dD_part);
     return launched();
   }
@@ -194,7 +227,9 @@ template <int MODE>
 struct GroupLaunch {
   const void* a;
   Strides3 sa;
-  const float *s, *dt, *dA;
+  const void* s;
+  int s_dtype;
+  const float *dt, *dA;
   const void* bc;
   Strides3 sbc;
   float *out, *ddA;
@@ -203,13 +238,19 @@ struct GroupLaunch {
   hipStream_t st;
   template <typename T, int P, int N>
   int run() const {
-    auto kernel = ssd_group_grad_kernel<T, P, N, MODE>;
+    if constexpr (!std::is_same<T, float>::value)
+      if (s_dtype != SSD_F32) return run_as<T, P, N, T>();
+    return run_as<T, P, N, float>();
+  }
+  template <typename T, int P, int N, typename TS>
+  int run_as() const {
+    auto kernel = ssd_group_grad_kernel<T, P, N, MODE, TS>;
     constexpr int smem = GroupSmem<T, P, N>::kBytes;
     SSD_TRY(allow_smem(kernel, smem));
     const int mtiles = (int)((d.Q + 63) / 64);
     if (d.batch * d.C * d.g * mtiles > 0x7fffffff) return SSD_ERR_SHAPE;
     hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.g * mtiles)), dim3(256), smem, st, (const T*)a, sa,
-                       s, dt, dA, (const T*)bc, sbc, out, ddA, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L,
+                       (const TS*)s, dt, dA, (const T*)bc, sbc, out, ddA, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L,
                        (int)d.Q, (int)d.C, mtiles, seq);
     return launched();
   }
@@ -275,16 +316,17 @@ int ssd_chunk_state_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64_t b_sg,
   SSD_TRY(check_f32(states));
   return dispatch_tpn(dtype, hdim, dstate,
                       StateLaunch<0>{x, B, Strides3{x_sb, x_sl, x_sh}, Strides3{b_sb, b_sl, b_sg}, dt, dA_cumsum,
-                                     states, d, as_seq(seq_idx, seq_sb, seq_sl), as_stream(stream)});
+                                     states, SSD_F32, d, as_seq(seq_idx, seq_sb, seq_sl), as_stream(stream)});
 }
 
 int ssd_state_passing_fwd(const float* states, const float* dA_chunk, int64_t da_sb, int64_t da_sh,
-                          int64_t da_sc, const float* initial, float* out, float* final_states,
+                          int64_t da_sc, const float* initial, void* out, int out_dtype, float* final_states,
                           int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, const int32_t* seq_idx,
                           int64_t seq_sb, int64_t seq_sl, int64_t seqlen, int64_t chunk, void* stream) {
   if (batch <= 0 || nchunks <= 0 || nheads <= 0 || dim <= 0) return SSD_ERR_SHAPE;
   if (dim % 4) return SSD_ERR_ALIGN;
   if (!dA_chunk) return SSD_ERR_NULL;
+  SSD_TRY(check_dtype(out_dtype));
   SSD_TRY(check_seq_chunks(seq_idx, seqlen, chunk, nchunks));
   SSD_TRY(check_f32(states));
   SSD_TRY(check_f32(out));
@@ -293,9 +335,14 @@ int ssd_state_passing_fwd(const float* states, const float* dA_chunk, int64_t da
   const int tiles = (int)((dim + 1023) / 1024);
   const int64_t grid = batch * nheads * tiles;
   if (grid > 0x7fffffff || dim > (1 << 24)) return SSD_ERR_SHAPE;
-  hipLaunchKernelGGL(ssd_state_passing_kernel, dim3((unsigned)grid), dim3(256), 0, as_stream(stream), states,
-                     dA_chunk, da_sb, da_sh, da_sc, initial, out, final_states, (int)nheads, (int)nchunks, (int)dim,
-                     tiles, as_seq(seq_idx, seq_sb, seq_sl), (int)seqlen, (int)chunk);
+  if (out_dtype == SSD_BF16)
+    hipLaunchKernelGGL(ssd_state_passing_kernel<bf16_t>, dim3((unsigned)grid), dim3(256), 0, as_stream(stream), states,
+                       dA_chunk, da_sb, da_sh, da_sc, initial, (bf16_t*)out, final_states, (int)nheads, (int)nchunks,
+                       (int)dim, tiles, as_seq(seq_idx, seq_sb, seq_sl), (int)seqlen, (int)chunk);
+  else
+    hipLaunchKernelGGL(ssd_state_passing_kernel<float>, dim3((unsigned)grid), dim3(256), 0, as_stream(stream), states,
+                       dA_chunk, da_sb, da_sh, da_sc, initial, (float*)out, final_states, (int)nheads, (int)nchunks,
+                       (int)dim, tiles, as_seq(seq_idx, seq_sb, seq_sl), (int)seqlen, (int)chunk);
   return launched();
 }
 
@@ -329,8 +376,8 @@ int ssd_bmm_chunk_fwd(const void* a, int64_t a_sb, int64_t a_sl, int64_t a_sg, c
 int ssd_chunk_scan_fwd(const float* cb, const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
                        const void* z, int64_t z_sb, int64_t z_sl, int64_t z_sh, int dtype,
                        const float* dt, const float* dA_cumsum, const void* C, int64_t c_sb, int64_t c_sl,
-                       int64_t c_sg, const float* prev_states, const float* D, int d_has_hdim, void* out,
-                       int64_t o_sb, int64_t o_sl, int64_t o_sh, void* out_x, int64_t batch,
+                       int64_t c_sg, const void* prev_states, int states_dtype, const float* D, int d_has_hdim,
+                       void* out, int64_t o_sb, int64_t o_sl, int64_t o_sh, void* out_x, int64_t batch,
                        int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate,
                        int64_t chunk, const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream) {
   Dims d;
@@ -344,19 +391,20 @@ int ssd_chunk_scan_fwd(const float* cb, const void* x, int64_t x_sb, int64_t x_s
   if (out_x && reinterpret_cast<uintptr_t>(out_x) % 16) return SSD_ERR_ALIGN;
   if (!dt || !dA_cumsum) return SSD_ERR_NULL;
   SSD_TRY(check_f32(cb));
-  SSD_TRY(check_f32(prev_states));
+  SSD_TRY(check_state(prev_states, states_dtype, dtype));
   if (batch * d.C * nheads * ((chunk + 63) / 64) > 0x7fffffff) return SSD_ERR_SHAPE;
   return dispatch_tpn(dtype, hdim, dstate,
                       ScanLaunch{cb, x, z, C, Strides3{x_sb, x_sl, x_sh}, Strides3{z_sb, z_sl, z_sh},
                                  Strides3{c_sb, c_sl, c_sg}, Strides3{o_sb, o_sl, o_sh}, dt, dA_cumsum,
-                                 prev_states, D, d_has_hdim, out, out_x, d, as_seq(seq_idx, seq_sb, seq_sl),
+                                 prev_states, states_dtype, D, d_has_hdim, out, out_x, d,
+                                 as_seq(seq_idx, seq_sb, seq_sl),
                                  as_stream(stream)});
 }
 
 int ssd_chunk_scan_bwd_dstates(const void* C, int64_t c_sb, int64_t c_sl, int64_t c_sg, const void* dout,
                                int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype, const float* dA_cumsum,
-                               float* dprev_states, int64_t batch, int64_t seqlen, int64_t nheads,
-                               int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
+                               void* dprev_states, int states_dtype, int64_t batch, int64_t seqlen,
+                               int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
                                const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream) {
   Dims d;
   SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
@@ -365,10 +413,10 @@ int ssd_chunk_scan_bwd_dstates(const void* C, int64_t c_sb, int64_t c_sl, int64_
   SSD_TRY(check_vec(dout, d_sb, d_sl, d_sh, dtype, hdim));
   SSD_TRY(check_vec(C, c_sb, c_sl, c_sg, dtype, dstate));
   if (!dA_cumsum) return SSD_ERR_NULL;
-  SSD_TRY(check_f32(dprev_states));
+  SSD_TRY(check_state(dprev_states, states_dtype, dtype));
   return dispatch_tpn(dtype, hdim, dstate,
                       StateLaunch<1>{dout, C, Strides3{d_sb, d_sl, d_sh}, Strides3{c_sb, c_sl, c_sg}, dA_cumsum,
-                                     dA_cumsum, dprev_states, d, as_seq(seq_idx, seq_sb, seq_sl),
+                                     dA_cumsum, dprev_states, states_dtype, d, as_seq(seq_idx, seq_sb, seq_sl),
                                      as_stream(stream)});
 }
 
@@ -378,8 +426,9 @@ size_t ssd_state_passing_bwd_workspace_bytes(int64_t batch, int64_t nchunks, int
   return (size_t)(batch * nheads * nchunks * tiles * 4) * sizeof(float);
 }
 
-int ssd_state_passing_bwd(const float* states, const float* dA_chunk, int64_t da_sb, int64_t da_sh,
-                          int64_t da_sc, const float* dout, const float* dfinal, float* dstates,
+int ssd_state_passing_bwd(const void* states, int states_dtype, const float* dA_chunk, int64_t da_sb, int64_t da_sh,
+                          int64_t da_sc, const void* dout, int dout_dtype, const float* dfinal, void* dstates,
+                          int dstates_dtype,
                           float* ddA_chunk, float* dinit, void* workspace, size_t workspace_bytes,
                           int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, const int32_t* seq_idx,
                           int64_t seq_sb, int64_t seq_sl, int64_t seqlen, int64_t chunk, void* stream) {
@@ -388,6 +437,9 @@ int ssd_state_passing_bwd(const float* states, const float* dA_chunk, int64_t da
   if (!dA_chunk || !ddA_chunk) return SSD_ERR_NULL;
   SSD_TRY(check_seq_chunks(seq_idx, seqlen, chunk, nchunks));
   const SeqIdx seq = as_seq(seq_idx, seq_sb, seq_sl);
+  SSD_TRY(check_dtype(states_dtype));
+  SSD_TRY(check_dtype(dout_dtype));
+  SSD_TRY(check_dtype(dstates_dtype));
   SSD_TRY(check_f32(states));
   SSD_TRY(check_f32(dout));
   SSD_TRY(check_f32(dstates));
@@ -400,9 +452,25 @@ int ssd_state_passing_bwd(const float* states, const float* dA_chunk, int64_t da
   if (grid > 0x7fffffff || dim > (1 << 24)) return SSD_ERR_SHAPE;
   hipStream_t st = as_stream(stream);
   float* part = static_cast<float*>(workspace);
-  hipLaunchKernelGGL(ssd_state_passing_bwd_kernel, dim3((unsigned)grid), dim3(256), 0, st, states, dA_chunk, da_sb,
-                     da_sh, da_sc, dout, dfinal, dstates, part, dinit, (int)nheads, (int)nchunks, (int)dim, tiles, seq,
-                     (int)seqlen, (int)chunk);
+  // the three tensors are float32 or bfloat16 independently of each other
+  auto launch = [&](auto ts, auto td, auto tg) {
+    using TS = decltype(ts);
+    using TD = decltype(td);
+    using TG = decltype(tg);
+    hipLaunchKernelGGL((ssd_state_passing_bwd_kernel<TS, TD, TG>), dim3((unsigned)grid), dim3(256), 0, st,
+                       (const TS*)states, dA_chunk, da_sb, da_sh, da_sc, (const TD*)dout, dfinal, (TG*)dstates, part,
+                       dinit, (int)nheads, (int)nchunks, (int)dim, tiles, seq, (int)seqlen, (int)chunk);
+  };
+  auto pick_g = [&](auto ts, auto td) {
+    if (dstates_dtype == SSD_BF16) launch(ts, td, bf16_t());
+    else launch(ts, td, float());
+  };
+  auto pick_d = [&](auto ts) {
+    if (dout_dtype == SSD_BF16) pick_g(ts, bf16_t());
+    else pick_g(ts, float());
+  };
+  if (states_dtype == SSD_BF16) pick_d(bf16_t());
+  else pick_d(float());
   SSD_TRY(launched());
   const int64_t total = batch * nheads * nchunks;
   hipLaunchKernelGGL(ssd_state_passing_bwd_finish_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
@@ -412,8 +480,8 @@ int ssd_state_passing_bwd(const float* states, const float* dA_chunk, int64_t da
 }
 
 int ssd_chunk_state_bwd_db(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype,
-                           const float* dt, const float* dA_cumsum, const float* dstates, const void* B,
-                           int64_t b_sb, int64_t b_sl, int64_t b_sg, float* dB, float* ddA_cumsum,
+                           const float* dt, const float* dA_cumsum, const void* dstates, int states_dtype,
+                           const void* B, int64_t b_sb, int64_t b_sl, int64_t b_sg, float* dB, float* ddA_cumsum,
                            int64_t batch, int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim,
                            int64_t dstate, int64_t chunk, const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl,
                            void* stream) {
@@ -423,12 +491,12 @@ int ssd_chunk_state_bwd_db(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_
   if (!dim_ok(hdim) || !dim_ok(dstate)) return SSD_ERR_UNSUPPORTED;
   SSD_TRY(check_vec(x, x_sb, x_sl, x_sh, dtype, hdim));
   if (!dt || !dA_cumsum || !dB) return SSD_ERR_NULL;
-  SSD_TRY(check_f32(dstates));
+  SSD_TRY(check_state(dstates, states_dtype, dtype));
   if (B && !ddA_cumsum) return SSD_ERR_NULL;
   if (B) SSD_TRY(check_vec(B, b_sb, b_sl, b_sg, dtype, dstate));
   hipStream_t st = as_stream(stream);
   SSD_TRY(dispatch_tpn(dtype, hdim, dstate,
-                       GroupLaunch<0>{x, Strides3{x_sb, x_sl, x_sh}, dstates, dt, dA_cumsum, B,
+                       GroupLaunch<0>{x, Strides3{x_sb, x_sl, x_sh}, dstates, states_dtype, dt, dA_cumsum, B,
                                       Strides3{b_sb, b_sl, b_sg}, dB, ddA_cumsum, d,
                                       as_seq(seq_idx, seq_sb, seq_sl), st}));
   if (!B) return SSD_OK;
@@ -436,7 +504,8 @@ int ssd_chunk_state_bwd_db(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_
 }
 
 int ssd_chunk_scan_bwd_dc(const void* dout, int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype,
-                          const float* dA_cumsum, const float* prev_states, const void* C, int64_t c_sb,
+                          const float* dA_cumsum, const void* prev_states, int states_dtype, const void* C,
+                          int64_t c_sb,
                           int64_t c_sl, int64_t c_sg, float* dC, float* ddA_cumsum_prev, int64_t batch,
                           int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t hdim, int64_t dstate,
                           int64_t chunk, const int32_t* seq_idx, int64_t seq_sb, int64_t seq_sl, void* stream) {
@@ -446,11 +515,12 @@ int ssd_chunk_scan_bwd_dc(const void* dout, int64_t d_sb, int64_t d_sl, int64_t 
   if (!dim_ok(hdim) || !dim_ok(dstate)) return SSD_ERR_UNSUPPORTED;
   SSD_TRY(check_vec(dout, d_sb, d_sl, d_sh, dtype, hdim));
   if (!dA_cumsum || !dC) return SSD_ERR_NULL;
-  SSD_TRY(check_f32(prev_states));
+  SSD_TRY(check_state(prev_states, states_dtype, dtype));
   if (C && !ddA_cumsum_prev) return SSD_ERR_NULL;
   if (C) SSD_TRY(check_vec(C, c_sb, c_sl, c_sg, dtype, dstate));
   return dispatch_tpn(dtype, hdim, dstate,
-                      GroupLaunch<1>{dout, Strides3{d_sb, d_sl, d_sh}, prev_states, dA_cumsum, dA_cumsum, C,
+                      GroupLaunch<1>{dout, Strides3{d_sb, d_sl, d_sh}, prev_states, states_dtype, dA_cumsum, dA_cumsum,
+                                     C,
                                      Strides3{c_sb, c_sl, c_sg}, dC, ddA_cumsum_prev, d,
                                      as_seq(seq_idx, seq_sb, seq_sl), as_stream(stream)});
 }
@@ -458,7 +528,7 @@ int ssd_chunk_scan_bwd_dc(const void* dout, int64_t d_sb, int64_t d_sl, int64_t 
 int ssd_chunk_scan_chunk_state_bwd_dx(const float* cb, const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
                                       const void* dout, int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype,
                                       const float* dt, const float* dA_cumsum, const void* B, int64_t b_sb,
-                                      int64_t b_sl, int64_t b_sg, const float* dstates, const float* D,
+                                      int64_t b_sl, int64_t b_sg, const void* dstates, int states_dtype, const float* D,
                                       int d_has_hdim, void* dx, int64_t dx_sb, int64_t dx_sl, int64_t dx_sh,
                                       float* ddt, int64_t batch, int64_t seqlen, int64_t nheads,
                                       int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk,
@@ -476,11 +546,12 @@ int ssd_chunk_scan_chunk_state_bwd_dx(const float* cb, const void* x, int64_t x_
   SSD_TRY(check_vec(B, b_sb, b_sl, b_sg, dtype, dstate));
   if (!dt || !dA_cumsum || !ddt) return SSD_ERR_NULL;
   SSD_TRY(check_f32(cb));
-  SSD_TRY(check_f32(dstates));
+  SSD_TRY(check_state(dstates, states_dtype, dtype));
   if (batch * d.C * nheads * ((chunk + 63) / 64) > 0x7fffffff) return SSD_ERR_SHAPE;
   return dispatch_tpn(dtype, hdim, dstate,
                       DxLaunch{cb, x, dout, B, Strides3{x_sb, x_sl, x_sh}, Strides3{d_sb, d_sl, d_sh},
-                               Strides3{b_sb, b_sl, b_sg}, Strides3{dx_sb, dx_sl, dx_sh}, dt, dA_cumsum, dstates, D,
+                               Strides3{b_sb, b_sl, b_sg}, Strides3{dx_sb, dx_sl, dx_sh}, dt, dA_cumsum, dstates,
+                               states_dtype, D,
                                d_has_hdim, dx, ddt, d, as_seq(seq_idx, seq_sb, seq_sl), dD_partial,
                                as_stream(stream)});
 }

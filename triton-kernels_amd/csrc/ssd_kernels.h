@@ -288,10 +288,10 @@ struct StateSmem {
   static constexpr int kBytes = 2 * kStage;  // two stages: one being multiplied, one being filled
 };
 
-template <typename T, int P, int N, int MODE>
+template <typename T, int P, int N, int MODE, typename TO>
 __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
     const T* __restrict__ x, Strides3 sx, const T* __restrict__ B, Strides3 sB,
-    const float* __restrict__ dt, const float* __restrict__ dA_cs, float* __restrict__ states, int nh,
+    const float* __restrict__ dt, const float* __restrict__ dA_cs, TO* __restrict__ states, int nh,
     int heads_per_group, int L, int Q, int C, SeqIdx seq) {
   using S = StateSmem<T, P, N>;
   constexpr int KT = S::KT, PX = S::PX, PB = S::PB, KG = Tile<T>::KG;
@@ -358,13 +358,13 @@ __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
       }
     }
   }
-  float* out = states + (((b * C + c) * nh + h) * (int64_t)P) * N;
+  TO* out = states + (((b * C + c) * nh + h) * (int64_t)P) * N;
 #pragma unroll
   for (int i = 0; i < BPW; ++i) {
     const int j = wave + 4 * i, mi = j % MB, ni = j / MB;
 #pragma unroll
     for (int v = 0; v < 16; ++v)
-      __builtin_nontemporal_store(acc[i][v], out + (int64_t)(32 * mi + acc_row(v, lane)) * N + 32 * ni + (lane & 31));
+      __builtin_nontemporal_store((TO)acc[i][v], out + (int64_t)(32 * mi + acc_row(v, lane)) * N + 32 * ni + (lane & 31));
   }
 }
 
@@ -379,6 +379,25 @@ __device__ __forceinline__ void stream_store4(float* p, float4 v) {
   __builtin_nontemporal_store(w, reinterpret_cast<f32x4*>(p));
 }
 
+// Four adjacent elements of a carried-state tensor, which is float32 or already rounded to
+// bfloat16 (what the reference's combined forward hands from its state passing to its chunk scan,
+// kernels/ema_combined.py:48-50: out_dtype = C.dtype).  STREAM: the non-temporal hint.
+template <bool STREAM>
+__device__ __forceinline__ float4 state_load4(const float* p) {
+  return STREAM ? stream_load4(p) : *reinterpret_cast<const float4*>(p);
+}
+template <bool STREAM>
+__device__ __forceinline__ float4 state_load4(const bf16_t* p) {
+  const ema::bf16x4 v = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const ema::bf16x4*>(p))
+                               : *reinterpret_cast<const ema::bf16x4*>(p);
+  return make_float4((float)v[0], (float)v[1], (float)v[2], (float)v[3]);
+}
+__device__ __forceinline__ void state_store4(float* p, float4 v) { stream_store4(p, v); }
+__device__ __forceinline__ void state_store4(bf16_t* p, float4 v) {
+  const ema::bf16x4 w = {(bf16_t)v.x, (bf16_t)v.y, (bf16_t)v.z, (bf16_t)v.w};
+  __builtin_nontemporal_store(w, reinterpret_cast<ema::bf16x4*>(p));
+}
+
 // ------------------------------------------------------------------------------------
 // state_passing.  out[b, c] = state entering chunk c, state <- exp(dA_chunk[c]) * state +
 // states[b, c]; the value after the last chunk goes to final.  One thread per four adjacent
@@ -387,9 +406,10 @@ __device__ __forceinline__ void stream_store4(float* p, float4 v) {
 // last column of dA_cumsum).  In a packed batch the state is dropped across a chunk whose last
 // position has another id than the previous chunk's last position.
 // ------------------------------------------------------------------------------------
+template <typename TO>
 __global__ __launch_bounds__(256) void ssd_state_passing_kernel(
     const float* __restrict__ states, const float* __restrict__ dA_chunk, int64_t da_sb, int64_t da_sh,
-    int64_t da_sc, const float* __restrict__ initial, float* __restrict__ out, float* __restrict__ final_states,
+    int64_t da_sc, const float* __restrict__ initial, TO* __restrict__ out, float* __restrict__ final_states,
     int nh, int C, int dim, int tiles, SeqIdx seq, int L, int Q) {
   const int tile = blockIdx.x % tiles;
   const int h = (blockIdx.x / tiles) % nh;
@@ -398,7 +418,7 @@ __global__ __launch_bounds__(256) void ssd_state_passing_kernel(
   if (e >= dim) return;
   const int64_t chunk_stride = (int64_t)nh * dim;
   const float* src = states + (b * C * nh + h) * (int64_t)dim + e;
-  float* dst = out + (b * C * nh + h) * (int64_t)dim + e;
+  TO* dst = out + (b * C * nh + h) * (int64_t)dim + e;
   const float* da = dA_chunk + b * da_sb + h * da_sh;
   float4 s = initial ? *reinterpret_cast<const float4*>(initial + (b * nh + h) * (int64_t)dim + e)
                      : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -417,7 +437,7 @@ __global__ __launch_bounds__(256) void ssd_state_passing_kernel(
     for (int u = 0; u < U; ++u) {
       const int c = c0 + u;
       if (c < C) {
-        stream_store4(dst + c * chunk_stride, s);
+        state_store4(dst + c * chunk_stride, s);
         s.x = fmaf(a[u], s.x, nv[u].x);
         s.y = fmaf(a[u], s.y, nv[u].y);
         s.z = fmaf(a[u], s.z, nv[u].z);
@@ -446,10 +466,11 @@ __device__ __forceinline__ float half_wave_sum(float v) {
 // The finish kernel sums the wave partials: ddA[b,h,c] = exp(dA_chunk[c]) * sum, and 0 for
 // c = 0 when there is no initial state.
 // ------------------------------------------------------------------------------------
+template <typename TS, typename TD, typename TG>
 __global__ __launch_bounds__(256) void ssd_state_passing_bwd_kernel(
-    const float* __restrict__ states, const float* __restrict__ dA_chunk, int64_t da_sb, int64_t da_sh,
-    int64_t da_sc, const float* __restrict__ dout, const float* __restrict__ dfinal,
-    float* __restrict__ dstates, float* __restrict__ part, float* __restrict__ dinit, int nh, int C, int dim,
+    const TS* __restrict__ states, const float* __restrict__ dA_chunk, int64_t da_sb, int64_t da_sh,
+    int64_t da_sc, const TD* __restrict__ dout, const float* __restrict__ dfinal,
+    TG* __restrict__ dstates, float* __restrict__ part, float* __restrict__ dinit, int nh, int C, int dim,
     int tiles, SeqIdx seq, int L, int Q) {
   const int tile = blockIdx.x % tiles;
   const int h = (blockIdx.x / tiles) % nh;
@@ -471,8 +492,8 @@ __global__ __launch_bounds__(256) void ssd_state_passing_bwd_kernel(
     for (int u = 0; u < U; ++u) {
       const int c = c1 - u;
       const bool in = c >= 0 && ok;
-      sv[u] = in ? stream_load4(states + base + c * chunk_stride) : zero4;
-      dv[u] = in ? stream_load4(dout + base + c * chunk_stride) : zero4;
+      sv[u] = in ? state_load4<true>(states + base + c * chunk_stride) : zero4;
+      dv[u] = in ? state_load4<true>(dout + base + c * chunk_stride) : zero4;
       a[u] = c >= 0 ? __expf(da[(int64_t)c * da_sc]) : 0.f;
       if (c >= 0 && !chunk_keeps_state(seq, b, c, Q, L)) a[u] = 0.f;
     }
@@ -480,7 +501,7 @@ __global__ __launch_bounds__(256) void ssd_state_passing_bwd_kernel(
     for (int u = 0; u < U; ++u) {
       const int c = c1 - u;
       if (c >= 0) {  // uniform across the workgroup
-        if (ok) stream_store4(dstates + base + c * chunk_stride, G);
+        if (ok) state_store4(dstates + base + c * chunk_stride, G);
         const float dot = ema::wave_sum(sv[u].x * G.x + sv[u].y * G.y + sv[u].z * G.z + sv[u].w * G.w);
         if (lane == 0) part[((b * nh + h) * C + c) * (int64_t)nw + wave_id] = dot;
         G.x = fmaf(a[u], G.x, dv[u].x);
@@ -556,9 +577,9 @@ struct GroupSmem {
   static constexpr int kBytes = P * PS * (int)sizeof(T) + (4 * 64 + 64) * (int)sizeof(float);
 };
 
-template <typename T, int P, int N, int MODE>
+template <typename T, int P, int N, int MODE, typename TS>
 __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
-    const T* __restrict__ a, Strides3 sa, const float* __restrict__ s, const float* __restrict__ dt,
+    const T* __restrict__ a, Strides3 sa, const TS* __restrict__ s, const float* __restrict__ dt,
     const float* __restrict__ dA_cs, const T* __restrict__ bc, Strides3 sbc, float* __restrict__ out,
     float* __restrict__ ddA, int nh, int heads_per_group, int ngroups, int L, int Q, int C, int mtiles,
     SeqIdx seq) {
@@ -618,7 +639,7 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
     const int64_t chunk = (b * nh + h) * C + c;
     const float* dAp = dA_cs + chunk * Q;
     const float* dtp = dt + chunk * Q;
-    const float* sg = s + (((b * C + c) * nh + h) * (int64_t)P) * N;
+    const TS* sg = s + (((b * C + c) * nh + h) * (int64_t)P) * N;
     const T* ag = a + b * sa.sb + (int64_t)c * Q * sa.sl + h * sa.sh;
     // every global load of this head goes out here, before the first wait: the state tile, the
     // wave's rows of a (its blocks share them), the row weights
@@ -627,7 +648,7 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int idx = tid + 256 * i;
-      sv[i] = *reinterpret_cast<const float4*>(sg + (int64_t)(idx / VPR) * N + (idx % VPR) * 4);
+      sv[i] = state_load4<false>(sg + (int64_t)(idx / VPR) * N + (idx % VPR) * 4);
     }
     const int m_lane = m0 + 32 * mi[0] + l32;
     Vec16<T> av[KS];
@@ -762,7 +783,7 @@ __global__ __launch_bounds__(256) void ssd_bmm_kernel(const T* __restrict__ a, S
 // LDS tile so that z, out and out_x move in 16-byte pieces.  In a packed batch the carried state
 // only reaches the rows whose id equals that of the previous chunk's last position (cb already
 // holds zeros between positions of different ids).
-// cb is float32 (b, C, g, Q, Q); prev is float32 (b, C, nh, P, N).
+// cb is float32 (b, C, g, Q, Q); prev is (b, C, nh, P, N) in float32 or in T (type TS).
 // ------------------------------------------------------------------------------------
 template <typename T, int P, int N>
 struct ScanSmem {
@@ -774,11 +795,11 @@ struct ScanSmem {
   static constexpr int kBytes = (kMax1 > kPhaseC ? kMax1 : kPhaseC) + 64 * (int)sizeof(float);
 };
 
-template <typename T, int P, int N>
+template <typename T, int P, int N, typename TS>
 __global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(
     const float* __restrict__ cb, const T* __restrict__ x, Strides3 sx, const T* __restrict__ z, Strides3 sz,
     const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Cm, Strides3 sC,
-    const float* __restrict__ prev, const float* __restrict__ D, int d_has_hdim, T* __restrict__ out,
+    const TS* __restrict__ prev, const float* __restrict__ D, int d_has_hdim, T* __restrict__ out,
     Strides3 so, T* __restrict__ out_x, int nh, int heads_per_group, int ngroups, int L, int Q, int C,
     int mtiles, SeqIdx seq) {
   using S = ScanSmem<T, P, N>;
@@ -807,7 +828,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(
   const float* dtp = dt + chunk * Q;
   const T* xg = x + b * sx.sb + (int64_t)c * Q * sx.sl + h * sx.sh;
   const T* Cg = Cm + b * sC.sb + (int64_t)c * Q * sC.sl + g * sC.sh;
-  const float* pg = prev + (((b * C + c) * nh + h) * (int64_t)P) * N;
+  const TS* pg = prev + (((b * C + c) * nh + h) * (int64_t)P) * N;
   const float* cbg = cb + (((b * C + c) * ngroups + g) * (int64_t)Q) * Q;
 
   // wave -> output blocks: rows 32*mi.., columns 32*(pi0 + 2*i)..
@@ -824,7 +845,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(
     for (int i = 0; i < P * VPR / 256; ++i) {
       const int idx = tid + 256 * i;
       const int r = idx / VPR, cv = (idx % VPR) * 4;
-      const float4 v = *reinterpret_cast<const float4*>(pg + (int64_t)r * N + cv);
+      const float4 v = state_load4<false>(pg + (int64_t)r * N + cv);
       T* d = Ps + r * S::PC + cv;
       d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
     }
@@ -954,11 +975,11 @@ struct WideSmem {
   static constexpr int kBytes = kMain + 3 * ST * (int)sizeof(float);            // + dA_k, dt_k, exp(dA_m)
 };
 
-template <typename T, int P, int N>
+template <typename T, int P, int N, typename TS>
 __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
     const float* __restrict__ cb, const T* __restrict__ x, Strides3 sx, const T* __restrict__ z, Strides3 sz,
     const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Cm, Strides3 sC,
-    const float* __restrict__ prev, const float* __restrict__ D, int d_has_hdim, T* __restrict__ out,
+    const TS* __restrict__ prev, const float* __restrict__ D, int d_has_hdim, T* __restrict__ out,
     Strides3 so, T* __restrict__ out_x, int nh, int heads_per_group, int ngroups, int L, int Q, int C,
     int stiles, SeqIdx seq) {
   using S = WideSmem<T, P, N>;
@@ -987,7 +1008,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
   const float* dtp = dt + chunk * Q;
   const T* xg = x + b * sx.sb + (int64_t)c * Q * sx.sl + h * sx.sh;
   const T* Cg = Cm + b * sC.sb + (int64_t)c * Q * sC.sl + g * sC.sh;
-  const float* pg = prev + (((b * C + c) * nh + h) * (int64_t)P) * N;
+  const TS* pg = prev + (((b * C + c) * nh + h) * (int64_t)P) * N;
   const float* cbg = cb + (((b * C + c) * ngroups + g) * (int64_t)Q) * Q;
 
   int mrow[2];
@@ -1007,7 +1028,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
     for (int i = 0; i < P * VPR / 256; ++i) {
       const int idx = tid + 256 * i;
       const int r = idx / VPR, cv = (idx % VPR) * 4;
-      const float4 v = stream_load4(pg + (int64_t)r * N + cv);
+      const float4 v = state_load4<true>(pg + (int64_t)r * N + cv);
       T* d = Pv + r * S::PC + cv;
       d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
     }
@@ -1188,11 +1209,11 @@ __device__ __forceinline__ void store_dD_partial(float* __restrict__ slot, float
 // its rows.  In a packed batch the dstates term only reaches the rows whose id equals that of the
 // chunk's last position.
 // ------------------------------------------------------------------------------------
-template <typename T, int P, int N>
+template <typename T, int P, int N, typename TS>
 __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
     const float* __restrict__ cb, const T* __restrict__ x, Strides3 sx, const T* __restrict__ dout, Strides3 sd,
     const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Bm, Strides3 sB,
-    const float* __restrict__ dstates, const float* __restrict__ D, int d_has_hdim, T* __restrict__ dx,
+    const TS* __restrict__ dstates, const float* __restrict__ D, int d_has_hdim, T* __restrict__ dx,
     Strides3 sdx, float* __restrict__ ddt, int nh, int heads_per_group, int ngroups, int L, int Q, int C,
     int mtiles, SeqIdx seq, float* __restrict__ dD_part) {
   using S = ScanSmem<T, P, N>;
@@ -1231,7 +1252,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
   const T* xg = x + b * sx.sb + (int64_t)c * Q * sx.sl + h * sx.sh;
   const T* dg = dout + b * sd.sb + (int64_t)c * Q * sd.sl + h * sd.sh;
   const T* Bg = Bm + b * sB.sb + (int64_t)c * Q * sB.sl + g * sB.sh;
-  const float* sg = dstates + (((b * C + c) * nh + h) * (int64_t)P) * N;
+  const TS* sg = dstates + (((b * C + c) * nh + h) * (int64_t)P) * N;
   const float* cbg = cb + (((b * C + c) * ngroups + g) * (int64_t)Q) * Q;
 
   const int mi = wave & 1, pi0 = wave >> 1;
@@ -1247,7 +1268,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_bwd_dx_kernel(
     for (int i = 0; i < P * VPR / 256; ++i) {
       const int idx = tid + 256 * i;
       const int r = idx / VPR, cv = (idx % VPR) * 4;
-      const float4 v = *reinterpret_cast<const float4*>(sg + (int64_t)r * N + cv);
+      const float4 v = state_load4<false>(sg + (int64_t)r * N + cv);
       T* d = Ps + r * S::PC + cv;
       d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
     }
@@ -1493,11 +1514,11 @@ __global__ __launch_bounds__(256) void ssd_ddA_causal_kernel(
 // chunk; the weight fragment of a lane (row m, consecutive k) is a column piece of cb, read as
 // one 4-byte load per k that is contiguous across the 32 lanes of a half-wave.
 // ------------------------------------------------------------------------------------
-template <typename T, int P, int N>
+template <typename T, int P, int N, typename TS>
 __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_wide_kernel(
     const float* __restrict__ cb, const T* __restrict__ x, Strides3 sx, const T* __restrict__ dout, Strides3 sd,
     const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Bm, Strides3 sB,
-    const float* __restrict__ dstates, const float* __restrict__ D, int d_has_hdim, T* __restrict__ dx,
+    const TS* __restrict__ dstates, const float* __restrict__ D, int d_has_hdim, T* __restrict__ dx,
     Strides3 sdx, float* __restrict__ ddt, int nh, int heads_per_group, int ngroups, int L, int Q, int C,
     int stiles, SeqIdx seq, float* __restrict__ dD_part) {
   using S = WideSmem<T, P, N>;
@@ -1534,7 +1555,7 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
   const float* dtp = dt + chunk * Q;
   const T* dg = dout + b * sd.sb + (int64_t)c * Q * sd.sl + h * sd.sh;
   const T* Bg = Bm + b * sB.sb + (int64_t)c * Q * sB.sl + g * sB.sh;
-  const float* sg = dstates + (((b * C + c) * nh + h) * (int64_t)P) * N;
+  const TS* sg = dstates + (((b * C + c) * nh + h) * (int64_t)P) * N;
   const float* cbg = cb + (((b * C + c) * ngroups + g) * (int64_t)Q) * Q;
 
   int mrow[2];
@@ -1554,7 +1575,7 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
     for (int i = 0; i < P * VPR / 256; ++i) {
       const int idx = tid + 256 * i;
       const int r = idx / VPR, cv = (idx % VPR) * 4;
-      const float4 v = stream_load4(sg + (int64_t)r * N + cv);
+      const float4 v = state_load4<true>(sg + (int64_t)r * N + cv);
       T* d = Pv + r * S::PC + cv;
       d[0] = (T)v.x, d[1] = (T)v.y, d[2] = (T)v.z, d[3] = (T)v.w;
     }

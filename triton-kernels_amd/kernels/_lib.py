@@ -51,16 +51,16 @@ _SIGNATURES = {
     # SSD forward stages (include/ssd_hip.h)
     "ssd_chunk_cumsum_fwd": (c_int, [_P, c_int, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, c_int, c_float, c_float, _P]),
     "ssd_chunk_state_fwd": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
-    "ssd_state_passing_fwd": (c_int, [_P, _P, _I, _I, _I, _P, _P, _P, _I, _I, _I, _I] + _IDS + [_I, _I, _P]),
+    "ssd_state_passing_fwd": (c_int, [_P, _P, _I, _I, _I, _P, _P, c_int, _P, _I, _I, _I, _I] + _IDS + [_I, _I, _P]),
     "ssd_bmm_chunk_fwd": (c_int, _SEQ + _SEQ + [c_int, _P, c_int, _I, _I, _I, _I, _I] + _IDS + [_P]),
-    "ssd_chunk_scan_fwd": (c_int, [_P] + _SEQ + _SEQ + [c_int, _P, _P] + _SEQ + [_P, _P, c_int] + _SEQ + [_P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
+    "ssd_chunk_scan_fwd": (c_int, [_P] + _SEQ + _SEQ + [c_int, _P, _P] + _SEQ + [_P, c_int, _P, c_int] + _SEQ + [_P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
     # SSD backward stages
-    "ssd_chunk_scan_bwd_dstates": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
+    "ssd_chunk_scan_bwd_dstates": (c_int, _SEQ + _SEQ + [c_int, _P, _P, c_int, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
     "ssd_state_passing_bwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
-    "ssd_state_passing_bwd": (c_int, [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I] + _IDS + [_I, _I, _P]),
-    "ssd_chunk_state_bwd_db": (c_int, _SEQ + [c_int, _P, _P, _P] + _SEQ + [_P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
-    "ssd_chunk_scan_bwd_dc": (c_int, _SEQ + [c_int, _P, _P] + _SEQ + [_P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
-    "ssd_chunk_scan_chunk_state_bwd_dx": (c_int, [_P] + _SEQ + _SEQ + [c_int, _P, _P] + _SEQ + [_P, _P, c_int] + _SEQ + [_P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P, _P]),
+    "ssd_state_passing_bwd": (c_int, [_P, c_int, _P, _I, _I, _I, _P, c_int, _P, _P, c_int, _P, _P, _P, c_size_t, _I, _I, _I, _I] + _IDS + [_I, _I, _P]),
+    "ssd_chunk_state_bwd_db": (c_int, _SEQ + [c_int, _P, _P, _P, c_int] + _SEQ + [_P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
+    "ssd_chunk_scan_bwd_dc": (c_int, _SEQ + [c_int, _P, _P, c_int] + _SEQ + [_P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
+    "ssd_chunk_scan_chunk_state_bwd_dx": (c_int, [_P] + _SEQ + _SEQ + [c_int, _P, _P] + _SEQ + [_P, c_int, _P, c_int] + _SEQ + [_P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P, _P]),
     "ssd_chunk_scan_chunk_state_bwd_dx_dD_slots": (c_int64, [c_int, _I, _I, _I]),
     "ssd_chunk_scan_bwd_ddAcs_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "ssd_chunk_scan_bwd_ddAcs": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _I, _P]),
@@ -174,6 +174,14 @@ def f32c(t: torch.Tensor) -> torch.Tensor:
     if t.dtype != torch.float32:
         t = t.float()
     return t.contiguous()
+
+
+def state_tensor(t: torch.Tensor, like: torch.Tensor = None):
+    """(dense tensor, dtype code) of a carried-state tensor: kept in bfloat16 when the kernels that
+    read it compute in bfloat16 (`like`, None for any), brought to float32 otherwise."""
+    if t.dtype == torch.bfloat16 and (like is None or like.dtype == torch.bfloat16):
+        return t.contiguous(), EMA_BF16
+    return f32c(t), EMA_F32
 
 
 def seq_ids(seq_idx, batch: int, seqlen: int, dev: torch.device):

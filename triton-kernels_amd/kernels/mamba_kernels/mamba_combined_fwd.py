@@ -16,7 +16,8 @@ from kernels.mamba_kernels.mamba_state_pass import _state_passing_fwd
 def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
                                    initial_states=None, seq_idx=None, cu_seqlens=None, dt_softplus=False,
                                    dt_limit=(0.0, float("inf"))):
-    """Returns (out, out_x, dt_out, dA_cumsum, states, final_states), and as a seventh item the state
+    """Returns (out, out_x, dt_out, dA_cumsum, states, final_states), states (the state entering
+    each chunk) in the dtype of C as in kernels/ema_combined.py:48-50, and as a seventh item the state
     at the end of each packed sequence when cu_seqlens is given (batch must be 1 then; the boundaries
     are the ones seq_idx marks), as kernels/ema_combined.py:56-62 of the reference does."""
     batch, seqlen, nheads, headdim = x.shape
@@ -32,7 +33,7 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
     init = None if initial_states is None else initial_states.reshape(batch, nheads, headdim * dstate)
     states, final_states = _state_passing_fwd(states.reshape(batch, -1, nheads, headdim * dstate),
                                               dA_cumsum[:, :, :, -1], initial_states=init, seq_idx=seq_idx,
-                                              chunk_size=chunk_size, out_dtype=torch.float32)
+                                              chunk_size=chunk_size, out_dtype=C.dtype)
     states = states.reshape(batch, -1, nheads, headdim, dstate)
     final_states = final_states.reshape(batch, nheads, headdim, dstate)
     CB = _bmm_chunk_fwd(C, B, chunk_size, seq_idx=seq_idx, output_dtype=torch.float32)

@@ -39,11 +39,12 @@ def _chunk_scan_fwd(cb, x, dt, dA_cumsum, C, states, D=None, z=None, seq_idx=Non
     out = torch.empty(batch, seqlen, nheads, headdim, device=dev, dtype=x.dtype)
     out_x = torch.empty_like(out) if z is not None else None
     Df = None if D is None else _lib.f32c(D)
+    states, st_code = _lib.state_tensor(states, like=x)
     with torch.cuda.device(dev):
         _lib.check(
             _lib.lib().ssd_chunk_scan_fwd(
                 _lib.f32c(cb).data_ptr(), *xs, *zs, _lib.dtype_code(x), _lib.f32c(dt).data_ptr(),
-                _lib.f32c(dA_cumsum).data_ptr(), *cs, _lib.f32c(states).data_ptr(),
+                _lib.f32c(dA_cumsum).data_ptr(), *cs, states.data_ptr(), st_code,
                 None if Df is None else Df.data_ptr(), int(D is not None and D.dim() == 2), out.data_ptr(),
                 out.stride(0), out.stride(1), out.stride(2), None if out_x is None else out_x.data_ptr(), batch,
                 seqlen, nheads, ngroups, headdim, dstate, chunk_size, *ids, _lib.stream_ptr(dev)),

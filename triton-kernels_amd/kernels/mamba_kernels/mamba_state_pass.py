@@ -30,13 +30,15 @@ def _state_passing_fwd(states, dA_chunk_cumsum, initial_states=None, seq_idx=Non
     st = _lib.f32c(states)
     da = dA_chunk_cumsum if dA_chunk_cumsum.dtype == torch.float32 else dA_chunk_cumsum.float()
     init = None if initial_states is None else _lib.f32c(initial_states)
-    out = torch.empty(batch, nchunks, nheads, dim, device=dev, dtype=torch.float32)
+    # float32 and bfloat16 copies of the carried states are written by the kernel itself
+    native = out_dtype if out_dtype in (torch.float32, torch.bfloat16) else torch.float32
+    out = torch.empty(batch, nchunks, nheads, dim, device=dev, dtype=native)
     final_states = torch.empty(batch, nheads, dim, device=dev, dtype=torch.float32)
     with torch.cuda.device(dev):
         _lib.check(
             _lib.lib().ssd_state_passing_fwd(st.data_ptr(), da.data_ptr(), da.stride(0), da.stride(1), da.stride(2),
                                              None if init is None else init.data_ptr(), out.data_ptr(),
-                                             final_states.data_ptr(), batch, nchunks, nheads, dim, *ids, seqlen,
-                                             chunk_size or 0, _lib.stream_ptr(dev)),
+                                             _lib.dtype_code(out), final_states.data_ptr(), batch, nchunks, nheads,
+                                             dim, *ids, seqlen, chunk_size or 0, _lib.stream_ptr(dev)),
             "ssd_state_passing_fwd")
-    return (out if out_dtype == torch.float32 else out.to(out_dtype)), final_states
+    return (out if out_dtype == native else out.to(out_dtype)), final_states

@@ -41,6 +41,7 @@ def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum, B, CB, dout, dstates, D=Non
         assert dx.shape == x.shape and dx.dtype == x.dtype and dx.stride(-1) == 1
     ddt = torch.empty(batch, nheads, nchunks, chunk_size, device=dev, dtype=torch.float32)
     Df = None if D is None else _lib.f32c(D)
+    dstates, ds_code = _lib.state_tensor(dstates, like=x)
     dD_part = None
     if D is not None:  # per-wave partial sums of dout * x, summed below like the reference's per-block ones
         slots = _lib.lib().ssd_chunk_scan_chunk_state_bwd_dx_dD_slots(_lib.dtype_code(x), headdim, dstate, chunk_size)
@@ -50,7 +51,7 @@ def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum, B, CB, dout, dstates, D=Non
         _lib.check(
             _lib.lib().ssd_chunk_scan_chunk_state_bwd_dx(
                 _lib.f32c(CB).data_ptr(), *xs, *ds, _lib.dtype_code(x), _lib.f32c(dt).data_ptr(),
-                _lib.f32c(dA_cumsum).data_ptr(), *bs, _lib.f32c(dstates).data_ptr(),
+                _lib.f32c(dA_cumsum).data_ptr(), *bs, dstates.data_ptr(), ds_code,
                 None if Df is None else Df.data_ptr(), int(D is not None and D.dim() == 2), dx.data_ptr(),
                 dx.stride(0), dx.stride(1), dx.stride(2), ddt.data_ptr(), batch, seqlen, nheads, ngroups, headdim,
                 dstate, chunk_size, *ids, None if dD_part is None else dD_part.data_ptr(), _lib.stream_ptr(dev)),

@@ -27,11 +27,13 @@ def _chunk_scan_bwd_dstates(C, dA_cumsum, dout, seq_idx=None, dtype=None):
     if C.dtype != dout.dtype:
         C = C.to(dout.dtype)
     C, cs = _lib.strided4(C)
-    out = torch.empty(batch, nchunks, nheads, headdim, dstate, device=dev, dtype=torch.float32)
+    # the kernel stores float32, or bfloat16 next to bfloat16 inputs; any other type is cast afterwards
+    native = dtype if dtype == torch.float32 or (dtype == torch.bfloat16 and dout.dtype == dtype) else torch.float32
+    out = torch.empty(batch, nchunks, nheads, headdim, dstate, device=dev, dtype=native)
     with torch.cuda.device(dev):
         _lib.check(
             _lib.lib().ssd_chunk_scan_bwd_dstates(*cs, *ds, _lib.dtype_code(dout), _lib.f32c(dA_cumsum).data_ptr(),
-                                                  out.data_ptr(), batch, seqlen, nheads, ngroups, headdim, dstate,
+                                                  out.data_ptr(), _lib.dtype_code(out), batch, seqlen, nheads, ngroups, headdim, dstate,
                                                   chunk_size, *ids, _lib.stream_ptr(dev)),
             "ssd_chunk_scan_bwd_dstates")
-    return out if dtype == torch.float32 else out.to(dtype)
+    return out if dtype == native else out.to(dtype)

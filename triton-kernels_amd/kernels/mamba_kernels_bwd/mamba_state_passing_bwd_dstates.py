@@ -33,25 +33,28 @@ def _state_passing_bwd(states, dA_chunk_cumsum, dout, dfinal_states=None, seq_id
         seqlen = seq_idx.shape[-1]
         assert nchunks == (seqlen + chunk_size - 1) // chunk_size
     seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)
-    st, do = _lib.f32c(states), _lib.f32c(dout)
+    (st, st_code), (do, do_code) = _lib.state_tensor(states), _lib.state_tensor(dout)
+    out_dtype = dstates_dtype if dstates_dtype is not None else dout.dtype
+    native = out_dtype if out_dtype in (torch.float32, torch.bfloat16) else torch.float32
     da = dA_chunk_cumsum if dA_chunk_cumsum.dtype == torch.float32 else dA_chunk_cumsum.float()
     dfin = None if dfinal_states is None else _lib.f32c(dfinal_states)
-    dstates = torch.empty(batch, nchunks, nheads, dim, device=dev, dtype=torch.float32)
+    dstates = torch.empty(batch, nchunks, nheads, dim, device=dev, dtype=native)
     ddA = torch.empty(batch, nheads, nchunks, device=dev, dtype=torch.float32)
     dinit = torch.empty(batch, nheads, dim, device=dev, dtype=torch.float32) if has_initial_states else None
     nbytes = lib.ssd_state_passing_bwd_workspace_bytes(batch, nchunks, nheads, dim)
     ws = torch.empty(max(nbytes, 16), device=dev, dtype=torch.uint8)
     with torch.cuda.device(dev):
         _lib.check(
-            lib.ssd_state_passing_bwd(st.data_ptr(), da.data_ptr(), da.stride(0), da.stride(1), da.stride(2),
-                                      do.data_ptr(), None if dfin is None else dfin.data_ptr(), dstates.data_ptr(),
+            lib.ssd_state_passing_bwd(st.data_ptr(), st_code, da.data_ptr(), da.stride(0), da.stride(1), da.stride(2),
+                                      do.data_ptr(), do_code, None if dfin is None else dfin.data_ptr(),
+                                      dstates.data_ptr(), _lib.dtype_code(dstates),
                                       ddA.data_ptr(), None if dinit is None else dinit.data_ptr(), ws.data_ptr(),
                                       nbytes, batch, nchunks, nheads, dim, *ids, seqlen, chunk_size or 0,
                                       _lib.stream_ptr(dev)),
             "ssd_state_passing_bwd")
-    out_dtype = dstates_dtype if dstates_dtype is not None else dout.dtype
-    if out_dtype != torch.float32:
+    if out_dtype != native:
         dstates = dstates.to(out_dtype)
+    if out_dtype != torch.float32:
         dinit = None if dinit is None else dinit.to(out_dtype)
     ddA = ddA.to(dA_chunk_cumsum.dtype)
     if states_dtype is None:
