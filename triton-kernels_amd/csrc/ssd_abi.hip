@@ -287,17 +287,23 @@ int ssd_chunk_cumsum_fwd(const void* dt, int dt_dtype, int64_t dt_sb, int64_t dt
   SSD_TRY(check_dims(batch, seqlen, nheads, 1, 0, 0, chunk, &d));
   SSD_TRY(check_dtype(dt_dtype));
   if (!dt || !A || !dA_cumsum || !dt_out) return SSD_ERR_NULL;
-  const int64_t total = batch * nheads * d.C;
   const Strides3 sd{dt_sb, dt_sl, dt_sh};
-  const unsigned grid = (unsigned)((total + 3) / 4);
+  // heads per workgroup: a power of two up to 32 whose Q x HT tile stays within 64 KB of LDS
+  int HT = 32;
+  while (HT > 1 && (HT / 2 >= nheads || (int64_t)HT * (chunk + 1) * 4 > 64 * 1024)) HT /= 2;
+  const int hgroups = (int)((nheads + HT - 1) / HT);
+  const int64_t blocks = batch * d.C * hgroups;
+  if (blocks > 0x7fffffff) return SSD_ERR_SHAPE;
+  const unsigned grid = (unsigned)blocks;
+  const int smem = HT * (int)(chunk + 1) * 4;
   if (dt_dtype == SSD_BF16)
-    hipLaunchKernelGGL(ssd_cumsum_kernel<bf16_t>, dim3(grid), dim3(256), 0, as_stream(stream), (const bf16_t*)dt,
-                       sd, A, dt_bias, dA_cumsum, dt_out, (int)nheads, (int)seqlen, (int)chunk, (int)d.C,
-                       dt_softplus, dt_min, dt_max, total);
+    hipLaunchKernelGGL(ssd_cumsum_kernel<bf16_t>, dim3(grid), dim3(256), smem, as_stream(stream), (const bf16_t*)dt,
+                       sd, A, dt_bias, dA_cumsum, dt_out, (int)nheads, (int)seqlen, (int)chunk, (int)d.C, dt_softplus,
+                       dt_min, dt_max, HT, hgroups);
   else
-    hipLaunchKernelGGL(ssd_cumsum_kernel<float>, dim3(grid), dim3(256), 0, as_stream(stream), (const float*)dt, sd,
+    hipLaunchKernelGGL(ssd_cumsum_kernel<float>, dim3(grid), dim3(256), smem, as_stream(stream), (const float*)dt, sd,
                        A, dt_bias, dA_cumsum, dt_out, (int)nheads, (int)seqlen, (int)chunk, (int)d.C, dt_softplus,
-                       dt_min, dt_max, total);
+                       dt_min, dt_max, HT, hgroups);
   return launched();
 }
 

@@ -224,9 +224,12 @@ struct RowPieces {
 };
 
 // ------------------------------------------------------------------------------------
-// chunk_cumsum.  One wave per (b, c, h).  dt is processed (bias, softplus with the identity
-// above 20, clamp), positions past the sequence give 0; dA = dt * A[h] is scanned across the
-// chunk with DPP.  Outputs are (b, nh, C, Q) float32.
+// chunk_cumsum.  One workgroup per (b, c, group of HT heads), HT a power of two up to 32.  dt is
+// (batch, seqlen, nheads) with the heads innermost, so the workgroup reads its Q x HT tile with the
+// heads across adjacent lanes, processes it (bias, softplus with the identity above 20, clamp; 0
+// past the sequence) and transposes it through LDS; then one wave per head scans dA = dt * A[h]
+// across the chunk with DPP, each lane owning ceil(Q/64) consecutive positions.  Outputs are
+// (b, nh, C, Q) float32.  LDS: HT * (Q + 1) floats.
 // ------------------------------------------------------------------------------------
 template <typename TD>
 __global__ __launch_bounds__(256) void ssd_cumsum_kernel(const TD* __restrict__ dt, Strides3 sd,
@@ -234,38 +237,58 @@ __global__ __launch_bounds__(256) void ssd_cumsum_kernel(const TD* __restrict__ 
                                                          const float* __restrict__ dt_bias,
                                                          float* __restrict__ dA_cs, float* __restrict__ dt_out,
                                                          int nh, int L, int Q, int C, int softplus,
-                                                         float dt_min, float dt_max, int64_t total) {
-  const int lane = threadIdx.x & 63;
-  const int64_t id = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // ((b * nh) + h) * C + c
-  if (id >= total) return;
-  const int c = (int)(id % C);
-  const int64_t bh = id / C;
-  const int h = (int)(bh % nh);
-  const int64_t b = bh / nh;
+                                                         float dt_min, float dt_max, int HT, int hgroups) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  float* tile = reinterpret_cast<float*>(smem);  // [HT][Q + 1]
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int hg = blockIdx.x % hgroups;
+  const int c = (blockIdx.x / hgroups) % C;
+  const int64_t b = blockIdx.x / (hgroups * C);
+  const int h0 = hg * HT;
+  const int limit = min(Q, L - c * Q);
+  const int pitch = Q + 1;
+  {
+    const int j = tid % HT, qstep = 256 / HT;
+    const int h = min(h0 + j, nh - 1);
+    const TD* src = dt + b * sd.sb + (int64_t)c * Q * sd.sl + (int64_t)h * sd.sh;
+    const float bias = dt_bias ? dt_bias[h] : 0.f;
+    constexpr int U = 8;  // loads in flight per thread
+    for (int qb = tid / HT; qb < Q; qb += U * qstep) {
+      float v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = (float)src[(int64_t)min(qb + u * qstep, limit - 1) * sd.sl];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int q = qb + u * qstep;
+        float t = v[u] + bias;
+        if (softplus && t <= 20.f) t = log1pf(__expf(t));
+        t = fminf(fmaxf(t, dt_min), dt_max);
+        if (q < Q) tile[j * pitch + q] = q < limit ? t : 0.f;
+      }
+    }
+  }
+  __syncthreads();
   const int per = (Q + 63) >> 6;
   const int q0 = lane * per;
-  const int limit = min(Q, L - c * Q);
-  const TD* src = dt + b * sd.sb + h * sd.sh + (int64_t)c * Q * sd.sl;
-  const float a = A[h];
-  const float bias = dt_bias ? dt_bias[h] : 0.f;
-  auto value = [&](int q) {
-    if (q >= limit) return 0.f;
-    float v = (float)src[(int64_t)q * sd.sl] + bias;
-    if (softplus && v <= 20.f) v = log1pf(__expf(v));
-    return fminf(fmaxf(v, dt_min), dt_max);
-  };
-  float local = 0.f;
-  for (int i = 0; i < per; ++i) local += value(q0 + i) * a;
-  float run = wave_inclusive_scan(local) - local;
-  float* o_cs = dA_cs + id * Q;
-  float* o_dt = dt_out + id * Q;
-  for (int i = 0; i < per; ++i) {
-    const int q = q0 + i;
-    if (q < Q) {
-      const float v = value(q);
-      run += v * a;
-      o_dt[q] = v;
-      o_cs[q] = run;
+  for (int jj = wave; jj < HT && h0 + jj < nh; jj += 4) {
+    const int h = h0 + jj;
+    const float a = A[h];
+    const float* row = tile + jj * pitch;
+    float local = 0.f;
+    for (int i = 0; i < per; ++i)
+      if (q0 + i < Q) local += row[q0 + i] * a;
+    float run = wave_inclusive_scan(local) - local;
+    const int64_t id = (b * nh + h) * C + c;
+    float* o_cs = dA_cs + id * Q;
+    float* o_dt = dt_out + id * Q;
+    for (int i = 0; i < per; ++i) {
+      const int q = q0 + i;
+      if (q < Q) {
+        const float v = row[q];
+        run += v * a;
+        o_dt[q] = v;
+        o_cs[q] = run;
+      }
     }
   }
 }
