@@ -30,9 +30,9 @@ for p in (ROOT, os.path.join(ROOT, "triton-kernels_amd")):
 TRAFFIC_BYTES = {"fwd_single_pass": 589083033, "bwd_single_pass": 841025145}
 # the same for the SSD stage kernels at configuration 5 (finishing kernels added to their stage)
 SSD_TRAFFIC_BYTES = {
-    "chunk_cumsum": 25728185, "chunk_state": 571561815, "state_passing": 553727051, "bmm_chunk": 100777471,
-    "chunk_scan": 878544586, "bwd_dstates": 562102058, "bwd_state_passing": 827459644, "bwd_db": 630374066,
-    "bwd_dc": 604094138, "bwd_dx": 1156650141, "bwd_ddAcs": 599910406,
+    "chunk_cumsum": 25311987, "chunk_state": 571562572, "state_passing": 419497855, "bmm_chunk": 100778356,
+    "chunk_scan": 742659408, "bwd_dstates": 448841641, "bwd_state_passing": 423804876, "bwd_db": 496062416,
+    "bwd_dc": 469832558, "bwd_dx": 1020231743, "bwd_ddAcs": 599940259,
 }
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published

@@ -288,8 +288,9 @@ int ssd_chunk_cumsum_fwd(const void* dt, int dt_dtype, int64_t dt_sb, int64_t dt
   SSD_TRY(check_dtype(dt_dtype));
   if (!dt || !A || !dA_cumsum || !dt_out) return SSD_ERR_NULL;
   const Strides3 sd{dt_sb, dt_sl, dt_sh};
-  // heads per workgroup: a power of two up to 32 whose Q x HT tile stays within 64 KB of LDS
-  int HT = 32;
+  // heads per workgroup: a power of two up to 8 (32-byte pieces of dt rows; more heads per workgroup
+  // leave too few workgroups to hide their latency) whose Q x HT tile stays within 64 KB of LDS
+  int HT = 8;
   while (HT > 1 && (HT / 2 >= nheads || (int64_t)HT * (chunk + 1) * 4 > 64 * 1024)) HT /= 2;
   const int hgroups = (int)((nheads + HT - 1) / HT);
   const int64_t blocks = batch * d.C * hgroups;

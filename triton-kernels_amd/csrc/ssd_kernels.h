@@ -224,7 +224,7 @@ struct RowPieces {
 };
 
 // ------------------------------------------------------------------------------------
-// chunk_cumsum.  One workgroup per (b, c, group of HT heads), HT a power of two up to 32.  dt is
+// chunk_cumsum.  One workgroup per (b, c, group of HT heads), HT a power of two up to 8.  dt is
 // (batch, seqlen, nheads) with the heads innermost, so the workgroup reads its Q x HT tile with the
 // heads across adjacent lanes, processes it (bias, softplus with the identity above 20, clamp; 0
 // past the sequence) and transposes it through LDS; then one wave per head scans dA = dt * A[h]
@@ -241,9 +241,10 @@ __global__ __launch_bounds__(256) void ssd_cumsum_kernel(const TD* __restrict__ 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   float* tile = reinterpret_cast<float*>(smem);  // [HT][Q + 1]
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int hg = blockIdx.x % hgroups;
-  const int c = (blockIdx.x / hgroups) % C;
-  const int64_t b = blockIdx.x / (hgroups * C);
+  const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);  // a chunk's head groups share lines of dt
+  const int hg = bid % hgroups;
+  const int c = (bid / hgroups) % C;
+  const int64_t b = bid / (hgroups * C);
   const int h0 = hg * HT;
   const int limit = min(Q, L - c * Q);
   const int pitch = Q + 1;
@@ -281,6 +282,17 @@ __global__ __launch_bounds__(256) void ssd_cumsum_kernel(const TD* __restrict__ 
     const int64_t id = (b * nh + h) * C + c;
     float* o_cs = dA_cs + id * Q;
     float* o_dt = dt_out + id * Q;
+    if (per == 4 && Q == 256) {  // the lane's four positions leave as one 16-byte store per output
+      float4 v4, c4;
+      v4.x = row[q0], v4.y = row[q0 + 1], v4.z = row[q0 + 2], v4.w = row[q0 + 3];
+      c4.x = run += v4.x * a;
+      c4.y = run += v4.y * a;
+      c4.z = run += v4.z * a;
+      c4.w = run += v4.w * a;
+      *reinterpret_cast<float4*>(o_dt + q0) = v4;
+      *reinterpret_cast<float4*>(o_cs + q0) = c4;
+      continue;
+    }
     for (int i = 0; i < per; ++i) {
       const int q = q0 + i;
       if (q < Q) {
