@@ -221,16 +221,16 @@ int ssd_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t 
  * back): cu_seqlens (nseq + 1, int32, device memory) holds the first position of each sequence and
  * the total length.  B (seqlen, ngroups, dstate) and x (seqlen, nheads, hdim) with element strides
  * for position and group / head (innermost contiguous); dt, dA_cumsum (nheads, nchunks, chunk)
- * float32 contiguous; chunk_states (nchunks, nheads, hdim, dstate) float32 contiguous, the state
- * entering each chunk (what ssd_state_passing_fwd writes).  states (nseq, nheads, hdim, dstate)
+ * float32 contiguous; chunk_states (nchunks, nheads, hdim, dstate) contiguous, float32 or `dtype`
+ * (states_dtype), the state entering each chunk (what ssd_state_passing_fwd writes).  states (nseq, nheads, hdim, dstate)
  * float32 is written in full; a sequence of length 0, or bounds outside [0, seqlen], give zeros.
  * Any hdim and dstate up to 4096.  For sequence s ending (exclusive) at e in chunk c = (e-1)/chunk:
  *   states[s] = sum_{k in s, k in chunk c} exp(min(dA[e-1] - dA[k], 0)) dt[k] x[k] (outer) B[k]
  *             + (s began before chunk c) * exp(dA[e-1]) * chunk_states[c].
  * Replaces chunk_state_varlen, kernels/ema_chunk_state.py:578-604 (kernel at :500-575). */
 int ssd_chunk_state_varlen(const void* B, int64_t b_sl, int64_t b_sg, const void* x, int64_t x_sl, int64_t x_sh,
-                           int dtype, const float* dt, const float* dA_cumsum, const float* chunk_states,
-                           const int32_t* cu_seqlens, float* states, int64_t nseq, int64_t seqlen, int64_t nheads,
+                           int dtype, const float* dt, const float* dA_cumsum, const void* chunk_states,
+                           int states_dtype, const int32_t* cu_seqlens, float* states, int64_t nseq, int64_t seqlen, int64_t nheads,
                            int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk, void* stream);
 
 #ifdef __cplusplus

@@ -643,25 +643,33 @@ int ssd_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t 
 }
 
 int ssd_chunk_state_varlen(const void* B, int64_t b_sl, int64_t b_sg, const void* x, int64_t x_sl, int64_t x_sh,
-                           int dtype, const float* dt, const float* dA_cumsum, const float* chunk_states,
-                           const int32_t* cu_seqlens, float* states, int64_t nseq, int64_t seqlen, int64_t nheads,
+                           int dtype, const float* dt, const float* dA_cumsum, const void* chunk_states,
+                           int states_dtype, const int32_t* cu_seqlens, float* states, int64_t nseq, int64_t seqlen, int64_t nheads,
                            int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk, void* stream) {
   Dims d;
   SSD_TRY(check_dims(1, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
   SSD_TRY(check_dtype(dtype));
   if (nseq <= 0 || nseq > 65535 || hdim <= 0 || dstate <= 0 || hdim > 4096 || dstate > 4096) return SSD_ERR_SHAPE;
+  if (states_dtype != SSD_F32 && states_dtype != dtype) return SSD_ERR_DTYPE;
   if (!B || !x || !dt || !dA_cumsum || !chunk_states || !cu_seqlens || !states) return SSD_ERR_NULL;
   const int64_t tiles = ((hdim + 63) / 64) * ((dstate + 63) / 64);
   const dim3 grid((unsigned)tiles, (unsigned)nseq, (unsigned)nheads);
   const int hpg = (int)(nheads / ngroups);
-  if (dtype == SSD_BF16)
-    hipLaunchKernelGGL(ssd_chunk_state_varlen_kernel<bf16_t>, grid, dim3(256), 0, as_stream(stream), (const bf16_t*)x,
-                       x_sl, x_sh, (const bf16_t*)B, b_sl, b_sg, dt, dA_cumsum, chunk_states, cu_seqlens, states,
-                       (int)seqlen, (int)nheads, hpg, (int)hdim, (int)dstate, (int)chunk, (int)d.C);
+  if (dtype == SSD_BF16 && states_dtype == SSD_BF16)
+    hipLaunchKernelGGL((ssd_chunk_state_varlen_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, as_stream(stream),
+                       (const bf16_t*)x, x_sl, x_sh, (const bf16_t*)B, b_sl, b_sg, dt, dA_cumsum,
+                       (const bf16_t*)chunk_states, cu_seqlens, states, (int)seqlen, (int)nheads, hpg, (int)hdim,
+                       (int)dstate, (int)chunk, (int)d.C);
+  else if (dtype == SSD_BF16)
+    hipLaunchKernelGGL((ssd_chunk_state_varlen_kernel<bf16_t, float>), grid, dim3(256), 0, as_stream(stream),
+                       (const bf16_t*)x, x_sl, x_sh, (const bf16_t*)B, b_sl, b_sg, dt, dA_cumsum,
+                       (const float*)chunk_states, cu_seqlens, states, (int)seqlen, (int)nheads, hpg, (int)hdim,
+                       (int)dstate, (int)chunk, (int)d.C);
   else
-    hipLaunchKernelGGL(ssd_chunk_state_varlen_kernel<float>, grid, dim3(256), 0, as_stream(stream), (const float*)x,
-                       x_sl, x_sh, (const float*)B, b_sl, b_sg, dt, dA_cumsum, chunk_states, cu_seqlens, states,
-                       (int)seqlen, (int)nheads, hpg, (int)hdim, (int)dstate, (int)chunk, (int)d.C);
+    hipLaunchKernelGGL((ssd_chunk_state_varlen_kernel<float, float>), grid, dim3(256), 0, as_stream(stream),
+                       (const float*)x, x_sl, x_sh, (const float*)B, b_sl, b_sg, dt, dA_cumsum,
+                       (const float*)chunk_states, cu_seqlens, states, (int)seqlen, (int)nheads, hpg, (int)hdim,
+                       (int)dstate, (int)chunk, (int)d.C);
   return launched();
 }
 

@@ -1768,10 +1768,10 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
 // Grid (P tiles * N tiles, sequences, heads).  The weighted B is rounded to T before the product,
 // as the reference does; an empty or out-of-range sequence gives zeros.
 // ------------------------------------------------------------------------------------
-template <typename T>
+template <typename T, typename TS>
 __global__ __launch_bounds__(256) void ssd_chunk_state_varlen_kernel(
     const T* __restrict__ x, int64_t x_sl, int64_t x_sh, const T* __restrict__ Bm, int64_t b_sl, int64_t b_sg,
-    const float* __restrict__ dt, const float* __restrict__ dA_cs, const float* __restrict__ chunk_states,
+    const float* __restrict__ dt, const float* __restrict__ dA_cs, const TS* __restrict__ chunk_states,
     const int32_t* __restrict__ cu_seqlens, float* __restrict__ out, int L, int nh, int hpg, int P, int N, int Q,
     int C) {
   constexpr int TP = 64, TN = 64, KB = 32;
@@ -1835,7 +1835,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_state_varlen_kernel(
       const int p = p0 + tp + i, n = n0 + tn + j;
       if (p < P && n < N) {
         float v = acc[i][j];
-        if (carried) v = fmaf(chunk_states[(((int64_t)c * nh + h) * P + p) * N + n], keep, v);
+        if (carried) v = fmaf((float)chunk_states[(((int64_t)c * nh + h) * P + p) * N + n], keep, v);
         out[(((int64_t)s * nh + h) * P + p) * N + n] = v;
       }
     }

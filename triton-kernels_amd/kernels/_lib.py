@@ -64,7 +64,7 @@ _SIGNATURES = {
     "ssd_chunk_scan_chunk_state_bwd_dx_dD_slots": (c_int64, [c_int, _I, _I, _I]),
     "ssd_chunk_scan_bwd_ddAcs_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "ssd_chunk_scan_bwd_ddAcs": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _I, _P]),
-    "ssd_chunk_state_varlen": (c_int, [_P, _I, _I, _P, _I, _I, c_int, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "ssd_chunk_state_varlen": (c_int, [_P, _I, _I, _P, _I, _I, c_int, _P, _P, _P, c_int, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
 }
 
 _lib = None

@@ -66,12 +66,13 @@ def chunk_state_varlen(B, x, dt, dA_cumsum, cu_seqlens, chunk_states):
     if B.stride(-1) != 1:
         B = B.contiguous()
     cu = cu_seqlens.to(torch.int32).contiguous()
+    st, st_code = _lib.state_tensor(chunk_states, like=x)
     states = torch.empty(batch, nheads, headdim, dstate, device=dev, dtype=torch.float32)
     with torch.cuda.device(dev):
         _lib.check(
             _lib.lib().ssd_chunk_state_varlen(B.data_ptr(), B.stride(0), B.stride(1), x.data_ptr(), x.stride(0),
                                               x.stride(1), _lib.dtype_code(x), _lib.f32c(dt).data_ptr(),
-                                              _lib.f32c(dA_cumsum).data_ptr(), _lib.f32c(chunk_states).data_ptr(),
+                                              _lib.f32c(dA_cumsum).data_ptr(), st.data_ptr(), st_code,
                                               cu.data_ptr(), states.data_ptr(), batch, total_seqlen, nheads, ngroups,
                                               headdim, dstate, chunk_size, _lib.stream_ptr(dev)),
             "ssd_chunk_state_varlen")
