@@ -105,13 +105,19 @@ size_t ema_fwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, in
  * sequence and prev128 must be NULL.  ev_start / ev_stop (hipEvent_t, may be NULL) are
  * recorded on the stream right before and after the kernel(s) that read x, so that a
  * caller can time them apart from the small set-up kernels.
+ * bwd_workspace (may be NULL; chunk a multiple of 128): the workspace of the ema_seq_bwd call
+ * (log-decay form, same shape) that will follow this forward pass, at least
+ * ema_seq_bwd_workspace_bytes(...) bytes.  The forward's set-up launch then also prepares it
+ * (status words of the reverse scan, the cumsum of A), and that ema_seq_bwd call, told so by its
+ * workspace_prepared argument, needs no set-up launch of its own.  The caller keeps the buffer
+ * untouched in between; a prepared workspace serves one backward call.
  * Replaces _ema_matmul_scan_combined_fwd, kernels/ema_kernels/ema_combined_fwd.py:12-45. */
 int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void* x,
             int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb,
             int64_t y_sl, int64_t y_sh, float* cs, float* prev, float* final_state,
-            float* prev128, void* workspace, size_t workspace_bytes, int64_t batch,
-            int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk, void* stream,
-            void* ev_start, void* ev_stop);
+            float* prev128, void* workspace, size_t workspace_bytes, void* bwd_workspace,
+            size_t bwd_workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
+            int64_t chunk, void* stream, void* ev_start, void* ev_stop);
 
 /* --------------------------------------------------------------- backward stages ---- */
 
@@ -244,13 +250,14 @@ size_t ema_seq_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen
  * (kernels/ema_kernels/ema_state_pass.py:129-130).  final_state (N,T), may be NULL: the state
  * after the last position.  prev128 (N, ceil(seqlen/128), T) float32, required: the state
  * entering each 128-row chunk, which ema_seq_bwd takes.  Chunking is internal; there is no
- * chunk argument.  ev_start / ev_stop as for ema_fwd. */
+ * chunk argument.  ev_start / ev_stop and bwd_workspace (the workspace of the ema_seq_bwd call of
+ * the same form and shape that will follow, prepared here; may be NULL) as for ema_fwd. */
 int ema_seq_fwd(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t c_sh,
                 const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y,
                 int64_t y_sb, int64_t y_sl, int64_t y_sh, const float* init, float* final_state,
-                float* prev128, void* workspace, size_t workspace_bytes, int64_t batch,
-                int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
-                void* ev_stop);
+                float* prev128, void* workspace, size_t workspace_bytes, void* bwd_workspace,
+                size_t bwd_workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
+                void* stream, void* ev_start, void* ev_stop);
 
 /* Backward of ema_seq_fwd in one pass over x and dy.  With r the reverse scan of dy,
  * r[t] = dy[t] + a[t+1] * r[t+1], started from dfinal (N,T) float32 (may be NULL = zero), the
@@ -262,14 +269,17 @@ int ema_seq_fwd(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t
  * (the reference leaves dP = -dA * exp(A) commented out, kernels/tests/ema_bwd/_ema_full_bwd.py:128-130,
  * and rearranges dA from (b,c,q) to (b,l) in torch, :71).  dcoef is float32 in the layout of
  * coef, given by its own strides; dinit (N,T) float32, may be NULL, receives a[0] * r[0], the
- * gradient of init.  prev128 is the forward's output of that name. */
+ * gradient of init.  prev128 is the forward's output of that name.  workspace_prepared: non-zero
+ * if the forward pass was given this workspace as its bwd_workspace and nothing has written to it
+ * since; the call then skips its set-up launch.  Only without dfinal (EMA_ERR_UNSUPPORTED
+ * otherwise), and once per forward pass. */
 int ema_seq_bwd(int form, const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh,
                 const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, const float* coef,
                 int64_t c_sb, int64_t c_sl, int64_t c_sh, const float* prev128,
                 const float* dfinal, int dtype, void* dx, int64_t dx_sb, int64_t dx_sl,
                 int64_t dx_sh, float* dcoef, int64_t dc_sb, int64_t dc_sl, int64_t dc_sh,
-                float* dinit, void* workspace, size_t workspace_bytes, int64_t batch,
-                int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
+                float* dinit, void* workspace, size_t workspace_bytes, int workspace_prepared,
+                int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
                 void* ev_stop);
 
 #ifdef __cplusplus

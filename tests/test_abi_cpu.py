@@ -71,8 +71,22 @@ def test_validation_happens_before_any_launch():
     # workspace too small
     assert (
         handle.ema_fwd(fake, 8, 1, 0, fake, 64, 8, 0, _lib.EMA_F32, fake, 64, 8, 0, fake, fake, fake,
-                       None, fake, 16, 1, 1, 8, 8, 4, None, None, None)
+                       None, fake, 16, None, 0, 1, 1, 8, 8, 4, None, None, None)
         == -2
+    )
+    # a prepared backward workspace needs the single-pass forward (chunk a multiple of 128) ...
+    assert (
+        handle.ema_fwd(fake, 8, 1, 0, fake, 64, 8, 0, _lib.EMA_F32, fake, 64, 8, 0, fake, fake, fake,
+                       None, fake, 1 << 30, fake, 1 << 30, 1, 1, 8, 8, 4, None, None, None)
+        == -5
+    )
+    # ... and a backward pass that nothing enters through the final state
+    seq = [fake, 64, 8, 0]
+    coef = [fake, 8, 1, 0]
+    assert (
+        handle.ema_seq_bwd(0, *seq, *seq, *coef, fake, fake, _lib.EMA_F32, *seq, *coef, None, fake, 1 << 30, 1,
+                           1, 1, 8, 8, None, None, None)
+        == -5
     )
 
 

@@ -235,3 +235,55 @@ def test_seq_packed_sequences_probability_form(dtype, device):
     check_close("dx", xg.grad, dx_ref, dtype)
     check_close("dp", pg.grad, dp_ref, dtype)
     check_close("dinit", ig.grad, dinit_ref, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("form", ["log_decay", "probability"])
+def test_backward_workspace_prepared_by_forward(form, dtype, device):
+    """A forward pass can set up the workspace of the backward pass that follows in its own set-up
+    launch.  The backward then gives bit-identical results, a second backward on the same
+    workspace falls back to its own set-up, and so does one with a gradient entering through the
+    final state; the autograd entry points use the hand-over."""
+    from kernels.ema_kernels.ema_combined_fwd import ema_matmul_scan_combined
+    from kernels.ema_seq import ema_seq_bwd, ema_seq_fwd, ema_seq_scan
+
+    announce(f"prepared backward workspace {form} {dtype}")
+    b, L, nh, d = 2, 700, 2, 320  # ragged last tile, two column tiles
+    gen = torch.Generator().manual_seed(11)
+    x = torch.randn(b, L, nh, d, generator=gen).to(dtype).to(device)
+    dy = torch.randn(b, L, nh, d, generator=gen).to(dtype).to(device)
+    p = torch.sigmoid(torch.randn(b, L, nh, generator=gen) - 1.0)
+    coef = (p if form == "probability" else torch.log1p(-p)).to(device)
+    dfin = torch.randn(b, nh, d, generator=gen).to(device)
+
+    y0, fin0, prev0 = ema_seq_fwd(coef, x, form)
+    y1, fin1, prev1, ws = ema_seq_fwd(coef, x, form, prepare_backward=True)
+    assert torch.equal(y0, y1) and torch.equal(fin0, fin1) and torch.equal(prev0, prev1)
+    ref = ema_seq_bwd(dy, x, coef, prev0, form)
+    assert ws.fresh
+    got = ema_seq_bwd(dy, x, coef, prev1, form, workspace=ws)
+    assert not ws.fresh
+    assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1])
+    again = ema_seq_bwd(dy, x, coef, prev1, form, workspace=ws)  # the workspace is used up: own set-up
+    assert torch.equal(again[0], ref[0]) and torch.equal(again[1], ref[1])
+    # a gradient through the final state cannot use the prepared words (they hold a zero entry state)
+    ref_f = ema_seq_bwd(dy, x, coef, prev0, form, dfinal_states=dfin)
+    _, _, prev2, ws2 = ema_seq_fwd(coef, x, form, prepare_backward=True)
+    got_f = ema_seq_bwd(dy, x, coef, prev2, form, dfinal_states=dfin, workspace=ws2)
+    assert torch.equal(got_f[0], ref_f[0]) and torch.equal(got_f[1], ref_f[1])
+
+    # autograd: two backward passes through one forward (the second finds the workspace used up)
+    xg, cg = x.clone().requires_grad_(), coef.clone().requires_grad_()
+    y = ema_seq_scan(cg, xg, form=form)
+    y.backward(dy, retain_graph=True)
+    g1 = (xg.grad.clone(), cg.grad.clone())
+    xg.grad = cg.grad = None
+    y.backward(dy)
+    assert torch.equal(xg.grad, g1[0]) and torch.equal(cg.grad, g1[1])
+    assert torch.equal(g1[0], ref[0]) and torch.equal(g1[1], ref[1])
+    if form == "log_decay":
+        xg, cg = x.clone().requires_grad_(), coef.clone().requires_grad_()
+        ema_matmul_scan_combined(cg, xg, 128).backward(dy)
+        assert torch.equal(xg.grad, ref[0]) and torch.equal(cg.grad, ref[1])
+        with torch.no_grad():  # no gradient wanted: no backward workspace is set up
+            assert torch.equal(ema_matmul_scan_combined(coef, x, 128), y0)

@@ -296,19 +296,35 @@ inline ChainWs chain_carve(void* base, const Dims& di) {
 // carries `seed` (N, T), or 0.  With cs_out the same launch also computes the cumsum of the
 // coefficient over the 128-row tiles (prob = 1: the coefficient is a probability), which the
 // look-back of the kernel that follows reads: one launch and one gap less per pass.
+// The backward pass that will follow a forward pass: its status words and the place of its copy
+// of the cumsum (both in the backward's workspace), prepared by the forward's set-up launch.
+struct NextPass {
+  ChainWs chain;
+  float* cs;
+  int BN;  // columns per tile of the backward kernel
+};
 int launch_chain_init(const ChainWs& w, int64_t cols, int BN, const Dims& di, bool reverse,
                       const float* seed, int ntiles, hipStream_t st, const float* A = nullptr,
-                      SeqStrides sa = SeqStrides{0, 0, 0}, float* cs_out = nullptr, int prob = 0) {
+                      SeqStrides sa = SeqStrides{0, 0, 0}, float* cs_out = nullptr, int prob = 0,
+                      const NextPass* next = nullptr) {
+  auto blocks_of = [](int64_t pairs) { return ((pairs > 4 ? pairs : 4) + 255) / 256; };
   const int64_t pairs = cols * (di.C + 1) * BN / 2;
-  const int64_t threads = pairs > 4 ? pairs : 4;
-  const int64_t init_blocks = (threads + 255) / 256;
+  const int64_t init_blocks = blocks_of(pairs);
   const int64_t chunks = di.N * di.C;
   const int64_t cumsum_blocks = cs_out ? (chunks + 3) / 4 : 0;
-  if (init_blocks + cumsum_blocks > 0x7fffffff) return EMA_ERR_SHAPE;
-  hipLaunchKernelGGL(chain_init_kernel, dim3((unsigned)(init_blocks + cumsum_blocks)), dim3(256), 0, st,
+  ChainNext nx{nullptr, 0, nullptr, 2, 0, 0, nullptr};
+  if (next) {
+    if (!cs_out || reverse) return EMA_ERR_UNSUPPORTED;  // prepared by a forward pass with its cumsum
+    const int64_t ntiles2 = (di.T + next->BN - 1) / next->BN;
+    const int64_t pairs2 = di.N * ntiles2 * (di.C + 1) * next->BN / 2;
+    nx = ChainNext{reinterpret_cast<uint4*>(next->chain.status), pairs2, next->chain.counters, next->BN,
+                   (int)di.C, (int)blocks_of(pairs2), next->cs};
+  }
+  if (init_blocks + nx.blocks + cumsum_blocks > 0x7fffffff) return EMA_ERR_SHAPE;
+  hipLaunchKernelGGL(chain_init_kernel, dim3((unsigned)(init_blocks + nx.blocks + cumsum_blocks)), dim3(256), 0, st,
                      reinterpret_cast<uint4*>(w.status), pairs, w.counters, BN, (int)di.C + 1,
                      reverse ? (int)di.C : 0, ntiles, (int)di.T, seed, (int)init_blocks, A, sa, cs_out,
-                     (int)di.nh, (int)di.L, (int)di.C, chunks, prob);
+                     (int)di.nh, (int)di.L, (int)di.C, chunks, prob, nx);
   return launched();
 }
 
@@ -327,13 +343,16 @@ template <typename T, typename S, bool XP>
 int launch_fwd_tile_t(const void* x, SeqStrides sx, const float* A, SeqStrides sa, float* cs128,
                       void* y, SeqStrides sy, float* prev128, float* prev_coarse, int ratio, float* fin,
                       const float* init, const ChainWs& w, const Dims& di, hipStream_t st, void* ev0,
-                      void* ev1) {
+                      void* ev1, const ChainWs* next_chain = nullptr, float* next_cs = nullptr) {
   using Cfg = TileCfg<T, S::FWD_CPL, S::RPL>;
   constexpr int BN = Cfg::BN, NT = Cfg::NT;
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
-  EMA_TRY(launch_chain_init(w, cols, BN, di, false, init, ntiles, st, A, sa, cs128, XP ? 1 : 0));
+  NextPass next{};
+  if (next_chain) next = NextPass{*next_chain, next_cs, TileCfg<T, S::BWD_CPL, S::RPL>::BN};
+  EMA_TRY(launch_chain_init(w, cols, BN, di, false, init, ntiles, st, A, sa, cs128, XP ? 1 : 0,
+                            next_chain ? &next : nullptr));
   auto kernel = fwd_tile_kernel<T, S::FWD_CPL, S::RPL, S::FWD_MINW, XP>;
   const int64_t cap = resident_blocks(kernel, NT, 0);
   launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx, A,
@@ -347,14 +366,16 @@ template <typename T, typename S, bool WRITE_Y, bool XP>
 int launch_bwd_tile_k(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* A,
                       SeqStrides sa, float* cs128, bool cumsum_here, const float* prev128, void* dx,
                       SeqStrides sdx, void* y, SeqStrides sy, float* part, const float* dfinal, float* dinit,
-                      const ChainWs& w, const Dims& di, hipStream_t st, void* ev0, void* ev1) {
+                      const ChainWs& w, const Dims& di, hipStream_t st, void* ev0, void* ev1,
+                      bool prepared = false) {
   using Cfg = TileCfg<T, S::BWD_CPL, S::RPL>;
   constexpr int BN = Cfg::BN, NT = Cfg::NT;
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
-  EMA_TRY(launch_chain_init(w, cols, BN, di, true, dfinal, ntiles, st, A, sa, cumsum_here ? cs128 : nullptr,
-                            XP ? 1 : 0));
+  if (!prepared)  // otherwise the forward pass has cleared the words and left cs128 in place
+    EMA_TRY(launch_chain_init(w, cols, BN, di, true, dfinal, ntiles, st, A, sa, cumsum_here ? cs128 : nullptr,
+                              XP ? 1 : 0));
   auto kernel = bwd_tile_kernel<T, S::BWD_CPL, S::RPL, S::BWD_MINW, WRITE_Y, XP>;
   const int64_t cap = resident_blocks(kernel, NT, 0);
   launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx,
@@ -368,12 +389,13 @@ template <typename T, typename S, bool XP>
 int launch_bwd_tile_t(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* A,
                       SeqStrides sa, float* cs128, bool cumsum_here, const float* prev128, void* dx,
                       SeqStrides sdx, void* y, SeqStrides sy, float* part, const float* dfinal, float* dinit,
-                      const ChainWs& w, const Dims& di, hipStream_t st, void* ev0, void* ev1) {
+                      const ChainWs& w, const Dims& di, hipStream_t st, void* ev0, void* ev1,
+                      bool prepared = false) {
   if (y)
     return launch_bwd_tile_k<T, S, true, XP>(x, sx, dy, sd, A, sa, cs128, cumsum_here, prev128, dx, sdx, y, sy,
-                                             part, dfinal, dinit, w, di, st, ev0, ev1);
+                                             part, dfinal, dinit, w, di, st, ev0, ev1, prepared);
   return launch_bwd_tile_k<T, S, false, XP>(x, sx, dy, sd, A, sa, cs128, cumsum_here, prev128, dx, sdx, nullptr,
-                                            sy, part, dfinal, dinit, w, di, st, ev0, ev1);
+                                            sy, part, dfinal, dinit, w, di, st, ev0, ev1, prepared);
 }
 
 template <typename S>
@@ -398,6 +420,34 @@ int run_bwd_fused(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, i
   hipLaunchKernelGGL(dA_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, part,
                      ddA, (int)d.L, (int)d.Q, (int)d.C, (int)di.C, bwd_col_tiles(di, dtype), total);
   return launched();
+}
+
+// Workspace of the sequence-level entry points (the backward adds its dA partials).
+struct SeqWs {
+  float *cs, *part;
+  ChainWs chain;
+  size_t bytes;
+};
+SeqWs carve_seq(void* base, const Dims& di, bool backward) {
+  SeqWs w;
+  size_t off = 0;
+  char* p = static_cast<char*>(base);
+  auto take = [&](size_t floats) {
+    float* r = reinterpret_cast<float*>(p + off);
+    off += align_up(floats * sizeof(float), 256);
+    return r;
+  };
+  const size_t ncq = (size_t)(di.N * di.C * di.Q);
+  w.cs = take(ncq);
+  w.part = nullptr;
+  if (backward) {
+    const int pb = tile_parts_per_dim<TileBf16>(di.T), pf = tile_parts_per_dim<TileF32>(di.T);
+    w.part = take(ncq * (size_t)(pb > pf ? pb : pf));
+  }
+  w.chain = chain_carve(p + off, di);
+  off += chain_ws_bytes(di);
+  w.bytes = off;
+  return w;
 }
 
 }  // namespace
@@ -499,10 +549,12 @@ size_t ema_fwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, in
 int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void* x, int64_t x_sb,
             int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb, int64_t y_sl,
             int64_t y_sh, float* cs, float* prev, float* final_state, float* prev128,
-            void* workspace, size_t workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen,
-            int64_t dim, int64_t chunk, void* stream, void* ev_start, void* ev_stop) {
+            void* workspace, size_t workspace_bytes, void* bwd_workspace, size_t bwd_workspace_bytes,
+            int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk, void* stream,
+            void* ev_start, void* ev_stop) {
   Dims d;
   EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
+  if (bwd_workspace && chunk % kTileRows) return EMA_ERR_UNSUPPORTED;
   EMA_TRY(check_dtype(dtype));
   EMA_TRY(check_seq(x, x_sb, x_sl, x_sh, dtype, dim));
   EMA_TRY(check_seq(y, y_sb, y_sl, y_sh, dtype, dim));
@@ -524,13 +576,21 @@ int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void
     float* cs128 = ratio == 1 ? cs : w.cs128;
     float* p128 = prev128 ? prev128 : (ratio == 1 ? prev : w.prev128);
     float* coarse = p128 == prev ? nullptr : prev;
+    SeqWs bw{};
+    if (bwd_workspace) {
+      EMA_TRY(check_f32(bwd_workspace));
+      if (bwd_workspace_bytes < carve_seq(nullptr, di, true).bytes) return EMA_ERR_SHAPE;
+      bw = carve_seq(bwd_workspace, di, true);
+    }
+    const ChainWs* nc = bwd_workspace ? &bw.chain : nullptr;
     if (dtype == EMA_BF16) {
       return launch_fwd_tile_t<bf16_t, TileBf16, false>(x, sx, A, sa, cs128, y, sy, p128, coarse, ratio,
                                                         final_state, nullptr, w.chain, di, st, ev_start,
-                                                        ev_stop);
+                                                        ev_stop, nc, bw.cs);
     }
     return launch_fwd_tile_t<float, TileF32, false>(x, sx, A, sa, cs128, y, sy, p128, coarse, ratio,
-                                                    final_state, nullptr, w.chain, di, st, ev_start, ev_stop);
+                                                    final_state, nullptr, w.chain, di, st, ev_start, ev_stop, nc,
+                                                    bw.cs);
   }
   if (prev128) return EMA_ERR_UNSUPPORTED;  // only produced when chunk is a multiple of 128
   float* states = static_cast<float*>(workspace);
@@ -767,33 +827,6 @@ int ema_bwd_dx_dA_fused(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
 
 // ---- sequence-level entry points: either form of the recurrence, optional boundary states
 
-struct SeqWs {
-  float *cs, *part;
-  ChainWs chain;
-  size_t bytes;
-};
-static SeqWs carve_seq(void* base, const Dims& di, bool backward) {
-  SeqWs w;
-  size_t off = 0;
-  char* p = static_cast<char*>(base);
-  auto take = [&](size_t floats) {
-    float* r = reinterpret_cast<float*>(p + off);
-    off += align_up(floats * sizeof(float), 256);
-    return r;
-  };
-  const size_t ncq = (size_t)(di.N * di.C * di.Q);
-  w.cs = take(ncq);
-  w.part = nullptr;
-  if (backward) {
-    const int pb = tile_parts_per_dim<TileBf16>(di.T), pf = tile_parts_per_dim<TileF32>(di.T);
-    w.part = take(ncq * (size_t)(pb > pf ? pb : pf));
-  }
-  w.chain = chain_carve(p + off, di);
-  off += chain_ws_bytes(di);
-  w.bytes = off;
-  return w;
-}
-
 static int check_form(int form) {
   return (form == EMA_FORM_LOG_DECAY || form == EMA_FORM_PROBABILITY) ? EMA_OK : EMA_ERR_UNSUPPORTED;
 }
@@ -807,8 +840,9 @@ size_t ema_seq_fwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen
 int ema_seq_fwd(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t c_sh, const void* x,
                 int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb,
                 int64_t y_sl, int64_t y_sh, const float* init, float* final_state, float* prev128,
-                void* workspace, size_t workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen,
-                int64_t dim, void* stream, void* ev_start, void* ev_stop) {
+                void* workspace, size_t workspace_bytes, void* bwd_workspace, size_t bwd_workspace_bytes,
+                int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
+                void* ev_stop) {
   Dims d;
   EMA_TRY(check_form(form));
   EMA_TRY(check_dims(batch, nheads, seqlen, dim, kTileRows, true, &d));
@@ -820,20 +854,31 @@ int ema_seq_fwd(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t
   if (workspace_bytes < ema_seq_fwd_workspace_bytes(batch, nheads, seqlen, dim)) return EMA_ERR_SHAPE;
   hipStream_t st = as_stream(stream);
   const SeqWs w = carve_seq(workspace, d, false);
+  SeqWs bw{};
+  if (bwd_workspace) {
+    EMA_TRY(check_f32(bwd_workspace));
+    if (bwd_workspace_bytes < carve_seq(nullptr, d, true).bytes) return EMA_ERR_SHAPE;
+    bw = carve_seq(bwd_workspace, d, true);
+  }
+  const ChainWs* nc = bwd_workspace ? &bw.chain : nullptr;
   const SeqStrides sx{x_sb, x_sl, x_sh}, sy{y_sb, y_sl, y_sh}, sc{c_sb, c_sl, c_sh};
   const bool xp = form == EMA_FORM_PROBABILITY;  // the cumsum of the coefficient is part of the set-up launch
   if (dtype == EMA_BF16) {
     if (xp)
       return launch_fwd_tile_t<bf16_t, TileBf16, true>(x, sx, coef, sc, w.cs, y, sy, prev128, nullptr, 1,
-                                                       final_state, init, w.chain, d, st, ev_start, ev_stop);
+                                                       final_state, init, w.chain, d, st, ev_start, ev_stop, nc,
+        bw.cs);
     return launch_fwd_tile_t<bf16_t, TileBf16, false>(x, sx, coef, sc, w.cs, y, sy, prev128, nullptr, 1,
-                                                      final_state, init, w.chain, d, st, ev_start, ev_stop);
+                                                      final_state, init, w.chain, d, st, ev_start, ev_stop, nc,
+        bw.cs);
   }
   if (xp)
     return launch_fwd_tile_t<float, TileF32, true>(x, sx, coef, sc, w.cs, y, sy, prev128, nullptr, 1,
-                                                   final_state, init, w.chain, d, st, ev_start, ev_stop);
+                                                   final_state, init, w.chain, d, st, ev_start, ev_stop, nc,
+        bw.cs);
   return launch_fwd_tile_t<float, TileF32, false>(x, sx, coef, sc, w.cs, y, sy, prev128, nullptr, 1,
-                                                  final_state, init, w.chain, d, st, ev_start, ev_stop);
+                                                  final_state, init, w.chain, d, st, ev_start, ev_stop, nc,
+        bw.cs);
 }
 
 size_t ema_seq_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim) {
@@ -846,8 +891,8 @@ int ema_seq_bwd(int form, const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t 
                 int64_t x_sb, int64_t x_sl, int64_t x_sh, const float* coef, int64_t c_sb, int64_t c_sl,
                 int64_t c_sh, const float* prev128, const float* dfinal, int dtype, void* dx,
                 int64_t dx_sb, int64_t dx_sl, int64_t dx_sh, float* dcoef, int64_t dc_sb, int64_t dc_sl,
-                int64_t dc_sh, float* dinit, void* workspace, size_t workspace_bytes, int64_t batch,
-                int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
+                int64_t dc_sh, float* dinit, void* workspace, size_t workspace_bytes, int workspace_prepared,
+                int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
                 void* ev_stop) {
   Dims d;
   EMA_TRY(check_form(form));
@@ -859,6 +904,9 @@ int ema_seq_bwd(int form, const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t 
   if (!coef || !prev128 || !dcoef) return EMA_ERR_NULL;
   EMA_TRY(check_f32(workspace));
   if (workspace_bytes < ema_seq_bwd_workspace_bytes(batch, nheads, seqlen, dim)) return EMA_ERR_SHAPE;
+  // a prepared workspace holds nothing entering the reverse scan from outside
+  if (workspace_prepared && dfinal) return EMA_ERR_UNSUPPORTED;
+  const bool prep = workspace_prepared != 0;
   hipStream_t st = as_stream(stream);
   const SeqWs w = carve_seq(workspace, d, true);
   const SeqStrides sx{x_sb, x_sl, x_sh}, sd{dy_sb, dy_sl, dy_sh}, sdx{dx_sb, dx_sl, dx_sh};
@@ -869,22 +917,19 @@ int ema_seq_bwd(int form, const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t 
     parts = tile_parts_per_dim<TileBf16>(d.T);
     if (xp)
       EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, true>(x, sx, dy, sd, coef, sc, w.cs, true, prev128, dx, sdx, nullptr,
-                                                         none, w.part, dfinal, dinit, w.chain, d, st, ev_start,
-                                                         ev_stop)));
+                                                         none, w.part, dfinal, dinit, w.chain, d, st, ev_start, ev_stop, prep)));
     else
       EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, false>(x, sx, dy, sd, coef, sc, w.cs, true, prev128, dx, sdx,
                                                           nullptr, none, w.part, dfinal, dinit, w.chain, d, st,
-                                                          ev_start, ev_stop)));
+                                                          ev_start, ev_stop, prep)));
   } else {
     parts = tile_parts_per_dim<TileF32>(d.T);
     if (xp)
       EMA_TRY((launch_bwd_tile_t<float, TileF32, true>(x, sx, dy, sd, coef, sc, w.cs, true, prev128, dx, sdx, nullptr,
-                                                       none, w.part, dfinal, dinit, w.chain, d, st, ev_start,
-                                                       ev_stop)));
+                                                       none, w.part, dfinal, dinit, w.chain, d, st, ev_start, ev_stop, prep)));
     else
       EMA_TRY((launch_bwd_tile_t<float, TileF32, false>(x, sx, dy, sd, coef, sc, w.cs, true, prev128, dx, sdx, nullptr,
-                                                        none, w.part, dfinal, dinit, w.chain, d, st, ev_start,
-                                                        ev_stop)));
+                                                        none, w.part, dfinal, dinit, w.chain, d, st, ev_start, ev_stop, prep)));
   }
   const int64_t total = d.N * d.L;
   hipLaunchKernelGGL(dcoef_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w.part,

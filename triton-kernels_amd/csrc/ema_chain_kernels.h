@@ -63,18 +63,34 @@ __device__ __forceinline__ unsigned chain_wait(const u64* p, float* v, unsigned*
 // The set-up of a single-pass kernel in one launch: the first init_blocks workgroups clear the
 // status words (and seed the virtual slot), the rest, if any, compute the per-tile cumsum of the
 // log-decay that the look-back reads (cumsum_block; cs null = no such workgroups are launched).
+// A forward pass whose backward will follow can have the backward's status words prepared in the
+// same launch (next: the words of the reverse scan with nothing entering it, next_blocks
+// workgroups after the first init_blocks) together with a second copy of the cumsum (cs_next).
+struct ChainNext {
+  uint4* words;
+  int64_t n_pairs;
+  unsigned* counters;
+  int BN, virt_slot, blocks;
+  float* cs;
+};
 __global__ __launch_bounds__(256) void chain_init_kernel(uint4* __restrict__ words, int64_t n_pairs,
                                                          unsigned* __restrict__ counters, int BN,
                                                          int slots, int virt_slot, int ntiles, int Tdim,
                                                          const float* __restrict__ seed, int init_blocks,
                                                          const float* __restrict__ A, SeqStrides sa,
                                                          float* __restrict__ cs, int nh, int L, int C,
-                                                         int64_t total_chunks, int prob) {
-  if ((int)blockIdx.x >= init_blocks) {
-    cumsum_block((int64_t)blockIdx.x - init_blocks, A, sa, cs, nh, L, kTileRows, C, total_chunks, prob);
+                                                         int64_t total_chunks, int prob, ChainNext next) {
+  int64_t blk = blockIdx.x;
+  if (blk >= init_blocks + next.blocks) {
+    cumsum_block(blk - init_blocks - next.blocks, A, sa, cs, nh, L, kTileRows, C, total_chunks, prob, next.cs);
     return;
   }
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (blk >= init_blocks) {  // the pass that follows: same layout, its own column width, no seed
+    blk -= init_blocks;
+    words = next.words, n_pairs = next.n_pairs, counters = next.counters, BN = next.BN;
+    virt_slot = next.virt_slot, seed = nullptr;
+  }
+  const int64_t i = blk * 256 + threadIdx.x;
   if (i < 4) counters[i] = 0u;
   if (i >= n_pairs) return;
   const int64_t w = 2 * i;

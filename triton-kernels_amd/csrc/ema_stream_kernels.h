@@ -22,7 +22,7 @@ __device__ __forceinline__ float cumsum_term(float v, int prob) {
 // The work of workgroup `block` (four chunks, one per wave).
 __device__ __forceinline__ void cumsum_block(int64_t block, const float* __restrict__ A, SeqStrides sa,
                                              float* __restrict__ cs, int nh, int L, int Q, int C,
-                                             int64_t total_chunks, int prob) {
+                                             int64_t total_chunks, int prob, float* __restrict__ cs2 = nullptr) {
   const int lane = threadIdx.x & 63;
   const int64_t chunk_id = block * 4 + (threadIdx.x >> 6);
   if (chunk_id >= total_chunks) return;
@@ -45,7 +45,10 @@ __device__ __forceinline__ void cumsum_block(int64_t block, const float* __restr
   for (int i = 0; i < per; ++i) {
     const int q = q0 + i;
     if (q < limit) run += cumsum_term(a[(int64_t)q * sa.sl], prob);
-    if (q < Q) out[q] = run;
+    if (q < Q) {
+      out[q] = run;
+      if (cs2) cs2[chunk_id * Q + q] = run;  // a second copy for the pass that follows
+    }
   }
 }
 

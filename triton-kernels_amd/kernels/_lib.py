@@ -31,7 +31,7 @@ _SIGNATURES = {
     "ema_state_passing_fwd": (c_int, [_P, _P, _I, _I, _P, _P, _I, _I, _I, _P]),
     "ema_scan_fwd": (c_int, _SEQ + [c_int, _P, _P] + _SEQ + [_I, _I, _I, _I, _I, _P]),
     "ema_fwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I]),
-    "ema_fwd": (c_int, _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _P, _P, _P]),
+    "ema_fwd": (c_int, _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, _P, c_size_t, _P, c_size_t, _I, _I, _I, _I, _I, _P, _P, _P]),
     "ema_chunk_scan_bwd_dstates": (c_int, _SEQ + [c_int, _P, _P, _I, _I, _I, _I, _I, _P]),
     "ema_state_passing_bwd_workspace_bytes": (c_size_t, [_I, _I, _I]),
     "ema_state_passing_bwd": (c_int, [_P, _P, _I, _I, _P, _P, _P, _P, c_size_t, _I, _I, _I, _P]),
@@ -46,8 +46,8 @@ _SIGNATURES = {
     "ema_bwd": (c_int, _SEQ + _SEQ + _SEQ + [_P, c_int] + _SEQ + [_P] + _SEQ + [_P, c_size_t, _I, _I, _I, _I, _I, _P, _P, _P]),
     "ema_seq_fwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "ema_seq_bwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
-    "ema_seq_fwd": (c_int, [c_int] + _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _P, _P, _P]),
-    "ema_seq_bwd": (c_int, [c_int] + _SEQ + _SEQ + _SEQ + [_P, _P, c_int] + _SEQ + _SEQ + [_P, _P, c_size_t, _I, _I, _I, _I, _P, _P, _P]),
+    "ema_seq_fwd": (c_int, [c_int] + _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, c_size_t, _P, c_size_t, _I, _I, _I, _I, _P, _P, _P]),
+    "ema_seq_bwd": (c_int, [c_int] + _SEQ + _SEQ + _SEQ + [_P, _P, c_int] + _SEQ + _SEQ + [_P, _P, c_size_t, c_int, _I, _I, _I, _I, _P, _P, _P]),
     # SSD forward stages (include/ssd_hip.h)
     "ssd_chunk_cumsum_fwd": (c_int, [_P, c_int, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, c_int, c_float, c_float, _P]),
     "ssd_chunk_state_fwd": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
@@ -174,6 +174,23 @@ def f32c(t: torch.Tensor) -> torch.Tensor:
     if t.dtype != torch.float32:
         t = t.float()
     return t.contiguous()
+
+
+class BackwardWorkspace:
+    """Workspace of the ema_seq_bwd call that follows a forward pass, prepared by that forward
+    pass's set-up launch (status words of the reverse scan, cumsum of the coefficient), so that the
+    backward needs no set-up launch of its own.  Good for one backward call: take() hands the
+    buffer out once and reports whether it is still as the forward left it."""
+
+    def __init__(self, batch: int, nh: int, L: int, T: int, dev: torch.device):
+        self.nbytes = lib().ema_seq_bwd_workspace_bytes(batch, nh, L, T)
+        assert self.nbytes > 0, "unsupported shape"
+        self.buf = torch.empty(self.nbytes, dtype=torch.uint8, device=dev)
+        self.fresh = True
+
+    def take(self):
+        fresh, self.fresh = self.fresh, False
+        return self.buf, fresh
 
 
 def state_tensor(t: torch.Tensor, like: torch.Tensor = None):
