@@ -54,3 +54,79 @@ def test_step_in_hip_graph(dtype, device):
         check_close(f"replay {rep} dA", dA_g, dA_ref, torch.float32)
     xf, Af = O.to_flat(x2.float(), A2)
     check_close("last replay vs oracle", y_g, O.from_flat(O.ema_loop(xf, Af), b, nh), dtype)
+
+
+@pytest.mark.parametrize("packed", [False, True], ids=["plain", "packed"])
+def test_ssd_forward_and_backward_stages_in_hip_graph(packed, device):
+    """The Mamba-2 SSD launchers enqueue kernels only as well: the five forward stages and the six
+    backward stage launchers captured in one graph, replayed with new inputs in the static buffers
+    and eager work in between, every replay bit-identical to the eager run."""
+    from kernels.mamba_kernels.mamba_combined_fwd import _mamba_chunk_scan_combined_fwd
+    from kernels.mamba_kernels.mamba_bmm import _bmm_chunk_fwd
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_bwd_da import _chunk_scan_bwd_ddAcs_stable
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_bwd_dc import _chunk_scan_bwd_dC
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_chunk_state_bwd_dx import _chunk_scan_chunk_state_bwd_dx
+    from kernels.mamba_kernels_bwd.mamba_chunk_state_bwd_db import _chunk_state_bwd_db
+    from kernels.mamba_kernels_bwd.mamba_scan_bwd import _chunk_scan_bwd_dstates
+    from kernels.mamba_kernels_bwd.mamba_state_passing_bwd_dstates import _state_passing_bwd
+    from oracle import ssd_oracle as S
+
+    announce(f"hip graph: ssd forward + backward stages, packed={packed}")
+    b, L, nh, P, g, N, Q = 2, 600, 4, 64, 1, 128, 256
+    BF16 = torch.bfloat16
+
+    def inputs(seed):
+        x, dt, A, B, C, _, _ = S.make_inputs(b, L, nh, P, g, N, seed=seed, dtype=BF16)
+        dout = torch.randn(b, L, nh, P, generator=torch.Generator().manual_seed(seed)).to(BF16)
+        return [t.to(device) for t in (x, dt, A, B, C, dout)]
+
+    static = inputs(1)
+    seq = None
+    if packed:
+        ids = torch.zeros(b, L, dtype=torch.int32)
+        ids[0, 100:] += 1
+        ids[0, 256:] += 1
+        ids[1, 300:] += 1
+        seq = ids.to(device)
+
+    def step():
+        x, dt, A, B, C, dout = static
+        out, _, dt_out, dA_cs, states, final = _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, Q, seq_idx=seq)
+        nc = dt_out.shape[2]
+        cb = _bmm_chunk_fwd(C, B, Q, seq_idx=seq, output_dtype=torch.float32)
+        dprev = _chunk_scan_bwd_dstates(C, dA_cs, dout, seq_idx=seq)
+        dstates, ddA_chunk, _ = _state_passing_bwd(states.view(b, nc, nh, P * N), dA_cs[..., -1],
+                                                   dprev.view(b, nc, nh, P * N), seq_idx=seq, chunk_size=Q)
+        dstates = dstates.view(b, nc, nh, P, N)
+        dB, ddA_b = _chunk_state_bwd_db(x, dt_out, dA_cs, dstates, seq_idx=seq, B=B, ngroups=g)
+        dC, ddA_c = _chunk_scan_bwd_dC(states, dA_cs, dout, seq_idx=seq, C=C, ngroups=g)
+        dx, ddt, _ = _chunk_scan_chunk_state_bwd_dx(x, dt_out, dA_cs, B, cb, dout, dstates, seq_idx=seq)
+        ddA = _chunk_scan_bwd_ddAcs_stable(x, dt_out, dA_cs, dout, cb)
+        return out, final, dstates, ddA_chunk, dB, ddA_b, dC, ddA_c, dx, ddt, ddA
+
+    eager = [t.clone() for t in step()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream(device)
+    side.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream(device).wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    names = "out final dstates ddA_chunk dB ddA_b dC ddA_c dx ddt ddA".split()
+    for rep in range(3):
+        for dst, src in zip(static, inputs(10 + rep)):
+            dst.copy_(src)
+        ref = [t.clone() for t in step()]
+        torch.cuda.synchronize()
+        for t in captured:
+            t.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, got, want in zip(names, captured, ref):
+            assert torch.equal(got, want), f"replay {rep}: {name} differs from the eager result"
+    x, dt, A, B, C, _ = [t.cpu() for t in static]
+    y_ref, _ = S.ssd_loop(x.float(), dt, A, B.float(), C.float(), seq_idx=None if seq is None else seq.cpu())
+    check_close("last replay vs the recurrence", captured[0], y_ref, BF16, loose=True)
