@@ -105,7 +105,7 @@ def cpu_baseline(args, torch):
 
     threads = torch.get_num_threads()
     nseq_total = args.batch * args.nheads
-    sample_b = 1
+    sample_b = min(4, args.batch)  # about 10 s of CPU work: 20 to 30 repetitions of a quarter of the batch
     x, A, dy = O.make_inputs(sample_b, args.nheads, args.seqlen, args.dim, seed=1, dtype=torch.bfloat16)
     xf, Af = O.to_flat(x.float(), A)
     dyf, _ = O.to_flat(dy.float(), A)
@@ -115,7 +115,7 @@ def cpu_baseline(args, torch):
         O.ema_loop(xf, Af)
         O.ema_loop_bwd(dyf, xf, Af)
         reps += 1
-        if time.perf_counter() - t0 > 10.0 or reps >= 20:
+        if time.perf_counter() - t0 > 10.0 or reps >= 40:
             break
     per = (time.perf_counter() - t0) / reps
     scale = nseq_total / (sample_b * args.nheads)
@@ -243,7 +243,7 @@ def ssd_main(args):
         x, dt, A, B, Cm, _, _ = S.make_inputs(1, 512, nh, P, g, N, seed=5, dtype=torch.bfloat16)
         t0 = time.perf_counter()
         reps = 0
-        while time.perf_counter() - t0 < 10.0 and reps < 20:
+        while time.perf_counter() - t0 < 10.0 and reps < 400:  # about 10 s of CPU work
             S.ssd_loop(x.float(), dt, A, B.float(), Cm.float())
             reps += 1
         per = (time.perf_counter() - t0) / reps
