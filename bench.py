@@ -2,7 +2,7 @@
 """Benchmark of the EMA chunked scan, forward + backward, on one MI355X.
 
 One step = one forward and one backward through the autograd entry point
-(ema_matmul_scan_combined(...).backward(dy)) of BASELINE configuration 3 at chunk size 128:
+(ema_matmul_scan_combined(...).backward(dy)) of benchmark configuration 3 at chunk size 128:
 b16 nh2 d1024 L4096, bf16 x / dy, fp32 log-decay and accumulation.  The forward is one pass
 over x (cumsum + single-pass chained scan), the backward one pass over x and dy.  Inputs are synthetic and resident in HBM before the timed
 region; the step rotates over several input sets so that no step finds its inputs in the
@@ -54,7 +54,7 @@ def parse():
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel timing pass")
     ap.add_argument("--workload", default="ema", choices=["ema", "ssd"],
                     help="ema: the headline EMA scan step (default); ssd: the Mamba-2 SSD forward stages at "
-                    "BASELINE configuration 5 (b8 nh32 hdim64 dstate128 g1 L8192 chunk256, bf16)")
+                    "benchmark configuration 5 (b8 nh32 hdim64 dstate128 g1 L8192 chunk256, bf16)")
     ap.add_argument("--stage", default=None,
                     help="time only this stage (a name from the `kernels` table, or fwd, bwd, copy) "
                     "and print a short JSON line; used for counter collection")
@@ -130,7 +130,7 @@ def cpu_baseline(args, torch):
 
 
 def ssd_main(args):
-    """Mamba-2 SSD forward at BASELINE configuration 5: the five stage launchers and their sum,
+    """Mamba-2 SSD forward at benchmark configuration 5: the five stage launchers and their sum,
     timed with events on the launch stream; per stage the algorithmic bytes (inputs read once,
     outputs written once) against the HBM peak and, for the three MFMA stages, dense FLOPs
     against the bf16 MFMA peak."""

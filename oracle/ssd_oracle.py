@@ -270,7 +270,7 @@ def combined_fwd(x, dt, A, B, C, Q, D=None, z=None, dt_bias=None, initial_states
 
 
 def make_inputs(b, L, nh, p, g, n, seed, dtype=torch.float32, with_z=False):
-    """BASELINE configuration 5's distributions: x, B, C ~ N(0,1); dt = softplus(N(-2, 0.5));
+    """benchmark configuration 5's distributions: x, B, C ~ N(0,1); dt = softplus(N(-2, 0.5));
     A = -exp(U(log 1, log 16)) per head; D = 0 is the configuration's choice (a non-zero D is
     returned for the tests that want one); z ~ N(0,1)."""
     gen = torch.Generator().manual_seed(seed)

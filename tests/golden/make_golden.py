@@ -10,7 +10,7 @@ with oracle/ or the HIP library:
     dx_t = dy_t + exp(A_{t+1}) * dx_{t+1}
     dA_t = exp(A_t) * <dx_t, y_{t-1}>
 
-Inputs are drawn as BASELINE config 1 describes (x ~ N(0,1), alpha = sigmoid(u), u ~ N(2,1),
+Inputs are drawn as benchmark configuration 1 describes (x ~ N(0,1), alpha = sigmoid(u), u ~ N(2,1),
 log-decay log(alpha), input (1 - alpha) * x) and stored as float32; the bf16 cases store
 values already rounded to bfloat16.  Run `python tests/golden/make_golden.py` to rewrite."""
 import os

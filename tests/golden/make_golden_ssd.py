@@ -12,7 +12,7 @@ here in float64 with plain numpy loops and no code shared with oracle/ or the HI
       z_t = (1 - p_t) * z_{t-1} + p_t * x_t,  z_{-1} = init, and the gradients of
       sum(z * dz) + sum(final * dfinal) with respect to x, p and init by the reverse recurrence.
 
-Inputs as BASELINE configuration 5 describes (x, B, C ~ N(0,1), dt = softplus(N(-2, 0.5)),
+Inputs as benchmark configuration 5 describes (x, B, C ~ N(0,1), dt = softplus(N(-2, 0.5)),
 A = -exp(U(log 1, log 16))) and stored as float32.  Run `python tests/golden/make_golden_ssd.py`
 to rewrite."""
 import os

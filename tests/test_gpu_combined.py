@@ -1,5 +1,5 @@
 """GPU parity of the combined forward / backward and of the autograd entry point against
-the sequential CPU oracle, including BASELINE configurations 1-4 at their full sizes."""
+the sequential CPU oracle, including benchmark configurations 1-4 at their full sizes."""
 import pytest
 import torch
 
@@ -132,7 +132,7 @@ def _autograd_headed(x, A, dy, Q, device):
 
 
 def test_config1_fp32_forward(device):
-    """BASELINE config 1: b1 nh2 L512 d64 Q128 fp32, input scaled by (1 - alpha), compared
+    """benchmark configuration 1: b1 nh2 L512 d64 Q128 fp32, input scaled by (1 - alpha), compared
     with y_t = alpha_t y_{t-1} + (1 - alpha_t) x_t."""
     from kernels.ema_kernels.ema_combined_fwd import ema_matmul_scan_combined
 
@@ -163,7 +163,7 @@ def test_autograd_headed_small(dtype, device):
 
 @pytest.mark.parametrize("Q", [128, 256, 512])
 def test_config3_bf16_fwd_bwd_full_size(Q, device):
-    """BASELINE configs 2 and 3: b16 nh2 d1024 L4096, bf16, chunk size swept, seed fixed per
+    """benchmark configurations 2 and 3: b16 nh2 d1024 L4096, bf16, chunk size swept, seed fixed per
     chunk size; forward, dx and dA against the sequential oracle at full size."""
     announce(f"config 2/3 full size Q{Q}")
     x, A, dy = O.make_inputs(16, 2, 4096, 1024, seed=1000 + Q, dtype=BF16)
@@ -175,7 +175,7 @@ def test_config3_bf16_fwd_bwd_full_size(Q, device):
 
 
 def test_config4_long_sequence(device):
-    """BASELINE config 4: b4 nh2 d1024 L32768 Q256, bf16, u ~ N(4,1) (long memory)."""
+    """benchmark configuration 4: b4 nh2 d1024 L32768 Q256, bf16, u ~ N(4,1) (long memory)."""
     announce("config 4 full size")
     x, A, dy = O.make_inputs(4, 2, 32768, 1024, seed=4, dtype=BF16, u_mean=4.0)
     y, dx, dA = _autograd_headed(x, A, dy, 256, device)

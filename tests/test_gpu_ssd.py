@@ -1,6 +1,6 @@
 """GPU parity of the Mamba-2 SSD forward stages (through the C ABI) against the CPU oracle:
 each stage against its restatement on the same inputs, the five stages together against the
-sequential state-space recurrence, and BASELINE configuration 5 at full size through one
+sequential state-space recurrence, and benchmark configuration 5 at full size through one
 sequence checked against the recurrence plus chunk-size invariance for the rest."""
 import pytest
 import torch

@@ -59,7 +59,7 @@ def test_loop_first_step_ignores_first_decay():
 
 
 def test_probability_form_config1():
-    # BASELINE config 1: y_t = alpha_t y_{t-1} + (1 - alpha_t) x_t with X = (1-alpha) x
+    # benchmark configuration 1: y_t = alpha_t y_{t-1} + (1 - alpha_t) x_t with X = (1-alpha) x
     x, A, _ = O.make_inputs(1, 2, 512, 64, seed=11, scale_x=False)
     xs, _, _ = O.make_inputs(1, 2, 512, 64, seed=11, scale_x=True)
     alpha = torch.exp(A)
