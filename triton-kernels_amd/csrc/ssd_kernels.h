@@ -436,6 +436,51 @@ __device__ __forceinline__ void state_store4(bf16_t* p, float4 v) {
   __builtin_nontemporal_store(w, reinterpret_cast<ema::bf16x4*>(p));
 }
 
+// E adjacent elements of a state-sized tensor per thread: 4, or 8 where that makes the bfloat16
+// accesses 16 bytes; a workgroup covers 256 * E elements of the state.
+template <int E>
+struct StateVec {
+  float v[E];
+};
+template <int E>
+__device__ __forceinline__ StateVec<E> state_load(const float* p) {
+  StateVec<E> r;
+#pragma unroll
+  for (int i = 0; i < E; i += 4) {
+    const float4 t = stream_load4(p + i);
+    r.v[i] = t.x, r.v[i + 1] = t.y, r.v[i + 2] = t.z, r.v[i + 3] = t.w;
+  }
+  return r;
+}
+template <int E>
+__device__ __forceinline__ StateVec<E> state_load(const bf16_t* p) {
+  StateVec<E> r;
+  if constexpr (E == 8) {
+    const Vec16<bf16_t> t = load16_stream(p);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r.v[i] = t.get(i);
+  } else {
+    const float4 t = state_load4<true>(p);
+    r.v[0] = t.x, r.v[1] = t.y, r.v[2] = t.z, r.v[3] = t.w;
+  }
+  return r;
+}
+template <int E>
+__device__ __forceinline__ void state_store(float* p, const StateVec<E>& s) {
+#pragma unroll
+  for (int i = 0; i < E; i += 4) stream_store4(p + i, make_float4(s.v[i], s.v[i + 1], s.v[i + 2], s.v[i + 3]));
+}
+template <int E>
+__device__ __forceinline__ void state_store(bf16_t* p, const StateVec<E>& s) {
+  if constexpr (E == 8) {
+    Vec16<bf16_t> t;
+    t.set_all(s.v);
+    store16_stream(p, t);
+  } else {
+    state_store4(p, make_float4(s.v[0], s.v[1], s.v[2], s.v[3]));
+  }
+}
+
 // ------------------------------------------------------------------------------------
 // state_passing.  out[b, c] = state entering chunk c, state <- exp(dA_chunk[c]) * state +
 // states[b, c]; the value after the last chunk goes to final.  One thread per four adjacent
@@ -444,7 +489,7 @@ __device__ __forceinline__ void state_store4(bf16_t* p, float4 v) {
 // last column of dA_cumsum).  In a packed batch the state is dropped across a chunk whose last
 // position has another id than the previous chunk's last position.
 // ------------------------------------------------------------------------------------
-template <typename TO>
+template <typename TO, int E>
 __global__ __launch_bounds__(256) void ssd_state_passing_kernel(
     const float* __restrict__ states, const float* __restrict__ dA_chunk, int64_t da_sb, int64_t da_sh,
     int64_t da_sc, const float* __restrict__ initial, TO* __restrict__ out, float* __restrict__ final_states,
@@ -452,38 +497,39 @@ __global__ __launch_bounds__(256) void ssd_state_passing_kernel(
   const int tile = blockIdx.x % tiles;
   const int h = (blockIdx.x / tiles) % nh;
   const int64_t b = blockIdx.x / (tiles * nh);
-  const int e = (tile * 256 + threadIdx.x) * 4;
+  const int e = (tile * 256 + threadIdx.x) * E;
   if (e >= dim) return;
   const int64_t chunk_stride = (int64_t)nh * dim;
   const float* src = states + (b * C * nh + h) * (int64_t)dim + e;
   TO* dst = out + (b * C * nh + h) * (int64_t)dim + e;
   const float* da = dA_chunk + b * da_sb + h * da_sh;
-  float4 s = initial ? *reinterpret_cast<const float4*>(initial + (b * nh + h) * (int64_t)dim + e)
-                     : make_float4(0.f, 0.f, 0.f, 0.f);
+  StateVec<E> s;
+#pragma unroll
+  for (int i = 0; i < E; ++i) s.v[i] = initial ? initial[(b * nh + h) * (int64_t)dim + e + i] : 0.f;
   constexpr int U = 4;
   for (int c0 = 0; c0 < C; c0 += U) {
-    float4 nv[U];
+    StateVec<E> nv[U];
     float a[U];
+    // unconditional loads from chunk indices clamped into the tensor
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int c = c0 + u;
-      nv[u] = c < C ? stream_load4(src + c * chunk_stride) : make_float4(0.f, 0.f, 0.f, 0.f);
-      a[u] = c < C ? __expf(da[(int64_t)c * da_sc]) : 0.f;
-      if (c < C && !chunk_keeps_state(seq, b, c, Q, L)) a[u] = 0.f;
+      const int c = min(c0 + u, C - 1);
+      nv[u] = state_load<E>(src + c * chunk_stride);
+      a[u] = __expf(da[(int64_t)c * da_sc]);
+      if (!chunk_keeps_state(seq, b, c, Q, L)) a[u] = 0.f;
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int c = c0 + u;
       if (c < C) {
-        state_store4(dst + c * chunk_stride, s);
-        s.x = fmaf(a[u], s.x, nv[u].x);
-        s.y = fmaf(a[u], s.y, nv[u].y);
-        s.z = fmaf(a[u], s.z, nv[u].z);
-        s.w = fmaf(a[u], s.w, nv[u].w);
+        state_store<E>(dst + c * chunk_stride, s);
+#pragma unroll
+        for (int i = 0; i < E; ++i) s.v[i] = fmaf(a[u], s.v[i], nv[u].v[i]);
       }
     }
   }
-  *reinterpret_cast<float4*>(final_states + (b * nh + h) * (int64_t)dim + e) = s;
+#pragma unroll
+  for (int i = 0; i < E; ++i) final_states[(b * nh + h) * (int64_t)dim + e + i] = s.v[i];
 }
 
 // Sum over the 32 lanes of each half of a wave (lanes 0..31 and 32..63 apart), left in lanes 31
@@ -504,7 +550,7 @@ __device__ __forceinline__ float half_wave_sum(float v) {
 // The finish kernel sums the wave partials: ddA[b,h,c] = exp(dA_chunk[c]) * sum, and 0 for
 // c = 0 when there is no initial state.
 // ------------------------------------------------------------------------------------
-template <typename TS, typename TD, typename TG>
+template <typename TS, typename TD, typename TG, int E>
 __global__ __launch_bounds__(256) void ssd_state_passing_bwd_kernel(
     const TS* __restrict__ states, const float* __restrict__ dA_chunk, int64_t da_sb, int64_t da_sh,
     int64_t da_sc, const TD* __restrict__ dout, const float* __restrict__ dfinal,
@@ -513,43 +559,48 @@ __global__ __launch_bounds__(256) void ssd_state_passing_bwd_kernel(
   const int tile = blockIdx.x % tiles;
   const int h = (blockIdx.x / tiles) % nh;
   const int64_t b = blockIdx.x / (tiles * nh);
-  const int e = (tile * 256 + threadIdx.x) * 4;
+  const int e = (tile * 256 + threadIdx.x) * E;
   const bool ok = e < dim;
   const int lane = threadIdx.x & 63;
   const int wave_id = tile * 4 + (threadIdx.x >> 6), nw = tiles * 4;
   const int64_t chunk_stride = (int64_t)nh * dim;
   const int64_t base = (b * C * nh + h) * (int64_t)dim + (ok ? e : 0);
   const float* da = dA_chunk + b * da_sb + h * da_sh;
-  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
-  float4 G = (dfinal && ok) ? *reinterpret_cast<const float4*>(dfinal + (b * nh + h) * (int64_t)dim + e) : zero4;
+  StateVec<E> G;
+#pragma unroll
+  for (int i = 0; i < E; ++i) G.v[i] = (dfinal && ok) ? dfinal[(b * nh + h) * (int64_t)dim + e + i] : 0.f;
   constexpr int U = 4;
   for (int c1 = C - 1; c1 >= 0; c1 -= U) {
-    float4 sv[U], dv[U];
+    StateVec<E> sv[U], dv[U];
     float a[U];
+    // unconditional loads from chunk indices clamped into the tensor; what lies outside is zeroed
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int c = c1 - u;
-      const bool in = c >= 0 && ok;
-      sv[u] = in ? state_load4<true>(states + base + c * chunk_stride) : zero4;
-      dv[u] = in ? state_load4<true>(dout + base + c * chunk_stride) : zero4;
-      a[u] = c >= 0 ? __expf(da[(int64_t)c * da_sc]) : 0.f;
-      if (c >= 0 && !chunk_keeps_state(seq, b, c, Q, L)) a[u] = 0.f;
+      const int c = max(c1 - u, 0);
+      sv[u] = state_load<E>(states + base + c * chunk_stride);
+      dv[u] = state_load<E>(dout + base + c * chunk_stride);
+      a[u] = __expf(da[(int64_t)c * da_sc]);
+      if (!chunk_keeps_state(seq, b, c, Q, L)) a[u] = 0.f;
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int c = c1 - u;
       if (c >= 0) {  // uniform across the workgroup
-        if (ok) state_store4(dstates + base + c * chunk_stride, G);
-        const float dot = ema::wave_sum(sv[u].x * G.x + sv[u].y * G.y + sv[u].z * G.z + sv[u].w * G.w);
+        if (ok) state_store<E>(dstates + base + c * chunk_stride, G);
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < E; ++i) dot = fmaf(sv[u].v[i], G.v[i], dot);
+        dot = ema::wave_sum(ok ? dot : 0.f);
         if (lane == 0) part[((b * nh + h) * C + c) * (int64_t)nw + wave_id] = dot;
-        G.x = fmaf(a[u], G.x, dv[u].x);
-        G.y = fmaf(a[u], G.y, dv[u].y);
-        G.z = fmaf(a[u], G.z, dv[u].z);
-        G.w = fmaf(a[u], G.w, dv[u].w);
+#pragma unroll
+        for (int i = 0; i < E; ++i) G.v[i] = fmaf(a[u], G.v[i], dv[u].v[i]);
       }
     }
   }
-  if (dinit && ok) *reinterpret_cast<float4*>(dinit + (b * nh + h) * (int64_t)dim + e) = G;
+  if (dinit && ok) {
+#pragma unroll
+    for (int i = 0; i < E; ++i) dinit[(b * nh + h) * (int64_t)dim + e + i] = G.v[i];
+  }
 }
 
 __global__ __launch_bounds__(256) void ssd_state_passing_bwd_finish_kernel(
