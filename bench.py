@@ -30,9 +30,9 @@ for p in (ROOT, os.path.join(ROOT, "triton-kernels_amd")):
 TRAFFIC_BYTES = {"fwd_single_pass": 589083033, "bwd_single_pass": 841025145}
 # the same for the SSD stage kernels at configuration 5 (finishing kernels added to their stage)
 SSD_TRAFFIC_BYTES = {
-    "chunk_cumsum": 25311987, "chunk_state": 571562572, "state_passing": 419497855, "bmm_chunk": 100778356,
-    "chunk_scan": 742659408, "bwd_dstates": 448841641, "bwd_state_passing": 423804876, "bwd_db": 496062416,
-    "bwd_dc": 469832558, "bwd_dx": 1020231743, "bwd_ddAcs": 599940259,
+    "chunk_cumsum": 25320408, "chunk_state": 571591572, "state_passing": 419465499, "bmm_chunk": 100772767,
+    "chunk_scan": 742659447, "bwd_dstates": 446640967, "bwd_state_passing": 409601722, "bwd_db": 496071800,
+    "bwd_dc": 469831534, "bwd_dx": 1020235822, "bwd_ddAcs": 599926788,
 }
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
