@@ -137,19 +137,29 @@ struct ScanLaunch {
       if (prev_dtype != SSD_F32) return run_as<T, P, N, T>();
     return run_as<T, P, N, float>();
   }
+  template <typename T, int P, int N, typename TS, int HP>
+  int launch_wide() const {
+    auto kernel = ssd_chunk_scan_wide_kernel<T, P, N, TS, HP>;
+    constexpr int smem = WideSmem<T, P * HP, N>::bytes_for(HP);
+    SSD_TRY(allow_smem(kernel, smem));
+    const int stiles = (int)(d.Q / 256);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * (d.nh / HP) * stiles)), dim3(256), smem, st, cb,
+                       (const T*)x, sx, (const T*)z, sz, dt, dA, (const T*)C, sC, (const TS*)prev, D, d_has_hdim,
+                       (T*)out, so, (T*)out_x, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C,
+                       stiles, seq);
+    return launched();
+  }
   template <typename T, int P, int N, typename TS>
   int run_as() const {
     constexpr int wide_smem = WideSmem<T, P, N>::kBytes;
     if (d.Q % 256 == 0 && wide_smem <= kLdsBytes) {  // 256-row super-tiles, no barrier inside the k loop
-      auto kernel = ssd_chunk_scan_wide_kernel<T, P, N, TS>;
-      constexpr int smem = wide_smem;
-      SSD_TRY(allow_smem(kernel, smem));
-      const int stiles = (int)(d.Q / 256);
-      hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.nh * stiles)), dim3(256), smem, st, cb,
-                         (const T*)x, sx, (const T*)z, sz, dt, dA, (const T*)C, sC, (const TS*)prev, D, d_has_hdim,
-                         (T*)out, so, (T*)out_x, (int)d.nh, (int)(d.nh / d.g), (int)d.g, (int)d.L, (int)d.Q, (int)d.C,
-                         stiles, seq);
-      return launched();
+      // Two adjacent heads of a group per workgroup where they are adjacent in memory too (dense
+      // heads of 64 features): they share the fragments of cb and the rows of C.
+      if constexpr (P == 64 && WideSmem<T, 128, N>::bytes_for(2) <= kLdsBytes / 2) {
+        const bool dense = sx.sh == P && so.sh == P && (!z || sz.sh == P);
+        if (dense && (d.nh / d.g) % 2 == 0) return launch_wide<T, P, N, TS, 2>();
+      }
+      return launch_wide<T, P, N, TS, 1>();
     }
     auto kernel = ssd_chunk_scan_kernel<T, P, N, TS>;
     constexpr int smem = ScanSmem<T, P, N>::kBytes;

@@ -1062,39 +1062,54 @@ struct WideSmem {
   static constexpr int kXP = kX > kPrev ? kX : kPrev;
   static constexpr int kMain = kXP > kOut ? kXP : kOut;
   static constexpr int kBytes = kMain + 3 * ST * (int)sizeof(float);            // + dA_k, dt_k, exp(dA_m)
+  // the same with those three vectors for each of `heads` heads sharing a tile of this width
+  static constexpr int bytes_for(int heads) { return kMain + heads * 3 * ST * (int)sizeof(float); }
 };
 
-template <typename T, int P, int N, typename TS>
+// HP heads per workgroup (1 or 2).  Two adjacent heads of one group share everything that does not
+// depend on the head: the fragments of cb and the rows of C, which are the costly per-lane loads of
+// this kernel.  Their x / z / out rows and their carried states are adjacent in memory (heads are
+// dense in those tensors; the host checks), so the pair is staged and stored like one head of twice
+// the width; the weights, the scale of the carried-state term and D are per head.
+template <typename T, int P, int N, typename TS, int HP>
 __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
     const float* __restrict__ cb, const T* __restrict__ x, Strides3 sx, const T* __restrict__ z, Strides3 sz,
     const float* __restrict__ dt, const float* __restrict__ dA_cs, const T* __restrict__ Cm, Strides3 sC,
     const TS* __restrict__ prev, const float* __restrict__ D, int d_has_hdim, T* __restrict__ out,
     Strides3 so, T* __restrict__ out_x, int nh, int heads_per_group, int ngroups, int L, int Q, int C,
     int stiles, SeqIdx seq) {
-  using S = WideSmem<T, P, N>;
-  constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, PB = P / 32, ST = S::ST;
+  constexpr int PW = P * HP;  // width of the tile of x, z and out
+  using S = WideSmem<T, PW, N>;
+  constexpr int EPL = Vec16<T>::N, KG = Tile<T>::KG, PB = PW / 32, PBH = P / 32, ST = S::ST;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* Xs = reinterpret_cast<T*>(smem);
   T* Pv = reinterpret_cast<T*>(smem);
   float* Os = reinterpret_cast<float*>(smem);
-  float* dAk = reinterpret_cast<float*>(smem + S::kMain);
-  float* dtk = dAk + ST;
-  float* sm = dtk + ST;  // exp(dA_m) of the carried-state term, then
-  float* fk = sm;        // the per-position factor of the causal term
+  float* vec = reinterpret_cast<float*>(smem + S::kMain);  // per head: dA_k, dt_k, exp(dA_m) / factor
+  auto dAk = [&](int hh) { return vec + (3 * hh) * ST; };
+  auto dtk = [&](int hh) { return vec + (3 * hh + 1) * ST; };
+  auto sm = [&](int hh) { return vec + (3 * hh + 2) * ST; };  // exp(dA_m) of the carried-state term, then
+  auto fk = [&](int hh) { return vec + (3 * hh + 2) * ST; };  // the per-position factor of the causal term
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31, half = lane >> 5;
   const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
+  const int nhp = nh / HP;
   const int st = bid % stiles;
-  const int h = (bid / stiles) % nh;
-  const int c = (bid / (stiles * nh)) % C;
-  const int64_t b = bid / ((int64_t)stiles * nh * C);
+  const int h = ((bid / stiles) % nhp) * HP;  // first head of the workgroup
+  const int c = (bid / (stiles * nhp)) % C;
+  const int64_t b = bid / ((int64_t)stiles * nhp * C);
   const int limit = min(Q, L - c * Q);
   const int m0 = ST * st;
   if (m0 >= limit) return;
   const int g = h / heads_per_group;
-  const int64_t chunk = (b * nh + h) * C + c;
-  const float* dAp = dA_cs + chunk * Q;
-  const float* dtp = dt + chunk * Q;
+  const float* dAp[HP];
+  const float* dtp[HP];
+#pragma unroll
+  for (int hh = 0; hh < HP; ++hh) {
+    const int64_t chunk = (b * nh + h + hh) * C + c;
+    dAp[hh] = dA_cs + chunk * Q;
+    dtp[hh] = dt + chunk * Q;
+  }
   const T* xg = x + b * sx.sb + (int64_t)c * Q * sx.sl + h * sx.sh;
   const T* Cg = Cm + b * sC.sb + (int64_t)c * Q * sC.sl + g * sC.sh;
   const TS* pg = prev + (((b * C + c) * nh + h) * (int64_t)P) * N;
@@ -1114,7 +1129,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
   {
     constexpr int VPR = N / 4;
 #pragma unroll
-    for (int i = 0; i < P * VPR / 256; ++i) {
+    for (int i = 0; i < PW * VPR / 256; ++i) {
       const int idx = tid + 256 * i;
       const int r = idx / VPR, cv = (idx % VPR) * 4;
       const float4 v = state_load4<true>(pg + (int64_t)r * N + cv);
@@ -1125,7 +1140,8 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
   {
     const ChunkSeq sq = chunk_seq(seq, b, c, Q);
     const bool live = !sq.on() || sq.at(min(m0 + tid, limit - 1)) == sq.entering(c);
-    sm[tid] = live ? __expf(dAp[m0 + tid]) : 0.f;
+#pragma unroll
+    for (int hh = 0; hh < HP; ++hh) sm(hh)[tid] = live ? __expf(dAp[hh][m0 + tid]) : 0.f;
   }
   __syncthreads();
   SSD_TSTAMP(1);
@@ -1141,11 +1157,13 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
       for (int pb = 0; pb < PB; ++pb) mma_group(a, frag_rows(Pv, S::PC, 32 * pb, kk, lane), acc[mb][pb]);
     }
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const float sc = sm[mrow[mb] + acc_row(v, lane)];
+    for (int hh = 0; hh < HP; ++hh)
 #pragma unroll
-      for (int pb = 0; pb < PB; ++pb) acc[mb][pb][v] *= sc;
-    }
+      for (int v = 0; v < 16; ++v) {
+        const float sc = sm(hh)[mrow[mb] + acc_row(v, lane)];
+#pragma unroll
+        for (int pb = hh * PBH; pb < (hh + 1) * PBH; ++pb) acc[mb][pb][v] *= sc;
+      }
   }
 
   // ---- phase B: the k super-tiles up to the diagonal one
@@ -1154,17 +1172,18 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
   SSD_TSTAMP(3);
   for (int kt = 0; kt <= st; ++kt) {
     const int k0 = ST * kt;
-    stage_rows<T, ST, P, NoScale, true>(Xs, xg, sx.sl, k0, limit, tid, NoScale());
-    {
+    stage_rows<T, ST, PW, NoScale, true>(Xs, xg, sx.sl, k0, limit, tid, NoScale());
+#pragma unroll
+    for (int hh = 0; hh < HP; ++hh) {
       // Below the diagonal the weight of (m, k) is split at the last position r of k's group of
       // 32: exp(dA_m - dA_r) is one exponential per row and group, exp(dA_r - dA_k) * dt_k one
       // per position k, shared by all rows.  Each exponent is clamped at 0 like the whole is in
       // the reference; for a dA_cumsum that is monotone inside the chunk (A of one sign,
       // dt >= 0) the product is the reference's clamped exponential.
-      const float ak = dAp[k0 + tid], ar = dAp[k0 + (tid | 31)], tk = dtp[k0 + tid];
-      dAk[tid] = ak;
-      dtk[tid] = tk;
-      fk[tid] = __expf(fminf(ar - ak, 0.f)) * tk;
+      const float ak = dAp[hh][k0 + tid], ar = dAp[hh][k0 + (tid | 31)], tk = dtp[hh][k0 + tid];
+      dAk(hh)[tid] = ak;
+      dtk(hh)[tid] = tk;
+      fk(hh)[tid] = __expf(fminf(ar - ak, 0.f)) * tk;
     }
     __syncthreads();
     SSD_TSTAMP(4);
@@ -1172,13 +1191,15 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) {
       const int mloc = mrow[mb] + l32;  // row inside the super-tile
-      const float am = dAp[m0 + mloc];
+      float am[HP];
+#pragma unroll
+      for (int hh = 0; hh < HP; ++hh) am[hh] = dAp[hh][m0 + mloc];
       const float* cbrow = cbg + (int64_t)(m0 + mloc) * Q + k0 + EPL * half;
       const int kend = diag ? mrow[mb] + 32 : ST;
       // NS steps at a time (the step count is even): their cb fragments are all requested before
       // the first is used, so the wave waits for memory once per NS steps.  Only where the
       // registers allow it without losing a wave per SIMD.
-      constexpr int NS = (P == 64 && sizeof(T) == 2) ? 2 : 1;
+      constexpr int NS = (PW == 64 && sizeof(T) == 2) ? 2 : 1;
       for (int kk0 = 0; kk0 < kend; kk0 += NS * KG) {
         float w[NS][EPL];
 #pragma unroll
@@ -1191,32 +1212,36 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
         // the group of 32 positions that holds the diagonal takes the exact, masked form
         const int grp_last = (kk0 & ~31) + 31;
         const bool exact = diag && grp_last >= mrow[mb];
-        const float gm = __expf(fminf(am - dAk[grp_last], 0.f));
 #pragma unroll
-        for (int u = 0; u < NS; ++u) {
-          const int kk = kk0 + KG * u, kb = kk + EPL * half;
-          Vec16<T> a;
-          float wf[EPL];
-          if (exact) {
+        for (int hh = 0; hh < HP; ++hh) {
+          const float gm = __expf(fminf(am[hh] - dAk(hh)[grp_last], 0.f));
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) {
-              const float f = w[u][e] * __expf(fminf(am - dAk[kb + e], 0.f)) * dtk[kb + e];
-              wf[e] = kb + e > mloc ? 0.f : f;
+          for (int u = 0; u < NS; ++u) {
+            const int kk = kk0 + KG * u, kb = kk + EPL * half;
+            Vec16<T> a;
+            float wf[EPL];
+            if (exact) {
+#pragma unroll
+              for (int e = 0; e < EPL; ++e) {
+                const float f = w[u][e] * __expf(fminf(am[hh] - dAk(hh)[kb + e], 0.f)) * dtk(hh)[kb + e];
+                wf[e] = kb + e > mloc ? 0.f : f;
+              }
+            } else {
+#pragma unroll
+              for (int e = 0; e < EPL; ++e) wf[e] = w[u][e] * fk(hh)[kb + e] * gm;
             }
-          } else {
+            a.set_all(wf);
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) wf[e] = w[u][e] * fk[kb + e] * gm;
+            for (int pb = hh * PBH; pb < (hh + 1) * PBH; ++pb)
+              mma_group(a, frag_cols(Xs, S::PX, kk, 32 * pb, lane), acc[mb][pb]);
           }
-          a.set_all(wf);
-#pragma unroll
-          for (int pb = 0; pb < PB; ++pb) mma_group(a, frag_cols(Xs, S::PX, kk, 32 * pb, lane), acc[mb][pb]);
         }
       }
       if (diag && D) {
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) {
-          const int col = 32 * pb + l32;
-          const float dv = d_has_hdim ? D[h * P + col] : D[h];
+          const int col = 32 * pb + l32;  // column of the tile = feature of head h + col / P
+          const float dv = d_has_hdim ? D[h * P + col] : D[h + pb / PBH];
 #pragma unroll
           for (int v = 0; v < 16; ++v)
             acc[mb][pb][v] = fmaf(dv, (float)Xs[(mrow[mb] + acc_row(v, lane)) * S::PX + col], acc[mb][pb][v]);
@@ -1230,7 +1255,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
 
   // ---- phase C: each wave moves its two blocks through its own staging area
   float* mine = Os + wave * 32 * S::PO;
-  constexpr int VPR = P / EPL;
+  constexpr int VPR = PW / EPL;
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {
 #pragma unroll
