@@ -1642,6 +1642,7 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
   T* Pv = reinterpret_cast<T*>(smem);
   float* Os = reinterpret_cast<float*>(smem);
   float* dAk = reinterpret_cast<float*>(smem + S::kMain);
+  float* fk = dAk + ST;  // per-position factor of the weights past the diagonal
   float* sm = dAk + 2 * ST;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31, half = lane >> 5;
@@ -1727,7 +1728,16 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
   for (int kt = st; kt < stiles && ST * kt < limit; ++kt) {
     const int k0 = ST * kt;
     stage_rows<T, ST, P>(Ds, dg, sd.sl, k0, limit, tid, NoScale());
-    dAk[tid] = dAp[k0 + tid];
+    {
+      // Past the diagonal the weight of (m, k) is split at the first position r of k's group of
+      // 32: exp(dA_k - dA_r) is one exponential per position k, shared by all rows, and
+      // exp(dA_r - dA_m) one per row and group.  Each exponent is clamped at 0 like the whole is
+      // in the reference; for a dA_cumsum that is monotone inside the chunk the product is the
+      // reference's clamped exponential.  Positions past the end of the sequence get factor 0.
+      const float ak = dAp[k0 + tid], ar = dAp[k0 + (tid & ~31)];
+      dAk[tid] = ak;
+      fk[tid] = k0 + tid < limit ? __expf(fminf(ak - ar, 0.f)) : 0.f;
+    }
     __syncthreads();
     SSD_TSTAMP(4);
     const bool diag = kt == st;
@@ -1736,22 +1746,40 @@ __global__ __launch_bounds__(256, (P == 64 ? 3 : 2)) void ssd_chunk_scan_bwd_dx_
       const int mloc = mrow[mb] + l32;
       const float am = dAp[m0 + mloc];
       const float* cbcol = cbg + (int64_t)k0 * Q + m0 + mloc;  // cb[k0 + k][m]: stride Q along k
-      for (int kk = diag ? mrow[mb] : 0; kk < ST; kk += KG) {
-        const int kb = kk + EPL * half;
-        float w[EPL];
+      // NS steps at a time (the step count is even): their cb pieces are all requested before the
+      // first is used, so the wave waits for memory once per NS steps.  Only where the registers
+      // allow it.
+      constexpr int NS = (P == 64 && sizeof(T) == 2) ? 2 : 1;
+      for (int kk0 = diag ? mrow[mb] : 0; kk0 < ST; kk0 += NS * KG) {
+        float w[NS][EPL];
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) w[e] = cbcol[(int64_t)(kb + e) * Q];
-        Vec16<T> a;
-        float wf[EPL];
+        for (int u = 0; u < NS; ++u)
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) {
-          const int k = kb + e;
-          const float f = w[e] * __expf(fminf(dAk[k] - am, 0.f));
-          wf[e] = ((diag && k < mloc) || k0 + k >= limit) ? 0.f : f;
+          for (int e = 0; e < EPL; ++e) w[u][e] = cbcol[(int64_t)(kk0 + KG * u + EPL * half + e) * Q];
+        // the group of 32 positions that holds the diagonal takes the exact, masked form
+        const int grp_first = kk0 & ~31;
+        const bool exact = diag && grp_first <= mrow[mb] + 31;
+        const float gm = __expf(fminf(dAk[grp_first] - am, 0.f));
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+          const int kk = kk0 + KG * u, kb = kk + EPL * half;
+          Vec16<T> a;
+          float wf[EPL];
+          if (exact) {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+              const int k = kb + e;
+              const float f = w[u][e] * __expf(fminf(dAk[k] - am, 0.f));
+              wf[e] = (k < mloc || k0 + k >= limit) ? 0.f : f;
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) wf[e] = w[u][e] * fk[kb + e] * gm;
+          }
+          a.set_all(wf);
+#pragma unroll
+          for (int pb = 0; pb < PB; ++pb) mma_group(a, frag_cols(Ds, S::PX, kk, 32 * pb, lane), acc[mb][pb]);
         }
-        a.set_all(wf);
-#pragma unroll
-        for (int pb = 0; pb < PB; ++pb) mma_group(a, frag_cols(Ds, S::PX, kk, 32 * pb, lane), acc[mb][pb]);
       }
     }
     SSD_TSTAMP(5);
