@@ -32,7 +32,7 @@ TRAFFIC_BYTES = {"fwd_single_pass": 589083033, "bwd_single_pass": 841025145}
 SSD_TRAFFIC_BYTES = {
     "chunk_cumsum": 25320408, "chunk_state": 571591572, "state_passing": 419465499, "bmm_chunk": 100772767,
     "chunk_scan": 742930943, "bwd_dstates": 446640967, "bwd_state_passing": 409601722, "bwd_db": 496071800,
-    "bwd_dc": 469831534, "bwd_dx": 1020235822, "bwd_ddAcs": 599926788,
+    "bwd_dc": 469831534, "bwd_dx": 1029628081, "bwd_ddAcs": 599926788,
 }
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
