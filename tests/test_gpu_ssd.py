@@ -26,6 +26,8 @@ CASES = [
     (1, 130, 2, 128, 2, 128, 64),
     (1, 900, 2, 64, 1, 64, 512),    # two 256-row super-tiles per chunk, the last chunk ragged
     (1, 512, 2, 128, 2, 128, 256),
+    (1, 300, 3, 64, 1, 128, 256),   # an odd number of heads per group: one head per workgroup
+    (1, 512, 6, 64, 2, 64, 256),
     (1, 150, 2, 64, 1, 64, 48),     # chunk sizes that are no multiple of the 64-row tiles
     (1, 333, 2, 64, 2, 64, 200),
     (1, 1100, 2, 64, 1, 128, 1024),  # the largest chunk size, second chunk ragged
@@ -124,6 +126,42 @@ def test_combined_vs_recurrence(b, L, nh, P, g, N, Q, dtype, device):
         check_close("final states, same", fin, fin_rnd, BF16)
     check_close("y", y, y_ref, dtype, loose=True)
     check_close("final states", fin, fin_ref, F32 if dtype == F32 else BF16, loose=True)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+def test_views_of_a_fused_projection(dtype, device):
+    """x, B, C and z as a Mamba-2 layer holds them: slices of one projected tensor, so the position
+    stride exceeds nheads * hdim while the heads stay dense (the chunk scan then pairs heads), and
+    x with every other head of a wider tensor (head stride 2 * hdim: one head per workgroup).
+    Strides only change addresses, so the results must equal those of contiguous copies."""
+    from kernels.mamba_kernels.mamba_combined_fwd import mamba_chunk_scan_combined_fwd
+
+    b, L, nh, P, g, N, Q = 2, 520, 4, 64, 1, 128, 256
+    announce(f"ssd strided views b{b} L{L} nh{nh} P{P} g{g} N{N} Q{Q} {dtype}")
+    x, dt, A, B, C, D, z = S.make_inputs(b, L, nh, P, g, N, seed=99, dtype=dtype, with_z=True)
+    xd, dtd, Ad, Bd, Cd, Dd, zd = _dev(device, x, dt, A, B, C, D, z)
+    y0, fin0 = mamba_chunk_scan_combined_fwd(xd, dtd, Ad, Bd, Cd, Q, D=Dd, z=zd, return_final_states=True)
+
+    d_in = nh * P
+    zxbc = torch.zeros(b, L, 2 * d_in + 2 * g * N + 8, device=device, dtype=dtype)
+    zxbc[..., :d_in] = zd.reshape(b, L, d_in)
+    zxbc[..., d_in:2 * d_in] = xd.reshape(b, L, d_in)
+    zxbc[..., 2 * d_in:2 * d_in + g * N] = Bd.reshape(b, L, g * N)
+    zxbc[..., 2 * d_in + g * N:2 * d_in + 2 * g * N] = Cd.reshape(b, L, g * N)
+    zv = zxbc[..., :d_in].unflatten(-1, (nh, P))
+    xv = zxbc[..., d_in:2 * d_in].unflatten(-1, (nh, P))
+    Bv = zxbc[..., 2 * d_in:2 * d_in + g * N].unflatten(-1, (g, N))
+    Cv = zxbc[..., 2 * d_in + g * N:2 * d_in + 2 * g * N].unflatten(-1, (g, N))
+    assert not xv.is_contiguous() and xv.stride(2) == P
+    y1, fin1 = mamba_chunk_scan_combined_fwd(xv, dtd, Ad, Bv, Cv, Q, D=Dd, z=zv, return_final_states=True)
+    assert torch.equal(y1, y0) and torch.equal(fin1, fin0)
+
+    wide = torch.zeros(b, L, 2 * nh, P, device=device, dtype=dtype)
+    wide[:, :, ::2] = xd
+    xs = wide[:, :, ::2]
+    assert xs.stride(2) == 2 * P
+    y2, fin2 = mamba_chunk_scan_combined_fwd(xs, dtd, Ad, Bd, Cd, Q, D=Dd, z=zd, return_final_states=True)
+    assert torch.equal(y2, y0) and torch.equal(fin2, fin0)
 
 
 def test_unsupported_shapes_are_refused(device):
