@@ -170,6 +170,50 @@ def test_ddAcs_vs_oracle(b, L, nh, P, g, N, Q, dtype, device):
     check_close("ddA_cumsum (causal term)", got, ref, dtype, loose=dtype == BF16)
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+def test_backward_stages_on_views(dtype, device):
+    """x, B, C as slices of one projected tensor and dout as a slice of a wider gradient: the
+    position strides exceed the dense ones.  Strides only change addresses, so every backward
+    launcher must return exactly what it returns for contiguous copies."""
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_bwd_da import _chunk_scan_bwd_ddAcs_stable
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_bwd_dc import _chunk_scan_bwd_dC
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_chunk_state_bwd_dx import _chunk_scan_chunk_state_bwd_dx
+    from kernels.mamba_kernels_bwd.mamba_chunk_state_bwd_db import _chunk_state_bwd_db
+    from kernels.mamba_kernels_bwd.mamba_scan_bwd import _chunk_scan_bwd_dstates
+
+    b, L, nh, P, g, N, Q = 2, 520, 4, 64, 2, 128, 256
+    announce(f"ssd bwd on views b{b} L{L} nh{nh} P{P} g{g} N{N} Q{Q} {dtype}")
+    x, dt, dA_cs, B, C, D, dout, prev, dstates = [t.to(device) for t in _inputs(b, L, nh, P, g, N, Q, dtype)]
+    cb = S.bmm_chunk(C.cpu(), B.cpu(), Q).to(device)
+    d_in = nh * P
+    xbc = torch.zeros(b, L, d_in + 2 * g * N + 8, device=device, dtype=dtype)
+    xbc[..., :d_in] = x.reshape(b, L, d_in)
+    xbc[..., d_in:d_in + g * N] = B.reshape(b, L, g * N)
+    xbc[..., d_in + g * N:d_in + 2 * g * N] = C.reshape(b, L, g * N)
+    xv = xbc[..., :d_in].unflatten(-1, (nh, P))
+    Bv = xbc[..., d_in:d_in + g * N].unflatten(-1, (g, N))
+    Cv = xbc[..., d_in + g * N:d_in + 2 * g * N].unflatten(-1, (g, N))
+    dwide = torch.zeros(b, L, 2 * d_in, device=device, dtype=dtype)
+    dwide[..., d_in:] = dout.reshape(b, L, d_in)
+    dv = dwide[..., d_in:].unflatten(-1, (nh, P))
+    assert not xv.is_contiguous() and not dv.is_contiguous()
+
+    def same(name, got, want):
+        got = got if isinstance(got, tuple) else (got,)
+        want = want if isinstance(want, tuple) else (want,)
+        for i, (a, w) in enumerate(zip(got, want)):
+            assert (a is None and w is None) or torch.equal(a, w), f"{name}[{i}] differs on views"
+
+    same("dstates", _chunk_scan_bwd_dstates(Cv, dA_cs, dv), _chunk_scan_bwd_dstates(C, dA_cs, dout))
+    same("dB", _chunk_state_bwd_db(xv, dt, dA_cs, dstates, B=Bv, ngroups=g),
+         _chunk_state_bwd_db(x, dt, dA_cs, dstates, B=B, ngroups=g))
+    same("dC", _chunk_scan_bwd_dC(prev, dA_cs, dv, C=Cv, ngroups=g),
+         _chunk_scan_bwd_dC(prev, dA_cs, dout, C=C, ngroups=g))
+    same("dx", _chunk_scan_chunk_state_bwd_dx(xv, dt, dA_cs, Bv, cb, dv, dstates, D=D),
+         _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cs, B, cb, dout, dstates, D=D))
+    same("ddA", _chunk_scan_bwd_ddAcs_stable(xv, dt, dA_cs, dv, cb), _chunk_scan_bwd_ddAcs_stable(x, dt, dA_cs, dout, cb))
+
+
 def test_config5_backward_stages_full_size(device):
     """b8 nh32 hdim64 dstate128 g1 L8192 Q256 bf16: every backward launcher runs on the whole
     workload; batch element 0 of each result is compared with the oracle."""
