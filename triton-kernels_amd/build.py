@@ -1,28 +1,27 @@
 """Builds lib/libema_hip.so (gfx950) from csrc/ with hipcc: the EMA scan (ema_abi.hip) and the
-SSD forward stages (ssd_abi.hip).  Usage: python build.py"""
+SSD stages (ssd_abi.hip).  The translation units are compiled side by side and then linked.
+Usage: python build.py"""
 import os
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SRC = [os.path.join(HERE, "csrc", "ema_abi.hip"), os.path.join(HERE, "csrc", "ssd_abi.hip")]
 OUT = os.path.join(HERE, "lib", "libema_hip.so")
+OBJ_DIR = os.path.join(HERE, "build")
 
 FLAGS = [
     "-O3",
     "-std=c++17",
     "--offload-arch=gfx950",
-    "-shared",
     "-fPIC",
     # packed FP32 VALU ops are kept off for every HIP translation unit of this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 
 
-def build(verbose: bool = True) -> str:
-    os.makedirs(os.path.dirname(OUT), exist_ok=True)
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + FLAGS + ["-o", OUT] + SRC
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -31,10 +30,22 @@ def build(verbose: bool = True) -> str:
     )
     if res.returncode != 0:
         sys.stderr.write(err + "\n")
-        raise RuntimeError("hipcc failed")
+        raise RuntimeError("hipcc failed: " + " ".join(cmd))
     if verbose and err.strip():
         print(err)
-    return OUT
+
+
+def build(verbose: bool = True, extra_flags=(), out: str = OUT) -> str:
+    os.makedirs(os.path.dirname(out), exist_ok=True)
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    tag = os.path.splitext(os.path.basename(out))[0]
+    objs = [os.path.join(OBJ_DIR, tag + "_" + os.path.basename(s) + ".o") for s in SRC]
+    with ThreadPoolExecutor(len(SRC)) as pool:
+        list(pool.map(lambda so: _run([hipcc] + FLAGS + list(extra_flags) + ["-c", so[0], "-o", so[1]], verbose),
+                      zip(SRC, objs)))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs, verbose)
+    return out
 
 
 if __name__ == "__main__":
