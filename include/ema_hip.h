@@ -45,7 +45,8 @@ typedef enum {
   EMA_ERR_ALIGN = -3,       /* dim / strides / pointers break the 16-byte rule */
   EMA_ERR_DTYPE = -4,       /* unknown ema_dtype */
   EMA_ERR_UNSUPPORTED = -5, /* a feature the reference also rejects */
-  EMA_ERR_LAUNCH = -6       /* hipGetLastError() after a launch was not hipSuccess */
+  EMA_ERR_LAUNCH = -6,      /* hipGetLastError() after a launch was not hipSuccess */
+  EMA_ERR_TOO_LARGE = -7    /* the problem needs more than the fixed scratch of ema_seq_fwd_static */
 } ema_status;
 
 typedef enum { EMA_F32 = 0, EMA_BF16 = 1 } ema_dtype;
@@ -281,6 +282,33 @@ int ema_seq_bwd(int form, const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t 
                 float* dinit, void* workspace, size_t workspace_bytes, int workspace_prepared,
                 int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
                 void* ev_stop);
+
+/* ------------------------------------------- entry point that allocates nothing ---- */
+
+/* Size of the file-scope device array that ema_seq_fwd_static works in. */
+#define EMA_STATIC_SCRATCH_BYTES (16u << 20)
+size_t ema_seq_fwd_static_max_workspace_bytes(void);
+
+/* ema_seq_fwd without a workspace argument.  This entry point has no counterpart in the
+ * reference; it is for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The status words of the
+ * chained scan and the other scratch that ema_seq_fwd takes as `workspace` live in a
+ * file-scope device array of EMA_STATIC_SCRATCH_BYTES bytes (one copy per GPU, held until
+ * the process ends); the call performs no allocation of any kind, on the device or through a
+ * library.  Inputs and outputs are the caller's, with the meaning they have in ema_seq_fwd
+ * (prev128 required, init and final_state may be NULL); there is no bwd_workspace and there
+ * are no timing events.  Problems whose ema_seq_fwd_workspace_bytes(...) exceeds
+ * EMA_STATIC_SCRATCH_BYTES are rejected with EMA_ERR_TOO_LARGE before anything is launched
+ * (the b16 nh2 L4096 d1024 problem needs 8.9 MiB).  All calls on one GPU share that GPU's array:
+ * every call clears what it needs cleared itself, so calls may follow each other on one stream
+ * in any order of shapes, but calls that overlap in time on one GPU (different streams or
+ * threads) race and must be serialised by the caller.  The current device must be the one
+ * `stream` belongs to. */
+int ema_seq_fwd_static(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t c_sh,
+                       const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y,
+                       int64_t y_sb, int64_t y_sl, int64_t y_sh, const float* init,
+                       float* final_state, float* prev128, int64_t batch, int64_t nheads,
+                       int64_t seqlen, int64_t dim, void* stream);
 
 #ifdef __cplusplus
 }

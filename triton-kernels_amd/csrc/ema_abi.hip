@@ -5,6 +5,8 @@
 #include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "ema_device.h"
 #include "ema_gemm_kernels.h"
 #include "ema_stream_kernels.h"
@@ -450,6 +452,31 @@ SeqWs carve_seq(void* base, const Dims& di, bool backward) {
   return w;
 }
 
+// ---------------------------------------------------------------- file-scope scratch
+// Workspace of ema_seq_fwd_static: one copy per GPU that loads the library, held until the
+// process ends.  In host code the array's name is only a handle for hipGetSymbolAddress; the
+// address the kernels get is looked up once per device and kept.
+constexpr size_t kScratchBytes = EMA_STATIC_SCRATCH_BYTES;
+__device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device.
+int scratch_address(void** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return EMA_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return EMA_ERR_LAUNCH;
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return EMA_OK;
+}
+
 }  // namespace
 
 // ====================================================================================
@@ -467,6 +494,7 @@ const char* ema_status_string(int status) {
     case EMA_ERR_DTYPE: return "unknown dtype";
     case EMA_ERR_UNSUPPORTED: return "unsupported";
     case EMA_ERR_LAUNCH: return "kernel launch failed";
+    case EMA_ERR_TOO_LARGE: return "problem exceeds the fixed scratch of the allocation-free entry point";
     default: return "unknown status";
   }
 }
@@ -837,7 +865,7 @@ size_t ema_seq_fwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen
   return carve_seq(nullptr, d, false).bytes;
 }
 
-int ema_seq_fwd(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t c_sh, const void* x,
+static int seq_fwd_impl(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t c_sh, const void* x,
                 int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb,
                 int64_t y_sl, int64_t y_sh, const float* init, float* final_state, float* prev128,
                 void* workspace, size_t workspace_bytes, void* bwd_workspace, size_t bwd_workspace_bytes,
@@ -879,6 +907,35 @@ int ema_seq_fwd(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t
   return launch_fwd_tile_t<float, TileF32, false>(x, sx, coef, sc, w.cs, y, sy, prev128, nullptr, 1,
                                                   final_state, init, w.chain, d, st, ev_start, ev_stop, nc,
         bw.cs);
+}
+
+int ema_seq_fwd(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t c_sh, const void* x,
+                int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb,
+                int64_t y_sl, int64_t y_sh, const float* init, float* final_state, float* prev128,
+                void* workspace, size_t workspace_bytes, void* bwd_workspace, size_t bwd_workspace_bytes,
+                int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
+                void* ev_stop) {
+  return seq_fwd_impl(form, coef, c_sb, c_sl, c_sh, x, x_sb, x_sl, x_sh, dtype, y, y_sb, y_sl, y_sh, init,
+                      final_state, prev128, workspace, workspace_bytes, bwd_workspace, bwd_workspace_bytes,
+                      batch, nheads, seqlen, dim, stream, ev_start, ev_stop);
+}
+
+// ---- the entry point that allocates nothing: ema_seq_fwd with its workspace in a file-scope array
+
+size_t ema_seq_fwd_static_max_workspace_bytes(void) { return kScratchBytes; }
+
+int ema_seq_fwd_static(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t c_sh, const void* x,
+                       int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb,
+                       int64_t y_sl, int64_t y_sh, const float* init, float* final_state, float* prev128,
+                       int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim, void* stream) {
+  const size_t need = ema_seq_fwd_workspace_bytes(batch, nheads, seqlen, dim);
+  if (need == 0) return EMA_ERR_SHAPE;
+  if (need > kScratchBytes) return EMA_ERR_TOO_LARGE;
+  void* ws = nullptr;
+  EMA_TRY(scratch_address(&ws));
+  return seq_fwd_impl(form, coef, c_sb, c_sl, c_sh, x, x_sb, x_sl, x_sh, dtype, y, y_sb, y_sl, y_sh, init,
+                      final_state, prev128, ws, kScratchBytes, nullptr, 0, batch, nheads, seqlen, dim, stream,
+                      nullptr, nullptr);
 }
 
 size_t ema_seq_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim) {

@@ -48,6 +48,8 @@ _SIGNATURES = {
     "ema_seq_bwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "ema_seq_fwd": (c_int, [c_int] + _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, c_size_t, _P, c_size_t, _I, _I, _I, _I, _P, _P, _P]),
     "ema_seq_bwd": (c_int, [c_int] + _SEQ + _SEQ + _SEQ + [_P, _P, c_int] + _SEQ + _SEQ + [_P, _P, c_size_t, c_int, _I, _I, _I, _I, _P, _P, _P]),
+    "ema_seq_fwd_static_max_workspace_bytes": (c_size_t, []),
+    "ema_seq_fwd_static": (c_int, [c_int] + _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _I, _I, _I, _I, _P]),
     # SSD forward stages (include/ssd_hip.h)
     "ssd_chunk_cumsum_fwd": (c_int, [_P, c_int, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, c_int, c_float, c_float, _P]),
     "ssd_chunk_state_fwd": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
@@ -100,6 +102,7 @@ _ERRORS = {
     -4: (TypeError, "unsupported dtype"),
     -5: (NotImplementedError, "unsupported"),
     -6: (RuntimeError, "kernel launch failed"),
+    -7: (ValueError, "problem exceeds the fixed scratch of the allocation-free entry point"),
 }
 
 
