@@ -27,6 +27,21 @@
  *     be 16-byte aligned.
  *   - Return value: EMA_OK (0) or a negative ema_status.  Arguments are validated before
  *     anything is launched; nothing is thrown across the boundary.
+ *   - Workspaces of the single-pass entry points (ema_fwd, ema_bwd, ema_seq_fwd, ema_seq_bwd)
+ *     begin with an ema_chain_header followed by the words through which the tiles of the
+ *     chained scan hand their state to each other (the chained part); per-call scratch follows.
+ *     Every word of the chained part is tagged with the epoch of the call that wrote it, so
+ *     nothing has to be cleared between calls: a buffer that was zero-filled once
+ *     (ema_workspace_clear, or any memset) serves any number of calls of these four entry points
+ *     on one problem shape (batch * nheads, seqlen, dim), forward and backward alike, one after
+ *     the other.  Pass workspace_ready = 1 for such a buffer and the call launches no clearing
+ *     kernel; with workspace_ready = 0 the call first clears the chained part (one more small
+ *     launch), which is right for a buffer of unknown contents.  A ready buffer must have held
+ *     nothing but this library's words since it was cleared (the tags are compared as plain
+ *     words); ema_seq_fwd, whose workspace is the chained part alone, may change shape from
+ *     call to call on one buffer.  Calls that share a workspace must not overlap in time.  A
+ *     buffer must be cleared again after 2^30 calls, and after a call that was aborted or that
+ *     the header's error word reports.
  */
 #ifndef EMA_HIP_H
 #define EMA_HIP_H
@@ -56,6 +71,28 @@ typedef enum {
   EMA_FORM_LOG_DECAY = 0,  /* A:  y[t] = exp(min(A[t], 0)) * y[t-1] + x[t]           */
   EMA_FORM_PROBABILITY = 1 /* p:  y[t] = (1 - p[t]) * y[t-1] + p[t] * x[t]           */
 } ema_form;
+
+/* What a workspace of the single-pass entry points begins with (256 bytes, device memory).  The
+ * library maintains it; a caller may read `error` (for instance together with the results) and
+ * may set `spin_limit` between calls.
+ *   error      non-zero once a tile's bounded wait for its predecessor has run out in some call
+ *              since the buffer was last cleared (a predecessor that never published: a
+ *              workspace that was not ready, overlapping calls on one workspace, or a device so
+ *              oversubscribed that resident workgroups stopped making progress).  The affected
+ *              outputs are NaN; the call itself still returns EMA_OK, since nothing is read back.
+ *   spin_limit polls of one word before a wait gives up; 0 = the built-in 2^20. */
+typedef struct {
+  uint32_t ticket;     /* next tile to hand out; zero between calls */
+  uint32_t done;       /* workgroups that have left the running call; zero between calls */
+  uint32_t epoch;      /* epoch of the last completed call */
+  uint32_t error;
+  uint32_t spin_limit;
+  uint32_t reserved[59];
+} ema_chain_header;
+
+/* Zero-fills `bytes` bytes of device memory at `workspace` (16-byte aligned) with a kernel on
+ * `stream`: the state in which workspace_ready = 1 may be passed. */
+int ema_workspace_clear(void* workspace, size_t bytes, void* stream);
 
 /* Largest chunk size accepted by every entry point. */
 #define EMA_MAX_CHUNK 1024
@@ -105,20 +142,15 @@ size_t ema_fwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, in
  * ema_bwd accepts to skip their recomputation.  For other chunk sizes F1..F4 run in
  * sequence and prev128 must be NULL.  ev_start / ev_stop (hipEvent_t, may be NULL) are
  * recorded on the stream right before and after the kernel(s) that read x, so that a
- * caller can time them apart from the small set-up kernels.
- * bwd_workspace (may be NULL; chunk a multiple of 128): the workspace of the ema_seq_bwd call
- * (log-decay form, same shape) that will follow this forward pass, at least
- * ema_seq_bwd_workspace_bytes(...) bytes.  The forward's set-up launch then also prepares it
- * (status words of the reverse scan, the cumsum of A), and that ema_seq_bwd call, told so by its
- * workspace_prepared argument, needs no set-up launch of its own.  The caller keeps the buffer
- * untouched in between; a prepared workspace serves one backward call.
+ * caller can time them apart from the small kernel that writes cs.  workspace_ready: see the
+ * conventions above (ignored when chunk is not a multiple of 128).
  * Replaces _ema_matmul_scan_combined_fwd, kernels/ema_kernels/ema_combined_fwd.py:12-45. */
 int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void* x,
             int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb,
             int64_t y_sl, int64_t y_sh, float* cs, float* prev, float* final_state,
-            float* prev128, void* workspace, size_t workspace_bytes, void* bwd_workspace,
-            size_t bwd_workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
-            int64_t chunk, void* stream, void* ev_start, void* ev_stop);
+            float* prev128, void* workspace, size_t workspace_bytes, int workspace_ready,
+            int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk, void* stream,
+            void* ev_start, void* ev_stop);
 
 /* --------------------------------------------------------------- backward stages ---- */
 
@@ -219,14 +251,15 @@ size_t ema_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, in
  * ddA[n,c,q] = dL/dA[n, c*Q+q] (0 in the slots past seqlen); when y is not NULL the forward
  * output is recomputed into it (the reference's recompute_output=True).  ev_start / ev_stop
  * (hipEvent_t, may be NULL) are recorded right before and after the single-pass kernel.
+ * workspace_ready: see the conventions above.
  * Replaces _ema_chunk_scan_combined_bwd,
  * kernels/ema_kernels_bwd/ema_combined_bwd.py:13-83. */
 int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const void* x,
             int64_t x_sb, int64_t x_sl, int64_t x_sh, const float* A, int64_t a_sb,
             int64_t a_sl, int64_t a_sh, const float* prev128, int dtype, void* dx,
             int64_t dx_sb, int64_t dx_sl, int64_t dx_sh, float* ddA, void* y, int64_t y_sb,
-            int64_t y_sl, int64_t y_sh, void* workspace, size_t workspace_bytes, int64_t batch,
-            int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk, void* stream,
+            int64_t y_sl, int64_t y_sh, void* workspace, size_t workspace_bytes, int workspace_ready,
+            int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk, void* stream,
             void* ev_start, void* ev_stop);
 
 /* ------------------------------------------------- sequence-level entry points ---- */
@@ -251,14 +284,14 @@ size_t ema_seq_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen
  * (kernels/ema_kernels/ema_state_pass.py:129-130).  final_state (N,T), may be NULL: the state
  * after the last position.  prev128 (N, ceil(seqlen/128), T) float32, required: the state
  * entering each 128-row chunk, which ema_seq_bwd takes.  Chunking is internal; there is no
- * chunk argument.  ev_start / ev_stop and bwd_workspace (the workspace of the ema_seq_bwd call of
- * the same form and shape that will follow, prepared here; may be NULL) as for ema_fwd. */
+ * chunk argument.  ev_start / ev_stop and workspace_ready as for ema_fwd.  The call is one
+ * kernel launch when the workspace is ready. */
 int ema_seq_fwd(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t c_sh,
                 const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y,
                 int64_t y_sb, int64_t y_sl, int64_t y_sh, const float* init, float* final_state,
-                float* prev128, void* workspace, size_t workspace_bytes, void* bwd_workspace,
-                size_t bwd_workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
-                void* stream, void* ev_start, void* ev_stop);
+                float* prev128, void* workspace, size_t workspace_bytes, int workspace_ready,
+                int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim, void* stream,
+                void* ev_start, void* ev_stop);
 
 /* Backward of ema_seq_fwd in one pass over x and dy.  With r the reverse scan of dy,
  * r[t] = dy[t] + a[t+1] * r[t+1], started from dfinal (N,T) float32 (may be NULL = zero), the
@@ -270,16 +303,14 @@ int ema_seq_fwd(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t
  * (the reference leaves dP = -dA * exp(A) commented out, kernels/tests/ema_bwd/_ema_full_bwd.py:128-130,
  * and rearranges dA from (b,c,q) to (b,l) in torch, :71).  dcoef is float32 in the layout of
  * coef, given by its own strides; dinit (N,T) float32, may be NULL, receives a[0] * r[0], the
- * gradient of init.  prev128 is the forward's output of that name.  workspace_prepared: non-zero
- * if the forward pass was given this workspace as its bwd_workspace and nothing has written to it
- * since; the call then skips its set-up launch.  Only without dfinal (EMA_ERR_UNSUPPORTED
- * otherwise), and once per forward pass. */
+ * gradient of init.  prev128 is the forward's output of that name.  workspace_ready: see the
+ * conventions above; the same buffer may serve the forward and the backward call. */
 int ema_seq_bwd(int form, const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh,
                 const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, const float* coef,
                 int64_t c_sb, int64_t c_sl, int64_t c_sh, const float* prev128,
                 const float* dfinal, int dtype, void* dx, int64_t dx_sb, int64_t dx_sl,
                 int64_t dx_sh, float* dcoef, int64_t dc_sb, int64_t dc_sl, int64_t dc_sh,
-                float* dinit, void* workspace, size_t workspace_bytes, int workspace_prepared,
+                float* dinit, void* workspace, size_t workspace_bytes, int workspace_ready,
                 int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
                 void* ev_stop);
 
@@ -299,11 +330,12 @@ size_t ema_seq_fwd_static_max_workspace_bytes(void);
  * (prev128 required, init and final_state may be NULL); there is no bwd_workspace and there
  * are no timing events.  Problems whose ema_seq_fwd_workspace_bytes(...) exceeds
  * EMA_STATIC_SCRATCH_BYTES are rejected with EMA_ERR_TOO_LARGE before anything is launched
- * (the b16 nh2 L4096 d1024 problem needs 8.9 MiB).  All calls on one GPU share that GPU's array:
- * every call clears what it needs cleared itself, so calls may follow each other on one stream
- * in any order of shapes, but calls that overlap in time on one GPU (different streams or
- * threads) race and must be serialised by the caller.  The current device must be the one
- * `stream` belongs to. */
+ * (the b16 nh2 L4096 d1024 problem needs 8.3 MiB).  All calls on one GPU share that GPU's array,
+ * which keeps what the last call left in it: the array starts out zero-filled, every call leaves
+ * it ready for the next (epoch-tagged words, see the conventions above), so nothing has to be
+ * cleared and calls may follow each other on one stream in any order of shapes; calls that
+ * overlap in time on one GPU (different streams or threads) race and must be serialised by the
+ * caller.  The current device must be the one `stream` belongs to. */
 int ema_seq_fwd_static(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t c_sh,
                        const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y,
                        int64_t y_sb, int64_t y_sl, int64_t y_sh, const float* init,

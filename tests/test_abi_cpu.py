@@ -42,8 +42,12 @@ def test_status_strings():
 def test_workspace_sizes():
     handle = _lib.lib()
     # config 2: N=32, C=32, T=1024, Q=128
-    assert handle.ema_fwd_workspace_bytes(16, 2, 4096, 1024, 64) == 32 * 64 * 1024 * 4
-    assert handle.ema_fwd_workspace_bytes(16, 2, 4096, 1024, 128) > 32 * 32 * 1024 * 8
+    # header + one word per (sequence, 128-row tile) + one per (sequence, tile, column), then scratch
+    chain = 256 + 32 * 32 * 8 + 32 * 32 * 1024 * 8
+    assert handle.ema_seq_fwd_workspace_bytes(16, 2, 4096, 1024) == chain
+    assert handle.ema_fwd_workspace_bytes(16, 2, 4096, 1024, 64) == chain + 32 * 64 * 1024 * 4
+    assert handle.ema_fwd_workspace_bytes(16, 2, 4096, 1024, 128) == chain + 32 * 32 * 1024 * 4
+    assert handle.ema_seq_bwd_workspace_bytes(16, 2, 4096, 1024) == chain + 8 * 32 * 4096 * 4  # partials per 128 (float32) columns
     assert handle.ema_state_passing_bwd_workspace_bytes(32, 32, 1024) == 32 * 32 * 16 * 4
     assert handle.ema_chunk_scan_bwd_ddAcs_workspace_bytes(16, 2, 4096, 128) == 2 * 32 * 32 * 128 * 4
     assert handle.ema_bwd_workspace_bytes(16, 2, 4096, 1024, 128) > 4 * 32 * 32 * 1024 * 4
@@ -71,23 +75,33 @@ def test_validation_happens_before_any_launch():
     # workspace too small
     assert (
         handle.ema_fwd(fake, 8, 1, 0, fake, 64, 8, 0, _lib.EMA_F32, fake, 64, 8, 0, fake, fake, fake,
-                       None, fake, 16, None, 0, 1, 1, 8, 8, 4, None, None, None)
+                       None, fake, 16, 0, 1, 1, 8, 8, 4, None, None, None)
         == -2
     )
-    # a prepared backward workspace needs the single-pass forward (chunk a multiple of 128) ...
-    assert (
-        handle.ema_fwd(fake, 8, 1, 0, fake, 64, 8, 0, _lib.EMA_F32, fake, 64, 8, 0, fake, fake, fake,
-                       None, fake, 1 << 30, fake, 1 << 30, 1, 1, 8, 8, 4, None, None, None)
-        == -5
-    )
-    # ... and a backward pass that nothing enters through the final state
     seq = [fake, 64, 8, 0]
     coef = [fake, 8, 1, 0]
     assert (
-        handle.ema_seq_bwd(0, *seq, *seq, *coef, fake, fake, _lib.EMA_F32, *seq, *coef, None, fake, 1 << 30, 1,
+        handle.ema_seq_bwd(0, *seq, *seq, *coef, fake, None, _lib.EMA_F32, *seq, *coef, None, fake, 16, 1,
+                           1, 1, 8, 8, None, None, None)
+        == -2
+    )
+    # unknown form of the recurrence, misaligned workspace
+    assert (
+        handle.ema_seq_bwd(5, *seq, *seq, *coef, fake, None, _lib.EMA_F32, *seq, *coef, None, fake, 1 << 30, 1,
                            1, 1, 8, 8, None, None, None)
         == -5
     )
+    assert handle.ema_workspace_clear(fake + 4, 64, None) == -3
+    assert handle.ema_workspace_clear(None, 64, None) == -1
+
+
+def test_chain_header_layout():
+    # the header the library declares, the one the kernels use and the binding's view agree
+    src = open(HEADERS[0]).read()
+    body = src[src.index("typedef struct {"):src.index("} ema_chain_header;")]
+    fields = re.findall(r"uint32_t\s+(\w+)(?:\[(\d+)\])?;", body)
+    assert [f[0] for f in fields] == ["ticket", "done", "epoch", "error", "spin_limit", "reserved"]
+    assert 4 * (5 + int(fields[-1][1])) == _lib.HEADER_BYTES == 256
 
 
 def test_ssd_validation_happens_before_any_launch():

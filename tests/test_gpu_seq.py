@@ -239,15 +239,16 @@ def test_seq_packed_sequences_probability_form(dtype, device):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("form", ["log_decay", "probability"])
-def test_backward_workspace_prepared_by_forward(form, dtype, device):
-    """A forward pass can set up the workspace of the backward pass that follows in its own set-up
-    launch.  The backward then gives bit-identical results, a second backward on the same
-    workspace falls back to its own set-up, and so does one with a gradient entering through the
-    final state; the autograd entry points use the hand-over."""
+def test_workspace_ready_or_not(form, dtype, device):
+    """A call on a fresh buffer of unknown contents (workspace_ready = 0: the call clears what it
+    uses) and calls on one zero-filled buffer that forward and backward share call after call
+    (workspace_ready = 1: no clearing launch, words of earlier calls are told apart by their epoch)
+    give bit-identical results; so do the autograd entry points, which use the shared buffer."""
+    from kernels import _lib
     from kernels.ema_kernels.ema_combined_fwd import ema_matmul_scan_combined
     from kernels.ema_seq import ema_seq_bwd, ema_seq_fwd, ema_seq_scan
 
-    announce(f"prepared backward workspace {form} {dtype}")
+    announce(f"workspace ready / not ready {form} {dtype}")
     b, L, nh, d = 2, 700, 2, 320  # ragged last tile, two column tiles
     gen = torch.Generator().manual_seed(11)
     x = torch.randn(b, L, nh, d, generator=gen).to(dtype).to(device)
@@ -256,23 +257,29 @@ def test_backward_workspace_prepared_by_forward(form, dtype, device):
     coef = (p if form == "probability" else torch.log1p(-p)).to(device)
     dfin = torch.randn(b, nh, d, generator=gen).to(device)
 
-    y0, fin0, prev0 = ema_seq_fwd(coef, x, form)
-    y1, fin1, prev1, ws = ema_seq_fwd(coef, x, form, prepare_backward=True)
-    assert torch.equal(y0, y1) and torch.equal(fin0, fin1) and torch.equal(prev0, prev1)
-    ref = ema_seq_bwd(dy, x, coef, prev0, form)
-    assert ws.fresh
-    got = ema_seq_bwd(dy, x, coef, prev1, form, workspace=ws)
-    assert not ws.fresh
-    assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1])
-    again = ema_seq_bwd(dy, x, coef, prev1, form, workspace=ws)  # the workspace is used up: own set-up
-    assert torch.equal(again[0], ref[0]) and torch.equal(again[1], ref[1])
-    # a gradient through the final state cannot use the prepared words (they hold a zero entry state)
-    ref_f = ema_seq_bwd(dy, x, coef, prev0, form, dfinal_states=dfin)
-    _, _, prev2, ws2 = ema_seq_fwd(coef, x, form, prepare_backward=True)
-    got_f = ema_seq_bwd(dy, x, coef, prev2, form, dfinal_states=dfin, workspace=ws2)
-    assert torch.equal(got_f[0], ref_f[0]) and torch.equal(got_f[1], ref_f[1])
+    def fresh():  # a buffer of unknown contents (here: all bits set)
+        n = _lib.lib().ema_seq_bwd_workspace_bytes(b, nh, L, d)
+        return torch.full((n,), 0xFF, dtype=torch.uint8, device=device), 0
 
-    # autograd: two backward passes through one forward (the second finds the workspace used up)
+    y0, fin0, prev0 = ema_seq_fwd(coef, x, form, workspace=fresh())
+    ref = ema_seq_bwd(dy, x, coef, prev0, form, workspace=fresh())
+    ref_f = ema_seq_bwd(dy, x, coef, prev0, form, dfinal_states=dfin, workspace=fresh())
+
+    n = _lib.lib().ema_seq_bwd_workspace_bytes(b, nh, L, d)
+    shared = torch.zeros(n, dtype=torch.uint8, device=device)
+    for rep in range(3):  # the same buffer, forward and backward in turn, never cleared
+        y1, fin1, prev1 = ema_seq_fwd(coef, x, form, workspace=(shared, 1))
+        assert torch.equal(y0, y1) and torch.equal(fin0, fin1) and torch.equal(prev0, prev1), rep
+        got = ema_seq_bwd(dy, x, coef, prev1, form, workspace=(shared, 1))
+        assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1]), rep
+        got_f = ema_seq_bwd(dy, x, coef, prev1, form, dfinal_states=dfin, workspace=(shared, 1))
+        assert torch.equal(got_f[0], ref_f[0]) and torch.equal(got_f[1], ref_f[1]), rep
+    hdr = shared[:256].view(torch.int32).cpu()
+    assert hdr[0] == 0 and hdr[1] == 0, "ticket and exit counters are left at zero"
+    assert hdr[2] == 9, "one epoch per call"
+    assert hdr[3] == 0, "no wait ran out"
+
+    # autograd: two backward passes through one forward, on the wrappers' own shared buffer
     xg, cg = x.clone().requires_grad_(), coef.clone().requires_grad_()
     y = ema_seq_scan(cg, xg, form=form)
     y.backward(dy, retain_graph=True)
@@ -285,5 +292,120 @@ def test_backward_workspace_prepared_by_forward(form, dtype, device):
         xg, cg = x.clone().requires_grad_(), coef.clone().requires_grad_()
         ema_matmul_scan_combined(cg, xg, 128).backward(dy)
         assert torch.equal(xg.grad, ref[0]) and torch.equal(cg.grad, ref[1])
-        with torch.no_grad():  # no gradient wanted: no backward workspace is set up
+        with torch.no_grad():
             assert torch.equal(ema_matmul_scan_combined(coef, x, 128), y0)
+    _lib.check_chain_errors(device)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_unused_final_state_brings_no_gradient_tensor(dtype, device):
+    """When only y is used, autograd hands the backward None for the final state's gradient (not
+    zeros), and the result equals that of a call without it."""
+    from kernels.ema_seq import EMASeqFn, ema_seq_bwd, ema_seq_fwd
+
+    gen = torch.Generator().manual_seed(3)
+    x = torch.randn(1, 300, 2, 64, generator=gen).to(dtype).to(device)
+    dy = torch.randn(1, 300, 2, 64, generator=gen).to(dtype).to(device)
+    A = torch.nn.functional.logsigmoid(torch.randn(1, 300, 2, generator=gen) + 2).to(device)
+    xg, Ag = x.clone().requires_grad_(), A.clone().requires_grad_()
+    y, fin = EMASeqFn.apply(Ag, xg, None, "log_decay")
+    seen = []
+    fin.register_hook(lambda g: seen.append(g))
+    y.backward(dy)
+    assert seen in ([], [None]), "no tensor of zeros is made up for the unused final state"
+    _, _, prev = ema_seq_fwd(A, x)
+    dx, dA, _ = ema_seq_bwd(dy, x, A, prev)
+    assert torch.equal(xg.grad, dx) and torch.equal(Ag.grad, dA)
+    # only the final state is used: dy arrives as None
+    xg, Ag = x.clone().requires_grad_(), A.clone().requires_grad_()
+    y, fin = EMASeqFn.apply(Ag, xg, None, "log_decay")
+    dfin = torch.randn_like(fin)
+    fin.backward(dfin)
+    dx2, dA2, _ = ema_seq_bwd(torch.zeros_like(x), x, A, prev, dfinal_states=dfin)
+    assert torch.equal(xg.grad, dx2) and torch.equal(Ag.grad, dA2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("form", ["log_decay", "probability"])
+@pytest.mark.parametrize("row", [126, 127, 128, 254, 255])
+def test_single_reset_near_tile_end(form, dtype, row, device):
+    """One sequence boundary at a row whose position inside its 128-row tile is 126, 127 or 0,
+    with nothing reset in the tile that follows (and the same with p = 1 there): the tile's total
+    decay is exactly zero, the later tiles must not see anything from before the boundary, and
+    the gradients follow the per-sequence oracle."""
+    from kernels.ema_seq import ema_seq_scan
+
+    announce(f"single reset at row {row} {form} {dtype}")
+    b, L, nh, d = 2, 640, 1, 256
+    gen = torch.Generator().manual_seed(100 + row)
+    x = torch.randn(b, L, nh, d, generator=gen).to(dtype)
+    dy = torch.randn(b, L, nh, d, generator=gen).to(dtype)
+    p = torch.sigmoid(torch.randn(b, L, nh, generator=gen) - 3.0)  # long memory: a leak would show
+    seq_idx = torch.zeros(b, L, dtype=torch.int32)
+    seq_idx[:, row:] = 1
+    for variant in ("seq_idx", "p_is_one"):
+        if variant == "p_is_one":
+            if form != "probability":
+                continue
+            pv = p.clone()
+            pv[:, row] = 1.0  # y[row] = x[row]: the state before is dropped without any flag
+            ids = None
+        else:
+            pv, ids = p, seq_idx
+        coef = pv if form == "probability" else torch.log1p(-pv)
+        xg = x.to(device).requires_grad_()
+        cg = coef.to(device).requires_grad_()
+        y = ema_seq_scan(cg, xg, form=form, seq_idx=None if ids is None else ids.to(device))
+        y.backward(dy.to(device))
+        # oracle: every piece on its own
+        xf, cf = O.to_flat(x.float(), coef)
+        dyf, _ = O.to_flat(dy.float(), coef)
+        if ids is None:
+            y_ref, _ = O.ema_seq_loop(xf, cf, form)
+            dx_ref, dc_ref, _ = O.ema_seq_loop_bwd(dyf, xf, cf, form)
+        else:
+            ys, dxs, dcs = [], [], []
+            for sl in (slice(0, row), slice(row, L)):
+                yy, _ = O.ema_seq_loop(xf[:, sl], cf[:, sl], form)
+                dxx, dcc, _ = O.ema_seq_loop_bwd(dyf[:, sl], xf[:, sl], cf[:, sl], form)
+                ys.append(yy), dxs.append(dxx), dcs.append(dcc)
+            y_ref, dx_ref, dc_ref = torch.cat(ys, 1), torch.cat(dxs, 1), torch.cat(dcs, 1)
+        check_close(f"y[{variant}]", O.to_flat(y.detach().cpu().float(), coef)[0], y_ref, dtype)
+        check_close(f"dx[{variant}]", O.to_flat(xg.grad.cpu().float(), coef)[0], dx_ref, dtype)
+        dc = cg.grad.cpu().permute(0, 2, 1).reshape(b * nh, L)
+        if form == "log_decay" and ids is not None:
+            # the gradient with respect to the -inf that marks the boundary is 0 * <...> = 0
+            assert torch.equal(dc[:, row], torch.zeros(b * nh))
+        check_close(f"dcoef[{variant}]", dc, dc_ref, dtype)
+
+
+def test_chain_error_is_reported(device):
+    """A tile whose predecessor never publishes gives up after spin_limit polls, raises the error
+    word of the workspace header and hands on NaN; every kernel still ends.  Forced from the host:
+    the ticket counter of a ready workspace is set past the first chunk's tiles, so those tiles
+    are never processed and the tiles of the second chunk wait in vain."""
+    from kernels import _lib
+    from kernels.ema_seq import ema_seq_fwd
+
+    announce("chained scan: bounded wait runs out")
+    b, L, nh, d = 1, 512, 2, 256
+    gen = torch.Generator().manual_seed(5)
+    x = torch.randn(b, L, nh, d, generator=gen).to(device)
+    A = torch.nn.functional.logsigmoid(torch.randn(b, L, nh, generator=gen) + 2).to(device)
+    n = _lib.lib().ema_seq_fwd_workspace_bytes(b, nh, L, d)
+    ws = torch.zeros(n, dtype=torch.uint8, device=device)
+    y_ok, _, _ = ema_seq_fwd(A, x, workspace=(ws, 1))
+    assert not _lib.chain_error(ws)
+    hdr = ws[:256].view(torch.int32)
+    cols = b * nh * 2  # sequences x column tiles of 128 float32 columns
+    hdr[0] = cols      # tickets of chunk 0 are skipped
+    hdr[4] = 64        # polls before a wait gives up
+    torch.cuda.synchronize()
+    y_bad, _, _ = ema_seq_fwd(A, x, workspace=(ws, 1))
+    torch.cuda.synchronize()
+    assert _lib.chain_error(ws), "the error word must be raised"
+    assert torch.isnan(y_bad[:, 128:]).all(), "everything computed from the missing state is NaN"
+    # clearing the workspace puts it back in order
+    _lib._clear(ws, device)
+    y_again, _, _ = ema_seq_fwd(A, x, workspace=(ws, 1))
+    assert torch.equal(y_again, y_ok) and not _lib.chain_error(ws)

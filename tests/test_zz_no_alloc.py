@@ -34,7 +34,7 @@ def _call(entry, form, coef, x, init, dev):
             nbytes = lib.ema_seq_fwd_workspace_bytes(batch, nh, L, T)
             ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
             st = lib.ema_seq_fwd(form, *cs_, *xs, _lib.dtype_code(x), *ys, init_ptr, final.data_ptr(),
-                                 prev128.data_ptr(), ws.data_ptr(), nbytes, None, 0, batch, nh, L, T, stream,
+                                 prev128.data_ptr(), ws.data_ptr(), nbytes, 0, batch, nh, L, T, stream,
                                  None, None)
     _lib.check(st, "ema_seq_fwd_" + entry)
     torch.cuda.synchronize(dev)

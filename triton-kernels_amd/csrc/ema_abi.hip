@@ -278,55 +278,37 @@ int resident_blocks(K kernel, int threads, int smem) {
 
 inline int64_t padded_dim(int64_t T) { return (T + 255) / 256 * 256; }
 
-// status words + counters of one chained kernel: C tile slots and one virtual slot per column
+// Workspace of one chained kernel: the header, one total-decay word per (sequence, tile) and one
+// status word per (sequence, tile, column).  The header sits at the start of the buffer whatever
+// the shape, so that a buffer can serve calls of different shapes one after the other.
 struct ChainWs {
+  ChainHeader* hdr;
+  u64* decw;
   u64* status;
-  unsigned* counters;
 };
+inline size_t chain_decw_bytes(const Dims& di) { return align_up((size_t)(di.N * di.C) * sizeof(u64), 256); }
 inline size_t chain_status_bytes(const Dims& di) {
-  return align_up((size_t)(di.N * (di.C + 1) * padded_dim(di.T)) * sizeof(u64), 256);
+  return align_up((size_t)(di.N * di.C * padded_dim(di.T)) * sizeof(u64), 256);
 }
-inline size_t chain_ws_bytes(const Dims& di) { return chain_status_bytes(di) + 256; }
+inline size_t chain_ws_bytes(const Dims& di) {
+  return sizeof(ChainHeader) + chain_decw_bytes(di) + chain_status_bytes(di);
+}
 inline ChainWs chain_carve(void* base, const Dims& di) {
   ChainWs w;
-  w.status = static_cast<u64*>(base);
-  w.counters = reinterpret_cast<unsigned*>(static_cast<char*>(base) + chain_status_bytes(di));
+  char* p = static_cast<char*>(base);
+  w.hdr = reinterpret_cast<ChainHeader*>(p);
+  w.decw = reinterpret_cast<u64*>(p + sizeof(ChainHeader));
+  w.status = reinterpret_cast<u64*>(p + sizeof(ChainHeader) + chain_decw_bytes(di));
   return w;
 }
 
-// Clears the words of cols column sets of BN columns; the virtual slot (0 forward, C reverse)
-// carries `seed` (N, T), or 0.  With cs_out the same launch also computes the cumsum of the
-// coefficient over the 128-row tiles (prob = 1: the coefficient is a probability), which the
-// look-back of the kernel that follows reads: one launch and one gap less per pass.
-// The backward pass that will follow a forward pass: its status words and the place of its copy
-// of the cumsum (both in the backward's workspace), prepared by the forward's set-up launch.
-struct NextPass {
-  ChainWs chain;
-  float* cs;
-  int BN;  // columns per tile of the backward kernel
-};
-int launch_chain_init(const ChainWs& w, int64_t cols, int BN, const Dims& di, bool reverse,
-                      const float* seed, int ntiles, hipStream_t st, const float* A = nullptr,
-                      SeqStrides sa = SeqStrides{0, 0, 0}, float* cs_out = nullptr, int prob = 0,
-                      const NextPass* next = nullptr) {
-  auto blocks_of = [](int64_t pairs) { return ((pairs > 4 ? pairs : 4) + 255) / 256; };
-  const int64_t pairs = cols * (di.C + 1) * BN / 2;
-  const int64_t init_blocks = blocks_of(pairs);
-  const int64_t chunks = di.N * di.C;
-  const int64_t cumsum_blocks = cs_out ? (chunks + 3) / 4 : 0;
-  ChainNext nx{nullptr, 0, nullptr, 2, 0, 0, nullptr};
-  if (next) {
-    if (!cs_out || reverse) return EMA_ERR_UNSUPPORTED;  // prepared by a forward pass with its cumsum
-    const int64_t ntiles2 = (di.T + next->BN - 1) / next->BN;
-    const int64_t pairs2 = di.N * ntiles2 * (di.C + 1) * next->BN / 2;
-    nx = ChainNext{reinterpret_cast<uint4*>(next->chain.status), pairs2, next->chain.counters, next->BN,
-                   (int)di.C, (int)blocks_of(pairs2), next->cs};
-  }
-  if (init_blocks + nx.blocks + cumsum_blocks > 0x7fffffff) return EMA_ERR_SHAPE;
-  hipLaunchKernelGGL(chain_init_kernel, dim3((unsigned)(init_blocks + nx.blocks + cumsum_blocks)), dim3(256), 0, st,
-                     reinterpret_cast<uint4*>(w.status), pairs, w.counters, BN, (int)di.C + 1,
-                     reverse ? (int)di.C : 0, ntiles, (int)di.T, seed, (int)init_blocks, A, sa, cs_out,
-                     (int)di.nh, (int)di.L, (int)di.C, chunks, prob, nx);
+// Zero fill with a kernel (a memset node in a captured graph is not wanted here).
+int launch_clear(void* base, size_t bytes, hipStream_t st) {
+  const int64_t n16 = (int64_t)((bytes + 15) / 16);
+  if (n16 == 0) return EMA_OK;
+  if ((n16 + 255) / 256 > 0x7fffffff) return EMA_ERR_SHAPE;
+  hipLaunchKernelGGL(chain_clear_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, st,
+                     static_cast<uint4*>(base), n16);
   return launched();
 }
 
@@ -340,64 +322,57 @@ struct TileF32 {
   static constexpr int FWD_CPL = 2, BWD_CPL = 2, RPL = 8, FWD_MINW = 8, BWD_MINW = 4;
 };
 
-// cs128 is computed by the set-up launch (the caller does not launch a cumsum for it).
+// ready: the chained part of the workspace is as a zero fill or an earlier call left it;
+// otherwise it is cleared first.
 template <typename T, typename S, bool XP>
-int launch_fwd_tile_t(const void* x, SeqStrides sx, const float* A, SeqStrides sa, float* cs128,
-                      void* y, SeqStrides sy, float* prev128, float* prev_coarse, int ratio, float* fin,
-                      const float* init, const ChainWs& w, const Dims& di, hipStream_t st, void* ev0,
-                      void* ev1, const ChainWs* next_chain = nullptr, float* next_cs = nullptr) {
+int launch_fwd_tile_t(const void* x, SeqStrides sx, const float* A, SeqStrides sa, void* y, SeqStrides sy,
+                      float* prev128, float* prev_coarse, int ratio, float* fin, const float* init,
+                      void* chain_base, bool ready, const Dims& di, hipStream_t st, void* ev0, void* ev1) {
   using Cfg = TileCfg<T, S::FWD_CPL, S::RPL>;
   constexpr int BN = Cfg::BN, NT = Cfg::NT;
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
-  NextPass next{};
-  if (next_chain) next = NextPass{*next_chain, next_cs, TileCfg<T, S::BWD_CPL, S::RPL>::BN};
-  EMA_TRY(launch_chain_init(w, cols, BN, di, false, init, ntiles, st, A, sa, cs128, XP ? 1 : 0,
-                            next_chain ? &next : nullptr));
+  if (!ready) EMA_TRY(launch_clear(chain_base, chain_ws_bytes(di), st));
+  const ChainWs w = chain_carve(chain_base, di);
   auto kernel = fwd_tile_kernel<T, S::FWD_CPL, S::RPL, S::FWD_MINW, XP>;
   const int64_t cap = resident_blocks(kernel, NT, 0);
   launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx, A,
-               sa, (const float*)cs128, (T*)y, sy, prev128, prev_coarse, ratio, fin, init ? 1 : 0, w.status, w.counters,
-               (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total);
+               sa, (T*)y, sy, prev128, prev_coarse, ratio, fin, init, w.hdr, w.decw, w.status, (int)di.nh,
+               (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total);
   return launched();
 }
 
-// cumsum_here: cs128 is computed by the set-up launch; otherwise the caller has filled it.
 template <typename T, typename S, bool WRITE_Y, bool XP>
 int launch_bwd_tile_k(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* A,
-                      SeqStrides sa, float* cs128, bool cumsum_here, const float* prev128, void* dx,
-                      SeqStrides sdx, void* y, SeqStrides sy, float* part, const float* dfinal, float* dinit,
-                      const ChainWs& w, const Dims& di, hipStream_t st, void* ev0, void* ev1,
-                      bool prepared = false) {
+                      SeqStrides sa, const float* prev128, void* dx, SeqStrides sdx, void* y, SeqStrides sy,
+                      float* part, const float* dfinal, float* dinit, void* chain_base, bool ready,
+                      const Dims& di, hipStream_t st, void* ev0, void* ev1) {
   using Cfg = TileCfg<T, S::BWD_CPL, S::RPL>;
   constexpr int BN = Cfg::BN, NT = Cfg::NT;
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
-  if (!prepared)  // otherwise the forward pass has cleared the words and left cs128 in place
-    EMA_TRY(launch_chain_init(w, cols, BN, di, true, dfinal, ntiles, st, A, sa, cumsum_here ? cs128 : nullptr,
-                              XP ? 1 : 0));
+  if (!ready) EMA_TRY(launch_clear(chain_base, chain_ws_bytes(di), st));
+  const ChainWs w = chain_carve(chain_base, di);
   auto kernel = bwd_tile_kernel<T, S::BWD_CPL, S::RPL, S::BWD_MINW, WRITE_Y, XP>;
   const int64_t cap = resident_blocks(kernel, NT, 0);
   launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx,
-               (const T*)dy, sd, A, sa, (const float*)cs128, prev128, (T*)dx, sdx, (T*)y, sy, part, dfinal ? 1 : 0, dinit,
-               w.status, w.counters, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols,
-               (int)total);
+               (const T*)dy, sd, A, sa, prev128, (T*)dx, sdx, (T*)y, sy, part, dfinal, dinit, w.hdr, w.decw,
+               w.status, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total);
   return launched();
 }
 
 template <typename T, typename S, bool XP>
 int launch_bwd_tile_t(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* A,
-                      SeqStrides sa, float* cs128, bool cumsum_here, const float* prev128, void* dx,
-                      SeqStrides sdx, void* y, SeqStrides sy, float* part, const float* dfinal, float* dinit,
-                      const ChainWs& w, const Dims& di, hipStream_t st, void* ev0, void* ev1,
-                      bool prepared = false) {
+                      SeqStrides sa, const float* prev128, void* dx, SeqStrides sdx, void* y, SeqStrides sy,
+                      float* part, const float* dfinal, float* dinit, void* chain_base, bool ready,
+                      const Dims& di, hipStream_t st, void* ev0, void* ev1) {
   if (y)
-    return launch_bwd_tile_k<T, S, true, XP>(x, sx, dy, sd, A, sa, cs128, cumsum_here, prev128, dx, sdx, y, sy,
-                                             part, dfinal, dinit, w, di, st, ev0, ev1, prepared);
-  return launch_bwd_tile_k<T, S, false, XP>(x, sx, dy, sd, A, sa, cs128, cumsum_here, prev128, dx, sdx, nullptr,
-                                            sy, part, dfinal, dinit, w, di, st, ev0, ev1, prepared);
+    return launch_bwd_tile_k<T, S, true, XP>(x, sx, dy, sd, A, sa, prev128, dx, sdx, y, sy, part, dfinal, dinit,
+                                             chain_base, ready, di, st, ev0, ev1);
+  return launch_bwd_tile_k<T, S, false, XP>(x, sx, dy, sd, A, sa, prev128, dx, sdx, nullptr, sy, part, dfinal,
+                                            dinit, chain_base, ready, di, st, ev0, ev1);
 }
 
 template <typename S>
@@ -424,30 +399,24 @@ int run_bwd_fused(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, i
   return launched();
 }
 
-// Workspace of the sequence-level entry points (the backward adds its dA partials).
+// Workspace of the sequence-level entry points: the chained part first, then (backward) the
+// dA partials.
 struct SeqWs {
-  float *cs, *part;
-  ChainWs chain;
+  void* chain;
+  float* part;
   size_t bytes;
 };
 SeqWs carve_seq(void* base, const Dims& di, bool backward) {
   SeqWs w;
-  size_t off = 0;
   char* p = static_cast<char*>(base);
-  auto take = [&](size_t floats) {
-    float* r = reinterpret_cast<float*>(p + off);
-    off += align_up(floats * sizeof(float), 256);
-    return r;
-  };
-  const size_t ncq = (size_t)(di.N * di.C * di.Q);
-  w.cs = take(ncq);
+  size_t off = chain_ws_bytes(di);
+  w.chain = base;
   w.part = nullptr;
   if (backward) {
     const int pb = tile_parts_per_dim<TileBf16>(di.T), pf = tile_parts_per_dim<TileF32>(di.T);
-    w.part = take(ncq * (size_t)(pb > pf ? pb : pf));
+    w.part = reinterpret_cast<float*>(p + off);
+    off += align_up((size_t)(di.N * di.C * di.Q) * (size_t)(pb > pf ? pb : pf) * sizeof(float), 256);
   }
-  w.chain = chain_carve(p + off, di);
-  off += chain_ws_bytes(di);
   w.bytes = off;
   return w;
 }
@@ -544,22 +513,23 @@ int ema_scan_fwd(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dt
                                   SeqStrides{y_sb, y_sl, y_sh}, d, as_stream(stream));
 }
 
-// Workspace of the single-pass forward (chunk size a multiple of 128).
+// Workspace of ema_fwd: the chained part first (left alone by the staged path, so that the
+// buffer stays ready for the single-pass kernels), then room for the 128-row chunk-entry states
+// when the caller keeps none, or for the chunk states of the staged path.
 struct FwdWs {
-  float *cs128, *prev128;
-  ChainWs chain;
+  void* chain;
+  float* scratch;
   size_t bytes;
 };
-static FwdWs carve_fwd(void* base, const Dims& di) {
+static FwdWs carve_fwd(void* base, const Dims& d) {
+  const Dims di = internal_dims(d);
   FwdWs w;
-  size_t off = 0;
   char* p = static_cast<char*>(base);
-  w.cs128 = reinterpret_cast<float*>(p + off);
-  off += align_up((size_t)(di.N * di.C * di.Q) * sizeof(float), 256);
-  w.prev128 = reinterpret_cast<float*>(p + off);
-  off += align_up((size_t)(di.N * di.C * di.T) * sizeof(float), 256);
-  w.chain = chain_carve(p + off, di);
-  off += chain_ws_bytes(di);
+  size_t off = chain_ws_bytes(di);
+  w.chain = base;
+  w.scratch = reinterpret_cast<float*>(p + off);
+  const size_t n128 = (size_t)(di.N * di.C * di.T), nq = (size_t)(d.N * d.C * d.T);
+  off += align_up((n128 > nq ? n128 : nq) * sizeof(float), 256);
   w.bytes = off;
   return w;
 }
@@ -568,21 +538,21 @@ size_t ema_fwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, in
                                int64_t chunk) {
   Dims d;
   if (check_dims(batch, nheads, seqlen, dim, chunk, true, &d) != EMA_OK) return 0;
-  const size_t staged = align_up((size_t)(d.N * d.C * d.T) * sizeof(float), 256);
-  if (chunk % kTileRows) return staged;
-  const size_t chained = carve_fwd(nullptr, internal_dims(d)).bytes;
-  return chained > staged ? chained : staged;
+  return carve_fwd(nullptr, d).bytes;
+}
+
+int ema_workspace_clear(void* workspace, size_t bytes, void* stream) {
+  EMA_TRY(check_f32(workspace));
+  return launch_clear(workspace, bytes, as_stream(stream));
 }
 
 int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void* x, int64_t x_sb,
             int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb, int64_t y_sl,
             int64_t y_sh, float* cs, float* prev, float* final_state, float* prev128,
-            void* workspace, size_t workspace_bytes, void* bwd_workspace, size_t bwd_workspace_bytes,
-            int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim, int64_t chunk, void* stream,
-            void* ev_start, void* ev_stop) {
+            void* workspace, size_t workspace_bytes, int workspace_ready, int64_t batch, int64_t nheads,
+            int64_t seqlen, int64_t dim, int64_t chunk, void* stream, void* ev_start, void* ev_stop) {
   Dims d;
   EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
-  if (bwd_workspace && chunk % kTileRows) return EMA_ERR_UNSUPPORTED;
   EMA_TRY(check_dtype(dtype));
   EMA_TRY(check_seq(x, x_sb, x_sl, x_sh, dtype, dim));
   EMA_TRY(check_seq(y, y_sb, y_sl, y_sh, dtype, dim));
@@ -592,36 +562,26 @@ int ema_fwd(const float* A, int64_t a_sb, int64_t a_sl, int64_t a_sh, const void
     return EMA_ERR_SHAPE;
   hipStream_t st = as_stream(stream);
   const SeqStrides sx{x_sb, x_sl, x_sh}, sy{y_sb, y_sl, y_sh}, sa{a_sb, a_sl, a_sh};
-  if (chunk != kTileRows) EMA_TRY(launch_cumsum(A, sa, cs, d, st));
+  EMA_TRY(launch_cumsum(A, sa, cs, d, st));  // an output of this entry point; the scan below does not read it
   if (chunk % kTileRows == 0) {
     // Single pass over x: the scan is computed on 128-row chunks with the inter-chunk state
     // handed over inside the kernel; the states at the caller's chunk boundaries are every
-    // (chunk/128)-th of them.  The cumsum over the 128-row chunks is part of the kernel's set-up
-    // launch; for chunk = 128 it is the caller's cs.
+    // (chunk/128)-th of them.
     const Dims di = internal_dims(d);
-    const FwdWs w = carve_fwd(workspace, di);
+    const FwdWs w = carve_fwd(workspace, d);
     const int ratio = (int)(chunk / kTileRows);
-    float* cs128 = ratio == 1 ? cs : w.cs128;
-    float* p128 = prev128 ? prev128 : (ratio == 1 ? prev : w.prev128);
+    float* p128 = prev128 ? prev128 : (ratio == 1 ? prev : w.scratch);
     float* coarse = p128 == prev ? nullptr : prev;
-    SeqWs bw{};
-    if (bwd_workspace) {
-      EMA_TRY(check_f32(bwd_workspace));
-      if (bwd_workspace_bytes < carve_seq(nullptr, di, true).bytes) return EMA_ERR_SHAPE;
-      bw = carve_seq(bwd_workspace, di, true);
-    }
-    const ChainWs* nc = bwd_workspace ? &bw.chain : nullptr;
-    if (dtype == EMA_BF16) {
-      return launch_fwd_tile_t<bf16_t, TileBf16, false>(x, sx, A, sa, cs128, y, sy, p128, coarse, ratio,
-                                                        final_state, nullptr, w.chain, di, st, ev_start,
-                                                        ev_stop, nc, bw.cs);
-    }
-    return launch_fwd_tile_t<float, TileF32, false>(x, sx, A, sa, cs128, y, sy, p128, coarse, ratio,
-                                                    final_state, nullptr, w.chain, di, st, ev_start, ev_stop, nc,
-                                                    bw.cs);
+    if (dtype == EMA_BF16)
+      return launch_fwd_tile_t<bf16_t, TileBf16, false>(x, sx, A, sa, y, sy, p128, coarse, ratio, final_state,
+                                                        nullptr, w.chain, workspace_ready != 0, di, st,
+                                                        ev_start, ev_stop);
+    return launch_fwd_tile_t<float, TileF32, false>(x, sx, A, sa, y, sy, p128, coarse, ratio, final_state,
+                                                    nullptr, w.chain, workspace_ready != 0, di, st, ev_start,
+                                                    ev_stop);
   }
   if (prev128) return EMA_ERR_UNSUPPORTED;  // only produced when chunk is a multiple of 128
-  float* states = static_cast<float*>(workspace);
+  float* states = carve_fwd(workspace, d).scratch;
   EMA_TRY(record_event(ev_start, st));
   EMA_TRY(launch_chunk_reduce<0>(x, sx, dtype, cs, states, d, st));
   EMA_TRY(launch_state_passing_fwd(states, cs + (d.Q - 1), d.C * d.Q, d.Q, prev, final_state, d.N,
@@ -734,16 +694,18 @@ int ema_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t 
                    ddA_intra, part, rowsum, d, as_stream(stream));
 }
 
-// Workspace of ema_bwd.
+// Workspace of ema_bwd: the chained part first, then the dA partials and what the recomputation
+// of the chunk-entry states needs.
 struct BwdWs {
+  void* chain;
   float *cs, *states, *prev, *part;
-  ChainWs chain;
   size_t bytes;
 };
 static BwdWs carve_bwd(void* base, const Dims& di) {
   BwdWs w;
-  size_t off = 0;
+  size_t off = chain_ws_bytes(di);
   char* p = static_cast<char*>(base);
+  w.chain = base;
   auto take = [&](size_t floats) {
     float* r = reinterpret_cast<float*>(p + off);
     off += align_up(floats * sizeof(float), 256);
@@ -755,8 +717,6 @@ static BwdWs carve_bwd(void* base, const Dims& di) {
   w.prev = take(nct);
   const int parts_bf16 = tile_parts_per_dim<TileBf16>(di.T), parts_f32 = tile_parts_per_dim<TileF32>(di.T);
   w.part = take(ncq * (size_t)(parts_bf16 > parts_f32 ? parts_bf16 : parts_f32));
-  w.chain = chain_carve(p + off, di);
-  off += chain_ws_bytes(di);
   w.bytes = off;
   return w;
 }
@@ -772,8 +732,8 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
             int64_t x_sb, int64_t x_sl, int64_t x_sh, const float* A, int64_t a_sb, int64_t a_sl,
             int64_t a_sh, const float* prev128, int dtype, void* dx, int64_t dx_sb, int64_t dx_sl,
             int64_t dx_sh, float* ddA, void* y, int64_t y_sb, int64_t y_sl, int64_t y_sh,
-            void* workspace, size_t workspace_bytes, int64_t batch, int64_t nheads, int64_t seqlen,
-            int64_t dim, int64_t chunk, void* stream, void* ev_start, void* ev_stop) {
+            void* workspace, size_t workspace_bytes, int workspace_ready, int64_t batch, int64_t nheads,
+            int64_t seqlen, int64_t dim, int64_t chunk, void* stream, void* ev_start, void* ev_stop) {
   Dims d;
   EMA_TRY(check_dims(batch, nheads, seqlen, dim, chunk, true, &d));
   EMA_TRY(check_dtype(dtype));
@@ -795,7 +755,6 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
   const SeqStrides sy{y_sb, y_sl, y_sh};
 
   const SeqStrides sa{a_sb, a_sl, a_sh};
-  const bool cumsum_here = prev128 != nullptr;  // otherwise the recomputation below needs cs first
   if (!prev128) {
     // states entering each chunk, recomputed: chunk states, then the inter-chunk recurrence
     // (its final state is not needed and lands in `part`, which is free until the main kernel)
@@ -809,13 +768,13 @@ int ema_bwd(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t dy_sh, const v
   // the reverse inter-chunk state is handed over inside the kernel
   int parts = dtype == EMA_BF16 ? tile_parts_per_dim<TileBf16>(di.T) : tile_parts_per_dim<TileF32>(di.T);
   if (dtype == EMA_BF16) {
-    EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, false>(x, sx, dy, sd, A, sa, w.cs, cumsum_here, prev128, dx, sdx, y, sy,
-                                                        w.part, nullptr, nullptr, w.chain, di, st, ev_start,
-                                                        ev_stop)));
+    EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, false>(x, sx, dy, sd, A, sa, prev128, dx, sdx, y, sy, w.part,
+                                                        nullptr, nullptr, w.chain, workspace_ready != 0, di,
+                                                        st, ev_start, ev_stop)));
   } else
-    EMA_TRY((launch_bwd_tile_t<float, TileF32, false>(x, sx, dy, sd, A, sa, w.cs, cumsum_here, prev128, dx, sdx, y, sy,
-                                                      w.part, nullptr, nullptr, w.chain, di, st, ev_start,
-                                                      ev_stop)));
+    EMA_TRY((launch_bwd_tile_t<float, TileF32, false>(x, sx, dy, sd, A, sa, prev128, dx, sdx, y, sy, w.part,
+                                                      nullptr, nullptr, w.chain, workspace_ready != 0, di, st,
+                                                      ev_start, ev_stop)));
   const int64_t total = d.N * d.C * d.Q;
   hipLaunchKernelGGL(dA_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w.part,
                      ddA, (int)d.L, (int)d.Q, (int)d.C, (int)di.C, parts, total);
@@ -866,11 +825,11 @@ size_t ema_seq_fwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen
 }
 
 static int seq_fwd_impl(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t c_sh, const void* x,
-                int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb,
-                int64_t y_sl, int64_t y_sh, const float* init, float* final_state, float* prev128,
-                void* workspace, size_t workspace_bytes, void* bwd_workspace, size_t bwd_workspace_bytes,
-                int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
-                void* ev_stop) {
+                        int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb,
+                        int64_t y_sl, int64_t y_sh, const float* init, float* final_state, float* prev128,
+                        void* workspace, size_t workspace_bytes, int workspace_ready, int64_t batch,
+                        int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
+                        void* ev_stop) {
   Dims d;
   EMA_TRY(check_form(form));
   EMA_TRY(check_dims(batch, nheads, seqlen, dim, kTileRows, true, &d));
@@ -882,42 +841,30 @@ static int seq_fwd_impl(int form, const float* coef, int64_t c_sb, int64_t c_sl,
   if (workspace_bytes < ema_seq_fwd_workspace_bytes(batch, nheads, seqlen, dim)) return EMA_ERR_SHAPE;
   hipStream_t st = as_stream(stream);
   const SeqWs w = carve_seq(workspace, d, false);
-  SeqWs bw{};
-  if (bwd_workspace) {
-    EMA_TRY(check_f32(bwd_workspace));
-    if (bwd_workspace_bytes < carve_seq(nullptr, d, true).bytes) return EMA_ERR_SHAPE;
-    bw = carve_seq(bwd_workspace, d, true);
-  }
-  const ChainWs* nc = bwd_workspace ? &bw.chain : nullptr;
   const SeqStrides sx{x_sb, x_sl, x_sh}, sy{y_sb, y_sl, y_sh}, sc{c_sb, c_sl, c_sh};
-  const bool xp = form == EMA_FORM_PROBABILITY;  // the cumsum of the coefficient is part of the set-up launch
+  const bool xp = form == EMA_FORM_PROBABILITY, ready = workspace_ready != 0;
   if (dtype == EMA_BF16) {
     if (xp)
-      return launch_fwd_tile_t<bf16_t, TileBf16, true>(x, sx, coef, sc, w.cs, y, sy, prev128, nullptr, 1,
-                                                       final_state, init, w.chain, d, st, ev_start, ev_stop, nc,
-        bw.cs);
-    return launch_fwd_tile_t<bf16_t, TileBf16, false>(x, sx, coef, sc, w.cs, y, sy, prev128, nullptr, 1,
-                                                      final_state, init, w.chain, d, st, ev_start, ev_stop, nc,
-        bw.cs);
+      return launch_fwd_tile_t<bf16_t, TileBf16, true>(x, sx, coef, sc, y, sy, prev128, nullptr, 1, final_state,
+                                                       init, w.chain, ready, d, st, ev_start, ev_stop);
+    return launch_fwd_tile_t<bf16_t, TileBf16, false>(x, sx, coef, sc, y, sy, prev128, nullptr, 1, final_state,
+                                                      init, w.chain, ready, d, st, ev_start, ev_stop);
   }
   if (xp)
-    return launch_fwd_tile_t<float, TileF32, true>(x, sx, coef, sc, w.cs, y, sy, prev128, nullptr, 1,
-                                                   final_state, init, w.chain, d, st, ev_start, ev_stop, nc,
-        bw.cs);
-  return launch_fwd_tile_t<float, TileF32, false>(x, sx, coef, sc, w.cs, y, sy, prev128, nullptr, 1,
-                                                  final_state, init, w.chain, d, st, ev_start, ev_stop, nc,
-        bw.cs);
+    return launch_fwd_tile_t<float, TileF32, true>(x, sx, coef, sc, y, sy, prev128, nullptr, 1, final_state, init,
+                                                   w.chain, ready, d, st, ev_start, ev_stop);
+  return launch_fwd_tile_t<float, TileF32, false>(x, sx, coef, sc, y, sy, prev128, nullptr, 1, final_state, init,
+                                                  w.chain, ready, d, st, ev_start, ev_stop);
 }
 
 int ema_seq_fwd(int form, const float* coef, int64_t c_sb, int64_t c_sl, int64_t c_sh, const void* x,
                 int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, void* y, int64_t y_sb,
                 int64_t y_sl, int64_t y_sh, const float* init, float* final_state, float* prev128,
-                void* workspace, size_t workspace_bytes, void* bwd_workspace, size_t bwd_workspace_bytes,
-                int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
-                void* ev_stop) {
+                void* workspace, size_t workspace_bytes, int workspace_ready, int64_t batch, int64_t nheads,
+                int64_t seqlen, int64_t dim, void* stream, void* ev_start, void* ev_stop) {
   return seq_fwd_impl(form, coef, c_sb, c_sl, c_sh, x, x_sb, x_sl, x_sh, dtype, y, y_sb, y_sl, y_sh, init,
-                      final_state, prev128, workspace, workspace_bytes, bwd_workspace, bwd_workspace_bytes,
-                      batch, nheads, seqlen, dim, stream, ev_start, ev_stop);
+                      final_state, prev128, workspace, workspace_bytes, workspace_ready, batch, nheads, seqlen,
+                      dim, stream, ev_start, ev_stop);
 }
 
 // ---- the entry point that allocates nothing: ema_seq_fwd with its workspace in a file-scope array
@@ -933,9 +880,11 @@ int ema_seq_fwd_static(int form, const float* coef, int64_t c_sb, int64_t c_sl, 
   if (need > kScratchBytes) return EMA_ERR_TOO_LARGE;
   void* ws = nullptr;
   EMA_TRY(scratch_address(&ws));
+  // the array starts out zero-filled and is only ever written by this entry point's kernels,
+  // which leave it ready for the next call: nothing has to be cleared
   return seq_fwd_impl(form, coef, c_sb, c_sl, c_sh, x, x_sb, x_sl, x_sh, dtype, y, y_sb, y_sl, y_sh, init,
-                      final_state, prev128, ws, kScratchBytes, nullptr, 0, batch, nheads, seqlen, dim, stream,
-                      nullptr, nullptr);
+                      final_state, prev128, ws, kScratchBytes, 1, batch, nheads, seqlen, dim, stream, nullptr,
+                      nullptr);
 }
 
 size_t ema_seq_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim) {
@@ -948,7 +897,7 @@ int ema_seq_bwd(int form, const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t 
                 int64_t x_sb, int64_t x_sl, int64_t x_sh, const float* coef, int64_t c_sb, int64_t c_sl,
                 int64_t c_sh, const float* prev128, const float* dfinal, int dtype, void* dx,
                 int64_t dx_sb, int64_t dx_sl, int64_t dx_sh, float* dcoef, int64_t dc_sb, int64_t dc_sl,
-                int64_t dc_sh, float* dinit, void* workspace, size_t workspace_bytes, int workspace_prepared,
+                int64_t dc_sh, float* dinit, void* workspace, size_t workspace_bytes, int workspace_ready,
                 int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim, void* stream, void* ev_start,
                 void* ev_stop) {
   Dims d;
@@ -961,32 +910,33 @@ int ema_seq_bwd(int form, const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t 
   if (!coef || !prev128 || !dcoef) return EMA_ERR_NULL;
   EMA_TRY(check_f32(workspace));
   if (workspace_bytes < ema_seq_bwd_workspace_bytes(batch, nheads, seqlen, dim)) return EMA_ERR_SHAPE;
-  // a prepared workspace holds nothing entering the reverse scan from outside
-  if (workspace_prepared && dfinal) return EMA_ERR_UNSUPPORTED;
-  const bool prep = workspace_prepared != 0;
+  const bool ready = workspace_ready != 0;
   hipStream_t st = as_stream(stream);
   const SeqWs w = carve_seq(workspace, d, true);
   const SeqStrides sx{x_sb, x_sl, x_sh}, sd{dy_sb, dy_sl, dy_sh}, sdx{dx_sb, dx_sl, dx_sh};
   const SeqStrides sc{c_sb, c_sl, c_sh}, none{0, 0, 0};
-  const bool xp = form == EMA_FORM_PROBABILITY;  // the cumsum of the coefficient is part of the set-up launch
+  const bool xp = form == EMA_FORM_PROBABILITY;
   int parts;
   if (dtype == EMA_BF16) {
     parts = tile_parts_per_dim<TileBf16>(d.T);
     if (xp)
-      EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, true>(x, sx, dy, sd, coef, sc, w.cs, true, prev128, dx, sdx, nullptr,
-                                                         none, w.part, dfinal, dinit, w.chain, d, st, ev_start, ev_stop, prep)));
+      EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, true>(x, sx, dy, sd, coef, sc, prev128, dx, sdx, nullptr, none,
+                                                         w.part, dfinal, dinit, w.chain, ready, d, st, ev_start,
+                                                         ev_stop)));
     else
-      EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, false>(x, sx, dy, sd, coef, sc, w.cs, true, prev128, dx, sdx,
-                                                          nullptr, none, w.part, dfinal, dinit, w.chain, d, st,
-                                                          ev_start, ev_stop, prep)));
+      EMA_TRY((launch_bwd_tile_t<bf16_t, TileBf16, false>(x, sx, dy, sd, coef, sc, prev128, dx, sdx, nullptr, none,
+                                                          w.part, dfinal, dinit, w.chain, ready, d, st, ev_start,
+                                                          ev_stop)));
   } else {
     parts = tile_parts_per_dim<TileF32>(d.T);
     if (xp)
-      EMA_TRY((launch_bwd_tile_t<float, TileF32, true>(x, sx, dy, sd, coef, sc, w.cs, true, prev128, dx, sdx, nullptr,
-                                                       none, w.part, dfinal, dinit, w.chain, d, st, ev_start, ev_stop, prep)));
+      EMA_TRY((launch_bwd_tile_t<float, TileF32, true>(x, sx, dy, sd, coef, sc, prev128, dx, sdx, nullptr, none,
+                                                       w.part, dfinal, dinit, w.chain, ready, d, st, ev_start,
+                                                       ev_stop)));
     else
-      EMA_TRY((launch_bwd_tile_t<float, TileF32, false>(x, sx, dy, sd, coef, sc, w.cs, true, prev128, dx, sdx, nullptr,
-                                                        none, w.part, dfinal, dinit, w.chain, d, st, ev_start, ev_stop, prep)));
+      EMA_TRY((launch_bwd_tile_t<float, TileF32, false>(x, sx, dy, sd, coef, sc, prev128, dx, sdx, nullptr, none,
+                                                        w.part, dfinal, dinit, w.chain, ready, d, st, ev_start,
+                                                        ev_stop)));
   }
   const int64_t total = d.N * d.L;
   hipLaunchKernelGGL(dcoef_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w.part,

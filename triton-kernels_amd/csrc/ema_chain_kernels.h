@@ -5,17 +5,23 @@
 // sequential recurrence) but inside the one kernel that also computes the outputs:
 //
 //   * every tile (n, chunk c, column tile) publishes the chunk-local state of its columns
-//     as soon as it has reduced its rows (flag AGGREGATE), then looks back over the tiles
-//     of the earlier chunks of the same sequence and columns, adding decayed aggregates
-//     until it meets a tile that already knows its inclusive state (flag PREFIX); it then
-//     publishes its own inclusive state.
-//   * a published word is 64 bits, {flag, f32 value}, written and polled with relaxed
-//     agent-scope atomics, so flag and value arrive together and no fence is needed.
+//     as soon as it has reduced its rows (state AGGREGATE) together with the tile's total
+//     decay, then looks back over the tiles of the earlier chunks of the same sequence and
+//     columns, adding decayed aggregates until it meets a tile that already knows its
+//     inclusive state (state PREFIX); it then publishes its own inclusive state.
+//   * a published word is 64 bits, {tag, f32 value}, written and polled with relaxed
+//     agent-scope atomics, so tag and value arrive together and no fence is needed.
+//   * the tag holds the launch's epoch besides the state, so words left by earlier launches
+//     read as "not published" and nothing has to be cleared between launches: a workspace that
+//     was zero-filled once serves any number of launches of any shapes, one after the other.
+//     The header of the workspace carries the epoch; the last workgroup to leave a launch
+//     advances it and puts the ticket counter back to zero.
 //   * tiles are handed out by an atomic ticket counter in chunk-major order (all columns
 //     of chunk 0, then chunk 1, ...; the backward runs the chunks from last to first), so
 //     a tile only ever waits for tiles with smaller tickets, which are running or done:
 //     the wait cannot deadlock whatever the number of resident workgroups.  Every poll
-//     loop is bounded; on exhaustion it raises the error word and the kernel still ends.
+//     loop is bounded; on exhaustion it raises the error word of the header, hands on NaN
+//     (which reaches the outputs) and the kernel still ends.
 #pragma once
 #include "ema_walk_kernels.h"
 
@@ -28,88 +34,94 @@ typedef unsigned long long u64;
 __device__ long long* g_ema_timing = nullptr;
 #endif
 
-constexpr unsigned kFlagAggregate = 1u;
-constexpr unsigned kFlagPrefix = 2u;
-constexpr int kSpinLimit = 1 << 20;
+// First 256 bytes of a chained-scan workspace (ema_chain_header in ema_hip.h).
+struct ChainHeader {
+  unsigned ticket;      // next tile to hand out; zero between launches
+  unsigned done;        // workgroups that have left the running launch; zero between launches
+  unsigned epoch;       // epoch of the last completed launch
+  unsigned error;       // sticky: a bounded wait ran out in some launch since the last clear
+  unsigned spin_limit;  // polls before a wait gives up; 0 = kSpinLimitDefault
+  unsigned reserved[59];
+};
+static_assert(sizeof(ChainHeader) == 256, "header size is part of the ABI");
 
-__device__ __forceinline__ void chain_publish(u64* p, unsigned flag, float v) {
-  const u64 w = ((u64)flag << 32) | (u64)__float_as_uint(v);
+constexpr unsigned kStateAggregate = 1u;
+constexpr unsigned kStatePrefix = 2u;
+constexpr unsigned kSpinLimitDefault = 1u << 20;
+constexpr unsigned kEpochMask = 0x3fffffffu;
+constexpr int kLookWindow = 4;  // predecessors whose words are requested together
+
+// Epoch of the launch that finds `last` in the header: 1 .. 2^30 - 1, never 0 (the tag of
+// zero-filled memory).
+__device__ __forceinline__ unsigned chain_next_epoch(unsigned last) {
+  const unsigned e = (last + 1u) & kEpochMask;
+  return e ? e : 1u;
+}
+
+__device__ __forceinline__ void chain_publish(u64* p, unsigned epoch, unsigned state, float v) {
+  const u64 w = ((u64)((epoch << 2) | state) << 32) | (u64)__float_as_uint(v);
   __hip_atomic_store(p, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Polls one word until it carries a flag.  Gives up after kSpinLimit polls: raises *err and
-// reports a zero PREFIX so that the caller's walk ends.
-__device__ __forceinline__ unsigned chain_wait(const u64* p, float* v, unsigned* err) {
-  for (int i = 0; i < kSpinLimit; ++i) {
-    const u64 w = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const unsigned f = (unsigned)(w >> 32);
-    if (f) {
-      *v = __uint_as_float((unsigned)w);
-      return f;
-    }
-    __builtin_amdgcn_s_sleep(1);
-  }
-  atomicExch(err, 1u);
-  *v = 0.f;
-  return kFlagPrefix;
+__device__ __forceinline__ u64 chain_peek(const u64* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Prepares the status words, the ticket counters and the error word before a chained kernel.
-// The words of one column set are laid out [slot][BN] with C + 1 slots: C tiles and one
-// virtual neighbour before the first tile (forward: slot 0, tiles at slot c + 1) or after the
-// last (reverse: slot C, tiles at slot c).  Tile slots are zeroed; the virtual slot carries
-// PREFIX with the state that enters the scan from outside, seed[n, column] or 0.  Each thread
-// writes two adjacent words (BN is even, so both lie in one slot).
-// The set-up of a single-pass kernel in one launch: the first init_blocks workgroups clear the
-// status words (and seed the virtual slot), the rest, if any, compute the per-tile cumsum of the
-// log-decay that the look-back reads (cumsum_block; cs null = no such workgroups are launched).
-// A forward pass whose backward will follow can have the backward's status words prepared in the
-// same launch (next: the words of the reverse scan with nothing entering it, next_blocks
-// workgroups after the first init_blocks) together with a second copy of the cumsum (cs_next).
-struct ChainNext {
-  uint4* words;
-  int64_t n_pairs;
-  unsigned* counters;
-  int BN, virt_slot, blocks;
-  float* cs;
+// State of a word under this launch's epoch; 0 = not published by this launch.
+__device__ __forceinline__ unsigned chain_state(u64 w, unsigned epoch) {
+  const unsigned tag = (unsigned)(w >> 32);
+  return (tag >> 2) == epoch ? (tag & 3u) : 0u;
+}
+
+__device__ __forceinline__ float chain_value(u64 w) { return __uint_as_float((unsigned)w); }
+
+struct ChainCtl {
+  unsigned epoch, spin_limit;
+  unsigned* err;
 };
-__global__ __launch_bounds__(256) void chain_init_kernel(uint4* __restrict__ words, int64_t n_pairs,
-                                                         unsigned* __restrict__ counters, int BN,
-                                                         int slots, int virt_slot, int ntiles, int Tdim,
-                                                         const float* __restrict__ seed, int init_blocks,
-                                                         const float* __restrict__ A, SeqStrides sa,
-                                                         float* __restrict__ cs, int nh, int L, int C,
-                                                         int64_t total_chunks, int prob, ChainNext next) {
-  int64_t blk = blockIdx.x;
-  if (blk >= init_blocks + next.blocks) {
-    cumsum_block(blk - init_blocks - next.blocks, A, sa, cs, nh, L, kTileRows, C, total_chunks, prob, next.cs);
-    return;
-  }
-  if (blk >= init_blocks) {  // the pass that follows: same layout, its own column width, no seed
-    blk -= init_blocks;
-    words = next.words, n_pairs = next.n_pairs, counters = next.counters, BN = next.BN;
-    virt_slot = next.virt_slot, seed = nullptr;
-  }
-  const int64_t i = blk * 256 + threadIdx.x;
-  if (i < 4) counters[i] = 0u;
-  if (i >= n_pairs) return;
-  const int64_t w = 2 * i;
-  const int64_t row = w / BN;  // (column set, slot)
-  const int k = (int)(w - row * BN);
-  const int64_t col_id = row / slots;
-  const int slot = (int)(row - col_id * slots);
-  uint4 v = make_uint4(0u, 0u, 0u, 0u);
-  if (slot == virt_slot) {
-    float s0 = 0.f, s1 = 0.f;
-    if (seed) {
-      const int64_t n = col_id / ntiles;
-      const int col = (int)(col_id - n * ntiles) * BN + k;
-      if (col < Tdim) s0 = seed[n * Tdim + col];
-      if (col + 1 < Tdim) s1 = seed[n * Tdim + col + 1];
+
+// w is what a first look at *p returned.  Polls until the word is published by this launch.
+// Gives up after spin_limit polls: raises the error word and reports a PREFIX of NaN, which ends
+// the caller's walk and poisons everything computed from it.
+__device__ __forceinline__ u64 chain_wait(const u64* p, u64 w, const ChainCtl& ctl) {
+  unsigned polls = 0;
+  while (chain_state(w, ctl.epoch) == 0u) {
+    if (++polls > ctl.spin_limit) {
+      atomicExch(ctl.err, 1u);
+      return ((u64)((ctl.epoch << 2) | kStatePrefix) << 32) | 0x7fc00000ull;
     }
-    v = make_uint4(__float_as_uint(s0), kFlagPrefix, __float_as_uint(s1), kFlagPrefix);
+    __builtin_amdgcn_s_sleep(1);
+    w = chain_peek(p);
   }
-  words[i] = v;
+  return w;
+}
+
+// Start and end of a launch.  Every workgroup reads the epoch before its first tile; the last
+// one to leave (all tickets are taken by then and nobody reads the header again) advances the
+// epoch and zeroes the counters for the next launch on the stream.
+__device__ __forceinline__ ChainCtl chain_enter(ChainHeader* hdr) {
+  ChainCtl ctl;
+  ctl.epoch = chain_next_epoch(__hip_atomic_load(&hdr->epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  const unsigned lim = __hip_atomic_load(&hdr->spin_limit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  ctl.spin_limit = lim ? lim : kSpinLimitDefault;
+  ctl.err = &hdr->error;
+  return ctl;
+}
+__device__ __forceinline__ void chain_leave(ChainHeader* hdr, const ChainCtl& ctl) {
+  // called by one thread per workgroup after the workgroup's last tile
+  const unsigned before = __hip_atomic_fetch_add(&hdr->done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (before == gridDim.x - 1) {
+    __hip_atomic_store(&hdr->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&hdr->done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&hdr->epoch, ctl.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+// Zero fill of a workspace (or of its leading part) in 16-byte pieces: the state in which the
+// chained kernels expect to find a workspace they have not used before.
+__global__ __launch_bounds__(256) void chain_clear_kernel(uint4* __restrict__ p, int64_t n16) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n16) p[i] = make_uint4(0u, 0u, 0u, 0u);
 }
 
 struct ChainTile {
@@ -135,29 +147,46 @@ __device__ __forceinline__ ChainTile chain_decode(int ticket, int cols, int ntil
   return t;
 }
 
-
-// Inclusive state entering chunk c for one column: walks the published words of the chunks
-// before (forward) or after (reverse) c, ending at the virtual neighbour at the latest.
-// status points at the words of this column set, laid out [slot][BN] as chain_init_kernel
-// describes; cs_n[j * 128 + 127] is the total log-decay of chunk j.
+// Look-back of one column, in two parts so that other work can sit between the requests and
+// their use.  words: the status words of this column, words[j * BN] that of tile j; decw[j]: the
+// total decay of tile j of this sequence.  The walk starts at the neighbour of tile c (c - 1
+// forward, c + 1 reverse) and ends at the first PREFIX; the first tile of a scan always
+// publishes one, so the walk stays inside [0, C).
 template <bool REV, int BN>
-__device__ __forceinline__ float chain_look(const u64* status, const float* __restrict__ cs_n,
-                                            int c, int C, int t, unsigned* err) {
-  float carry = 0.f, scale = 1.f;
-  for (int j = REV ? c + 1 : c - 1; REV ? j <= C : j >= -1; j += REV ? 1 : -1) {
-    float v;
-    const unsigned f = chain_wait(status + (int64_t)(REV ? j : j + 1) * BN + t, &v, err);
-    carry = fmaf(scale, v, carry);
-    if (f == kFlagPrefix) break;  // always so at the virtual neighbour
-    scale *= __expf(fminf(cs_n[(int64_t)j * kTileRows + kTileRows - 1], 0.f));
-  }
-  return carry;
-}
+struct ChainLook {
+  u64 w[kLookWindow], d[kLookWindow];
+  int j;  // neighbour the window starts at
 
-// Slot of tile c of a column set.
-template <bool REV>
-__device__ __forceinline__ int chain_slot(int c) {
-  return REV ? c : c + 1;
-}
+  __device__ __forceinline__ int clampj(int jj, int C) const { return REV ? min(jj, C - 1) : max(jj, 0); }
+
+  __device__ __forceinline__ void request(const u64* words, const u64* decw, int C) {
+#pragma unroll
+    for (int i = 0; i < kLookWindow; ++i) {
+      const int jj = clampj(REV ? j + i : j - i, C);
+      w[i] = chain_peek(words + (int64_t)jj * BN);
+      d[i] = chain_peek(decw + jj);
+    }
+  }
+  __device__ __forceinline__ void begin(const u64* words, const u64* decw, int c, int C) {
+    j = REV ? c + 1 : c - 1;
+    request(words, decw, C);
+  }
+  __device__ __forceinline__ float finish(const u64* words, const u64* decw, int C, const ChainCtl& ctl) {
+    float carry = 0.f, scale = 1.f;
+    for (;;) {
+#pragma unroll
+      for (int i = 0; i < kLookWindow; ++i) {
+        const int jj = REV ? j + i : j - i;
+        if (REV ? jj >= C : jj < 0) return carry;
+        const u64 sw = chain_wait(words + (int64_t)jj * BN, w[i], ctl);
+        carry = fmaf(scale, chain_value(sw), carry);
+        if (chain_state(sw, ctl.epoch) == kStatePrefix) return carry;
+        scale *= chain_value(chain_wait(decw + jj, d[i], ctl));
+      }
+      j += REV ? kLookWindow : -kLookWindow;
+      request(words, decw, C);
+    }
+  }
+};
 
 }  // namespace ema

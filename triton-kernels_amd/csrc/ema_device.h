@@ -41,6 +41,14 @@ __device__ __forceinline__ float wave_inclusive_scan(float v) {
   return v;
 }
 
+// Exclusive prefix sum over the 64 lanes: the inclusive sum of the lane before, 0 in lane 0.
+// Formed by a shift and not as `inclusive - own value`, which is NaN for an infinite term (a
+// log-decay of -inf marks a state reset and must stay -inf in every later sum).
+__device__ __forceinline__ float wave_exclusive_scan(float v) {
+  const float up = __shfl_up(wave_inclusive_scan(v), 1, 64);
+  return (threadIdx.x & 63) == 0 ? 0.f : up;
+}
+
 // Sum over the 64 lanes, returned in every lane.
 __device__ __forceinline__ float wave_sum(float v) {
   v = wave_inclusive_scan(v);

@@ -22,7 +22,7 @@ __device__ __forceinline__ float cumsum_term(float v, int prob) {
 // The work of workgroup `block` (four chunks, one per wave).
 __device__ __forceinline__ void cumsum_block(int64_t block, const float* __restrict__ A, SeqStrides sa,
                                              float* __restrict__ cs, int nh, int L, int Q, int C,
-                                             int64_t total_chunks, int prob, float* __restrict__ cs2 = nullptr) {
+                                             int64_t total_chunks, int prob) {
   const int lane = threadIdx.x & 63;
   const int64_t chunk_id = block * 4 + (threadIdx.x >> 6);
   if (chunk_id >= total_chunks) return;
@@ -40,15 +40,12 @@ __device__ __forceinline__ void cumsum_block(int64_t block, const float* __restr
     const int q = q0 + i;
     if (q < limit) local += cumsum_term(a[(int64_t)q * sa.sl], prob);
   }
-  float run = wave_inclusive_scan(local) - local;  // exclusive prefix of the lane totals
+  float run = wave_exclusive_scan(local);  // prefix of the lane totals before this lane
   float* out = cs + chunk_id * Q;
   for (int i = 0; i < per; ++i) {
     const int q = q0 + i;
     if (q < limit) run += cumsum_term(a[(int64_t)q * sa.sl], prob);
-    if (q < Q) {
-      out[q] = run;
-      if (cs2) cs2[chunk_id * Q + q] = run;  // a second copy for the pass that follows
-    }
+    if (q < Q) out[q] = run;
   }
 }
 
@@ -305,7 +302,7 @@ __global__ __launch_bounds__(256) void row_dot_kernel(const T* __restrict__ x, S
     float local = 0.f;
     for (int i = 0; i < per; ++i)
       if (q0 + i < Q) local += rbuf[q0 + i];
-    float run = wave_inclusive_scan(local) - local;
+    float run = wave_exclusive_scan(local);
     for (int i = 0; i < per; ++i) {
       const int q = q0 + i;
       if (q < Q) {
@@ -341,7 +338,7 @@ __global__ __launch_bounds__(256) void combine_dA_kernel(const float* __restrict
     const int p = p0 + i;
     if (p < Q) local += sp[Q - 1 - p] + (p == 0 ? extra : 0.f);
   }
-  float run = wave_inclusive_scan(local) - local;
+  float run = wave_exclusive_scan(local);
   for (int i = 0; i < per; ++i) {
     const int p = p0 + i;
     if (p < Q) {

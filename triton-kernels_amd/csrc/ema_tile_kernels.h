@@ -194,41 +194,43 @@ __device__ __forceinline__ float tile_keep(float coef) {
   return coef;
 }
 
-template <bool REV, int BN>
-__device__ __forceinline__ float tile_look(const u64* status, const float* __restrict__ cs_n, int c,
-                                           int C, int k, unsigned* err) {
-  return chain_look<REV, BN>(status, cs_n, c, C, k, err);
-}
-
 // ------------------------------------------------------------------------------------
 // Forward.  Writes y, prev[n,c,:] (state entering each 128-row chunk), optionally a copy at
-// a coarser chunking and the final state.  With has_init the state before the first row is
-// what the virtual slot of the status words carries.  status: N*ntiles*C*BN zeroed words; counters[0]
-// ticket, counters[3] error word.  One ticket = one tile; the next ticket is fetched while
-// the tile is processed.
+// a coarser chunking and the final state.  init (may be null): the state before the first row,
+// (N, T).  hdr / decw / status: the chained-scan workspace (zero-filled once, see
+// ema_chain_kernels.h); decw has N*C words, status N*ntiles*C*BN.  One ticket = one tile; the
+// next ticket is fetched while the tile is processed.
+//
+// Per tile and column the row groups are combined in one chain of NG steps by the workgroup's
+// first BN threads (one per column), straight after the local pass: the chain leaves in LDS, for
+// every row group, the state entering it if nothing entered the tile, and yields the tile's
+// aggregate, which is published at once.  What the look-back then returns enters every group
+// scaled by the decay of the groups before it, so the final pass starts from two LDS reads.
 // ------------------------------------------------------------------------------------
 template <typename T, int CPL, int RPL, int MINW, bool XP>
 __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
     const T* __restrict__ x, SeqStrides sx, const float* __restrict__ A, SeqStrides sa,
-    const float* __restrict__ cs, T* __restrict__ y, SeqStrides sy, float* __restrict__ prev,
-    float* __restrict__ prev_coarse, int ratio, float* __restrict__ final_state,
-    int has_init, u64* __restrict__ status, unsigned* __restrict__ counters, int nh, int L, int Tdim, int C,
-    int ntiles, int cols, int total) {
+    T* __restrict__ y, SeqStrides sy, float* __restrict__ prev, float* __restrict__ prev_coarse, int ratio,
+    float* __restrict__ final_state, const float* __restrict__ init, ChainHeader* __restrict__ hdr,
+    u64* __restrict__ decw, u64* __restrict__ status, int nh, int L, int Tdim, int C, int ntiles, int cols,
+    int total) {
   using W = TileCfg<T, CPL, RPL>;
   constexpr int BN = W::BN, NW = W::NW, NG = W::NG;
   __shared__ __attribute__((aligned(16))) float sS[2][NG][BN];  // group states, double-buffered by tile
+  __shared__ __attribute__((aligned(16))) float sP[2][BN];      // state entering the tile
   __shared__ float sD[2][NG];                                   // total decay of each row group
+  __shared__ float sW[2][NG];                                   // decay of the groups before each group
   __shared__ int s_ticket[2];
   const int lane = threadIdx.x & 63;
   const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-  unsigned* err = counters + 3;
+  const ChainCtl ctl = chain_enter(hdr);
 
-  if (threadIdx.x == 0) s_ticket[0] = (int)atomicAdd(counters, 1u);
+  if (threadIdx.x == 0) s_ticket[0] = (int)atomicAdd(&hdr->ticket, 1u);
   __syncthreads();
   int cur = s_ticket[0], buf = 0, slot = 1;
   while (cur < total) {
     int future = 0;
-    if (threadIdx.x == 0) future = (int)atomicAdd(counters, 1u);
+    if (threadIdx.x == 0) future = (int)atomicAdd(&hdr->ticket, 1u);
     const ChainTile t = chain_decode<false, BN>(cur, cols, ntiles, C, nh, L);
     const bool cok = t.col0 + lane * CPL < Tdim;
     const int nrows = t.limit - RPL * grp;  // valid rows of this wave (may be <= 0)
@@ -259,37 +261,38 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
     __syncthreads();
     EMA_TSTAMP(1);
 
-    // 2. tile aggregate, look-back, states entering the row groups (one thread per column)
+    // 2. one thread per column: chain over the row groups, publish, look back
     if (threadIdx.x < BN) {
       const int k = threadIdx.x;
-      u64* st = status + (int64_t)t.col_id * (C + 1) * BN;
-      u64* mine = st + (int64_t)chain_slot<false>(t.c) * BN + k;
+      u64* words = status + ((int64_t)t.col_id * C) * BN + k;
+      u64* dws = decw + (int64_t)t.n * C;
       float loc = 0.f, dec = 1.f;
 #pragma unroll
       for (int g = 0; g < NG; ++g) {
-        const float d = sD[buf][g];
-        loc = fmaf(d, loc, sS[buf][g][k]);
-        dec *= d;
+        const float sg = sS[buf][g][k], dg = sD[buf][g];
+        sS[buf][g][k] = loc;
+        if (k == 0) sW[buf][g] = dec;
+        loc = fmaf(dg, loc, sg);
+        dec *= dg;
       }
-      float p_in = 0.f;
-      if (t.c > 0 || has_init) {  // the first tile's only neighbour is the virtual one
-        chain_publish(mine, kFlagAggregate, loc);
-        p_in = tile_look<false, BN>(st, cs + (int64_t)t.n * C * kTileRows, t.c, C, k, err);
+      float p_in;
+      if (t.c > 0) {
+        if (k == 0) chain_publish(dws + t.c, ctl.epoch, kStateAggregate, dec);
+        chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStateAggregate, loc);
+        ChainLook<false, BN> look;
+        look.begin(words, dws, t.c, C);
+        p_in = look.finish(words, dws, C, ctl);
+      } else {
+        p_in = (init && t.col0 + k < Tdim) ? init[(int64_t)t.n * Tdim + t.col0 + k] : 0.f;
       }
       const float p_out = fmaf(dec, p_in, loc);
-      chain_publish(mine, kFlagPrefix, p_out);
+      chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStatePrefix, p_out);
+      sP[buf][k] = p_in;
       if (t.col0 + k < Tdim) {
         prev[(int64_t)t.chunk_id * Tdim + t.col0 + k] = p_in;
         if (prev_coarse && t.c % ratio == 0)
           prev_coarse[((int64_t)t.n * ((C + ratio - 1) / ratio) + t.c / ratio) * Tdim + t.col0 + k] = p_in;
         if (final_state && t.c == C - 1) final_state[(int64_t)t.n * Tdim + t.col0 + k] = p_out;
-      }
-      float E = p_in;
-#pragma unroll
-      for (int g = 0; g < NG; ++g) {
-        const float sg = sS[buf][g][k];
-        sS[buf][g][k] = E;
-        E = fmaf(sD[buf][g], E, sg);
       }
     }
     if (threadIdx.x == 0) s_ticket[slot] = future;
@@ -297,9 +300,10 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
     EMA_TSTAMP(2);
 
     // 3. final pass from the true state
-#pragma unroll
-    for (int e = 0; e < CPL; ++e) s[e] = sS[buf][grp][lane * CPL + e];
     {
+      const float wg = sW[buf][grp];
+#pragma unroll
+      for (int e = 0; e < CPL; ++e) s[e] = fmaf(wg, sP[buf][lane * CPL + e], sS[buf][grp][lane * CPL + e]);
       T* g = y + (int64_t)t.b * sy.sb + (int64_t)t.h * sy.sh +
              ((int64_t)t.c * kTileRows + RPL * grp) * sy.sl + t.col0;
       const unsigned off = (unsigned)lane * CPL;
@@ -315,6 +319,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
     slot ^= 1;
     buf ^= 1;
   }
+  if (threadIdx.x == 0) chain_leave(hdr, ctl);
 }
 
 // ------------------------------------------------------------------------------------
@@ -322,33 +327,41 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
 // the reverse state entering each tile from the rows after it, H = a[next row] * dx[next row],
 // comes from the chained scan over dy, last chunk first.  Writes dx, optionally y, and the
 // column partials part[(chunk*ntiles + ctile)*128 + m] = a[m] * <dx[m], y[m-1]> over the
-// tile's columns (probability form: <r[m], x[m] - y[m-1]>).  With has_dfinal the virtual slot
-// of the status words carries the gradient reaching the state after the last row; dinit (may
-// be null) receives the gradient of the state before the first.  counters[1] ticket, counters[3] error word.
+// tile's columns (probability form: <r[m], x[m] - y[m-1]>).  dfinal (may be null): the gradient
+// reaching the state after the last row, (N, T); dinit (may be null) receives the gradient of
+// the state before the first.
+//
+// After the local passes the first BN threads chain the reverse group states (and publish the
+// aggregate), the next BN threads chain the forward group states from the saved chunk-entry
+// state; the forward values y are then recomputed while the reverse look-back is under way.
 // ------------------------------------------------------------------------------------
 template <typename T, int CPL, int RPL, int MINW, bool WRITE_Y, bool XP>
 __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     const T* __restrict__ x, SeqStrides sx, const T* __restrict__ dy, SeqStrides sd,
-    const float* __restrict__ A, SeqStrides sa, const float* __restrict__ cs,
-    const float* __restrict__ prev, T* __restrict__ dx, SeqStrides sdx, T* __restrict__ y,
-    SeqStrides sy, float* __restrict__ part, int has_dfinal,
-    float* __restrict__ dinit, u64* __restrict__ status, unsigned* __restrict__ counters, int nh, int L, int Tdim, int C, int ntiles, int cols, int total) {
+    const float* __restrict__ A, SeqStrides sa, const float* __restrict__ prev, T* __restrict__ dx,
+    SeqStrides sdx, T* __restrict__ y, SeqStrides sy, float* __restrict__ part,
+    const float* __restrict__ dfinal, float* __restrict__ dinit, ChainHeader* __restrict__ hdr,
+    u64* __restrict__ decw, u64* __restrict__ status, int nh, int L, int Tdim, int C, int ntiles, int cols,
+    int total) {
   using W = TileCfg<T, CPL, RPL>;
-  constexpr int BN = W::BN, NW = W::NW, NG = W::NG;
+  constexpr int BN = W::BN, NW = W::NW, NG = W::NG, NT = W::NT;
+  static_assert(2 * BN <= NT, "one thread per column and direction");
   __shared__ __attribute__((aligned(16))) float sS[2][NG][BN];  // forward group states
   __shared__ __attribute__((aligned(16))) float sR[2][NG][BN];  // reverse group states
+  __shared__ __attribute__((aligned(16))) float sH[2][BN];      // reverse state entering the tile
   __shared__ float sD[2][NG];
+  __shared__ float sW[2][NG];  // decay of the groups after each group
   __shared__ int s_ticket[2];
   const int lane = threadIdx.x & 63;
   const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-  unsigned* err = counters + 3;
+  const ChainCtl ctl = chain_enter(hdr);
 
-  if (threadIdx.x == 0) s_ticket[0] = (int)atomicAdd(counters + 1, 1u);
+  if (threadIdx.x == 0) s_ticket[0] = (int)atomicAdd(&hdr->ticket, 1u);
   __syncthreads();
   int cur = s_ticket[0], buf = 0, slot = 1;
   while (cur < total) {
     int future = 0;
-    if (threadIdx.x == 0) future = (int)atomicAdd(counters + 1, 1u);
+    if (threadIdx.x == 0) future = (int)atomicAdd(&hdr->ticket, 1u);
     const ChainTile t = chain_decode<true, BN>(cur, cols, ntiles, C, nh, L);
     const bool cok = t.col0 + lane * CPL < Tdim;
     const int nrows = t.limit - RPL * grp;
@@ -359,9 +372,10 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
                                 sd.sl, nrows, cok, lane);
     tile_load_rows<T, CPL, RPL, kStreamBwdLoad>(xr, x + (int64_t)t.b * sx.sb + (int64_t)t.h * sx.sh + row0 * sx.sl + t.col0,
                                 sx.sl, nrows, cok, lane);
+    // the threads that will chain the forward group states fetch the state entering the tile
+    const int kf = (int)threadIdx.x - BN;
     float p_in = 0.f;
-    if (threadIdx.x < BN && t.col0 + (int)threadIdx.x < Tdim)
-      p_in = prev[(int64_t)t.chunk_id * Tdim + t.col0 + threadIdx.x];
+    if (kf >= 0 && kf < BN && t.col0 + kf < Tdim) p_in = prev[(int64_t)t.chunk_id * Tdim + t.col0 + kf];
     // a: factor of the state per row; pc: the row's coefficient as tile_step takes it
     float a[RPL], pc[RPL];
     tile_decays<RPL, XP>(pc, A + (int64_t)t.b * sa.sb + (int64_t)t.h * sa.sh + row0 * sa.sl, sa.sl, nrows);
@@ -396,46 +410,42 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     __syncthreads();
     EMA_TSTAMP(1);
 
-    // 2a. publish the reverse aggregate; forward states entering the row groups
-    u64* st = status + (int64_t)t.col_id * (C + 1) * BN;
+    // 2a. chains over the row groups, one thread per column and direction
+    u64* words = status + ((int64_t)t.col_id * C) * BN + (threadIdx.x < BN ? (int)threadIdx.x : 0);
+    u64* dws = decw + (int64_t)t.n * C;
+    const bool last = t.c == C - 1;
     float loc = 0.f, dec = 1.f;
+    ChainLook<true, BN> look;
     if (threadIdx.x < BN) {
       const int k = threadIdx.x;
+      float rg[NG], dg[NG];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) rg[g] = sR[buf][g][k], dg[g] = sD[buf][g];
 #pragma unroll
       for (int g = NG - 1; g >= 0; --g) {
-        const float d = sD[buf][g];
-        loc = fmaf(d, loc, sR[buf][g][k]);
-        dec *= d;
+        sR[buf][g][k] = loc;
+        if (k == 0) sW[buf][g] = dec;
+        loc = fmaf(dg[g], loc, rg[g]);
+        dec *= dg[g];
       }
-      if (t.c < C - 1 || has_dfinal) chain_publish(st + (int64_t)t.c * BN + k, kFlagAggregate, loc);
+      if (!last) {
+        if (k == 0) chain_publish(dws + t.c, ctl.epoch, kStateAggregate, dec);
+        chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStateAggregate, loc);
+        look.begin(words, dws, t.c, C);
+      }
+    } else if (kf < BN) {
+      float sg[NG], dg[NG];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) sg[g] = sS[buf][g][kf], dg[g] = sD[buf][g];
       float E = p_in;
 #pragma unroll
       for (int g = 0; g < NG; ++g) {
-        const float sg = sS[buf][g][k];
-        sS[buf][g][k] = E;
-        E = fmaf(sD[buf][g], E, sg);
+        sS[buf][g][kf] = E;
+        E = fmaf(dg[g], E, sg[g]);
       }
     }
     __syncthreads();
     EMA_TSTAMP(2);
-
-    // 2b. look-back for the reverse state (the waves that own no column go straight on)
-    if (threadIdx.x < BN) {
-      const int k = threadIdx.x;
-      float h_in = 0.f;
-      if (t.c < C - 1 || has_dfinal)
-        h_in = tile_look<true, BN>(st, cs + (int64_t)t.n * C * kTileRows, t.c, C, k, err);
-      const float h_out = fmaf(dec, h_in, loc);
-      chain_publish(st + (int64_t)t.c * BN + k, kFlagPrefix, h_out);
-      if (dinit && t.c == 0 && t.col0 + k < Tdim) dinit[(int64_t)t.n * Tdim + t.col0 + k] = h_out;
-      float G = h_in;
-#pragma unroll
-      for (int g = NG - 1; g >= 0; --g) {
-        const float rg = sR[buf][g][k];
-        sR[buf][g][k] = G;
-        G = fmaf(sD[buf][g], G, rg);
-      }
-    }
 
     // 1c. forward values y from the true state (kept in float32 for the dots)
     float E[CPL];
@@ -457,6 +467,18 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
         if (WRITE_Y && i < nrows && cok) row_store<NW>(g + (int64_t)i * sy.sl + off, row_pack<T, CPL, NW>(s));
       }
     }
+
+    // 2b. the reverse state entering the tile (the waves that own no column go straight on)
+    if (threadIdx.x < BN) {
+      const int k = threadIdx.x;
+      float h_in;
+      if (!last) h_in = look.finish(words, dws, C, ctl);
+      else h_in = (dfinal && t.col0 + k < Tdim) ? dfinal[(int64_t)t.n * Tdim + t.col0 + k] : 0.f;
+      const float h_out = fmaf(dec, h_in, loc);
+      chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStatePrefix, h_out);
+      if (dinit && t.c == 0 && t.col0 + k < Tdim) dinit[(int64_t)t.n * Tdim + t.col0 + k] = h_out;
+      sH[buf][k] = h_in;
+    }
     if (threadIdx.x == 0) s_ticket[slot] = future;
     __syncthreads();
     EMA_TSTAMP(3);
@@ -466,8 +488,9 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
       T* g = dx + (int64_t)t.b * sdx.sb + (int64_t)t.h * sdx.sh + row0 * sdx.sl + t.col0;
       const unsigned off = (unsigned)lane * CPL;
       float dA = 0.f;  // lane i reports row i of the wave
+      const float wg = sW[buf][grp];
 #pragma unroll
-      for (int e = 0; e < CPL; ++e) r[e] = sR[buf][grp][lane * CPL + e];
+      for (int e = 0; e < CPL; ++e) r[e] = fmaf(wg, sH[buf][lane * CPL + e], sR[buf][grp][lane * CPL + e]);
 #pragma unroll
       for (int i = RPL - 1; i >= 0; --i) {
         float dot = 0.f;
@@ -503,6 +526,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     slot ^= 1;
     buf ^= 1;
   }
+  if (threadIdx.x == 0) chain_leave(hdr, ctl);
 }
 
 // out[b, p, h] = sum over the column tiles of part[n, p / 128, tile, p % 128]: the gradient of

@@ -31,7 +31,8 @@ _SIGNATURES = {
     "ema_state_passing_fwd": (c_int, [_P, _P, _I, _I, _P, _P, _I, _I, _I, _P]),
     "ema_scan_fwd": (c_int, _SEQ + [c_int, _P, _P] + _SEQ + [_I, _I, _I, _I, _I, _P]),
     "ema_fwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I]),
-    "ema_fwd": (c_int, _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, _P, c_size_t, _P, c_size_t, _I, _I, _I, _I, _I, _P, _P, _P]),
+    "ema_workspace_clear": (c_int, [_P, c_size_t, _P]),
+    "ema_fwd": (c_int, _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, _P, c_size_t, c_int, _I, _I, _I, _I, _I, _P, _P, _P]),
     "ema_chunk_scan_bwd_dstates": (c_int, _SEQ + [c_int, _P, _P, _I, _I, _I, _I, _I, _P]),
     "ema_state_passing_bwd_workspace_bytes": (c_size_t, [_I, _I, _I]),
     "ema_state_passing_bwd": (c_int, [_P, _P, _I, _I, _P, _P, _P, _P, c_size_t, _I, _I, _I, _P]),
@@ -43,10 +44,10 @@ _SIGNATURES = {
     "ema_bwd_dx_dA_fused_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "ema_bwd_dx_dA_fused": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P] + _SEQ + [_P] + _SEQ + [_P, c_size_t, _I, _I, _I, _I, _P]),
     "ema_bwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I]),
-    "ema_bwd": (c_int, _SEQ + _SEQ + _SEQ + [_P, c_int] + _SEQ + [_P] + _SEQ + [_P, c_size_t, _I, _I, _I, _I, _I, _P, _P, _P]),
+    "ema_bwd": (c_int, _SEQ + _SEQ + _SEQ + [_P, c_int] + _SEQ + [_P] + _SEQ + [_P, c_size_t, c_int, _I, _I, _I, _I, _I, _P, _P, _P]),
     "ema_seq_fwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "ema_seq_bwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
-    "ema_seq_fwd": (c_int, [c_int] + _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, c_size_t, _P, c_size_t, _I, _I, _I, _I, _P, _P, _P]),
+    "ema_seq_fwd": (c_int, [c_int] + _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, c_size_t, c_int, _I, _I, _I, _I, _P, _P, _P]),
     "ema_seq_bwd": (c_int, [c_int] + _SEQ + _SEQ + _SEQ + [_P, _P, c_int] + _SEQ + _SEQ + [_P, _P, c_size_t, c_int, _I, _I, _I, _I, _P, _P, _P]),
     "ema_seq_fwd_static_max_workspace_bytes": (c_size_t, []),
     "ema_seq_fwd_static": (c_int, [c_int] + _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _I, _I, _I, _I, _P]),
@@ -179,21 +180,80 @@ def f32c(t: torch.Tensor) -> torch.Tensor:
     return t.contiguous()
 
 
-class BackwardWorkspace:
-    """Workspace of the ema_seq_bwd call that follows a forward pass, prepared by that forward
-    pass's set-up launch (status words of the reverse scan, cumsum of the coefficient), so that the
-    backward needs no set-up launch of its own.  Good for one backward call: take() hands the
-    buffer out once and reports whether it is still as the forward left it."""
+# ---------------------------------------------------------------------------------------------
+# Workspace of the single-pass entry points.  The library tags every word it writes to the
+# chained part of a workspace with the epoch of the call, so a buffer that was zero-filled once
+# serves every later call without being cleared (workspace_ready = 1: the call is the tile kernel
+# alone).  The wrappers keep one such buffer per device and problem shape (the chained part is
+# laid out by (sequences, 128-row tiles, dim), and only tagged words may ever be written there),
+# shared by the forward and the backward of that shape.  Calls that share a buffer must not
+# overlap in time: code that runs these operators on several streams of one device at once
+# switches to a fresh buffer per call with private_workspaces(True), at the price of one small
+# clearing launch per call.
+# ---------------------------------------------------------------------------------------------
+HEADER_BYTES = 256
+_RECLEAR_AFTER = 1 << 29  # calls; the epoch tag wraps at 2**30
+_MAX_SHARED = 16          # buffers kept (the least recently created goes first)
 
-    def __init__(self, batch: int, nh: int, L: int, T: int, dev: torch.device):
-        self.nbytes = lib().ema_seq_bwd_workspace_bytes(batch, nh, L, T)
-        assert self.nbytes > 0, "unsupported shape"
-        self.buf = torch.empty(self.nbytes, dtype=torch.uint8, device=dev)
-        self.fresh = True
+_shared = {}  # (device index, N, tiles, dim) -> [buffer, calls since the last clear]
+_private = False
 
-    def take(self):
-        fresh, self.fresh = self.fresh, False
-        return self.buf, fresh
+
+def private_workspaces(on: bool) -> None:
+    global _private
+    _private = bool(on)
+
+
+def _clear(buf: torch.Tensor, dev: torch.device) -> None:
+    with torch.cuda.device(dev):
+        check(lib().ema_workspace_clear(buf.data_ptr(), buf.numel(), stream_ptr(dev)), "ema_workspace_clear")
+
+
+def workspace(dev: torch.device, nbytes: int, batch: int, nh: int, L: int, T: int):
+    """(uint8 buffer of at least nbytes, workspace_ready flag) for one call on `dev` of a
+    single-pass entry point on a (batch, L, nh, T) problem."""
+    assert nbytes > 0, "unsupported shape"
+    capturing = torch.cuda.is_current_stream_capturing()
+    key = (dev.index, batch * nh, -(-L // 128), T)
+    entry = _shared.get(key)
+    fits = entry is not None and entry[0].numel() >= nbytes
+    if _private or (capturing and not fits):
+        # under graph capture nothing persistent may be created: the call clears what it uses
+        return torch.empty(nbytes, dtype=torch.uint8, device=dev), 0
+    if not fits:
+        size = max(nbytes, 0 if entry is None else entry[0].numel())
+        _shared.pop(key, None)
+        while len(_shared) >= _MAX_SHARED:
+            _shared.pop(next(iter(_shared)))
+        entry = _shared[key] = [torch.empty(size, dtype=torch.uint8, device=dev), 0]
+        _clear(entry[0], dev)
+    elif entry[1] >= _RECLEAR_AFTER and not capturing:
+        _clear(entry[0], dev)
+        entry[1] = 0
+    entry[1] += 1
+    return entry[0], 1
+
+
+def chain_error(buf: torch.Tensor) -> bool:
+    """Whether a tile's bounded wait ran out in some call on this workspace (synchronises)."""
+    return bool(buf[:HEADER_BYTES].view(torch.int32)[3].item())
+
+
+def check_chain_errors(device=None) -> None:
+    """Raises if any call since the last check gave up waiting for a predecessor tile (the
+    outputs of that call hold NaN).  Reads one word per device back: call it where the program
+    synchronises anyway, not between kernels.  The workspace is cleared after a report."""
+    for key, entry in list(_shared.items()):
+        index = key[0]
+        if device is not None and torch.device(device).index not in (None, index):
+            continue
+        if chain_error(entry[0]):
+            _clear(entry[0], entry[0].device)
+            entry[1] = 0
+            raise RuntimeError(
+                f"EMA chained scan on cuda:{index}: a tile gave up waiting for its predecessor; the "
+                "results of that call are NaN (overlapping calls on one workspace, or a workspace "
+                "that was not ready)")
 
 
 def state_tensor(t: torch.Tensor, like: torch.Tensor = None):

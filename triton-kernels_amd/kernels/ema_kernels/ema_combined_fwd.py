@@ -11,7 +11,7 @@ from kernels import _lib
 
 
 def _ema_matmul_scan_combined_fwd(A_ema, X_ema, chunk_size, dtype=torch.float32, return_prev128=False,
-                                  kernel_events=None, prepare_backward=False):
+                                  kernel_events=None):
     """A_ema: (B, L) or (b, L, nh) float32 log-decay; X_ema: (B, L, T) or (b, L, nh, d).
 
     Returns (out, dA_cumsum (N, C, Q), states entering each chunk (N, C, T), final (N, T)).
@@ -19,9 +19,7 @@ def _ema_matmul_scan_combined_fwd(A_ema, X_ema, chunk_size, dtype=torch.float32,
     return_prev128 a fifth value follows: the states entering each 128-row chunk, which the
     backward accepts to skip their recomputation (None when chunk_size is not a multiple
     of 128).  kernel_events: optional (start, stop) torch.cuda.Event pair recorded around the
-    kernel that reads x.  prepare_backward (chunk_size a multiple of 128): a sixth value
-    follows, the workspace of the backward pass, prepared by this pass's set-up launch
-    (_lib.BackwardWorkspace; kernels.ema_seq.ema_seq_bwd takes it)."""
+    kernel that reads x."""
     dev = _lib.require_gpu(A_ema, X_ema)
     x, x_args, batch, nh, seqlen, token_dim = _lib.seq_view(X_ema)
     a_args, a_batch, a_nh, a_len = _lib.decay_view(A_ema)
@@ -39,24 +37,18 @@ def _ema_matmul_scan_combined_fwd(A_ema, X_ema, chunk_size, dtype=torch.float32,
             N, math.ceil(seqlen / 128), token_dim, device=dev, dtype=torch.float32)
     L = _lib.lib()
     ws_bytes = L.ema_fwd_workspace_bytes(batch, nh, seqlen, token_dim, chunk_size)
-    assert ws_bytes > 0, "unsupported shape"
-    ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
-    bwd_ws = None
-    if prepare_backward and chunk_size % 128 == 0:
-        bwd_ws = _lib.BackwardWorkspace(batch, nh, seqlen, token_dim, dev)
+    ws, ready = _lib.workspace(dev, ws_bytes, batch, nh, seqlen, token_dim)
     with torch.cuda.device(dev):
         st = L.ema_fwd(
             *a_args, *x_args, _lib.dtype_code(x), *y_args, cs.data_ptr(), prev.data_ptr(),
             final.data_ptr(), None if prev128 is None or prev128 is prev else prev128.data_ptr(),
-            ws.data_ptr(), ws_bytes, None if bwd_ws is None else bwd_ws.buf.data_ptr(),
-            0 if bwd_ws is None else bwd_ws.nbytes, batch, nh, seqlen, token_dim, chunk_size,
+            ws.data_ptr(), ws.numel(), ready, batch, nh, seqlen, token_dim, chunk_size,
             _lib.stream_ptr(dev), *_lib.event_ptrs(kernel_events),
         )
     _lib.check(st, "_ema_matmul_scan_combined_fwd")
     if dtype != torch.float32:
         prev = prev.to(dtype)
-    res = (out, cs, prev, final) + ((prev128,) if return_prev128 else ())
-    return res + ((bwd_ws,) if prepare_backward else ())
+    return (out, cs, prev, final) + ((prev128,) if return_prev128 else ())
 
 
 def _unchunk_dA(ddA, A_like, seqlen):
@@ -70,31 +62,38 @@ def _unchunk_dA(ddA, A_like, seqlen):
 
 
 class EMAMatmulCombinedFn(torch.autograd.Function):
+    """forward / backward of ema_matmul_scan_combined.  For chunk sizes that are multiples of 128
+    both directions are one kernel launch each plus the small reduction of the log-decay
+    gradient: the scan does not depend on the chunking, so the sequence-level entry points are
+    used and the chunked intermediates of the reference's forward (which its backward, being
+    unimplemented, never read) are not formed."""
+
     @staticmethod
     def forward(ctx, A_ema, X_ema, chunk_size):
-        wants_grad = any(ctx.needs_input_grad)
-        out, dA_cumsum, states, final_states, prev128, bwd_ws = _ema_matmul_scan_combined_fwd(
-            A_ema, X_ema, chunk_size=chunk_size, return_prev128=True, prepare_backward=True
-        ) if wants_grad else _ema_matmul_scan_combined_fwd(
-            A_ema, X_ema, chunk_size=chunk_size, return_prev128=True) + (None,)
-        ctx.save_for_backward(out, dA_cumsum, states, final_states, A_ema, X_ema)
-        ctx.prev128 = prev128  # a small float32 tensor the backward reuses; not an input or output
-        ctx.bwd_ws = bwd_ws    # the backward's workspace, set up by the forward's set-up launch
         ctx.chunk_size = chunk_size
+        if chunk_size % 128 == 0:
+            from kernels.ema_seq import ema_seq_fwd
+
+            out, _, prev128 = ema_seq_fwd(A_ema, X_ema, form="log_decay")
+            ctx.save_for_backward(A_ema, X_ema, prev128)
+            return out
+        out, dA_cumsum, states, final_states = _ema_matmul_scan_combined_fwd(A_ema, X_ema, chunk_size=chunk_size)
+        ctx.save_for_backward(A_ema, X_ema)
         return out
 
     @staticmethod
     def backward(ctx, dout, *args):
-        from kernels.ema_kernels_bwd.ema_combined_bwd import _ema_chunk_scan_combined_bwd
-
-        out, dA_cumsum, states, final_states, A_ema, X_ema = ctx.saved_tensors
-        if ctx.prev128 is not None:
-            # the same single-pass kernel through the entry point that returns the gradient of the
-            # log-decay in the layout of A itself: nothing to rearrange afterwards
+        if len(ctx.saved_tensors) == 3:
+            # the gradient of the log-decay comes back in the layout of A itself: nothing to
+            # rearrange afterwards
             from kernels.ema_seq import ema_seq_bwd
 
-            dx, dA, _ = ema_seq_bwd(dout, X_ema, A_ema, ctx.prev128, form="log_decay", workspace=ctx.bwd_ws)
+            A_ema, X_ema, prev128 = ctx.saved_tensors
+            dx, dA, _ = ema_seq_bwd(dout, X_ema, A_ema, prev128, form="log_decay")
             return dA, dx, None
+        from kernels.ema_kernels_bwd.ema_combined_bwd import _ema_chunk_scan_combined_bwd
+
+        A_ema, X_ema = ctx.saved_tensors
         dx, ddA = _ema_chunk_scan_combined_bwd(dout, X_ema, A_ema, ctx.chunk_size)
         dA = _unchunk_dA(ddA, A_ema, X_ema.shape[1])
         return dA, dx, None

@@ -42,13 +42,12 @@ def _ema_chunk_scan_combined_bwd(dout, x, A, chunk_size, dt_limit=(0.0, float("i
         y, y_args = None, [None, 0, 0, 0]
     L = _lib.lib()
     ws_bytes = L.ema_bwd_workspace_bytes(batch, nh, seqlen, token_dim, chunk_size)
-    assert ws_bytes > 0, "unsupported shape"
-    ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
+    ws, ready = _lib.workspace(dev, ws_bytes, batch, nh, seqlen, token_dim)
     with torch.cuda.device(dev):
         st = L.ema_bwd(
             *d_args, *x_args, *a_args, None if prev128 is None else prev128.data_ptr(),
             _lib.dtype_code(x), *dx_args, ddA.data_ptr(), *y_args,
-            ws.data_ptr(), ws_bytes, batch, nh, seqlen, token_dim, chunk_size, _lib.stream_ptr(dev),
+            ws.data_ptr(), ws.numel(), ready, batch, nh, seqlen, token_dim, chunk_size, _lib.stream_ptr(dev),
             *_lib.event_ptrs(kernel_events),
         )
     _lib.check(st, "_ema_chunk_scan_combined_bwd")

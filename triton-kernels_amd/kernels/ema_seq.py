@@ -30,10 +30,10 @@ def _state_2d(s, batch, nh, T, name):
     return _lib.f32c(s).reshape(batch * nh, T)
 
 
-def ema_seq_fwd(coef, x, form="log_decay", initial_states=None, kernel_events=None, prepare_backward=False):
+def ema_seq_fwd(coef, x, form="log_decay", initial_states=None, kernel_events=None, workspace=None):
     """Forward pass.  Returns (y, final_states, prev128); prev128 (N, ceil(L/128), T) float32 is
-    what ema_seq_bwd needs from the forward.  With prepare_backward a fourth value follows: the
-    workspace of the backward pass, set up by this pass's set-up launch (pass it to ema_seq_bwd)."""
+    what ema_seq_bwd needs from the forward.  workspace: optional (uint8 buffer, ready flag) to
+    use instead of the device's shared one."""
     dev = _lib.require_gpu(x, coef)
     x, xs, batch, nh, L, T = _lib.seq_view(x)
     cs_, cb, cnh, cL = _lib.decay_view(coef)
@@ -46,28 +46,24 @@ def ema_seq_fwd(coef, x, form="log_decay", initial_states=None, kernel_events=No
     prev128 = torch.empty(N, -(-L // 128), T, dtype=torch.float32, device=dev)
     init = None if initial_states is None else _state_2d(initial_states, batch, nh, T, "initial_states")
     nbytes = lib.ema_seq_fwd_workspace_bytes(batch, nh, L, T)
-    assert nbytes > 0, "unsupported shape"
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-    bwd_ws = _lib.BackwardWorkspace(batch, nh, L, T, dev) if prepare_backward else None
+    ws, ready = _lib.workspace(dev, nbytes, batch, nh, L, T) if workspace is None else workspace
+    assert ws.numel() >= nbytes
     ev0, ev1 = _lib.event_ptrs(kernel_events)
     with torch.cuda.device(dev):
         _lib.check(
             lib.ema_seq_fwd(FORMS[form], *cs_, *xs, _lib.dtype_code(x), *ys,
                             None if init is None else init.data_ptr(), final.data_ptr(),
-                            prev128.data_ptr(), ws.data_ptr(), nbytes,
-                            None if bwd_ws is None else bwd_ws.buf.data_ptr(),
-                            0 if bwd_ws is None else bwd_ws.nbytes, batch, nh, L, T,
+                            prev128.data_ptr(), ws.data_ptr(), ws.numel(), ready, batch, nh, L, T,
                             _lib.stream_ptr(dev), ev0, ev1),
             "ema_seq_fwd")
     final = final.reshape(batch, T) if x.dim() == 3 else final.reshape(batch, nh, T)
-    return (y, final, prev128, bwd_ws) if prepare_backward else (y, final, prev128)
+    return y, final, prev128
 
 
 def ema_seq_bwd(dy, x, coef, prev128, form="log_decay", dfinal_states=None, want_dinit=False,
                 kernel_events=None, workspace=None):
-    """Backward pass.  Returns (dx, dcoef, dinitial_states or None).  workspace: the
-    _lib.BackwardWorkspace a forward pass of the same form and shape prepared; it saves this pass's
-    set-up launch the first time it is used and when no gradient enters through the final state."""
+    """Backward pass.  Returns (dx, dcoef, dinitial_states or None).  workspace: optional
+    (uint8 buffer, ready flag) to use instead of the device's shared one."""
     dev = _lib.require_gpu(dy, x, coef, prev128)
     x, xs, batch, nh, L, T = _lib.seq_view(x)
     if dy.dtype != x.dtype:
@@ -86,21 +82,15 @@ def ema_seq_bwd(dy, x, coef, prev128, form="log_decay", dfinal_states=None, want
     dfin = None if dfinal_states is None else _state_2d(dfinal_states, batch, nh, T, "dfinal_states")
     dinit = torch.empty(N, T, dtype=torch.float32, device=dev) if want_dinit else None
     nbytes = lib.ema_seq_bwd_workspace_bytes(batch, nh, L, T)
-    assert nbytes > 0, "unsupported shape"
-    prepared = False
-    if workspace is not None:
-        assert workspace.nbytes == nbytes and workspace.buf.device == dev
-        ws, prepared = workspace.take()
-        prepared = prepared and dfin is None
-    else:
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    ws, ready = _lib.workspace(dev, nbytes, batch, nh, L, T) if workspace is None else workspace
+    assert ws.numel() >= nbytes
     ev0, ev1 = _lib.event_ptrs(kernel_events)
     with torch.cuda.device(dev):
         _lib.check(
             lib.ema_seq_bwd(FORMS[form], *ds, *xs, *cs_, prev128.data_ptr(),
                             None if dfin is None else dfin.data_ptr(), _lib.dtype_code(x), *dxs, *dcs,
-                            None if dinit is None else dinit.data_ptr(), ws.data_ptr(), nbytes,
-                            int(prepared), batch, nh, L, T, _lib.stream_ptr(dev), ev0, ev1),
+                            None if dinit is None else dinit.data_ptr(), ws.data_ptr(), ws.numel(),
+                            ready, batch, nh, L, T, _lib.stream_ptr(dev), ev0, ev1),
             "ema_seq_bwd")
     if dinit is not None:
         dinit = dinit.reshape(batch, T) if x.dim() == 3 else dinit.reshape(batch, nh, T)
@@ -110,21 +100,21 @@ def ema_seq_bwd(dy, x, coef, prev128, form="log_decay", dfinal_states=None, want
 class EMASeqFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, coef, x, initial_states, form):
-        wants_grad = any(ctx.needs_input_grad)
-        y, final, prev128, bwd_ws = ema_seq_fwd(coef, x, form, initial_states, prepare_backward=True) \
-            if wants_grad else ema_seq_fwd(coef, x, form, initial_states) + (None,)
+        y, final, prev128 = ema_seq_fwd(coef, x, form, initial_states)
         ctx.save_for_backward(coef, x, prev128)
-        ctx.bwd_ws = bwd_ws  # the backward's workspace, set up by the forward's set-up launch
         ctx.form = form
         ctx.has_init = initial_states is not None
         ctx.init_dtype = None if initial_states is None else initial_states.dtype
+        ctx.set_materialize_grads(False)  # an unused final state brings None, not a tensor of zeros
         return y, final
 
     @staticmethod
     def backward(ctx, dy, dfinal):
         coef, x, prev128 = ctx.saved_tensors
+        if dy is None:
+            dy = torch.zeros_like(x)
         dx, dcoef, dinit = ema_seq_bwd(dy.contiguous(), x, coef, prev128, ctx.form,
-                                       dfinal_states=dfinal, want_dinit=ctx.has_init, workspace=ctx.bwd_ws)
+                                       dfinal_states=dfinal, want_dinit=ctx.has_init)
         if dinit is not None:
             dinit = dinit.to(ctx.init_dtype)
         return dcoef, dx, dinit, None
