@@ -265,6 +265,9 @@ void launch_timed(void (*kernel)(Args...), dim3 grid, dim3 block, hipStream_t st
 }
 
 // Workgroups of a persistent kernel that can be resident at once on the current device.
+#ifndef EMA_MAX_WGS_PER_CU  // development knob: cap on the resident workgroups per compute unit
+#define EMA_MAX_WGS_PER_CU 64
+#endif
 template <typename K>
 int resident_blocks(K kernel, int threads, int smem) {
   int dev = 0, ncu = 0, per_cu = 0;
@@ -273,6 +276,7 @@ int resident_blocks(K kernel, int threads, int smem) {
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel),
                                                    threads, smem) != hipSuccess || per_cu < 1)
     per_cu = 1;
+  if (per_cu > EMA_MAX_WGS_PER_CU) per_cu = EMA_MAX_WGS_PER_CU;
   return ncu * per_cu;
 }
 
@@ -315,11 +319,23 @@ int launch_clear(void* base, size_t bytes, hipStream_t st) {
 // Shape of the register-tile single-pass kernels: columns per lane (a tile is 128 rows by
 // 64 times that many columns), rows per lane (128 / RPL waves per workgroup), waves per SIMD
 // the register allocation must allow.
+#ifndef EMA_FWD_SHAPE  // columns per lane, rows per lane, waves per SIMD
+#define EMA_FWD_SHAPE 4, 8, 8
+#endif
+#ifndef EMA_BWD_SHAPE
+#define EMA_BWD_SHAPE 4, 8, 4
+#endif
+struct TileShape {
+  int cpl, rpl, minw;
+};
 struct TileBf16 {
-  static constexpr int FWD_CPL = 4, BWD_CPL = 4, RPL = 8, FWD_MINW = 8, BWD_MINW = 4;
+  static constexpr TileShape F{EMA_FWD_SHAPE}, B{EMA_BWD_SHAPE};
+  static constexpr int FWD_CPL = F.cpl, FWD_RPL = F.rpl, FWD_MINW = F.minw;
+  static constexpr int BWD_CPL = B.cpl, BWD_RPL = B.rpl, BWD_MINW = B.minw;
 };
 struct TileF32 {
-  static constexpr int FWD_CPL = 2, BWD_CPL = 2, RPL = 8, FWD_MINW = 8, BWD_MINW = 4;
+  static constexpr int FWD_CPL = 2, FWD_RPL = 8, FWD_MINW = 8;
+  static constexpr int BWD_CPL = 2, BWD_RPL = 8, BWD_MINW = 4;
 };
 
 // ready: the chained part of the workspace is as a zero fill or an earlier call left it;
@@ -328,14 +344,14 @@ template <typename T, typename S, bool XP>
 int launch_fwd_tile_t(const void* x, SeqStrides sx, const float* A, SeqStrides sa, void* y, SeqStrides sy,
                       float* prev128, float* prev_coarse, int ratio, float* fin, const float* init,
                       void* chain_base, bool ready, const Dims& di, hipStream_t st, void* ev0, void* ev1) {
-  using Cfg = TileCfg<T, S::FWD_CPL, S::RPL>;
+  using Cfg = TileCfg<T, S::FWD_CPL, S::FWD_RPL>;
   constexpr int BN = Cfg::BN, NT = Cfg::NT;
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
   if (!ready) EMA_TRY(launch_clear(chain_base, chain_ws_bytes(di), st));
   const ChainWs w = chain_carve(chain_base, di);
-  auto kernel = fwd_tile_kernel<T, S::FWD_CPL, S::RPL, S::FWD_MINW, XP>;
+  auto kernel = fwd_tile_kernel<T, S::FWD_CPL, S::FWD_RPL, S::FWD_MINW, XP>;
   const int64_t cap = resident_blocks(kernel, NT, 0);
   launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx, A,
                sa, (T*)y, sy, prev128, prev_coarse, ratio, fin, init, w.hdr, w.decw, w.status, (int)di.nh,
@@ -348,14 +364,14 @@ int launch_bwd_tile_k(const void* x, SeqStrides sx, const void* dy, SeqStrides s
                       SeqStrides sa, const float* prev128, void* dx, SeqStrides sdx, void* y, SeqStrides sy,
                       float* part, const float* dfinal, float* dinit, void* chain_base, bool ready,
                       const Dims& di, hipStream_t st, void* ev0, void* ev1) {
-  using Cfg = TileCfg<T, S::BWD_CPL, S::RPL>;
+  using Cfg = TileCfg<T, S::BWD_CPL, S::BWD_RPL>;
   constexpr int BN = Cfg::BN, NT = Cfg::NT;
   const int ntiles = (int)((di.T + BN - 1) / BN);
   const int64_t cols = di.N * ntiles, total = cols * di.C;
   if (total > 0x7fffffff) return EMA_ERR_SHAPE;
   if (!ready) EMA_TRY(launch_clear(chain_base, chain_ws_bytes(di), st));
   const ChainWs w = chain_carve(chain_base, di);
-  auto kernel = bwd_tile_kernel<T, S::BWD_CPL, S::RPL, S::BWD_MINW, WRITE_Y, XP>;
+  auto kernel = bwd_tile_kernel<T, S::BWD_CPL, S::BWD_RPL, S::BWD_MINW, WRITE_Y, XP>;
   const int64_t cap = resident_blocks(kernel, NT, 0);
   launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx,
                (const T*)dy, sd, A, sa, prev128, (T*)dx, sdx, (T*)y, sy, part, dfinal, dinit, w.hdr, w.decw,

@@ -49,7 +49,6 @@ constexpr unsigned kStateAggregate = 1u;
 constexpr unsigned kStatePrefix = 2u;
 constexpr unsigned kSpinLimitDefault = 1u << 20;
 constexpr unsigned kEpochMask = 0x3fffffffu;
-constexpr int kLookWindow = 4;  // predecessors whose words are requested together
 
 // Epoch of the launch that finds `last` in the header: 1 .. 2^30 - 1, never 0 (the tag of
 // zero-filled memory).
@@ -152,16 +151,17 @@ __device__ __forceinline__ ChainTile chain_decode(int ticket, int cols, int ntil
 // total decay of tile j of this sequence.  The walk starts at the neighbour of tile c (c - 1
 // forward, c + 1 reverse) and ends at the first PREFIX; the first tile of a scan always
 // publishes one, so the walk stays inside [0, C).
-template <bool REV, int BN>
+// W: predecessors whose words are requested together.
+template <bool REV, int BN, int W>
 struct ChainLook {
-  u64 w[kLookWindow], d[kLookWindow];
+  u64 w[W], d[W];
   int j;  // neighbour the window starts at
 
   __device__ __forceinline__ int clampj(int jj, int C) const { return REV ? min(jj, C - 1) : max(jj, 0); }
 
   __device__ __forceinline__ void request(const u64* words, const u64* decw, int C) {
 #pragma unroll
-    for (int i = 0; i < kLookWindow; ++i) {
+    for (int i = 0; i < W; ++i) {
       const int jj = clampj(REV ? j + i : j - i, C);
       w[i] = chain_peek(words + (int64_t)jj * BN);
       d[i] = chain_peek(decw + jj);
@@ -175,7 +175,7 @@ struct ChainLook {
     float carry = 0.f, scale = 1.f;
     for (;;) {
 #pragma unroll
-      for (int i = 0; i < kLookWindow; ++i) {
+      for (int i = 0; i < W; ++i) {
         const int jj = REV ? j + i : j - i;
         if (REV ? jj >= C : jj < 0) return carry;
         const u64 sw = chain_wait(words + (int64_t)jj * BN, w[i], ctl);
@@ -183,7 +183,7 @@ struct ChainLook {
         if (chain_state(sw, ctl.epoch) == kStatePrefix) return carry;
         scale *= chain_value(chain_wait(decw + jj, d[i], ctl));
       }
-      j += REV ? kLookWindow : -kLookWindow;
+      j += REV ? W : -W;
       request(words, decw, C);
     }
   }

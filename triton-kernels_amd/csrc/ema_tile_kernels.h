@@ -37,12 +37,33 @@
 namespace ema {
 
 #ifdef EMA_TIMING
-#define EMA_TSTAMP(slot)                                                                            \
-  do {                                                                                              \
-    if (threadIdx.x == 0 && g_ema_timing) g_ema_timing[(int64_t)cur * 8 + (slot)] = wall_clock64(); \
+// Development builds only: thread 0 keeps up to 8 timestamps per tile in registers and writes them
+// out when the tile is finished, so that taking a stamp waits for nothing.
+#define EMA_TSTAMP_DECL long long ema_ts[8] = {0, 0, 0, 0, 0, 0, 0, 0}
+#define EMA_TSTAMP(slot)                               \
+  do {                                                 \
+    if (threadIdx.x == 0) ema_ts[slot] = wall_clock64(); \
+  } while (0)
+#define EMA_TSTAMP_VALUE(slot, v)       \
+  do {                                  \
+    if (threadIdx.x == 0) ema_ts[slot] = (v); \
+  } while (0)
+#define EMA_TSTAMP_FLUSH                                                    \
+  do {                                                                      \
+    if (threadIdx.x == 0 && g_ema_timing)                                   \
+      for (int q = 0; q < 8; ++q) g_ema_timing[(int64_t)cur * 8 + q] = ema_ts[q]; \
   } while (0)
 #else
+#define EMA_TSTAMP_DECL \
+  do {                  \
+  } while (0)
 #define EMA_TSTAMP(slot) \
+  do {                   \
+  } while (0)
+#define EMA_TSTAMP_VALUE(slot, v) \
+  do {                            \
+  } while (0)
+#define EMA_TSTAMP_FLUSH \
   do {                   \
   } while (0)
 #endif
@@ -57,13 +78,19 @@ namespace ema {
 constexpr bool kStreamFwdLoad = (EMA_STREAM_FLAGS & 1) != 0, kStreamFwdStore = (EMA_STREAM_FLAGS & 2) != 0,
                kStreamBwdLoad = (EMA_STREAM_FLAGS & 4) != 0, kStreamBwdStore = (EMA_STREAM_FLAGS & 8) != 0;
 
+// Predecessors whose words a look-back requests together (the forward runs at 64 registers).
+#ifndef EMA_FWD_LOOK_WINDOW
+#define EMA_FWD_LOOK_WINDOW 3
+#endif
+constexpr int kFwdLookWindow = EMA_FWD_LOOK_WINDOW, kBwdLookWindow = 4;
+
 template <typename T, int CPL, int RPL>
 struct TileCfg {
   static constexpr int NG = kTileRows / RPL;            // row groups = waves of the workgroup
   static constexpr int NT = 64 * NG;                    // threads
   static constexpr int BN = 64 * CPL;                   // columns of a tile
   static constexpr int NW = CPL * (int)sizeof(T) / 4;   // 32-bit words of one lane's row
-  static_assert(NW == 2 || NW == 4, "a lane's row is 8 or 16 bytes");
+  static_assert(NW == 1 || NW == 2 || NW == 4, "a lane's row is 4, 8 or 16 bytes");
   static_assert(NG * RPL == kTileRows && NG <= 16 && BN <= NT, "tile shape");
 };
 
@@ -82,10 +109,13 @@ __device__ __forceinline__ RowWords<NW> row_load(const void* p) {
     const uintx4 v = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const uintx4*>(p))
                             : *reinterpret_cast<const uintx4*>(p);
     r.w[0] = v[0], r.w[1] = v[1], r.w[2] = v[2], r.w[3] = v[3];
-  } else {
+  } else if constexpr (NW == 2) {
     const uintx2 v = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const uintx2*>(p))
                             : *reinterpret_cast<const uintx2*>(p);
     r.w[0] = v[0], r.w[1] = v[1];
+  } else {
+    r.w[0] = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const unsigned*>(p))
+                    : *reinterpret_cast<const unsigned*>(p);
   }
   return r;
 }
@@ -95,10 +125,13 @@ __device__ __forceinline__ void row_store(void* p, const RowWords<NW>& r) {
     const uintx4 v = {r.w[0], r.w[1], r.w[2], r.w[3]};
     if (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<uintx4*>(p));
     else *reinterpret_cast<uintx4*>(p) = v;
-  } else {
+  } else if constexpr (NW == 2) {
     const uintx2 v = {r.w[0], r.w[1]};
     if (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<uintx2*>(p));
     else *reinterpret_cast<uintx2*>(p) = v;
+  } else {
+    if (STREAM) __builtin_nontemporal_store(r.w[0], reinterpret_cast<unsigned*>(p));
+    else *reinterpret_cast<unsigned*>(p) = r.w[0];
   }
 }
 template <int NW>
@@ -146,34 +179,45 @@ __device__ __forceinline__ void rows_opaque(RowWords<NW>* rows) {
     for (int k = 0; k < NW; ++k) asm volatile("" : "+v"(rows[i].w[k]));
 }
 
-// The RPL rows of this lane.  g points at (first row of the wave, first column of the tile);
-// rows at or past `nrows` and columns past the end read as 0.
-template <typename T, int CPL, int RPL, bool STREAM = false>
-__device__ __forceinline__ void tile_load_rows(RowWords<TileCfg<T, CPL, RPL>::NW>* rows,
-                                               const T* __restrict__ g, int64_t sl, int nrows, bool cok,
-                                               int lane) {
-  constexpr int NW = TileCfg<T, CPL, RPL>::NW;
-  const unsigned off = (unsigned)lane * CPL;
-  if (nrows >= RPL && __all(cok)) {
-#pragma unroll
-    for (int i = 0; i < RPL; ++i) rows[i] = row_load<NW, STREAM>(g + (int64_t)i * sl + off);
-  } else {
-#pragma unroll
-    for (int i = 0; i < RPL; ++i)
-      rows[i] = (i < nrows && cok) ? row_load<NW, STREAM>(g + (int64_t)i * sl + off) : row_zero<NW>();
-  }
+// Where a workgroup finds its part of a tile of a sequence tensor.
+struct TileAt {
+  int nrows;  // valid rows of this wave (may be <= 0)
+  bool cok;   // this lane's columns lie inside the tensor
+  bool full;  // all rows and all lanes of the wave are inside: no per-row predicates needed
+};
+template <int RPL>
+__device__ __forceinline__ TileAt tile_at(int limit, int grp, bool cok) {
+  TileAt a;
+  a.nrows = limit - RPL * grp;
+  a.cok = cok;
+  a.full = a.nrows >= RPL && __all(cok);
+  return a;
+}
+// Row i of this lane: g points at (first row of the wave, this lane's first column).  Rows at or
+// past nrows and columns past the end read as 0.
+template <int NW, bool STREAM, typename T>
+__device__ __forceinline__ RowWords<NW> tile_load_row(const T* __restrict__ g, int64_t sl, int i, const TileAt& at) {
+  if (at.full) return row_load<NW, STREAM>(g + (int64_t)i * sl);
+  return (i < at.nrows && at.cok) ? row_load<NW, STREAM>(g + (int64_t)i * sl) : row_zero<NW>();
 }
 
-// Row coefficients of the wave's rows; the addresses are uniform over the wave.  Log-decay
-// form: a[i] = exp(min(A[row], 0)), 1 past the end of the sequence.  Probability form:
-// a[i] = p[row], 0 past the end.
-template <int RPL, bool XP>
-__device__ __forceinline__ void tile_decays(float* a, const float* __restrict__ A, int64_t a_sl, int nrows) {
+// A value that is the same in every lane, moved to a scalar register.
+__device__ __forceinline__ float wave_uniform(float v) {
+  return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
+}
+
+// Raw coefficients of the wave's RPL rows (uniform addresses), requested ahead of their use;
+// rows at or past nrows get the neutral value (log-decay 0, probability 0).
+template <int RPL>
+__device__ __forceinline__ void tile_coef_load(float* raw, const float* __restrict__ A, int64_t a_sl, int nrows) {
 #pragma unroll
-  for (int i = 0; i < RPL; ++i) {
-    if (XP) a[i] = i < nrows ? A[(int64_t)i * a_sl] : 0.f;
-    else a[i] = i < nrows ? __expf(fminf(A[(int64_t)i * a_sl], 0.f)) : 1.f;
-  }
+  for (int i = 0; i < RPL; ++i) raw[i] = i < nrows ? A[(int64_t)i * a_sl] : 0.f;
+}
+// Log-decay form: a[i] = exp(min(A[row], 0)).  Probability form: a[i] = p[row].  Scalar registers.
+template <int RPL, bool XP>
+__device__ __forceinline__ void tile_decays(float* a, const float* raw) {
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) a[i] = wave_uniform(XP ? raw[i] : __expf(fminf(raw[i], 0.f)));
 }
 
 // Probability form: the sign bit of a coefficient marks the first position of a packed sequence.
@@ -223,26 +267,34 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
   __shared__ int s_ticket[2];
   const int lane = threadIdx.x & 63;
   const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const unsigned off = (unsigned)lane * CPL;
   const ChainCtl ctl = chain_enter(hdr);
 
   if (threadIdx.x == 0) s_ticket[0] = (int)atomicAdd(&hdr->ticket, 1u);
   __syncthreads();
   int cur = s_ticket[0], buf = 0, slot = 1;
+  // The rows of a tile are requested while the tile before is being stored (row i of the next
+  // tile goes into the registers that row i of this one has just left), so that loads and stores
+  // are under way together; the first tile's rows are requested here.
+  RowWords<NW> rows[RPL];
+  float araw[RPL];
+  ChainTile t = chain_decode<false, BN>(cur < total ? cur : 0, cols, ntiles, C, nh, L);
+  TileAt at = tile_at<RPL>(t.limit, grp, t.col0 + lane * CPL < Tdim);
+  if (cur < total) {
+    const T* g = x + (int64_t)t.b * sx.sb + (int64_t)t.h * sx.sh +
+                 ((int64_t)t.c * kTileRows + RPL * grp) * sx.sl + t.col0 + off;
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) rows[i] = tile_load_row<NW, kStreamFwdLoad>(g, sx.sl, i, at);
+    tile_coef_load<RPL>(araw, A + (int64_t)t.b * sa.sb + (int64_t)t.h * sa.sh +
+                                  ((int64_t)t.c * kTileRows + RPL * grp) * sa.sl, sa.sl, at.nrows);
+  }
   while (cur < total) {
     int future = 0;
     if (threadIdx.x == 0) future = (int)atomicAdd(&hdr->ticket, 1u);
-    const ChainTile t = chain_decode<false, BN>(cur, cols, ntiles, C, nh, L);
-    const bool cok = t.col0 + lane * CPL < Tdim;
-    const int nrows = t.limit - RPL * grp;  // valid rows of this wave (may be <= 0)
+    EMA_TSTAMP_DECL;
     EMA_TSTAMP(0);
-    RowWords<NW> rows[RPL];
-    tile_load_rows<T, CPL, RPL, kStreamFwdLoad>(rows, x + (int64_t)t.b * sx.sb + (int64_t)t.h * sx.sh +
-                                          ((int64_t)t.c * kTileRows + RPL * grp) * sx.sl + t.col0,
-                                sx.sl, nrows, cok, lane);
     float a[RPL];
-    tile_decays<RPL, XP>(a, A + (int64_t)t.b * sa.sb + (int64_t)t.h * sa.sh +
-                                ((int64_t)t.c * kTileRows + RPL * grp) * sa.sl,
-                         sa.sl, nrows);
+    tile_decays<RPL, XP>(a, araw);
     // 1. local pass
     float s[CPL];
     float D = 1.f;
@@ -266,22 +318,39 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
       const int k = threadIdx.x;
       u64* words = status + ((int64_t)t.col_id * C) * BN + k;
       u64* dws = decw + (int64_t)t.n * C;
+      // all reads first (the group decays are the same for every column: scalar registers),
+      // then the chain: otherwise every step waits for its own LDS read
+      float sg[NG], dg[NG];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) sg[g] = sS[buf][g][k];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) dg[g] = wave_uniform(sD[buf][g]);
       float loc = 0.f, dec = 1.f;
 #pragma unroll
       for (int g = 0; g < NG; ++g) {
-        const float sg = sS[buf][g][k], dg = sD[buf][g];
         sS[buf][g][k] = loc;
         if (k == 0) sW[buf][g] = dec;
-        loc = fmaf(dg, loc, sg);
-        dec *= dg;
+        loc = fmaf(dg[g], loc, sg[g]);
+        dec *= dg[g];
       }
       float p_in;
+#ifdef EMA_EXP_NO_LOOK
+      if (false) {
+#else
       if (t.c > 0) {
+#endif
         if (k == 0) chain_publish(dws + t.c, ctl.epoch, kStateAggregate, dec);
         chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStateAggregate, loc);
-        ChainLook<false, BN> look;
+        ChainLook<false, BN, kFwdLookWindow> look;
+        EMA_TSTAMP(4);
         look.begin(words, dws, t.c, C);
+#ifdef EMA_TIMING
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        EMA_TSTAMP(5);
+        EMA_TSTAMP_VALUE(7, chain_state(look.w[0], ctl.epoch) * 10 + chain_state(look.w[1], ctl.epoch));
+#endif
         p_in = look.finish(words, dws, C, ctl);
+        EMA_TSTAMP(6);
       } else {
         p_in = (init && t.col0 + k < Tdim) ? init[(int64_t)t.n * Tdim + t.col0 + k] : 0.f;
       }
@@ -299,23 +368,36 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
     __syncthreads();
     EMA_TSTAMP(2);
 
-    // 3. final pass from the true state
+    // 3. final pass from the true state; behind each stored row the same row of the next tile
+    // is requested
+    const int next = s_ticket[slot];
+    const bool more = next < total;
+    const ChainTile tn = chain_decode<false, BN>(more ? next : 0, cols, ntiles, C, nh, L);
+    const TileAt atn = tile_at<RPL>(tn.limit, grp, tn.col0 + lane * CPL < Tdim);
     {
       const float wg = sW[buf][grp];
 #pragma unroll
       for (int e = 0; e < CPL; ++e) s[e] = fmaf(wg, sP[buf][lane * CPL + e], sS[buf][grp][lane * CPL + e]);
       T* g = y + (int64_t)t.b * sy.sb + (int64_t)t.h * sy.sh +
-             ((int64_t)t.c * kTileRows + RPL * grp) * sy.sl + t.col0;
-      const unsigned off = (unsigned)lane * CPL;
+             ((int64_t)t.c * kTileRows + RPL * grp) * sy.sl + t.col0 + off;
+      const T* gn = x + (int64_t)tn.b * sx.sb + (int64_t)tn.h * sx.sh +
+                    ((int64_t)tn.c * kTileRows + RPL * grp) * sx.sl + tn.col0 + off;
 #pragma unroll
       for (int i = 0; i < RPL; ++i) {
 #pragma unroll
         for (int e = 0; e < CPL; ++e) s[e] = tile_step<XP>(a[i], s[e], row_get<T, NW>(rows[i], e));
-        if (i < nrows && cok) row_store<NW, kStreamFwdStore>(g + (int64_t)i * sy.sl + off, row_pack<T, CPL, NW>(s));
+        if (i < at.nrows && at.cok) row_store<NW, kStreamFwdStore>(g + (int64_t)i * sy.sl, row_pack<T, CPL, NW>(s));
+        if (more) rows[i] = tile_load_row<NW, kStreamFwdLoad>(gn, sx.sl, i, atn);
       }
+      if (more)
+        tile_coef_load<RPL>(araw, A + (int64_t)tn.b * sa.sb + (int64_t)tn.h * sa.sh +
+                                      ((int64_t)tn.c * kTileRows + RPL * grp) * sa.sl, sa.sl, atn.nrows);
     }
     EMA_TSTAMP(3);
-    cur = s_ticket[slot];
+    EMA_TSTAMP_FLUSH;
+    cur = next;
+    t = tn;
+    at = atn;
     slot ^= 1;
     buf ^= 1;
   }
@@ -334,6 +416,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
 // After the local passes the first BN threads chain the reverse group states (and publish the
 // aggregate), the next BN threads chain the forward group states from the saved chunk-entry
 // state; the forward values y are then recomputed while the reverse look-back is under way.
+// As in the forward, the rows of the next tile are requested behind the stores of this one.
 // ------------------------------------------------------------------------------------
 template <typename T, int CPL, int RPL, int MINW, bool WRITE_Y, bool XP>
 __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
@@ -354,31 +437,38 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
   __shared__ int s_ticket[2];
   const int lane = threadIdx.x & 63;
   const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const unsigned off = (unsigned)lane * CPL;
+  const int kf = (int)threadIdx.x - BN;  // column of the threads that chain the forward group states
   const ChainCtl ctl = chain_enter(hdr);
 
   if (threadIdx.x == 0) s_ticket[0] = (int)atomicAdd(&hdr->ticket, 1u);
   __syncthreads();
   int cur = s_ticket[0], buf = 0, slot = 1;
+  RowWords<NW> dr[RPL], xr[RPL];
+  float araw[RPL];
+  float p_in = 0.f;
+  ChainTile t = chain_decode<true, BN>(cur < total ? cur : 0, cols, ntiles, C, nh, L);
+  TileAt at = tile_at<RPL>(t.limit, grp, t.col0 + lane * CPL < Tdim);
+  if (cur < total) {
+    const int64_t row0 = (int64_t)t.c * kTileRows + RPL * grp;
+    const T* gd = dy + (int64_t)t.b * sd.sb + (int64_t)t.h * sd.sh + row0 * sd.sl + t.col0 + off;
+    const T* gx = x + (int64_t)t.b * sx.sb + (int64_t)t.h * sx.sh + row0 * sx.sl + t.col0 + off;
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) dr[i] = tile_load_row<NW, kStreamBwdLoad>(gd, sd.sl, i, at);
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) xr[i] = tile_load_row<NW, kStreamBwdLoad>(gx, sx.sl, i, at);
+    tile_coef_load<RPL>(araw, A + (int64_t)t.b * sa.sb + (int64_t)t.h * sa.sh + row0 * sa.sl, sa.sl, at.nrows);
+    if (kf >= 0 && kf < BN && t.col0 + kf < Tdim) p_in = prev[(int64_t)t.chunk_id * Tdim + t.col0 + kf];
+  }
   while (cur < total) {
     int future = 0;
     if (threadIdx.x == 0) future = (int)atomicAdd(&hdr->ticket, 1u);
-    const ChainTile t = chain_decode<true, BN>(cur, cols, ntiles, C, nh, L);
-    const bool cok = t.col0 + lane * CPL < Tdim;
-    const int nrows = t.limit - RPL * grp;
+    EMA_TSTAMP_DECL;
     EMA_TSTAMP(0);
-    RowWords<NW> dr[RPL], xr[RPL];
     const int64_t row0 = (int64_t)t.c * kTileRows + RPL * grp;
-    tile_load_rows<T, CPL, RPL, kStreamBwdLoad>(dr, dy + (int64_t)t.b * sd.sb + (int64_t)t.h * sd.sh + row0 * sd.sl + t.col0,
-                                sd.sl, nrows, cok, lane);
-    tile_load_rows<T, CPL, RPL, kStreamBwdLoad>(xr, x + (int64_t)t.b * sx.sb + (int64_t)t.h * sx.sh + row0 * sx.sl + t.col0,
-                                sx.sl, nrows, cok, lane);
-    // the threads that will chain the forward group states fetch the state entering the tile
-    const int kf = (int)threadIdx.x - BN;
-    float p_in = 0.f;
-    if (kf >= 0 && kf < BN && t.col0 + kf < Tdim) p_in = prev[(int64_t)t.chunk_id * Tdim + t.col0 + kf];
     // a: factor of the state per row; pc: the row's coefficient as tile_step takes it
     float a[RPL], pc[RPL];
-    tile_decays<RPL, XP>(pc, A + (int64_t)t.b * sa.sb + (int64_t)t.h * sa.sh + row0 * sa.sl, sa.sl, nrows);
+    tile_decays<RPL, XP>(pc, araw);
 #pragma unroll
     for (int i = 0; i < RPL; ++i) a[i] = tile_keep<XP>(pc[i]);
 
@@ -415,12 +505,14 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     u64* dws = decw + (int64_t)t.n * C;
     const bool last = t.c == C - 1;
     float loc = 0.f, dec = 1.f;
-    ChainLook<true, BN> look;
+    ChainLook<true, BN, kBwdLookWindow> look;
     if (threadIdx.x < BN) {
       const int k = threadIdx.x;
       float rg[NG], dg[NG];
 #pragma unroll
-      for (int g = 0; g < NG; ++g) rg[g] = sR[buf][g][k], dg[g] = sD[buf][g];
+      for (int g = 0; g < NG; ++g) rg[g] = sR[buf][g][k];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) dg[g] = wave_uniform(sD[buf][g]);
 #pragma unroll
       for (int g = NG - 1; g >= 0; --g) {
         sR[buf][g][k] = loc;
@@ -436,7 +528,9 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     } else if (kf < BN) {
       float sg[NG], dg[NG];
 #pragma unroll
-      for (int g = 0; g < NG; ++g) sg[g] = sS[buf][g][kf], dg[g] = sD[buf][g];
+      for (int g = 0; g < NG; ++g) sg[g] = sS[buf][g][kf];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) dg[g] = wave_uniform(sD[buf][g]);
       float E = p_in;
 #pragma unroll
       for (int g = 0; g < NG; ++g) {
@@ -453,8 +547,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     for (int e = 0; e < CPL; ++e) E[e] = sS[buf][grp][lane * CPL + e];
     float yv[RPL][CPL];
     {
-      T* g = WRITE_Y ? y + (int64_t)t.b * sy.sb + (int64_t)t.h * sy.sh + row0 * sy.sl + t.col0 : nullptr;
-      const unsigned off = (unsigned)lane * CPL;
+      T* g = WRITE_Y ? y + (int64_t)t.b * sy.sb + (int64_t)t.h * sy.sh + row0 * sy.sl + t.col0 + off : nullptr;
 #pragma unroll
       for (int e = 0; e < CPL; ++e) s[e] = E[e];
 #pragma unroll
@@ -464,7 +557,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
           s[e] = tile_step<XP>(pc[i], s[e], row_get<T, NW>(xr[i], e));
           yv[i][e] = s[e];
         }
-        if (WRITE_Y && i < nrows && cok) row_store<NW>(g + (int64_t)i * sy.sl + off, row_pack<T, CPL, NW>(s));
+        if (WRITE_Y && i < at.nrows && at.cok) row_store<NW>(g + (int64_t)i * sy.sl, row_pack<T, CPL, NW>(s));
       }
     }
 
@@ -483,10 +576,17 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     __syncthreads();
     EMA_TSTAMP(3);
 
-    // 3. final reverse pass: dx, and the dots with the row before
+    // 3. final reverse pass: dx, and the dots with the row before; behind each stored row the
+    // same rows of the next tile are requested
+    const int next = s_ticket[slot];
+    const bool more = next < total;
+    const ChainTile tn = chain_decode<true, BN>(more ? next : 0, cols, ntiles, C, nh, L);
+    const TileAt atn = tile_at<RPL>(tn.limit, grp, tn.col0 + lane * CPL < Tdim);
     {
-      T* g = dx + (int64_t)t.b * sdx.sb + (int64_t)t.h * sdx.sh + row0 * sdx.sl + t.col0;
-      const unsigned off = (unsigned)lane * CPL;
+      T* g = dx + (int64_t)t.b * sdx.sb + (int64_t)t.h * sdx.sh + row0 * sdx.sl + t.col0 + off;
+      const int64_t rown = (int64_t)tn.c * kTileRows + RPL * grp;
+      const T* gd = dy + (int64_t)tn.b * sd.sb + (int64_t)tn.h * sd.sh + rown * sd.sl + tn.col0 + off;
+      const T* gx = x + (int64_t)tn.b * sx.sb + (int64_t)tn.h * sx.sh + rown * sx.sl + tn.col0 + off;
       float dA = 0.f;  // lane i reports row i of the wave
       const float wg = sW[buf][grp];
 #pragma unroll
@@ -507,9 +607,13 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
           float o[CPL];
 #pragma unroll
           for (int e = 0; e < CPL; ++e) o[e] = fabsf(pc[i]) * r[e];
-          if (i < nrows && cok) row_store<NW, kStreamBwdStore>(g + (int64_t)i * sdx.sl + off, row_pack<T, CPL, NW>(o));
+          if (i < at.nrows && at.cok) row_store<NW, kStreamBwdStore>(g + (int64_t)i * sdx.sl, row_pack<T, CPL, NW>(o));
         } else {
-          if (i < nrows && cok) row_store<NW, kStreamBwdStore>(g + (int64_t)i * sdx.sl + off, row_pack<T, CPL, NW>(r));
+          if (i < at.nrows && at.cok) row_store<NW, kStreamBwdStore>(g + (int64_t)i * sdx.sl, row_pack<T, CPL, NW>(r));
+        }
+        if (more) {
+          dr[i] = tile_load_row<NW, kStreamBwdLoad>(gd, sd.sl, i, atn);
+          xr[i] = tile_load_row<NW, kStreamBwdLoad>(gx, sx.sl, i, atn);
         }
 #pragma unroll
         for (int e = 0; e < CPL; ++e) r[e] *= a[i];
@@ -519,10 +623,17 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
         if (lane == i) dA = dot;
       }
       if (lane < RPL)
-        part[((int64_t)t.chunk_id * ntiles + t.ctile) * kTileRows + RPL * grp + lane] = lane < nrows ? dA : 0.f;
+        part[((int64_t)t.chunk_id * ntiles + t.ctile) * kTileRows + RPL * grp + lane] = lane < at.nrows ? dA : 0.f;
+      if (more) {
+        tile_coef_load<RPL>(araw, A + (int64_t)tn.b * sa.sb + (int64_t)tn.h * sa.sh + rown * sa.sl, sa.sl, atn.nrows);
+        p_in = (kf >= 0 && kf < BN && tn.col0 + kf < Tdim) ? prev[(int64_t)tn.chunk_id * Tdim + tn.col0 + kf] : 0.f;
+      }
     }
     EMA_TSTAMP(4);
-    cur = s_ticket[slot];
+    EMA_TSTAMP_FLUSH;
+    cur = next;
+    t = tn;
+    at = atn;
     slot ^= 1;
     buf ^= 1;
   }

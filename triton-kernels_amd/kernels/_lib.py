@@ -12,7 +12,8 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libema_hip.so")
+# EMA_HIP_LIB names another build of the library (same ABI), e.g. one with a different tile shape
+LIB_PATH = os.environ.get("EMA_HIP_LIB") or os.path.join(os.path.dirname(_HERE), "lib", "libema_hip.so")
 
 EMA_F32, EMA_BF16 = 0, 1
 EMA_FORM_LOG_DECAY, EMA_FORM_PROBABILITY = 0, 1
