@@ -146,45 +146,34 @@ __device__ __forceinline__ ChainTile chain_decode(int ticket, int cols, int ntil
   return t;
 }
 
-// Look-back of one column, in two parts so that other work can sit between the requests and
-// their use.  words: the status words of this column, words[j * BN] that of tile j; decw[j]: the
+// Look-back of one column, in two parts so that other work can sit between the first request and
+// its use.  words: the status words of this column, words[j * BN] that of tile j; decw[j]: the
 // total decay of tile j of this sequence.  The walk starts at the neighbour of tile c (c - 1
 // forward, c + 1 reverse) and ends at the first PREFIX; the first tile of a scan always
-// publishes one, so the walk stays inside [0, C).
-// W: predecessors whose words are requested together.
-template <bool REV, int BN, int W>
+// publishes one, so the walk stays inside [0, C).  Polls are not free (every one is a trip to
+// device-coherent memory), so only what is needed is requested: the neighbour's word first; a
+// tile's decay only once its word shows an aggregate, together with the word of the tile beyond.
+template <bool REV, int BN>
 struct ChainLook {
-  u64 w[W], d[W];
-  int j;  // neighbour the window starts at
+  u64 w;  // first look at the neighbour's word
+  int j;
 
-  __device__ __forceinline__ int clampj(int jj, int C) const { return REV ? min(jj, C - 1) : max(jj, 0); }
-
-  __device__ __forceinline__ void request(const u64* words, const u64* decw, int C) {
-#pragma unroll
-    for (int i = 0; i < W; ++i) {
-      const int jj = clampj(REV ? j + i : j - i, C);
-      w[i] = chain_peek(words + (int64_t)jj * BN);
-      d[i] = chain_peek(decw + jj);
-    }
-  }
-  __device__ __forceinline__ void begin(const u64* words, const u64* decw, int c, int C) {
+  __device__ __forceinline__ void begin(const u64* words, int c) {
     j = REV ? c + 1 : c - 1;
-    request(words, decw, C);
+    w = chain_peek(words + (int64_t)j * BN);
   }
   __device__ __forceinline__ float finish(const u64* words, const u64* decw, int C, const ChainCtl& ctl) {
     float carry = 0.f, scale = 1.f;
     for (;;) {
-#pragma unroll
-      for (int i = 0; i < W; ++i) {
-        const int jj = REV ? j + i : j - i;
-        if (REV ? jj >= C : jj < 0) return carry;
-        const u64 sw = chain_wait(words + (int64_t)jj * BN, w[i], ctl);
-        carry = fmaf(scale, chain_value(sw), carry);
-        if (chain_state(sw, ctl.epoch) == kStatePrefix) return carry;
-        scale *= chain_value(chain_wait(decw + jj, d[i], ctl));
-      }
-      j += REV ? W : -W;
-      request(words, decw, C);
+      const u64 sw = chain_wait(words + (int64_t)j * BN, w, ctl);
+      carry = fmaf(scale, chain_value(sw), carry);
+      if (chain_state(sw, ctl.epoch) == kStatePrefix) return carry;
+      const int jn = REV ? j + 1 : j - 1;
+      if (REV ? jn >= C : jn < 0) return carry;
+      const u64 d = chain_peek(decw + j);
+      w = chain_peek(words + (int64_t)jn * BN);
+      scale *= chain_value(chain_wait(decw + j, d, ctl));
+      j = jn;
     }
   }
 };

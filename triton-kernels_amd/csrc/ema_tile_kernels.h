@@ -78,12 +78,11 @@ namespace ema {
 constexpr bool kStreamFwdLoad = (EMA_STREAM_FLAGS & 1) != 0, kStreamFwdStore = (EMA_STREAM_FLAGS & 2) != 0,
                kStreamBwdLoad = (EMA_STREAM_FLAGS & 4) != 0, kStreamBwdStore = (EMA_STREAM_FLAGS & 8) != 0;
 
-// Predecessors whose words a look-back requests together (the forward runs at 64 registers).
-#ifndef EMA_FWD_LOOK_WINDOW
-#define EMA_FWD_LOOK_WINDOW 3
+// Development builds only (wrong results, to price the parts of the look-back): 1 no aggregate
+// publish and no polls, 4 nothing published at all.
+#ifndef EMA_EXP
+#define EMA_EXP 0
 #endif
-constexpr int kFwdLookWindow = EMA_FWD_LOOK_WINDOW, kBwdLookWindow = 4;
-
 template <typename T, int CPL, int RPL>
 struct TileCfg {
   static constexpr int NG = kTileRows / RPL;            // row groups = waves of the workgroup
@@ -334,28 +333,19 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
         dec *= dg[g];
       }
       float p_in;
-#ifdef EMA_EXP_NO_LOOK
-      if (false) {
-#else
-      if (t.c > 0) {
-#endif
+      if (t.c > 0 && EMA_EXP == 0) {
         if (k == 0) chain_publish(dws + t.c, ctl.epoch, kStateAggregate, dec);
         chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStateAggregate, loc);
-        ChainLook<false, BN, kFwdLookWindow> look;
+        ChainLook<false, BN> look;
         EMA_TSTAMP(4);
-        look.begin(words, dws, t.c, C);
-#ifdef EMA_TIMING
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        EMA_TSTAMP(5);
-        EMA_TSTAMP_VALUE(7, chain_state(look.w[0], ctl.epoch) * 10 + chain_state(look.w[1], ctl.epoch));
-#endif
+        look.begin(words, t.c);
         p_in = look.finish(words, dws, C, ctl);
         EMA_TSTAMP(6);
       } else {
-        p_in = (init && t.col0 + k < Tdim) ? init[(int64_t)t.n * Tdim + t.col0 + k] : 0.f;
+        p_in = (init && t.c == 0 && t.col0 + k < Tdim) ? init[(int64_t)t.n * Tdim + t.col0 + k] : 0.f;
       }
       const float p_out = fmaf(dec, p_in, loc);
-      chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStatePrefix, p_out);
+      if (EMA_EXP != 4) chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStatePrefix, p_out);
       sP[buf][k] = p_in;
       if (t.col0 + k < Tdim) {
         prev[(int64_t)t.chunk_id * Tdim + t.col0 + k] = p_in;
@@ -505,7 +495,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     u64* dws = decw + (int64_t)t.n * C;
     const bool last = t.c == C - 1;
     float loc = 0.f, dec = 1.f;
-    ChainLook<true, BN, kBwdLookWindow> look;
+    ChainLook<true, BN> look;
     if (threadIdx.x < BN) {
       const int k = threadIdx.x;
       float rg[NG], dg[NG];
@@ -520,10 +510,10 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
         loc = fmaf(dg[g], loc, rg[g]);
         dec *= dg[g];
       }
-      if (!last) {
+      if (!last && EMA_EXP == 0) {
         if (k == 0) chain_publish(dws + t.c, ctl.epoch, kStateAggregate, dec);
         chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStateAggregate, loc);
-        look.begin(words, dws, t.c, C);
+        look.begin(words, t.c);
       }
     } else if (kf < BN) {
       float sg[NG], dg[NG];
@@ -565,10 +555,10 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     if (threadIdx.x < BN) {
       const int k = threadIdx.x;
       float h_in;
-      if (!last) h_in = look.finish(words, dws, C, ctl);
-      else h_in = (dfinal && t.col0 + k < Tdim) ? dfinal[(int64_t)t.n * Tdim + t.col0 + k] : 0.f;
+      if (!last && EMA_EXP == 0) h_in = look.finish(words, dws, C, ctl);
+      else h_in = (dfinal && last && t.col0 + k < Tdim) ? dfinal[(int64_t)t.n * Tdim + t.col0 + k] : 0.f;
       const float h_out = fmaf(dec, h_in, loc);
-      chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStatePrefix, h_out);
+      if (EMA_EXP != 4) chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStatePrefix, h_out);
       if (dinit && t.c == 0 && t.col0 + k < Tdim) dinit[(int64_t)t.n * Tdim + t.col0 + k] = h_out;
       sH[buf][k] = h_in;
     }
