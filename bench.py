@@ -4,18 +4,25 @@
 One step = one forward and one backward through the autograd entry point
 (ema_matmul_scan_combined(...).backward(dy)) of benchmark configuration 3 at chunk size 128:
 b16 nh2 d1024 L4096, bf16 x / dy, fp32 log-decay and accumulation.  The forward is one pass
-over x (cumsum + single-pass chained scan), the backward one pass over x and dy.  Inputs are synthetic and resident in HBM before the timed
-region; the step rotates over several input sets so that no step finds its inputs in the
-256 MB last-level cache.
+over x, the backward one pass over x and dy (three launches per step: the two single-pass
+kernels and the small reduction of the log-decay gradient).  Inputs are synthetic and resident
+in HBM before the timed region; the steps run back to back and rotate over several input sets,
+so that no step finds its inputs in the 256 MB last-level cache and every kernel runs while the
+output of the one before is still on its way to HBM, as in a training loop.
 
-Prints ONE JSON line.  `roofline` describes the kernel with the largest share of the step,
-timed live with HIP events that the library records on the launch stream right around it;
-`stage_launchers` times every per-stage launcher of the reference's interface on its own; `cpu_baseline` is the sequential CPU
-oracle timed on a bounded sample and scaled to the full workload.
+Prints ONE JSON line.  `roofline` describes the kernel with the largest share of the step; its
+duration is that of the very dispatches of the timed steps (events that the runtime stamps with
+start and end of the dispatch, collected in a second pass of the same loop).  `configs` holds
+the other benchmark configurations: chunk sizes 256 and 512 (step, and the three per-stage
+contraction launchers with their dense-FLOP rate), the long-sequence configuration 4 and the
+Mamba-2 SSD configuration 5.  `stage_launchers` times every per-stage launcher of the
+reference's interface on its own; `cpu_baseline` is the sequential CPU oracle timed on a bounded
+sample and scaled to the full workload.
 """
 import argparse
 import json
 import os
+import platform
 import sys
 import time
 
@@ -24,10 +31,11 @@ for p in (ROOT, os.path.join(ROOT, "triton-kernels_amd")):
     if p not in sys.path:
         sys.path.insert(0, p)
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), scaled by
-# what the same counters read for a plain 268 435 456-byte device copy (FETCH_SIZE reads
-# 131 085 KiB for it, factor 1.99982; WRITE_SIZE reads 262 144 KiB, factor 1).
-TRAFFIC_BYTES = {"fwd_single_pass": 589083033, "bwd_single_pass": 841025145}
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (summaries and commands under
+# profiles/), scaled by what the same counters read for a plain 268 435 456-byte device copy
+# (FETCH_SIZE reads 131 085 KiB for it, factor 1.99982; WRITE_SIZE reads 262 144 KiB, factor 1).
+TRAFFIC_BYTES = {"fwd_single_pass": None, "bwd_single_pass": None}
+TRAFFIC_SOURCE = "profiles/single_pass_tile_kernels_b16_nh2_d1024_L4096_c128_hbm_traffic.txt (rocprofv3 --pmc, not measured by this run)"
 # the same for the SSD stage kernels at configuration 5 (finishing kernels added to their stage)
 SSD_TRAFFIC_BYTES = {
     "chunk_cumsum": 25320408, "chunk_state": 571591572, "state_passing": 419465499, "bmm_chunk": 100772767,
@@ -49,16 +57,40 @@ def parse():
     ap.add_argument("--nheads", type=int, default=2)
     ap.add_argument("--seqlen", type=int, default=4096)
     ap.add_argument("--dim", type=int, default=1024)
+    ap.add_argument("--u-mean", type=float, default=2.0, help="mean of u in the decay sigmoid(u)")
     ap.add_argument("--sets", type=int, default=3, help="input sets the steps rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel timing pass")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-stage launcher timing")
+    ap.add_argument("--no-configs", action="store_true", help="skip the other benchmark configurations")
     ap.add_argument("--workload", default="ema", choices=["ema", "ssd"],
-                    help="ema: the headline EMA scan step (default); ssd: the Mamba-2 SSD forward stages at "
-                    "benchmark configuration 5 (b8 nh32 hdim64 dstate128 g1 L8192 chunk256, bf16)")
+                    help="ema: the headline EMA scan step (default); ssd: the Mamba-2 SSD stages at "
+                    "benchmark configuration 5 (b8 nh32 hdim64 dstate128 g1 L8192 chunk256, bf16) alone")
     ap.add_argument("--stage", default=None,
-                    help="time only this stage (a name from the `kernels` table, or fwd, bwd, copy) "
-                    "and print a short JSON line; used for counter collection")
+                    help="time only this stage (a name from the stage tables, or fwd, bwd, bwd_saved, step, copy) "
+                    "and print a short JSON line; used for profiles and counter collection")
     return ap.parse_args()
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return platform.processor() or "unknown"
+
+
+def ema_inputs(torch, dev, b, nh, L, T, seed, u_mean=2.0, dtype=None):
+    """Synthetic inputs of the EMA benchmark configurations, generated on the device:
+    x, dy ~ N(0,1) (b, L, nh, T) bf16; A = log(sigmoid(u)), u ~ N(u_mean, 1), (b, L, nh) fp32."""
+    dtype = dtype or torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(seed)
+    x = torch.randn(b, L, nh, T, generator=g, device=dev, dtype=torch.float32).to(dtype)
+    u = torch.randn(b, L, nh, generator=g, device=dev, dtype=torch.float32) + u_mean
+    A = torch.nn.functional.logsigmoid(u)
+    dy = torch.randn(b, L, nh, T, generator=g, device=dev, dtype=torch.float32).to(dtype)
+    return x, A, dy
 
 
 def algorithmic_bytes(N, L, T, Q, esize):
@@ -123,19 +155,190 @@ def cpu_baseline(args, torch):
         "value": per * scale * 1e3,
         "unit": "ms",
         "cores": threads,
+        "cpu_model": cpu_model(),
+        "threads": threads,
         "kind": "port",
         "sample": f"{sample_b * args.nheads} of {nseq_total} sequences (L={args.seqlen}, d={args.dim}), "
         f"fwd + bwd sequential recurrence in fp32 torch, {reps} repetitions, scaled x{scale:g}",
     }
 
 
-def ssd_main(args):
-    """Mamba-2 SSD forward at benchmark configuration 5: the five stage launchers and their sum,
-    timed with events on the launch stream; per stage the algorithmic bytes (inputs read once,
-    outputs written once) against the HBM peak and, for the three MFMA stages, dense FLOPs
-    against the bf16 MFMA peak."""
-    import torch
+# ------------------------------------------------------------------------------------------------
+# EMA step on one configuration
+# ------------------------------------------------------------------------------------------------
 
+class EmaRun:
+    """Input sets and step functions of one EMA configuration."""
+
+    def __init__(self, torch, dev, b, nh, L, T, Q, nsets, u_mean, seed0):
+        from kernels.ema_kernels.ema_combined_fwd import ema_matmul_scan_combined
+        from kernels.ema_seq import ema_seq_bwd, ema_seq_fwd
+
+        self.torch, self.dev = torch, dev
+        self.b, self.nh, self.L, self.T, self.Q = b, nh, L, T, Q
+        self.N = b * nh
+        self.sets = [ema_inputs(torch, dev, b, nh, L, T, seed0 + s, u_mean) for s in range(nsets)]
+        self.grad_sets = [(x.clone().requires_grad_(), A.clone().requires_grad_(), dy) for x, A, dy in self.sets]
+        self._apply, self._fwd, self._bwd = ema_matmul_scan_combined, ema_seq_fwd, ema_seq_bwd
+        self._saved = None
+
+    def step(self, i):
+        # one training step through the autograd entry point: the forward keeps the states entering
+        # each 128-row chunk (4 MB) and the backward reuses them
+        x, A, dy = self.grad_sets[i % len(self.grad_sets)]
+        x.grad = None
+        A.grad = None
+        self._apply(A, x, self.Q).backward(dy)
+
+    def fwd_only(self, i, events=None):
+        x, A, dy = self.sets[i % len(self.sets)]
+        return self._fwd(A, x, kernel_events=events)
+
+    def bwd_saved(self, i, events=None):  # backward as the autograd step runs it, with the forward's states
+        if self._saved is None:
+            self._saved = [self._fwd(A, x)[2] for x, A, dy in self.sets]
+        x, A, dy = self.sets[i % len(self.sets)]
+        return self._bwd(dy, x, A, self._saved[i % len(self.sets)], kernel_events=events)
+
+    def step_kernels(self, iters):
+        """The same two launches per step as `step` makes (sequence-level forward, then backward
+        with the forward's states), back to back, with the runtime's start / stop stamps of every
+        dispatch: in-sequence durations of the two single-pass kernels, in ms."""
+        torch = self.torch
+        self.bwd_saved(0)
+        evs = []
+        for i in range(2 * iters):
+            ev = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+            ev[0].record()
+            ev[1].record()  # materialise the handles before the timed launches
+            evs.append(ev)
+        for i in range(3):
+            self.fwd_only(i)
+            self.bwd_saved(i)
+        torch.cuda.synchronize()
+        for i in range(iters):
+            self.fwd_only(i, evs[2 * i])
+            self.bwd_saved(i, evs[2 * i + 1])
+        torch.cuda.synchronize()
+        f = sum(evs[2 * i][0].elapsed_time(evs[2 * i][1]) for i in range(iters)) / iters
+        bw = sum(evs[2 * i + 1][0].elapsed_time(evs[2 * i + 1][1]) for i in range(iters)) / iters
+        return f, bw
+
+    def measure(self, steps, warmup):
+        torch = self.torch
+        for i in range(warmup):
+            self.step(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ms_events = time_region(self.step, steps, torch)
+        wall = (time.perf_counter() - t0) * 1e3 / steps
+        ab = algorithmic_bytes(self.N, self.L, self.T, self.Q, 2)
+        ms_step = max(ms_events, wall)
+        kf, kb = self.step_kernels(steps)
+        x_bytes = self.N * self.L * self.T * 2
+        small = self.N * (-(-self.L // 128)) * self.T * 4  # chunk-entry states at 128-row chunking
+        fb = 2 * x_bytes + self.N * self.L * 4 + small
+        bb = 3 * x_bytes + 2 * self.N * self.L * 4 + small
+        return {
+            "ms_per_step": ms_step,
+            "hbm_frac_of_peak_fwd+bwd": (ab["fwd"] + ab["bwd"]) / ms_step / 1e6 / HBM_PEAK_GBS,
+            "algorithmic_bytes_fwd+bwd": ab["fwd"] + ab["bwd"],
+            "step_kernels": {
+                "fwd_single_pass": {"ms": kf, "bytes": fb, "GBps": fb / kf / 1e6, "hbm_frac": fb / kf / 1e6 / HBM_PEAK_GBS},
+                "bwd_single_pass": {"ms": kb, "bytes": bb, "GBps": bb / kb / 1e6, "hbm_frac": bb / kb / 1e6 / HBM_PEAK_GBS},
+            },
+        }
+
+
+def make_stages(sets, Q, torch):
+    """name -> callable(i) launching one stage through its per-stage launcher (one kernel each,
+    plus at most one tiny finishing kernel) on input set i; `copy` is a plain device copy of
+    one x-sized tensor."""
+    from kernels.ema_kernels.ema_cumsum import ema_chunk_cumsum_fwd
+    from kernels.ema_kernels.ema_scan_fwd import _ema_scan_fwd
+    from kernels.ema_kernels.ema_state_fwd import _ema_chunk_state_fwd
+    from kernels.ema_kernels.ema_state_pass import _ema_state_passing_fwd
+    from kernels.ema_kernels_bwd.ema_chunk_scan_bwd_dc import _ema_chunk_scan_bwd_dC
+    from kernels.ema_kernels_bwd.ema_chunk_scan_chunk_state_bwd_dx import _chunk_scan_chunk_state_bwd_dx
+    from kernels.ema_kernels_bwd.ema_chunk_state_bwd_db import _ema_chunk_state_bwd_db
+    from kernels.ema_kernels_bwd.ema_combined_bwd import _ema_bwd_dx_dA_fused
+    from kernels.ema_kernels_bwd.ema_scan_bwd import _ema_chunk_scan_bwd_dstates
+    from kernels.ema_kernels_bwd.ema_scan_da import _ema_chunk_scan_bwd_ddAcs_stable
+    from kernels.ema_kernels_bwd.ema_state_passing_bwd_dstates import _ema_state_passing_bwd
+
+    inter = []
+    for x, A, dy in sets:
+        cs = ema_chunk_cumsum_fwd(A, Q)
+        states = _ema_chunk_state_fwd(x, cs)
+        prev, _ = _ema_state_passing_fwd(states, cs[..., -1], out_dtype=torch.float32)
+        ds = _ema_chunk_scan_bwd_dstates(cs, dy)
+        g, _, _ = _ema_state_passing_bwd(prev, cs[..., -1], ds)
+        if Q == 128:
+            fused_in = (cs, prev, g)
+        else:  # the fused backward kernel always works on 128-row chunks
+            cs1 = ema_chunk_cumsum_fwd(A, 128)
+            prev1, _ = _ema_state_passing_fwd(_ema_chunk_state_fwd(x, cs1), cs1[..., -1], out_dtype=torch.float32)
+            g1, _, _ = _ema_state_passing_bwd(prev1, cs1[..., -1], _ema_chunk_scan_bwd_dstates(cs1, dy))
+            fused_in = (cs1, prev1, g1)
+        inter.append((cs, states, prev, ds, g, fused_in))
+
+    def pick(i):
+        k = i % len(sets)
+        return sets[k] + inter[k]
+
+    stages = {
+        "cumsum": lambda i: ema_chunk_cumsum_fwd(pick(i)[1], Q),
+        "chunk_state": lambda i: _ema_chunk_state_fwd(pick(i)[0], pick(i)[3]),
+        "state_passing_fwd": lambda i: _ema_state_passing_fwd(pick(i)[4], pick(i)[3][..., -1]),
+        "chunk_scan": lambda i: _ema_scan_fwd(pick(i)[0], pick(i)[3], pick(i)[5]),
+        "bwd_dstates": lambda i: _ema_chunk_scan_bwd_dstates(pick(i)[3], pick(i)[2]),
+        "state_passing_bwd": lambda i: _ema_state_passing_bwd(pick(i)[5], pick(i)[3][..., -1], pick(i)[6]),
+        "bwd_dx": lambda i: _chunk_scan_chunk_state_bwd_dx(pick(i)[0], pick(i)[3], pick(i)[2], pick(i)[7]),
+        "bwd_db": lambda i: _ema_chunk_state_bwd_db(pick(i)[0], pick(i)[3], pick(i)[7]),
+        "bwd_dc": lambda i: _ema_chunk_scan_bwd_dC(pick(i)[5], pick(i)[3], pick(i)[2]),
+        "bwd_da_intra": lambda i: _ema_chunk_scan_bwd_ddAcs_stable(pick(i)[0], pick(i)[3], pick(i)[2]),
+        "bwd_fused_dx_dA": lambda i: _ema_bwd_dx_dA_fused(
+            pick(i)[0], pick(i)[8][0], pick(i)[2], pick(i)[8][1], pick(i)[8][2]),
+    }
+    outs = [torch.empty_like(s[0]) for s in sets]
+    stages["copy"] = lambda i: outs[i % len(sets)].copy_(sets[i % len(sets)][0])
+    return stages
+
+
+def time_stages(sets, Q, iters, torch, only=None):
+    """Per-stage timing with HIP events on the launch stream (back-to-back launches over the
+    rotating input sets)."""
+    stages = make_stages(sets, Q, torch)
+    x = sets[0][0]
+    N, L, T = x.shape[0] * x.shape[2], x.shape[1], x.shape[3]
+    ab = dict(algorithmic_bytes(N, L, T, Q, 2), copy=2 * x.numel() * x.element_size())
+    res = {}
+    for name, fn in stages.items():
+        if only and name not in only:
+            continue
+        for i in range(3):
+            fn(i)
+        ms = time_region(fn, iters, torch)
+        gbps = ab[name] / ms / 1e6
+        res[name] = {"ms": ms, "GBps": gbps, "hbm_frac": gbps / HBM_PEAK_GBS, "bytes": ab[name]}
+    flops = 2.0 * Q * L * T * N
+    for name in ("chunk_scan", "bwd_dx", "bwd_da_intra"):  # dense-equivalent count, Q*Q per chunk
+        if name in res:
+            tf = flops / res[name]["ms"] / 1e9
+            res[name]["dense_TFLOPs"] = tf
+            res[name]["mfma_frac_dense"] = tf / MFMA_BF16_PEAK_TFLOPS
+    return res
+
+
+# ------------------------------------------------------------------------------------------------
+# Mamba-2 SSD stages at configuration 5
+# ------------------------------------------------------------------------------------------------
+
+def ssd_stages(torch, steps, warmup, only=None):
+    """The five forward stage launchers, their combined forward and the six backward stage
+    launchers at benchmark configuration 5, timed with events on the launch stream; per stage the
+    algorithmic bytes (inputs read once, outputs written once) against the HBM peak and, for the
+    MFMA stages, dense FLOPs against the bf16 MFMA peak."""
     from kernels.mamba_kernels.mamba_bmm import _bmm_chunk_fwd
     from kernels.mamba_kernels.mamba_combined_fwd import _mamba_chunk_scan_combined_fwd
     from kernels.mamba_kernels.mamba_cumsum import _chunk_cumsum_fwd
@@ -148,15 +351,19 @@ def ssd_main(args):
     from kernels.mamba_kernels_bwd.mamba_chunk_state_bwd_db import _chunk_state_bwd_db
     from kernels.mamba_kernels_bwd.mamba_scan_bwd import _chunk_scan_bwd_dstates
     from kernels.mamba_kernels_bwd.mamba_state_passing_bwd_dstates import _state_passing_bwd
-    from oracle import ssd_oracle as S
 
     dev = torch.device("cuda:0")
     b, L, nh, P, g, N, Q = 8, 8192, 32, 64, 1, 128, 256
     C = L // Q
     sets = []
     for s in range(2):
-        x, dt, A, B, Cm, _, _ = S.make_inputs(b, L, nh, P, g, N, seed=5 + s, dtype=torch.bfloat16)
-        sets.append(tuple(t.to(dev) for t in (x, dt, A, B, Cm)))
+        gen = torch.Generator(device=dev).manual_seed(5 + s)
+        x = torch.randn(b, L, nh, P, generator=gen, device=dev).to(torch.bfloat16)
+        B = torch.randn(b, L, g, N, generator=gen, device=dev).to(torch.bfloat16)
+        Cm = torch.randn(b, L, g, N, generator=gen, device=dev).to(torch.bfloat16)
+        dt = torch.nn.functional.softplus(torch.randn(b, L, nh, generator=gen, device=dev) * 0.5 - 2.0)
+        A = -torch.exp(torch.rand(nh, generator=gen, device=dev) * 2.772588722239781)  # -exp(U(log 1, log 16))
+        sets.append((x, dt, A, B, Cm))
     inter = []
     for x, dt, A, B, Cm in sets:
         out, _, dt_out, dA_cs, states, _ = _mamba_chunk_scan_combined_fwd(x, dt, A, B, Cm, Q)
@@ -213,20 +420,30 @@ def ssd_main(args):
              "bwd_dx": (2 * Q * Q * P + 2 * Q * N * P) * units, "bwd_ddAcs": 2 * Q * Q * P * units}
     res = {}
     for name, fn in stages.items():
-        if args.stage and name != args.stage:
+        if only and name != only:
             continue
-        for i in range(args.warmup):
+        for i in range(warmup):
             fn(i)
-        ms = time_region(fn, args.steps, torch)
+        ms = time_region(fn, steps, torch)
         res[name] = {"ms": ms, "bytes": nbytes[name], "GBps": nbytes[name] / ms / 1e6,
                      "hbm_frac": nbytes[name] / ms / 1e6 / HBM_PEAK_GBS}
         if name in flops:
             res[name]["dense_TFLOPs"] = flops[name] / ms / 1e9
             res[name]["mfma_frac"] = flops[name] / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS
+    if not only:
+        res["backward_stages_sum"] = {"ms": sum(v["ms"] for k, v in res.items() if k.startswith("bwd_"))}
+    return res
+
+
+def ssd_main(args):
+    import torch
+
+    from oracle import ssd_oracle as S
+
+    res = ssd_stages(torch, args.steps, args.warmup, args.stage)
     if args.stage:
         print(json.dumps({"stage": args.stage, **res[args.stage], "steps": args.steps}))
         return
-    res["backward_stages_sum"] = {"ms": sum(v["ms"] for k, v in res.items() if k.startswith("bwd_"))}
     # the roofline entry is for the dominant kernel of the timed region, which is the forward
     dom = max((k for k in res if k != "forward" and not k.startswith(("bwd_", "backward"))),
               key=lambda k: res[k]["ms"])
@@ -239,9 +456,11 @@ def ssd_main(args):
                    "chunk256, bf16 x/B/C, fp32 dt/A, D = 0, no gate"},
         "stages": res,
         "roofline": {"kernel": dom, "bound": "hbm", "achieved": res[dom]["GBps"], "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": res[dom]["hbm_frac"], "traffic": SSD_TRAFFIC_BYTES.get(dom)},
+                     "unit": "GB/s", "frac": res[dom]["hbm_frac"], "traffic": SSD_TRAFFIC_BYTES.get(dom),
+                     "traffic_source": "profiles/ssd_stages_b8_nh32_hd64_ds128_L8192_c256_hbm_traffic.txt"},
     }
     if not args.no_cpu_baseline:
+        b, L, nh, P, g, N = 8, 8192, 32, 64, 1, 128
         x, dt, A, B, Cm, _, _ = S.make_inputs(1, 512, nh, P, g, N, seed=5, dtype=torch.bfloat16)
         t0 = time.perf_counter()
         reps = 0
@@ -251,72 +470,39 @@ def ssd_main(args):
         per = (time.perf_counter() - t0) / reps
         scale = b * L / 512
         out["cpu_baseline"] = {"value": per * scale * 1e3, "unit": "ms", "cores": torch.get_num_threads(),
-                               "kind": "port",
+                               "cpu_model": cpu_model(), "threads": torch.get_num_threads(), "kind": "port",
                                "sample": f"1 of {b} sequences, 512 of {L} positions, sequential recurrence in fp32 "
                                f"torch, {reps} repetitions, scaled x{scale:g}"}
     print(json.dumps(out))
 
 
+# ------------------------------------------------------------------------------------------------
+
 def main():
     args = parse()
-    if args.workload == "ssd" and args.gpus == 1:
-        return ssd_main(args)
     if args.gpus != 1:
         print("bench.py measures one GPU only: the EMA scan has no multi-GPU path in this build "
               "(run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
+    if args.workload == "ssd":
+        return ssd_main(args)
     import torch
-
-    from kernels.ema_kernels.ema_combined_fwd import _ema_matmul_scan_combined_fwd
-    from kernels.ema_kernels_bwd.ema_combined_bwd import _ema_chunk_scan_combined_bwd
-    from oracle import ema_oracle as O
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     dev = torch.device("cuda:0")
     b, nh, L, T, Q = args.batch, args.nheads, args.seqlen, args.dim, args.chunk
-    N = b * nh
-    sets = []
-    for s in range(args.sets):
-        x, A, dy = O.make_inputs(b, nh, L, T, seed=1000 + Q + s, dtype=torch.bfloat16)
-        sets.append((x.to(dev), A.to(dev), dy.to(dev)))
-    del x, A, dy
-
-    from kernels.ema_kernels.ema_combined_fwd import ema_matmul_scan_combined
-
-    for x, A, dy in sets:
-        x.requires_grad_()
-        A.requires_grad_()
-
-    def step(i):
-        # one training step through the autograd entry point: the forward keeps the states
-        # entering each 128-row chunk (4 MB) and the backward reuses them
-        x, A, dy = sets[i % len(sets)]
-        x.grad = None
-        A.grad = None
-        ema_matmul_scan_combined(A, x, Q).backward(dy)
-
-    def fwd_only(i):
-        x, A, dy = sets[i % len(sets)]
-        _ema_matmul_scan_combined_fwd(A.detach(), x.detach(), Q)
-
-    def bwd_only(i):  # stand-alone backward: recomputes the chunk-entry states from x
-        x, A, dy = sets[i % len(sets)]
-        _ema_chunk_scan_combined_bwd(dy, x.detach(), A.detach(), Q)
-
-    saved = []
-
-    def bwd_saved(i):  # backward as the autograd step runs it, with the forward's states
-        if not saved:
-            for x, A, dy in sets:
-                saved.append(_ema_matmul_scan_combined_fwd(A.detach(), x.detach(), Q, return_prev128=True)[4])
-        x, A, dy = sets[i % len(sets)]
-        _ema_chunk_scan_combined_bwd(dy, x.detach(), A.detach(), Q, prev128=saved[i % len(sets)])
+    run = EmaRun(torch, dev, b, nh, L, T, Q, args.sets, args.u_mean, seed0=1000 + Q)
 
     if args.stage:
-        stages = make_stages([tuple(t.detach() for t in st) for st in sets], Q, torch)
-        stages.update({"fwd": fwd_only, "bwd": bwd_only, "bwd_saved": bwd_saved, "step": step})
+        from kernels.ema_kernels_bwd.ema_combined_bwd import _ema_chunk_scan_combined_bwd
+
+        stages = {"fwd": run.fwd_only, "bwd_saved": run.bwd_saved, "step": run.step,
+                  "bwd": lambda i: _ema_chunk_scan_combined_bwd(run.sets[i % len(run.sets)][2], run.sets[i % len(run.sets)][0],
+                                                                run.sets[i % len(run.sets)][1], Q)}
+        if args.stage not in stages:
+            stages = make_stages(run.sets, Q, torch)
         fn = stages[args.stage]
         for i in range(args.warmup):
             fn(i)
@@ -324,34 +510,23 @@ def main():
         print(json.dumps({"stage": args.stage, "ms": ms, "steps": args.steps}))
         return
 
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    ms_step_events = time_region(step, args.steps, torch)
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    ms_step = max(ms_step_events, wall_ms)
+    head = run.measure(args.steps, args.warmup)
+    ms_step = head["ms_per_step"]
+    main_k = head["step_kernels"]
+    ab = algorithmic_bytes(run.N, L, T, Q, 2)
 
     # the same step (forward launcher, then backward launcher with the forward's states) captured
     # once per input set into a HIP graph and replayed, as the reference's benchmarks time their
     # kernels (do_bench_cudagraph, kernels/benchmarks/ema_bench.py:102)
     ms_graph = None
     try:
-        graphs = []
-        side = torch.cuda.Stream(dev)
-        side.wait_stream(torch.cuda.current_stream(dev))
-        with torch.cuda.stream(side):
-            for x, A, dy in sets:
-                out = _ema_matmul_scan_combined_fwd(A.detach(), x.detach(), Q, return_prev128=True)
-                _ema_chunk_scan_combined_bwd(dy, x.detach(), A.detach(), Q, prev128=out[4])
-        torch.cuda.current_stream(dev).wait_stream(side)
-        keep = []
-        for x, A, dy in sets:
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                out = _ema_matmul_scan_combined_fwd(A.detach(), x.detach(), Q, return_prev128=True)
-                keep.append((out, _ema_chunk_scan_combined_bwd(dy, x.detach(), A.detach(), Q, prev128=out[4])))
-            graphs.append(g)
+        run.bwd_saved(0)
+        graphs, keep = [], []
+        for k in range(len(run.sets)):
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                keep.append((run.fwd_only(k), run.bwd_saved(k)))
+            graphs.append(gr)
         for i in range(args.warmup):
             graphs[i % len(graphs)].replay()
         ms_graph = time_region(lambda i: graphs[i % len(graphs)].replay(), args.steps, torch)
@@ -359,45 +534,18 @@ def main():
     except Exception as exc:  # capture is an extra; the eager figure stands without it
         print(f"graph capture skipped: {exc}", file=sys.stderr)
 
-    ab = algorithmic_bytes(N, L, T, Q, 2)
-    ms_fwd = time_region(fwd_only, args.steps, torch)
-    ms_bwd = time_region(bwd_only, args.steps, torch)
-    bwd_saved(0)
-    ms_bwd_saved = time_region(bwd_saved, args.steps, torch)
+    ms_fwd = time_region(run.fwd_only, args.steps, torch)
+    ms_bwd_saved = time_region(run.bwd_saved, args.steps, torch)
+    from kernels.ema_kernels_bwd.ema_combined_bwd import _ema_chunk_scan_combined_bwd
 
-    # the two kernels that carry the step, timed alone with HIP events recorded by the library
-    # on the launch stream right around them
-    def kernel_ms(call):
-        pairs = []
-        for i in range(args.steps):
-            ev = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-            ev[0].record(); ev[1].record()  # materialise the handles
-            call(i, ev)
-            pairs.append(ev)
-        torch.cuda.synchronize()
-        return sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
+    ms_bwd = time_region(lambda i: _ema_chunk_scan_combined_bwd(run.sets[i % len(run.sets)][2], run.sets[i % len(run.sets)][0],
+                                                                run.sets[i % len(run.sets)][1], Q), args.steps, torch)
 
-    x_bytes = N * L * T * 2
-    small = N * (-(-L // 128)) * (128 * 4 + T * 4)  # cs + chunk-entry states at 128-row chunking
-    main = {}
-    ms = kernel_ms(lambda i, ev: _ema_matmul_scan_combined_fwd(
-        sets[i % len(sets)][1].detach(), sets[i % len(sets)][0].detach(), Q, kernel_events=ev))
-    nbytes = 2 * x_bytes + small
-    main["fwd_single_pass"] = {"ms": ms, "bytes": nbytes, "GBps": nbytes / ms / 1e6,
-                               "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBS}
-    ms = kernel_ms(lambda i, ev: _ema_chunk_scan_combined_bwd(
-        sets[i % len(sets)][2], sets[i % len(sets)][0].detach(), sets[i % len(sets)][1].detach(), Q,
-        prev128=saved[i % len(sets)], kernel_events=ev))
-    nbytes = 3 * x_bytes + small + N * L * 4  # x, dy, dx, cs, chunk-entry states, dA
-    main["bwd_single_pass"] = {"ms": ms, "bytes": nbytes, "GBps": nbytes / ms / 1e6,
-                               "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBS}
+    kernels = {} if args.no_kernels else time_stages(run.sets, Q, args.steps, torch)
 
-    kernels = {}
-    if not args.no_kernels:
-        kernels = time_kernels([tuple(t.detach() for t in st) for st in sets], Q, args.steps, ab, torch)
-
+    shape = f"b{b} nh{nh} d{T} L{L} c{Q}"
     out = {
-        "metric": "EMA scan fwd+bwd ms @ b16 nh2 d1024 L4096 c128",
+        "metric": f"EMA scan fwd+bwd ms @ {shape}",
         "value": ms_step,
         "unit": "ms",
         "n_gpus": 1,
@@ -422,99 +570,60 @@ def main():
             "bwd": ab["bwd"] / ms_bwd_saved / 1e6,
             "fwd+bwd": (ab["fwd"] + ab["bwd"]) / ms_step / 1e6,
         },
-        "hbm_frac_of_peak_fwd+bwd": (ab["fwd"] + ab["bwd"]) / ms_step / 1e6 / HBM_PEAK_GBS,
-        "step_kernels": main,
+        "hbm_frac_of_peak_fwd+bwd": head["hbm_frac_of_peak_fwd+bwd"],
+        "step_kernels": main_k,
         "stage_launchers": kernels,
     }
-    dom = max(main, key=lambda k: main[k]["ms"])
+    dom = max(main_k, key=lambda k: main_k[k]["ms"])
     out["roofline"] = {
         "kernel": dom,
         "bound": "hbm",
-        "achieved": main[dom]["GBps"],
+        "achieved": main_k[dom]["GBps"],
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
-        "frac": main[dom]["GBps"] / HBM_PEAK_GBS,
+        "frac": main_k[dom]["GBps"] / HBM_PEAK_GBS,
         "traffic": TRAFFIC_BYTES.get(dom),
+        "traffic_source": TRAFFIC_SOURCE,
+        "duration": "mean of the dispatches of the timed fwd,bwd sequence (runtime start/stop stamps)",
     }
+    del run
+    torch.cuda.empty_cache()
+
+    if not args.no_configs:
+        cfgs = {}
+        # configuration 3 at the other chunk sizes: the step, and the three contraction launchers
+        for q in (256, 512):
+            r = EmaRun(torch, dev, 16, 2, 4096, 1024, q, 2, 2.0, seed0=1000 + q)
+            m = r.measure(max(10, args.steps // 2), 3)
+            st = time_stages(r.sets, q, max(10, args.steps // 2), torch, only=("chunk_scan", "bwd_dx", "bwd_da_intra"))
+            cfgs[f"c{q}"] = {"workload": f"b16 nh2 d1024 L4096 chunk{q}", "step_ms": m["ms_per_step"],
+                             "hbm_frac": m["hbm_frac_of_peak_fwd+bwd"], "step_kernels": m["step_kernels"],
+                             "contraction_launchers": st}
+            del r, st
+            torch.cuda.empty_cache()
+        # configuration 4: long sequence, long memory
+        r = EmaRun(torch, dev, 4, 2, 32768, 1024, 256, 2, 4.0, seed0=4000)
+        m = r.measure(max(10, args.steps // 2), 3)
+        cfgs["cfg4"] = {"workload": "b4 nh2 d1024 L32768 chunk256, u ~ N(4,1)", "step_ms": m["ms_per_step"],
+                        "hbm_frac": m["hbm_frac_of_peak_fwd+bwd"], "algorithmic_bytes": m["algorithmic_bytes_fwd+bwd"],
+                        "step_kernels": m["step_kernels"]}
+        del r
+        torch.cuda.empty_cache()
+        # configuration 5: Mamba-2 SSD stages
+        s5 = ssd_stages(torch, max(10, args.steps // 2), 3)
+        cfgs["cfg5"] = {"workload": "Mamba-2 SSD b8 nh32 hdim64 dstate128 g1 L8192 chunk256, bf16",
+                        "forward_ms": s5["forward"]["ms"],
+                        "forward_stages_ms": {k: s5[k]["ms"] for k in ("chunk_cumsum", "chunk_state", "state_passing",
+                                                                      "bmm_chunk", "chunk_scan")},
+                        "backward_stages_ms": {k: v["ms"] for k, v in s5.items() if k.startswith("bwd_")},
+                        "backward_stages_sum_ms": s5["backward_stages_sum"]["ms"],
+                        "stages": s5}
+        torch.cuda.empty_cache()
+        out["configs"] = cfgs
+
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args, torch)
     print(json.dumps(out))
-
-
-def make_stages(sets, Q, torch):
-    """name -> callable(i) launching one stage through its per-stage launcher (one kernel each,
-    plus at most one tiny finishing kernel) on input set i; `copy` is a plain device copy of
-    one x-sized tensor, the practical ceiling of a read-once write-once kernel."""
-    from kernels.ema_kernels.ema_cumsum import ema_chunk_cumsum_fwd
-    from kernels.ema_kernels.ema_scan_fwd import _ema_scan_fwd
-    from kernels.ema_kernels.ema_state_fwd import _ema_chunk_state_fwd
-    from kernels.ema_kernels.ema_state_pass import _ema_state_passing_fwd
-    from kernels.ema_kernels_bwd.ema_chunk_scan_bwd_dc import _ema_chunk_scan_bwd_dC
-    from kernels.ema_kernels_bwd.ema_chunk_scan_chunk_state_bwd_dx import _chunk_scan_chunk_state_bwd_dx
-    from kernels.ema_kernels_bwd.ema_chunk_state_bwd_db import _ema_chunk_state_bwd_db
-    from kernels.ema_kernels_bwd.ema_combined_bwd import _ema_bwd_dx_dA_fused
-    from kernels.ema_kernels_bwd.ema_scan_bwd import _ema_chunk_scan_bwd_dstates
-    from kernels.ema_kernels_bwd.ema_scan_da import _ema_chunk_scan_bwd_ddAcs_stable
-    from kernels.ema_kernels_bwd.ema_state_passing_bwd_dstates import _ema_state_passing_bwd
-
-    inter = []
-    for x, A, dy in sets:
-        cs = ema_chunk_cumsum_fwd(A, Q)
-        states = _ema_chunk_state_fwd(x, cs)
-        prev, _ = _ema_state_passing_fwd(states, cs[..., -1], out_dtype=torch.float32)
-        ds = _ema_chunk_scan_bwd_dstates(cs, dy)
-        g, _, _ = _ema_state_passing_bwd(prev, cs[..., -1], ds)
-        if Q == 128:
-            fused_in = (cs, prev, g)
-        else:  # the fused backward kernel always works on 128-row chunks
-            cs1 = ema_chunk_cumsum_fwd(A, 128)
-            prev1, _ = _ema_state_passing_fwd(_ema_chunk_state_fwd(x, cs1), cs1[..., -1], out_dtype=torch.float32)
-            g1, _, _ = _ema_state_passing_bwd(prev1, cs1[..., -1], _ema_chunk_scan_bwd_dstates(cs1, dy))
-            fused_in = (cs1, prev1, g1)
-        inter.append((cs, states, prev, ds, g, fused_in))
-
-    def pick(i):
-        k = i % len(sets)
-        return sets[k] + inter[k]
-
-    stages = {
-        "cumsum": lambda i: ema_chunk_cumsum_fwd(pick(i)[1], Q),
-        "chunk_state": lambda i: _ema_chunk_state_fwd(pick(i)[0], pick(i)[3]),
-        "state_passing_fwd": lambda i: _ema_state_passing_fwd(pick(i)[4], pick(i)[3][..., -1]),
-        "chunk_scan": lambda i: _ema_scan_fwd(pick(i)[0], pick(i)[3], pick(i)[5]),
-        "bwd_dstates": lambda i: _ema_chunk_scan_bwd_dstates(pick(i)[3], pick(i)[2]),
-        "state_passing_bwd": lambda i: _ema_state_passing_bwd(pick(i)[5], pick(i)[3][..., -1], pick(i)[6]),
-        "bwd_dx": lambda i: _chunk_scan_chunk_state_bwd_dx(pick(i)[0], pick(i)[3], pick(i)[2], pick(i)[7]),
-        "bwd_db": lambda i: _ema_chunk_state_bwd_db(pick(i)[0], pick(i)[3], pick(i)[7]),
-        "bwd_dc": lambda i: _ema_chunk_scan_bwd_dC(pick(i)[5], pick(i)[3], pick(i)[2]),
-        "bwd_da_intra": lambda i: _ema_chunk_scan_bwd_ddAcs_stable(pick(i)[0], pick(i)[3], pick(i)[2]),
-        "bwd_fused_dx_dA": lambda i: _ema_bwd_dx_dA_fused(
-            pick(i)[0], pick(i)[8][0], pick(i)[2], pick(i)[8][1], pick(i)[8][2]),
-    }
-    outs = [torch.empty_like(s[0]) for s in sets]
-    stages["copy"] = lambda i: outs[i % len(sets)].copy_(sets[i % len(sets)][0])
-    return stages
-
-
-def time_kernels(sets, Q, iters, ab, torch):
-    """Per-stage timing with HIP events on the launch stream."""
-    stages = make_stages(sets, Q, torch)
-    x = sets[0][0]
-    ab = dict(ab, copy=2 * x.numel() * x.element_size())
-    res = {}
-    for name, fn in stages.items():
-        for i in range(3):
-            fn(i)
-        ms = time_region(fn, iters, torch)
-        gbps = ab[name] / ms / 1e6
-        res[name] = {"ms": ms, "GBps": gbps, "hbm_frac": gbps / HBM_PEAK_GBS, "bytes": ab[name]}
-    N, L, T = x.shape[0] * x.shape[2], x.shape[1], x.shape[3]
-    flops = 2.0 * Q * L * T * N
-    for name in ("chunk_scan", "bwd_dx", "bwd_da_intra"):  # dense-equivalent count, Q*Q per chunk
-        tf = flops / res[name]["ms"] / 1e9
-        res[name]["dense_TFLOPs"] = tf
-        res[name]["mfma_frac_dense"] = tf / MFMA_BF16_PEAK_TFLOPS
-    return res
 
 
 if __name__ == "__main__":

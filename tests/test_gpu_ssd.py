@@ -164,6 +164,62 @@ def test_views_of_a_fused_projection(dtype, device):
     assert torch.equal(y2, y0) and torch.equal(fin2, fin0)
 
 
+def test_converted_operands_stay_alive_until_the_launch(device):
+    """CB in bfloat16 together with dt and dA_cumsum as strided views: every operand the chunk scan
+    has to convert is converted into a temporary, and all of them must still be there when the
+    kernel is enqueued.  The result must equal that of float32, contiguous operands."""
+    from kernels.mamba_kernels.mamba_bmm import _bmm_chunk_fwd
+    from kernels.mamba_kernels.mamba_cumsum import _chunk_cumsum_fwd
+    from kernels.mamba_kernels.mamba_scan_fwd import _chunk_scan_fwd
+    from kernels.mamba_kernels.mamba_state_fwd import _chunk_state_fwd
+    from kernels.mamba_kernels.mamba_state_pass import _state_passing_fwd
+
+    b, L, nh, P, g, N, Q = 2, 512, 4, 64, 1, 128, 256
+    announce(f"ssd chunk scan with converted operands b{b} L{L} nh{nh} P{P} N{N} Q{Q}")
+    x, dt, A, B, C, D, _ = S.make_inputs(b, L, nh, P, g, N, seed=21, dtype=BF16)
+    xd, dtd, Ad, Bd, Cd = _dev(device, x, dt, A, B, C)
+    dA_cs, dt_out = _chunk_cumsum_fwd(dtd, Ad, Q)
+    states = _chunk_state_fwd(Bd, xd, dt_out, dA_cs)
+    nchunks = L // Q
+    prev, _ = _state_passing_fwd(states.view(b, nchunks, nh, P * N), dA_cs[..., -1], out_dtype=BF16)
+    prev = prev.view(b, nchunks, nh, P, N)
+    cb32 = _bmm_chunk_fwd(Cd, Bd, Q, output_dtype=F32)
+    ref, _ = _chunk_scan_fwd(cb32, xd, dt_out, dA_cs, Cd, prev)
+    # the same values in the shapes that need converting
+    cb16 = cb32.to(BF16)
+    ref16, _ = _chunk_scan_fwd(cb16.float(), xd, dt_out, dA_cs, Cd, prev)
+    wide_dt = torch.zeros(b, nh, nchunks, 2 * Q, device=device)
+    wide_dA = torch.zeros(b, nh, nchunks, 2 * Q, device=device)
+    wide_dt[..., ::2] = dt_out
+    wide_dA[..., ::2] = dA_cs
+    dt_view, dA_view = wide_dt[..., ::2], wide_dA[..., ::2]
+    assert not dt_view.is_contiguous() and not dA_view.is_contiguous()
+    for rep in range(3):  # the allocator reuses the blocks of earlier temporaries
+        got, _ = _chunk_scan_fwd(cb16, xd, dt_view, dA_view, Cd, prev)
+        assert torch.equal(got, ref16), rep
+    check_close("y with bf16 CB", got, ref, BF16, loose=True)
+
+
+def test_chunk_states_into_a_given_buffer(device):
+    """A preallocated float32 result is written in place (no second tensor, no copy)."""
+    from kernels.mamba_kernels.mamba_cumsum import _chunk_cumsum_fwd
+    from kernels.mamba_kernels.mamba_state_fwd import _chunk_state_fwd
+
+    b, L, nh, P, g, N, Q = 1, 512, 2, 64, 1, 128, 256
+    x, dt, A, B, C, D, _ = S.make_inputs(b, L, nh, P, g, N, seed=22, dtype=BF16)
+    xd, dtd, Ad, Bd = _dev(device, x, dt, A, B)
+    dA_cs, dt_out = _chunk_cumsum_fwd(dtd, Ad, Q)
+    ref = _chunk_state_fwd(Bd, xd, dt_out, dA_cs)
+    buf = torch.full_like(ref, float("nan"))
+    ptr = buf.data_ptr()
+    before = torch.cuda.memory_allocated(device)
+    out = _chunk_state_fwd(Bd, xd, dt_out, dA_cs, states=buf)
+    assert out is buf and buf.data_ptr() == ptr and torch.equal(buf, ref)
+    assert torch.cuda.memory_allocated(device) - before < ref.numel() * 4, "no second result tensor"
+    half = torch.empty(ref.shape, device=device, dtype=BF16)  # another dtype still goes through a copy
+    assert torch.equal(_chunk_state_fwd(Bd, xd, dt_out, dA_cs, states=half), ref.to(BF16))
+
+
 def test_unsupported_shapes_are_refused(device):
     from kernels.mamba_kernels.mamba_state_fwd import _chunk_state_fwd
 

@@ -40,11 +40,15 @@ def _chunk_scan_fwd(cb, x, dt, dA_cumsum, C, states, D=None, z=None, seq_idx=Non
     out_x = torch.empty_like(out) if z is not None else None
     Df = None if D is None else _lib.f32c(D)
     states, st_code = _lib.state_tensor(states, like=x)
+    # float32 views / copies are bound to names so that they outlive the launch below
+    cb_f = _lib.f32c(cb)
+    dt_f = _lib.f32c(dt)
+    dA_cumsum_f = _lib.f32c(dA_cumsum)
     with torch.cuda.device(dev):
         _lib.check(
             _lib.lib().ssd_chunk_scan_fwd(
-                _lib.f32c(cb).data_ptr(), *xs, *zs, _lib.dtype_code(x), _lib.f32c(dt).data_ptr(),
-                _lib.f32c(dA_cumsum).data_ptr(), *cs, states.data_ptr(), st_code,
+                cb_f.data_ptr(), *xs, *zs, _lib.dtype_code(x), dt_f.data_ptr(),
+                dA_cumsum_f.data_ptr(), *cs, states.data_ptr(), st_code,
                 None if Df is None else Df.data_ptr(), int(D is not None and D.dim() == 2), out.data_ptr(),
                 out.stride(0), out.stride(1), out.stride(2), None if out_x is None else out_x.data_ptr(), batch,
                 seqlen, nheads, ngroups, headdim, dstate, chunk_size, *ids, _lib.stream_ptr(dev)),

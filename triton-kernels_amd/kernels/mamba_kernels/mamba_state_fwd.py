@@ -28,16 +28,25 @@ def _chunk_state_fwd(B, x, dt, dA_cumsum, seq_idx=None, states=None, states_in_f
     seq_idx, ids = _lib.seq_ids(seq_idx, batch, seqlen, dev)
     x, xs = _lib.strided4(x)
     B, bs = _lib.strided4(B)
-    out = torch.empty(batch, nchunks, nheads, headdim, dstate, device=dev, dtype=torch.float32)
+    # a preallocated dense float32 result is written in place, as the reference's launcher does
+    # (kernels/mamba_kernels/mamba_state_fwd.py:147-151); any other goes through a copy
+    in_place = (states is not None and states.dtype == torch.float32 and states.is_contiguous()
+                and states.device == dev and states.shape == (batch, nchunks, nheads, headdim, dstate))
+    out = states if in_place else torch.empty(batch, nchunks, nheads, headdim, dstate, device=dev,
+                                              dtype=torch.float32)
+    # float32 views / copies are bound to names so that they outlive the launch below
+    dt_f = _lib.f32c(dt)
+    dA_cumsum_f = _lib.f32c(dA_cumsum)
     with torch.cuda.device(dev):
         _lib.check(
-            _lib.lib().ssd_chunk_state_fwd(*bs, *xs, _lib.dtype_code(x), _lib.f32c(dt).data_ptr(),
-                                           _lib.f32c(dA_cumsum).data_ptr(), out.data_ptr(), batch, seqlen, nheads,
+            _lib.lib().ssd_chunk_state_fwd(*bs, *xs, _lib.dtype_code(x), dt_f.data_ptr(),
+                                           dA_cumsum_f.data_ptr(), out.data_ptr(), batch, seqlen, nheads,
                                            ngroups, headdim, dstate, chunk_size, *ids, _lib.stream_ptr(dev)),
             "ssd_chunk_state_fwd")
     if states is not None:
         assert states.shape == (batch, nchunks, nheads, headdim, dstate)
-        states.copy_(out)
+        if not in_place:
+            states.copy_(out)
         return states
     return out if states_in_fp32 else out.to(B.dtype)
 
@@ -68,11 +77,14 @@ def chunk_state_varlen(B, x, dt, dA_cumsum, cu_seqlens, chunk_states):
     cu = cu_seqlens.to(torch.int32).contiguous()
     st, st_code = _lib.state_tensor(chunk_states, like=x)
     states = torch.empty(batch, nheads, headdim, dstate, device=dev, dtype=torch.float32)
+    # float32 views / copies are bound to names so that they outlive the launch below
+    dt_f = _lib.f32c(dt)
+    dA_cumsum_f = _lib.f32c(dA_cumsum)
     with torch.cuda.device(dev):
         _lib.check(
             _lib.lib().ssd_chunk_state_varlen(B.data_ptr(), B.stride(0), B.stride(1), x.data_ptr(), x.stride(0),
-                                              x.stride(1), _lib.dtype_code(x), _lib.f32c(dt).data_ptr(),
-                                              _lib.f32c(dA_cumsum).data_ptr(), st.data_ptr(), st_code,
+                                              x.stride(1), _lib.dtype_code(x), dt_f.data_ptr(),
+                                              dA_cumsum_f.data_ptr(), st.data_ptr(), st_code,
                                               cu.data_ptr(), states.data_ptr(), batch, total_seqlen, nheads, ngroups,
                                               headdim, dstate, chunk_size, _lib.stream_ptr(dev)),
             "ssd_chunk_state_varlen")

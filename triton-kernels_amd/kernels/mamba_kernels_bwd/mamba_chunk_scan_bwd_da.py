@@ -29,10 +29,14 @@ def _chunk_scan_bwd_ddAcs_stable(x, dt, dA_cumsum, dout, cb):
     nbytes = lib.ssd_chunk_scan_bwd_ddAcs_workspace_bytes(batch, seqlen, nheads, chunk_size)
     assert nbytes > 0, "unsupported shape"
     ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
+    # float32 views / copies are bound to names so that they outlive the launch below
+    dt_f = _lib.f32c(dt)
+    dA_cumsum_f = _lib.f32c(dA_cumsum)
+    cb_f = _lib.f32c(cb)
     with torch.cuda.device(dev):
         _lib.check(
-            lib.ssd_chunk_scan_bwd_ddAcs(*xs, *ds, _lib.dtype_code(x), _lib.f32c(dt).data_ptr(),
-                                         _lib.f32c(dA_cumsum).data_ptr(), _lib.f32c(cb).data_ptr(),
+            lib.ssd_chunk_scan_bwd_ddAcs(*xs, *ds, _lib.dtype_code(x), dt_f.data_ptr(),
+                                         dA_cumsum_f.data_ptr(), cb_f.data_ptr(),
                                          ddA_cumsum.data_ptr(), ws.data_ptr(), nbytes, batch, seqlen, nheads, ngroups,
                                          headdim, chunk_size, _lib.stream_ptr(dev)),
             "ssd_chunk_scan_bwd_ddAcs")

@@ -34,9 +34,11 @@ def _chunk_scan_bwd_dC(prev_states, dA_cumsum, dout, seq_idx=None, C=None, ngrou
         ddA_prev = torch.empty(batch, nheads, nchunks, chunk_size, device=dev, dtype=torch.float32)
     dC = torch.empty(batch, seqlen, ngroups, dstate, device=dev, dtype=torch.float32)
     prev_states, st_code = _lib.state_tensor(prev_states, like=dout)
+    # float32 views / copies are bound to names so that they outlive the launch below
+    dA_cumsum_f = _lib.f32c(dA_cumsum)
     with torch.cuda.device(dev):
         _lib.check(
-            _lib.lib().ssd_chunk_scan_bwd_dc(*ds, _lib.dtype_code(dout), _lib.f32c(dA_cumsum).data_ptr(),
+            _lib.lib().ssd_chunk_scan_bwd_dc(*ds, _lib.dtype_code(dout), dA_cumsum_f.data_ptr(),
                                              prev_states.data_ptr(), st_code, *cs, dC.data_ptr(),
                                              None if ddA_prev is None else ddA_prev.data_ptr(), batch, seqlen,
                                              nheads, ngroups, headdim, dstate, chunk_size, *ids,

@@ -47,11 +47,15 @@ def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum, B, CB, dout, dstates, D=Non
         slots = _lib.lib().ssd_chunk_scan_chunk_state_bwd_dx_dD_slots(_lib.dtype_code(x), headdim, dstate, chunk_size)
         assert slots > 0, "unsupported shape"
         dD_part = torch.empty(batch, nchunks, nheads, slots, headdim, device=dev, dtype=torch.float32)
+    # float32 views / copies are bound to names so that they outlive the launch below
+    CB_f = _lib.f32c(CB)
+    dt_f = _lib.f32c(dt)
+    dA_cumsum_f = _lib.f32c(dA_cumsum)
     with torch.cuda.device(dev):
         _lib.check(
             _lib.lib().ssd_chunk_scan_chunk_state_bwd_dx(
-                _lib.f32c(CB).data_ptr(), *xs, *ds, _lib.dtype_code(x), _lib.f32c(dt).data_ptr(),
-                _lib.f32c(dA_cumsum).data_ptr(), *bs, dstates.data_ptr(), ds_code,
+                CB_f.data_ptr(), *xs, *ds, _lib.dtype_code(x), dt_f.data_ptr(),
+                dA_cumsum_f.data_ptr(), *bs, dstates.data_ptr(), ds_code,
                 None if Df is None else Df.data_ptr(), int(D is not None and D.dim() == 2), dx.data_ptr(),
                 dx.stride(0), dx.stride(1), dx.stride(2), ddt.data_ptr(), batch, seqlen, nheads, ngroups, headdim,
                 dstate, chunk_size, *ids, None if dD_part is None else dD_part.data_ptr(), _lib.stream_ptr(dev)),

@@ -34,10 +34,13 @@ def _chunk_state_bwd_db(x, dt, dA_cumsum, dstates, seq_idx=None, B=None, ngroups
         ddA_cumsum = torch.empty(batch, nheads, nchunks, chunk_size, device=dev, dtype=torch.float32)
     dB = torch.empty(batch, seqlen, ngroups, dstate, device=dev, dtype=torch.float32)
     dstates, ds_code = _lib.state_tensor(dstates, like=x)
+    # float32 views / copies are bound to names so that they outlive the launch below
+    dt_f = _lib.f32c(dt)
+    dA_cumsum_f = _lib.f32c(dA_cumsum)
     with torch.cuda.device(dev):
         _lib.check(
-            _lib.lib().ssd_chunk_state_bwd_db(*xs, _lib.dtype_code(x), _lib.f32c(dt).data_ptr(),
-                                              _lib.f32c(dA_cumsum).data_ptr(), dstates.data_ptr(), ds_code, *bs,
+            _lib.lib().ssd_chunk_state_bwd_db(*xs, _lib.dtype_code(x), dt_f.data_ptr(),
+                                              dA_cumsum_f.data_ptr(), dstates.data_ptr(), ds_code, *bs,
                                               dB.data_ptr(), None if ddA_cumsum is None else ddA_cumsum.data_ptr(),
                                               batch, seqlen, nheads, ngroups, headdim, dstate, chunk_size, *ids,
                                               _lib.stream_ptr(dev)),

@@ -30,9 +30,11 @@ def _chunk_scan_bwd_dstates(C, dA_cumsum, dout, seq_idx=None, dtype=None):
     # the kernel stores float32, or bfloat16 next to bfloat16 inputs; any other type is cast afterwards
     native = dtype if dtype == torch.float32 or (dtype == torch.bfloat16 and dout.dtype == dtype) else torch.float32
     out = torch.empty(batch, nchunks, nheads, headdim, dstate, device=dev, dtype=native)
+    # float32 views / copies are bound to names so that they outlive the launch below
+    dA_cumsum_f = _lib.f32c(dA_cumsum)
     with torch.cuda.device(dev):
         _lib.check(
-            _lib.lib().ssd_chunk_scan_bwd_dstates(*cs, *ds, _lib.dtype_code(dout), _lib.f32c(dA_cumsum).data_ptr(),
+            _lib.lib().ssd_chunk_scan_bwd_dstates(*cs, *ds, _lib.dtype_code(dout), dA_cumsum_f.data_ptr(),
                                                   out.data_ptr(), _lib.dtype_code(out), batch, seqlen, nheads, ngroups, headdim, dstate,
                                                   chunk_size, *ids, _lib.stream_ptr(dev)),
             "ssd_chunk_scan_bwd_dstates")
