@@ -194,11 +194,11 @@ int launch_row_dot(const void* x, SeqStrides sx, int dtype, const float* vec, co
                    float* out, int raw, const Dims& d, hipStream_t st) {
   const unsigned grid = (unsigned)(d.N * d.C);
   if (dtype == EMA_BF16)
-    hipLaunchKernelGGL((row_dot_kernel<bf16_t, MODE>), dim3(grid), dim3(256), 0, st,
+    hipLaunchKernelGGL((row_dot_kernel<bf16_t, MODE>), dim3(grid), dim3(kRowDotThreads), 0, st,
                        (const bf16_t*)x, sx, vec, cs, out, (int)d.nh, (int)d.L, (int)d.T, (int)d.Q,
                        (int)d.C, raw);
   else
-    hipLaunchKernelGGL((row_dot_kernel<float, MODE>), dim3(grid), dim3(256), 0, st, (const float*)x,
+    hipLaunchKernelGGL((row_dot_kernel<float, MODE>), dim3(grid), dim3(kRowDotThreads), 0, st, (const float*)x,
                        sx, vec, cs, out, (int)d.nh, (int)d.L, (int)d.T, (int)d.Q, (int)d.C, raw);
   return launched();
 }

@@ -21,7 +21,7 @@ constexpr int kBM = 128;  // rows of a chunk handled by one workgroup (4 waves x
 // da_finish_kernel turns these into ddA_intra.
 // ------------------------------------------------------------------------------------
 template <typename T>
-__global__ __launch_bounds__(256) void da_gemm_kernel(const T* __restrict__ x, SeqStrides sx,
+__global__ __launch_bounds__(256, 2) void da_gemm_kernel(const T* __restrict__ x, SeqStrides sx,
                                                       const T* __restrict__ dy, SeqStrides sd,
                                                       const float* __restrict__ cs,
                                                       float* __restrict__ part,
@@ -70,6 +70,26 @@ __global__ __launch_bounds__(256) void da_gemm_kernel(const T* __restrict__ x, S
 
   constexpr int VPR = DK / EPL;   // 8 vectors per row
   constexpr int RPP = 256 / VPR;  // 32 rows per pass
+  constexpr int NP = kBM / RPP;   // passes (row pieces per thread and operand)
+  const int vcol = (tid % VPR) * EPL;
+  const int r0 = tid / VPR;
+  // One stage of both operands in registers: requested before the products of the stage before
+  // are formed, so that the loads travel meanwhile (the LDS tiles themselves are single).
+  Vec16<T> pd[NP], px[NP];
+  auto request = [&](int kt_base, int d0) {
+    const bool cok = d0 + vcol < Tdim;
+    const int dcol = cok ? d0 + vcol : 0;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      // unconditional loads from indices clamped into the tensor, zeroed afterwards
+      const int m = mt_base + r0 + p * RPP, k = kt_base + r0 + p * RPP;
+      pd[p] = load16(dp + (int64_t)min(m, limit - 1) * sd.sl + dcol);
+      px[p] = load16(xp + (int64_t)min(k, limit - 1) * sx.sl + dcol);
+      if (m >= limit || !cok) pd[p].zero();
+      if (k >= limit || !cok) px[p].zero();
+    }
+  };
+  request(0, 0);
   for (int kt = 0; kt <= mt; ++kt) {
     const int kt_base = kt * kBM;
     const int ncb = kt == mt ? wave + 1 : 4;  // column blocks at or below the diagonal
@@ -81,23 +101,15 @@ __global__ __launch_bounds__(256) void da_gemm_kernel(const T* __restrict__ x, S
 
     for (int d0 = 0; d0 < Tdim; d0 += DK) {
       __syncthreads();
-      {
-        const int vcol = (tid % VPR) * EPL;
-        const bool cok = d0 + vcol < Tdim;
 #pragma unroll
-        for (int r = tid / VPR; r < kBM; r += RPP) {
-          // unconditional loads from indices clamped into the tensor, zeroed afterwards
-          const int m = mt_base + r, k = kt_base + r;
-          const int dcol = cok ? d0 + vcol : 0;
-          Vec16<T> vd = load16(dp + (int64_t)min(m, limit - 1) * sd.sl + dcol);
-          Vec16<T> vx = load16(xp + (int64_t)min(k, limit - 1) * sx.sl + dcol);
-          if (m >= limit || !cok) vd.zero();
-          if (k >= limit || !cok) vx.zero();
-          store16(&dys[r * ROW + vcol], vd);
-          store16(&xs[r * ROW + vcol], vx);
-        }
+      for (int p = 0; p < NP; ++p) {
+        store16(&dys[(r0 + p * RPP) * ROW + vcol], pd[p]);
+        store16(&xs[(r0 + p * RPP) * ROW + vcol], px[p]);
       }
       __syncthreads();
+      // the stage after this one: next feature columns, or the first ones of the next column tile
+      if (d0 + DK < Tdim) request(kt_base, d0 + DK);
+      else if (kt < mt) request(kt_base + kBM, 0);
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int doff = g * KG + EPL * half;

@@ -231,16 +231,19 @@ __global__ __launch_bounds__(256) void state_passing_bwd_finish_kernel(
 //                chunk limit give 0; out[0] = 0, out[j] = r[j-1] (raw) or
 //                out[j] = sum_{m<j} r[m] (cumulative).
 //   MODE 1 (dc): out[m] = exp(cs[m]) * <dy[n,cQ+m], prev[n,c]>, 0 past the limit.
-// One workgroup per (n, c); wave w takes rows 4*w + 16*i + {0..3}; a wave covers the
-// feature axis with 16-byte loads per lane and reduces with DPP.
+// One workgroup of kRowDotThreads per (n, c); wave w takes rows R*w + R*NWV*i + {0..R-1}; a wave
+// covers the feature axis with 16-byte loads per lane (R of them in flight per lane and column
+// step) and reduces with DPP.
 // ------------------------------------------------------------------------------------
+constexpr int kRowDotThreads = 512;
 template <typename T, int MODE>
-__global__ __launch_bounds__(256) void row_dot_kernel(const T* __restrict__ x, SeqStrides sx,
-                                                      const float* __restrict__ vec,
-                                                      const float* __restrict__ cs,
-                                                      float* __restrict__ out, int nh, int L,
-                                                      int Tdim, int Q, int C, int raw) {
+__global__ __launch_bounds__(kRowDotThreads) void row_dot_kernel(const T* __restrict__ x, SeqStrides sx,
+                                                                 const float* __restrict__ vec,
+                                                                 const float* __restrict__ cs,
+                                                                 float* __restrict__ out, int nh, int L,
+                                                                 int Tdim, int Q, int C, int raw) {
   constexpr int VEC = Vec16<T>::N;
+  constexpr int NWV = kRowDotThreads / 64;
   __shared__ float rbuf[EMA_MAX_CHUNK_DEV];
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
@@ -255,8 +258,8 @@ __global__ __launch_bounds__(256) void row_dot_kernel(const T* __restrict__ x, S
   const float* vp = vec + chunk_id * Tdim;
   const T* xp = x + b * sx.sb + h * sx.sh + (int64_t)c * Q * sx.sl;
 
-  constexpr int R = 4;
-  for (int m0 = wave * R; m0 < Q; m0 += 4 * R) {
+  constexpr int R = 8;
+  for (int m0 = wave * R; m0 < Q; m0 += NWV * R) {
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = 0.f;
@@ -292,9 +295,9 @@ __global__ __launch_bounds__(256) void row_dot_kernel(const T* __restrict__ x, S
   __syncthreads();
   float* op = out + chunk_id * Q;
   if (MODE == 1) {
-    for (int m = tid; m < Q; m += 256) op[m] = rbuf[m];
+    for (int m = tid; m < Q; m += kRowDotThreads) op[m] = rbuf[m];
   } else if (raw) {
-    for (int m = tid; m < Q; m += 256) op[m] = m == 0 ? 0.f : rbuf[m - 1];
+    for (int m = tid; m < Q; m += kRowDotThreads) op[m] = m == 0 ? 0.f : rbuf[m - 1];
   } else if (wave == 0) {
     // out[j] = sum_{m<j} r[m]: exclusive scan, lane l owns positions l*per .. l*per+per-1
     const int per = (Q + 63) >> 6;
