@@ -302,6 +302,18 @@ def make_stages(sets, Q, torch):
     }
     outs = [torch.empty_like(s[0]) for s in sets]
     stages["copy"] = lambda i: outs[i % len(sets)].copy_(sets[i % len(sets)][0])
+    # the plainest streaming kernels, as ceilings: x -> out (the forward's traffic) and
+    # x, dy -> out (the backward's)
+    from kernels import _lib
+
+    def stream(i, two):
+        x, A, dy = sets[i % len(sets)]
+        o = outs[i % len(sets)]
+        _lib.check(_lib.lib().ema_stream_copy(x.data_ptr(), dy.data_ptr() if two else None, o.data_ptr(),
+                                              x.numel() * x.element_size(), _lib.stream_ptr(x.device)), "ema_stream_copy")
+
+    stages["stream_copy"] = lambda i: stream(i, False)
+    stages["stream_2in_1out"] = lambda i: stream(i, True)
     return stages
 
 
@@ -311,7 +323,8 @@ def time_stages(sets, Q, iters, torch, only=None):
     stages = make_stages(sets, Q, torch)
     x = sets[0][0]
     N, L, T = x.shape[0] * x.shape[2], x.shape[1], x.shape[3]
-    ab = dict(algorithmic_bytes(N, L, T, Q, 2), copy=2 * x.numel() * x.element_size())
+    xb = x.numel() * x.element_size()
+    ab = dict(algorithmic_bytes(N, L, T, Q, 2), copy=2 * xb, stream_copy=2 * xb, stream_2in_1out=3 * xb)
     res = {}
     for name, fn in stages.items():
         if only and name not in only:

@@ -94,6 +94,13 @@ typedef struct {
  * `stream`: the state in which workspace_ready = 1 may be passed. */
 int ema_workspace_clear(void* workspace, size_t bytes, void* stream);
 
+/* Measurement aid (no counterpart in the reference): dst = a, or dst = a ^ b when b is not NULL,
+ * `bytes` bytes (a multiple of 16; pointers 16-byte aligned), one 16-byte piece per thread with
+ * non-temporal accesses.  bench.py times it back to back over rotating buffers: what the plainest
+ * streaming kernel sustains on the device is the practical ceiling next to which the scan
+ * kernels' rates are reported. */
+int ema_stream_copy(const void* a, const void* b, void* dst, size_t bytes, void* stream);
+
 /* Largest chunk size accepted by every entry point. */
 #define EMA_MAX_CHUNK 1024
 

@@ -2,7 +2,6 @@
 // reference launcher each entry point replaces are in include/ema_hip.h.
 #include "../../include/ema_hip.h"
 
-#include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 
 #include <mutex>
@@ -251,17 +250,18 @@ inline int record_event(void* ev, hipStream_t st) {
   return hipEventRecord(reinterpret_cast<hipEvent_t>(ev), st) == hipSuccess ? EMA_OK : EMA_ERR_LAUNCH;
 }
 
-// Launches a kernel that uses no dynamic LDS.  With events (hipEvent_t, either may be NULL) the
-// runtime stamps them with the start and the end of this very dispatch, so their difference is
-// the kernel's own duration, free of the gaps around it.
+// Launches a kernel that uses no dynamic LDS, with optional events (hipEvent_t, either may be NULL)
+// recorded on the stream right before and right after it.  In a sequence of launches the interval
+// between them is the kernel's share of the stream's time: it starts when the work before is
+// complete (written back), which is also how a kernel trace accounts a dispatch; the runtime's own
+// start / stop stamps of the dispatch leave out what the hand-over between two kernels costs.
 template <typename... Args>
-void launch_timed(void (*kernel)(Args...), dim3 grid, dim3 block, hipStream_t st, void* ev0, void* ev1,
-                  Args... args) {
-  if (ev0 || ev1)
-    hipExtLaunchKernelGGL(kernel, grid, block, 0, st, reinterpret_cast<hipEvent_t>(ev0),
-                          reinterpret_cast<hipEvent_t>(ev1), 0, args...);
-  else
-    hipLaunchKernelGGL(kernel, grid, block, 0, st, args...);
+int launch_timed(void (*kernel)(Args...), dim3 grid, dim3 block, hipStream_t st, void* ev0, void* ev1,
+                 Args... args) {
+  if (ev0 && hipEventRecord(reinterpret_cast<hipEvent_t>(ev0), st) != hipSuccess) return EMA_ERR_LAUNCH;
+  hipLaunchKernelGGL(kernel, grid, block, 0, st, args...);
+  if (ev1 && hipEventRecord(reinterpret_cast<hipEvent_t>(ev1), st) != hipSuccess) return EMA_ERR_LAUNCH;
+  return EMA_OK;
 }
 
 // Workgroups of a persistent kernel that can be resident at once on the current device.
@@ -320,7 +320,7 @@ int launch_clear(void* base, size_t bytes, hipStream_t st) {
 // 64 times that many columns), rows per lane (128 / RPL waves per workgroup), waves per SIMD
 // the register allocation must allow.
 #ifndef EMA_FWD_SHAPE  // columns per lane, rows per lane, waves per SIMD
-#define EMA_FWD_SHAPE 4, 8, 8
+#define EMA_FWD_SHAPE 4, 8, 4
 #endif
 #ifndef EMA_BWD_SHAPE
 #define EMA_BWD_SHAPE 4, 8, 4
@@ -334,7 +334,7 @@ struct TileBf16 {
   static constexpr int BWD_CPL = B.cpl, BWD_RPL = B.rpl, BWD_MINW = B.minw;
 };
 struct TileF32 {
-  static constexpr int FWD_CPL = 2, FWD_RPL = 8, FWD_MINW = 8;
+  static constexpr int FWD_CPL = 2, FWD_RPL = 8, FWD_MINW = 4;
   static constexpr int BWD_CPL = 2, BWD_RPL = 8, BWD_MINW = 4;
 };
 
@@ -353,9 +353,9 @@ int launch_fwd_tile_t(const void* x, SeqStrides sx, const float* A, SeqStrides s
   const ChainWs w = chain_carve(chain_base, di);
   auto kernel = fwd_tile_kernel<T, S::FWD_CPL, S::FWD_RPL, S::FWD_MINW, XP>;
   const int64_t cap = resident_blocks(kernel, NT, 0);
-  launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx, A,
-               sa, (T*)y, sy, prev128, prev_coarse, ratio, fin, init, w.hdr, w.decw, w.status, (int)di.nh,
-               (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total);
+  EMA_TRY(launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x,
+                       sx, A, sa, (T*)y, sy, prev128, prev_coarse, ratio, fin, init, w.hdr, w.decw, w.status,
+                       (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total));
   return launched();
 }
 
@@ -373,9 +373,10 @@ int launch_bwd_tile_k(const void* x, SeqStrides sx, const void* dy, SeqStrides s
   const ChainWs w = chain_carve(chain_base, di);
   auto kernel = bwd_tile_kernel<T, S::BWD_CPL, S::BWD_RPL, S::BWD_MINW, WRITE_Y, XP>;
   const int64_t cap = resident_blocks(kernel, NT, 0);
-  launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x, sx,
-               (const T*)dy, sd, A, sa, prev128, (T*)dx, sdx, (T*)y, sy, part, dfinal, dinit, w.hdr, w.decw,
-               w.status, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total);
+  EMA_TRY(launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x,
+                       sx, (const T*)dy, sd, A, sa, prev128, (T*)dx, sdx, (T*)y, sy, part, dfinal, dinit, w.hdr,
+                       w.decw, w.status, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols,
+                       (int)total));
   return launched();
 }
 
@@ -555,6 +556,19 @@ size_t ema_fwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, in
   Dims d;
   if (check_dims(batch, nheads, seqlen, dim, chunk, true, &d) != EMA_OK) return 0;
   return carve_fwd(nullptr, d).bytes;
+}
+
+int ema_stream_copy(const void* a, const void* b, void* dst, size_t bytes, void* stream) {
+  if (!a || !dst) return EMA_ERR_NULL;
+  if (bytes % 16 || reinterpret_cast<uintptr_t>(a) % 16 || reinterpret_cast<uintptr_t>(dst) % 16 ||
+      reinterpret_cast<uintptr_t>(b) % 16)
+    return EMA_ERR_ALIGN;
+  const int64_t n16 = (int64_t)(bytes / 16);
+  if (n16 == 0) return EMA_OK;
+  if ((n16 + 255) / 256 > 0x7fffffff) return EMA_ERR_SHAPE;
+  hipLaunchKernelGGL(stream_copy_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, as_stream(stream),
+                     static_cast<const uint4*>(a), static_cast<const uint4*>(b), static_cast<uint4*>(dst), n16);
+  return launched();
 }
 
 int ema_workspace_clear(void* workspace, size_t bytes, void* stream) {

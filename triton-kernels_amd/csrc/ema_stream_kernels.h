@@ -7,6 +7,21 @@
 namespace ema {
 
 // ------------------------------------------------------------------------------------
+// Measurement aid: the plainest streaming kernel, one 16-byte piece per thread, non-temporal;
+// dst = a (one source) or dst = a ^ b (two sources).  What it sustains is the practical ceiling
+// the scan kernels are held against.
+// ------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void stream_copy_kernel(const uint4* __restrict__ a, const uint4* __restrict__ b,
+                                                          uint4* __restrict__ dst, int64_t n16) {
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n16) return;
+  u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a) + i);
+  if (b) v ^= __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(b) + i);
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst) + i);
+}
+
+// ------------------------------------------------------------------------------------
 // F1: per-chunk inclusive cumsum of the log-decay.  One wave per (n, c); lane l owns the
 // `per` consecutive positions starting at l * per, sums them serially, and the lane totals
 // are scanned across the wave with DPP.  With prob != 0 the input holds probabilities p and

@@ -275,33 +275,46 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
   __shared__ __attribute__((aligned(16))) float sP[2][BN];      // state entering the tile
   __shared__ float sD[2][NG];                                   // total decay of each row group
   __shared__ float sW[2][NG];                                   // decay of the groups before each group
-  __shared__ int s_ticket[2];
+  __shared__ int s_ticket[3];
   const int lane = threadIdx.x & 63;
   const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const unsigned off = (unsigned)lane * CPL;
+  const bool looks = grp * 64 < BN;  // this wave's threads own a column each in step 2
   const ChainCtl ctl = chain_enter(hdr);
 
-  if (threadIdx.x == 0) s_ticket[0] = (int)atomicAdd(&hdr->ticket, 1u);
+  if (threadIdx.x == 0) {
+    s_ticket[0] = (int)atomicAdd(&hdr->ticket, 1u);
+    s_ticket[1] = (int)atomicAdd(&hdr->ticket, 1u);
+  }
   __syncthreads();
-  int cur = s_ticket[0], buf = 0, slot = 1;
-  // The rows of a tile are requested while the tile before is being stored (row i of the next
-  // tile goes into the registers that row i of this one has just left), so that loads and stores
-  // are under way together; the first tile's rows are requested here.
-  RowWords<NW> rows[RPL];
-  float araw[RPL];
+  int cur = s_ticket[0], nxt = s_ticket[1], buf = 0, slot = 2;
+
+  // Two register sets hold the tile being processed and the one after it: the rows of the next
+  // tile are requested right after the first barrier, so they travel while this tile waits for
+  // its look-back, makes its final pass and stores.  The waves whose threads look back request
+  // theirs after the look-back: loads return in the order of their requests, and a poll queued
+  // behind eight row loads would wait for all of them.
+  RowWords<NW> rowsA[RPL], rowsB[RPL];
+  float arawA[RPL], arawB[RPL];
+  auto request = [&](RowWords<NW>* rows, float* araw, const ChainTile& tt, const TileAt& aa) {
+    const T* g = x + (int64_t)tt.b * sx.sb + (int64_t)tt.h * sx.sh +
+                 ((int64_t)tt.c * kTileRows + RPL * grp) * sx.sl + tt.col0 + off;
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) rows[i] = tile_load_row<NW, kStreamFwdLoad>(g, sx.sl, i, aa);
+    tile_coef_load<RPL>(araw, A + (int64_t)tt.b * sa.sb + (int64_t)tt.h * sa.sh +
+                                  ((int64_t)tt.c * kTileRows + RPL * grp) * sa.sl, sa.sl, aa.nrows);
+  };
   ChainTile t = chain_decode<false, BN>(cur < total ? cur : 0, cols, ntiles, C, nh, L);
   TileAt at = tile_at<RPL>(t.limit, grp, t.col0 + lane * CPL < Tdim);
-  if (cur < total) {
-    const T* g = x + (int64_t)t.b * sx.sb + (int64_t)t.h * sx.sh +
-                 ((int64_t)t.c * kTileRows + RPL * grp) * sx.sl + t.col0 + off;
-#pragma unroll
-    for (int i = 0; i < RPL; ++i) rows[i] = tile_load_row<NW, kStreamFwdLoad>(g, sx.sl, i, at);
-    tile_coef_load<RPL>(araw, A + (int64_t)t.b * sa.sb + (int64_t)t.h * sa.sh +
-                                  ((int64_t)t.c * kTileRows + RPL * grp) * sa.sl, sa.sl, at.nrows);
-  }
-  while (cur < total) {
+  if (cur < total) request(rowsA, arawA, t, at);
+
+  // one tile: `rows` / `araw` hold it, `rows_n` / `araw_n` receive the next one
+  auto tile = [&](RowWords<NW>* rows, float* araw, RowWords<NW>* rows_n, float* araw_n) {
     int future = 0;
     if (threadIdx.x == 0) future = (int)atomicAdd(&hdr->ticket, 1u);
+    const bool more = nxt < total;
+    const ChainTile tn = chain_decode<false, BN>(more ? nxt : 0, cols, ntiles, C, nh, L);
+    const TileAt atn = tile_at<RPL>(tn.limit, grp, tn.col0 + lane * CPL < Tdim);
     EMA_TSTAMP_DECL;
     EMA_TSTAMP(0);
     float a[RPL];
@@ -323,6 +336,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
     rows_opaque<NW, RPL>(rows);
     __syncthreads();
     EMA_TSTAMP(1);
+    if (more && !looks) request(rows_n, araw_n, tn, atn);
 
     // 2. one thread per column: chain over the row groups, publish, look back
     if (threadIdx.x < BN) {
@@ -366,42 +380,38 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
         if (final_state && t.c == C - 1) final_state[(int64_t)t.n * Tdim + t.col0 + k] = p_out;
       }
     }
+    if (more && looks) request(rows_n, araw_n, tn, atn);
     if (threadIdx.x == 0) s_ticket[slot] = future;
     __syncthreads();
     EMA_TSTAMP(2);
 
-    // 3. final pass from the true state; behind each stored row the same row of the next tile
-    // is requested
-    const int next = s_ticket[slot];
-    const bool more = next < total;
-    const ChainTile tn = chain_decode<false, BN>(more ? next : 0, cols, ntiles, C, nh, L);
-    const TileAt atn = tile_at<RPL>(tn.limit, grp, tn.col0 + lane * CPL < Tdim);
+    // 3. final pass from the true state
     {
       const float wg = sW[buf][grp];
 #pragma unroll
       for (int e = 0; e < CPL; ++e) s[e] = fmaf(wg, sP[buf][lane * CPL + e], sS[buf][grp][lane * CPL + e]);
       T* g = y + (int64_t)t.b * sy.sb + (int64_t)t.h * sy.sh +
              ((int64_t)t.c * kTileRows + RPL * grp) * sy.sl + t.col0 + off;
-      const T* gn = x + (int64_t)tn.b * sx.sb + (int64_t)tn.h * sx.sh +
-                    ((int64_t)tn.c * kTileRows + RPL * grp) * sx.sl + tn.col0 + off;
 #pragma unroll
       for (int i = 0; i < RPL; ++i) {
 #pragma unroll
         for (int e = 0; e < CPL; ++e) s[e] = tile_step<XP>(a[i], s[e], row_get<T, NW>(rows[i], e));
         if (i < at.nrows && at.cok) row_store<NW, kStreamFwdStore>(g + (int64_t)i * sy.sl, row_pack<T, CPL, NW>(s));
-        if (more) rows[i] = tile_load_row<NW, kStreamFwdLoad>(gn, sx.sl, i, atn);
       }
-      if (more)
-        tile_coef_load<RPL>(araw, A + (int64_t)tn.b * sa.sb + (int64_t)tn.h * sa.sh +
-                                      ((int64_t)tn.c * kTileRows + RPL * grp) * sa.sl, sa.sl, atn.nrows);
     }
     EMA_TSTAMP(3);
     EMA_TSTAMP_FLUSH;
-    cur = next;
+    cur = nxt;
+    nxt = s_ticket[slot];
     t = tn;
     at = atn;
-    slot ^= 1;
+    slot = slot == 2 ? 0 : slot + 1;
     buf ^= 1;
+  };
+  while (cur < total) {
+    tile(rowsA, arawA, rowsB, arawB);
+    if (cur >= total) break;
+    tile(rowsB, arawB, rowsA, arawA);
   }
   if (threadIdx.x == 0) chain_leave(hdr, ctl);
 }
