@@ -34,7 +34,7 @@ for p in (ROOT, os.path.join(ROOT, "triton-kernels_amd")):
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (summaries and commands under
 # profiles/), scaled by what the same counters read for a plain 268 435 456-byte device copy
 # (FETCH_SIZE reads 131 085 KiB for it, factor 1.99982; WRITE_SIZE reads 262 144 KiB, factor 1).
-TRAFFIC_BYTES = {"fwd_single_pass": None, "bwd_single_pass": None}
+TRAFFIC_BYTES = {"fwd_single_pass": 570370042, "bwd_single_pass": 841222651}
 TRAFFIC_SOURCE = "profiles/single_pass_tile_kernels_b16_nh2_d1024_L4096_c128_hbm_traffic.txt (rocprofv3 --pmc, not measured by this run)"
 # the same for the SSD stage kernels at configuration 5 (finishing kernels added to their stage)
 SSD_TRAFFIC_BYTES = {
@@ -597,7 +597,7 @@ def main():
         "frac": main_k[dom]["GBps"] / HBM_PEAK_GBS,
         "traffic": TRAFFIC_BYTES.get(dom),
         "traffic_source": TRAFFIC_SOURCE,
-        "duration": "mean of the dispatches of the timed fwd,bwd sequence (runtime start/stop stamps)",
+        "duration": "mean over the timed fwd,bwd sequence of the time between events recorded on the launch stream directly before and after the launch",
     }
     del run
     torch.cuda.empty_cache()
