@@ -82,6 +82,23 @@ int ssd_state_passing_fwd(const float* states, const float* dA_chunk, int64_t da
                           int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, const int32_t* seq_idx,
                           int64_t seq_sb, int64_t seq_sl, int64_t seqlen, int64_t chunk, void* stream);
 
+/* ssd_chunk_state_fwd and ssd_state_passing_fwd in one pass over x and B: the chunk-local states,
+ * which are float32 and twice the bytes of x, stay in registers instead of going through memory.
+ * out (batch, C, nheads, hdim, dstate), float32 or bfloat16 (out_dtype), receives the state entering
+ * each chunk; final_states (batch, nheads, hdim, dstate) float32 the state after the last chunk;
+ * initial of that shape, float32, may be NULL.  The results equal those of the two entry points
+ * called one after the other bit for bit.  chunk must be a multiple of 64 (SSD_ERR_UNSUPPORTED
+ * otherwise); packed batches (seq_idx) go through the two separate entry points.
+ * Replaces the pair _chunk_state_fwd, kernels/mamba_kernels/mamba_state_fwd.py:138-169, and
+ * _state_passing_fwd, kernels/mamba_kernels/mamba_state_pass.py:84-115, where a caller runs them
+ * back to back (the single-kernel chunk walk of kernels/mamba_3_kernels/mamba_ssd_fwd.py:247-258
+ * carries its state the same way). */
+int ssd_chunk_state_passing_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64_t b_sg, const void* x,
+                                int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, const float* dt,
+                                const float* dA_cumsum, const float* initial, void* out, int out_dtype,
+                                float* final_states, int64_t batch, int64_t seqlen, int64_t nheads,
+                                int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk, void* stream);
+
 /* out[b,c,g,m,k] = sum_n a[b,cQ+m,g,n] * bm[b,cQ+k,g,n]; rows past seqlen are zero.  out is
  * float32 or `dtype` (out_dtype).  With seq_idx, out[m,k] = 0 where the ids of m and k differ
  * (mamba_bmm.py:70-73).  Replaces _bmm_chunk_fwd, kernels/mamba_kernels/mamba_bmm.py:88-126

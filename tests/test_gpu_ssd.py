@@ -220,6 +220,79 @@ def test_chunk_states_into_a_given_buffer(device):
     assert torch.equal(_chunk_state_fwd(Bd, xd, dt_out, dA_cs, states=half), ref.to(BF16))
 
 
+WALK_CASES = [
+    # b, L, nh, P, g, N, Q
+    (2, 300, 4, 64, 1, 64, 64),     # last chunk ragged, last stage ragged
+    (1, 256, 2, 64, 2, 128, 128),
+    (2, 200, 4, 64, 1, 128, 256),   # a single ragged chunk
+    (1, 520, 2, 128, 1, 64, 128),
+    (1, 130, 2, 128, 2, 128, 64),
+    (1, 900, 3, 64, 1, 64, 512),
+    (1, 1100, 2, 64, 1, 128, 1024),
+    (3, 64, 2, 64, 1, 128, 64),     # one stage in all
+]
+
+
+@pytest.mark.parametrize("out_dtype", [F32, BF16], ids=["out_f32", "out_bf16"])
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("b,L,nh,P,g,N,Q", WALK_CASES)
+def test_chunk_state_passing_in_one_kernel(b, L, nh, P, g, N, Q, dtype, out_dtype, device):
+    """The kernel that keeps the chunk-local states on chip against the two launchers it replaces:
+    the same bits, with and without an initial state, and the oracle's restatements on top."""
+    from kernels.mamba_kernels.mamba_combined_fwd import _chunk_state_passing_fwd
+    from kernels.mamba_kernels.mamba_cumsum import _chunk_cumsum_fwd
+    from kernels.mamba_kernels.mamba_state_fwd import _chunk_state_fwd
+    from kernels.mamba_kernels.mamba_state_pass import _state_passing_fwd
+
+    if dtype == F32 and out_dtype == BF16:
+        pytest.skip("float32 inputs carry float32 states")
+    announce(f"ssd state walk b{b} L{L} nh{nh} P{P} g{g} N{N} Q{Q} {dtype} -> {out_dtype}")
+    x, dt, A, B, _, _, _ = S.make_inputs(b, L, nh, P, g, N, seed=L + N + Q, dtype=dtype)
+    init = torch.randn(b, nh, P, N, generator=torch.Generator().manual_seed(9))
+    xd, dtd, Ad, Bd, initd = _dev(device, x, dt, A, B, init)
+    dA_cs, dt_out = _chunk_cumsum_fwd(dtd, Ad, Q)
+    C = dA_cs.shape[2]
+    for ini in (None, initd):
+        local = _chunk_state_fwd(Bd, xd, dt_out, dA_cs)
+        ref, ref_fin = _state_passing_fwd(local.view(b, C, nh, P * N), dA_cs[..., -1],
+                                          initial_states=None if ini is None else ini.view(b, nh, P * N),
+                                          out_dtype=out_dtype)
+        got, fin = _chunk_state_passing_fwd(Bd, xd, dt_out, dA_cs, initial_states=ini, out_dtype=out_dtype)
+        torch.cuda.synchronize()
+        assert got.dtype == out_dtype and got.shape == (b, C, nh, P, N) and fin.shape == (b, nh, P, N)
+        assert torch.equal(got.view(b, C, nh, P * N), ref), "states entering the chunks differ from the two launchers"
+        assert torch.equal(fin.view(b, nh, P * N), ref_fin), "final states differ from the two launchers"
+    # against the oracle (no initial state)
+    dA_ref, dt_ref = S.chunk_cumsum(dt, A, Q)
+    st_ref = S.chunk_state(B, x, dt_ref, dA_ref, round_to=None if dtype == F32 else BF16)
+    prev_ref, fin_ref = S.state_passing(st_ref.reshape(b, C, nh, P * N), dA_ref[..., -1])
+    got, fin = _chunk_state_passing_fwd(Bd, xd, dt_out, dA_cs, out_dtype=F32)
+    check_close("states entering the chunks", got, prev_ref.view(b, C, nh, P, N), dtype)
+    check_close("final states", fin, fin_ref.view(b, nh, P, N), dtype)
+
+
+def test_chunk_state_passing_views_and_limits(device):
+    """x and B as slices of a wider projection give the bits of contiguous copies; chunk sizes the
+    kernel does not take are left to the two launchers (None)."""
+    from kernels.mamba_kernels.mamba_combined_fwd import _chunk_state_passing_fwd
+    from kernels.mamba_kernels.mamba_cumsum import _chunk_cumsum_fwd
+
+    b, L, nh, P, g, N, Q = 2, 384, 4, 64, 1, 128, 128
+    x, dt, A, B, _, _, _ = S.make_inputs(b, L, nh, P, g, N, seed=31, dtype=BF16)
+    xd, dtd, Ad, Bd = _dev(device, x, dt, A, B)
+    wide = torch.randn(b, L, nh * P + g * N + 24, device=device).to(BF16)
+    xv = wide[..., : nh * P].view(b, L, nh, P)
+    Bv = wide[..., nh * P : nh * P + g * N].view(b, L, g, N)
+    xv.copy_(xd)
+    Bv.copy_(Bd)
+    dA_cs, dt_out = _chunk_cumsum_fwd(dtd, Ad, Q)
+    a = _chunk_state_passing_fwd(Bd, xd, dt_out, dA_cs, out_dtype=BF16)
+    v = _chunk_state_passing_fwd(Bv, xv, dt_out, dA_cs, out_dtype=BF16)
+    assert torch.equal(a[0], v[0]) and torch.equal(a[1], v[1])
+    dA48, dt48 = _chunk_cumsum_fwd(dtd, Ad, 48)
+    assert _chunk_state_passing_fwd(Bd, xd, dt48, dA48) is None
+
+
 def test_unsupported_shapes_are_refused(device):
     from kernels.mamba_kernels.mamba_state_fwd import _chunk_state_fwd
 

@@ -118,6 +118,36 @@ struct StateLaunch {
   }
 };
 
+struct WalkLaunch {
+  const void *x, *B;
+  Strides3 sx, sB;
+  const float *dt, *dA, *initial;
+  void* out;
+  int out_dtype;
+  float* final_states;
+  Dims d;
+  hipStream_t st;
+  template <typename T, int P, int N>
+  int run() const {
+    if (out_dtype == SSD_BF16) return run_as<T, P, N, bf16_t>();
+    return run_as<T, P, N, float>();
+  }
+  template <typename T, int P, int N, typename TO>
+  int run_as() const {
+#ifndef SSD_WALK_NSPLIT  // 2: two workgroups per (b, h), half the state columns each (measured no faster: x crosses the L2 twice)
+#define SSD_WALK_NSPLIT 1
+#endif
+    constexpr int NSPLIT = (SSD_WALK_NSPLIT == 2 && ((P / 32) * (N / 64)) % 4 == 0 && P * N <= 64 * 128) ? 2 : 1;
+    auto kernel = ssd_state_walk_kernel<T, P, N, TO, NSPLIT>;
+    constexpr int smem = WalkSmem<T, P, N / NSPLIT>::kBytes;
+    SSD_TRY(allow_smem(kernel, smem));
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.nh * NSPLIT)), dim3(256), smem, st, (const T*)x, sx,
+                       (const T*)B, sB, dt, dA, initial, (TO*)out, final_states, (int)d.nh, (int)(d.nh / d.g),
+                       (int)d.L, (int)d.Q, (int)d.C);
+    return launched();
+  }
+};
+
 struct ScanLaunch {
   const float* cb;
   const void *x, *z, *C;
@@ -334,6 +364,27 @@ int ssd_chunk_state_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64_t b_sg,
   return dispatch_tpn(dtype, hdim, dstate,
                       StateLaunch<0>{x, B, Strides3{x_sb, x_sl, x_sh}, Strides3{b_sb, b_sl, b_sg}, dt, dA_cumsum,
                                      states, SSD_F32, d, as_seq(seq_idx, seq_sb, seq_sl), as_stream(stream)});
+}
+
+int ssd_chunk_state_passing_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64_t b_sg, const void* x,
+                                int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype, const float* dt,
+                                const float* dA_cumsum, const float* initial, void* out, int out_dtype,
+                                float* final_states, int64_t batch, int64_t seqlen, int64_t nheads,
+                                int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk, void* stream) {
+  Dims d;
+  SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
+  SSD_TRY(check_dtype(dtype));
+  SSD_TRY(check_dtype(out_dtype));
+  if (!dim_ok(hdim) || !dim_ok(dstate) || chunk % 64) return SSD_ERR_UNSUPPORTED;
+  SSD_TRY(check_vec(x, x_sb, x_sl, x_sh, dtype, hdim));
+  SSD_TRY(check_vec(B, b_sb, b_sl, b_sg, dtype, dstate));
+  if (!dt || !dA_cumsum) return SSD_ERR_NULL;
+  SSD_TRY(check_f32(out));
+  SSD_TRY(check_f32(final_states));
+  if (initial) SSD_TRY(check_f32(initial));
+  return dispatch_tpn(dtype, hdim, dstate,
+                      WalkLaunch{x, B, Strides3{x_sb, x_sl, x_sh}, Strides3{b_sb, b_sl, b_sg}, dt, dA_cumsum, initial,
+                                 out, out_dtype, final_states, d, as_stream(stream)});
 }
 
 int ssd_state_passing_fwd(const float* states, const float* dA_chunk, int64_t da_sb, int64_t da_sh,

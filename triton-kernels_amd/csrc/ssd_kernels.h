@@ -187,7 +187,8 @@ struct RowPieces {
   static_assert((ROWS * VPR) % 256 == 0 && CNT <= 8, "tile must split evenly over 256 threads");
   Vec16<T> v[CNT];
   float a0[CNT], a1[CNT];
-  template <bool STREAM = false>
+  // BOTH: aux0 and aux1 are given (no test of the pointers between the loads)
+  template <bool STREAM = false, bool BOTH = false>
   __device__ __forceinline__ void load(const T* __restrict__ g, int64_t row_stride, int row0, int limit, int tid,
                                        const float* __restrict__ aux0 = nullptr,
                                        const float* __restrict__ aux1 = nullptr) {
@@ -197,8 +198,8 @@ struct RowPieces {
       const int row = min(row0 + idx / VPR, limit - 1);
       const T* src = g + (int64_t)row * row_stride + (idx % VPR) * EPL;
       v[i] = STREAM ? load16_stream(src) : load16(src);
-      if (aux0) a0[i] = aux0[row];
-      if (aux1) a1[i] = aux1[row];
+      if (BOTH || aux0) a0[i] = aux0[row];
+      if (BOTH || aux1) a1[i] = aux1[row];
     }
   }
   // scale(row, aux0[row], aux1[row]) multiplies the row; NoScale leaves it
@@ -530,6 +531,169 @@ __global__ __launch_bounds__(256) void ssd_state_passing_kernel(
   }
 #pragma unroll
   for (int i = 0; i < E; ++i) final_states[(b * nh + h) * (int64_t)dim + e + i] = s.v[i];
+}
+
+// ------------------------------------------------------------------------------------
+// chunk_state and state_passing in one pass over x and B.  One workgroup (4 waves) per (b, h)
+// walks the whole sequence in stages of 64 rows.  The local state of a chunk accumulates on MFMA
+// exactly as in ssd_chunk_state_kernel (MODE 0); when a chunk ends the running state (float32, in
+// the accumulator layout) becomes exp(dA_last) * state + local, as in ssd_state_passing_kernel, and
+// when a chunk begins it is written out as the state entering that chunk.  The results equal those
+// of the two kernels run one after the other bit for bit (same products in the same order, same
+// fused multiply-add), while the chunk-local float32 states, twice the bytes of x, never touch
+// memory.  The rows of D stages are in flight in registers at any time (a workgroup is alone on its
+// compute unit and walks its rows in sequence, so the depth of this ring is what keeps its share
+// of the memory system busy); LDS holds two stages, so a stage costs one barrier.  Q must be a
+// multiple of 64 (a stage lies inside one chunk).  dt and dA_cs are (b, nh, C, Q), so position r of
+// the sequence sits at offset r of the (b, h) row whatever the chunk.  No packed batches.
+// ------------------------------------------------------------------------------------
+#ifndef SSD_WALK_DIAG  // diagnostic builds (wrong results on purpose): 1 no state stores, 2 no products, 3 neither LDS stores nor products
+#define SSD_WALK_DIAG 0
+#endif
+template <typename T, int P, int NL>
+struct WalkSmem {
+  static constexpr int KT = 64, PX = Tile<T>::pitch(P), PB = Tile<T>::pitch(NL);
+  static constexpr int kStageElems = KT * (PX + PB);
+  static constexpr int kBytes = 2 * kStageElems * (int)sizeof(T);
+};
+
+// NSPLIT workgroups share one (b, h), each with N / NSPLIT columns of the state: with two of them
+// per compute unit one multiplies while the other waits for its rows.  They read the same rows of
+// x (adjacent workgroups, the same L2).
+template <typename T, int P, int N, typename TO, int NSPLIT>
+__global__ __launch_bounds__(256, NSPLIT) void ssd_state_walk_kernel(
+    const T* __restrict__ x, Strides3 sx, const T* __restrict__ B, Strides3 sB, const float* __restrict__ dt,
+    const float* __restrict__ dA_cs, const float* __restrict__ initial, TO* __restrict__ out,
+    float* __restrict__ final_states, int nh, int heads_per_group, int L, int Q, int C) {
+  constexpr int NL = N / NSPLIT;
+  using S = WalkSmem<T, P, NL>;
+  constexpr int KT = S::KT, PX = S::PX, PB = S::PB, KG = Tile<T>::KG;
+  constexpr int MB = P / 32, NB = NL / 32, BPW = MB * NB / 4;
+  static_assert(MB * NB % 4 == 0, "output blocks must split over 4 waves");
+  // stages in flight: as many as the registers hold next to the two sets of accumulators
+  constexpr int kPieceRegs = NSPLIT == 2
+      ? (RowPieces<T, KT, P>::CNT + RowPieces<T, KT, NL>::CNT) * 6 + 2 * RowPieces<T, KT, NL>::CNT
+      : (RowPieces<T, KT, P>::CNT + RowPieces<T, KT, NL>::CNT) * 4 + 2 * RowPieces<T, KT, NL>::CNT;
+  constexpr int kRoom = 256 - 2 * BPW * 16 - (NSPLIT == 2 ? 140 : 40 + 8 * BPW + (sizeof(T) == 4 ? 16 : 0));
+#ifdef SSD_WALK_D
+  constexpr int D = SSD_WALK_D;
+#else
+  constexpr int D = kRoom >= 4 * kPieceRegs ? 4 : (kRoom >= 3 * kPieceRegs ? 3 : (kRoom >= 2 * kPieceRegs ? 2 : 1));
+#endif
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T* lds = reinterpret_cast<T*>(smem);
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
+  const int part = bid % NSPLIT;
+  const int h = (bid / NSPLIT) % nh;
+  const int64_t b = bid / (NSPLIT * nh);
+  const int n0 = part * NL;  // first state column of this workgroup
+  const float* dAb = dA_cs + (b * nh + h) * (int64_t)C * Q;
+  const float* dtb = dt + (b * nh + h) * (int64_t)C * Q;
+  const T* xg = x + b * sx.sb + h * sx.sh;
+  const T* Bg = B + b * sB.sb + (h / heads_per_group) * sB.sh + n0;
+  const int G = (L + KT - 1) / KT;
+
+  // element (p, n) of the state <-> accumulator i, component v of this lane
+  auto elem = [&](int i, int v) {
+    const int j = wave + 4 * i, mi = j % MB, ni = j / MB;
+    return (32 * mi + acc_row(v, lane)) * N + n0 + 32 * ni + (lane & 31);
+  };
+  // Every request is unconditional (a load inside a branch would have to complete before the next
+  // is issued): stages past the end are requested again as the last one and never used.
+  RowPieces<T, KT, P> px[D];
+  RowPieces<T, KT, NL> pb[D];
+  auto request = [&](RowPieces<T, KT, P>& rx, RowPieces<T, KT, NL>& rb, int g) {
+    const int row0 = min(g, G - 1) * KT;
+#ifndef SSD_WALK_XNT
+#define SSD_WALK_XNT true
+#endif
+    if (SSD_WALK_DIAG != 4) rx.template load<SSD_WALK_XNT>(xg, sx.sl, row0, L, tid);
+    if (SSD_WALK_DIAG != 5) rb.template load<false, true>(Bg, sB.sl, row0, L, tid, dAb, dtb);
+  };
+#pragma unroll
+  for (int u = 0; u < D; ++u) request(px[u], pb[u], u);
+
+  floatx16 acc[BPW], st[BPW];
+#pragma unroll
+  for (int i = 0; i < BPW; ++i) {
+    zero_acc(acc[i]);
+    zero_acc(st[i]);
+  }
+  if (initial) {
+    const float* ini = initial + (b * nh + h) * (int64_t)(P * N);
+#pragma unroll
+    for (int i = 0; i < BPW; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) st[i][v] = ini[elem(i, v)];
+  }
+  // the decay sum at the end of the chunk a stage belongs to, fetched one chunk ahead
+  float dal_next = dAb[Q - 1], dal = 0.f;
+
+  // one stage: rx / rb hold its rows and receive those of stage g + D
+  auto stage = [&](RowPieces<T, KT, P>& rx, RowPieces<T, KT, NL>& rb, int g) {
+    const int row0 = g * KT;
+    const int c = row0 / Q, k0 = row0 - c * Q;
+    if (k0 == 0) {
+      dal = dal_next;
+      dal_next = dAb[(int64_t)min(c + 1, C - 1) * Q + Q - 1];
+      TO* o = out + ((b * C + c) * nh + h) * (int64_t)(P * N);
+      if (SSD_WALK_DIAG != 1 || c == 0) {
+#pragma unroll
+        for (int i = 0; i < BPW; ++i)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) __builtin_nontemporal_store((TO)st[i][v], o + elem(i, v));
+      }
+    }
+    T* xb = lds + (g & 1) * S::kStageElems;
+    T* bb = xb + KT * PX;
+    const float dA_last = dal;
+    if (SSD_WALK_DIAG < 3) {
+      rx.store(xb, row0, L, tid, NoScale());
+      rb.store(bb, row0, L, tid, [&](int, float dA_k, float dt_k) { return __expf(fminf(dA_last - dA_k, 0.f)) * dt_k; });
+    } else {  // the rows must still arrive
+#pragma unroll
+      for (int i = 0; i < RowPieces<T, KT, P>::CNT; ++i)
+        if (SSD_WALK_DIAG != 4) acc[0][0] += rx.v[i].get(0);
+#pragma unroll
+      for (int i = 0; i < RowPieces<T, KT, NL>::CNT; ++i)
+        if (SSD_WALK_DIAG != 5) acc[0][1] += rb.v[i].get(0) + rb.a0[i] + rb.a1[i];
+    }
+    __syncthreads();
+    request(rx, rb, g + D);
+#pragma unroll
+    for (int kk = 0; kk < (SSD_WALK_DIAG >= 2 ? 0 : KT); kk += KG) {
+#pragma unroll
+      for (int i = 0; i < BPW; ++i) {
+        const int j = wave + 4 * i, mi = j % MB, ni = j / MB;
+        mma_group(frag_cols(xb, PX, kk, 32 * mi, lane), frag_cols(bb, PB, kk, 32 * ni, lane), acc[i]);
+      }
+    }
+    if (k0 + KT >= Q || g == G - 1) {  // the chunk ends with this stage
+      const float a = __expf(dA_last);
+#pragma unroll
+      for (int i = 0; i < BPW; ++i) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) st[i][v] = fmaf(a, st[i][v], acc[i][v]);
+        zero_acc(acc[i]);
+      }
+    }
+  };
+  // Whole rounds of D stages run without a test between the stages: every path through a round
+  // issues the same loads, so the waits for a stage's rows leave the rounds behind it in flight.
+  int g0 = 0;
+  for (; g0 + D <= G; g0 += D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) stage(px[u], pb[u], g0 + u);
+  }
+#pragma unroll
+  for (int u = 0; u < D - 1; ++u)
+    if (g0 + u < G) stage(px[u], pb[u], g0 + u);
+  float* f = final_states + (b * nh + h) * (int64_t)(P * N);
+#pragma unroll
+  for (int i = 0; i < BPW; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) f[elem(i, v)] = st[i][v];
 }
 
 // Sum over the 32 lanes of each half of a wave (lanes 0..31 and 32..63 apart), left in lanes 31
