@@ -696,6 +696,283 @@ __global__ __launch_bounds__(256, NSPLIT) void ssd_state_walk_kernel(
     for (int v = 0; v < 16; ++v) f[elem(i, v)] = st[i][v];
 }
 
+// ------------------------------------------------------------------------------------
+// The whole forward behind the cumsum in one pass: one workgroup (4 waves) per (b, h) walks the
+// sequence in stages of 64 rows and carries the (hdim x dstate) state in float32 registers, so
+// neither chunk-local states nor carried states nor C B^T go through memory.  Per stage, with
+// a_k the chunk's running sum of dA at position k, a_0 the sum before the stage and a_e at its
+// last row:
+//   out[m] = exp(a_m - a_0) * C_m . S  +  sum_{k <= m} (C_m . B_k) exp(min(a_m - a_k, 0)) dt_k x_k  +  D x_m
+//   S     <- exp(a_e - a_0) * S  +  sum_k exp(a_e - a_k) dt_k  x_k (x) B_k
+// which is the state-space recurrence itself, regrouped; the state entering each chunk of Q rows
+// is written out as the staged path writes it (Q a multiple of 64).  The operands of the products
+// are rounded to the input type where the staged kernels round them (carried state, weighted
+// C B^T), here per stage instead of per chunk, and the weight of the state update sits on x
+// instead of B: results agree with the staged path to rounding, not bit for bit.
+// Wave w owns output rows 32 * (w / 2) .. and hdim / 2 columns; it forms its own 32-row band of
+// C B^T (two waves form the same band, which is cheaper than handing it over) and turns it into an
+// MFMA operand through a private piece of LDS.  Two barriers per stage; the rows of the next D
+// stages are in flight in registers.  No packed batches.
+// ------------------------------------------------------------------------------------
+#ifndef SSD_FUSED_DIAG  // diagnostic builds (wrong results on purpose): 1 no C.S / C B^T products, 2 no band (weights, LDS), 3 no causal product, 4 no state update, 5 no output epilogue, 6 no loads past the first
+#define SSD_FUSED_DIAG 0
+#endif
+template <typename T, int P, int N>
+struct FusedSmem {
+  static constexpr int KT = 64, EPL = Vec16<T>::N;
+  static constexpr int PX = Tile<T>::pitch(P), PB = Tile<T>::pitch(N), PW = Tile<T>::pitch(32), PO = P + 4;
+  // the carried state is kept as St[n][p] and a wave's band of C B^T as W[k][m]: the accumulator
+  // layout gives a lane four consecutive rows of one column, which are adjacent that way
+  static constexpr int oXr = 0, oXw = oXr + KT * PX, oB = oXw + KT * PX, oC = oB + KT * PB, oS = oC + KT * PB,
+                       oW = oS + N * PX, kElems = oW + 4 * KT * PW;
+  static constexpr int kOutBytes = KT * PO * (int)sizeof(float);
+  static constexpr int kBytes = kElems * (int)sizeof(T) + kOutBytes + 2 * KT * (int)sizeof(float);
+};
+
+template <typename T, int P, int N, typename TS>
+__global__ __launch_bounds__(256) void ssd_fused_fwd_kernel(
+    const T* __restrict__ x, Strides3 sx, const T* __restrict__ B, Strides3 sB, const T* __restrict__ Cm, Strides3 sC,
+    const T* __restrict__ z, Strides3 sz, const float* __restrict__ dt, const float* __restrict__ dA_cs,
+    const float* __restrict__ Dv, int d_has_hdim, const float* __restrict__ initial, T* __restrict__ out, Strides3 so,
+    T* __restrict__ out_x, TS* __restrict__ states, float* __restrict__ final_states, int nh, int heads_per_group,
+    int L, int Q, int C) {
+  using S = FusedSmem<T, P, N>;
+  constexpr int KT = S::KT, EPL = S::EPL, KG = Tile<T>::KG, PX = S::PX, PB = S::PB, PW = S::PW, PO = S::PO;
+  constexpr int MB = P / 32, NB = N / 32, BPW = MB * NB / 4;  // state blocks per wave
+  constexpr int OB = P / 64;                                  // output column blocks per wave
+#ifdef SSD_FUSED_D
+  constexpr int D = SSD_FUSED_D;
+#else
+  constexpr int D = (P == 64 && N == 64) ? 2 : 1;  // stages in flight
+#endif
+  static_assert(MB * NB % 4 == 0 && P % 64 == 0, "blocks must split over 4 waves");
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T* lds = reinterpret_cast<T*>(smem);
+  T *Xr = lds + S::oXr, *Xw = lds + S::oXw, *Bt = lds + S::oB, *Ct = lds + S::oC, *St = lds + S::oS;
+  float* Os = reinterpret_cast<float*>(smem + S::kElems * sizeof(T));
+  float* dAs = Os + KT * PO;
+  float* dts = dAs + KT;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31;
+  T* Wr = lds + S::oW + wave * KT * PW;
+  const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
+  const int h = bid % nh;
+  const int64_t b = bid / nh;
+  const int g = h / heads_per_group;
+  const float* dAb = dA_cs + (b * nh + h) * (int64_t)C * Q;
+  const float* dtb = dt + (b * nh + h) * (int64_t)C * Q;
+  const T* xg = x + b * sx.sb + h * sx.sh;
+  const T* Bg = B + b * sB.sb + g * sB.sh;
+  const T* Cg = Cm + b * sC.sb + g * sC.sh;
+  const int G = (L + KT - 1) / KT;
+  const int mi = wave >> 1;            // 32-row band of the stage this wave writes
+  const int pc0 = (wave & 1) * OB;     // its first 32-column block
+
+  auto selem = [&](int i, int v) {  // element (p, n) of the state <-> state block i, component v
+    const int j = wave + 4 * i, bm = j % MB, bn = j / MB;
+    return (32 * bm + acc_row(v, lane)) * N + 32 * bn + l32;
+  };
+  // four consecutive components of an accumulator (rows r .. r + 3 of one column) as one piece
+  auto pack4 = [&](const floatx16& a, int q) {
+    float f[4] = {a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]};
+    ema::bf16x4 r;
+    if constexpr (std::is_same<T, bf16_t>::value) {
+      typedef float f32x2 __attribute__((ext_vector_type(2)));
+      typedef bf16_t b16x2 __attribute__((ext_vector_type(2)));
+      const b16x2 lo = __builtin_convertvector((f32x2){f[0], f[1]}, b16x2), hi = __builtin_convertvector((f32x2){f[2], f[3]}, b16x2);
+      r[0] = lo[0], r[1] = lo[1], r[2] = hi[0], r[3] = hi[1];
+    }
+    return r;
+  };
+
+  RowPieces<T, KT, P> px[D];
+  RowPieces<T, KT, N> pb[D], pc[D];
+  float dae[D];  // a_e of the stage in flight
+  auto request = [&](int u, int gq) {
+    const int row0 = min(gq, G - 1) * KT;
+    px[u].template load<true, true>(xg, sx.sl, row0, L, tid, dAb, dtb);
+    pb[u].load(Bg, sB.sl, row0, L, tid);
+    pc[u].load(Cg, sC.sl, row0, L, tid);
+    dae[u] = dAb[min(row0 + KT - 1, L - 1)];
+  };
+#pragma unroll
+  for (int u = 0; u < D; ++u) request(u, u);
+
+  floatx16 st[BPW];
+#pragma unroll
+  for (int i = 0; i < BPW; ++i) zero_acc(st[i]);
+  if (initial) {
+    const float* ini = initial + (b * nh + h) * (int64_t)(P * N);
+#pragma unroll
+    for (int i = 0; i < BPW; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) st[i][v] = ini[selem(i, v)];
+  }
+  float a0 = 0.f;  // a_0 of the stage: the running sum at the last row of the stage before, 0 at a chunk's start
+
+  auto stage = [&](int u, int gq) {
+    const int row0 = gq * KT;
+    const int c = row0 / Q, k0 = row0 - c * Q;
+    if (k0 == 0) {
+      a0 = 0.f;
+      TS* o = states + ((b * C + c) * nh + h) * (int64_t)(P * N);
+#pragma unroll
+      for (int i = 0; i < BPW; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) __builtin_nontemporal_store((TS)st[i][v], o + selem(i, v));
+    }
+    const float ae = dae[u];
+    // 1. the carried state, rounded, for the C . S product
+#pragma unroll
+    for (int i = 0; i < BPW; ++i) {
+      const int j = wave + 4 * i, bm = j % MB, bn = j / MB;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)  // rows p = 32 bm + 8 q + 4 (lane / 32) .. + 3 of column n = 32 bn + l32
+        *reinterpret_cast<ema::bf16x4*>(St + (32 * bn + l32) * PX + 32 * bm + 8 * q + 4 * (lane >> 5)) = pack4(st[i], q);
+    }
+    // 2. the stage's rows: x as it is and weighted for the state update, B, C, and a_k, dt_k
+    {
+      constexpr int VPR = RowPieces<T, KT, P>::VPR;
+#pragma unroll
+      for (int i = 0; i < RowPieces<T, KT, P>::CNT; ++i) {
+        const int idx = tid + 256 * i;
+        if (idx % VPR == 0) {
+          dAs[idx / VPR] = px[u].a0[i];
+          dts[idx / VPR] = px[u].a1[i];
+        }
+      }
+    }
+    px[u].store(Xr, row0, L, tid, NoScale());
+    px[u].store(Xw, row0, L, tid, [&](int, float a_k, float dt_k) { return __expf(fminf(ae - a_k, 0.f)) * dt_k; });
+    pb[u].store(Bt, row0, L, tid, NoScale());
+    pc[u].store(Ct, row0, L, tid, NoScale());
+    __syncthreads();
+    if (SSD_FUSED_DIAG != 6) request(u, gq + D);
+
+    // 3. this wave's band of C B^T, weighted and masked, as an operand
+    floatx16 acc[OB];
+#pragma unroll
+    for (int ob = 0; ob < OB; ++ob) zero_acc(acc[ob]);
+    float am[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) am[v] = dAs[32 * mi + acc_row(v, lane)];
+    // C . S and the band of C B^T share the fragments of C
+    floatx16 cb[2];
+    zero_acc(cb[0]);
+    zero_acc(cb[1]);
+#pragma unroll
+    for (int n0 = 0; n0 < (SSD_FUSED_DIAG == 1 ? 0 : N); n0 += KG) {
+      const Vec16<T> a = frag_rows(Ct, PB, 32 * mi, n0, lane);
+#pragma unroll
+      for (int ob = 0; ob < OB; ++ob) mma_group(a, frag_cols(St, PX, n0, 32 * (pc0 + ob), lane), acc[ob]);
+      mma_group(a, frag_rows(Bt, PB, 0, n0, lane), cb[0]);
+      if (mi) mma_group(a, frag_rows(Bt, PB, 32, n0, lane), cb[1]);
+    }
+#pragma unroll
+    for (int kb = 0; kb < (SSD_FUSED_DIAG == 2 ? 0 : 2); ++kb) {
+      if (kb > mi) break;
+      const int k = 32 * kb + l32;
+      const float ak = dAs[k], tk = dts[k];
+      float w[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = 32 * mi + acc_row(v, lane);
+        const float f = cb[kb][v] * __expf(fminf(am[v] - ak, 0.f)) * tk;
+        w[v] = k > m ? 0.f : f;
+      }
+      floatx16 wv;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) wv[v] = w[v];
+#pragma unroll
+      for (int q = 0; q < 4; ++q)  // rows m = 8 q + 4 (lane / 32) .. + 3 of the band, column k
+        *reinterpret_cast<ema::bf16x4*>(Wr + k * PW + 8 * q + 4 * (lane >> 5)) = pack4(wv, q);
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const float sc = __expf(fminf(am[v] - a0, 0.f));
+#pragma unroll
+      for (int ob = 0; ob < OB; ++ob) acc[ob][v] *= sc;
+    }
+    // the wave's own writes of its band are visible to its own reads once the LDS counter has drained
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    // 5. the causal product with x
+    for (int kk = 0; kk < (SSD_FUSED_DIAG == 3 ? 0 : 32 * (mi + 1)); kk += KG) {
+      const Vec16<T> a = frag_cols(Wr, PW, kk, 0, lane);
+#pragma unroll
+      for (int ob = 0; ob < OB; ++ob) mma_group(a, frag_cols(Xr, PX, kk, 32 * (pc0 + ob), lane), acc[ob]);
+    }
+    if (Dv) {
+#pragma unroll
+      for (int ob = 0; ob < OB; ++ob) {
+        const int col = 32 * (pc0 + ob) + l32;
+        const float dv = d_has_hdim ? Dv[h * P + col] : Dv[h];
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          acc[ob][v] = fmaf(dv, (float)Xr[(32 * mi + acc_row(v, lane)) * PX + col], acc[ob][v]);
+      }
+    }
+    // 6. the state after the stage
+    {
+      const float dec = __expf(fminf(ae - a0, 0.f));
+#pragma unroll
+      for (int i = 0; i < BPW; ++i) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) st[i][v] *= dec;
+        const int j = wave + 4 * i, bm = j % MB, bn = j / MB;
+#pragma unroll
+        for (int kk = 0; kk < (SSD_FUSED_DIAG == 4 ? 0 : KT); kk += KG)
+          mma_group(frag_cols(Xw, PX, kk, 32 * bm, lane), frag_cols(Bt, PB, kk, 32 * bn, lane), st[i]);
+      }
+    }
+    a0 = ae;
+    // 7. the stage's output rows through LDS, so that they leave in 16-byte pieces
+#pragma unroll
+    for (int ob = 0; ob < OB; ++ob)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) Os[(32 * mi + acc_row(v, lane)) * PO + 32 * (pc0 + ob) + l32] = acc[ob][v];
+    __syncthreads();
+    constexpr int VPR = P / EPL;
+#pragma unroll
+    for (int i = 0; i < (SSD_FUSED_DIAG == 5 ? 0 : KT * VPR / 256); ++i) {
+      const int idx = tid + 256 * i;
+      const int r = idx / VPR, cv = (idx % VPR) * EPL;
+      const int64_t pos = (int64_t)row0 + r;
+      if (pos < L) {
+        float vv[EPL];
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) vv[e] = Os[r * PO + cv + e];
+        Vec16<T> o;
+        if (z) {
+          if (out_x) {
+            o.set_all(vv);
+            store16(out_x + b * so.sb + pos * so.sl + h * so.sh + cv, o);
+          }
+          const Vec16<T> zv = load16(z + b * sz.sb + pos * sz.sl + h * sz.sh + cv);
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) {
+            const float zf = zv.get(e);
+            vv[e] *= zf / (1.f + __expf(-zf));
+          }
+        }
+        o.set_all(vv);
+        store16_stream(out + b * so.sb + pos * so.sl + h * so.sh + cv, o);
+      }
+    }
+  };
+  int g0 = 0;
+  for (; g0 + D <= G; g0 += D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) stage(u, g0 + u);
+  }
+#pragma unroll
+  for (int u = 0; u < D - 1; ++u)
+    if (g0 + u < G) stage(u, g0 + u);
+  float* f = final_states + (b * nh + h) * (int64_t)(P * N);
+#pragma unroll
+  for (int i = 0; i < BPW; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) f[selem(i, v)] = st[i][v];
+}
+
 // Sum over the 32 lanes of each half of a wave (lanes 0..31 and 32..63 apart), left in lanes 31
 // and 63: the DPP prefix steps of wave_inclusive_scan without the last one.
 __device__ __forceinline__ float half_wave_sum(float v) {

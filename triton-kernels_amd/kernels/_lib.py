@@ -58,6 +58,7 @@ _SIGNATURES = {
     "ssd_chunk_state_fwd": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
     "ssd_state_passing_fwd": (c_int, [_P, _P, _I, _I, _I, _P, _P, c_int, _P, _I, _I, _I, _I] + _IDS + [_I, _I, _P]),
     "ssd_chunk_state_passing_fwd": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, _P, c_int, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "ssd_fused_fwd": (c_int, _SEQ + _SEQ + _SEQ + _SEQ + [c_int, _P, _P, _P, c_int, _P] + _SEQ + [_P, _P, c_int, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "ssd_bmm_chunk_fwd": (c_int, _SEQ + _SEQ + [c_int, _P, c_int, _I, _I, _I, _I, _I] + _IDS + [_P]),
     "ssd_chunk_scan_fwd": (c_int, [_P] + _SEQ + _SEQ + [c_int, _P, _P] + _SEQ + [_P, c_int, _P, c_int] + _SEQ + [_P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
     # SSD backward stages
