@@ -726,7 +726,7 @@ struct FusedSmem {
   static constexpr int oXr = 0, oXw = oXr + KT * PX, oB = oXw + KT * PX, oC = oB + KT * PB, oS = oC + KT * PB,
                        oW = oS + N * PX, kElems = oW + 4 * KT * PW;
   static constexpr int kOutBytes = KT * PO * (int)sizeof(float);
-  static constexpr int kBytes = kElems * (int)sizeof(T) + kOutBytes + 2 * KT * (int)sizeof(float);
+  static constexpr int kBytes = kElems * (int)sizeof(T) + kOutBytes + 4 * KT * (int)sizeof(float);
 };
 
 template <typename T, int P, int N, typename TS>
@@ -752,6 +752,8 @@ __global__ __launch_bounds__(256) void ssd_fused_fwd_kernel(
   float* Os = reinterpret_cast<float*>(smem + S::kElems * sizeof(T));
   float* dAs = Os + KT * PO;
   float* dts = dAs + KT;
+  float* sms = dts + KT;  // exp(a_m - a_0): the scale of row m's C . S
+  float* fgs = sms + KT;  // rows 0..31: exp(a_31 - a_k) dt_k; rows 32..63: exp(a_m - a_31)
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31;
   T* Wr = lds + S::oW + wave * KT * PW;
   const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
@@ -786,13 +788,14 @@ __global__ __launch_bounds__(256) void ssd_fused_fwd_kernel(
 
   RowPieces<T, KT, P> px[D];
   RowPieces<T, KT, N> pb[D], pc[D];
-  float dae[D];  // a_e of the stage in flight
+  float dae[D], dam[D];  // a_e and a_31 of the stage in flight
   auto request = [&](int u, int gq) {
     const int row0 = min(gq, G - 1) * KT;
     px[u].template load<true, true>(xg, sx.sl, row0, L, tid, dAb, dtb);
     pb[u].load(Bg, sB.sl, row0, L, tid);
     pc[u].load(Cg, sC.sl, row0, L, tid);
     dae[u] = dAb[min(row0 + KT - 1, L - 1)];
+    dam[u] = dAb[min(row0 + 31, L - 1)];
   };
 #pragma unroll
   for (int u = 0; u < D; ++u) request(u, u);
@@ -807,6 +810,19 @@ __global__ __launch_bounds__(256) void ssd_fused_fwd_kernel(
 #pragma unroll
       for (int v = 0; v < 16; ++v) st[i][v] = ini[selem(i, v)];
   }
+#ifdef SSD_TIMING
+  long long tacc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, tlast = clock64();
+#define SSD_FPHASE(i)                 \
+  do {                                \
+    const long long now = clock64();  \
+    tacc[i] += now - tlast;           \
+    tlast = now;                      \
+  } while (0)
+#else
+#define SSD_FPHASE(i) \
+  do {                \
+  } while (0)
+#endif
   float a0 = 0.f;  // a_0 of the stage: the running sum at the last row of the stage before, 0 at a chunk's start
 
   auto stage = [&](int u, int gq) {
@@ -820,6 +836,7 @@ __global__ __launch_bounds__(256) void ssd_fused_fwd_kernel(
 #pragma unroll
         for (int v = 0; v < 16; ++v) __builtin_nontemporal_store((TS)st[i][v], o + selem(i, v));
     }
+    SSD_FPHASE(7);
     const float ae = dae[u];
     // 1. the carried state, rounded, for the C . S product
 #pragma unroll
@@ -836,8 +853,15 @@ __global__ __launch_bounds__(256) void ssd_fused_fwd_kernel(
       for (int i = 0; i < RowPieces<T, KT, P>::CNT; ++i) {
         const int idx = tid + 256 * i;
         if (idx % VPR == 0) {
-          dAs[idx / VPR] = px[u].a0[i];
-          dts[idx / VPR] = px[u].a1[i];
+          // Below the diagonal block the weight of (m, k) splits at row 31, the last of k's block:
+          // exp(a_m - a_31) per row times exp(a_31 - a_k) dt_k per column, both exponents <= 0
+          // for sums that fall along the chunk (each is clamped like the whole is).
+          const int r = idx / VPR;
+          const float ar = px[u].a0[i], tr = px[u].a1[i];
+          dAs[r] = ar;
+          dts[r] = tr;
+          sms[r] = __expf(fminf(ar - a0, 0.f));
+          fgs[r] = r < 32 ? __expf(fminf(dam[u] - ar, 0.f)) * tr : __expf(fminf(ar - dam[u], 0.f));
         }
       }
     }
@@ -845,16 +869,15 @@ __global__ __launch_bounds__(256) void ssd_fused_fwd_kernel(
     px[u].store(Xw, row0, L, tid, [&](int, float a_k, float dt_k) { return __expf(fminf(ae - a_k, 0.f)) * dt_k; });
     pb[u].store(Bt, row0, L, tid, NoScale());
     pc[u].store(Ct, row0, L, tid, NoScale());
+    SSD_FPHASE(0);
     __syncthreads();
+    SSD_FPHASE(1);
     if (SSD_FUSED_DIAG != 6) request(u, gq + D);
 
     // 3. this wave's band of C B^T, weighted and masked, as an operand
     floatx16 acc[OB];
 #pragma unroll
     for (int ob = 0; ob < OB; ++ob) zero_acc(acc[ob]);
-    float am[16];
-#pragma unroll
-    for (int v = 0; v < 16; ++v) am[v] = dAs[32 * mi + acc_row(v, lane)];
     // C . S and the band of C B^T share the fragments of C
     floatx16 cb[2];
     zero_acc(cb[0]);
@@ -867,33 +890,39 @@ __global__ __launch_bounds__(256) void ssd_fused_fwd_kernel(
       mma_group(a, frag_rows(Bt, PB, 0, n0, lane), cb[0]);
       if (mi) mma_group(a, frag_rows(Bt, PB, 32, n0, lane), cb[1]);
     }
+    if (SSD_FUSED_DIAG != 2) {
+      if (mi) {  // the block below the diagonal one: a factor per row times a factor per column
+        const float gk = fgs[l32];
 #pragma unroll
-    for (int kb = 0; kb < (SSD_FUSED_DIAG == 2 ? 0 : 2); ++kb) {
-      if (kb > mi) break;
-      const int k = 32 * kb + l32;
-      const float ak = dAs[k], tk = dts[k];
-      float w[16];
+        for (int v = 0; v < 16; ++v) cb[0][v] *= fgs[32 + acc_row(v, lane)] * gk;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = 32 * mi + acc_row(v, lane);
-        const float f = cb[kb][v] * __expf(fminf(am[v] - ak, 0.f)) * tk;
-        w[v] = k > m ? 0.f : f;
+        for (int q = 0; q < 4; ++q)
+          *reinterpret_cast<ema::bf16x4*>(Wr + l32 * PW + 8 * q + 4 * (lane >> 5)) = pack4(cb[0], q);
       }
-      floatx16 wv;
+      {  // the diagonal block: the exact weight, masked
+        floatx16& cd = cb[mi ? 1 : 0];
+        const int k = 32 * mi + l32;
+        const float ak = dAs[k], tk = dts[k];
 #pragma unroll
-      for (int v = 0; v < 16; ++v) wv[v] = w[v];
+        for (int v = 0; v < 16; ++v) {
+          const int m = 32 * mi + acc_row(v, lane);
+          const float f = cd[v] * __expf(fminf(dAs[m] - ak, 0.f)) * tk;
+          cd[v] = k > m ? 0.f : f;
+        }
 #pragma unroll
-      for (int q = 0; q < 4; ++q)  // rows m = 8 q + 4 (lane / 32) .. + 3 of the band, column k
-        *reinterpret_cast<ema::bf16x4*>(Wr + k * PW + 8 * q + 4 * (lane >> 5)) = pack4(wv, q);
+        for (int q = 0; q < 4; ++q)  // rows m = 8 q + 4 (lane / 32) .. + 3 of the band, column k
+          *reinterpret_cast<ema::bf16x4*>(Wr + k * PW + 8 * q + 4 * (lane >> 5)) = pack4(cd, q);
+      }
     }
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      const float sc = __expf(fminf(am[v] - a0, 0.f));
+      const float sc = sms[32 * mi + acc_row(v, lane)];
 #pragma unroll
       for (int ob = 0; ob < OB; ++ob) acc[ob][v] *= sc;
     }
     // the wave's own writes of its band are visible to its own reads once the LDS counter has drained
     __builtin_amdgcn_s_waitcnt(0xc07f);
+    SSD_FPHASE(2);
     // 5. the causal product with x
     for (int kk = 0; kk < (SSD_FUSED_DIAG == 3 ? 0 : 32 * (mi + 1)); kk += KG) {
       const Vec16<T> a = frag_cols(Wr, PW, kk, 0, lane);
@@ -910,6 +939,7 @@ __global__ __launch_bounds__(256) void ssd_fused_fwd_kernel(
           acc[ob][v] = fmaf(dv, (float)Xr[(32 * mi + acc_row(v, lane)) * PX + col], acc[ob][v]);
       }
     }
+    SSD_FPHASE(3);
     // 6. the state after the stage
     {
       const float dec = __expf(fminf(ae - a0, 0.f));
@@ -924,12 +954,14 @@ __global__ __launch_bounds__(256) void ssd_fused_fwd_kernel(
       }
     }
     a0 = ae;
+    SSD_FPHASE(4);
     // 7. the stage's output rows through LDS, so that they leave in 16-byte pieces
 #pragma unroll
     for (int ob = 0; ob < OB; ++ob)
 #pragma unroll
       for (int v = 0; v < 16; ++v) Os[(32 * mi + acc_row(v, lane)) * PO + 32 * (pc0 + ob) + l32] = acc[ob][v];
     __syncthreads();
+    SSD_FPHASE(5);
     constexpr int VPR = P / EPL;
 #pragma unroll
     for (int i = 0; i < (SSD_FUSED_DIAG == 5 ? 0 : KT * VPR / 256); ++i) {
@@ -971,6 +1003,11 @@ __global__ __launch_bounds__(256) void ssd_fused_fwd_kernel(
   for (int i = 0; i < BPW; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) f[selem(i, v)] = st[i][v];
+#ifdef SSD_TIMING
+  SSD_FPHASE(6);
+  if ((tid & 63) == 0 && g_ssd_timing)
+    for (int i = 0; i < 8; ++i) g_ssd_timing[((int64_t)blockIdx.x * 4 + wave) * 8 + i] = tacc[i];
+#endif
 }
 
 // Sum over the 32 lanes of each half of a wave (lanes 0..31 and 32..63 apart), left in lanes 31
