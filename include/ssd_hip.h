@@ -111,8 +111,8 @@ int ssd_chunk_state_passing_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64
  * state entering each chunk, final_states (batch, nheads, hdim, dstate) float32 the last one.  The
  * operands of the products are rounded to the input type where the staged entry points round them,
  * per 64-row stage instead of per chunk: results agree with the staged path to rounding, not bit for
- * bit.  bfloat16 inputs, chunk a multiple of 64, no packed batches (SSD_ERR_UNSUPPORTED otherwise:
- * run the staged entry points).
+ * bit.  bfloat16 inputs, hdim 64, dstate 64 or 128, chunk a multiple of 64, no packed batches
+ * (SSD_ERR_UNSUPPORTED otherwise: run the staged entry points).
  * Replaces, run back to back, _chunk_state_fwd (kernels/mamba_kernels/mamba_state_fwd.py:138-169),
  * _state_passing_fwd (mamba_state_pass.py:84-115), _bmm_chunk_fwd (mamba_bmm.py:80) and
  * _chunk_scan_fwd (mamba_scan_fwd.py:162); the reference's own single-kernel forward is

@@ -298,8 +298,8 @@ FUSED_CASES = [
     (2, 300, 4, 64, 1, 64, 64),     # last chunk and last stage ragged
     (1, 256, 2, 64, 2, 128, 128),
     (2, 200, 4, 64, 1, 128, 256),   # a single ragged chunk
-    (1, 520, 2, 128, 1, 64, 128),
-    (1, 130, 2, 128, 2, 128, 64),
+    (1, 520, 3, 64, 1, 64, 128),
+    (1, 130, 2, 64, 2, 128, 64),
     (1, 900, 3, 64, 1, 64, 512),
     (1, 1100, 2, 64, 1, 128, 1024),
     (3, 64, 2, 64, 1, 128, 64),     # one stage in all
@@ -368,6 +368,8 @@ def test_forward_in_one_kernel_limits(device):
     assert _fused_fwd(xd, dto, dA, Bd, Cd, 64) is None  # float32 inputs
     dA48, dt48 = _chunk_cumsum_fwd(dtd, Ad, 48)
     assert _fused_fwd(xd.to(BF16), dt48, dA48, Bd.to(BF16), Cd.to(BF16), 48) is None  # chunk no multiple of 64
+    wide = torch.zeros(b, L, nh, 128, device=device, dtype=BF16)
+    assert _fused_fwd(wide, dto, dA, Bd.to(BF16), Cd.to(BF16), 64) is None  # head size 128
 
 
 def test_unsupported_shapes_are_refused(device):

@@ -697,11 +697,11 @@ __global__ __launch_bounds__(256, NSPLIT) void ssd_state_walk_kernel(
 }
 
 // ------------------------------------------------------------------------------------
-// The whole forward behind the cumsum in one pass: one workgroup (4 waves) per (b, h) walks the
-// sequence in stages of 64 rows and carries the (hdim x dstate) state in float32 registers, so
-// neither chunk-local states nor carried states nor C B^T go through memory.  Per stage, with
-// a_k the chunk's running sum of dA at position k, a_0 the sum before the stage and a_e at its
-// last row:
+// The whole forward behind the cumsum in one pass (hdim 64): one workgroup of 8 waves per (b, h)
+// walks the sequence in stages of 64 rows and carries the (64 x dstate) state in float32
+// registers, so neither chunk-local states nor carried states nor C B^T go through memory.  Per
+// stage, with a_k the chunk's running sum of dA at position k, a_0 the sum before the stage and a_e
+// at its last row:
 //   out[m] = exp(a_m - a_0) * C_m . S  +  sum_{k <= m} (C_m . B_k) exp(min(a_m - a_k, 0)) dt_k x_k  +  D x_m
 //   S     <- exp(a_e - a_0) * S  +  sum_k exp(a_e - a_k) dt_k  x_k (x) B_k
 // which is the state-space recurrence itself, regrouped; the state entering each chunk of Q rows
@@ -709,48 +709,91 @@ __global__ __launch_bounds__(256, NSPLIT) void ssd_state_walk_kernel(
 // are rounded to the input type where the staged kernels round them (carried state, weighted
 // C B^T), here per stage instead of per chunk, and the weight of the state update sits on x
 // instead of B: results agree with the staged path to rounding, not bit for bit.
-// Wave w owns output rows 32 * (w / 2) .. and hdim / 2 columns; it forms its own 32-row band of
-// C B^T (two waves form the same band, which is cheaper than handing it over) and turns it into an
-// MFMA operand through a private piece of LDS.  Two barriers per stage; the rows of the next D
-// stages are in flight in registers.  No packed batches.
+//
+// Work of a stage over the waves: the 64 x 64 output is four 32 x 32 blocks; two waves share a
+// block and split the state dimension between them (each forms C . S and its 32-row band of
+// C B^T over half of dstate, weights its partial band, multiplies it with x; the two partial
+// outputs meet in the output pass).  The state's 32 x 32 blocks go one to a wave.  The two waves
+// that a SIMD holds work on the upper and the lower band, whose causal work differs by half.
+// Two barriers per stage; the rows of the next D stages are in flight in registers.
+// No packed batches.
 // ------------------------------------------------------------------------------------
-#ifndef SSD_FUSED_DIAG  // diagnostic builds (wrong results on purpose): 1 no C.S / C B^T products, 2 no band (weights, LDS), 3 no causal product, 4 no state update, 5 no output epilogue, 6 no loads past the first
+#ifndef SSD_FUSED_DIAG  // diagnostic builds (wrong results on purpose): 1 no C.S / C B^T products, 2 no band, 3 no causal product, 4 no state update, 5 no output pass, 6 no loads past the first
 #define SSD_FUSED_DIAG 0
 #endif
-template <typename T, int P, int N>
+template <typename T, int N>
 struct FusedSmem {
-  static constexpr int KT = 64, EPL = Vec16<T>::N;
+  static constexpr int P = 64, KT = 64, NT = 512, EPL = Vec16<T>::N;
   static constexpr int PX = Tile<T>::pitch(P), PB = Tile<T>::pitch(N), PW = Tile<T>::pitch(32), PO = P + 4;
   // the carried state is kept as St[n][p] and a wave's band of C B^T as W[k][m]: the accumulator
   // layout gives a lane four consecutive rows of one column, which are adjacent that way
   static constexpr int oXr = 0, oXw = oXr + KT * PX, oB = oXw + KT * PX, oC = oB + KT * PB, oS = oC + KT * PB,
-                       oW = oS + N * PX, kElems = oW + 4 * KT * PW;
-  static constexpr int kOutBytes = KT * PO * (int)sizeof(float);
+                       oW = oS + N * PX, kElems = oW + 8 * KT * PW;
+  static constexpr int kOutBytes = 2 * KT * PO * (int)sizeof(float);
   static constexpr int kBytes = kElems * (int)sizeof(T) + kOutBytes + 4 * KT * (int)sizeof(float);
 };
 
-template <typename T, int P, int N, typename TS>
-__global__ __launch_bounds__(256) void ssd_fused_fwd_kernel(
+// The rows of a 64-row stage as 16-byte pieces over NT threads (RowPieces for another thread count).
+template <typename T, int COLS, int NT>
+struct StagePieces {
+  static constexpr int EPL = Vec16<T>::N, VPR = COLS / EPL, CNT = 64 * VPR / NT;
+  static_assert((64 * VPR) % NT == 0, "tile must split evenly over the threads");
+  Vec16<T> v[CNT];
+  template <bool STREAM>
+  __device__ __forceinline__ void load(const T* __restrict__ g, int64_t row_stride, int row0, int limit, int tid) {
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) {
+      const int idx = tid + NT * i;
+      const int row = min(row0 + idx / VPR, limit - 1);
+      const T* src = g + (int64_t)row * row_stride + (idx % VPR) * EPL;
+      v[i] = STREAM ? load16_stream(src) : load16(src);
+    }
+  }
+  // rows at or past limit are stored as zeros; scale(r) multiplies row r of the stage
+  template <typename F>
+  __device__ __forceinline__ void store(T* tile, int row0, int limit, int tid, F scale) const {
+    constexpr int PT = Tile<T>::pitch(COLS);
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) {
+      const int idx = tid + NT * i;
+      const int r = idx / VPR, cv = (idx % VPR) * EPL;
+      Vec16<T> w = v[i];
+      if constexpr (!std::is_same<F, NoScale>::value) {
+        const float sc = scale(r);
+        float t[EPL];
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) t[e] = w.get(e) * sc;
+        w.set_all(t);
+      }
+      if (row0 + r >= limit) w.zero();
+      store16(tile + r * PT + cv, w);
+    }
+  }
+};
+
+template <typename T, int N, typename TS, bool HAS_Z>
+__global__ __launch_bounds__(512) void ssd_fused_fwd_kernel(
     const T* __restrict__ x, Strides3 sx, const T* __restrict__ B, Strides3 sB, const T* __restrict__ Cm, Strides3 sC,
     const T* __restrict__ z, Strides3 sz, const float* __restrict__ dt, const float* __restrict__ dA_cs,
     const float* __restrict__ Dv, int d_has_hdim, const float* __restrict__ initial, T* __restrict__ out, Strides3 so,
     T* __restrict__ out_x, TS* __restrict__ states, float* __restrict__ final_states, int nh, int heads_per_group,
     int L, int Q, int C) {
-  using S = FusedSmem<T, P, N>;
-  constexpr int KT = S::KT, EPL = S::EPL, KG = Tile<T>::KG, PX = S::PX, PB = S::PB, PW = S::PW, PO = S::PO;
-  constexpr int MB = P / 32, NB = N / 32, BPW = MB * NB / 4;  // state blocks per wave
-  constexpr int OB = P / 64;                                  // output column blocks per wave
+  using S = FusedSmem<T, N>;
+  constexpr int P = S::P, KT = S::KT, NT = S::NT, EPL = S::EPL, KG = Tile<T>::KG;
+  constexpr int PX = S::PX, PB = S::PB, PW = S::PW, PO = S::PO;
+  constexpr int MB = P / 32, NBLK = N / 32;  // state blocks: MB x NBLK, one per wave (the first MB * NBLK waves)
+  constexpr int NH = N / 2;                 // the half of dstate a wave contracts over
 #ifdef SSD_FUSED_D
   constexpr int D = SSD_FUSED_D;
 #else
-  constexpr int D = (P == 64 && N == 64) ? 2 : 1;  // stages in flight
+  constexpr int D = 1;  // stages in flight (two spill)
 #endif
-  static_assert(MB * NB % 4 == 0 && P % 64 == 0, "blocks must split over 4 waves");
+  static_assert(MB * NBLK <= 8 && NH % KG == 0, "one state block per wave");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* lds = reinterpret_cast<T*>(smem);
   T *Xr = lds + S::oXr, *Xw = lds + S::oXw, *Bt = lds + S::oB, *Ct = lds + S::oC, *St = lds + S::oS;
-  float* Os = reinterpret_cast<float*>(smem + S::kElems * sizeof(T));
-  float* dAs = Os + KT * PO;
+  float* Os = reinterpret_cast<float*>(smem + S::kElems * sizeof(T));  // [2][KT][PO]: one partial output per half
+  float* dAs = Os + 2 * KT * PO;
   float* dts = dAs + KT;
   float* sms = dts + KT;  // exp(a_m - a_0): the scale of row m's C . S
   float* fgs = sms + KT;  // rows 0..31: exp(a_31 - a_k) dt_k; rows 32..63: exp(a_m - a_31)
@@ -765,131 +808,116 @@ __global__ __launch_bounds__(256) void ssd_fused_fwd_kernel(
   const T* xg = x + b * sx.sb + h * sx.sh;
   const T* Bg = B + b * sB.sb + g * sB.sh;
   const T* Cg = Cm + b * sC.sb + g * sC.sh;
+  const T* zg = HAS_Z ? z + b * sz.sb + h * sz.sh : nullptr;
   const int G = (L + KT - 1) / KT;
-  const int mi = wave >> 1;            // 32-row band of the stage this wave writes
-  const int pc0 = (wave & 1) * OB;     // its first 32-column block
+  const int mi = wave >> 2;        // 32-row band of the stage this wave works on
+  const int pcb = (wave >> 1) & 1; // its 32-column block of the output
+  const int half = wave & 1;       // its half of dstate
+  const bool owns = wave < MB * NBLK;  // this wave keeps a block of the state:
+  const int bm = wave % MB, bn = wave / MB;  // rows 32 bm .. of p, columns 32 bn .. of n
 
-  auto selem = [&](int i, int v) {  // element (p, n) of the state <-> state block i, component v
-    const int j = wave + 4 * i, bm = j % MB, bn = j / MB;
-    return (32 * bm + acc_row(v, lane)) * N + 32 * bn + l32;
-  };
+  auto selem = [&](int v) { return (32 * bm + acc_row(v, lane)) * N + 32 * bn + l32; };
   // four consecutive components of an accumulator (rows r .. r + 3 of one column) as one piece
   auto pack4 = [&](const floatx16& a, int q) {
-    float f[4] = {a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]};
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef bf16_t b16x2 __attribute__((ext_vector_type(2)));
+    const b16x2 lo = __builtin_convertvector((f32x2){a[4 * q], a[4 * q + 1]}, b16x2);
+    const b16x2 hi = __builtin_convertvector((f32x2){a[4 * q + 2], a[4 * q + 3]}, b16x2);
     ema::bf16x4 r;
-    if constexpr (std::is_same<T, bf16_t>::value) {
-      typedef float f32x2 __attribute__((ext_vector_type(2)));
-      typedef bf16_t b16x2 __attribute__((ext_vector_type(2)));
-      const b16x2 lo = __builtin_convertvector((f32x2){f[0], f[1]}, b16x2), hi = __builtin_convertvector((f32x2){f[2], f[3]}, b16x2);
-      r[0] = lo[0], r[1] = lo[1], r[2] = hi[0], r[3] = hi[1];
-    }
+    r[0] = lo[0], r[1] = lo[1], r[2] = hi[0], r[3] = hi[1];
     return r;
   };
 
-  RowPieces<T, KT, P> px[D];
-  RowPieces<T, KT, N> pb[D], pc[D];
-  float dae[D], dam[D];  // a_e and a_31 of the stage in flight
+  // Every request is unconditional (a load inside a branch would have to complete before the next
+  // is issued): stages past the end are requested again as the last one and never used.
+  StagePieces<T, P, NT> px[D], pz[HAS_Z ? D : 1];
+  StagePieces<T, N, NT> pb[D], pc[D];
+  float pa[D], pt[D], dae[D], dam[D];  // a_k and dt_k of this thread's row; a_e and a_31 of the stage
+  const int vrow = tid >> 3;  // the row whose a_k, dt_k this thread brings (threads 8 r .. 8 r + 7 the same)
   auto request = [&](int u, int gq) {
     const int row0 = min(gq, G - 1) * KT;
-    px[u].template load<true, true>(xg, sx.sl, row0, L, tid, dAb, dtb);
-    pb[u].load(Bg, sB.sl, row0, L, tid);
-    pc[u].load(Cg, sC.sl, row0, L, tid);
+    px[u].template load<true>(xg, sx.sl, row0, L, tid);
+    pb[u].template load<false>(Bg, sB.sl, row0, L, tid);
+    pc[u].template load<false>(Cg, sC.sl, row0, L, tid);
+    if constexpr (HAS_Z) pz[u].template load<true>(zg, sz.sl, row0, L, tid);
+    const int r = min(row0 + vrow, L - 1);
+    pa[u] = dAb[r];
+    pt[u] = dtb[r];
     dae[u] = dAb[min(row0 + KT - 1, L - 1)];
     dam[u] = dAb[min(row0 + 31, L - 1)];
   };
 #pragma unroll
   for (int u = 0; u < D; ++u) request(u, u);
 
-  floatx16 st[BPW];
-#pragma unroll
-  for (int i = 0; i < BPW; ++i) zero_acc(st[i]);
-  if (initial) {
+  floatx16 st;
+  zero_acc(st);
+  if (initial && owns) {
     const float* ini = initial + (b * nh + h) * (int64_t)(P * N);
 #pragma unroll
-    for (int i = 0; i < BPW; ++i)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) st[i][v] = ini[selem(i, v)];
+    for (int v = 0; v < 16; ++v) st[v] = ini[selem(v)];
   }
-#ifdef SSD_TIMING
-  long long tacc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, tlast = clock64();
-#define SSD_FPHASE(i)                 \
-  do {                                \
-    const long long now = clock64();  \
-    tacc[i] += now - tlast;           \
-    tlast = now;                      \
-  } while (0)
-#else
-#define SSD_FPHASE(i) \
-  do {                \
-  } while (0)
-#endif
   float a0 = 0.f;  // a_0 of the stage: the running sum at the last row of the stage before, 0 at a chunk's start
 
-  auto stage = [&](int u, int gq) {
+  // FULL: every row of the stage lies inside the sequence, so that its stores are unconditional
+  // and the waits for rows requested before them can count them.  (Loads and stores of a wave
+  // complete in order; a store the compiler cannot count makes every later wait for a load wait
+  // for the store as well.)
+  auto stage = [&](int u, int gq, auto full_tag) {
+    constexpr bool FULL = decltype(full_tag)::value;
     const int row0 = gq * KT;
     const int c = row0 / Q, k0 = row0 - c * Q;
-    if (k0 == 0) {
-      a0 = 0.f;
-      TS* o = states + ((b * C + c) * nh + h) * (int64_t)(P * N);
-#pragma unroll
-      for (int i = 0; i < BPW; ++i)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) __builtin_nontemporal_store((TS)st[i][v], o + selem(i, v));
-    }
-    SSD_FPHASE(7);
-    const float ae = dae[u];
+    if (k0 == 0) a0 = 0.f;
+    const float ae = dae[u], a31 = dam[u];
     // 1. the carried state, rounded, for the C . S product
-#pragma unroll
-    for (int i = 0; i < BPW; ++i) {
-      const int j = wave + 4 * i, bm = j % MB, bn = j / MB;
+    if (owns) {
 #pragma unroll
       for (int q = 0; q < 4; ++q)  // rows p = 32 bm + 8 q + 4 (lane / 32) .. + 3 of column n = 32 bn + l32
-        *reinterpret_cast<ema::bf16x4*>(St + (32 * bn + l32) * PX + 32 * bm + 8 * q + 4 * (lane >> 5)) = pack4(st[i], q);
+        *reinterpret_cast<ema::bf16x4*>(St + (32 * bn + l32) * PX + 32 * bm + 8 * q + 4 * (lane >> 5)) = pack4(st, q);
     }
-    // 2. the stage's rows: x as it is and weighted for the state update, B, C, and a_k, dt_k
-    {
-      constexpr int VPR = RowPieces<T, KT, P>::VPR;
-#pragma unroll
-      for (int i = 0; i < RowPieces<T, KT, P>::CNT; ++i) {
-        const int idx = tid + 256 * i;
-        if (idx % VPR == 0) {
-          // Below the diagonal block the weight of (m, k) splits at row 31, the last of k's block:
-          // exp(a_m - a_31) per row times exp(a_31 - a_k) dt_k per column, both exponents <= 0
-          // for sums that fall along the chunk (each is clamped like the whole is).
-          const int r = idx / VPR;
-          const float ar = px[u].a0[i], tr = px[u].a1[i];
-          dAs[r] = ar;
-          dts[r] = tr;
-          sms[r] = __expf(fminf(ar - a0, 0.f));
-          fgs[r] = r < 32 ? __expf(fminf(dam[u] - ar, 0.f)) * tr : __expf(fminf(ar - dam[u], 0.f));
-        }
-      }
+    // 2. the stage's rows: x as it is and weighted for the state update, B, C, and the vectors of the weights
+    if ((tid & 7) == 0) {
+      // Below the diagonal block the weight of (m, k) splits at row 31, the last of k's block:
+      // exp(a_m - a_31) per row times exp(a_31 - a_k) dt_k per column, both exponents <= 0 for
+      // sums that fall along the chunk (each is clamped like the whole is).
+      const float ar = pa[u], tr = pt[u];
+      dAs[vrow] = ar;
+      dts[vrow] = tr;
+      sms[vrow] = __expf(fminf(ar - a0, 0.f));
+      fgs[vrow] = vrow < 32 ? __expf(fminf(a31 - ar, 0.f)) * tr : __expf(fminf(ar - a31, 0.f));
     }
     px[u].store(Xr, row0, L, tid, NoScale());
-    px[u].store(Xw, row0, L, tid, [&](int, float a_k, float dt_k) { return __expf(fminf(ae - a_k, 0.f)) * dt_k; });
+    {
+      // x has 8 pieces to a row: the rows of this thread's pieces are vrow (NT / 8 = 64 rows, one piece each)
+      static_assert(StagePieces<T, P, NT>::CNT == 1 && StagePieces<T, P, NT>::VPR == 8, "one piece of x per thread");
+      const float wx = __expf(fminf(ae - pa[u], 0.f)) * pt[u];
+      px[u].store(Xw, row0, L, tid, [&](int) { return wx; });
+    }
     pb[u].store(Bt, row0, L, tid, NoScale());
     pc[u].store(Ct, row0, L, tid, NoScale());
-    SSD_FPHASE(0);
+    Vec16<T> zrow;
+    if constexpr (HAS_Z) zrow = pz[u].v[0];
     __syncthreads();
-    SSD_FPHASE(1);
+    if (k0 == 0 && owns) {  // the state entering the chunk (st is untouched until step 6)
+      TS* o = states + ((b * C + c) * nh + h) * (int64_t)(P * N);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) __builtin_nontemporal_store((TS)st[v], o + selem(v));
+    }
     if (SSD_FUSED_DIAG != 6) request(u, gq + D);
 
-    // 3. this wave's band of C B^T, weighted and masked, as an operand
-    floatx16 acc[OB];
-#pragma unroll
-    for (int ob = 0; ob < OB; ++ob) zero_acc(acc[ob]);
-    // C . S and the band of C B^T share the fragments of C
-    floatx16 cb[2];
+    // 3. C . S and this wave's band of C B^T over its half of dstate; they share the fragments of C
+    floatx16 acc, cb[2];
+    zero_acc(acc);
     zero_acc(cb[0]);
     zero_acc(cb[1]);
 #pragma unroll
-    for (int n0 = 0; n0 < (SSD_FUSED_DIAG == 1 ? 0 : N); n0 += KG) {
-      const Vec16<T> a = frag_rows(Ct, PB, 32 * mi, n0, lane);
-#pragma unroll
-      for (int ob = 0; ob < OB; ++ob) mma_group(a, frag_cols(St, PX, n0, 32 * (pc0 + ob), lane), acc[ob]);
-      mma_group(a, frag_rows(Bt, PB, 0, n0, lane), cb[0]);
-      if (mi) mma_group(a, frag_rows(Bt, PB, 32, n0, lane), cb[1]);
+    for (int n0 = 0; n0 < (SSD_FUSED_DIAG == 1 ? 0 : NH); n0 += KG) {
+      const int nn = half * NH + n0;
+      const Vec16<T> a = frag_rows(Ct, PB, 32 * mi, nn, lane);
+      mma_group(a, frag_cols(St, PX, nn, 32 * pcb, lane), acc);
+      mma_group(a, frag_rows(Bt, PB, 0, nn, lane), cb[0]);
+      if (mi) mma_group(a, frag_rows(Bt, PB, 32, nn, lane), cb[1]);
     }
+    asm volatile("" ::: "memory");  // keeps the phases apart: reads hoisted across them cost registers
     if (SSD_FUSED_DIAG != 2) {
       if (mi) {  // the block below the diagonal one: a factor per row times a factor per column
         const float gk = fgs[l32];
@@ -914,74 +942,58 @@ __global__ __launch_bounds__(256) void ssd_fused_fwd_kernel(
           *reinterpret_cast<ema::bf16x4*>(Wr + k * PW + 8 * q + 4 * (lane >> 5)) = pack4(cd, q);
       }
     }
+    asm volatile("" ::: "memory");  // keeps the phases apart: reads hoisted across them cost registers
+    // 4. the C . S part takes the decay from the stage's start to its row
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const float sc = sms[32 * mi + acc_row(v, lane)];
-#pragma unroll
-      for (int ob = 0; ob < OB; ++ob) acc[ob][v] *= sc;
-    }
+    for (int v = 0; v < 16; ++v) acc[v] *= sms[32 * mi + acc_row(v, lane)];
     // the wave's own writes of its band are visible to its own reads once the LDS counter has drained
     __builtin_amdgcn_s_waitcnt(0xc07f);
-    SSD_FPHASE(2);
-    // 5. the causal product with x
-    for (int kk = 0; kk < (SSD_FUSED_DIAG == 3 ? 0 : 32 * (mi + 1)); kk += KG) {
-      const Vec16<T> a = frag_cols(Wr, PW, kk, 0, lane);
+    // 5. the causal product with x, and the skip term once
+    for (int kk = 0; kk < (SSD_FUSED_DIAG == 3 ? 0 : 32 * (mi + 1)); kk += KG)
+      mma_group(frag_cols(Wr, PW, kk, 0, lane), frag_cols(Xr, PX, kk, 32 * pcb, lane), acc);
+    if (Dv && half == 0) {
+      const int col = 32 * pcb + l32;
+      const float dv = d_has_hdim ? Dv[h * P + col] : Dv[h];
 #pragma unroll
-      for (int ob = 0; ob < OB; ++ob) mma_group(a, frag_cols(Xr, PX, kk, 32 * (pc0 + ob), lane), acc[ob]);
+      for (int v = 0; v < 16; ++v) acc[v] = fmaf(dv, (float)Xr[(32 * mi + acc_row(v, lane)) * PX + col], acc[v]);
     }
-    if (Dv) {
-#pragma unroll
-      for (int ob = 0; ob < OB; ++ob) {
-        const int col = 32 * (pc0 + ob) + l32;
-        const float dv = d_has_hdim ? Dv[h * P + col] : Dv[h];
-#pragma unroll
-        for (int v = 0; v < 16; ++v)
-          acc[ob][v] = fmaf(dv, (float)Xr[(32 * mi + acc_row(v, lane)) * PX + col], acc[ob][v]);
-      }
-    }
-    SSD_FPHASE(3);
+    asm volatile("" ::: "memory");  // keeps the phases apart: reads hoisted across them cost registers
     // 6. the state after the stage
-    {
+    if (owns) {
       const float dec = __expf(fminf(ae - a0, 0.f));
 #pragma unroll
-      for (int i = 0; i < BPW; ++i) {
+      for (int v = 0; v < 16; ++v) st[v] *= dec;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) st[i][v] *= dec;
-        const int j = wave + 4 * i, bm = j % MB, bn = j / MB;
-#pragma unroll
-        for (int kk = 0; kk < (SSD_FUSED_DIAG == 4 ? 0 : KT); kk += KG)
-          mma_group(frag_cols(Xw, PX, kk, 32 * bm, lane), frag_cols(Bt, PB, kk, 32 * bn, lane), st[i]);
-      }
+      for (int kk = 0; kk < (SSD_FUSED_DIAG == 4 ? 0 : KT); kk += KG)
+        mma_group(frag_cols(Xw, PX, kk, 32 * bm, lane), frag_cols(Bt, PB, kk, 32 * bn, lane), st);
     }
     a0 = ae;
-    SSD_FPHASE(4);
-    // 7. the stage's output rows through LDS, so that they leave in 16-byte pieces
+    asm volatile("" ::: "memory");  // keeps the phases apart: reads hoisted across them cost registers
+    // 7. the two partial outputs of a block meet in the output pass, which moves 16-byte pieces
+    {
+      float* mine = Os + half * KT * PO;
 #pragma unroll
-    for (int ob = 0; ob < OB; ++ob)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) Os[(32 * mi + acc_row(v, lane)) * PO + 32 * (pc0 + ob) + l32] = acc[ob][v];
+      for (int v = 0; v < 16; ++v) mine[(32 * mi + acc_row(v, lane)) * PO + 32 * pcb + l32] = acc[v];
+    }
     __syncthreads();
-    SSD_FPHASE(5);
-    constexpr int VPR = P / EPL;
-#pragma unroll
-    for (int i = 0; i < (SSD_FUSED_DIAG == 5 ? 0 : KT * VPR / 256); ++i) {
-      const int idx = tid + 256 * i;
-      const int r = idx / VPR, cv = (idx % VPR) * EPL;
+    if (SSD_FUSED_DIAG != 5) {
+      constexpr int VPR = P / EPL;
+      static_assert(KT * VPR == NT, "one piece of the output per thread");
+      const int r = tid / VPR, cv = (tid % VPR) * EPL;
       const int64_t pos = (int64_t)row0 + r;
-      if (pos < L) {
+      if (FULL || pos < L) {
         float vv[EPL];
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) vv[e] = Os[r * PO + cv + e];
+        for (int e = 0; e < EPL; ++e) vv[e] = Os[r * PO + cv + e] + Os[KT * PO + r * PO + cv + e];
         Vec16<T> o;
-        if (z) {
+        if constexpr (HAS_Z) {
           if (out_x) {
             o.set_all(vv);
             store16(out_x + b * so.sb + pos * so.sl + h * so.sh + cv, o);
           }
-          const Vec16<T> zv = load16(z + b * sz.sb + pos * sz.sl + h * sz.sh + cv);
 #pragma unroll
           for (int e = 0; e < EPL; ++e) {
-            const float zf = zv.get(e);
+            const float zf = zrow.get(e);
             vv[e] *= zf / (1.f + __expf(-zf));
           }
         }
@@ -990,24 +1002,21 @@ __global__ __launch_bounds__(256) void ssd_fused_fwd_kernel(
       }
     }
   };
+  const int Gfull = L / KT;  // stages that lie inside the sequence
   int g0 = 0;
-  for (; g0 + D <= G; g0 += D) {
+  for (; g0 + D <= Gfull; g0 += D) {
 #pragma unroll
-    for (int u = 0; u < D; ++u) stage(u, g0 + u);
+    for (int u = 0; u < D; ++u) stage(u, g0 + u, std::true_type());
   }
+  // what is left: fewer than D whole stages and at most one ragged one
 #pragma unroll
-  for (int u = 0; u < D - 1; ++u)
-    if (g0 + u < G) stage(u, g0 + u);
-  float* f = final_states + (b * nh + h) * (int64_t)(P * N);
+  for (int u = 0; u < D; ++u)
+    if (g0 + u < G) stage(u, g0 + u, std::false_type());
+  if (owns) {
+    float* f = final_states + (b * nh + h) * (int64_t)(P * N);
 #pragma unroll
-  for (int i = 0; i < BPW; ++i)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) f[selem(i, v)] = st[i][v];
-#ifdef SSD_TIMING
-  SSD_FPHASE(6);
-  if ((tid & 63) == 0 && g_ssd_timing)
-    for (int i = 0; i < 8; ++i) g_ssd_timing[((int64_t)blockIdx.x * 4 + wave) * 8 + i] = tacc[i];
-#endif
+    for (int v = 0; v < 16; ++v) f[selem(v)] = st[v];
+  }
 }
 
 // Sum over the 32 lanes of each half of a wave (lanes 0..31 and 32..63 apart), left in lanes 31

@@ -58,7 +58,7 @@ def _fused_fwd(x, dt_out, dA_cumsum, B, C, chunk_size, D=None, z=None, initial_s
     batch, seqlen, nheads, headdim = x.shape
     _, _, ngroups, dstate = B.shape
     bf16 = torch.bfloat16
-    if (chunk_size % 64 or headdim not in (64, 128) or dstate not in (64, 128) or x.dtype != bf16 or B.dtype != bf16
+    if (chunk_size % 64 or headdim != 64 or dstate not in (64, 128) or x.dtype != bf16 or B.dtype != bf16
             or C.dtype != bf16 or (z is not None and z.dtype != bf16)):
         return None
     dev = _lib.require_gpu(x, B, C, dt_out, dA_cumsum)
