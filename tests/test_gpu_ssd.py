@@ -233,8 +233,8 @@ WALK_CASES = [
 ]
 
 
-@pytest.mark.parametrize("out_dtype", [F32, BF16], ids=["out_f32", "out_bf16"])
-@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype,out_dtype", [(F32, F32), (BF16, F32), (BF16, BF16)],
+                         ids=["f32-out_f32", "bf16-out_f32", "bf16-out_bf16"])  # float32 inputs carry float32 states
 @pytest.mark.parametrize("b,L,nh,P,g,N,Q", WALK_CASES)
 def test_chunk_state_passing_in_one_kernel(b, L, nh, P, g, N, Q, dtype, out_dtype, device):
     """The kernel that keeps the chunk-local states on chip against the two launchers it replaces:
@@ -244,8 +244,6 @@ def test_chunk_state_passing_in_one_kernel(b, L, nh, P, g, N, Q, dtype, out_dtyp
     from kernels.mamba_kernels.mamba_state_fwd import _chunk_state_fwd
     from kernels.mamba_kernels.mamba_state_pass import _state_passing_fwd
 
-    if dtype == F32 and out_dtype == BF16:
-        pytest.skip("float32 inputs carry float32 states")
     announce(f"ssd state walk b{b} L{L} nh{nh} P{P} g{g} N{N} Q{Q} {dtype} -> {out_dtype}")
     x, dt, A, B, _, _, _ = S.make_inputs(b, L, nh, P, g, N, seed=L + N + Q, dtype=dtype)
     init = torch.randn(b, nh, P, N, generator=torch.Generator().manual_seed(9))
