@@ -230,6 +230,8 @@ WALK_CASES = [
     (1, 900, 3, 64, 1, 64, 512),
     (1, 1100, 2, 64, 1, 128, 1024),
     (3, 64, 2, 64, 1, 128, 64),     # one stage in all
+    (1, 50, 2, 64, 1, 64, 64),      # less than one stage
+    (1, 8256, 1, 64, 1, 128, 256),  # 129 stages: rounds of the ring and a remainder
 ]
 
 
@@ -301,6 +303,8 @@ FUSED_CASES = [
     (1, 900, 3, 64, 1, 64, 512),
     (1, 1100, 2, 64, 1, 128, 1024),
     (3, 64, 2, 64, 1, 128, 64),     # one stage in all
+    (1, 50, 2, 64, 1, 64, 64),      # less than one stage
+    (1, 2100, 1, 64, 1, 128, 256),  # a ragged last stage behind many whole ones
 ]
 
 
