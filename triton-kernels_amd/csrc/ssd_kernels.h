@@ -121,6 +121,13 @@ struct Tile {
   static constexpr int KG = 2 * EPL;  // contraction extent of one mma_group
   // LDS pitch (elements) of a tile with `cols` dense columns: 16 bytes of padding
   static constexpr int pitch(int cols) { return cols + EPL; }
+  // LDS pitch of a tile that is contracted along its rows (read with frag_cols).  The LDS has 64
+  // banks of 4 bytes.  One transposing read takes, per half wave, 64 adjacent bytes of four
+  // consecutive rows: with 64 bytes of padding (bf16 rows are multiples of 128 bytes here) the
+  // four rows fall into four different quarters of the 256-byte bank period.  The float32 form
+  // reads 128 adjacent bytes of two rows four apart per instruction: 32 bytes of padding put them
+  // into different halves.
+  static constexpr int kpitch(int cols) { return cols + (sizeof(T) == 2 ? 32 : 8); }
 };
 
 __device__ __forceinline__ void zero_acc(floatx16& a) {
@@ -181,7 +188,7 @@ __device__ __forceinline__ void stage_rows(T* tile, const T* __restrict__ g, int
 // tile's loads in flight while it works on the current one calls them apart.  Up to two float32
 // values per row (aux0[row], aux1[row]; null = not wanted) travel with the pieces, so that a
 // row scale computed from them costs no load at store time.
-template <typename T, int ROWS, int COLS>
+template <typename T, int ROWS, int COLS, int PITCH = Tile<T>::pitch(COLS)>
 struct RowPieces {
   static constexpr int EPL = Vec16<T>::N, VPR = COLS / EPL, CNT = ROWS * VPR / 256;
   static_assert((ROWS * VPR) % 256 == 0 && CNT <= 8, "tile must split evenly over 256 threads");
@@ -205,7 +212,7 @@ struct RowPieces {
   // scale(row, aux0[row], aux1[row]) multiplies the row; NoScale leaves it
   template <typename F>
   __device__ __forceinline__ void store(T* tile, int row0, int limit, int tid, F scale) {
-    constexpr int P = Tile<T>::pitch(COLS);
+    constexpr int P = PITCH;
 #pragma unroll
     for (int i = 0; i < CNT; ++i) {
       const int idx = tid + 256 * i;
@@ -319,7 +326,7 @@ __global__ __launch_bounds__(256) void ssd_cumsum_kernel(const TD* __restrict__ 
 // ------------------------------------------------------------------------------------
 template <typename T, int P, int N>
 struct StateSmem {
-  static constexpr int KT = 64, PX = Tile<T>::pitch(P), PB = Tile<T>::pitch(N);
+  static constexpr int KT = 64, PX = Tile<T>::kpitch(P), PB = Tile<T>::kpitch(N);
   static constexpr int kStage = KT * (PX + PB) * (int)sizeof(T);
   // One stage in LDS.  The next stage waits in registers while this one is multiplied, so a second
   // LDS buffer only saves a barrier per stage, and at 53 KB it allowed three workgroups per CU
@@ -368,8 +375,8 @@ __global__ __launch_bounds__(256) void ssd_chunk_state_kernel(
     const float w = __expf(dA_k);
     return (sq.on() && sq.at(k) != seq_ref) ? 0.f : w;
   };
-  RowPieces<T, KT, P> px;
-  RowPieces<T, KT, N> pb;
+  RowPieces<T, KT, P, PX> px;
+  RowPieces<T, KT, N, PB> pb;
   auto request = [&](int k0) {  // the pieces of a stage and the per-row values their scale needs
     px.template load<true>(xg, sx.sl, k0, limit, tid, MODE == 1 ? dAp : nullptr);
     pb.load(Bg, sB.sl, k0, limit, tid, MODE == 0 ? dAp : nullptr, MODE == 0 ? dtp : nullptr);
@@ -552,7 +559,7 @@ __global__ __launch_bounds__(256) void ssd_state_passing_kernel(
 #endif
 template <typename T, int P, int NL>
 struct WalkSmem {
-  static constexpr int KT = 64, PX = Tile<T>::pitch(P), PB = Tile<T>::pitch(NL);
+  static constexpr int KT = 64, PX = Tile<T>::kpitch(P), PB = Tile<T>::kpitch(NL);
   static constexpr int kStageElems = KT * (PX + PB);
   static constexpr int kBytes = 2 * kStageElems * (int)sizeof(T);
 };
@@ -572,8 +579,8 @@ __global__ __launch_bounds__(256, NSPLIT) void ssd_state_walk_kernel(
   static_assert(MB * NB % 4 == 0, "output blocks must split over 4 waves");
   // stages in flight: as many as the registers hold next to the two sets of accumulators
   constexpr int kPieceRegs = NSPLIT == 2
-      ? (RowPieces<T, KT, P>::CNT + RowPieces<T, KT, NL>::CNT) * 6 + 2 * RowPieces<T, KT, NL>::CNT
-      : (RowPieces<T, KT, P>::CNT + RowPieces<T, KT, NL>::CNT) * 4 + 2 * RowPieces<T, KT, NL>::CNT;
+      ? (RowPieces<T, KT, P, S::PX>::CNT + RowPieces<T, KT, NL, S::PB>::CNT) * 6 + 2 * RowPieces<T, KT, NL, S::PB>::CNT
+      : (RowPieces<T, KT, P, S::PX>::CNT + RowPieces<T, KT, NL, S::PB>::CNT) * 4 + 2 * RowPieces<T, KT, NL, S::PB>::CNT;
   constexpr int kRoom = 256 - 2 * BPW * 16 - (NSPLIT == 2 ? 140 : 40 + 8 * BPW + (sizeof(T) == 4 ? 16 : 0));
 #ifdef SSD_WALK_D
   constexpr int D = SSD_WALK_D;
@@ -601,9 +608,9 @@ __global__ __launch_bounds__(256, NSPLIT) void ssd_state_walk_kernel(
   };
   // Every request is unconditional (a load inside a branch would have to complete before the next
   // is issued): stages past the end are requested again as the last one and never used.
-  RowPieces<T, KT, P> px[D];
-  RowPieces<T, KT, NL> pb[D];
-  auto request = [&](RowPieces<T, KT, P>& rx, RowPieces<T, KT, NL>& rb, int g) {
+  RowPieces<T, KT, P, S::PX> px[D];
+  RowPieces<T, KT, NL, S::PB> pb[D];
+  auto request = [&](RowPieces<T, KT, P, S::PX>& rx, RowPieces<T, KT, NL, S::PB>& rb, int g) {
     const int row0 = min(g, G - 1) * KT;
 #ifndef SSD_WALK_XNT
 #define SSD_WALK_XNT true
@@ -631,7 +638,7 @@ __global__ __launch_bounds__(256, NSPLIT) void ssd_state_walk_kernel(
   float dal_next = dAb[Q - 1], dal = 0.f;
 
   // one stage: rx / rb hold its rows and receive those of stage g + D
-  auto stage = [&](RowPieces<T, KT, P>& rx, RowPieces<T, KT, NL>& rb, int g) {
+  auto stage = [&](RowPieces<T, KT, P, S::PX>& rx, RowPieces<T, KT, NL, S::PB>& rb, int g) {
     const int row0 = g * KT;
     const int c = row0 / Q, k0 = row0 - c * Q;
     if (k0 == 0) {
@@ -653,10 +660,10 @@ __global__ __launch_bounds__(256, NSPLIT) void ssd_state_walk_kernel(
       rb.store(bb, row0, L, tid, [&](int, float dA_k, float dt_k) { return __expf(fminf(dA_last - dA_k, 0.f)) * dt_k; });
     } else {  // the rows must still arrive
 #pragma unroll
-      for (int i = 0; i < RowPieces<T, KT, P>::CNT; ++i)
+      for (int i = 0; i < RowPieces<T, KT, P, S::PX>::CNT; ++i)
         if (SSD_WALK_DIAG != 4) acc[0][0] += rx.v[i].get(0);
 #pragma unroll
-      for (int i = 0; i < RowPieces<T, KT, NL>::CNT; ++i)
+      for (int i = 0; i < RowPieces<T, KT, NL, S::PB>::CNT; ++i)
         if (SSD_WALK_DIAG != 5) acc[0][1] += rb.v[i].get(0) + rb.a0[i] + rb.a1[i];
     }
     __syncthreads();
@@ -1149,7 +1156,7 @@ __global__ __launch_bounds__(256) void ssd_row_cumsum_kernel(float* __restrict__
 // ------------------------------------------------------------------------------------
 template <typename T, int P, int N>
 struct GroupSmem {
-  static constexpr int PS = Tile<T>::pitch(N);
+  static constexpr int PS = Tile<T>::kpitch(N);  // the state tile is contracted along its rows
   static constexpr int kBytes = P * PS * (int)sizeof(T) + (4 * 64 + 64) * (int)sizeof(float);
 };
 
