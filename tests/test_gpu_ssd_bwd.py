@@ -22,6 +22,8 @@ CASES = [
     (1, 150, 2, 64, 1, 64, 48),     # chunk sizes that are no multiple of the 64-row tiles
     (1, 333, 2, 64, 2, 64, 200),
     (1, 1100, 2, 64, 1, 128, 1024),  # the largest chunk size, second chunk ragged
+    (1, 320, 7, 64, 1, 128, 64),    # seven heads in a group: the three head slots of the dB / dC kernel wrap twice
+    (1, 192, 2, 64, 2, 128, 64),    # one head per group
     # head and state sizes the kernels do not take natively (split into sub-heads / zero-padded
     # around them); the reference's EMA tests and benchmarks call its Mamba launchers with
     # dstate = 1 and head sizes 8, 32 and 512

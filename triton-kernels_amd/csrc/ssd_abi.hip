@@ -284,6 +284,23 @@ struct GroupLaunch {
   }
   template <typename T, int P, int N, typename TS>
   int run_as() const {
+#ifndef SSD_GROUP_DMA  // 0: development builds without the kernel that copies its operands straight into LDS
+#define SSD_GROUP_DMA 1
+#endif
+    if constexpr (SSD_GROUP_DMA && std::is_same<T, bf16_t>::value && std::is_same<TS, bf16_t>::value && P == 64 && N == 128) {
+      // (the kernel keeps the byte offset of a row inside a chunk in 32 bits)
+      if (d.Q % 64 == 0 && !seq.p && d.Q * sa.sl < (int64_t(1) << 30)) {
+        auto kernel = ssd_group_grad_dma_kernel<MODE>;
+        constexpr int smem = GroupDmaSmem::kBytes;
+        SSD_TRY(allow_smem(kernel, smem));
+        const int mtiles = (int)(d.Q / 64);
+        if (d.batch * d.C * d.g * mtiles > 0x7fffffff) return SSD_ERR_SHAPE;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.C * d.g * mtiles)), dim3(256), smem, st, (const bf16_t*)a,
+                           sa, (const bf16_t*)s, dt, dA, (const bf16_t*)bc, sbc, out, ddA, (int)d.nh, (int)(d.nh / d.g),
+                           (int)d.g, (int)d.L, (int)d.Q, (int)d.C, mtiles);
+        return launched();
+      }
+    }
     auto kernel = ssd_group_grad_kernel<T, P, N, MODE, TS>;
     constexpr int smem = GroupSmem<T, P, N>::kBytes;
     SSD_TRY(allow_smem(kernel, smem));

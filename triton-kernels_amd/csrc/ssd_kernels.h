@@ -1307,6 +1307,243 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
 }
 
 // ------------------------------------------------------------------------------------
+// The same for bfloat16 operands and states, hdim 64, dstate 128, chunk sizes that are multiples of
+// 64, no packed batch.  A workgroup spends most of a head waiting for the head's state tile and rows,
+// and the registers do not hold a second head next to the accumulators, so here everything a head
+// needs is copied from global memory straight into LDS by the load unit (no registers in between):
+// three heads' worth of LDS, the copies of heads h + 1 and h + 2 under way while head h is
+// multiplied, one barrier per head.  A copy puts the 16-byte pieces that the 64 lanes ask for side
+// by side (1 KB per instruction), so the tiles have no padding; bank conflicts are avoided by
+// the order of the pieces inside a row, which the requesting lane chooses through the address it
+// asks for:
+//   state tile [64 p][128 n] (256-byte rows, read with the transposing read): piece j of row r in slot
+//     j ^ 4 (r % 4), so that four consecutive rows fall into four different quarters of the bank period;
+//   rows of a [64 m][64 p] (128-byte rows, read 16 bytes per lane, a lane per row): piece j of row r in
+//     slot j ^ ((r / 2) % 8), so that sixteen consecutive rows cover all banks;
+//   one more instruction brings dA[m0 .. m0 + 63], dt[m0 .. m0 + 63] and dA[Q - 4 .. Q - 1].
+// The copies count as vector-memory loads of the requesting wave and complete in order; a wave waits
+// until only the copies of the head after the current one are outstanding, then passes the barrier.
+// ------------------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+// 64 lanes x 16 bytes from global memory into LDS: lane l's piece lands at lds_base + 16 * l
+// (lds_base is the same for the whole wave).  Written as assembly so that the compiler does not
+// make every later LDS read wait for all copies under way; the caller waits for the counter.
+__device__ __forceinline__ void copy16_to_lds(const void* g, void* lds_base) {
+  const unsigned lds = (unsigned)(uintptr_t)(lds_void_t*)lds_base;
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds) : "memory", "m0");
+}
+
+// The same with the address split into a base that is the same for the whole wave (scalar registers)
+// and a byte offset per lane: a loop that only moves the base spends no vector instructions on addresses.
+__device__ __forceinline__ void copy16_to_lds(const void* base, unsigned lane_offset, void* lds_base) {
+  const unsigned lds = (unsigned)(uintptr_t)(lds_void_t*)lds_base;
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base), "s"(lds)
+               : "memory", "m0");
+}
+
+struct GroupDmaSmem {
+  static constexpr int R = 3;  // heads in LDS
+  static constexpr int kState = 64 * 128 * (int)sizeof(bf16_t), kRows = 64 * 64 * (int)sizeof(bf16_t), kVec = 2048;
+  static constexpr int kHead = kState + kRows + kVec;
+  static constexpr int kBytes = R * kHead + 2 * 4 * 32 * (int)sizeof(float);  // + the row sums of two heads
+  // copies a wave requests per head (the first wave one more: the vectors)
+  static constexpr int kCopiesPerWave = 16 / 4 + 8 / 4;
+};
+
+template <int MODE>
+__global__ __launch_bounds__(256, 2) void ssd_group_grad_dma_kernel(
+    const bf16_t* __restrict__ a, Strides3 sa, const bf16_t* __restrict__ s, const float* __restrict__ dt,
+    const float* __restrict__ dA_cs, const bf16_t* __restrict__ bc, Strides3 sbc, float* __restrict__ out,
+    float* __restrict__ ddA, int nh, int heads_per_group, int ngroups, int L, int Q, int C, int mtiles) {
+  using S = GroupDmaSmem;
+  using T = bf16_t;
+  constexpr int P = 64, N = 128, EPL = 8, KG = 16, BPW = 2, KS = P / KG;
+  static_assert(S::kCopiesPerWave == 6, "the wait below counts six copies per wave and head");
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  float* rs = reinterpret_cast<float*>(smem + S::R * S::kHead);  // [2 heads][4 waves][32 rows]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31, half = lane >> 5;
+  const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
+  const int mt = bid % mtiles;
+  const int g = (bid / mtiles) % ngroups;
+  const int c = (bid / (mtiles * ngroups)) % C;
+  const int64_t b = bid / ((int64_t)mtiles * ngroups * C);
+  const int limit = min(Q, L - c * Q);
+  const int m0 = 64 * mt;
+
+  // block i of this wave: rows 32 * mi .., columns 32 * ni[i] ..
+  const int mi = wave & 1;
+  int ni[BPW];
+#pragma unroll
+  for (int i = 0; i < BPW; ++i) ni[i] = (wave + 4 * i) >> 1;
+  const int rloc = 32 * mi + l32;  // this lane's row inside the tile
+  const int m = m0 + rloc;
+  const bool want_ddA = bc != nullptr;
+  floatx16 total[BPW];
+#pragma unroll
+  for (int i = 0; i < BPW; ++i) zero_acc(total[i]);
+
+  // The copies of head hh into LDS set u.  What depends on the lane is the same for every head and is
+  // kept as byte offsets; a head only moves the (scalar) bases.
+  unsigned s_off[4], a_off[2];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {  // four rows of the state tile per instruction
+    const int r = 4 * (4 * wave + j) + (lane >> 4);
+    s_off[j] = (unsigned)(r * N + 8 * ((lane & 15) ^ (4 * (r & 3)))) * (unsigned)sizeof(T);
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {  // eight rows of a per instruction
+    const int r = 8 * (2 * wave + j) + (lane >> 3);
+    a_off[j] = (unsigned)((int64_t)min(m0 + r, limit - 1) * sa.sl + 8 * ((lane & 7) ^ ((r >> 1) & 7))) * (unsigned)sizeof(T);
+  }
+  // waves 0 and 1 bring dA[m0 .. m0 + 63] with dA[Q - 4 .. Q - 1] behind it, and dt[m0 .. m0 + 63]
+  const unsigned v_off = (unsigned)(lane < 16 ? m0 + 4 * lane : (wave == 0 ? Q - 4 : m0)) * (unsigned)sizeof(float);
+  const T* s_first = s + (((b * C + c) * nh + g * heads_per_group) * (int64_t)P) * N;
+  const T* a_first = a + b * sa.sb + (int64_t)c * Q * sa.sl + (int64_t)g * heads_per_group * sa.sh;
+  const int64_t chunk_first = (b * nh + g * heads_per_group) * (int64_t)C + c;
+  auto request = [&](int hh, int u) {
+    unsigned char* base = smem + u * S::kHead;
+    const T* sg = s_first + (int64_t)hh * P * N;
+    const T* ag = a_first + (int64_t)hh * sa.sh;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) copy16_to_lds(sg, s_off[j], base + (4 * wave + j) * 1024);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) copy16_to_lds(ag, a_off[j], base + S::kState + (2 * wave + j) * 1024);
+    if (wave < 2) {
+      const float* vg = (wave == 0 ? dA_cs : dt) + (chunk_first + (int64_t)hh * C) * Q;
+      copy16_to_lds(vg, v_off, base + S::kState + S::kRows + wave * 1024);
+    }
+  };
+  request(0, 0);
+  if (heads_per_group > 1) request(1, 1);
+  // bc in the (transposed) accumulator layout: this lane's row m, columns n of each block.  Loaded
+  // behind the first copies and waited for here, so that no wait for ordinary loads (which would wait
+  // for every copy before them as well) falls into the loop.
+  float bcv[BPW][16];
+#pragma unroll
+  for (int i = 0; i < BPW; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) bcv[i][v] = 0.f;
+  if (want_ddA) {
+    const T* bcg = bc + b * sbc.sb + (int64_t)c * Q * sbc.sl + g * sbc.sh;
+#pragma unroll
+    for (int i = 0; i < BPW; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const float t = (float)bcg[(int64_t)min(m, limit - 1) * sbc.sl + 32 * ni[i] + acc_row(v, lane)];
+        bcv[i][v] = m < limit ? t : 0.f;
+      }
+  }
+#pragma unroll
+  for (int i = 0; i < BPW; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) asm volatile("" : "+v"(bcv[i][v]));
+
+  // where this lane reads its operand fragments inside a head's tiles (elements)
+  int r_off[KS], t_off[BPW];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) r_off[ks] = rloc * P + 8 * ((2 * ks + half) ^ ((rloc >> 1) & 7));
+#pragma unroll
+  for (int i = 0; i < BPW; ++i) {
+    const int i16 = lane & 15;
+    const int row = 8 * half + (i16 >> 2);
+    const int col = 32 * ni[i] + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+    t_off[i] = row * N + 8 * ((col >> 3) ^ (4 * (row & 3))) + (col & 7);
+  }
+
+  for (int hh = 0; hh < heads_per_group; ++hh) {
+    const int u = hh % S::R;
+    // the copies of this head have landed once only those of the next head are outstanding
+    if (hh + 1 < heads_per_group) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // every wave's part of the head is there; every wave is done with head hh - 1
+    if (hh + 2 < heads_per_group) request(hh + 2, (hh + 2) % S::R);
+    if (want_ddA && hh > 0 && tid < 64) {  // the row sums of head hh - 1 (see below)
+      const float* rp = rs + ((hh - 1) & 1) * 128;
+      const int w0 = tid >> 5;
+      const float r = rp[w0 * 32 + (tid & 31)] + rp[(w0 + 2) * 32 + (tid & 31)];
+      float* o = ddA + ((b * nh + g * heads_per_group + hh - 1) * C + c) * (int64_t)Q;
+      const int mm = m0 + tid;
+      if (MODE == 0) {
+        if (mm + 1 < Q) o[mm + 1] = r;
+        if (mm == 0) o[0] = 0.f;
+      } else {
+        o[mm] = r;
+      }
+    }
+    const unsigned char* base = smem + u * S::kHead;
+    const T* St = reinterpret_cast<const T*>(base);
+    const T* At = reinterpret_cast<const T*>(base + S::kState);
+    const float* vec = reinterpret_cast<const float*>(base + S::kState + S::kRows);  // dA rows, dA tail | dt rows
+    // the weight of this lane's row; rows past the sequence (their operand rows repeat the last
+    // valid one) get none
+    const float wr = MODE == 0 ? __expf(fminf(vec[67] - vec[rloc], 0.f)) * vec[256 + rloc] : __expf(vec[rloc]);
+    const float w = m < limit ? wr : 0.f;
+    floatx16 acc[BPW];
+#pragma unroll
+    for (int i = 0; i < BPW; ++i) zero_acc(acc[i]);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const Vec16<T> av = load16(At + r_off[ks]);
+#pragma unroll
+      for (int i = 0; i < BPW; ++i) {
+        // St[p][n] contracted along p: lane l receives eight consecutive p of column n = 32 ni + l % 32
+        // (sixteen rows further down the key of a row is the same)
+        const T* p = St + t_off[i] + KG * ks * N;
+        typedef __attribute__((address_space(3))) ema::bf16x4 lds_bf16x4;
+        const ema::bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)p);
+        const ema::bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(p + 4 * N));  // row + 4: the same key
+        Vec16<T> sf;
+        sf.raw = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        mma_group(sf, av, acc[i]);  // [n][m]
+      }
+    }
+    float part = 0.f;
+#pragma unroll
+    for (int i = 0; i < BPW; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        total[i][v] = fmaf(acc[i][v], w, total[i][v]);
+        part = fmaf(acc[i][v], bcv[i][v], part);  // bcv is zero where no row sums are asked for
+      }
+    if (want_ddA) {
+      // the halves of the wave hold different columns n of row m; the waves w and w + 2 too: their
+      // sums meet after the next barrier
+      part += __shfl_xor(part, 32);
+      if (half == 0) rs[(hh & 1) * 128 + wave * 32 + l32] = part * w;
+    }
+  }
+  if (want_ddA) {
+    __syncthreads();
+    if (tid < 64) {
+      const int hh = heads_per_group - 1;
+      const float* rp = rs + (hh & 1) * 128;
+      const int w0 = tid >> 5;
+      const float r = rp[w0 * 32 + (tid & 31)] + rp[(w0 + 2) * 32 + (tid & 31)];
+      float* o = ddA + ((b * nh + g * heads_per_group + hh) * C + c) * (int64_t)Q;
+      const int mm = m0 + tid;
+      if (MODE == 0) {
+        if (mm + 1 < Q) o[mm + 1] = r;
+        if (mm == 0) o[0] = 0.f;
+      } else {
+        o[mm] = r;
+      }
+    }
+  }
+  // total is [n][m] per block: a lane writes four adjacent n of its row m at a time
+  float* og = out + (b * L + (int64_t)c * Q) * ngroups * N + (int64_t)g * N;
+  if (m < limit) {
+#pragma unroll
+    for (int i = 0; i < BPW; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; v += 4)
+        *reinterpret_cast<float4*>(og + (int64_t)m * ngroups * N + 32 * ni[i] + acc_row(v, lane)) =
+            make_float4(total[i][v], total[i][v + 1], total[i][v + 2], total[i][v + 3]);
+  }
+}
+
+// ------------------------------------------------------------------------------------
 // bmm_chunk.  out[b, c, g, m, k] = sum_n a[b, cQ+m, g, n] * bm[b, cQ+k, g, n]; one workgroup
 // per 64 x 64 output tile, one 32 x 32 block per wave; rows past the sequence are zero, and so
 // are, in a packed batch, the entries whose two positions carry different ids.
