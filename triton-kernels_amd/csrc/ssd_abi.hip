@@ -134,6 +134,21 @@ struct WalkLaunch {
   }
   template <typename T, int P, int N, typename TO>
   int run_as() const {
+#ifndef SSD_WALK_DMA  // 0: development builds without the kernel that copies its rows straight into LDS
+#define SSD_WALK_DMA 1
+#endif
+    // (the kernel keeps the byte offset of a row inside a stage in 32 bits)
+    if constexpr (SSD_WALK_DMA && std::is_same<T, bf16_t>::value && P == 64 && N == 128) {
+      if (sx.sl < (int64_t(1) << 24) && sB.sl < (int64_t(1) << 24)) {
+        auto kernel = ssd_state_walk_dma_kernel<TO>;
+        constexpr int smem = WalkDmaSmem::kBytes;
+        SSD_TRY(allow_smem(kernel, smem));
+        hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.nh)), dim3(512), smem, st, (const bf16_t*)x, sx,
+                           (const bf16_t*)B, sB, dt, dA, initial, (TO*)out, final_states, (int)d.nh, (int)(d.nh / d.g),
+                           (int)d.L, (int)d.Q, (int)d.C);
+        return launched();
+      }
+    }
 #ifndef SSD_WALK_NSPLIT  // 2: two workgroups per (b, h), half the state columns each (measured no faster: x crosses the L2 twice)
 #define SSD_WALK_NSPLIT 1
 #endif

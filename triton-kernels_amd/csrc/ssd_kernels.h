@@ -130,6 +130,29 @@ struct Tile {
   static constexpr int kpitch(int cols) { return cols + (sizeof(T) == 2 ? 32 : 8); }
 };
 
+// ------------------------------------------------------------------ copies from global memory into LDS
+// The load unit can write what it fetches straight into LDS, without passing through registers:
+// such copies occupy no registers while they are under way, so how many a workgroup has in flight is
+// bounded by LDS alone.  They count as vector-memory loads of the requesting wave and complete in
+// order with its other loads and stores.
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+// 64 lanes x 16 bytes from global memory into LDS: lane l's piece lands at lds_base + 16 * l
+// (lds_base is the same for the whole wave).  Written as assembly so that the compiler does not
+// make every later LDS read wait for all copies under way; the caller waits for the counter.
+__device__ __forceinline__ void copy16_to_lds(const void* g, void* lds_base) {
+  const unsigned lds = (unsigned)(uintptr_t)(lds_void_t*)lds_base;
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds) : "memory", "m0");
+}
+
+// The same with the address split into a base that is the same for the whole wave (scalar registers)
+// and a byte offset per lane: a loop that only moves the base spends no vector instructions on addresses.
+__device__ __forceinline__ void copy16_to_lds(const void* base, unsigned lane_offset, void* lds_base) {
+  const unsigned lds = (unsigned)(uintptr_t)(lds_void_t*)lds_base;
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base), "s"(lds)
+               : "memory", "m0");
+}
+
 __device__ __forceinline__ void zero_acc(floatx16& a) {
 #pragma unroll
   for (int v = 0; v < 16; ++v) a[v] = 0.f;
@@ -701,6 +724,168 @@ __global__ __launch_bounds__(256, NSPLIT) void ssd_state_walk_kernel(
   for (int i = 0; i < BPW; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) f[elem(i, v)] = st[i][v];
+}
+
+// ------------------------------------------------------------------------------------
+// The same walk for bfloat16, hdim 64, dstate 128, with the rows copied from global memory straight
+// into LDS.  A workgroup is alone on its compute unit and walks its rows in sequence, so what keeps
+// its share of the memory system busy is the number of stages in flight; copies into LDS occupy no
+// registers, which also leaves room for eight waves (one 32 x 32 block of the state each) where the
+// register-staged kernel has four.  R stages live in LDS: while stage g is multiplied the copies of
+// stages g + 1 .. g + R - 1 are under way; one barrier per stage.  Per stage: 64 rows of x (128-byte
+// rows) and of B (256-byte rows), both read with the transposing read and therefore stored with
+// their 16-byte pieces permuted (see the dB / dC kernel below), and two small pieces with the stage's dA
+// and dt and the chunk's last dA.  B arrives unweighted, so the weight exp(min(dA_last - dA_k, 0)) dt_k
+// is applied to the operand fragment (float32 product, rounded to bfloat16: the same arithmetic as where
+// the register-staged kernels weight the rows on their way into LDS); each wave computes the stage's 64
+// weights once, a lane each, and passes them through 256 bytes of LDS of its own.  Results equal those
+// of the register-staged kernel (and of the two launchers) bit for bit.
+//
+// The waits are placed by hand.  Copies and stores of a wave complete in the order of their requests,
+// and the counter that s_waitcnt vmcnt(n) tests counts both; a stage's copies have landed once no more
+// than the requests made after them are outstanding: three copies for each later stage in flight (a
+// wave requests three or four per stage) and the sixteen stores of the state entering a chunk, if a
+// chunk began since.  No ordinary load may sit in the loop: its wait would wait for every copy before
+// it as well.
+// ------------------------------------------------------------------------------------
+struct WalkDmaSmem {
+  static constexpr int R = 4;  // stages in LDS (five and six measured slower)
+  static constexpr int kX = 64 * 64 * (int)sizeof(bf16_t), kB = 64 * 128 * (int)sizeof(bf16_t), kVec = 2048;
+  static constexpr int kStage = kX + kB + kVec;
+  static constexpr int kBytes = R * kStage + 8 * 64 * (int)sizeof(float);  // + the weights, a copy per wave
+};
+
+template <typename TO>
+__global__ __launch_bounds__(512) void ssd_state_walk_dma_kernel(
+    const bf16_t* __restrict__ x, Strides3 sx, const bf16_t* __restrict__ B, Strides3 sB, const float* __restrict__ dt,
+    const float* __restrict__ dA_cs, const float* __restrict__ initial, TO* __restrict__ out,
+    float* __restrict__ final_states, int nh, int heads_per_group, int L, int Q, int C) {
+  using S = WalkDmaSmem;
+  using T = bf16_t;
+  constexpr int P = 64, N = 128, KT = 64, KG = 16, MB = P / 32, R = S::R;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), half = lane >> 5;
+  float* wl = reinterpret_cast<float*>(smem + R * S::kStage) + wave * 64;  // this wave's copy of the weights
+  const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
+  const int h = bid % nh;
+  const int64_t b = bid / nh;
+  const float* dAb = dA_cs + (b * nh + h) * (int64_t)C * Q;
+  const float* dtb = dt + (b * nh + h) * (int64_t)C * Q;
+  const T* xg = x + b * sx.sb + h * sx.sh;
+  const T* Bg = B + b * sB.sb + (h / heads_per_group) * sB.sh;
+  const int G = (L + KT - 1) / KT;
+  const int mi = wave % MB, ni = wave / MB;  // this wave's block of the state: rows 32 mi .., columns 32 ni ..
+  auto elem = [&](int v) { return (32 * mi + acc_row(v, lane)) * N + 32 * ni + (lane & 31); };
+
+  // The copies of stage g into LDS set u: wave w brings rows 8 w .. 8 w + 7 of x (one instruction),
+  // rows 8 w .. of B (two), and waves 0 / 1 the pieces of dA / dt.  What depends on the lane is
+  // computed here; a request moves scalar bases (and clamps the rows of the last, ragged stage).
+  const int xr = 8 * wave + (lane >> 3);                                  // row of x inside the stage
+  const unsigned x_piece = 16u * ((lane & 7) ^ (4 * ((xr >> 1) & 1)));    // byte offset inside the row
+  int br[2];
+  unsigned b_piece[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    br[j] = 4 * (2 * wave + j) + (lane >> 4);
+    b_piece[j] = 16u * ((lane & 15) ^ (4 * (br[j] & 3)));
+  }
+  auto request = [&](int g, int u) {
+    const int row0 = min(g, G - 1) * KT;
+    const int last = L - 1 - row0;  // rows past the sequence repeat its last row (their weight is 0)
+    unsigned char* base = smem + u * S::kStage;
+    copy16_to_lds(xg + (int64_t)row0 * sx.sl, (unsigned)(min(xr, last) * sx.sl) * 2u + x_piece, base + wave * 1024);
+    const T* bg = Bg + (int64_t)row0 * sB.sl;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      copy16_to_lds(bg, (unsigned)(min(br[j], last) * sB.sl) * 2u + b_piece[j], base + S::kX + (2 * wave + j) * 1024);
+    if (wave < 2) {
+      // lanes 0 .. 15: the stage's 64 values; the others: the chunk's last four values of dA (dt: anything valid)
+      const int tail = (row0 / Q + 1) * Q - 4 - row0;
+      const unsigned off = 4u * (unsigned)(lane < 16 ? 4 * lane : (wave == 0 ? tail : 0));
+      copy16_to_lds((wave == 0 ? dAb : dtb) + row0, off, base + S::kX + S::kB + wave * 1024);
+    }
+  };
+#pragma unroll
+  for (int u = 0; u < R - 1; ++u) request(u, u);
+
+  floatx16 acc, st;
+  zero_acc(acc);
+  zero_acc(st);
+  if (initial) {
+    const float* ini = initial + (b * nh + h) * (int64_t)(P * N);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) st[v] = ini[elem(v)];
+  }
+  // (waited for here, so that no wait for ordinary loads falls into the loop)
+#pragma unroll
+  for (int v = 0; v < 16; ++v) asm volatile("" : "+v"(st[v]));
+
+  // where this lane reads its operand fragments inside a stage's tiles (elements)
+  int x_off, b_off;
+  {
+    const int i16 = lane & 15;
+    const int row = 8 * half + (i16 >> 2);
+    const int cx = 32 * mi + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+    const int cb = 32 * ni + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+    x_off = row * P + 8 * ((cx >> 3) ^ (4 * ((row >> 1) & 1))) + (cx & 7);
+    b_off = row * N + 8 * ((cb >> 3) ^ (4 * (row & 3))) + (cb & 7);
+  }
+  typedef __attribute__((address_space(3))) ema::bf16x4 lds_bf16x4;
+  auto tr_read = [&](const T* p, int pitch) {
+    const ema::bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)p);
+    const ema::bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(p + 4 * pitch));  // row + 4: the same key
+    Vec16<T> r;
+    r.raw = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return r;
+  };
+
+  int since = R;  // stages since the last chunk began (at least R: no stores in the queue)
+  for (int g = 0; g < G; ++g) {
+    const int u = g % R;
+    const int row0 = g * KT;
+    const int c = row0 / Q, k0 = row0 - c * Q;
+    // The copies of this stage have landed once only later requests are outstanding: those of the R - 2
+    // stages after it (three per wave and stage, four for two of the waves) and, if a chunk began
+    // 1 .. R - 2 stages ago, the sixteen stores of its entering state (with chunks of one or two stages
+    // there may be two such chunks: the lower count waits a little longer).
+    if (since <= R - 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (R - 2) + 16) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (R - 2)) : "memory");
+    __syncthreads();  // every wave's part of the stage is there; every wave is done with stage g - 1
+    if (k0 == 0) {  // the state entering the chunk
+      TO* o = out + ((b * C + c) * nh + h) * (int64_t)(P * N);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) __builtin_nontemporal_store((TO)st[v], o + elem(v));
+      since = 0;
+    }
+    ++since;
+    request(g + R - 1, (g + R - 1) % R);
+    const unsigned char* base = smem + u * S::kStage;
+    const T* xb = reinterpret_cast<const T*>(base);
+    const T* bb = reinterpret_cast<const T*>(base + S::kX);
+    const float* vec = reinterpret_cast<const float*>(base + S::kX + S::kB);  // dA rows, dA tail | dt rows
+    const float dA_last = vec[67];
+    wl[lane] = __expf(fminf(dA_last - vec[lane], 0.f)) * vec[256 + lane];
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // the wave's own LDS writes are visible to its own reads
+#pragma unroll
+    for (int ks = 0; ks < KT / KG; ++ks) {
+      const Vec16<T> xf = tr_read(xb + x_off + KG * ks * P, P);
+      Vec16<T> bf = tr_read(bb + b_off + KG * ks * N, N);
+      float t[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) t[e] = bf.get(e) * wl[KG * ks + 8 * half + e];
+      bf.set_all(t);
+      mma_group(xf, bf, acc);
+    }
+    if (k0 + KT >= Q || g == G - 1) {  // the chunk ends with this stage
+      const float a = __expf(dA_last);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) st[v] = fmaf(a, st[v], acc[v]);
+      zero_acc(acc);
+    }
+  }
+  float* f = final_states + (b * nh + h) * (int64_t)(P * N);
+#pragma unroll
+  for (int v = 0; v < 16; ++v) f[elem(v)] = st[v];
 }
 
 // ------------------------------------------------------------------------------------
@@ -1324,24 +1509,6 @@ __global__ __launch_bounds__(256) void ssd_group_grad_kernel(
 // The copies count as vector-memory loads of the requesting wave and complete in order; a wave waits
 // until only the copies of the head after the current one are outstanding, then passes the barrier.
 // ------------------------------------------------------------------------------------
-typedef __attribute__((address_space(3))) void lds_void_t;
-
-// 64 lanes x 16 bytes from global memory into LDS: lane l's piece lands at lds_base + 16 * l
-// (lds_base is the same for the whole wave).  Written as assembly so that the compiler does not
-// make every later LDS read wait for all copies under way; the caller waits for the counter.
-__device__ __forceinline__ void copy16_to_lds(const void* g, void* lds_base) {
-  const unsigned lds = (unsigned)(uintptr_t)(lds_void_t*)lds_base;
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds) : "memory", "m0");
-}
-
-// The same with the address split into a base that is the same for the whole wave (scalar registers)
-// and a byte offset per lane: a loop that only moves the base spends no vector instructions on addresses.
-__device__ __forceinline__ void copy16_to_lds(const void* base, unsigned lane_offset, void* lds_base) {
-  const unsigned lds = (unsigned)(uintptr_t)(lds_void_t*)lds_base;
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base), "s"(lds)
-               : "memory", "m0");
-}
-
 struct GroupDmaSmem {
   static constexpr int R = 3;  // heads in LDS
   static constexpr int kState = 64 * 128 * (int)sizeof(bf16_t), kRows = 64 * 64 * (int)sizeof(bf16_t), kVec = 2048;
