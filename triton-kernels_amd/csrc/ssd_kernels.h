@@ -137,20 +137,25 @@ struct Tile {
 // order with its other loads and stores.
 typedef __attribute__((address_space(3))) void lds_void_t;
 
-// 64 lanes x 16 bytes from global memory into LDS: lane l's piece lands at lds_base + 16 * l
-// (lds_base is the same for the whole wave).  Written as assembly so that the compiler does not
-// make every later LDS read wait for all copies under way; the caller waits for the counter.
-__device__ __forceinline__ void copy16_to_lds(const void* g, void* lds_base) {
-  const unsigned lds = (unsigned)(uintptr_t)(lds_void_t*)lds_base;
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds) : "memory", "m0");
-}
-
-// The same with the address split into a base that is the same for the whole wave (scalar registers)
-// and a byte offset per lane: a loop that only moves the base spends no vector instructions on addresses.
+// 64 lanes x 16 bytes from global memory into LDS: lane l's piece, at base + lane_offset bytes, lands at
+// lds_base + 16 * l.  base and lds_base are the same for the whole wave (scalar registers), so a loop that only
+// moves the base spends no vector instructions on addresses.  Written as assembly so that the compiler does
+// not make every later LDS read wait for all copies under way (given the builtin it does, whatever the
+// addresses); the caller waits for the counter (s_waitcnt vmcnt) and passes a barrier before another wave
+// reads the data.  m0, which carries the LDS address, is put back, so the compiler need not know that it
+// changes; five wait states precede the load because its scalar base may just have been written by vector
+// instructions (v_readfirstlane), which the compiler cannot see from outside the assembly.
 __device__ __forceinline__ void copy16_to_lds(const void* base, unsigned lane_offset, void* lds_base) {
   const unsigned lds = (unsigned)(uintptr_t)(lds_void_t*)lds_base;
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base), "s"(lds)
-               : "memory", "m0");
+  const uint64_t wide = reinterpret_cast<uint64_t>(base);
+  const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(wide >> 32));
+  const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)wide);  // (unsigned: no sign extension below)
+  base = reinterpret_cast<const void*>(((uint64_t)hi << 32) | (uint64_t)lo);
+  unsigned keep;
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b32 m0, %0"
+               : "=&s"(keep)
+               : "v"(lane_offset), "s"(base), "s"(lds)
+               : "memory");
 }
 
 __device__ __forceinline__ void zero_acc(floatx16& a) {
