@@ -72,6 +72,8 @@ def test_dstates_db_dc_vs_oracle(b, L, nh, P, g, N, Q, dtype, device):
     if dtype == BF16:  # gradient states already in bfloat16: the product rounds them there either way
         dB16, ddA16 = _chunk_state_bwd_db(d(x), d(dt), d(dA_cs), d(dstates).to(BF16), B=d(B), ngroups=g)
         assert torch.equal(dB16, dB) and torch.equal(ddA16, ddA)
+        dB16n = _chunk_state_bwd_db(d(x), d(dt), d(dA_cs), d(dstates).to(BF16), ngroups=g)  # no B: no row sums asked for
+        assert torch.equal(dB16n if not isinstance(dB16n, tuple) else dB16n[0], dB)
 
     dC_ref, ddAp_ref = S.chunk_scan_bwd_dC(prev, dA_cs, dout, C=C, ngroups=g, round_to=rt)
     dC, ddAp = _chunk_scan_bwd_dC(d(prev), d(dA_cs), d(dout), C=d(C), ngroups=g)
@@ -80,6 +82,8 @@ def test_dstates_db_dc_vs_oracle(b, L, nh, P, g, N, Q, dtype, device):
     if dtype == BF16:  # carried states already in bfloat16: the product rounds them there either way
         dC16, ddAp16 = _chunk_scan_bwd_dC(d(prev).to(BF16), d(dA_cs), d(dout), C=d(C), ngroups=g)
         assert torch.equal(dC16, dC) and torch.equal(ddAp16, ddAp)
+        dC16n = _chunk_scan_bwd_dC(d(prev).to(BF16), d(dA_cs), d(dout), ngroups=g)  # no C: no row sums asked for
+        assert torch.equal(dC16n if not isinstance(dC16n, tuple) else dC16n[0], dC)
 
 
 @pytest.mark.parametrize("has_init", [False, True])
