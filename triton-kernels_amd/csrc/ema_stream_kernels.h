@@ -273,7 +273,10 @@ __global__ __launch_bounds__(kRowDotThreads) void row_dot_kernel(const T* __rest
   const float* vp = vec + chunk_id * Tdim;
   const T* xp = x + b * sx.sb + h * sx.sh + (int64_t)c * Q * sx.sl;
 
-  constexpr int R = 8;
+  // rows per wave and turn.  Measured at b16 nh2 d1024 L4096 chunk 128 (db / dc, us): 8 rows 50 / 49, 4 rows
+  // 47.5 / 47, 2 rows 44.7 / 44.5, 1 row 47.7 / 47.5, 16 rows 58 / 56: fewer registers per wave keep more waves
+  // resident, and two 16-byte loads per lane and column step are enough to cover the latency with them.
+  constexpr int R = 2;
   for (int m0 = wave * R; m0 < Q; m0 += NWV * R) {
     float acc[R];
 #pragma unroll
