@@ -232,6 +232,8 @@ WALK_CASES = [
     (3, 64, 2, 64, 1, 128, 64),     # one stage in all
     (1, 50, 2, 64, 1, 64, 64),      # less than one stage
     (1, 8256, 1, 64, 1, 128, 256),  # 129 stages: rounds of the ring and a remainder
+    (1, 640, 2, 64, 1, 128, 64),    # every stage begins a chunk (the state stores of two chunks in the queue at a time)
+    (2, 1000, 2, 64, 2, 128, 128),  # two stages per chunk, last chunk and last stage ragged
 ]
 
 
