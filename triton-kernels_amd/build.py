@@ -48,5 +48,13 @@ def build(verbose: bool = True, extra_flags=(), out: str = OUT) -> str:
     return out
 
 
+# Development build with per-tile phase timestamps in the single-pass kernels (what
+# `bench.py --stage tile_phases` loads); never the library the operators use.
+TIMING_OUT = os.path.join(HERE, "lib", "libema_hip_timing.so")
+
+
 if __name__ == "__main__":
-    build()
+    if "--timing" in sys.argv[1:]:
+        build(extra_flags=["-DEMA_TIMING"], out=TIMING_OUT)
+    else:
+        build()

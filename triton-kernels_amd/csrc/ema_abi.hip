@@ -338,6 +338,10 @@ struct TileF32 {
   static constexpr int BWD_CPL = 2, BWD_RPL = 8, BWD_MINW = 4;
 };
 
+inline TileOrder make_order(const Dims& di, int ntiles) {
+  return tile_order_make((unsigned)di.batch, (unsigned)di.nh, (unsigned)di.C, (unsigned)ntiles);
+}
+
 // ready: the chained part of the workspace is as a zero fill or an earlier call left it;
 // otherwise it is cleared first.
 template <typename T, typename S, bool XP>
@@ -355,7 +359,8 @@ int launch_fwd_tile_t(const void* x, SeqStrides sx, const float* A, SeqStrides s
   const int64_t cap = resident_blocks(kernel, NT, 0);
   EMA_TRY(launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x,
                        sx, A, sa, (T*)y, sy, prev128, prev_coarse, ratio, fin, init, w.hdr, w.decw, w.status,
-                       (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total));
+                       (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols, (int)total,
+                       make_order(di, ntiles)));
   return launched();
 }
 
@@ -376,7 +381,7 @@ int launch_bwd_tile_k(const void* x, SeqStrides sx, const void* dy, SeqStrides s
   EMA_TRY(launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x,
                        sx, (const T*)dy, sd, A, sa, prev128, (T*)dx, sdx, (T*)y, sy, part, dfinal, dinit, w.hdr,
                        w.decw, w.status, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols,
-                       (int)total));
+                       (int)total, make_order(di, ntiles)));
   return launched();
 }
 

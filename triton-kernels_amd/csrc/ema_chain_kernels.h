@@ -123,24 +123,59 @@ __global__ __launch_bounds__(256) void chain_clear_kernel(uint4* __restrict__ p,
   if (i < n16) p[i] = make_uint4(0u, 0u, 0u, 0u);
 }
 
+// n / d for n < 2^31 by a multiplication: m = ceil(2^(31 + l) / d), l = ceil(log2 d), fits 32 bits
+// and floor(n * m / 2^(31 + l)) is exact for n < 2^31 (the error term n * (m * d - 2^(31 + l)) stays
+// below 2^(31 + l)).  d = 1 is encoded as m = 0.
+struct FastDiv {
+  unsigned m, sh;
+};
+inline FastDiv fast_div_make(unsigned d) {
+  FastDiv f{0u, 0u};
+  if (d <= 1u) return f;
+  unsigned l = 0;
+  while ((1ull << l) < d) ++l;
+  const unsigned long long num = 1ull << (31 + l);
+  f.m = (unsigned)((num + d - 1) / d);
+  f.sh = l - 1;
+  return f;
+}
+__device__ __forceinline__ unsigned fast_div(unsigned n, FastDiv f) {
+  return f.m ? (__umulhi(n, f.m) >> f.sh) : n;
+}
+
+// Tickets are handed out in chunk-major order: all sequences and column tiles of chunk 0, then
+// chunk 1, ... (REV: the chunks from last to first), so a tile's predecessor always has a smaller
+// ticket.  Within a chunk: batch element, head, column tile.  TileOrder holds the reciprocals that
+// turn a ticket into its tile without divisions.
+struct TileOrder {
+  unsigned cols;    // tiles per chunk: sequences * column tiles
+  unsigned C;       // chunks
+  unsigned ntiles, nh;
+  FastDiv dcols, dnt, dnh;
+};
+inline TileOrder tile_order_make(unsigned B, unsigned nh, unsigned C, unsigned ntiles) {
+  TileOrder o;
+  o.cols = B * nh * ntiles, o.C = C, o.ntiles = ntiles, o.nh = nh;
+  o.dcols = fast_div_make(o.cols), o.dnt = fast_div_make(ntiles), o.dnh = fast_div_make(nh);
+  return o;
+}
+
 struct ChainTile {
   int c, ctile, limit, col0, n, b, h, chunk_id, col_id;  // col_id = n * ntiles + ctile
 };
 
-// Ticket -> tile, chunk-major; REV runs the chunks from last to first.  All quantities fit
-// 32 bits (the host checks N * C * ntiles < 2^31).
+// Ticket -> tile.  All quantities fit 32 bits (the host checks N * C * ntiles < 2^31).
 template <bool REV, int BN>
-__device__ __forceinline__ ChainTile chain_decode(int ticket, int cols, int ntiles, int C, int nh,
-                                                  int L) {
+__device__ __forceinline__ ChainTile chain_decode(int ticket, const TileOrder& o, int L) {
   ChainTile t;
-  const unsigned cc = (unsigned)ticket / (unsigned)cols;
-  t.c = REV ? C - 1 - (int)cc : (int)cc;
-  t.col_id = ticket - (int)cc * cols;
-  t.n = (int)((unsigned)t.col_id / (unsigned)ntiles);
-  t.ctile = t.col_id - t.n * ntiles;
-  t.b = (int)((unsigned)t.n / (unsigned)nh);
-  t.h = t.n - t.b * nh;
-  t.chunk_id = t.n * C + t.c;
+  const unsigned cc = fast_div((unsigned)ticket, o.dcols);
+  t.c = REV ? (int)o.C - 1 - (int)cc : (int)cc;
+  t.col_id = ticket - (int)(cc * o.cols);
+  t.n = (int)fast_div((unsigned)t.col_id, o.dnt);
+  t.ctile = t.col_id - t.n * (int)o.ntiles;
+  t.b = (int)fast_div((unsigned)t.n, o.dnh);
+  t.h = t.n - t.b * (int)o.nh;
+  t.chunk_id = t.n * (int)o.C + t.c;
   t.limit = min(kTileRows, L - t.c * kTileRows);
   t.col0 = t.ctile * BN;
   return t;

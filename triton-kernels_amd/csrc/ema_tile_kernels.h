@@ -37,31 +37,41 @@
 namespace ema {
 
 #ifdef EMA_TIMING
-// Development builds only: thread 0 keeps up to 8 timestamps per tile in registers and writes them
-// out when the tile is finished, so that taking a stamp waits for nothing.
+// Development builds only: one thread per role keeps up to 8 timestamps per tile in registers and
+// writes them out when the tile is finished, so that taking a stamp waits for nothing.  A tile has
+// 16 slots in the buffer: 0..7 for thread 0 of the workgroup, 8..15 for the thread `EMA_TS_ROW`
+// (the first thread of a wave that only owns rows, where a kernel has such waves).
 #define EMA_TSTAMP_DECL long long ema_ts[8] = {0, 0, 0, 0, 0, 0, 0, 0}
-#define EMA_TSTAMP(slot)                               \
-  do {                                                 \
-    if (threadIdx.x == 0) ema_ts[slot] = wall_clock64(); \
+#define EMA_TSTAMP_T(tid, slot)                            \
+  do {                                                     \
+    if (threadIdx.x == (tid)) ema_ts[slot] = wall_clock64(); \
   } while (0)
-#define EMA_TSTAMP_VALUE(slot, v)       \
-  do {                                  \
+#define EMA_TSTAMP(slot) EMA_TSTAMP_T(0, slot)
+#define EMA_TSTAMP_VALUE(slot, v)             \
+  do {                                        \
     if (threadIdx.x == 0) ema_ts[slot] = (v); \
   } while (0)
-#define EMA_TSTAMP_FLUSH                                                    \
-  do {                                                                      \
-    if (threadIdx.x == 0 && g_ema_timing)                                   \
-      for (int q = 0; q < 8; ++q) g_ema_timing[(int64_t)cur * 8 + q] = ema_ts[q]; \
+#define EMA_TSTAMP_FLUSH_T(tid, base)                                                  \
+  do {                                                                                 \
+    if (threadIdx.x == (tid) && g_ema_timing)                                          \
+      for (int q = 0; q < 8; ++q) g_ema_timing[(int64_t)cur * 16 + (base) + q] = ema_ts[q]; \
   } while (0)
+#define EMA_TSTAMP_FLUSH EMA_TSTAMP_FLUSH_T(0, 0)
 #else
 #define EMA_TSTAMP_DECL \
   do {                  \
+  } while (0)
+#define EMA_TSTAMP_T(tid, slot) \
+  do {                          \
   } while (0)
 #define EMA_TSTAMP(slot) \
   do {                   \
   } while (0)
 #define EMA_TSTAMP_VALUE(slot, v) \
   do {                            \
+  } while (0)
+#define EMA_TSTAMP_FLUSH_T(tid, base) \
+  do {                                \
   } while (0)
 #define EMA_TSTAMP_FLUSH \
   do {                   \
@@ -268,7 +278,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
     T* __restrict__ y, SeqStrides sy, float* __restrict__ prev, float* __restrict__ prev_coarse, int ratio,
     float* __restrict__ final_state, const float* __restrict__ init, ChainHeader* __restrict__ hdr,
     u64* __restrict__ decw, u64* __restrict__ status, int nh, int L, int Tdim, int C, int ntiles, int cols,
-    int total) {
+    int total, const TileOrder ord) {
   using W = TileCfg<T, CPL, RPL>;
   constexpr int BN = W::BN, NW = W::NW, NG = W::NG;
   __shared__ __attribute__((aligned(16))) float sS[2][NG][BN];  // group states, double-buffered by tile
@@ -304,7 +314,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
     tile_coef_load<RPL>(araw, A + (int64_t)tt.b * sa.sb + (int64_t)tt.h * sa.sh +
                                   ((int64_t)tt.c * kTileRows + RPL * grp) * sa.sl, sa.sl, aa.nrows);
   };
-  ChainTile t = chain_decode<false, BN>(cur < total ? cur : 0, cols, ntiles, C, nh, L);
+  ChainTile t = chain_decode<false, BN>(cur < total ? cur : 0, ord, L);
   TileAt at = tile_at<RPL>(t.limit, grp, t.col0 + lane * CPL < Tdim);
   if (cur < total) request(rowsA, arawA, t, at);
 
@@ -313,12 +323,14 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
     int future = 0;
     if (threadIdx.x == 0) future = (int)atomicAdd(&hdr->ticket, 1u);
     const bool more = nxt < total;
-    const ChainTile tn = chain_decode<false, BN>(more ? nxt : 0, cols, ntiles, C, nh, L);
+    const ChainTile tn = chain_decode<false, BN>(more ? nxt : 0, ord, L);
     const TileAt atn = tile_at<RPL>(tn.limit, grp, tn.col0 + lane * CPL < Tdim);
     EMA_TSTAMP_DECL;
     EMA_TSTAMP(0);
+    EMA_TSTAMP_VALUE(7, (long long)blockIdx.x);
     float a[RPL];
     tile_decays<RPL, XP>(a, araw);
+    EMA_TSTAMP(5);
     // 1. local pass
     float s[CPL];
     float D = 1.f;
@@ -437,7 +449,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     SeqStrides sdx, T* __restrict__ y, SeqStrides sy, float* __restrict__ part,
     const float* __restrict__ dfinal, float* __restrict__ dinit, ChainHeader* __restrict__ hdr,
     u64* __restrict__ decw, u64* __restrict__ status, int nh, int L, int Tdim, int C, int ntiles, int cols,
-    int total) {
+    int total, const TileOrder ord) {
   using W = TileCfg<T, CPL, RPL>;
   constexpr int BN = W::BN, NW = W::NW, NG = W::NG, NT = W::NT;
   static_assert(2 * BN <= NT, "one thread per column and direction");
@@ -459,7 +471,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
   RowWords<NW> dr[RPL], xr[RPL];
   float araw[RPL];
   float p_in = 0.f;
-  ChainTile t = chain_decode<true, BN>(cur < total ? cur : 0, cols, ntiles, C, nh, L);
+  ChainTile t = chain_decode<true, BN>(cur < total ? cur : 0, ord, L);
   TileAt at = tile_at<RPL>(t.limit, grp, t.col0 + lane * CPL < Tdim);
   if (cur < total) {
     const int64_t row0 = (int64_t)t.c * kTileRows + RPL * grp;
@@ -477,10 +489,12 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     if (threadIdx.x == 0) future = (int)atomicAdd(&hdr->ticket, 1u);
     EMA_TSTAMP_DECL;
     EMA_TSTAMP(0);
+    EMA_TSTAMP_VALUE(7, (long long)blockIdx.x);
     const int64_t row0 = (int64_t)t.c * kTileRows + RPL * grp;
     // a: factor of the state per row; pc: the row's coefficient as tile_step takes it
     float a[RPL], pc[RPL];
     tile_decays<RPL, XP>(pc, araw);
+    EMA_TSTAMP(5);
 #pragma unroll
     for (int i = 0; i < RPL; ++i) a[i] = tile_keep<XP>(pc[i]);
 
@@ -579,6 +593,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
       float h_in;
       if (!last && EMA_EXP == 0) h_in = look.finish(words, dws, C, ctl);
       else h_in = (dfinal && last && t.col0 + k < Tdim) ? dfinal[(int64_t)t.n * Tdim + t.col0 + k] : 0.f;
+      EMA_TSTAMP(6);
       const float h_out = fmaf(dec, h_in, loc);
       if (EMA_EXP != 4) chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStatePrefix, h_out);
       if (dinit && t.c == 0 && t.col0 + k < Tdim) dinit[(int64_t)t.n * Tdim + t.col0 + k] = h_out;
@@ -592,7 +607,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     // same rows of the next tile are requested
     const int next = s_ticket[slot];
     const bool more = next < total;
-    const ChainTile tn = chain_decode<true, BN>(more ? next : 0, cols, ntiles, C, nh, L);
+    const ChainTile tn = chain_decode<true, BN>(more ? next : 0, ord, L);
     const TileAt atn = tile_at<RPL>(tn.limit, grp, tn.col0 + lane * CPL < Tdim);
     {
       T* g = dx + (int64_t)t.b * sdx.sb + (int64_t)t.h * sdx.sh + row0 * sdx.sl + t.col0 + off;

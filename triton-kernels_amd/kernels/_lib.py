@@ -188,18 +188,28 @@ def f32c(t: torch.Tensor) -> torch.Tensor:
 # Workspace of the single-pass entry points.  The library tags every word it writes to the
 # chained part of a workspace with the epoch of the call, so a buffer that was zero-filled once
 # serves every later call without being cleared (workspace_ready = 1: the call is the tile kernel
-# alone).  The wrappers keep one such buffer per device and problem shape (the chained part is
-# laid out by (sequences, 128-row tiles, dim), and only tagged words may ever be written there),
-# shared by the forward and the backward of that shape.  Calls that share a buffer must not
-# overlap in time: code that runs these operators on several streams of one device at once
-# switches to a fresh buffer per call with private_workspaces(True), at the price of one small
-# clearing launch per call.
+# alone).  Two calls that overlap in time must not share a buffer (they would draw tiles from one
+# ticket counter), so the wrappers keep one buffer per (device, stream, problem shape): calls on
+# one stream are ordered, calls on different streams get different buffers.  A buffer is created
+# at the largest size any entry point needs for its shape with chunk sizes that are multiples of
+# 128, and never grows or moves afterwards; a call that needs more (the staged forward with a
+# small chunk size, which does not use the chained part) gets a buffer of its own.  Buffers handed
+# out while a HIP graph is being captured are pinned: the graph holds their address, so they are
+# never dropped.  private_workspaces(True) switches to a fresh, cleared buffer per call.
 # ---------------------------------------------------------------------------------------------
 HEADER_BYTES = 256
 _RECLEAR_AFTER = 1 << 29  # calls; the epoch tag wraps at 2**30
-_MAX_SHARED = 16          # buffers kept (the least recently created goes first)
+_MAX_SHARED = 16          # unpinned buffers kept (the least recently created goes first)
 
-_shared = {}  # (device index, N, tiles, dim) -> [buffer, calls since the last clear]
+
+class _Shared:
+    __slots__ = ("buf", "calls", "pinned")
+
+    def __init__(self, buf):
+        self.buf, self.calls, self.pinned = buf, 0, False
+
+
+_shared = {}  # (device index, stream, N, tiles, dim) -> _Shared
 _private = False
 
 
@@ -213,29 +223,39 @@ def _clear(buf: torch.Tensor, dev: torch.device) -> None:
         check(lib().ema_workspace_clear(buf.data_ptr(), buf.numel(), stream_ptr(dev)), "ema_workspace_clear")
 
 
+def _shared_bytes(batch: int, nh: int, L: int, T: int) -> int:
+    """Largest workspace of the four single-pass entry points for this shape (chunk 128)."""
+    h = lib()
+    return max(h.ema_fwd_workspace_bytes(batch, nh, L, T, 128), h.ema_bwd_workspace_bytes(batch, nh, L, T, 128),
+               h.ema_seq_fwd_workspace_bytes(batch, nh, L, T), h.ema_seq_bwd_workspace_bytes(batch, nh, L, T))
+
+
 def workspace(dev: torch.device, nbytes: int, batch: int, nh: int, L: int, T: int):
-    """(uint8 buffer of at least nbytes, workspace_ready flag) for one call on `dev` of a
-    single-pass entry point on a (batch, L, nh, T) problem."""
+    """(uint8 buffer of at least nbytes, workspace_ready flag) for one call on the current
+    stream of `dev` of a single-pass entry point on a (batch, L, nh, T) problem."""
     assert nbytes > 0, "unsupported shape"
     capturing = torch.cuda.is_current_stream_capturing()
-    key = (dev.index, batch * nh, -(-L // 128), T)
+    key = (dev.index, stream_ptr(dev), batch * nh, -(-L // 128), T)
     entry = _shared.get(key)
-    fits = entry is not None and entry[0].numel() >= nbytes
-    if _private or (capturing and not fits):
-        # under graph capture nothing persistent may be created: the call clears what it uses
+    if _private or (entry is None and capturing) or (entry is not None and entry.buf.numel() < nbytes):
+        # under capture nothing persistent may be created; an oversized request is served apart
         return torch.empty(nbytes, dtype=torch.uint8, device=dev), 0
-    if not fits:
-        size = max(nbytes, 0 if entry is None else entry[0].numel())
-        _shared.pop(key, None)
-        while len(_shared) >= _MAX_SHARED:
-            _shared.pop(next(iter(_shared)))
-        entry = _shared[key] = [torch.empty(size, dtype=torch.uint8, device=dev), 0]
-        _clear(entry[0], dev)
-    elif entry[1] >= _RECLEAR_AFTER and not capturing:
-        _clear(entry[0], dev)
-        entry[1] = 0
-    entry[1] += 1
-    return entry[0], 1
+    if entry is None:
+        size = _shared_bytes(batch, nh, L, T)
+        if size < nbytes:
+            return torch.empty(nbytes, dtype=torch.uint8, device=dev), 0
+        unpinned = [k for k, e in _shared.items() if not e.pinned]
+        for k in unpinned[: max(0, len(unpinned) - _MAX_SHARED + 1)]:
+            del _shared[k]
+        entry = _shared[key] = _Shared(torch.empty(size, dtype=torch.uint8, device=dev))
+        _clear(entry.buf, dev)
+    elif entry.calls >= _RECLEAR_AFTER and not capturing:
+        _clear(entry.buf, dev)
+        entry.calls = 0
+    if capturing:
+        entry.pinned = True
+    entry.calls += 1
+    return entry.buf, 1
 
 
 def chain_error(buf: torch.Tensor) -> bool:
@@ -251,9 +271,12 @@ def check_chain_errors(device=None) -> None:
         index = key[0]
         if device is not None and torch.device(device).index not in (None, index):
             continue
-        if chain_error(entry[0]):
-            _clear(entry[0], entry[0].device)
-            entry[1] = 0
+        if chain_error(entry.buf):
+            # the buffer belongs to another stream, maybe: nothing may be in flight while it is cleared
+            torch.cuda.synchronize(entry.buf.device)
+            _clear(entry.buf, entry.buf.device)
+            torch.cuda.synchronize(entry.buf.device)
+            entry.calls = 0
             raise RuntimeError(
                 f"EMA chained scan on cuda:{index}: a tile gave up waiting for its predecessor; the "
                 "results of that call are NaN (overlapping calls on one workspace, or a workspace "
