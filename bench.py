@@ -200,15 +200,24 @@ class EmaRun:
         A.grad = None
         self._apply(A, x, self.Q).backward(dy)
 
-    def fwd_only(self, i, events=None):
+    def fwd_only(self, i, events=None, workspace=None):
         x, A, dy = self.sets[i % len(self.sets)]
-        return self._fwd(A, x, kernel_events=events)
+        return self._fwd(A, x, kernel_events=events, workspace=workspace)
 
-    def bwd_saved(self, i, events=None):  # backward as the autograd step runs it, with the forward's states
+    def bwd_saved(self, i, events=None, workspace=None):  # backward as the autograd step runs it, with the forward's states
         if self._saved is None:
             self._saved = [self._fwd(A, x)[2] for x, A, dy in self.sets]
         x, A, dy = self.sets[i % len(self.sets)]
-        return self._bwd(dy, x, A, self._saved[i % len(self.sets)], kernel_events=events)
+        return self._bwd(dy, x, A, self._saved[i % len(self.sets)], kernel_events=events, workspace=workspace)
+
+    def ready_workspace(self):
+        """A zero-filled workspace of the caller's own (passed as ready): what code that captures
+        its step into a HIP graph creates once before the capture, so that the graph holds no
+        clearing launches."""
+        from kernels import _lib
+
+        n = _lib.lib().ema_seq_bwd_workspace_bytes(self.b, self.nh, self.L, self.T)
+        return (self.torch.zeros(n, dtype=self.torch.uint8, device=self.dev), 1)
 
     def step_kernels(self, iters):
         """The same two launches per step as `step` makes (sequence-level forward, then backward
@@ -351,6 +360,21 @@ def make_stages(sets, Q, torch):
 
     stages["stream_copy"] = lambda i: stream(i, False)
     stages["stream_2in_1out"] = lambda i: stream(i, True)
+
+    # the same bytes in the access pattern of the single-pass kernels (tiles of 128 rows x 512
+    # bytes, persistent workgroups): with the row order a scanning wave needs, and with the one the
+    # memory system likes best
+    def tile_copy(i, rowmap):
+        x, A, dy = sets[i % len(sets)]
+        o = outs[i % len(sets)]
+        b, L, nh, d = x.shape
+        _lib.check(_lib.lib().ema_tile_pattern_copy(x.data_ptr(), o.data_ptr(), b, L, nh * d * x.element_size(), rowmap,
+                                                    _lib.stream_ptr(x.device)), "ema_tile_pattern_copy")
+
+    x0 = sets[0][0]
+    if x0.shape[1] % 128 == 0 and (x0.shape[2] * x0.shape[3] * x0.element_size()) % 512 == 0:
+        stages["tile_copy_scan_order"] = lambda i: tile_copy(i, 0)
+        stages["tile_copy_best_order"] = lambda i: tile_copy(i, 1)
     return stages
 
 
@@ -361,7 +385,8 @@ def time_stages(sets, Q, iters, torch, only=None):
     x = sets[0][0]
     N, L, T = x.shape[0] * x.shape[2], x.shape[1], x.shape[3]
     xb = x.numel() * x.element_size()
-    ab = dict(algorithmic_bytes(N, L, T, Q, 2), copy=2 * xb, stream_copy=2 * xb, stream_2in_1out=3 * xb)
+    ab = dict(algorithmic_bytes(N, L, T, Q, 2), copy=2 * xb, stream_copy=2 * xb, stream_2in_1out=3 * xb,
+              tile_copy_scan_order=2 * xb, tile_copy_best_order=2 * xb)
     res = {}
     for name, fn in stages.items():
         if only and name not in only:
@@ -441,7 +466,6 @@ def ssd_stages(torch, steps, warmup, only=None):
         "chunk_scan": lambda i: _chunk_scan_fwd(pick(i)[9], pick(i)[0], pick(i)[5], pick(i)[6], pick(i)[4], pick(i)[8]),
         "forward": lambda i: _mamba_chunk_scan_combined_fwd(*pick(i)[:5], Q),
         # the same with everything behind the cumsum in one kernel (all intermediates on chip)
-        "forward_one_kernel": lambda i: _mamba_chunk_scan_combined_fwd(*pick(i)[:5], Q, single_kernel=True),
         # backward stages (the reference has no combined backward): x dt A B C | dt_out dA st states cb dout dprev dstates
         "bwd_dstates": lambda i: _chunk_scan_bwd_dstates(pick(i)[4], pick(i)[6], pick(i)[10]),
         "bwd_state_passing": lambda i: _state_passing_bwd(pick(i)[8].view(b, C, nh, P * N), pick(i)[6][..., -1],
@@ -464,7 +488,7 @@ def ssd_stages(torch, steps, warmup, only=None):
         "chunk_cumsum": 3 * dtb, "chunk_state": xb + bc + 2 * dtb + stb, "state_passing": stb + pvb + dtb // Q,
         "chunk_state_passing": xb + bc + 2 * dtb + pvb,
         "bmm_chunk": 2 * bc + cbb, "chunk_scan": cbb + 2 * xb + bc + pvb + 2 * dtb,
-        "forward": 2 * xb + 2 * bc + dtb, "forward_one_kernel": 2 * xb + 2 * bc + dtb,
+        "forward": 2 * xb + 2 * bc + dtb,
         "bwd_dstates": xb + bc + dtb + pvb, "bwd_state_passing": 3 * pvb + 2 * dtb // Q,
         "bwd_db": xb + pvb + 2 * dtb + bc + 2 * bc + dtb, "bwd_dc": xb + pvb + dtb + bc + 2 * bc + dtb,
         "bwd_dx": cbb + 3 * xb + bc + pvb + 3 * dtb, "bwd_ddAcs": 2 * xb + 3 * dtb + cbb,
@@ -695,10 +719,12 @@ def main():
     try:
         run.bwd_saved(0)
         graphs, keep = [], []
+        ws = run.ready_workspace()  # the graphs replay one after the other on one stream: one buffer serves all
+        torch.cuda.synchronize()
         for k in range(len(run.sets)):
             gr = torch.cuda.CUDAGraph()
             with torch.cuda.graph(gr):
-                keep.append((run.fwd_only(k), run.bwd_saved(k)))
+                keep.append((run.fwd_only(k, workspace=ws), run.bwd_saved(k, workspace=ws)))
             graphs.append(gr)
         for i in range(args.warmup):
             graphs[i % len(graphs)].replay()
@@ -790,7 +816,6 @@ def main():
         s5 = ssd_stages(torch, max(10, args.steps // 2), 3)
         cfgs["cfg5"] = {"workload": "Mamba-2 SSD b8 nh32 hdim64 dstate128 g1 L8192 chunk256, bf16",
                         "forward_ms": s5["forward"]["ms"],
-                        "forward_one_kernel_ms": s5["forward_one_kernel"]["ms"],
                         # the combined forward runs chunk_cumsum, chunk_state_passing (chunk_state and
                         # state_passing in one kernel), bmm_chunk and chunk_scan
                         "forward_stages_ms": {k: s5[k]["ms"] for k in ("chunk_cumsum", "chunk_state", "state_passing",

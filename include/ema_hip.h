@@ -101,6 +101,17 @@ int ema_workspace_clear(void* workspace, size_t bytes, void* stream);
  * kernels' rates are reported. */
 int ema_stream_copy(const void* a, const void* b, void* dst, size_t bytes, void* stream);
 
+/* Measurement aid (no counterpart in the reference): copies a (slabs, rows, row_bytes) byte tensor
+ * (rows a multiple of 128, row_bytes a multiple of 512) in the access pattern of the single-pass
+ * kernels: persistent workgroups, tiles of 128 rows x 512 bytes in chunk-major order, 8 bytes per
+ * lane and row.  rowmap 0: a wave moves 16 consecutive rows of a tile, as a wave that scans down
+ * the rows has to; rowmap 1: the rows of a wave are 8 apart and slabs are rotated against each
+ * other, which is the order the memory system sustains the highest rate for.  bench.py reports
+ * both next to the plain streaming copy: the first is the ceiling of the scan kernels' own
+ * pattern. */
+int ema_tile_pattern_copy(const void* src, void* dst, int64_t slabs, int64_t rows, int64_t row_bytes,
+                          int rowmap, void* stream);
+
 /* Largest chunk size accepted by every entry point. */
 #define EMA_MAX_CHUNK 1024
 

@@ -99,33 +99,6 @@ int ssd_chunk_state_passing_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64
                                 float* final_states, int64_t batch, int64_t seqlen, int64_t nheads,
                                 int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk, void* stream);
 
-/* The forward behind ssd_chunk_cumsum_fwd in ONE kernel: chunk states, state passing, C B^T and the
- * chunk scan.  A workgroup per (batch, head) walks the sequence in 64-row stages with the state in
- * float32 registers, so neither the chunk-local states nor the carried states nor C B^T go through
- * memory: x, B, C (and z) are read once, out is written once.  Arguments as for the four entry points
- * it stands for: x, z, out (and out_x, dense like out, may be NULL unless z is given and the caller
- * wants the ungated result) are (batch, seqlen, nheads, hdim), B and C (batch, seqlen, ngroups, dstate),
- * dt and dA_cumsum (batch, nheads, nchunks, chunk) float32 from ssd_chunk_cumsum_fwd, D (nheads) or
- * (nheads, hdim) float32 or NULL, initial (batch, nheads, hdim, dstate) float32 or NULL.  states
- * (batch, nchunks, nheads, hdim, dstate), float32 or of the inputs' type (states_dtype), receives the
- * state entering each chunk, final_states (batch, nheads, hdim, dstate) float32 the last one.  The
- * operands of the products are rounded to the input type where the staged entry points round them,
- * per 64-row stage instead of per chunk: results agree with the staged path to rounding, not bit for
- * bit.  bfloat16 inputs, hdim 64, dstate 64 or 128, chunk a multiple of 64, no packed batches
- * (SSD_ERR_UNSUPPORTED otherwise: run the staged entry points).
- * Replaces, run back to back, _chunk_state_fwd (kernels/mamba_kernels/mamba_state_fwd.py:138-169),
- * _state_passing_fwd (mamba_state_pass.py:84-115), _bmm_chunk_fwd (mamba_bmm.py:80) and
- * _chunk_scan_fwd (mamba_scan_fwd.py:162); the reference's own single-kernel forward is
- * kernels/mamba_3_kernels/mamba_ssd_fwd.py:247-258 (one program per head and batch element walking
- * the chunks). */
-int ssd_fused_fwd(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, const void* B, int64_t b_sb,
-                  int64_t b_sl, int64_t b_sg, const void* C, int64_t c_sb, int64_t c_sl, int64_t c_sg,
-                  const void* z, int64_t z_sb, int64_t z_sl, int64_t z_sh, int dtype, const float* dt,
-                  const float* dA_cumsum, const float* D, int d_has_hdim, const float* initial, void* out,
-                  int64_t o_sb, int64_t o_sl, int64_t o_sh, void* out_x, void* states, int states_dtype,
-                  float* final_states, int64_t batch, int64_t seqlen, int64_t nheads, int64_t ngroups,
-                  int64_t hdim, int64_t dstate, int64_t chunk, void* stream);
-
 /* out[b,c,g,m,k] = sum_n a[b,cQ+m,g,n] * bm[b,cQ+k,g,n]; rows past seqlen are zero.  out is
  * float32 or `dtype` (out_dtype).  With seq_idx, out[m,k] = 0 where the ids of m and k differ
  * (mamba_bmm.py:70-73).  Replaces _bmm_chunk_fwd, kernels/mamba_kernels/mamba_bmm.py:88-126

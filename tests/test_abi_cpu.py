@@ -122,15 +122,11 @@ def test_ssd_validation_happens_before_any_launch():
     assert handle.ssd_state_passing_fwd(fake, fake, 2, 1, 1, None, fake, 7, fake, 1, 1, 2, 8, *ids, 0, 0, None) == -4
     # carried states are float32 or of the inputs' type: bfloat16 states with float32 inputs are refused
     assert handle.ssd_chunk_scan_bwd_dc(*seq, 0, fake, fake, 1, *grp, fake, fake, 1, 64, 2, 1, 64, 64, 64, *ids, None) == -4
-    # the fused forward entries: chunk sizes off the 64-row stages, float32 inputs and head size 128 go to the staged entries
+    # the fused chunk-state + state-passing entry: chunk sizes off the 64-row stages, float32 inputs and head size 128 go to the staged entries
     walk = lambda dtype, chunk, out_dtype=0: handle.ssd_chunk_state_passing_fwd(
         *grp, *seq, dtype, fake, fake, None, fake, out_dtype, fake, 1, 64, 2, 1, 64, 64, chunk, None)
     assert walk(0, 48) == -5 and walk(1, 64, 9) == -4 and walk(1, 0) == -2
     assert handle.ssd_chunk_state_passing_fwd(*grp, *seq, 1, None, fake, None, fake, 1, fake, 1, 64, 2, 1, 64, 64, 64, None) == -1
-    one = lambda dtype, hdim, chunk, out=fake: handle.ssd_fused_fwd(
-        *seq, *grp, *grp, None, 0, 0, 0, dtype, fake, fake, None, 0, None, out, *seq[1:], None, fake, 1, fake,
-        1, 64, 2, 1, hdim, 64, chunk, None)
-    assert one(0, 64, 64) == -5 and one(1, 128, 64) == -5 and one(1, 64, 48) == -5 and one(1, 64, 64, None) == -1
     # a packed batch must come with the chunking that gives nchunks
     assert handle.ssd_state_passing_fwd(fake, fake, 2, 1, 1, None, fake, 0, fake, 1, 2, 2, 8, fake, 64, 1, 64, 16, None) == -2
 

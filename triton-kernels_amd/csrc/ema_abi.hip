@@ -576,6 +576,20 @@ int ema_stream_copy(const void* a, const void* b, void* dst, size_t bytes, void*
   return launched();
 }
 
+int ema_tile_pattern_copy(const void* src, void* dst, int64_t slabs, int64_t rows, int64_t row_bytes, int rowmap,
+                          void* stream) {
+  if (!src || !dst) return EMA_ERR_NULL;
+  if (slabs <= 0 || rows <= 0 || row_bytes <= 0 || rows % 128 || row_bytes % 512) return EMA_ERR_SHAPE;
+  if (reinterpret_cast<uintptr_t>(src) % 16 || reinterpret_cast<uintptr_t>(dst) % 16) return EMA_ERR_ALIGN;
+  const int64_t pieces = row_bytes / 512, tiles = slabs * (rows / 128) * pieces;
+  if (tiles > 0x7fffffff || slabs > 0x7fffffff / pieces) return EMA_ERR_SHAPE;
+  const int64_t cap = resident_blocks(tile_copy_kernel, 512, 0);
+  hipLaunchKernelGGL(tile_copy_kernel, dim3((unsigned)(tiles < cap ? tiles : cap)), dim3(512), 0, as_stream(stream),
+                     static_cast<const char*>(src), static_cast<char*>(dst), (int)slabs, (int)(rows / 128), (int)pieces,
+                     row_bytes, rows * row_bytes, rowmap ? 1 : 0);
+  return launched();
+}
+
 int ema_workspace_clear(void* workspace, size_t bytes, void* stream) {
   EMA_TRY(check_f32(workspace));
   return launch_clear(workspace, bytes, as_stream(stream));

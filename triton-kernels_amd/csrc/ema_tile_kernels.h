@@ -88,11 +88,6 @@ namespace ema {
 constexpr bool kStreamFwdLoad = (EMA_STREAM_FLAGS & 1) != 0, kStreamFwdStore = (EMA_STREAM_FLAGS & 2) != 0,
                kStreamBwdLoad = (EMA_STREAM_FLAGS & 4) != 0, kStreamBwdStore = (EMA_STREAM_FLAGS & 8) != 0;
 
-// Development builds only (wrong results, to price the parts of the look-back): 1 no aggregate
-// publish and no polls, 4 nothing published at all.
-#ifndef EMA_EXP
-#define EMA_EXP 0
-#endif
 // Output rows are written through to device memory (1) instead of being left to the L2s' write-back
 // (0).  Measured at b16 nh2 d1024 L4096: forward 112 -> 105 us, step 279 -> 271 us.
 #ifndef EMA_STORE_WT
@@ -371,7 +366,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
         dec *= dg[g];
       }
       float p_in;
-      if (t.c > 0 && EMA_EXP == 0) {
+      if (t.c > 0) {
         if (k == 0) chain_publish(dws + t.c, ctl.epoch, kStateAggregate, dec);
         chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStateAggregate, loc);
         ChainLook<false, BN> look;
@@ -383,7 +378,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
         p_in = (init && t.c == 0 && t.col0 + k < Tdim) ? init[(int64_t)t.n * Tdim + t.col0 + k] : 0.f;
       }
       const float p_out = fmaf(dec, p_in, loc);
-      if (EMA_EXP != 4) chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStatePrefix, p_out);
+      chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStatePrefix, p_out);
       sP[buf][k] = p_in;
       if (t.col0 + k < Tdim) {
         prev[(int64_t)t.chunk_id * Tdim + t.col0 + k] = p_in;
@@ -546,7 +541,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
         loc = fmaf(dg[g], loc, rg[g]);
         dec *= dg[g];
       }
-      if (!last && EMA_EXP == 0) {
+      if (!last) {
         if (k == 0) chain_publish(dws + t.c, ctl.epoch, kStateAggregate, dec);
         chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStateAggregate, loc);
         look.begin(words, t.c);
@@ -591,11 +586,11 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     if (threadIdx.x < BN) {
       const int k = threadIdx.x;
       float h_in;
-      if (!last && EMA_EXP == 0) h_in = look.finish(words, dws, C, ctl);
+      if (!last) h_in = look.finish(words, dws, C, ctl);
       else h_in = (dfinal && last && t.col0 + k < Tdim) ? dfinal[(int64_t)t.n * Tdim + t.col0 + k] : 0.f;
       EMA_TSTAMP(6);
       const float h_out = fmaf(dec, h_in, loc);
-      if (EMA_EXP != 4) chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStatePrefix, h_out);
+      chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStatePrefix, h_out);
       if (dinit && t.c == 0 && t.col0 + k < Tdim) dinit[(int64_t)t.n * Tdim + t.col0 + k] = h_out;
       sH[buf][k] = h_in;
     }

@@ -349,34 +349,6 @@ int launch_bmm(const void* a, Strides3 sa, const void* bm, Strides3 sb, void* ou
 
 }  // namespace
 
-template <int N, typename TS, bool HAS_Z>
-static int launch_fused_fwd_z(const void* x, Strides3 sx, const void* B, Strides3 sB, const void* C, Strides3 sC,
-                              const void* z, Strides3 sz, const float* dt, const float* dA, const float* D,
-                              int d_has_hdim, const float* initial, void* out, Strides3 so, void* out_x, void* states,
-                              float* final_states, const Dims& d, hipStream_t st) {
-  auto kernel = ssd_fused_fwd_kernel<bf16_t, N, TS, HAS_Z>;
-  constexpr int smem = FusedSmem<bf16_t, N>::kBytes;
-  static_assert(smem <= kLdsBytes, "the stage tiles must fit the LDS of a compute unit");
-  SSD_TRY(allow_smem(kernel, smem));
-  hipLaunchKernelGGL(kernel, dim3((unsigned)(d.batch * d.nh)), dim3(512), smem, st, (const bf16_t*)x, sx,
-                     (const bf16_t*)B, sB, (const bf16_t*)C, sC, (const bf16_t*)z, sz, dt, dA, D, d_has_hdim, initial,
-                     (bf16_t*)out, so, (bf16_t*)out_x, (TS*)states, final_states, (int)d.nh, (int)(d.nh / d.g),
-                     (int)d.L, (int)d.Q, (int)d.C);
-  return launched();
-}
-
-template <int N, typename TS>
-static int launch_fused_fwd(const void* x, Strides3 sx, const void* B, Strides3 sB, const void* C, Strides3 sC,
-                            const void* z, Strides3 sz, const float* dt, const float* dA, const float* D,
-                            int d_has_hdim, const float* initial, void* out, Strides3 so, void* out_x, void* states,
-                            float* final_states, const Dims& d, hipStream_t st) {
-  if (z)
-    return launch_fused_fwd_z<N, TS, true>(x, sx, B, sB, C, sC, z, sz, dt, dA, D, d_has_hdim, initial, out, so, out_x,
-                                           states, final_states, d, st);
-  return launch_fused_fwd_z<N, TS, false>(x, sx, B, sB, C, sC, z, sz, dt, dA, D, d_has_hdim, initial, out, so, out_x,
-                                          states, final_states, d, st);
-}
-
 extern "C" {
 
 int ssd_chunk_cumsum_fwd(const void* dt, int dt_dtype, int64_t dt_sb, int64_t dt_sl, int64_t dt_sh,
@@ -445,41 +417,6 @@ int ssd_chunk_state_passing_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64
   return dispatch_tpn(dtype, hdim, dstate,
                       WalkLaunch{x, B, Strides3{x_sb, x_sl, x_sh}, Strides3{b_sb, b_sl, b_sg}, dt, dA_cumsum, initial,
                                  out, out_dtype, final_states, d, as_stream(stream)});
-}
-
-int ssd_fused_fwd(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, const void* B, int64_t b_sb,
-                  int64_t b_sl, int64_t b_sg, const void* C, int64_t c_sb, int64_t c_sl, int64_t c_sg,
-                  const void* z, int64_t z_sb, int64_t z_sl, int64_t z_sh, int dtype, const float* dt,
-                  const float* dA_cumsum, const float* D, int d_has_hdim, const float* initial, void* out,
-                  int64_t o_sb, int64_t o_sl, int64_t o_sh, void* out_x, void* states, int states_dtype,
-                  float* final_states, int64_t batch, int64_t seqlen, int64_t nheads, int64_t ngroups,
-                  int64_t hdim, int64_t dstate, int64_t chunk, void* stream) {
-  Dims d;
-  SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
-  SSD_TRY(check_dtype(dtype));
-  SSD_TRY(check_dtype(states_dtype));
-  if (dtype != SSD_BF16 || hdim != 64 || !dim_ok(dstate) || chunk % 64) return SSD_ERR_UNSUPPORTED;
-  SSD_TRY(check_vec(x, x_sb, x_sl, x_sh, dtype, hdim));
-  SSD_TRY(check_vec(out, o_sb, o_sl, o_sh, dtype, hdim));
-  SSD_TRY(check_vec(B, b_sb, b_sl, b_sg, dtype, dstate));
-  SSD_TRY(check_vec(C, c_sb, c_sl, c_sg, dtype, dstate));
-  if (z) SSD_TRY(check_vec(z, z_sb, z_sl, z_sh, dtype, hdim));
-  if (out_x && reinterpret_cast<uintptr_t>(out_x) % 16) return SSD_ERR_ALIGN;
-  if (!dt || !dA_cumsum) return SSD_ERR_NULL;
-  SSD_TRY(check_f32(states));
-  SSD_TRY(check_f32(final_states));
-  if (initial) SSD_TRY(check_f32(initial));
-  const Strides3 sx{x_sb, x_sl, x_sh}, sB{b_sb, b_sl, b_sg}, sC{c_sb, c_sl, c_sg}, sz{z_sb, z_sl, z_sh};
-  const Strides3 so{o_sb, o_sl, o_sh};
-  hipStream_t st = as_stream(stream);
-#define SSD_FUSED(NN)                                                                                           \
-  (states_dtype == SSD_BF16                                                                                     \
-       ? launch_fused_fwd<NN, bf16_t>(x, sx, B, sB, C, sC, z, sz, dt, dA_cumsum, D, d_has_hdim, initial, out, so,  \
-                                      out_x, states, final_states, d, st)                                       \
-       : launch_fused_fwd<NN, float>(x, sx, B, sB, C, sC, z, sz, dt, dA_cumsum, D, d_has_hdim, initial, out, so,   \
-                                     out_x, states, final_states, d, st))
-  return dstate == 64 ? SSD_FUSED(64) : SSD_FUSED(128);
-#undef SSD_FUSED
 }
 
 int ssd_state_passing_fwd(const float* states, const float* dA_chunk, int64_t da_sb, int64_t da_sh,

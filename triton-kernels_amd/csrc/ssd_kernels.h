@@ -582,9 +582,6 @@ __global__ __launch_bounds__(256) void ssd_state_passing_kernel(
 // multiple of 64 (a stage lies inside one chunk).  dt and dA_cs are (b, nh, C, Q), so position r of
 // the sequence sits at offset r of the (b, h) row whatever the chunk.  No packed batches.
 // ------------------------------------------------------------------------------------
-#ifndef SSD_WALK_DIAG  // diagnostic builds (wrong results on purpose): 1 no state stores, 2 no products, 3 neither LDS stores nor products
-#define SSD_WALK_DIAG 0
-#endif
 template <typename T, int P, int NL>
 struct WalkSmem {
   static constexpr int KT = 64, PX = Tile<T>::kpitch(P), PB = Tile<T>::kpitch(NL);
@@ -643,8 +640,8 @@ __global__ __launch_bounds__(256, NSPLIT) void ssd_state_walk_kernel(
 #ifndef SSD_WALK_XNT
 #define SSD_WALK_XNT true
 #endif
-    if (SSD_WALK_DIAG != 4) rx.template load<SSD_WALK_XNT>(xg, sx.sl, row0, L, tid);
-    if (SSD_WALK_DIAG != 5) rb.template load<false, true>(Bg, sB.sl, row0, L, tid, dAb, dtb);
+    rx.template load<SSD_WALK_XNT>(xg, sx.sl, row0, L, tid);
+    rb.template load<false, true>(Bg, sB.sl, row0, L, tid, dAb, dtb);
   };
 #pragma unroll
   for (int u = 0; u < D; ++u) request(px[u], pb[u], u);
@@ -673,31 +670,20 @@ __global__ __launch_bounds__(256, NSPLIT) void ssd_state_walk_kernel(
       dal = dal_next;
       dal_next = dAb[(int64_t)min(c + 1, C - 1) * Q + Q - 1];
       TO* o = out + ((b * C + c) * nh + h) * (int64_t)(P * N);
-      if (SSD_WALK_DIAG != 1 || c == 0) {
 #pragma unroll
-        for (int i = 0; i < BPW; ++i)
+      for (int i = 0; i < BPW; ++i)
 #pragma unroll
-          for (int v = 0; v < 16; ++v) __builtin_nontemporal_store((TO)st[i][v], o + elem(i, v));
-      }
+        for (int v = 0; v < 16; ++v) __builtin_nontemporal_store((TO)st[i][v], o + elem(i, v));
     }
     T* xb = lds + (g & 1) * S::kStageElems;
     T* bb = xb + KT * PX;
     const float dA_last = dal;
-    if (SSD_WALK_DIAG < 3) {
-      rx.store(xb, row0, L, tid, NoScale());
-      rb.store(bb, row0, L, tid, [&](int, float dA_k, float dt_k) { return __expf(fminf(dA_last - dA_k, 0.f)) * dt_k; });
-    } else {  // the rows must still arrive
-#pragma unroll
-      for (int i = 0; i < RowPieces<T, KT, P, S::PX>::CNT; ++i)
-        if (SSD_WALK_DIAG != 4) acc[0][0] += rx.v[i].get(0);
-#pragma unroll
-      for (int i = 0; i < RowPieces<T, KT, NL, S::PB>::CNT; ++i)
-        if (SSD_WALK_DIAG != 5) acc[0][1] += rb.v[i].get(0) + rb.a0[i] + rb.a1[i];
-    }
+    rx.store(xb, row0, L, tid, NoScale());
+    rb.store(bb, row0, L, tid, [&](int, float dA_k, float dt_k) { return __expf(fminf(dA_last - dA_k, 0.f)) * dt_k; });
     __syncthreads();
     request(rx, rb, g + D);
 #pragma unroll
-    for (int kk = 0; kk < (SSD_WALK_DIAG >= 2 ? 0 : KT); kk += KG) {
+    for (int kk = 0; kk < KT; kk += KG) {
 #pragma unroll
       for (int i = 0; i < BPW; ++i) {
         const int j = wave + 4 * i, mi = j % MB, ni = j / MB;
@@ -891,329 +877,6 @@ __global__ __launch_bounds__(512) void ssd_state_walk_dma_kernel(
   float* f = final_states + (b * nh + h) * (int64_t)(P * N);
 #pragma unroll
   for (int v = 0; v < 16; ++v) f[elem(v)] = st[v];
-}
-
-// ------------------------------------------------------------------------------------
-// The whole forward behind the cumsum in one pass (hdim 64): one workgroup of 8 waves per (b, h)
-// walks the sequence in stages of 64 rows and carries the (64 x dstate) state in float32
-// registers, so neither chunk-local states nor carried states nor C B^T go through memory.  Per
-// stage, with a_k the chunk's running sum of dA at position k, a_0 the sum before the stage and a_e
-// at its last row:
-//   out[m] = exp(a_m - a_0) * C_m . S  +  sum_{k <= m} (C_m . B_k) exp(min(a_m - a_k, 0)) dt_k x_k  +  D x_m
-//   S     <- exp(a_e - a_0) * S  +  sum_k exp(a_e - a_k) dt_k  x_k (x) B_k
-// which is the state-space recurrence itself, regrouped; the state entering each chunk of Q rows
-// is written out as the staged path writes it (Q a multiple of 64).  The operands of the products
-// are rounded to the input type where the staged kernels round them (carried state, weighted
-// C B^T), here per stage instead of per chunk, and the weight of the state update sits on x
-// instead of B: results agree with the staged path to rounding, not bit for bit.
-//
-// Work of a stage over the waves: the 64 x 64 output is four 32 x 32 blocks; two waves share a
-// block and split the state dimension between them (each forms C . S and its 32-row band of
-// C B^T over half of dstate, weights its partial band, multiplies it with x; the two partial
-// outputs meet in the output pass).  The state's 32 x 32 blocks go one to a wave.  The two waves
-// that a SIMD holds work on the upper and the lower band, whose causal work differs by half.
-// Two barriers per stage; the rows of the next D stages are in flight in registers.
-// No packed batches.
-// ------------------------------------------------------------------------------------
-#ifndef SSD_FUSED_DIAG  // diagnostic builds (wrong results on purpose): 1 no C.S / C B^T products, 2 no band, 3 no causal product, 4 no state update, 5 no output pass, 6 no loads past the first
-#define SSD_FUSED_DIAG 0
-#endif
-template <typename T, int N>
-struct FusedSmem {
-  static constexpr int P = 64, KT = 64, NT = 512, EPL = Vec16<T>::N;
-  static constexpr int PX = Tile<T>::pitch(P), PB = Tile<T>::pitch(N), PW = Tile<T>::pitch(32), PO = P + 4;
-  // the carried state is kept as St[n][p] and a wave's band of C B^T as W[k][m]: the accumulator
-  // layout gives a lane four consecutive rows of one column, which are adjacent that way
-  static constexpr int oXr = 0, oXw = oXr + KT * PX, oB = oXw + KT * PX, oC = oB + KT * PB, oS = oC + KT * PB,
-                       oW = oS + N * PX, kElems = oW + 8 * KT * PW;
-  static constexpr int kOutBytes = 2 * KT * PO * (int)sizeof(float);
-  static constexpr int kBytes = kElems * (int)sizeof(T) + kOutBytes + 4 * KT * (int)sizeof(float);
-};
-
-// The rows of a 64-row stage as 16-byte pieces over NT threads (RowPieces for another thread count).
-template <typename T, int COLS, int NT>
-struct StagePieces {
-  static constexpr int EPL = Vec16<T>::N, VPR = COLS / EPL, CNT = 64 * VPR / NT;
-  static_assert((64 * VPR) % NT == 0, "tile must split evenly over the threads");
-  Vec16<T> v[CNT];
-  template <bool STREAM>
-  __device__ __forceinline__ void load(const T* __restrict__ g, int64_t row_stride, int row0, int limit, int tid) {
-#pragma unroll
-    for (int i = 0; i < CNT; ++i) {
-      const int idx = tid + NT * i;
-      const int row = min(row0 + idx / VPR, limit - 1);
-      const T* src = g + (int64_t)row * row_stride + (idx % VPR) * EPL;
-      v[i] = STREAM ? load16_stream(src) : load16(src);
-    }
-  }
-  // rows at or past limit are stored as zeros; scale(r) multiplies row r of the stage
-  template <typename F>
-  __device__ __forceinline__ void store(T* tile, int row0, int limit, int tid, F scale) const {
-    constexpr int PT = Tile<T>::pitch(COLS);
-#pragma unroll
-    for (int i = 0; i < CNT; ++i) {
-      const int idx = tid + NT * i;
-      const int r = idx / VPR, cv = (idx % VPR) * EPL;
-      Vec16<T> w = v[i];
-      if constexpr (!std::is_same<F, NoScale>::value) {
-        const float sc = scale(r);
-        float t[EPL];
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) t[e] = w.get(e) * sc;
-        w.set_all(t);
-      }
-      if (row0 + r >= limit) w.zero();
-      store16(tile + r * PT + cv, w);
-    }
-  }
-};
-
-template <typename T, int N, typename TS, bool HAS_Z>
-__global__ __launch_bounds__(512) void ssd_fused_fwd_kernel(
-    const T* __restrict__ x, Strides3 sx, const T* __restrict__ B, Strides3 sB, const T* __restrict__ Cm, Strides3 sC,
-    const T* __restrict__ z, Strides3 sz, const float* __restrict__ dt, const float* __restrict__ dA_cs,
-    const float* __restrict__ Dv, int d_has_hdim, const float* __restrict__ initial, T* __restrict__ out, Strides3 so,
-    T* __restrict__ out_x, TS* __restrict__ states, float* __restrict__ final_states, int nh, int heads_per_group,
-    int L, int Q, int C) {
-  using S = FusedSmem<T, N>;
-  constexpr int P = S::P, KT = S::KT, NT = S::NT, EPL = S::EPL, KG = Tile<T>::KG;
-  constexpr int PX = S::PX, PB = S::PB, PW = S::PW, PO = S::PO;
-  constexpr int MB = P / 32, NBLK = N / 32;  // state blocks: MB x NBLK, one per wave (the first MB * NBLK waves)
-  constexpr int NH = N / 2;                 // the half of dstate a wave contracts over
-#ifdef SSD_FUSED_D
-  constexpr int D = SSD_FUSED_D;
-#else
-  constexpr int D = 1;  // stages in flight (two spill)
-#endif
-  static_assert(MB * NBLK <= 8 && NH % KG == 0, "one state block per wave");
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  T* lds = reinterpret_cast<T*>(smem);
-  T *Xr = lds + S::oXr, *Xw = lds + S::oXw, *Bt = lds + S::oB, *Ct = lds + S::oC, *St = lds + S::oS;
-  float* Os = reinterpret_cast<float*>(smem + S::kElems * sizeof(T));  // [2][KT][PO]: one partial output per half
-  float* dAs = Os + 2 * KT * PO;
-  float* dts = dAs + KT;
-  float* sms = dts + KT;  // exp(a_m - a_0): the scale of row m's C . S
-  float* fgs = sms + KT;  // rows 0..31: exp(a_31 - a_k) dt_k; rows 32..63: exp(a_m - a_31)
-  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31;
-  T* Wr = lds + S::oW + wave * KT * PW;
-  const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
-  const int h = bid % nh;
-  const int64_t b = bid / nh;
-  const int g = h / heads_per_group;
-  const float* dAb = dA_cs + (b * nh + h) * (int64_t)C * Q;
-  const float* dtb = dt + (b * nh + h) * (int64_t)C * Q;
-  const T* xg = x + b * sx.sb + h * sx.sh;
-  const T* Bg = B + b * sB.sb + g * sB.sh;
-  const T* Cg = Cm + b * sC.sb + g * sC.sh;
-  const T* zg = HAS_Z ? z + b * sz.sb + h * sz.sh : nullptr;
-  const int G = (L + KT - 1) / KT;
-  const int mi = wave >> 2;        // 32-row band of the stage this wave works on
-  const int pcb = (wave >> 1) & 1; // its 32-column block of the output
-  const int half = wave & 1;       // its half of dstate
-  const bool owns = wave < MB * NBLK;  // this wave keeps a block of the state:
-  const int bm = wave % MB, bn = wave / MB;  // rows 32 bm .. of p, columns 32 bn .. of n
-
-  auto selem = [&](int v) { return (32 * bm + acc_row(v, lane)) * N + 32 * bn + l32; };
-  // four consecutive components of an accumulator (rows r .. r + 3 of one column) as one piece
-  auto pack4 = [&](const floatx16& a, int q) {
-    typedef float f32x2 __attribute__((ext_vector_type(2)));
-    typedef bf16_t b16x2 __attribute__((ext_vector_type(2)));
-    const b16x2 lo = __builtin_convertvector((f32x2){a[4 * q], a[4 * q + 1]}, b16x2);
-    const b16x2 hi = __builtin_convertvector((f32x2){a[4 * q + 2], a[4 * q + 3]}, b16x2);
-    ema::bf16x4 r;
-    r[0] = lo[0], r[1] = lo[1], r[2] = hi[0], r[3] = hi[1];
-    return r;
-  };
-
-  // Every request is unconditional (a load inside a branch would have to complete before the next
-  // is issued): stages past the end are requested again as the last one and never used.
-  StagePieces<T, P, NT> px[D], pz[HAS_Z ? D : 1];
-  StagePieces<T, N, NT> pb[D], pc[D];
-  float pa[D], pt[D], dae[D], dam[D];  // a_k and dt_k of this thread's row; a_e and a_31 of the stage
-  const int vrow = tid >> 3;  // the row whose a_k, dt_k this thread brings (threads 8 r .. 8 r + 7 the same)
-  auto request = [&](int u, int gq) {
-    const int row0 = min(gq, G - 1) * KT;
-    px[u].template load<true>(xg, sx.sl, row0, L, tid);
-    pb[u].template load<false>(Bg, sB.sl, row0, L, tid);
-    pc[u].template load<false>(Cg, sC.sl, row0, L, tid);
-    if constexpr (HAS_Z) pz[u].template load<true>(zg, sz.sl, row0, L, tid);
-    const int r = min(row0 + vrow, L - 1);
-    pa[u] = dAb[r];
-    pt[u] = dtb[r];
-    dae[u] = dAb[min(row0 + KT - 1, L - 1)];
-    dam[u] = dAb[min(row0 + 31, L - 1)];
-  };
-#pragma unroll
-  for (int u = 0; u < D; ++u) request(u, u);
-
-  floatx16 st;
-  zero_acc(st);
-  if (initial && owns) {
-    const float* ini = initial + (b * nh + h) * (int64_t)(P * N);
-#pragma unroll
-    for (int v = 0; v < 16; ++v) st[v] = ini[selem(v)];
-  }
-  float a0 = 0.f;  // a_0 of the stage: the running sum at the last row of the stage before, 0 at a chunk's start
-
-  // FULL: every row of the stage lies inside the sequence, so that its stores are unconditional
-  // and the waits for rows requested before them can count them.  (Loads and stores of a wave
-  // complete in order; a store the compiler cannot count makes every later wait for a load wait
-  // for the store as well.)
-  auto stage = [&](int u, int gq, auto full_tag) {
-    constexpr bool FULL = decltype(full_tag)::value;
-    const int row0 = gq * KT;
-    const int c = row0 / Q, k0 = row0 - c * Q;
-    if (k0 == 0) a0 = 0.f;
-    const float ae = dae[u], a31 = dam[u];
-    // 1. the carried state, rounded, for the C . S product
-    if (owns) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q)  // rows p = 32 bm + 8 q + 4 (lane / 32) .. + 3 of column n = 32 bn + l32
-        *reinterpret_cast<ema::bf16x4*>(St + (32 * bn + l32) * PX + 32 * bm + 8 * q + 4 * (lane >> 5)) = pack4(st, q);
-    }
-    // 2. the stage's rows: x as it is and weighted for the state update, B, C, and the vectors of the weights
-    if ((tid & 7) == 0) {
-      // Below the diagonal block the weight of (m, k) splits at row 31, the last of k's block:
-      // exp(a_m - a_31) per row times exp(a_31 - a_k) dt_k per column, both exponents <= 0 for
-      // sums that fall along the chunk (each is clamped like the whole is).
-      const float ar = pa[u], tr = pt[u];
-      dAs[vrow] = ar;
-      dts[vrow] = tr;
-      sms[vrow] = __expf(fminf(ar - a0, 0.f));
-      fgs[vrow] = vrow < 32 ? __expf(fminf(a31 - ar, 0.f)) * tr : __expf(fminf(ar - a31, 0.f));
-    }
-    px[u].store(Xr, row0, L, tid, NoScale());
-    {
-      // x has 8 pieces to a row: the rows of this thread's pieces are vrow (NT / 8 = 64 rows, one piece each)
-      static_assert(StagePieces<T, P, NT>::CNT == 1 && StagePieces<T, P, NT>::VPR == 8, "one piece of x per thread");
-      const float wx = __expf(fminf(ae - pa[u], 0.f)) * pt[u];
-      px[u].store(Xw, row0, L, tid, [&](int) { return wx; });
-    }
-    pb[u].store(Bt, row0, L, tid, NoScale());
-    pc[u].store(Ct, row0, L, tid, NoScale());
-    Vec16<T> zrow;
-    if constexpr (HAS_Z) zrow = pz[u].v[0];
-    __syncthreads();
-    if (k0 == 0 && owns) {  // the state entering the chunk (st is untouched until step 6)
-      TS* o = states + ((b * C + c) * nh + h) * (int64_t)(P * N);
-#pragma unroll
-      for (int v = 0; v < 16; ++v) __builtin_nontemporal_store((TS)st[v], o + selem(v));
-    }
-    if (SSD_FUSED_DIAG != 6) request(u, gq + D);
-
-    // 3. C . S and this wave's band of C B^T over its half of dstate; they share the fragments of C
-    floatx16 acc, cb[2];
-    zero_acc(acc);
-    zero_acc(cb[0]);
-    zero_acc(cb[1]);
-#pragma unroll
-    for (int n0 = 0; n0 < (SSD_FUSED_DIAG == 1 ? 0 : NH); n0 += KG) {
-      const int nn = half * NH + n0;
-      const Vec16<T> a = frag_rows(Ct, PB, 32 * mi, nn, lane);
-      mma_group(a, frag_cols(St, PX, nn, 32 * pcb, lane), acc);
-      mma_group(a, frag_rows(Bt, PB, 0, nn, lane), cb[0]);
-      if (mi) mma_group(a, frag_rows(Bt, PB, 32, nn, lane), cb[1]);
-    }
-    asm volatile("" ::: "memory");  // keeps the phases apart: reads hoisted across them cost registers
-    if (SSD_FUSED_DIAG != 2) {
-      if (mi) {  // the block below the diagonal one: a factor per row times a factor per column
-        const float gk = fgs[l32];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) cb[0][v] *= fgs[32 + acc_row(v, lane)] * gk;
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-          *reinterpret_cast<ema::bf16x4*>(Wr + l32 * PW + 8 * q + 4 * (lane >> 5)) = pack4(cb[0], q);
-      }
-      {  // the diagonal block: the exact weight, masked
-        floatx16& cd = cb[mi ? 1 : 0];
-        const int k = 32 * mi + l32;
-        const float ak = dAs[k], tk = dts[k];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int m = 32 * mi + acc_row(v, lane);
-          const float f = cd[v] * __expf(fminf(dAs[m] - ak, 0.f)) * tk;
-          cd[v] = k > m ? 0.f : f;
-        }
-#pragma unroll
-        for (int q = 0; q < 4; ++q)  // rows m = 8 q + 4 (lane / 32) .. + 3 of the band, column k
-          *reinterpret_cast<ema::bf16x4*>(Wr + k * PW + 8 * q + 4 * (lane >> 5)) = pack4(cd, q);
-      }
-    }
-    asm volatile("" ::: "memory");  // keeps the phases apart: reads hoisted across them cost registers
-    // 4. the C . S part takes the decay from the stage's start to its row
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] *= sms[32 * mi + acc_row(v, lane)];
-    // the wave's own writes of its band are visible to its own reads once the LDS counter has drained
-    __builtin_amdgcn_s_waitcnt(0xc07f);
-    // 5. the causal product with x, and the skip term once
-    for (int kk = 0; kk < (SSD_FUSED_DIAG == 3 ? 0 : 32 * (mi + 1)); kk += KG)
-      mma_group(frag_cols(Wr, PW, kk, 0, lane), frag_cols(Xr, PX, kk, 32 * pcb, lane), acc);
-    if (Dv && half == 0) {
-      const int col = 32 * pcb + l32;
-      const float dv = d_has_hdim ? Dv[h * P + col] : Dv[h];
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[v] = fmaf(dv, (float)Xr[(32 * mi + acc_row(v, lane)) * PX + col], acc[v]);
-    }
-    asm volatile("" ::: "memory");  // keeps the phases apart: reads hoisted across them cost registers
-    // 6. the state after the stage
-    if (owns) {
-      const float dec = __expf(fminf(ae - a0, 0.f));
-#pragma unroll
-      for (int v = 0; v < 16; ++v) st[v] *= dec;
-#pragma unroll
-      for (int kk = 0; kk < (SSD_FUSED_DIAG == 4 ? 0 : KT); kk += KG)
-        mma_group(frag_cols(Xw, PX, kk, 32 * bm, lane), frag_cols(Bt, PB, kk, 32 * bn, lane), st);
-    }
-    a0 = ae;
-    asm volatile("" ::: "memory");  // keeps the phases apart: reads hoisted across them cost registers
-    // 7. the two partial outputs of a block meet in the output pass, which moves 16-byte pieces
-    {
-      float* mine = Os + half * KT * PO;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) mine[(32 * mi + acc_row(v, lane)) * PO + 32 * pcb + l32] = acc[v];
-    }
-    __syncthreads();
-    if (SSD_FUSED_DIAG != 5) {
-      constexpr int VPR = P / EPL;
-      static_assert(KT * VPR == NT, "one piece of the output per thread");
-      const int r = tid / VPR, cv = (tid % VPR) * EPL;
-      const int64_t pos = (int64_t)row0 + r;
-      if (FULL || pos < L) {
-        float vv[EPL];
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) vv[e] = Os[r * PO + cv + e] + Os[KT * PO + r * PO + cv + e];
-        Vec16<T> o;
-        if constexpr (HAS_Z) {
-          if (out_x) {
-            o.set_all(vv);
-            store16(out_x + b * so.sb + pos * so.sl + h * so.sh + cv, o);
-          }
-#pragma unroll
-          for (int e = 0; e < EPL; ++e) {
-            const float zf = zrow.get(e);
-            vv[e] *= zf / (1.f + __expf(-zf));
-          }
-        }
-        o.set_all(vv);
-        store16_stream(out + b * so.sb + pos * so.sl + h * so.sh + cv, o);
-      }
-    }
-  };
-  const int Gfull = L / KT;  // stages that lie inside the sequence
-  int g0 = 0;
-  for (; g0 + D <= Gfull; g0 += D) {
-#pragma unroll
-    for (int u = 0; u < D; ++u) stage(u, g0 + u, std::true_type());
-  }
-  // what is left: fewer than D whole stages and at most one ragged one
-#pragma unroll
-  for (int u = 0; u < D; ++u)
-    if (g0 + u < G) stage(u, g0 + u, std::false_type());
-  if (owns) {
-    float* f = final_states + (b * nh + h) * (int64_t)(P * N);
-#pragma unroll
-    for (int v = 0; v < 16; ++v) f[selem(v)] = st[v];
-  }
 }
 
 // Sum over the 32 lanes of each half of a wave (lanes 0..31 and 32..63 apart), left in lanes 31

@@ -49,50 +49,9 @@ def _chunk_state_passing_fwd(B, x, dt, dA_cumsum, initial_states=None, out_dtype
     return states, final_states
 
 
-def _fused_fwd(x, dt_out, dA_cumsum, B, C, chunk_size, D=None, z=None, initial_states=None):
-    """Everything behind the cumsum as one kernel (chunk states, state passing, C B^T, chunk scan:
-    kernels/mamba_kernels/mamba_state_fwd.py:138, mamba_state_pass.py:84, mamba_bmm.py:80,
-    mamba_scan_fwd.py:162 of the reference), or None where that kernel does not apply.  Returns
-    (out, out_x, states, final_states) as the four launchers give them; the values agree with theirs
-    to rounding (the products round their operands per 64-row stage instead of per chunk)."""
-    batch, seqlen, nheads, headdim = x.shape
-    _, _, ngroups, dstate = B.shape
-    bf16 = torch.bfloat16
-    if (chunk_size % 64 or headdim != 64 or dstate not in (64, 128) or x.dtype != bf16 or B.dtype != bf16
-            or C.dtype != bf16 or (z is not None and z.dtype != bf16)):
-        return None
-    dev = _lib.require_gpu(x, B, C, dt_out, dA_cumsum)
-    nchunks = dt_out.shape[2]
-    x, xs = _lib.strided4(x)
-    B, bs = _lib.strided4(B)
-    C, cs = _lib.strided4(C)
-    if z is not None:
-        z, zs = _lib.strided4(z)
-    else:
-        zs = (None, 0, 0, 0)
-    dt_f = _lib.f32c(dt_out)
-    dA_f = _lib.f32c(dA_cumsum)
-    Df = None if D is None else _lib.f32c(D)
-    init = None if initial_states is None else _lib.f32c(initial_states)
-    out = torch.empty(batch, seqlen, nheads, headdim, device=dev, dtype=x.dtype)
-    out_x = torch.empty_like(out) if z is not None else None
-    states = torch.empty(batch, nchunks, nheads, headdim, dstate, device=dev, dtype=C.dtype)
-    final_states = torch.empty(batch, nheads, headdim, dstate, device=dev, dtype=torch.float32)
-    with torch.cuda.device(dev):
-        _lib.check(
-            _lib.lib().ssd_fused_fwd(*xs, *bs, *cs, *zs, _lib.dtype_code(x), dt_f.data_ptr(), dA_f.data_ptr(),
-                                     None if Df is None else Df.data_ptr(), int(Df is not None and Df.dim() == 2),
-                                     None if init is None else init.data_ptr(), out.data_ptr(), out.stride(0),
-                                     out.stride(1), out.stride(2), None if out_x is None else out_x.data_ptr(),
-                                     states.data_ptr(), _lib.dtype_code(states), final_states.data_ptr(), batch,
-                                     seqlen, nheads, ngroups, headdim, dstate, chunk_size, _lib.stream_ptr(dev)),
-            "ssd_fused_fwd")
-    return out, out_x, states, final_states
-
-
 def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
                                    initial_states=None, seq_idx=None, cu_seqlens=None, dt_softplus=False,
-                                   dt_limit=(0.0, float("inf")), single_kernel=False):
+                                   dt_limit=(0.0, float("inf"))):
     """Returns (out, out_x, dt_out, dA_cumsum, states, final_states), states (the state entering
     each chunk) in the dtype of C as in kernels/ema_combined.py:48-50, and as a seventh item the state
     at the end of each packed sequence when cu_seqlens is given (batch must be 1 then; the boundaries
@@ -106,14 +65,6 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
         assert initial_states.shape == (batch, nheads, headdim, dstate)
     dA_cumsum, dt_out = _chunk_cumsum_fwd(dt, A, chunk_size, dt_bias=dt_bias, dt_softplus=dt_softplus,
                                           dt_limit=dt_limit)
-    # single_kernel: everything behind the cumsum in one launch where that kernel applies (it keeps all
-    # intermediates on chip; at benchmark configuration 5 it is measured slower than the staged path, so
-    # it is not the default)
-    if single_kernel and seq_idx is None and cu_seqlens is None:
-        whole = _fused_fwd(x, dt_out, dA_cumsum, B, C, chunk_size, D=D, z=z, initial_states=initial_states)
-        if whole is not None:
-            out, out_x, states, final_states = whole
-            return out, out_x, dt_out, dA_cumsum, states, final_states
     fused = None
     if seq_idx is None and C.dtype in (torch.float32, torch.bfloat16):
         fused = _chunk_state_passing_fwd(B, x, dt_out, dA_cumsum, initial_states=initial_states, out_dtype=C.dtype)
