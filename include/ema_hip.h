@@ -360,6 +360,21 @@ int ema_seq_fwd_static(int form, const float* coef, int64_t c_sb, int64_t c_sl, 
                        float* final_state, float* prev128, int64_t batch, int64_t nheads,
                        int64_t seqlen, int64_t dim, void* stream);
 
+/* Companions of ema_seq_fwd_static (no counterpart in the reference either; none of them
+ * allocates).
+ * ema_seq_fwd_static_init: looks up the device address of the array for the current device
+ * (the first look-up on a device may load the code object).  Call it once per device before
+ * ema_seq_fwd_static is captured into a HIP graph, so that nothing but kernel launches happens
+ * under capture; ema_seq_fwd_static itself does the look-up on its first eager call otherwise.
+ * ema_seq_fwd_static_error: copies the sticky error word of the array's chain header to *error
+ * (host memory) after synchronising `stream`: non-zero means that some call since the last reset
+ * gave up a bounded wait and its outputs hold NaN.
+ * ema_seq_fwd_static_reset: zero-fills the array with a kernel on `stream` (the state of a fresh
+ * process); needed after an aborted call or a reported error, never in normal operation. */
+int ema_seq_fwd_static_init(void);
+int ema_seq_fwd_static_error(int* error, void* stream);
+int ema_seq_fwd_static_reset(void* stream);
+
 #ifdef __cplusplus
 }
 #endif

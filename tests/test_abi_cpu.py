@@ -127,6 +127,9 @@ def test_ssd_validation_happens_before_any_launch():
         *grp, *seq, dtype, fake, fake, None, fake, out_dtype, fake, 1, 64, 2, 1, 64, 64, chunk, None)
     assert walk(0, 48) == -5 and walk(1, 64, 9) == -4 and walk(1, 0) == -2
     assert handle.ssd_chunk_state_passing_fwd(*grp, *seq, 1, None, fake, None, fake, 1, fake, 1, 64, 2, 1, 64, 64, 64, None) == -1
+    # dt and the decay sums are fetched in 16-byte pieces by the kernels that copy straight into LDS
+    assert handle.ssd_chunk_state_passing_fwd(*grp, *seq, 1, fake + 4, fake, None, fake, 1, fake, 1, 64, 2, 1, 64, 64, 64, None) == -3
+    assert handle.ssd_chunk_state_passing_fwd(*grp, *seq, 1, fake, fake + 8, None, fake, 1, fake, 1, 64, 2, 1, 64, 64, 64, None) == -3
     # a packed batch must come with the chunking that gives nchunks
     assert handle.ssd_state_passing_fwd(fake, fake, 2, 1, 1, None, fake, 0, fake, 1, 2, 2, 8, fake, 64, 1, 64, 16, None) == -2
 

@@ -78,3 +78,53 @@ def test_static_entry_rejects_what_does_not_fit(device):
     assert st == -7
     with pytest.raises(ValueError):
         _lib.check(st, "ema_seq_fwd_static")
+
+
+def test_static_entry_in_a_hip_graph_and_its_companions(device):
+    """After ema_seq_fwd_static_init nothing but kernel launches happens in a call, so it can be
+    captured; every replay must give the bits of ema_seq_fwd.  The error word reads 0 after normal
+    calls, and a reset leaves the array usable."""
+    import ctypes
+
+    lib = _lib.lib()
+    with torch.cuda.device(device):
+        assert lib.ema_seq_fwd_static_init() == 0
+    b, nh, L, T = 2, 2, 1024, 256
+    x, A, _ = O.make_inputs(b, nh, L, T, seed=51, dtype=torch.bfloat16)
+    xs, As = x.to(device), A.to(device)
+    y = torch.zeros_like(xs)
+    final = torch.zeros(b * nh, T, dtype=torch.float32, device=device)
+    prev128 = torch.zeros(b * nh, L // 128, T, dtype=torch.float32, device=device)
+    _, xa, *_ = _lib.seq_view(xs)
+    _, ya, *_ = _lib.seq_view(y)
+    ca, *_ = _lib.decay_view(As)
+
+    def launch():
+        with torch.cuda.device(device):
+            _lib.check(lib.ema_seq_fwd_static(_lib.EMA_FORM_LOG_DECAY, *ca, *xa, _lib.EMA_BF16, *ya, None,
+                                              final.data_ptr(), prev128.data_ptr(), b, nh, L, T,
+                                              _lib.stream_ptr(device)), "ema_seq_fwd_static")
+
+    announce("ema_seq_fwd_static captured into a graph")
+    launch()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        launch()
+    for rep in range(3):
+        x2, A2, _ = O.make_inputs(b, nh, L, T, seed=60 + rep, dtype=torch.bfloat16)
+        xs.copy_(x2.to(device)); As.copy_(A2.to(device))
+        want = _call("workspace", _lib.EMA_FORM_LOG_DECAY, As, xs, None, device)
+        y.zero_(); final.zero_(); prev128.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, a, w in zip(("y", "final", "prev128"), (y, final, prev128), want):
+            assert torch.equal(a, w), f"replay {rep}: {name} differs from ema_seq_fwd"
+    err = ctypes.c_int(-1)
+    with torch.cuda.device(device):
+        assert lib.ema_seq_fwd_static_error(ctypes.byref(err), _lib.stream_ptr(device)) == 0 and err.value == 0
+        assert lib.ema_seq_fwd_static_error(None, _lib.stream_ptr(device)) == -1
+        assert lib.ema_seq_fwd_static_reset(_lib.stream_ptr(device)) == 0
+    launch()
+    torch.cuda.synchronize()
+    assert torch.equal(y, want[0]), "after a reset the entry point gives the same bits"

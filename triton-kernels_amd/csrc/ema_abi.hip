@@ -936,6 +936,31 @@ int ema_seq_fwd_static(int form, const float* coef, int64_t c_sb, int64_t c_sl, 
                       nullptr);
 }
 
+int ema_seq_fwd_static_init(void) {
+  void* ws = nullptr;
+  return scratch_address(&ws);
+}
+
+int ema_seq_fwd_static_error(int* error, void* stream) {
+  if (!error) return EMA_ERR_NULL;
+  void* ws = nullptr;
+  EMA_TRY(scratch_address(&ws));
+  hipStream_t st = as_stream(stream);
+  unsigned word = 0;
+  const unsigned* src = &static_cast<const ChainHeader*>(ws)->error;
+  if (hipMemcpyAsync(&word, src, sizeof(word), hipMemcpyDeviceToHost, st) != hipSuccess ||
+      hipStreamSynchronize(st) != hipSuccess)
+    return EMA_ERR_LAUNCH;
+  *error = (int)word;
+  return EMA_OK;
+}
+
+int ema_seq_fwd_static_reset(void* stream) {
+  void* ws = nullptr;
+  EMA_TRY(scratch_address(&ws));
+  return launch_clear(ws, kScratchBytes, as_stream(stream));
+}
+
 size_t ema_seq_bwd_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim) {
   Dims d;
   if (check_dims(batch, nheads, seqlen, dim, kTileRows, true, &d) != EMA_OK) return 0;

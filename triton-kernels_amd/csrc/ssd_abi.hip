@@ -37,6 +37,10 @@ int check_f32(const void* p) {
   return reinterpret_cast<uintptr_t>(p) % 16 ? SSD_ERR_ALIGN : SSD_OK;
 }
 
+// The kernels that copy their operands straight into LDS form 32-bit unsigned byte offsets from
+// the strides: tensors addressed with a negative stride go to the register-staged kernels.
+inline bool forward_strides(const Strides3& s) { return s.sb >= 0 && s.sl >= 0 && s.sh >= 0; }
+
 // A carried-state tensor is float32 or of the inputs' type (16-byte aligned either way).
 int check_state(const void* p, int state_dtype, int dtype) {
   if (state_dtype != SSD_F32 && state_dtype != dtype) return SSD_ERR_DTYPE;
@@ -139,7 +143,7 @@ struct WalkLaunch {
 #endif
     // (the kernel keeps the byte offset of a row inside a stage in 32 bits)
     if constexpr (SSD_WALK_DMA && std::is_same<T, bf16_t>::value && P == 64 && N == 128) {
-      if (sx.sl < (int64_t(1) << 24) && sB.sl < (int64_t(1) << 24)) {
+      if (forward_strides(sx) && forward_strides(sB) && sx.sl < (int64_t(1) << 24) && sB.sl < (int64_t(1) << 24)) {
         auto kernel = ssd_state_walk_dma_kernel<TO>;
         constexpr int smem = WalkDmaSmem::kBytes;
         SSD_TRY(allow_smem(kernel, smem));
@@ -304,7 +308,7 @@ struct GroupLaunch {
 #endif
     if constexpr (SSD_GROUP_DMA && std::is_same<T, bf16_t>::value && std::is_same<TS, bf16_t>::value && P == 64 && N == 128) {
       // (the kernel keeps the byte offset of a row inside a chunk in 32 bits)
-      if (d.Q % 64 == 0 && !seq.p && d.Q * sa.sl < (int64_t(1) << 30)) {
+      if (d.Q % 64 == 0 && !seq.p && forward_strides(sa) && forward_strides(sbc) && d.Q * sa.sl < (int64_t(1) << 30)) {
         auto kernel = ssd_group_grad_dma_kernel<MODE>;
         constexpr int smem = GroupDmaSmem::kBytes;
         SSD_TRY(allow_smem(kernel, smem));
@@ -410,7 +414,8 @@ int ssd_chunk_state_passing_fwd(const void* B, int64_t b_sb, int64_t b_sl, int64
   if (!dim_ok(hdim) || !dim_ok(dstate) || chunk % 64) return SSD_ERR_UNSUPPORTED;
   SSD_TRY(check_vec(x, x_sb, x_sl, x_sh, dtype, hdim));
   SSD_TRY(check_vec(B, b_sb, b_sl, b_sg, dtype, dstate));
-  if (!dt || !dA_cumsum) return SSD_ERR_NULL;
+  SSD_TRY(check_f32(dt));  // fetched in 16-byte pieces
+  SSD_TRY(check_f32(dA_cumsum));
   SSD_TRY(check_f32(out));
   SSD_TRY(check_f32(final_states));
   if (initial) SSD_TRY(check_f32(initial));
@@ -599,7 +604,9 @@ int ssd_chunk_state_bwd_db(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_
   SSD_TRY(check_dtype(dtype));
   if (!dim_ok(hdim) || !dim_ok(dstate)) return SSD_ERR_UNSUPPORTED;
   SSD_TRY(check_vec(x, x_sb, x_sl, x_sh, dtype, hdim));
-  if (!dt || !dA_cumsum || !dB) return SSD_ERR_NULL;
+  if (!dB) return SSD_ERR_NULL;
+  SSD_TRY(check_f32(dt));  // fetched in 16-byte pieces
+  SSD_TRY(check_f32(dA_cumsum));
   SSD_TRY(check_state(dstates, states_dtype, dtype));
   if (B && !ddA_cumsum) return SSD_ERR_NULL;
   if (B) SSD_TRY(check_vec(B, b_sb, b_sl, b_sg, dtype, dstate));
@@ -623,7 +630,8 @@ int ssd_chunk_scan_bwd_dc(const void* dout, int64_t d_sb, int64_t d_sl, int64_t 
   SSD_TRY(check_dtype(dtype));
   if (!dim_ok(hdim) || !dim_ok(dstate)) return SSD_ERR_UNSUPPORTED;
   SSD_TRY(check_vec(dout, d_sb, d_sl, d_sh, dtype, hdim));
-  if (!dA_cumsum || !dC) return SSD_ERR_NULL;
+  if (!dC) return SSD_ERR_NULL;
+  SSD_TRY(check_f32(dA_cumsum));  // fetched in 16-byte pieces
   SSD_TRY(check_state(prev_states, states_dtype, dtype));
   if (C && !ddA_cumsum_prev) return SSD_ERR_NULL;
   if (C) SSD_TRY(check_vec(C, c_sb, c_sl, c_sg, dtype, dstate));

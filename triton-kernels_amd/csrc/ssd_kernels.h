@@ -771,12 +771,18 @@ __global__ __launch_bounds__(512) void ssd_state_walk_dma_kernel(
   // The copies of stage g into LDS set u: wave w brings rows 8 w .. 8 w + 7 of x (one instruction),
   // rows 8 w .. of B (two), and waves 0 / 1 the pieces of dA / dt.  What depends on the lane is
   // computed here; a request moves scalar bases (and clamps the rows of the last, ragged stage).
+  // Copies a wave requests per stage: kXCopies of x, kBCopies of B (and one more on waves 0 / 1).  The
+  // hand-placed waits below count on exactly these numbers.
+  constexpr int kXCopies = 1, kBCopies = 2, kMinCopies = kXCopies + kBCopies;
+  constexpr int kStateStores = 16;  // stores of the state entering a chunk, per lane
+  static_assert(8 * 8 * kXCopies == KT && 8 * 4 * kBCopies == KT, "eight waves bring the 64 rows of a stage");
+  static_assert(sizeof(floatx16) == kStateStores * sizeof(float), "one store per accumulator register");
   const int xr = 8 * wave + (lane >> 3);                                  // row of x inside the stage
   const unsigned x_piece = 16u * ((lane & 7) ^ (4 * ((xr >> 1) & 1)));    // byte offset inside the row
-  int br[2];
-  unsigned b_piece[2];
+  int br[kBCopies];
+  unsigned b_piece[kBCopies];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int j = 0; j < kBCopies; ++j) {
     br[j] = 4 * (2 * wave + j) + (lane >> 4);
     b_piece[j] = 16u * ((lane & 15) ^ (4 * (br[j] & 3)));
   }
@@ -787,7 +793,7 @@ __global__ __launch_bounds__(512) void ssd_state_walk_dma_kernel(
     copy16_to_lds(xg + (int64_t)row0 * sx.sl, (unsigned)(min(xr, last) * sx.sl) * 2u + x_piece, base + wave * 1024);
     const T* bg = Bg + (int64_t)row0 * sB.sl;
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < kBCopies; ++j)
       copy16_to_lds(bg, (unsigned)(min(br[j], last) * sB.sl) * 2u + b_piece[j], base + S::kX + (2 * wave + j) * 1024);
     if (wave < 2) {
       // lanes 0 .. 15: the stage's 64 values; the others: the chunk's last four values of dA (dt: anything valid)
@@ -839,13 +845,14 @@ __global__ __launch_bounds__(512) void ssd_state_walk_dma_kernel(
     // stages after it (three per wave and stage, four for two of the waves) and, if a chunk began
     // 1 .. R - 2 stages ago, the sixteen stores of its entering state (with chunks of one or two stages
     // there may be two such chunks: the lower count waits a little longer).
-    if (since <= R - 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (R - 2) + 16) : "memory");
-    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (R - 2)) : "memory");
+    static_assert(kMinCopies * (R - 2) + kStateStores < 64, "the counter holds 6 bits");
+    if (since <= R - 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kMinCopies * (R - 2) + kStateStores) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kMinCopies * (R - 2)) : "memory");
     __syncthreads();  // every wave's part of the stage is there; every wave is done with stage g - 1
     if (k0 == 0) {  // the state entering the chunk
       TO* o = out + ((b * C + c) * nh + h) * (int64_t)(P * N);
 #pragma unroll
-      for (int v = 0; v < 16; ++v) __builtin_nontemporal_store((TO)st[v], o + elem(v));
+      for (int v = 0; v < kStateStores; ++v) __builtin_nontemporal_store((TO)st[v], o + elem(v));
       since = 0;
     }
     ++since;
@@ -1221,14 +1228,18 @@ __global__ __launch_bounds__(256, 2) void ssd_group_grad_dma_kernel(
 
   // The copies of head hh into LDS set u.  What depends on the lane is the same for every head and is
   // kept as byte offsets; a head only moves the (scalar) bases.
-  unsigned s_off[4], a_off[2];
+  // Copies a wave requests per head: kSCopies of the state tile, kACopies of the rows (and one more on
+  // waves 0 / 1); the wait in the loop counts on these numbers.
+  constexpr int kSCopies = 4, kACopies = 2, kMinCopies = kSCopies + kACopies;
+  static_assert(4 * 4 * kSCopies == P && 4 * 8 * kACopies == 64, "four waves bring a head's state tile and 64 rows");
+  unsigned s_off[kSCopies], a_off[kACopies];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {  // four rows of the state tile per instruction
+  for (int j = 0; j < kSCopies; ++j) {  // four rows of the state tile per instruction
     const int r = 4 * (4 * wave + j) + (lane >> 4);
     s_off[j] = (unsigned)(r * N + 8 * ((lane & 15) ^ (4 * (r & 3)))) * (unsigned)sizeof(T);
   }
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {  // eight rows of a per instruction
+  for (int j = 0; j < kACopies; ++j) {  // eight rows of a per instruction
     const int r = 8 * (2 * wave + j) + (lane >> 3);
     a_off[j] = (unsigned)((int64_t)min(m0 + r, limit - 1) * sa.sl + 8 * ((lane & 7) ^ ((r >> 1) & 7))) * (unsigned)sizeof(T);
   }
@@ -1242,9 +1253,9 @@ __global__ __launch_bounds__(256, 2) void ssd_group_grad_dma_kernel(
     const T* sg = s_first + (int64_t)hh * P * N;
     const T* ag = a_first + (int64_t)hh * sa.sh;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) copy16_to_lds(sg, s_off[j], base + (4 * wave + j) * 1024);
+    for (int j = 0; j < kSCopies; ++j) copy16_to_lds(sg, s_off[j], base + (4 * wave + j) * 1024);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) copy16_to_lds(ag, a_off[j], base + S::kState + (2 * wave + j) * 1024);
+    for (int j = 0; j < kACopies; ++j) copy16_to_lds(ag, a_off[j], base + S::kState + (2 * wave + j) * 1024);
     if (wave < 2) {
       const float* vg = (wave == 0 ? dA_cs : dt) + (chunk_first + (int64_t)hh * C) * Q;
       copy16_to_lds(vg, v_off, base + S::kState + S::kRows + wave * 1024);
@@ -1290,7 +1301,7 @@ __global__ __launch_bounds__(256, 2) void ssd_group_grad_dma_kernel(
   for (int hh = 0; hh < heads_per_group; ++hh) {
     const int u = hh % S::R;
     // the copies of this head have landed once only those of the next head are outstanding
-    if (hh + 1 < heads_per_group) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    if (hh + 1 < heads_per_group) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kMinCopies) : "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();  // every wave's part of the head is there; every wave is done with head hh - 1
     if (hh + 2 < heads_per_group) request(hh + 2, (hh + 2) % S::R);

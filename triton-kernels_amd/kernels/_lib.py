@@ -53,6 +53,9 @@ _SIGNATURES = {
     "ema_seq_fwd": (c_int, [c_int] + _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, c_size_t, c_int, _I, _I, _I, _I, _P, _P, _P]),
     "ema_seq_bwd": (c_int, [c_int] + _SEQ + _SEQ + _SEQ + [_P, _P, c_int] + _SEQ + _SEQ + [_P, _P, c_size_t, c_int, _I, _I, _I, _I, _P, _P, _P]),
     "ema_seq_fwd_static_max_workspace_bytes": (c_size_t, []),
+    "ema_seq_fwd_static_init": (c_int, []),
+    "ema_seq_fwd_static_error": (c_int, [_P, _P]),
+    "ema_seq_fwd_static_reset": (c_int, [_P]),
     "ema_seq_fwd_static": (c_int, [c_int] + _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _I, _I, _I, _I, _P]),
     # SSD forward stages (include/ssd_hip.h)
     "ssd_chunk_cumsum_fwd": (c_int, [_P, c_int, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, c_int, c_float, c_float, _P]),
