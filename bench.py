@@ -431,6 +431,7 @@ def ssd_stages(torch, steps, warmup, only=None):
     from kernels.mamba_kernels_bwd.mamba_chunk_scan_chunk_state_bwd_dx import _chunk_scan_chunk_state_bwd_dx
     from kernels.mamba_kernels_bwd.mamba_chunk_state_bwd_db import _chunk_state_bwd_db
     from kernels.mamba_kernels_bwd.mamba_scan_bwd import _chunk_scan_bwd_dstates
+    from kernels.mamba_kernels_bwd.mamba_scan_state_passing_bwd import _chunk_scan_state_passing_bwd
     from kernels.mamba_kernels_bwd.mamba_state_passing_bwd_dstates import _state_passing_bwd
 
     dev = torch.device("cuda:0")
@@ -471,11 +472,13 @@ def ssd_stages(torch, steps, warmup, only=None):
         "bmm_chunk": lambda i: _bmm_chunk_fwd(pick(i)[4], pick(i)[3], Q, output_dtype=torch.float32),
         "chunk_scan": lambda i: _chunk_scan_fwd(pick(i)[9], pick(i)[0], pick(i)[5], pick(i)[6], pick(i)[4], pick(i)[8]),
         "forward": lambda i: _mamba_chunk_scan_combined_fwd(*pick(i)[:5], Q),
-        # the same with everything behind the cumsum in one kernel (all intermediates on chip)
         # backward stages (the reference has no combined backward): x dt A B C | dt_out dA st states cb dout dprev dstates
         "bwd_dstates": lambda i: _chunk_scan_bwd_dstates(pick(i)[4], pick(i)[6], pick(i)[10]),
         "bwd_state_passing": lambda i: _state_passing_bwd(pick(i)[8].view(b, C, nh, P * N), pick(i)[6][..., -1],
                                                           pick(i)[11].view(b, C, nh, P * N)),
+        # the two stages above in one kernel: the chunk's gradient stays in the accumulators
+        "bwd_dstates_state_passing": lambda i: _chunk_scan_state_passing_bwd(pick(i)[4], pick(i)[6], pick(i)[10],
+                                                                             pick(i)[8]),
         "bwd_db": lambda i: _chunk_state_bwd_db(pick(i)[0], pick(i)[5], pick(i)[6], pick(i)[12], B=pick(i)[3], ngroups=g),
         "bwd_dc": lambda i: _chunk_scan_bwd_dC(pick(i)[8], pick(i)[6], pick(i)[10], C=pick(i)[4], ngroups=g),
         "bwd_dx": lambda i: _chunk_scan_chunk_state_bwd_dx(pick(i)[0], pick(i)[5], pick(i)[6], pick(i)[3], pick(i)[9],
@@ -496,12 +499,14 @@ def ssd_stages(torch, steps, warmup, only=None):
         "bmm_chunk": 2 * bc + cbb, "chunk_scan": cbb + 2 * xb + bc + pvb + 2 * dtb,
         "forward": 2 * xb + 2 * bc + dtb,
         "bwd_dstates": xb + bc + dtb + pvb, "bwd_state_passing": 3 * pvb + 2 * dtb // Q,
+        "bwd_dstates_state_passing": xb + bc + dtb + 2 * pvb + dtb // Q,
         "bwd_db": xb + pvb + 2 * dtb + bc + 2 * bc + dtb, "bwd_dc": xb + pvb + dtb + bc + 2 * bc + dtb,
         "bwd_dx": cbb + 3 * xb + bc + pvb + 3 * dtb, "bwd_ddAcs": 2 * xb + 3 * dtb + cbb,
     }
     units = b * C * nh
     flops = {"chunk_state": 2 * Q * P * N * units, "chunk_state_passing": 2 * Q * P * N * units, "bmm_chunk": 2 * Q * Q * N * b * C * g,
              "chunk_scan": (2 * Q * Q * P + 2 * Q * N * P) * units, "bwd_dstates": 2 * Q * P * N * units,
+             "bwd_dstates_state_passing": 2 * Q * P * N * units,
              "bwd_db": 2 * Q * P * N * units, "bwd_dc": 2 * Q * P * N * units,
              "bwd_dx": (2 * Q * Q * P + 2 * Q * N * P) * units, "bwd_ddAcs": 2 * Q * Q * P * units}
     res = {}
@@ -517,7 +522,11 @@ def ssd_stages(torch, steps, warmup, only=None):
             res[name]["dense_TFLOPs"] = flops[name] / ms / 1e9
             res[name]["mfma_frac"] = flops[name] / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS
     if not only:
-        res["backward_stages_sum"] = {"ms": sum(v["ms"] for k, v in res.items() if k.startswith("bwd_"))}
+        six = ("bwd_dstates", "bwd_state_passing", "bwd_db", "bwd_dc", "bwd_dx", "bwd_ddAcs")
+        res["backward_stages_sum"] = {"ms": sum(res[k]["ms"] for k in six)}
+        # the same work with the first two stages in one kernel
+        res["backward_sum_with_reverse_walk"] = {
+            "ms": res["bwd_dstates_state_passing"]["ms"] + sum(res[k]["ms"] for k in six[2:])}
     return res
 
 
@@ -828,6 +837,8 @@ def main():
                                                                       "chunk_state_passing", "bmm_chunk", "chunk_scan")},
                         "backward_stages_ms": {k: v["ms"] for k, v in s5.items() if k.startswith("bwd_")},
                         "backward_stages_sum_ms": s5["backward_stages_sum"]["ms"],
+                        # with bwd_dstates and bwd_state_passing replaced by bwd_dstates_state_passing
+                        "backward_sum_with_reverse_walk_ms": s5["backward_sum_with_reverse_walk"]["ms"],
                         "stages": s5}
         torch.cuda.empty_cache()
         out["configs"] = cfgs

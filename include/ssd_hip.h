@@ -163,6 +163,30 @@ int ssd_state_passing_bwd(const void* states, int states_dtype, const float* dA_
                           int64_t batch, int64_t nchunks, int64_t nheads, int64_t dim, const int32_t* seq_idx,
                           int64_t seq_sb, int64_t seq_sl, int64_t seqlen, int64_t chunk, void* stream);
 
+/* Bytes of workspace ssd_chunk_scan_state_passing_bwd needs (per-wave partial dot products). */
+size_t ssd_chunk_scan_state_passing_bwd_workspace_bytes(int64_t batch, int64_t nchunks, int64_t nheads);
+
+/* ssd_chunk_scan_bwd_dstates followed by ssd_state_passing_bwd in one kernel (no counterpart among
+ * the reference's launchers, the mirror image of ssd_chunk_state_passing_fwd): a workgroup per
+ * (batch, head) walks the chunks from the last to the first, forms the chunk's gradient with respect
+ * to its entering state in the accumulators and feeds it to the reverse recurrence there, so that
+ * this state-sized float32 tensor is neither written nor read back.  C, dout, dA_cumsum as for
+ * ssd_chunk_scan_bwd_dstates; states, dfinal, dstates, ddA_chunk, dinit as for ssd_state_passing_bwd
+ * (dim = hdim * dstate, dA_chunk = dA_cumsum[..., chunk - 1]).  The results are those of the two
+ * entry points called one after the other with a float32 tensor between them: dstates bit for bit,
+ * ddA_chunk up to the order of its sums.  Written for bfloat16 dout / C / states, hdim 64,
+ * dstate 128, chunk a multiple of 64 and at least 128, non-negative strides; anything else, and a
+ * packed batch (seq_idx), returns SSD_ERR_UNSUPPORTED and goes through the two separate entry points.
+ * Replaces the pair _chunk_scan_bwd_dstates, kernels/mamba_kernels_bwd/mamba_scan_bwd.py:91-116, and
+ * _state_passing_bwd, kernels/mamba_kernels_bwd/mamba_state_passing_bwd_dstates.py:116-172, where a
+ * caller runs them back to back. */
+int ssd_chunk_scan_state_passing_bwd(const void* C, int64_t c_sb, int64_t c_sl, int64_t c_sg, const void* dout,
+                                     int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype, const float* dA_cumsum,
+                                     const void* states, int states_dtype, const float* dfinal, void* dstates,
+                                     int dstates_dtype, float* ddA_chunk, float* dinit, void* workspace,
+                                     size_t workspace_bytes, int64_t batch, int64_t seqlen, int64_t nheads,
+                                     int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk, void* stream);
+
 /* dB[b,l,g,n] = sum over the heads h of group g of (sum_p x[m,p] * round(dstates[b,c,h,p,n])) *
  * exp(min(dA_last - dA_m, 0)) * dt_m (float32, dense (batch, seqlen, ngroups, dstate)).  With B
  * (may be NULL, then ddA_cumsum is not written): r_h[m] = sum_n db_h[m,n] * B[m,n] and

@@ -132,6 +132,92 @@ def test_state_passing_bwd_vs_oracle(b, nc, nh, dim, has_init, device):
     check_close("dstates, float32 out of bfloat16 in", mixed[0], ref16[0], F32)
 
 
+WALK_CASES = [
+    # b, L, nh, g, Q: bfloat16, hdim 64, dstate 128 (what the single kernel is written for)
+    (2, 1024, 4, 1, 256),
+    (1, 700, 3, 1, 256),    # last chunk ragged: three stages, the last of them 60 rows
+    (1, 520, 2, 2, 128),    # two stages per chunk, the last chunk has one stage of 8 rows
+    (2, 384, 4, 2, 192),    # three stages per chunk
+    (1, 1536, 2, 1, 512),
+    (1, 100, 2, 1, 128),    # a single, ragged chunk
+    (1, 2100, 1, 1, 1024),
+]
+
+
+@pytest.mark.parametrize("has_init", [False, True])
+@pytest.mark.parametrize("b,L,nh,g,Q", WALK_CASES)
+def test_dstates_and_state_passing_in_one_kernel(b, L, nh, g, Q, has_init, device):
+    """The reverse walk against the oracle's two stages with the reference's rounding, and against
+    the two launchers with a float32 tensor between them (dstates bit for bit)."""
+    from kernels.mamba_kernels_bwd import mamba_scan_state_passing_bwd as M
+    from kernels.mamba_kernels_bwd.mamba_scan_bwd import _chunk_scan_bwd_dstates
+    from kernels.mamba_kernels_bwd.mamba_state_passing_bwd_dstates import _state_passing_bwd
+
+    P, N = 64, 128
+    announce(f"ssd reverse walk b{b} L{L} nh{nh} g{g} Q{Q} init={has_init}")
+    x, dt, dA_cs, B, C, D, dout, prev, _ = _inputs(b, L, nh, P, g, N, Q, BF16)
+    nc = dA_cs.shape[2]
+    states = prev.to(BF16)
+    gen = torch.Generator().manual_seed(L)
+    dfin = torch.randn(b, nh, P, N, generator=gen)
+    d = lambda t: t.to(device)
+
+    fused = M._fused(d(C), d(dA_cs), d(dout), d(states), d(dfin), has_init, F32)
+    assert fused is not None, "the single kernel must take this case"
+    got = M._chunk_scan_state_passing_bwd(d(C), d(dA_cs), d(dout), d(states), dfinal_states=d(dfin),
+                                          has_initial_states=has_init, dstates_dtype=F32)
+    assert torch.equal(got[0], fused[0])
+
+    dprev_ref = S.bwd_dstates(C, dA_cs, dout, round_to=BF16)
+    ref = S.state_passing_bwd(states.float().reshape(b, nc, nh, P * N), dA_cs[..., -1],
+                              dprev_ref.reshape(b, nc, nh, P * N), dfin.reshape(b, nh, P * N),
+                              has_initial_states=has_init)
+    check_close("dstates", got[0].reshape(b, nc, nh, P * N), ref[0], BF16)
+    check_close("ddA_chunk_cumsum", got[1], ref[1], BF16)
+    if has_init:
+        check_close("dinitstates", got[2].reshape(b, nh, P * N), ref[2], BF16)
+    else:
+        assert got[2] is None
+
+    dprev = _chunk_scan_bwd_dstates(d(C), d(dA_cs), d(dout), dtype=F32)
+    two = _state_passing_bwd(d(states).reshape(b, nc, nh, P * N), d(dA_cs)[..., -1], dprev.reshape(b, nc, nh, P * N),
+                             dfinal_states=d(dfin).reshape(b, nh, P * N), has_initial_states=has_init,
+                             dstates_dtype=F32)
+    assert torch.equal(got[0].reshape(b, nc, nh, P * N), two[0]), "dstates differ from the two launchers'"
+    check_close("ddA_chunk_cumsum against the two launchers", got[1], two[1].cpu(), F32)
+    if has_init:
+        assert torch.equal(got[2].reshape(b, nh, P * N), two[2])
+
+    # bfloat16 out (the type of the states) and no gradient of the final state
+    got16 = M._chunk_scan_state_passing_bwd(d(C), d(dA_cs), d(dout), d(states))
+    assert got16[0].dtype == BF16
+    ref0 = S.state_passing_bwd(states.float().reshape(b, nc, nh, P * N), dA_cs[..., -1],
+                               dprev_ref.reshape(b, nc, nh, P * N))
+    check_close("dstates, bfloat16, no dfinal", got16[0].reshape(b, nc, nh, P * N), ref0[0], BF16)
+    check_close("ddA_chunk_cumsum, no dfinal", got16[1], ref0[1], BF16)
+
+
+def test_reverse_walk_falls_back_to_the_two_launchers(device):
+    """Shapes and types the single kernel does not take go through the two launchers."""
+    from kernels.mamba_kernels_bwd import mamba_scan_state_passing_bwd as M
+
+    b, L, nh, P, g, N, Q = 1, 300, 2, 64, 1, 64, 64
+    for dtype in (F32, BF16):
+        x, dt, dA_cs, B, C, D, dout, prev, _ = _inputs(b, L, nh, P, g, N, Q, dtype)
+        nc = dA_cs.shape[2]
+        d = lambda t: t.to(device)
+        assert M._fused(d(C), d(dA_cs), d(dout), d(prev.to(dtype)), None, False, F32) is None
+        got = M._chunk_scan_state_passing_bwd(d(C), d(dA_cs), d(dout), d(prev.to(dtype)), has_initial_states=True,
+                                              dstates_dtype=F32)
+        rt = None if dtype == F32 else dtype
+        ref = S.state_passing_bwd(prev.to(dtype).float().reshape(b, nc, nh, P * N), dA_cs[..., -1],
+                                  S.bwd_dstates(C, dA_cs, dout, round_to=rt).reshape(b, nc, nh, P * N),
+                                  has_initial_states=True)
+        check_close("dstates", got[0].reshape(b, nc, nh, P * N), ref[0], F32)
+        check_close("ddA_chunk_cumsum", got[1], ref[1], F32)
+        check_close("dinitstates", got[2].reshape(b, nh, P * N), ref[2], F32)
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("b,L,nh,P,g,N,Q", CASES)
 def test_dx_vs_oracle(b, L, nh, P, g, N, Q, dtype, device):
@@ -174,6 +260,34 @@ def test_ddAcs_vs_oracle(b, L, nh, P, g, N, Q, dtype, device):
     ref = S.chunk_scan_bwd_ddAcs_stable(x, dt, dA_cs, dout, cb)
     got = _chunk_scan_bwd_ddAcs_stable(d(x), d(dt), d(dA_cs), d(dout), d(cb))
     check_close("ddA_cumsum (causal term)", got, ref, dtype, loose=dtype == BF16)
+
+
+@pytest.mark.parametrize("kind", ["steep", "rising", "mixed"])
+@pytest.mark.parametrize("Q", [64, 256])
+def test_ddAcs_decays_outside_the_factored_form(kind, Q, device):
+    """The kernel factors exp(dA_m - dA_n) below the diagonal blocks where dA falls along the chunk,
+    and inside a diagonal block where it falls by little there.  Steep decays (dA falls by far more
+    than float32's exponent range inside 32 positions), rising dA (A > 0: the clamp at 0 acts) and
+    dA that changes direction take the other forms; all against the oracle in float32."""
+    from kernels.mamba_kernels_bwd.mamba_chunk_scan_bwd_da import _chunk_scan_bwd_ddAcs_stable
+
+    b, L, nh, P, g, N = 1, 2 * Q, 2, 64, 1, 64
+    announce(f"ssd bwd ddAcs {kind} Q{Q}")
+    x, dt_raw, A, B, C, D, _ = S.make_inputs(b, L, nh, P, g, N, seed=7 + Q, dtype=F32)
+    gen = torch.Generator().manual_seed(Q)
+    if kind == "steep":
+        dt_raw, A = torch.full_like(dt_raw, 2.0), torch.tensor([-6.0, -1.5])
+    elif kind == "rising":
+        A = torch.tensor([0.5, 0.05])
+    dA_cs, dt = S.chunk_cumsum(dt_raw, A, Q)
+    if kind == "mixed":  # no cumsum of one sign: what the launcher is given need not come from chunk_cumsum
+        dA_cs = torch.randn(dA_cs.shape, generator=gen)
+    dout = torch.randn(b, L, nh, P, generator=gen)
+    cb = S.bmm_chunk(C, B, Q)
+    d = lambda t: t.to(device)
+    ref = S.chunk_scan_bwd_ddAcs_stable(x, dt, dA_cs, dout, cb)
+    got = _chunk_scan_bwd_ddAcs_stable(d(x), d(dt), d(dA_cs), d(dout), d(cb))
+    check_close("ddA_cumsum (causal term)", got, ref, F32)
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])

@@ -593,6 +593,61 @@ int ssd_state_passing_bwd(const void* states, int states_dtype, const float* dA_
   return launched();
 }
 
+size_t ssd_chunk_scan_state_passing_bwd_workspace_bytes(int64_t batch, int64_t nchunks, int64_t nheads) {
+  if (batch <= 0 || nchunks <= 0 || nheads <= 0) return 0;
+  return (size_t)(batch * nheads * nchunks * 8) * sizeof(float);  // a partial dot per wave
+}
+
+int ssd_chunk_scan_state_passing_bwd(const void* C, int64_t c_sb, int64_t c_sl, int64_t c_sg, const void* dout,
+                                     int64_t d_sb, int64_t d_sl, int64_t d_sh, int dtype, const float* dA_cumsum,
+                                     const void* states, int states_dtype, const float* dfinal, void* dstates,
+                                     int dstates_dtype, float* ddA_chunk, float* dinit, void* workspace,
+                                     size_t workspace_bytes, int64_t batch, int64_t seqlen, int64_t nheads,
+                                     int64_t ngroups, int64_t hdim, int64_t dstate, int64_t chunk, void* stream) {
+  Dims d;
+  SSD_TRY(check_dims(batch, seqlen, nheads, ngroups, hdim, dstate, chunk, &d));
+  SSD_TRY(check_dtype(dtype));
+  SSD_TRY(check_dtype(states_dtype));
+  SSD_TRY(check_dtype(dstates_dtype));
+  // what the kernel is written for: its tiles and its three state buffers in LDS have these sizes
+  if (dtype != SSD_BF16 || states_dtype != SSD_BF16 || hdim != 64 || dstate != 128 || chunk % 64 || chunk < 128)
+    return SSD_ERR_UNSUPPORTED;
+  SSD_TRY(check_vec(dout, d_sb, d_sl, d_sh, dtype, hdim));
+  SSD_TRY(check_vec(C, c_sb, c_sl, c_sg, dtype, dstate));
+  SSD_TRY(check_f32(dA_cumsum));  // fetched in 16-byte pieces
+  SSD_TRY(check_f32(states));
+  SSD_TRY(check_f32(dstates));
+  SSD_TRY(check_f32(workspace));
+  if (!ddA_chunk) return SSD_ERR_NULL;
+  if (dfinal) SSD_TRY(check_f32(dfinal));
+  if (dinit) SSD_TRY(check_f32(dinit));
+  if (workspace_bytes < ssd_chunk_scan_state_passing_bwd_workspace_bytes(batch, d.C, nheads)) return SSD_ERR_SHAPE;
+  const Strides3 sd{d_sb, d_sl, d_sh}, sc{c_sb, c_sl, c_sg};
+  // (the kernel keeps the byte offset of a row inside a stage in 32 bits)
+  if (!forward_strides(sd) || !forward_strides(sc) || sd.sl >= (int64_t(1) << 24) || sc.sl >= (int64_t(1) << 24))
+    return SSD_ERR_UNSUPPORTED;
+  if (batch * nheads > 0x7fffffff) return SSD_ERR_SHAPE;
+  hipStream_t st = as_stream(stream);
+  float* part = static_cast<float*>(workspace);
+  constexpr int smem = WalkBwdDmaSmem::kBytes;
+  auto launch = [&](auto tg) -> int {
+    using TG = decltype(tg);
+    auto kernel = ssd_state_walk_bwd_dma_kernel<TG>;
+    SSD_TRY(allow_smem(kernel, smem));
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(batch * nheads)), dim3(512), smem, st, (const bf16_t*)dout, sd,
+                       (const bf16_t*)C, sc, dA_cumsum, (const bf16_t*)states, dfinal, (TG*)dstates, part, dinit,
+                       (int)nheads, (int)(nheads / ngroups), (int)seqlen, (int)chunk, (int)d.C);
+    return launched();
+  };
+  SSD_TRY(dstates_dtype == SSD_BF16 ? launch(bf16_t()) : launch(float()));
+  // ddA_chunk[b,h,c] = exp(dA_cumsum[b,h,c,chunk-1]) * the sum of the eight partial dots
+  const int64_t total = batch * nheads * d.C;
+  hipLaunchKernelGGL(ssd_state_passing_bwd_finish_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                     part, dA_cumsum + (chunk - 1), nheads * d.C * chunk, d.C * chunk, chunk, ddA_chunk, (int)nheads,
+                     (int)d.C, 8, dinit ? 1 : 0, total, as_seq(nullptr, 0, 0), (int)seqlen, (int)chunk);
+  return launched();
+}
+
 int ssd_chunk_state_bwd_db(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh, int dtype,
                            const float* dt, const float* dA_cumsum, const void* dstates, int states_dtype,
                            const void* B, int64_t b_sb, int64_t b_sl, int64_t b_sg, float* dB, float* ddA_cumsum,

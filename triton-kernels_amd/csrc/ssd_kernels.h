@@ -886,6 +886,201 @@ __global__ __launch_bounds__(512) void ssd_state_walk_dma_kernel(
   for (int v = 0; v < 16; ++v) f[elem(v)] = st[v];
 }
 
+// ------------------------------------------------------------------------------------
+// The mirror image of that walk for the backward: the gradient of the chunk scan with respect to
+// the carried states (MODE 1 of ssd_chunk_state_kernel) and the reverse recurrence over the chunks
+// (ssd_state_passing_bwd_kernel) in one kernel, for bfloat16, hdim 64, dstate 128, bfloat16 carried
+// states and chunks of at least two stages.  A workgroup per (b, h) walks the chunks from the last
+// to the first (the 64-row stages of a chunk in ascending order, as the stage kernel sums them) with
+//   D_c   = sum_k round(dout[k] * exp(dA_k)) (x) C[k]          over the rows of chunk c (accumulators)
+//   dstates[c] = G,   part[(b,h,c), wave] = <states[c], G>     at the chunk's first stage
+//   G     = exp(dA_chunk[c]) * G + D_c                          at its last
+// where G starts from dfinal (or zero) and ends as dinit.  D_c never leaves the accumulators: the
+// float32 (or rounded) copy that the two launchers write and read back is gone, and the results
+// are those of the two launchers with a float32 D_c (dstates bit for bit; the per-chunk dots are
+// summed in another order).  The finish kernel of the state passing turns the partial dots into ddA.
+//
+// Rows arrive as in the forward walk: R stages of dout (128-byte rows), C (256-byte rows) and dA in
+// LDS by direct copies, the waits placed by hand.  states[c] (16 KB) comes the same way with the
+// request of the chunk's first stage, ahead of that stage's rows, into one of three buffers in turn:
+// the buffer of chunk c was read last at the first stage of chunk c + 3, at least six steps before
+// this request (chunks have two stages or more), and the request is made behind a barrier that every
+// wave passes after that step.  Counting: a wave requests kMinCopies copies per stage or more (two
+// for the state tile, one for dA), so once no more than kMinCopies * (R - 2) requests are
+// outstanding everything up to this stage's rows has landed; the stores of a chunk's first stage
+// (sixteen of dstates and one partial dot) share the counter and are allowed for while they can
+// still be in the queue.
+// ------------------------------------------------------------------------------------
+struct WalkBwdDmaSmem {
+  static constexpr int R = WalkDmaSmem::R;
+  static constexpr int kX = WalkDmaSmem::kX, kB = WalkDmaSmem::kB, kVec = 1024;
+  static constexpr int kStage = kX + kB + kVec;
+  static constexpr int kWeights = 8 * 64 * (int)sizeof(float);
+  static constexpr int kTile = 64 * 128 * (int)sizeof(bf16_t), kTiles = 3;
+  static constexpr int kBytes = R * kStage + kWeights + kTiles * kTile;
+};
+
+template <typename TG>
+__global__ __launch_bounds__(512) void ssd_state_walk_bwd_dma_kernel(
+    const bf16_t* __restrict__ dout, Strides3 sx, const bf16_t* __restrict__ Cm, Strides3 sC,
+    const float* __restrict__ dA_cs, const bf16_t* __restrict__ states, const float* __restrict__ dfinal,
+    TG* __restrict__ dstates, float* __restrict__ part, float* __restrict__ dinit, int nh, int heads_per_group, int L,
+    int Q, int C) {
+  using S = WalkBwdDmaSmem;
+  using T = bf16_t;
+  constexpr int P = 64, N = 128, KT = 64, KG = 16, MB = P / 32, R = S::R;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), half = lane >> 5;
+  float* wl = reinterpret_cast<float*>(smem + R * S::kStage) + wave * 64;  // this wave's copy of the weights
+  unsigned char* tiles = smem + R * S::kStage + S::kWeights;
+  const int bid = xcd_local_index((int)blockIdx.x, (int)gridDim.x);
+  const int h = bid % nh;
+  const int64_t b = bid / nh;
+  const float* dAb = dA_cs + (b * nh + h) * (int64_t)C * Q;
+  const T* xg = dout + b * sx.sb + h * sx.sh;
+  const T* Cg = Cm + b * sC.sb + (h / heads_per_group) * sC.sh;
+  const int SPC = Q / KT;                              // stages of a whole chunk
+  const int S_last = (L - (C - 1) * Q + KT - 1) / KT;  // stages of the last chunk, which comes first
+  const int G = S_last + (C - 1) * SPC;
+  const int mi = wave % MB, ni = wave / MB;  // this wave's block of the state: rows 32 mi .., columns 32 ni ..
+  auto elem = [&](int v) { return (32 * mi + acc_row(v, lane)) * N + 32 * ni + (lane & 31); };
+  // step i of the walk works on stage s of chunk c
+  auto stage_of = [&](int i, int& c, int& s) {
+    if (i < S_last) {
+      c = C - 1, s = i;
+    } else {
+      const int j = i - S_last;
+      c = C - 2 - j / SPC, s = j % SPC;
+    }
+  };
+
+  constexpr int kXCopies = 1, kCCopies = 2, kMinCopies = kXCopies + kCCopies, kTileCopies = 2;
+  constexpr int kChunkStores = 16 + 1;  // dstates, and the wave's partial dot
+  static_assert(8 * 8 * kXCopies == KT && 8 * 4 * kCCopies == KT, "eight waves bring the 64 rows of a stage");
+  static_assert(8 * kTileCopies * 1024 == S::kTile, "eight waves bring the state tile");
+  static_assert(sizeof(floatx16) == (kChunkStores - 1) * sizeof(float), "one store per accumulator register");
+  const int xr = 8 * wave + (lane >> 3);                                  // row of dout inside the stage
+  const unsigned x_piece = 16u * ((lane & 7) ^ (4 * ((xr >> 1) & 1)));    // byte offset inside the row
+  int cr[kCCopies];
+  unsigned c_piece[kCCopies];
+#pragma unroll
+  for (int j = 0; j < kCCopies; ++j) {
+    cr[j] = 4 * (2 * wave + j) + (lane >> 4);
+    c_piece[j] = 16u * ((lane & 15) ^ (4 * (cr[j] & 3)));
+  }
+  auto request = [&](int i, int u) {
+    int c, s;
+    stage_of(min(i, G - 1), c, s);
+    const int row0 = c * Q + s * KT;
+    const int last = L - 1 - row0;  // rows past the sequence repeat its last row (their weight is 0)
+    unsigned char* base = smem + u * S::kStage;
+    if (s == 0 && i < G) {  // the state entering the chunk, ahead of the rows
+      const T* sg = states + ((b * C + c) * nh + h) * (int64_t)(P * N) + wave * (kTileCopies * 512);
+      unsigned char* dst = tiles + (c % S::kTiles) * S::kTile + wave * (kTileCopies * 1024);
+#pragma unroll
+      for (int j = 0; j < kTileCopies; ++j) copy16_to_lds(sg + j * 512, 16u * (unsigned)lane, dst + j * 1024);
+    }
+    copy16_to_lds(xg + (int64_t)row0 * sx.sl, (unsigned)(min(xr, last) * sx.sl) * 2u + x_piece, base + wave * 1024);
+    const T* cg = Cg + (int64_t)row0 * sC.sl;
+#pragma unroll
+    for (int j = 0; j < kCCopies; ++j)
+      copy16_to_lds(cg, (unsigned)(min(cr[j], last) * sC.sl) * 2u + c_piece[j], base + S::kX + (2 * wave + j) * 1024);
+    if (wave == 0) {
+      // lanes 0 .. 15: the stage's 64 values of dA; the others: the chunk's last four
+      const int tail = (c + 1) * Q - 4 - row0;
+      copy16_to_lds(dAb + row0, 4u * (unsigned)(lane < 16 ? 4 * lane : tail), base + S::kX + S::kB);
+    }
+  };
+#pragma unroll
+  for (int u = 0; u < R - 1; ++u) request(u, u);
+
+  floatx16 acc, gr;
+  zero_acc(acc);
+  zero_acc(gr);
+  if (dfinal) {
+    const float* fin = dfinal + (b * nh + h) * (int64_t)(P * N);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) gr[v] = fin[elem(v)];
+  }
+  // (waited for here, so that no wait for ordinary loads falls into the loop)
+#pragma unroll
+  for (int v = 0; v < 16; ++v) asm volatile("" : "+v"(gr[v]));
+
+  // where this lane reads its operand fragments inside a stage's tiles (elements)
+  int x_off, c_off;
+  {
+    const int i16 = lane & 15;
+    const int row = 8 * half + (i16 >> 2);
+    const int cx = 32 * mi + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+    const int cc = 32 * ni + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+    x_off = row * P + 8 * ((cx >> 3) ^ (4 * ((row >> 1) & 1))) + (cx & 7);
+    c_off = row * N + 8 * ((cc >> 3) ^ (4 * (row & 3))) + (cc & 7);
+  }
+  typedef __attribute__((address_space(3))) ema::bf16x4 lds_bf16x4;
+  auto tr_read = [&](const T* p, int pitch) {
+    const ema::bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)p);
+    const ema::bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(p + 4 * pitch));  // row + 4: the same key
+    Vec16<T> r;
+    r.raw = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return r;
+  };
+
+  int since = R;  // steps since the last chunk began (at least R: no stores in the queue)
+  for (int i = 0; i < G; ++i) {
+    const int u = i % R;
+    int c, s;
+    stage_of(i, c, s);
+    const int row0 = c * Q + s * KT;
+    static_assert(kMinCopies * (R - 2) + kChunkStores < 64, "the counter holds 6 bits");
+    if (since <= R - 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kMinCopies * (R - 2) + kChunkStores) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kMinCopies * (R - 2)) : "memory");
+    __syncthreads();  // every wave's part of the stage is there; every wave is done with step i - 1
+    if (s == 0) {  // dstates[c] and the wave's share of <states[c], G>
+      TG* o = dstates + ((b * C + c) * nh + h) * (int64_t)(P * N);
+      const T* tile = reinterpret_cast<const T*>(tiles + (c % S::kTiles) * S::kTile);
+      float dot = 0.f;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        __builtin_nontemporal_store((TG)gr[v], o + elem(v));
+        dot = fmaf((float)tile[elem(v)], gr[v], dot);
+      }
+      dot = ema::wave_sum(dot);
+      if (lane == 0) part[((b * nh + h) * (int64_t)C + c) * 8 + wave] = dot;
+      since = 0;
+    }
+    ++since;
+    request(i + R - 1, (i + R - 1) % R);
+    const unsigned char* base = smem + u * S::kStage;
+    const T* xb = reinterpret_cast<const T*>(base);
+    const T* cb = reinterpret_cast<const T*>(base + S::kX);
+    const float* vec = reinterpret_cast<const float*>(base + S::kX + S::kB);  // dA of the rows, dA tail
+    const float dA_last = vec[67];
+    wl[lane] = row0 + lane < L ? __expf(vec[lane]) : 0.f;
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // the wave's own LDS writes are visible to its own reads
+#pragma unroll
+    for (int ks = 0; ks < KT / KG; ++ks) {
+      Vec16<T> xf = tr_read(xb + x_off + KG * ks * P, P);
+      const Vec16<T> cf = tr_read(cb + c_off + KG * ks * N, N);
+      float t[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) t[e] = xf.get(e) * wl[KG * ks + 8 * half + e];
+      xf.set_all(t);
+      mma_group(xf, cf, acc);
+    }
+    if (s == (c == C - 1 ? S_last : SPC) - 1) {  // the chunk ends with this stage
+      const float a = __expf(dA_last);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) gr[v] = fmaf(a, gr[v], acc[v]);
+      zero_acc(acc);
+    }
+  }
+  if (dinit) {
+    float* f = dinit + (b * nh + h) * (int64_t)(P * N);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) f[elem(v)] = gr[v];
+  }
+}
+
 // Sum over the 32 lanes of each half of a wave (lanes 0..31 and 32..63 apart), left in lanes 31
 // and 63: the DPP prefix steps of wave_inclusive_scan without the last one.
 __device__ __forceinline__ float half_wave_sum(float v) {
@@ -2107,6 +2302,9 @@ __global__ __launch_bounds__(256) void ssd_ddA_causal_kernel(
   const T* xg = x + b * sx.sb + (int64_t)c * Q * sx.sl + h * sx.sh;
   const T* dg = dout + b * sd.sb + (int64_t)c * Q * sd.sl + h * sd.sh;
 
+  // (raw buffer of 32-bit words, no bounds to speak of: the offsets stay inside the chunk's Q x Q block)
+  const __amdgpu_buffer_rsrc_t cb_desc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(cbg), 0, 0x7fffffff, 0x00020000);
+
   SSD_TSTAMP(0);
   // shared: the chunk's x rows (zero past the limit), dA, dt; cleared: the sums
   static_assert(S::PX == Tile<T>::pitch(P), "stage_rows writes rows at this pitch");
@@ -2122,6 +2320,8 @@ __global__ __launch_bounds__(256) void ssd_ddA_causal_kernel(
   for (int w = 0; w < 4; ++w) colpart[w * 256 + tid] = 0.f;
   __syncthreads();
   SSD_TSTAMP(1);
+  // (a ragged chunk keeps the direct form, whose masks keep whatever cb holds past the sequence out of the sums)
+  const bool falling = __syncthreads_and(tid + 1 >= Q || dAs[tid + 1] <= dAs[tid]) != 0 && limit == Q;
 
 #pragma unroll
   for (int slot = 0; slot < 2; ++slot) {
@@ -2135,31 +2335,65 @@ __global__ __launch_bounds__(256) void ssd_ddA_causal_kernel(
       a[ks] = load16(dg + (int64_t)min(m_lane, limit - 1) * sd.sl + KG * ks + EPL * half);
       if (m_lane >= limit) a[ks].zero();
     }
-    float rowacc[16], dAm[16];
+    // Below the diagonal blocks the decay factors as exp(dA_m - r) * exp(r - dA_n) with r = dA of the
+    // block row's first position: where dA does not increase along the chunk (`falling`; it is a cumsum
+    // of dt * A with A < 0) both exponents are <= 0 there, so neither factor overflows and the clamp of
+    // the exponent at 0 never acts.  That takes the exponential out of the element loop (one per row and
+    // block row, one per column and block); the diagonal blocks and any other dA keep the direct form.
+    const float r = dAs[32 * mb];
+    // the same inside the diagonal block if dA falls by so little over its 32 positions that neither
+    // factor leaves the range of float32
+    const bool narrow = r - dAs[32 * mb + 31] <= 60.f;
+    float rowacc[16], em[16];
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       rowacc[v] = 0.f;
-      dAm[v] = dAs[32 * mb + acc_row(v, lane)];
+      em[v] = __expf(dAs[32 * mb + acc_row(v, lane)] - r);
     }
+    // cb through a buffer descriptor: the part of the address that depends on the accumulator register,
+    // the block row and the turn is a scalar offset, the lane's part one register for all sixteen loads
+    const int cb_lane = (4 * half * Q + l32) * (int)sizeof(float);
     for (int nb = 0; nb <= mb; ++nb) {
+      const int n = 32 * nb + l32;
+      // every load is issued before the first use: none of them sits inside a branch
+      float cbv[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        cbv[v] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(
+            cb_desc, cb_lane, ((32 * mb + 8 * (v >> 2) + (v & 3)) * Q + 32 * nb) * (int)sizeof(float), 0));
       floatx16 acc;
       zero_acc(acc);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) mma_group(a[ks], frag_rows(Xs, S::PX, 32 * nb, KG * ks, lane), acc);
-      const int n = 32 * nb + l32;
       const float dAn = dAs[n], wn = dts[n];
       float col = 0.f;
-      // every load is issued before the first use: none of them sits inside a branch
-      float cbv[16];
+      if (falling && nb < mb) {
+        const float gn = wn * __expf(r - dAn);
 #pragma unroll
-      for (int v = 0; v < 16; ++v) cbv[v] = cbg[(int64_t)(32 * mb + acc_row(v, lane)) * Q + n];
+        for (int v = 0; v < 16; ++v) {
+          const float u = acc[v] * cbv[v] * em[v];
+          rowacc[v] = fmaf(u, gn, rowacc[v]);
+          col += u;
+        }
+        col *= gn;
+      } else if (falling && narrow) {  // the diagonal block: exp(r - dA_n) >= 1 here, and bounded
+        const float gn = wn * __expf(r - dAn);
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = 32 * mb + acc_row(v, lane);
-        const float f = acc[v] * cbv[v] * wn * __expf(fminf(dAm[v] - dAn, 0.f));
-        const float w = (n < m && m < limit) ? f : 0.f;
-        rowacc[v] += w;
-        col += w;
+        for (int v = 0; v < 16; ++v) {
+          const float u = n < 32 * mb + acc_row(v, lane) ? acc[v] * cbv[v] * em[v] : 0.f;
+          rowacc[v] = fmaf(u, gn, rowacc[v]);
+          col += u;
+        }
+        col *= gn;
+      } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int m = 32 * mb + acc_row(v, lane);
+          const float f = acc[v] * cbv[v] * wn * __expf(fminf(dAs[m] - dAn, 0.f));
+          const float w = (n < m && m < limit) ? f : 0.f;
+          rowacc[v] += w;
+          col += w;
+        }
       }
       col += __shfl_xor(col, 32);  // the two halves of the wave hold different rows of one column
       if (half == 0) colpart[wave * 256 + n] += col;

@@ -67,6 +67,9 @@ _SIGNATURES = {
     # SSD backward stages
     "ssd_chunk_scan_bwd_dstates": (c_int, _SEQ + _SEQ + [c_int, _P, _P, c_int, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
     "ssd_state_passing_bwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
+    "ssd_chunk_scan_state_passing_bwd_workspace_bytes": (c_size_t, [_I, _I, _I]),
+    "ssd_chunk_scan_state_passing_bwd": (c_int, _SEQ + _SEQ + [c_int, _P, _P, c_int, _P, _P, c_int, _P, _P, _P, c_size_t,
+                                                  _I, _I, _I, _I, _I, _I, _I, _P]),
     "ssd_state_passing_bwd": (c_int, [_P, c_int, _P, _I, _I, _I, _P, c_int, _P, _P, c_int, _P, _P, _P, c_size_t, _I, _I, _I, _I] + _IDS + [_I, _I, _P]),
     "ssd_chunk_state_bwd_db": (c_int, _SEQ + [c_int, _P, _P, _P, c_int] + _SEQ + [_P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
     "ssd_chunk_scan_bwd_dc": (c_int, _SEQ + [c_int, _P, _P, c_int] + _SEQ + [_P, _P, _I, _I, _I, _I, _I, _I, _I] + _IDS + [_P]),
