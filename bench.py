@@ -381,6 +381,7 @@ def make_stages(sets, Q, torch):
     if x0.shape[1] % 128 == 0 and (x0.shape[2] * x0.shape[3] * x0.element_size()) % 512 == 0:
         stages["tile_copy_scan_order"] = lambda i: tile_copy(i, 0)
         stages["tile_copy_best_order"] = lambda i: tile_copy(i, 1)
+        stages["tile_copy_exchange"] = lambda i: tile_copy(i, 2)
     return stages
 
 
@@ -392,7 +393,8 @@ def time_stages(sets, Q, iters, torch, only=None):
     N, L, T = x.shape[0] * x.shape[2], x.shape[1], x.shape[3]
     xb = x.numel() * x.element_size()
     ab = dict(algorithmic_bytes(N, L, T, Q, 2), copy=2 * xb, stream_copy=2 * xb, stream_2in_1out=3 * xb,
-              tile_copy_scan_order=2 * xb, tile_copy_best_order=2 * xb)
+              tile_copy_scan_order=2 * xb, tile_copy_best_order=2 * xb,
+              tile_copy_exchange=2 * xb)
     res = {}
     for name, fn in stages.items():
         if only and name not in only:

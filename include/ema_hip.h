@@ -106,9 +106,10 @@ int ema_stream_copy(const void* a, const void* b, void* dst, size_t bytes, void*
  * kernels: persistent workgroups, tiles of 128 rows x 512 bytes in chunk-major order, 8 bytes per
  * lane and row.  rowmap 0: a wave moves 16 consecutive rows of a tile, as a wave that scans down
  * the rows has to; rowmap 1: the rows of a wave are 8 apart and slabs are rotated against each
- * other, which is the order the memory system sustains the highest rate for.  bench.py reports
- * both next to the plain streaming copy: the first is the ceiling of the scan kernels' own
- * pattern. */
+ * other, which is the order the memory system sustains the highest rate for; rowmap 2: memory is
+ * touched as with rowmap 1 and every wave still gets 16 consecutive rows into its registers, the
+ * rows changing hands through LDS on the way in and on the way out.  bench.py reports all three
+ * next to the plain streaming copy: the first is the ceiling of the scan kernels' own pattern. */
 int ema_tile_pattern_copy(const void* src, void* dst, int64_t slabs, int64_t rows, int64_t row_bytes,
                           int rowmap, void* stream);
 

@@ -583,6 +583,17 @@ int ema_tile_pattern_copy(const void* src, void* dst, int64_t slabs, int64_t row
   if (reinterpret_cast<uintptr_t>(src) % 16 || reinterpret_cast<uintptr_t>(dst) % 16) return EMA_ERR_ALIGN;
   const int64_t pieces = row_bytes / 512, tiles = slabs * (rows / 128) * pieces;
   if (tiles > 0x7fffffff || slabs > 0x7fffffff / pieces) return EMA_ERR_SHAPE;
+  if (rowmap == 2) {
+    constexpr int smem = 2 * 128 * 512;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(tile_copy_exchange_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess)
+      return EMA_ERR_LAUNCH;
+    const int64_t cap = resident_blocks(tile_copy_exchange_kernel, 512, smem);
+    hipLaunchKernelGGL(tile_copy_exchange_kernel, dim3((unsigned)(tiles < cap ? tiles : cap)), dim3(512), smem,
+                       as_stream(stream), static_cast<const char*>(src), static_cast<char*>(dst), (int)slabs,
+                       (int)(rows / 128), (int)pieces, row_bytes, rows * row_bytes);
+    return launched();
+  }
   const int64_t cap = resident_blocks(tile_copy_kernel, 512, 0);
   hipLaunchKernelGGL(tile_copy_kernel, dim3((unsigned)(tiles < cap ? tiles : cap)), dim3(512), 0, as_stream(stream),
                      static_cast<const char*>(src), static_cast<char*>(dst), (int)slabs, (int)(rows / 128), (int)pieces,

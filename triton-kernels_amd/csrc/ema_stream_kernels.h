@@ -56,6 +56,61 @@ __global__ __launch_bounds__(512) void tile_copy_kernel(const char* __restrict__
   }
 }
 
+// The same copy with the interleaved order on the memory side and consecutive rows per wave in
+// registers, as a scanning kernel would need them: rows arrive interleaved, pass through a 64 KB
+// tile in LDS to the wave that owns them, and go back through a second tile to be stored
+// interleaved; the next tile's rows are requested while the current one is exchanged.
+__global__ __launch_bounds__(512) void tile_copy_exchange_kernel(const char* __restrict__ src, char* __restrict__ dst,
+                                                                 int slabs, int row_blocks, int pieces, int64_t row_bytes,
+                                                                 int64_t slab_bytes) {
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  u32x2* tin = reinterpret_cast<u32x2*>(smem);
+  u32x2* tout = reinterpret_cast<u32x2*>(smem + 128 * 512);
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int per_block = slabs * pieces, total = row_blocks * per_block;
+  auto base_of = [&](int id, int& slab) {
+    const int rb = id / per_block, r = id - rb * per_block;
+    slab = r / pieces;
+    const int piece = r - slab * pieces;
+    return (int64_t)slab * slab_bytes + (int64_t)rb * 128 * row_bytes + (int64_t)piece * 512 + lane * 8;
+  };
+  u32x2 v[16];
+  int id = blockIdx.x, slab = 0;
+  int64_t base = 0;
+  if (id < total) {
+    base = base_of(id, slab);
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      v[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(src + base + ((8 * i + g + slab) & 127) * row_bytes));
+  }
+  while (id < total) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) tin[((8 * i + g + slab) & 127) * 64 + lane] = v[i];
+    __syncthreads();
+    u32x2 w[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) w[i] = tin[(16 * g + i) * 64 + lane];
+    const int cur_slab = slab;
+    const int64_t cur_base = base;
+    id += gridDim.x;
+    if (id < total) {
+      base = base_of(id, slab);
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        v[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(src + base + ((8 * i + g + slab) & 127) * row_bytes));
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) tout[(16 * g + i) * 64 + lane] = w[i];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = (8 * i + g + cur_slab) & 127;
+      __builtin_nontemporal_store(tout[row * 64 + lane], reinterpret_cast<u32x2*>(dst + cur_base + row * row_bytes));
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------
 // F1: per-chunk inclusive cumsum of the log-decay.  One wave per (n, c); lane l owns the
 // `per` consecutive positions starting at l * per, sums them serially, and the lane totals
