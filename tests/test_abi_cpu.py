@@ -132,6 +132,18 @@ def test_ssd_validation_happens_before_any_launch():
     assert handle.ssd_chunk_state_passing_fwd(*grp, *seq, 1, fake, fake + 8, None, fake, 1, fake, 1, 64, 2, 1, 64, 64, 64, None) == -3
     # a packed batch must come with the chunking that gives nchunks
     assert handle.ssd_state_passing_fwd(fake, fake, 2, 1, 1, None, fake, 0, fake, 1, 2, 2, 8, fake, 64, 1, 64, 16, None) == -2
+    # the reverse walk (dstates + state passing in one kernel): what it is not written for goes to the two launchers
+    grp128 = [fake, 64 * 128, 128, 128]
+    need = handle.ssd_chunk_scan_state_passing_bwd_workspace_bytes(1, 1, 2)
+    assert need == 1 * 1 * 2 * 8 * 4 and handle.ssd_chunk_scan_state_passing_bwd_workspace_bytes(0, 1, 2) == 0
+
+    def rwalk(dtype=1, chunk=128, states_dtype=1, dA=fake, ddA=fake, ws_bytes=need, dout=seq, hdim=64, dstate=128, out_dtype=1):
+        return handle.ssd_chunk_scan_state_passing_bwd(*grp128, *dout, dtype, dA, fake, states_dtype, None, fake, out_dtype,
+                                                       ddA, None, fake, ws_bytes, 1, 64, 2, 1, hdim, dstate, chunk, None)
+    assert rwalk(dtype=0) == -5 and rwalk(chunk=64) == -5 and rwalk(chunk=160) == -5 and rwalk(states_dtype=0) == -5
+    assert rwalk(hdim=128) == -5 and rwalk(out_dtype=7) == -4
+    assert rwalk(ddA=None) == -1 and rwalk(dA=fake + 4) == -3 and rwalk(ws_bytes=need - 4) == -2
+    assert rwalk(dout=[fake, 64 * 2 * 64, -2 * 64, 64]) == -5  # a reversed view: byte offsets are formed unsigned
 
 
 def test_error_mapping():
