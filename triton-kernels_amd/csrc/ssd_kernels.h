@@ -1897,6 +1897,13 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
     for (int pb = 0; pb < PB; ++pb) zero_acc(acc[mb][pb]);
 
   SSD_TSTAMP(0);
+  // The carried state only takes the lower half of the region it shares with the x tile: the upper half
+  // of the first x tile, rows 128 .. 255, is requested now, ahead of the state, and written to LDS behind
+  // it, so that it costs no round trip of its own after phase A.
+  static_assert(S::kPrev <= (ST / 2) * S::PX * (int)sizeof(T), "the carried state must leave the upper half of the x tile free");
+  constexpr bool kEarly = (ST / 2) * (PW / EPL) / 256 <= 8;  // (eight pieces per thread travel in registers)
+  RowPieces<T, kEarly ? ST / 2 : 32, kEarly ? PW : EPL * 8, S::PX> upper;
+  if constexpr (kEarly) upper.template load<true>(xg, sx.sl, ST / 2, limit, tid);
   // ---- phase A: C . prev, scaled by exp(dA_m)
   {
     constexpr int VPR = N / 4;
@@ -1915,6 +1922,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
 #pragma unroll
     for (int hh = 0; hh < HP; ++hh) sm(hh)[tid] = live ? __expf(dAp[hh][m0 + tid]) : 0.f;
   }
+  if constexpr (kEarly) upper.store(Xs + (ST / 2) * S::PX, ST / 2, limit, tid, NoScale());
   __syncthreads();
   SSD_TSTAMP(1);
 #pragma unroll
@@ -1944,7 +1952,9 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_wide_kernel(
   SSD_TSTAMP(3);
   for (int kt = 0; kt <= st; ++kt) {
     const int k0 = ST * kt;
-    stage_rows<T, ST, PW, NoScale, true>(Xs, xg, sx.sl, k0, limit, tid, NoScale());
+    // (the upper half of the first tile is in LDS already, see above)
+    stage_rows<T, ST / 2, PW, NoScale, true>(Xs, xg, sx.sl, k0, limit, tid, NoScale());
+    if (kt > 0 || !kEarly) stage_rows<T, ST / 2, PW, NoScale, true>(Xs + (ST / 2) * S::PX, xg, sx.sl, k0 + ST / 2, limit, tid, NoScale());
 #pragma unroll
     for (int hh = 0; hh < HP; ++hh) {
       // Below the diagonal the weight of (m, k) is split at the last position r of k's group of
