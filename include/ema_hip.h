@@ -246,6 +246,9 @@ size_t ema_bwd_dx_dA_fused_workspace_bytes(int64_t batch, int64_t nheads, int64_
  * which equals ddA_intra + ddA_next + reverse-cumsum(ddA_prev, + ddA_chunk at the last
  * slot): dx[m] is the gradient of the scan state at row m and y[m-1] is the state that
  * exp(A[m]) multiplies.  When y is not NULL the forward output is written there too.
+ * The decay of a row is taken as exp(min(cs[m] - cs[m-1], 0)) (cs[-1] = 0 at a chunk's first row).
+ * Runs the backward single-pass kernel with both carried states given, so nothing is chained between
+ * workgroups and the workspace only holds the partials.
  * Replaces the four launchers _chunk_scan_chunk_state_bwd_dx, _ema_chunk_state_bwd_db,
  * _ema_chunk_scan_bwd_dC, _ema_chunk_scan_bwd_ddAcs_stable and the torch glue around them,
  * kernels/ema_kernels_bwd/ema_combined_bwd.py:70-79. */

@@ -164,30 +164,6 @@ int launch_chunk_gemm(const void* in, SeqStrides si, int dtype, const float* cs,
   return launch_chunk_scan_t<float, kWalkBnF32, REVERSE>(in, si, cs, vec, out, so, d, st);
 }
 
-template <typename T, int BN>
-int launch_bwd_fused_t(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* cs,
-                       const float* prev, const float* g, void* dx, SeqStrides sdx, void* y,
-                       SeqStrides sy, float* part, const Dims& di, hipStream_t st) {
-  const int ntiles = (int)((di.T + BN - 1) / BN);
-  const int64_t grid = di.N * di.C * ntiles;
-  if (grid > 0x7fffffff) return EMA_ERR_SHAPE;
-  const int smem = WalkCfg<T, BN>::smem_bytes(2, 2);
-  if (y) {
-    auto kernel = bwd_fused_kernel<T, BN, true>;
-    EMA_TRY(allow_smem(kernel, smem));
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), smem, st, (const T*)x, sx,
-                       (const T*)dy, sd, cs, prev, g, (T*)dx, sdx, (T*)y, sy, part, (int)di.nh,
-                       (int)di.L, (int)di.T, (int)di.C, ntiles);
-  } else {
-    auto kernel = bwd_fused_kernel<T, BN, false>;
-    EMA_TRY(allow_smem(kernel, smem));
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), smem, st, (const T*)x, sx,
-                       (const T*)dy, sd, cs, prev, g, (T*)dx, sdx, (T*)nullptr, sy, part, (int)di.nh,
-                       (int)di.L, (int)di.T, (int)di.C, ntiles);
-  }
-  return launched();
-}
-
 template <int MODE>
 int launch_row_dot(const void* x, SeqStrides sx, int dtype, const float* vec, const float* cs,
                    float* out, int raw, const Dims& d, hipStream_t st) {
@@ -381,7 +357,7 @@ int launch_bwd_tile_k(const void* x, SeqStrides sx, const void* dy, SeqStrides s
   EMA_TRY(launch_timed(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), st, ev0, ev1, (const T*)x,
                        sx, (const T*)dy, sd, A, sa, prev128, (T*)dx, sdx, (T*)y, sy, part, dfinal, dinit, w.hdr,
                        w.decw, w.status, (int)di.nh, (int)di.L, (int)di.T, (int)di.C, ntiles, (int)cols,
-                       (int)total, make_order(di, ntiles)));
+                       (int)total, make_order(di, ntiles), (const float*)nullptr));
   return launched();
 }
 
@@ -402,22 +378,47 @@ constexpr int tile_parts_per_dim(int64_t T) {
   return (int)((T + 64 * S::BWD_CPL - 1) / (64 * S::BWD_CPL));
 }
 
-// dx, optionally the recomputed y, and the log-decay gradient in one pass over x and dy.
-// di is the 128-row chunking the kernel works on (cs, prev, g follow it); d fixes the
-// (N, C, Q) layout of ddA.
+// dx, optionally the recomputed y, and the log-decay gradient in one pass over x and dy, with the
+// states entering every 128-row chunk from both sides given (prev, g): the backward single-pass
+// kernel with nothing to chain.  di is the 128-row chunking the kernel works on (cs, prev, g follow
+// it); d fixes the (N, C, Q) layout of ddA.
+template <typename T, typename S>
+int launch_bwd_tile_given(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* cs,
+                          const float* prev, const float* g, void* dx, SeqStrides sdx, void* y, SeqStrides sy,
+                          float* part, const Dims& di, hipStream_t st) {
+  using Cfg = TileCfg<T, S::BWD_CPL, S::BWD_RPL>;
+  constexpr int BN = Cfg::BN, NT = Cfg::NT;
+  const int ntiles = (int)((di.T + BN - 1) / BN);
+  const int64_t cols = di.N * ntiles, total = cols * di.C;
+  if (total > 0x7fffffff) return EMA_ERR_SHAPE;
+  const SeqStrides sa{di.nh * di.C * kTileRows, 1, di.C * kTileRows};  // cs is dense (N, C, 128)
+  auto launch = [&](auto kernel) {
+    const int64_t cap = resident_blocks(kernel, NT, 0);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(NT), 0, st, (const T*)x, sx,
+                       (const T*)dy, sd, cs, sa, prev, (T*)dx, sdx, (T*)y, sy, part, (const float*)nullptr,
+                       (float*)nullptr, (ChainHeader*)nullptr, (u64*)nullptr, (u64*)nullptr, (int)di.nh, (int)di.L,
+                       (int)di.T, (int)di.C, ntiles, (int)cols, (int)total, make_order(di, ntiles), g);
+  };
+  if (y) launch(bwd_tile_kernel<T, S::BWD_CPL, S::BWD_RPL, S::BWD_MINW, true, false, true>);
+  else launch(bwd_tile_kernel<T, S::BWD_CPL, S::BWD_RPL, S::BWD_MINW, false, false, true>);
+  return launched();
+}
+
 int run_bwd_fused(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, int dtype,
                   const float* cs, const float* prev, const float* g, void* dx, SeqStrides sdx,
                   void* y, SeqStrides sy, float* ddA, float* part, const Dims& d, const Dims& di,
                   hipStream_t st) {
-  if (dtype == EMA_BF16)
-    EMA_TRY((launch_bwd_fused_t<bf16_t, kWalkBnBf16>(x, sx, dy, sd, cs, prev, g, dx, sdx, y, sy, part,
-                                                     di, st)));
-  else
-    EMA_TRY((launch_bwd_fused_t<float, kWalkBnF32>(x, sx, dy, sd, cs, prev, g, dx, sdx, y, sy, part,
-                                                   di, st)));
+  int parts;
+  if (dtype == EMA_BF16) {
+    EMA_TRY((launch_bwd_tile_given<bf16_t, TileBf16>(x, sx, dy, sd, cs, prev, g, dx, sdx, y, sy, part, di, st)));
+    parts = tile_parts_per_dim<TileBf16>(di.T);
+  } else {
+    EMA_TRY((launch_bwd_tile_given<float, TileF32>(x, sx, dy, sd, cs, prev, g, dx, sdx, y, sy, part, di, st)));
+    parts = tile_parts_per_dim<TileF32>(di.T);
+  }
   const int64_t total = d.N * d.C * d.Q;
   hipLaunchKernelGGL(dA_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, part,
-                     ddA, (int)d.L, (int)d.Q, (int)d.C, (int)di.C, bwd_col_tiles(di, dtype), total);
+                     ddA, (int)d.L, (int)d.Q, (int)d.C, (int)di.C, parts, total);
   return launched();
 }
 

@@ -229,6 +229,20 @@ __device__ __forceinline__ void tile_coef_load(float* raw, const float* __restri
 #pragma unroll
   for (int i = 0; i < RPL; ++i) raw[i] = i < nrows ? A[(int64_t)i * a_sl] : 0.f;
 }
+// The same from the inclusive cumsum of the log-decay over the 128-row chunk that the tile is
+// (cs points at the wave's first row, dense along the rows): raw[i] = cs[i] - cs[i - 1], and cs[0]
+// itself for the chunk's first row.
+template <int RPL>
+__device__ __forceinline__ void tile_coef_load_cumsum(float* raw, const float* __restrict__ cs, int nrows,
+                                                      bool chunk_start) {
+  float before = chunk_start ? 0.f : cs[-1];
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) {
+    const float here = i < nrows ? cs[i] : before;
+    raw[i] = here - before;
+    before = here;
+  }
+}
 // Log-decay form: a[i] = exp(min(A[row], 0)).  Probability form: a[i] = p[row].  Scalar registers.
 template <int RPL, bool XP>
 __device__ __forceinline__ void tile_decays(float* a, const float* raw) {
@@ -437,14 +451,21 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void fwd_tile_kernel(
 // state; the forward values y are then recomputed while the reverse look-back is under way.
 // As in the forward, the rows of the next tile are requested behind the stores of this one.
 // ------------------------------------------------------------------------------------
-template <typename T, int CPL, int RPL, int MINW, bool WRITE_Y, bool XP>
+//
+// GIVEN: the reverse state entering every tile is an input as well (given[n,c,:], the gradient of the
+// state that leaves chunk c, as the reverse state passing of the per-stage path computes it), and A
+// is the per-chunk inclusive cumsum of the log-decay, dense (N, C, 128), described by sa.  Nothing
+// is chained then: no workspace words, no tickets (workgroup w takes the tiles w, w + grid, ...), and
+// hdr / decw / status are not touched.
+template <typename T, int CPL, int RPL, int MINW, bool WRITE_Y, bool XP, bool GIVEN = false>
 __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     const T* __restrict__ x, SeqStrides sx, const T* __restrict__ dy, SeqStrides sd,
     const float* __restrict__ A, SeqStrides sa, const float* __restrict__ prev, T* __restrict__ dx,
     SeqStrides sdx, T* __restrict__ y, SeqStrides sy, float* __restrict__ part,
     const float* __restrict__ dfinal, float* __restrict__ dinit, ChainHeader* __restrict__ hdr,
     u64* __restrict__ decw, u64* __restrict__ status, int nh, int L, int Tdim, int C, int ntiles, int cols,
-    int total, const TileOrder ord) {
+    int total, const TileOrder ord, const float* __restrict__ given = nullptr) {
+  static_assert(!(GIVEN && XP), "the given-state form reads a cumsum of log-decays");
   using W = TileCfg<T, CPL, RPL>;
   constexpr int BN = W::BN, NW = W::NW, NG = W::NG, NT = W::NT;
   static_assert(2 * BN <= NT, "one thread per column and direction");
@@ -458,11 +479,19 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
   const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const unsigned off = (unsigned)lane * CPL;
   const int kf = (int)threadIdx.x - BN;  // column of the threads that chain the forward group states
-  const ChainCtl ctl = chain_enter(hdr);
-
-  if (threadIdx.x == 0) s_ticket[0] = (int)atomicAdd(&hdr->ticket, 1u);
-  __syncthreads();
-  int cur = s_ticket[0], buf = 0, slot = 1;
+  ChainCtl ctl;
+  if constexpr (!GIVEN) {
+    ctl = chain_enter(hdr);
+    if (threadIdx.x == 0) s_ticket[0] = (int)atomicAdd(&hdr->ticket, 1u);
+    __syncthreads();
+  }
+  int cur = GIVEN ? (int)blockIdx.x : s_ticket[0], buf = 0, slot = 1;
+  // the coefficients of this wave's rows of tile tt
+  auto coef_load = [&](float* raw, const ChainTile& tt, int64_t row, int nrows) {
+    const float* ap = A + (int64_t)tt.b * sa.sb + (int64_t)tt.h * sa.sh + row * sa.sl;
+    if constexpr (GIVEN) tile_coef_load_cumsum<RPL>(raw, ap, nrows, grp == 0);
+    else tile_coef_load<RPL>(raw, ap, sa.sl, nrows);
+  };
   RowWords<NW> dr[RPL], xr[RPL];
   float araw[RPL];
   float p_in = 0.f;
@@ -476,12 +505,14 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     for (int i = 0; i < RPL; ++i) dr[i] = tile_load_row<NW, kStreamBwdLoad>(gd, sd.sl, i, at);
 #pragma unroll
     for (int i = 0; i < RPL; ++i) xr[i] = tile_load_row<NW, kStreamBwdLoad>(gx, sx.sl, i, at);
-    tile_coef_load<RPL>(araw, A + (int64_t)t.b * sa.sb + (int64_t)t.h * sa.sh + row0 * sa.sl, sa.sl, at.nrows);
+    coef_load(araw, t, row0, at.nrows);
     if (kf >= 0 && kf < BN && t.col0 + kf < Tdim) p_in = prev[(int64_t)t.chunk_id * Tdim + t.col0 + kf];
   }
   while (cur < total) {
-    int future = 0;
-    if (threadIdx.x == 0) future = (int)atomicAdd(&hdr->ticket, 1u);
+    int future = GIVEN ? cur + (int)gridDim.x : 0;
+    if constexpr (!GIVEN) {
+      if (threadIdx.x == 0) future = (int)atomicAdd(&hdr->ticket, 1u);
+    }
     EMA_TSTAMP_DECL;
     EMA_TSTAMP(0);
     EMA_TSTAMP_VALUE(7, (long long)blockIdx.x);
@@ -541,10 +572,12 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
         loc = fmaf(dg[g], loc, rg[g]);
         dec *= dg[g];
       }
-      if (!last) {
-        if (k == 0) chain_publish(dws + t.c, ctl.epoch, kStateAggregate, dec);
-        chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStateAggregate, loc);
-        look.begin(words, t.c);
+      if constexpr (!GIVEN) {
+        if (!last) {
+          if (k == 0) chain_publish(dws + t.c, ctl.epoch, kStateAggregate, dec);
+          chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStateAggregate, loc);
+          look.begin(words, t.c);
+        }
       }
     } else if (kf < BN) {
       float sg[NG], dg[NG];
@@ -586,21 +619,27 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     if (threadIdx.x < BN) {
       const int k = threadIdx.x;
       float h_in;
-      if (!last) h_in = look.finish(words, dws, C, ctl);
-      else h_in = (dfinal && last && t.col0 + k < Tdim) ? dfinal[(int64_t)t.n * Tdim + t.col0 + k] : 0.f;
-      EMA_TSTAMP(6);
-      const float h_out = fmaf(dec, h_in, loc);
-      chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStatePrefix, h_out);
-      if (dinit && t.c == 0 && t.col0 + k < Tdim) dinit[(int64_t)t.n * Tdim + t.col0 + k] = h_out;
+      if constexpr (GIVEN) {
+        h_in = t.col0 + k < Tdim ? given[(int64_t)t.chunk_id * Tdim + t.col0 + k] : 0.f;
+      } else {
+        if (!last) h_in = look.finish(words, dws, C, ctl);
+        else h_in = (dfinal && last && t.col0 + k < Tdim) ? dfinal[(int64_t)t.n * Tdim + t.col0 + k] : 0.f;
+        EMA_TSTAMP(6);
+        const float h_out = fmaf(dec, h_in, loc);
+        chain_publish(words + (int64_t)t.c * BN, ctl.epoch, kStatePrefix, h_out);
+        if (dinit && t.c == 0 && t.col0 + k < Tdim) dinit[(int64_t)t.n * Tdim + t.col0 + k] = h_out;
+      }
       sH[buf][k] = h_in;
     }
-    if (threadIdx.x == 0) s_ticket[slot] = future;
+    if constexpr (!GIVEN) {
+      if (threadIdx.x == 0) s_ticket[slot] = future;
+    }
     __syncthreads();
     EMA_TSTAMP(3);
 
     // 3. final reverse pass: dx, and the dots with the row before; behind each stored row the
     // same rows of the next tile are requested
-    const int next = s_ticket[slot];
+    const int next = GIVEN ? future : s_ticket[slot];
     const bool more = next < total;
     const ChainTile tn = chain_decode<true, BN>(more ? next : 0, ord, L);
     const TileAt atn = tile_at<RPL>(tn.limit, grp, tn.col0 + lane * CPL < Tdim);
@@ -647,7 +686,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
       if (lane < RPL)
         part[((int64_t)t.chunk_id * ntiles + t.ctile) * kTileRows + RPL * grp + lane] = lane < at.nrows ? dA : 0.f;
       if (more) {
-        tile_coef_load<RPL>(araw, A + (int64_t)tn.b * sa.sb + (int64_t)tn.h * sa.sh + rown * sa.sl, sa.sl, atn.nrows);
+        coef_load(araw, tn, rown, atn.nrows);
         p_in = (kf >= 0 && kf < BN && tn.col0 + kf < Tdim) ? prev[(int64_t)tn.chunk_id * Tdim + tn.col0 + kf] : 0.f;
       }
     }
@@ -659,7 +698,9 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
     slot ^= 1;
     buf ^= 1;
   }
-  if (threadIdx.x == 0) chain_leave(hdr, ctl);
+  if constexpr (!GIVEN) {
+    if (threadIdx.x == 0) chain_leave(hdr, ctl);
+  }
 }
 
 // out[b, p, h] = sum over the column tiles of part[n, p / 128, tile, p % 128]: the gradient of

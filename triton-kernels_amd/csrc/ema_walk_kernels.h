@@ -332,110 +332,6 @@ __global__ __launch_bounds__(256) void chunk_scan_walk_kernel(
   }
 }
 
-// ------------------------------------------------------------------------------------
-// Fused backward over one 128-row chunk (the caller chunks the sequence by 128 for this
-// kernel whatever the chunk size of the interface):
-//   dx[m]  = exp(cs[127]-cs[m]) * g + sum_{k>=m} exp(cs[k]-cs[m]) * dy[k]           (B3)
-//   y[m]   = exp(cs[m]) * prev + sum_{k<=m} exp(cs[m]-cs[k]) * x[k]                  (F4, not stored
-//            unless WRITE_Y)
-//   dA[m]  = exp(A[m]) * <dx[m], y[m-1]>,  y[-1] = prev, A[m] = cs[m] - cs[m-1]
-// The last line is the whole log-decay gradient (the sum of the reference's B4, B5, B6 and
-// chunk terms), because dx[m] is dL/dy-state at row m and y[m-1] is the state it multiplies.
-// Each workgroup reduces dA over its BN columns and writes the partial to
-// part[(chunk * ntiles + ctile) * 128 + m]; dA_reduce_kernel sums the column tiles.
-// ------------------------------------------------------------------------------------
-template <typename T, int BN, bool WRITE_Y>
-__global__ __launch_bounds__(256) void bwd_fused_kernel(
-    const T* __restrict__ x, SeqStrides sx, const T* __restrict__ dy, SeqStrides sd,
-    const float* __restrict__ cs, const float* __restrict__ prev, const float* __restrict__ g,
-    T* __restrict__ dx, SeqStrides sdx, T* __restrict__ y, SeqStrides sy, float* __restrict__ part,
-    int nh, int L, int Tdim, int C, int ntiles) {
-  using Cfg = WalkCfg<T, BN>;
-  constexpr int Q = kTileRows;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  T* xt = reinterpret_cast<T*>(smem);
-  T* dt = xt + Cfg::TILE;
-  const WalkScratch s = walk_scratch<T, BN, 2>(smem, 2);
-
-  const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63;
-  const int l32 = lane & 31;
-  const int ctile = (int)(blockIdx.x % ntiles);
-  const int64_t chunk_id = blockIdx.x / ntiles;
-  const int64_t n = chunk_id / C;
-  const int c = (int)(chunk_id - n * C);
-  const int64_t b = n / nh;
-  const int h = (int)(n - b * nh);
-  const int limit = min(Q, L - c * Q);
-  const int col0 = ctile * BN;
-  const float* csp = cs + chunk_id * Q;
-
-  float p_in = 0.f, h_in = 0.f;
-  if (tid < BN && col0 + tid < Tdim) {
-    p_in = prev[chunk_id * Tdim + col0 + tid];
-    h_in = g[chunk_id * Tdim + col0 + tid];
-  }
-  walk_load_cs<true, true>(s, csp, 0, Q, tid);
-  walk_load_tile<T, BN>(xt, x + b * sx.sb + h * sx.sh + (int64_t)c * Q * sx.sl, sx.sl, 0, limit, col0,
-                        Tdim, tid);
-  walk_load_tile<T, BN>(dt, dy + b * sd.sb + h * sd.sh + (int64_t)c * Q * sd.sl, sd.sl, 0, limit,
-                        col0, Tdim, tid);
-  __syncthreads();
-  walk_block_state<T, BN>(xt, s.wf, s.sj, wave, lane);
-  walk_block_state<T, BN>(dt, s.wr, s.rj, wave, lane);
-  __syncthreads();
-  if (tid < BN) {
-    walk_chain_fwd<BN>(s, p_in, tid);
-    walk_chain_rev<BN>(s, h_in, tid);
-  }
-  __syncthreads();
-
-  const float cm = s.csT[32 * wave + l32 + 1];
-  floatx16 dacc[Cfg::NDB];
-  {
-    Vec16<T> hi[Cfg::NG], lo[Cfg::NG];
-    walk_decay_frags<T, true>(s.csT, wave, lane, hi, lo);
-    const float u = __expf(fminf(s.csT[32 * wave + 32] - cm, 0.f));
-#pragma unroll
-    for (int db = 0; db < Cfg::NDB; ++db)
-      dacc[db] = walk_block_mma<T, BN>(dt, hi, lo, s.Hj + wave * BN, u, wave, db, lane);
-  }
-  float dot = 0.f;
-  {
-    Vec16<T> hi[Cfg::NG], lo[Cfg::NG];
-    walk_decay_frags<T, false>(s.csT, wave, lane, hi, lo);
-    const float u = __expf(fminf(cm - s.csT[32 * wave], 0.f));
-    const float* pw = s.Pj + wave * BN;
-#pragma unroll
-    for (int db = 0; db < Cfg::NDB; ++db) {
-      const floatx16 yacc = walk_block_mma<T, BN>(xt, hi, lo, pw, u, wave, db, lane);
-      // y[m-1] sits one lane to the left; the wave's first row takes the carried state P_w
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const float left = __int_as_float(
-            __builtin_amdgcn_update_dpp(0, __float_as_int(yacc[v]), 0x138 /* wave_shr:1 */, 0xf, 0xf, false));
-        const float ym1 = l32 == 0 ? pw[db * 32 + acc_row(v, lane)] : left;
-        dot = fmaf(dacc[db][v], ym1, dot);
-      }
-      if (WRITE_Y) walk_pack_block<T, BN>(xt, yacc, wave, db, lane);
-    }
-  }
-  // the two half-waves hold disjoint column subsets of the same rows
-  dot += __shfl_xor(dot, 32);
-  if (lane < 32) {
-    const int m = 32 * wave + lane;
-    const float a_m = cm - s.csT[m];  // A[m] = cs[m] - cs[m-1], cs[-1] = 0
-    part[(chunk_id * ntiles + ctile) * (int64_t)Q + m] = m < limit ? __expf(a_m) * dot : 0.f;
-  }
-#pragma unroll
-  for (int db = 0; db < Cfg::NDB; ++db) walk_pack_block<T, BN>(dt, dacc[db], wave, db, lane);
-  walk_store_rows<T, BN>(dt, dx + b * sdx.sb + h * sdx.sh + (int64_t)c * Q * sdx.sl, sdx.sl, 0, limit,
-                         col0, Tdim, wave, lane);
-  if (WRITE_Y)
-    walk_store_rows<T, BN>(xt, y + b * sy.sb + h * sy.sh + (int64_t)c * Q * sy.sl, sy.sl, 0, limit,
-                           col0, Tdim, wave, lane);
-}
-
 // ddA[n, p / Q, p % Q] = sum over column tiles of part[n, p / 128, tile, p % 128] for
 // positions p < L; the padded slots of the last chunk are set to 0.  One thread per slot.
 __global__ __launch_bounds__(256) void dA_reduce_kernel(const float* __restrict__ part,
