@@ -21,9 +21,10 @@ contraction launchers with their dense-FLOP rate), the long-sequence configurati
 Mamba-2 SSD configuration 5 and `ref_f32_fwd`, the forward on the workload of the reference's own
 benchmark script (float32, b16 L8192 d1024) beside the only figures the reference publishes.
 `stage_launchers` times every per-stage launcher of the reference's interface on its own, and
-four copies that bound what a kernel can reach here: a linear one, torch's, and two that move the
-tensor in the tile order of the single-pass kernels (rows of a wave consecutive, as a scan needs
-them, or interleaved, as the memory system prefers them).  `cpu_baseline` is the sequential CPU
+the copies that bound what a kernel can reach here: a linear one, torch's, and four that move the
+tensor in the tile order of the single-pass kernels (in the kernels' own shape, with fewer and
+longer waves, with the rows interleaved as the memory system prefers them, and interleaved with an
+exchange through LDS).  `cpu_baseline` is the sequential CPU
 oracle timed on a bounded sample and scaled to the full workload.
 """
 import argparse
@@ -368,8 +369,9 @@ def make_stages(sets, Q, torch):
     stages["stream_2in_1out"] = lambda i: stream(i, True)
 
     # the same bytes in the access pattern of the single-pass kernels (tiles of 128 rows x 512
-    # bytes, persistent workgroups): with the row order a scanning wave needs, and with the one the
-    # memory system likes best
+    # bytes, one persistent workgroup per compute unit): in the shape the two kernels load and
+    # store in (sixteen waves with 8 consecutive rows each), with eight waves of 16 rows, in the
+    # order the memory system likes best, and in that order with the rows handed on through LDS
     def tile_copy(i, rowmap):
         x, A, dy = sets[i % len(sets)]
         o = outs[i % len(sets)]
@@ -380,6 +382,7 @@ def make_stages(sets, Q, torch):
     x0 = sets[0][0]
     if x0.shape[1] % 128 == 0 and (x0.shape[2] * x0.shape[3] * x0.element_size()) % 512 == 0:
         stages["tile_copy_scan_order"] = lambda i: tile_copy(i, 0)
+        stages["tile_copy_scan_order_8_waves"] = lambda i: tile_copy(i, 3)
         stages["tile_copy_best_order"] = lambda i: tile_copy(i, 1)
         stages["tile_copy_exchange"] = lambda i: tile_copy(i, 2)
     return stages
@@ -393,8 +396,8 @@ def time_stages(sets, Q, iters, torch, only=None):
     N, L, T = x.shape[0] * x.shape[2], x.shape[1], x.shape[3]
     xb = x.numel() * x.element_size()
     ab = dict(algorithmic_bytes(N, L, T, Q, 2), copy=2 * xb, stream_copy=2 * xb, stream_2in_1out=3 * xb,
-              tile_copy_scan_order=2 * xb, tile_copy_best_order=2 * xb,
-              tile_copy_exchange=2 * xb)
+              tile_copy_scan_order=2 * xb, tile_copy_scan_order_8_waves=2 * xb,
+              tile_copy_best_order=2 * xb, tile_copy_exchange=2 * xb)
     res = {}
     for name, fn in stages.items():
         if only and name not in only:

@@ -103,13 +103,15 @@ int ema_stream_copy(const void* a, const void* b, void* dst, size_t bytes, void*
 
 /* Measurement aid (no counterpart in the reference): copies a (slabs, rows, row_bytes) byte tensor
  * (rows a multiple of 128, row_bytes a multiple of 512) in the access pattern of the single-pass
- * kernels: persistent workgroups, tiles of 128 rows x 512 bytes in chunk-major order, 8 bytes per
- * lane and row.  rowmap 0: a wave moves 16 consecutive rows of a tile, as a wave that scans down
- * the rows has to; rowmap 1: the rows of a wave are 8 apart and slabs are rotated against each
- * other, which is the order the memory system sustains the highest rate for; rowmap 2: memory is
- * touched as with rowmap 1 and every wave still gets 16 consecutive rows into its registers, the
- * rows changing hands through LDS on the way in and on the way out.  bench.py reports all three
- * next to the plain streaming copy: the first is the ceiling of the scan kernels' own pattern. */
+ * kernels: one persistent workgroup per compute unit, tiles of 128 rows x 512 bytes in chunk-major
+ * order, 8 bytes per lane and row.  rowmap 0: sixteen waves with 8 consecutive rows each, the shape
+ * in which the two kernels load and store; rowmap 3: eight waves with 16 consecutive rows each;
+ * rowmap 1: eight waves, the rows of a wave 8 apart and slabs rotated against each other, which is
+ * the order the memory system sustains the highest rate for; rowmap 2: memory is touched as with
+ * rowmap 1 and every wave still gets 16 consecutive rows into its registers, the rows changing
+ * hands through LDS on the way in and on the way out.  Other values: EMA_ERR_UNSUPPORTED.  bench.py
+ * reports all four next to the plain streaming copy: the first is the ceiling of the scan kernels'
+ * own pattern. */
 int ema_tile_pattern_copy(const void* src, void* dst, int64_t slabs, int64_t rows, int64_t row_bytes,
                           int rowmap, void* stream);
 

@@ -9,7 +9,7 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("slabs,rows,row_bytes", [(3, 256, 1024), (16, 128, 4096), (5, 384, 512)])
-@pytest.mark.parametrize("rowmap", [0, 1, 2], ids=["scan_order", "best_order", "exchange"])
+@pytest.mark.parametrize("rowmap", [0, 1, 2, 3], ids=["scan_order", "best_order", "exchange", "scan_order_8_waves"])
 def test_tile_pattern_copy_copies(rowmap, slabs, rows, row_bytes, device):
     from kernels import _lib
 
@@ -32,6 +32,7 @@ def test_tile_pattern_copy_rejects_other_shapes(device):
     assert f(buf.data_ptr(), buf.data_ptr(), 2, 100, 512, 0, s) == -2   # rows not a multiple of 128
     assert f(buf.data_ptr(), buf.data_ptr(), 2, 128, 500, 2, s) == -2   # row bytes not a multiple of 512
     assert f(None, buf.data_ptr(), 2, 128, 512, 1, s) == -1
+    assert f(buf.data_ptr(), buf.data_ptr(), 2, 128, 512, 9, s) == -5   # no such pattern
 
 
 @pytest.mark.parametrize("two", [False, True], ids=["one_input", "two_inputs"])

@@ -584,21 +584,34 @@ int ema_tile_pattern_copy(const void* src, void* dst, int64_t slabs, int64_t row
   if (reinterpret_cast<uintptr_t>(src) % 16 || reinterpret_cast<uintptr_t>(dst) % 16) return EMA_ERR_ALIGN;
   const int64_t pieces = row_bytes / 512, tiles = slabs * (rows / 128) * pieces;
   if (tiles > 0x7fffffff || slabs > 0x7fffffff / pieces) return EMA_ERR_SHAPE;
-  if (rowmap == 2) {
+  if (rowmap < 0 || rowmap > 3) return EMA_ERR_UNSUPPORTED;
+  // one workgroup per compute unit, as the single-pass kernels run
+  int dev = 0, ncu = 256;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+    return EMA_ERR_LAUNCH;
+  const dim3 grid((unsigned)(tiles < ncu ? tiles : ncu));
+  const char* s8 = static_cast<const char*>(src);
+  char* d8 = static_cast<char*>(dst);
+  const int rb = (int)(rows / 128);
+  hipStream_t st = as_stream(stream);
+  if (rowmap == 0) {
+    hipLaunchKernelGGL(tile_copy_shape_kernel<16>, grid, dim3(1024), 0, st, s8, d8, (int)slabs, rb, (int)pieces, row_bytes,
+                       rows * row_bytes);
+  } else if (rowmap == 3) {
+    hipLaunchKernelGGL(tile_copy_shape_kernel<8>, grid, dim3(512), 0, st, s8, d8, (int)slabs, rb, (int)pieces, row_bytes,
+                       rows * row_bytes);
+  } else if (rowmap == 1) {
+    hipLaunchKernelGGL(tile_copy_kernel, grid, dim3(512), 0, st, s8, d8, (int)slabs, rb, (int)pieces, row_bytes,
+                       rows * row_bytes);
+  } else {
     constexpr int smem = 2 * 128 * 512;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(tile_copy_exchange_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess)
       return EMA_ERR_LAUNCH;
-    const int64_t cap = resident_blocks(tile_copy_exchange_kernel, 512, smem);
-    hipLaunchKernelGGL(tile_copy_exchange_kernel, dim3((unsigned)(tiles < cap ? tiles : cap)), dim3(512), smem,
-                       as_stream(stream), static_cast<const char*>(src), static_cast<char*>(dst), (int)slabs,
-                       (int)(rows / 128), (int)pieces, row_bytes, rows * row_bytes);
-    return launched();
+    hipLaunchKernelGGL(tile_copy_exchange_kernel, grid, dim3(512), smem, st, s8, d8, (int)slabs, rb, (int)pieces,
+                       row_bytes, rows * row_bytes);
   }
-  const int64_t cap = resident_blocks(tile_copy_kernel, 512, 0);
-  hipLaunchKernelGGL(tile_copy_kernel, dim3((unsigned)(tiles < cap ? tiles : cap)), dim3(512), 0, as_stream(stream),
-                     static_cast<const char*>(src), static_cast<char*>(dst), (int)slabs, (int)(rows / 128), (int)pieces,
-                     row_bytes, rows * row_bytes, rowmap ? 1 : 0);
   return launched();
 }
 

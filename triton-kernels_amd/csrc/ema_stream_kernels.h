@@ -22,22 +22,42 @@ __global__ __launch_bounds__(256) void stream_copy_kernel(const uint4* __restric
 }
 
 // ------------------------------------------------------------------------------------
-// Copy in the access pattern of the single-pass kernels (measurement aid).  The tensor is
-// (slabs, rows, row_bytes) bytes; a tile is 128 rows x 512 bytes; one persistent workgroup of 8
-// waves per compute unit takes the tiles in chunk-major order (all slabs and row pieces of rows
-// 0..127, then of rows 128..255, ...), workgroup w the tiles w, w + grid, ...; a lane moves 8 bytes
-// of 16 rows per tile.
-//   rowmap 0: wave g moves rows 16 g .. 16 g + 15 of the tile: consecutive rows per wave, which is
-//             what a scan down the rows needs;
-//   rowmap 1: instruction i of wave g moves row (8 i + g + slab) % 128: the rows of a wave are 8
-//             apart, the waves of a workgroup touch neighbouring rows, and slabs (whose addresses
-//             differ by a large power of two) are rotated against each other.
-// On this part the second order is what the memory system likes (6.2 TB/s against 5.4 TB/s at
-// b16 nh2 d1024 L4096, bfloat16); a wave that scans needs the first.
+// Copies in the access pattern of the single-pass kernels (measurement aids).  The tensor is
+// (slabs, rows, row_bytes) bytes; a tile is 128 rows x 512 bytes; one persistent workgroup per
+// compute unit takes the tiles in chunk-major order (all slabs and row pieces of rows 0..127, then
+// of rows 128..255, ...), workgroup w the tiles w, w + grid, ...; a lane moves 8 bytes of each of
+// its rows, a wave's loads of a tile all go out before its stores.
+//   tile_copy_shape_kernel<16>: sixteen waves, wave g moves rows 8 g .. 8 g + 7: the shape in which
+//             fwd_tile_kernel and bwd_tile_kernel load and store;
+//   tile_copy_shape_kernel<8>:  eight waves with 16 consecutive rows each;
+//   tile_copy_kernel:           eight waves, instruction i of wave g moves row (8 i + g + slab) % 128:
+//             the rows of a wave are 8 apart, the waves of a workgroup touch neighbouring rows, and
+//             slabs (whose addresses differ by a large power of two) are rotated against each other.
+// At b16 nh2 d1024 L4096, bfloat16, these sustain 5.7, 5.2 and 6.0 TB/s.
 // ------------------------------------------------------------------------------------
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void tile_copy_shape_kernel(const char* __restrict__ src, char* __restrict__ dst,
+                                                                     int slabs, int row_blocks, int pieces,
+                                                                     int64_t row_bytes, int64_t slab_bytes) {
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+  constexpr int RPW = 128 / WAVES;  // rows of a wave
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int per_block = slabs * pieces, total = row_blocks * per_block;
+  for (int id = blockIdx.x; id < total; id += gridDim.x) {
+    const int rb = id / per_block, r = id - rb * per_block;
+    const int slab = r / pieces, piece = r - slab * pieces;
+    const int64_t base = (int64_t)slab * slab_bytes + ((int64_t)rb * 128 + RPW * g) * row_bytes + (int64_t)piece * 512 + lane * 8;
+    u32x2 v[RPW];
+#pragma unroll
+    for (int i = 0; i < RPW; ++i) v[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(src + base + i * row_bytes));
+#pragma unroll
+    for (int i = 0; i < RPW; ++i) __builtin_nontemporal_store(v[i], reinterpret_cast<u32x2*>(dst + base + i * row_bytes));
+  }
+}
+
 __global__ __launch_bounds__(512) void tile_copy_kernel(const char* __restrict__ src, char* __restrict__ dst,
                                                         int slabs, int row_blocks, int pieces, int64_t row_bytes,
-                                                        int64_t slab_bytes, int rowmap) {
+                                                        int64_t slab_bytes) {
   typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
   const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
   const int per_block = slabs * pieces, total = row_blocks * per_block;
@@ -48,7 +68,7 @@ __global__ __launch_bounds__(512) void tile_copy_kernel(const char* __restrict__
     u32x2 v[16];
     int row[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) row[i] = rowmap ? ((8 * i + g + slab) & 127) : 16 * g + i;
+    for (int i = 0; i < 16; ++i) row[i] = (8 * i + g + slab) & 127;
 #pragma unroll
     for (int i = 0; i < 16; ++i) v[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(src + base + row[i] * row_bytes));
 #pragma unroll
