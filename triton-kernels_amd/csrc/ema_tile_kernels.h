@@ -614,6 +614,20 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
         if (WRITE_Y && i < at.nrows && at.cok) row_store<NW>(g + (int64_t)i * sy.sl, row_pack<T, CPL, NW>(s));
       }
     }
+    // Given-state form: the x rows of the next tile are requested here, where this tile's have been
+    // used for the last time, and not behind the stores of the final pass (0.159 -> 0.152 ms at b16
+    // nh2 d1024 L4096).  The chained form must not: rows requested while the look-back is under way
+    // slow its polls down, and everybody waits for those (158 -> 163 us).
+    if constexpr (GIVEN) {
+      if (future < total) {
+        const ChainTile tx = chain_decode<true, BN>(future, ord, L);
+        const TileAt atx = tile_at<RPL>(tx.limit, grp, tx.col0 + lane * CPL < Tdim);
+        const T* gx = x + (int64_t)tx.b * sx.sb + (int64_t)tx.h * sx.sh +
+                      ((int64_t)tx.c * kTileRows + RPL * grp) * sx.sl + tx.col0 + off;
+#pragma unroll
+        for (int i = 0; i < RPL; ++i) xr[i] = tile_load_row<NW, kStreamBwdLoad>(gx, sx.sl, i, atx);
+      }
+    }
 
     // 2b. the reverse state entering the tile (the waves that own no column go straight on)
     if (threadIdx.x < BN) {
@@ -674,7 +688,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), MINW) void bwd_tile_kernel(
         }
         if (more) {
           dr[i] = tile_load_row<NW, kStreamBwdLoad>(gd, sd.sl, i, atn);
-          xr[i] = tile_load_row<NW, kStreamBwdLoad>(gx, sx.sl, i, atn);
+          if (!GIVEN) xr[i] = tile_load_row<NW, kStreamBwdLoad>(gx, sx.sl, i, atn);
         }
 #pragma unroll
         for (int e = 0; e < CPL; ++e) r[e] *= a[i];
