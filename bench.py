@@ -370,18 +370,21 @@ def make_stages(sets, Q, torch):
 
     # the same bytes in the access pattern of the single-pass kernels (tiles of 128 rows x 512
     # bytes, one persistent workgroup per compute unit): in the shape the two kernels load and
-    # store in (sixteen waves with 8 consecutive rows each), with eight waves of 16 rows, in the
-    # order the memory system likes best, and in that order with the rows handed on through LDS
-    def tile_copy(i, rowmap):
+    # store in (sixteen waves with 8 consecutive rows each; also with two inputs, as the backward
+    # kernel has), with eight waves of 16 rows, in the order the memory system likes best, and in
+    # that order with the rows handed on through LDS
+    def tile_copy(i, rowmap, two=False):
         x, A, dy = sets[i % len(sets)]
         o = outs[i % len(sets)]
         b, L, nh, d = x.shape
-        _lib.check(_lib.lib().ema_tile_pattern_copy(x.data_ptr(), o.data_ptr(), b, L, nh * d * x.element_size(), rowmap,
-                                                    _lib.stream_ptr(x.device)), "ema_tile_pattern_copy")
+        _lib.check(_lib.lib().ema_tile_pattern_copy(x.data_ptr(), dy.data_ptr() if two else None, o.data_ptr(), b, L,
+                                                    nh * d * x.element_size(), rowmap, _lib.stream_ptr(x.device)),
+                   "ema_tile_pattern_copy")
 
     x0 = sets[0][0]
     if x0.shape[1] % 128 == 0 and (x0.shape[2] * x0.shape[3] * x0.element_size()) % 512 == 0:
         stages["tile_copy_scan_order"] = lambda i: tile_copy(i, 0)
+        stages["tile_copy_scan_order_2in_1out"] = lambda i: tile_copy(i, 0, two=True)
         stages["tile_copy_scan_order_8_waves"] = lambda i: tile_copy(i, 3)
         stages["tile_copy_best_order"] = lambda i: tile_copy(i, 1)
         stages["tile_copy_exchange"] = lambda i: tile_copy(i, 2)
@@ -396,7 +399,7 @@ def time_stages(sets, Q, iters, torch, only=None):
     N, L, T = x.shape[0] * x.shape[2], x.shape[1], x.shape[3]
     xb = x.numel() * x.element_size()
     ab = dict(algorithmic_bytes(N, L, T, Q, 2), copy=2 * xb, stream_copy=2 * xb, stream_2in_1out=3 * xb,
-              tile_copy_scan_order=2 * xb, tile_copy_scan_order_8_waves=2 * xb,
+              tile_copy_scan_order=2 * xb, tile_copy_scan_order_2in_1out=3 * xb, tile_copy_scan_order_8_waves=2 * xb,
               tile_copy_best_order=2 * xb, tile_copy_exchange=2 * xb)
     res = {}
     for name, fn in stages.items():

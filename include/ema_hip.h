@@ -109,11 +109,12 @@ int ema_stream_copy(const void* a, const void* b, void* dst, size_t bytes, void*
  * rowmap 1: eight waves, the rows of a wave 8 apart and slabs rotated against each other, which is
  * the order the memory system sustains the highest rate for; rowmap 2: memory is touched as with
  * rowmap 1 and every wave still gets 16 consecutive rows into its registers, the rows changing
- * hands through LDS on the way in and on the way out.  Other values: EMA_ERR_UNSUPPORTED.  bench.py
- * reports all four next to the plain streaming copy: the first is the ceiling of the scan kernels'
- * own pattern. */
-int ema_tile_pattern_copy(const void* src, void* dst, int64_t slabs, int64_t rows, int64_t row_bytes,
-                          int rowmap, void* stream);
+ * hands through LDS on the way in and on the way out.  Other values: EMA_ERR_UNSUPPORTED.  src2 (may
+ * be NULL; rowmap 0 only): a second input of the same layout, dst = src ^ src2, the backward kernel's
+ * two inputs and one output.  bench.py reports all of them next to the plain streaming copy: rowmap 0
+ * is the ceiling of the scan kernels' own pattern. */
+int ema_tile_pattern_copy(const void* src, const void* src2, void* dst, int64_t slabs, int64_t rows,
+                          int64_t row_bytes, int rowmap, void* stream);
 
 /* Largest chunk size accepted by every entry point. */
 #define EMA_MAX_CHUNK 1024

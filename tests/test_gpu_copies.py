@@ -17,10 +17,16 @@ def test_tile_pattern_copy_copies(rowmap, slabs, rows, row_bytes, device):
     gen = torch.Generator(device=device).manual_seed(rowmap + rows)
     src = torch.randint(0, 256, (slabs, rows, row_bytes), generator=gen, device=device, dtype=torch.uint8)
     dst = torch.zeros_like(src)
-    _lib.check(_lib.lib().ema_tile_pattern_copy(src.data_ptr(), dst.data_ptr(), slabs, rows, row_bytes, rowmap,
+    _lib.check(_lib.lib().ema_tile_pattern_copy(src.data_ptr(), None, dst.data_ptr(), slabs, rows, row_bytes, rowmap,
                                                 _lib.stream_ptr(device)), "ema_tile_pattern_copy")
     torch.cuda.synchronize()
     assert torch.equal(src, dst)
+    if rowmap == 0:  # with a second input: the exclusive or of the two
+        other = torch.randint(0, 256, (slabs, rows, row_bytes), generator=gen, device=device, dtype=torch.uint8)
+        _lib.check(_lib.lib().ema_tile_pattern_copy(src.data_ptr(), other.data_ptr(), dst.data_ptr(), slabs, rows,
+                                                    row_bytes, rowmap, _lib.stream_ptr(device)), "ema_tile_pattern_copy")
+        torch.cuda.synchronize()
+        assert torch.equal(dst, src ^ other)
 
 
 def test_tile_pattern_copy_rejects_other_shapes(device):
@@ -29,10 +35,11 @@ def test_tile_pattern_copy_rejects_other_shapes(device):
     buf = torch.zeros(2 * 128 * 512, device=device, dtype=torch.uint8)
     f = _lib.lib().ema_tile_pattern_copy
     s = _lib.stream_ptr(device)
-    assert f(buf.data_ptr(), buf.data_ptr(), 2, 100, 512, 0, s) == -2   # rows not a multiple of 128
-    assert f(buf.data_ptr(), buf.data_ptr(), 2, 128, 500, 2, s) == -2   # row bytes not a multiple of 512
-    assert f(None, buf.data_ptr(), 2, 128, 512, 1, s) == -1
-    assert f(buf.data_ptr(), buf.data_ptr(), 2, 128, 512, 9, s) == -5   # no such pattern
+    assert f(buf.data_ptr(), None, buf.data_ptr(), 2, 100, 512, 0, s) == -2   # rows not a multiple of 128
+    assert f(buf.data_ptr(), None, buf.data_ptr(), 2, 128, 500, 2, s) == -2   # row bytes not a multiple of 512
+    assert f(None, None, buf.data_ptr(), 2, 128, 512, 1, s) == -1
+    assert f(buf.data_ptr(), None, buf.data_ptr(), 2, 128, 512, 9, s) == -5   # no such pattern
+    assert f(buf.data_ptr(), buf.data_ptr(), buf.data_ptr(), 2, 128, 512, 1, s) == -5   # two inputs: the kernels' shape only
 
 
 @pytest.mark.parametrize("two", [False, True], ids=["one_input", "two_inputs"])

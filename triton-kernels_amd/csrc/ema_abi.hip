@@ -577,9 +577,11 @@ int ema_stream_copy(const void* a, const void* b, void* dst, size_t bytes, void*
   return launched();
 }
 
-int ema_tile_pattern_copy(const void* src, void* dst, int64_t slabs, int64_t rows, int64_t row_bytes, int rowmap,
-                          void* stream) {
+int ema_tile_pattern_copy(const void* src, const void* src2, void* dst, int64_t slabs, int64_t rows, int64_t row_bytes,
+                          int rowmap, void* stream) {
   if (!src || !dst) return EMA_ERR_NULL;
+  if (src2 && rowmap != 0) return EMA_ERR_UNSUPPORTED;
+  if (reinterpret_cast<uintptr_t>(src2) % 16) return EMA_ERR_ALIGN;
   if (slabs <= 0 || rows <= 0 || row_bytes <= 0 || rows % 128 || row_bytes % 512) return EMA_ERR_SHAPE;
   if (reinterpret_cast<uintptr_t>(src) % 16 || reinterpret_cast<uintptr_t>(dst) % 16) return EMA_ERR_ALIGN;
   const int64_t pieces = row_bytes / 512, tiles = slabs * (rows / 128) * pieces;
@@ -592,15 +594,16 @@ int ema_tile_pattern_copy(const void* src, void* dst, int64_t slabs, int64_t row
     return EMA_ERR_LAUNCH;
   const dim3 grid((unsigned)(tiles < ncu ? tiles : ncu));
   const char* s8 = static_cast<const char*>(src);
+  const char* s28 = static_cast<const char*>(src2);
   char* d8 = static_cast<char*>(dst);
   const int rb = (int)(rows / 128);
   hipStream_t st = as_stream(stream);
   if (rowmap == 0) {
-    hipLaunchKernelGGL(tile_copy_shape_kernel<16>, grid, dim3(1024), 0, st, s8, d8, (int)slabs, rb, (int)pieces, row_bytes,
-                       rows * row_bytes);
+    hipLaunchKernelGGL(tile_copy_shape_kernel<16>, grid, dim3(1024), 0, st, s8, s28, d8, (int)slabs, rb, (int)pieces,
+                       row_bytes, rows * row_bytes);
   } else if (rowmap == 3) {
-    hipLaunchKernelGGL(tile_copy_shape_kernel<8>, grid, dim3(512), 0, st, s8, d8, (int)slabs, rb, (int)pieces, row_bytes,
-                       rows * row_bytes);
+    hipLaunchKernelGGL(tile_copy_shape_kernel<8>, grid, dim3(512), 0, st, s8, (const char*)nullptr, d8, (int)slabs, rb,
+                       (int)pieces, row_bytes, rows * row_bytes);
   } else if (rowmap == 1) {
     hipLaunchKernelGGL(tile_copy_kernel, grid, dim3(512), 0, st, s8, d8, (int)slabs, rb, (int)pieces, row_bytes,
                        rows * row_bytes);

@@ -33,10 +33,13 @@ __global__ __launch_bounds__(256) void stream_copy_kernel(const uint4* __restric
 //   tile_copy_kernel:           eight waves, instruction i of wave g moves row (8 i + g + slab) % 128:
 //             the rows of a wave are 8 apart, the waves of a workgroup touch neighbouring rows, and
 //             slabs (whose addresses differ by a large power of two) are rotated against each other.
-// At b16 nh2 d1024 L4096, bfloat16, these sustain 5.7, 5.2 and 6.0 TB/s.
+// At b16 nh2 d1024 L4096, bfloat16, these sustain 5.5, 5.4 and 6.0 TB/s; the first with two inputs 5.9 TB/s.
 // ------------------------------------------------------------------------------------
+// (src2, if not null: a second input of the same layout; dst = src ^ src2, as in the backward kernel's
+// two inputs and one output)
 template <int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void tile_copy_shape_kernel(const char* __restrict__ src, char* __restrict__ dst,
+__global__ __launch_bounds__(64 * WAVES) void tile_copy_shape_kernel(const char* __restrict__ src,
+                                                                     const char* __restrict__ src2, char* __restrict__ dst,
                                                                      int slabs, int row_blocks, int pieces,
                                                                      int64_t row_bytes, int64_t slab_bytes) {
   typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
@@ -50,6 +53,13 @@ __global__ __launch_bounds__(64 * WAVES) void tile_copy_shape_kernel(const char*
     u32x2 v[RPW];
 #pragma unroll
     for (int i = 0; i < RPW; ++i) v[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(src + base + i * row_bytes));
+    if (src2) {
+      u32x2 u[RPW];
+#pragma unroll
+      for (int i = 0; i < RPW; ++i) u[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(src2 + base + i * row_bytes));
+#pragma unroll
+      for (int i = 0; i < RPW; ++i) v[i] ^= u[i];
+    }
 #pragma unroll
     for (int i = 0; i < RPW; ++i) __builtin_nontemporal_store(v[i], reinterpret_cast<u32x2*>(dst + base + i * row_bytes));
   }

@@ -34,7 +34,7 @@ _SIGNATURES = {
     "ema_fwd_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I]),
     "ema_workspace_clear": (c_int, [_P, c_size_t, _P]),
     "ema_stream_copy": (c_int, [_P, _P, _P, c_size_t, _P]),
-    "ema_tile_pattern_copy": (c_int, [_P, _P, _I, _I, _I, c_int, _P]),
+    "ema_tile_pattern_copy": (c_int, [_P, _P, _P, _I, _I, _I, c_int, _P]),
     "ema_fwd": (c_int, _SEQ + _SEQ + [c_int] + _SEQ + [_P, _P, _P, _P, _P, c_size_t, c_int, _I, _I, _I, _I, _I, _P, _P, _P]),
     "ema_chunk_scan_bwd_dstates": (c_int, _SEQ + [c_int, _P, _P, _I, _I, _I, _I, _I, _P]),
     "ema_state_passing_bwd_workspace_bytes": (c_size_t, [_I, _I, _I]),
