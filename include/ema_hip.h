@@ -224,12 +224,16 @@ int ema_chunk_scan_bwd_dc(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t 
                           int64_t batch, int64_t nheads, int64_t seqlen, int64_t dim,
                           int64_t chunk, void* stream);
 
-/* Bytes of workspace ema_chunk_scan_bwd_ddAcs needs (per-row-tile partial sums). */
-size_t ema_chunk_scan_bwd_ddAcs_workspace_bytes(int64_t batch, int64_t nheads,
-                                                int64_t seqlen, int64_t chunk);
+/* Bytes of workspace ema_chunk_scan_bwd_ddAcs needs (partial sums per row tile and per column
+ * tile, one flag per chunk); 0 for a shape or dtype it does not take. */
+size_t ema_chunk_scan_bwd_ddAcs_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen,
+                                                int64_t dim, int64_t chunk, int dtype);
 
 /* B6: G[m,k] = exp(min(cs[m]-cs[k],0)) * <dy[m], x[k]> for k < m;
  * ddA_intra[j] = sum_{m>=j} sum_{k<j} G[m,k], ddA_intra[0] = 0.  Output (N,C,Q).
+ * Chunks of up to 512 rows in which cs never rises (every decay) are evaluated in the factored form
+ * ddA_intra[j] = exp(cs[j]-cs[j-1]) * <r[j], y[j-1]> with the chunk-local scans y of x and r of dy,
+ * in float32 and in a time that does not grow with the chunk; the others by the product itself.
  * Replaces _ema_chunk_scan_bwd_ddAcs_stable,
  * kernels/ema_kernels_bwd/ema_scan_da.py:113-137. */
 int ema_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,

@@ -170,6 +170,45 @@ def test_bwd_da_intra(case, device):
     assert float(got[..., 0].abs().max()) == 0.0
 
 
+# (N, L, T, Q) for B6 alone: chunks of one to four 128-row sub-tiles with ragged ends, a feature
+# width that is no multiple of the column tile, and a chunk too long for the factored form
+DA_SHAPES = [
+    (2, 1000, 320, 200),
+    (1, 900, 1024, 300),
+    (3, 1100, 264, 384),
+    (2, 2048, 512, 512),
+    (2, 1500, 136, 500),
+    (1, 1300, 72, 640),
+]
+
+
+@pytest.mark.parametrize("rising", ["nowhere", "some_chunks", "everywhere"])
+@pytest.mark.parametrize("shape", DA_SHAPES, ids=lambda s: "N%d_L%d_T%d_Q%d" % s)
+def test_bwd_da_intra_forms(shape, rising, dtype, device):
+    """B6 over both of its forms: a cumsum that never rises inside a chunk takes the factored form, a
+    chunk in which it rises anywhere the product with the pairwise minimum
+    (kernels/ema_kernels_bwd/ema_scan_da.py:92), and one call may hold both kinds."""
+    from kernels.ema_kernels_bwd.ema_scan_da import _ema_chunk_scan_bwd_ddAcs_stable
+
+    N, L, T, Q = shape
+    announce(f"bwd_da_intra forms {N}x{L}x{T} Q{Q} {dtype} rising {rising}")
+    A, X, dy = flat_case(N, L, T, seed=77 + L + Q, dtype=dtype)
+    if rising == "everywhere":
+        A = A.abs() * 0.05 - 0.02  # both signs in every chunk
+    elif rising == "some_chunks":
+        A = A.clone()
+        C = -(-L // Q)
+        for n in range(N):
+            for c in range(n % 2, C, 3):  # every third chunk, one or two positive steps in it
+                A[n, min(L - 1, c * Q + 1 + (37 * c) % (Q - 1))] = 0.3
+                A[n, min(L - 1, c * Q + Q // 2)] = 0.01
+    cs = O.chunk_cumsum(A, Q)
+    got = _ema_chunk_scan_bwd_ddAcs_stable(_dev(X, device), _dev(cs, device), _dev(dy, device))
+    ref = O.bwd_da_intra(X.float(), cs, dy.float())
+    check_close("ddA_intra", _valid(got, L), _valid(ref, L), dtype)
+    assert float(got[..., 0].abs().max()) == 0.0
+
+
 def test_headed_layout_stages(device):
     """(b, L, nh, d) tensors and a (b, L, nh) log-decay are consumed in place (strided)."""
     from kernels.ema_kernels.ema_cumsum import ema_chunk_cumsum_fwd

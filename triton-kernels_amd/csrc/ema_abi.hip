@@ -12,6 +12,7 @@
 #include "ema_walk_kernels.h"
 #include "ema_chain_kernels.h"
 #include "ema_tile_kernels.h"
+#include "ema_flat_kernels.h"
 
 using namespace ema;
 
@@ -176,32 +177,6 @@ int launch_row_dot(const void* x, SeqStrides sx, int dtype, const float* vec, co
     hipLaunchKernelGGL((row_dot_kernel<float, MODE>), dim3(grid), dim3(kRowDotThreads), 0, st, (const float*)x,
                        sx, vec, cs, out, (int)d.nh, (int)d.L, (int)d.T, (int)d.Q, (int)d.C, raw);
   return launched();
-}
-
-int launch_da(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, int dtype,
-              const float* cs, float* ddA_intra, float* part, float* rowsum, const Dims& d,
-              hipStream_t st) {
-  const int MT = (int)((d.Q + kBM - 1) / kBM);
-  const int64_t grid = d.N * d.C * MT;
-  if (grid > 0x7fffffff) return EMA_ERR_SHAPE;
-  if (dtype == EMA_BF16)
-    hipLaunchKernelGGL((da_gemm_kernel<bf16_t>), dim3((unsigned)grid), dim3(256), 0, st,
-                       (const bf16_t*)x, sx, (const bf16_t*)dy, sd, cs, part, rowsum, (int)d.nh,
-                       (int)d.L, (int)d.T, (int)d.Q, (int)d.C, MT, nullptr, nullptr, 1, 1);
-  else
-    hipLaunchKernelGGL((da_gemm_kernel<float>), dim3((unsigned)grid), dim3(256), 0, st,
-                       (const float*)x, sx, (const float*)dy, sd, cs, part, rowsum, (int)d.nh,
-                       (int)d.L, (int)d.T, (int)d.Q, (int)d.C, MT, nullptr, nullptr, 1, 1);
-  EMA_TRY(launched());
-  const int64_t total = d.N * d.C;
-  hipLaunchKernelGGL(da_finish_kernel<kBM>, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, st, part,
-                     rowsum, ddA_intra, (int)d.Q, MT, total);
-  return launched();
-}
-
-size_t da_part_floats(const Dims& d) {
-  const int64_t MT = (d.Q + kBM - 1) / kBM;
-  return (size_t)(d.N * d.C * MT * d.Q);
 }
 
 // The backward chunks the sequence by 128 internally, whatever the chunk size of the
@@ -419,6 +394,111 @@ int run_bwd_fused(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, i
   const int64_t total = d.N * d.C * d.Q;
   hipLaunchKernelGGL(dA_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, part,
                      ddA, (int)d.L, (int)d.Q, (int)d.C, (int)di.C, parts, total);
+  return launched();
+}
+
+// Workspace of B6: column sums per row tile and row sums of the kernel that forms the product, then
+// the per-column-tile dots of the factored form and one flag per chunk.
+struct DaWs {
+  float *part, *rowsum, *flat;
+  int* steep;
+  size_t bytes;
+};
+// Columns per workgroup of the factored form: the single-pass kernels' tile; for float32 chunks of
+// three or four 128-row sub-tiles half of it (a chunk's x rows stay in registers, and eight bytes per
+// row and lane are too many there).
+template <typename T>
+constexpr int kFlatLongDiv = sizeof(T) == 4 ? 2 : 1;
+inline int da_flat_cols(const Dims& d, int dtype) {
+  const int wide = dtype == EMA_BF16 ? 64 * TileBf16::BWD_CPL : 64 * TileF32::BWD_CPL;
+  const int div = dtype == EMA_BF16 ? kFlatLongDiv<bf16_t> : kFlatLongDiv<float>;
+  return d.Q > 2 * kTileRows ? wide / div : wide;
+}
+inline int da_flat_tiles(const Dims& d, int dtype) {
+  const int bn = da_flat_cols(d, dtype);
+  return (int)((d.T + bn - 1) / bn);
+}
+constexpr int kFlatMaxChunk = 4 * kTileRows;  // the factored form keeps a chunk's x rows in registers
+DaWs carve_da(void* base, const Dims& d, int dtype) {
+  DaWs w;
+  size_t off = 0;
+  char* p = static_cast<char*>(base);
+  auto take = [&](size_t bytes) {
+    char* r = p + off;
+    off += align_up(bytes, 256);
+    return r;
+  };
+  const int64_t MT = (d.Q + kBM - 1) / kBM;
+  w.part = reinterpret_cast<float*>(take((size_t)(d.N * d.C * MT * d.Q) * sizeof(float)));
+  w.rowsum = reinterpret_cast<float*>(take((size_t)(d.N * d.C * d.Q) * sizeof(float)));
+  const bool flat = d.Q <= kFlatMaxChunk;
+  w.flat = reinterpret_cast<float*>(take(flat ? (size_t)(d.N * d.C * d.Q) * da_flat_tiles(d, dtype) * sizeof(float) : 0));
+  w.steep = reinterpret_cast<int*>(take(flat ? (size_t)(d.N * d.C) * sizeof(int) : 0));
+  w.bytes = off;
+  return w;
+}
+
+template <typename T, int CPL, int RPL, int KT>
+int launch_da_flat_k(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* cs,
+                     const DaWs& w, const Dims& d, hipStream_t st) {
+  using Cfg = TileCfg<T, CPL, RPL>;
+  constexpr int smem = FlatCfg<T, CPL, RPL, KT>::smem_bytes;
+  const int ntiles = (int)((d.T + Cfg::BN - 1) / Cfg::BN);
+  const int64_t total = d.N * d.C * ntiles;
+  if (total > 0x7fffffff) return EMA_ERR_SHAPE;
+  auto kernel = da_flat_kernel<T, CPL, RPL, KT>;
+  EMA_TRY(allow_smem(kernel, smem));
+  const int64_t cap = resident_blocks(kernel, Cfg::NT, smem);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(Cfg::NT), smem, st, (const T*)x, sx,
+                     (const T*)dy, sd, cs, w.flat, w.steep, (int)d.nh, (int)d.L, (int)d.T, (int)d.Q, (int)d.C,
+                     ntiles, (int)total);
+  return launched();
+}
+template <typename T, typename S>
+int launch_da_flat(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* cs,
+                   const DaWs& w, const Dims& d, hipStream_t st) {
+  constexpr int CPL = S::BWD_CPL, RPL = S::BWD_RPL;
+  static_assert(CPL % kFlatLongDiv<T> == 0, "long chunks take a part of the columns");
+  switch ((d.Q + kTileRows - 1) / kTileRows) {
+    case 1: return launch_da_flat_k<T, CPL, RPL, 1>(x, sx, dy, sd, cs, w, d, st);
+    case 2: return launch_da_flat_k<T, CPL, RPL, 2>(x, sx, dy, sd, cs, w, d, st);
+    case 3: return launch_da_flat_k<T, CPL / kFlatLongDiv<T>, RPL, 3>(x, sx, dy, sd, cs, w, d, st);
+    default: return launch_da_flat_k<T, CPL / kFlatLongDiv<T>, RPL, 4>(x, sx, dy, sd, cs, w, d, st);
+  }
+}
+
+// B6.  Chunks of up to 512 rows go through the factored form first; the kernel that forms the
+// product then takes the chunks in which the cumsum rises somewhere (none, for decays), and the
+// finish kernel picks per chunk.
+int launch_da(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, int dtype,
+              const float* cs, float* ddA_intra, const DaWs& w, const Dims& d, hipStream_t st) {
+  const int MT = (int)((d.Q + kBM - 1) / kBM);
+  const int64_t grid = d.N * d.C * MT;
+  if (grid > 0x7fffffff) return EMA_ERR_SHAPE;
+  // the factored form reads a chunk's rows at 32-bit byte offsets from the chunk's first row and
+  // tells rows apart by their offset: rows must not overlap and a chunk must span less than 2 GiB
+  auto fits = [&](const SeqStrides& s) {
+    return s.sl >= d.T && (d.Q * s.sl + 256) * (int64_t)elem_size(dtype) < (int64_t)0x7fffffff;
+  };
+  const bool flat = d.Q <= kFlatMaxChunk && fits(sx) && fits(sd);
+  if (flat) {
+    if (dtype == EMA_BF16) EMA_TRY((launch_da_flat<bf16_t, TileBf16>(x, sx, dy, sd, cs, w, d, st)));
+    else EMA_TRY((launch_da_flat<float, TileF32>(x, sx, dy, sd, cs, w, d, st)));
+  }
+  const int* only = flat ? w.steep : nullptr;
+  if (dtype == EMA_BF16)
+    hipLaunchKernelGGL((da_gemm_kernel<bf16_t>), dim3((unsigned)grid), dim3(256), 0, st,
+                       (const bf16_t*)x, sx, (const bf16_t*)dy, sd, cs, w.part, w.rowsum, (int)d.nh,
+                       (int)d.L, (int)d.T, (int)d.Q, (int)d.C, MT, nullptr, nullptr, 1, 1, only);
+  else
+    hipLaunchKernelGGL((da_gemm_kernel<float>), dim3((unsigned)grid), dim3(256), 0, st,
+                       (const float*)x, sx, (const float*)dy, sd, cs, w.part, w.rowsum, (int)d.nh,
+                       (int)d.L, (int)d.T, (int)d.Q, (int)d.C, MT, nullptr, nullptr, 1, 1, only);
+  EMA_TRY(launched());
+  const int64_t total = d.N * d.C;
+  hipLaunchKernelGGL(da_finish_kernel<kBM>, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, st, w.part,
+                     w.rowsum, ddA_intra, (int)d.Q, MT, total, flat ? w.flat : nullptr, only,
+                     da_flat_tiles(d, dtype));
   return launched();
 }
 
@@ -743,11 +823,11 @@ int ema_chunk_scan_bwd_dc(const void* dy, int64_t dy_sb, int64_t dy_sl, int64_t 
 }
 
 size_t ema_chunk_scan_bwd_ddAcs_workspace_bytes(int64_t batch, int64_t nheads, int64_t seqlen,
-                                                int64_t chunk) {
+                                                int64_t dim, int64_t chunk, int dtype) {
   Dims d;
-  if (check_dims(batch, nheads, seqlen, 1, chunk, false, &d) != EMA_OK) return 0;
-  return align_up(da_part_floats(d) * sizeof(float), 256) +
-         align_up((size_t)(d.N * d.C * d.Q) * sizeof(float), 256);
+  if (check_dims(batch, nheads, seqlen, dim, chunk, true, &d) != EMA_OK) return 0;
+  if (check_dtype(dtype) != EMA_OK) return 0;
+  return carve_da(nullptr, d, dtype).bytes;
 }
 
 int ema_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,
@@ -762,13 +842,10 @@ int ema_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t 
   EMA_TRY(check_seq(dy, dy_sb, dy_sl, dy_sh, dtype, dim));
   if (!cs || !ddA_intra) return EMA_ERR_NULL;
   EMA_TRY(check_f32(workspace));
-  if (workspace_bytes < ema_chunk_scan_bwd_ddAcs_workspace_bytes(batch, nheads, seqlen, chunk))
-    return EMA_ERR_SHAPE;
-  float* part = static_cast<float*>(workspace);
-  float* rowsum = reinterpret_cast<float*>(static_cast<char*>(workspace) +
-                                           align_up(da_part_floats(d) * sizeof(float), 256));
+  const DaWs w = carve_da(workspace, d, dtype);
+  if (workspace_bytes < w.bytes) return EMA_ERR_SHAPE;
   return launch_da(x, SeqStrides{x_sb, x_sl, x_sh}, dy, SeqStrides{dy_sb, dy_sl, dy_sh}, dtype, cs,
-                   ddA_intra, part, rowsum, d, as_stream(stream));
+                   ddA_intra, w, d, as_stream(stream));
 }
 
 // Workspace of ema_bwd: the chained part first, then the dA partials and what the recomputation

@@ -29,7 +29,10 @@ __global__ __launch_bounds__(256, 2) void da_gemm_kernel(const T* __restrict__ x
                                                       int Tdim, int Q, int C, int MT,
                                                       const float* __restrict__ wk,
                                                       const float* __restrict__ wmk,
-                                                      int heads_per_group, int ngroups) {
+                                                      int heads_per_group, int ngroups,
+                                                      const int* __restrict__ only = nullptr) {
+  // only (may be null): the kernel works on the chunks whose entry is not 0 and leaves the rest alone
+  if (only && only[blockIdx.x / MT] == 0) return;
   constexpr int EPL = Vec16<T>::N;
   constexpr int KG = 2 * EPL;
   constexpr int DK = 4 * KG;        // feature columns per LDS stage (128 bytes per row)
@@ -174,14 +177,27 @@ __global__ __launch_bounds__(256, 2) void da_gemm_kernel(const T* __restrict__ x
 
 // B6, second part: ddA_intra[j] = sum_{i<j} (colsum[i] - rowsum[i]) with
 // colsum[i] = sum over the row tiles mt >= i / 128 of part[mt][i].  One wave per (n, c).
+// With flat (may be null) the chunks whose entry in steep is 0 take their result from there instead:
+// ddA_intra[j] = sum over the ntiles column tiles of flat[(chunk*ntiles + tile)*Q + j].
 template <int BM>
 __global__ __launch_bounds__(256) void da_finish_kernel(const float* __restrict__ part,
                                                         const float* __restrict__ rowsum,
                                                         float* __restrict__ ddA_intra, int Q,
-                                                        int MT, int64_t total_chunks) {
+                                                        int MT, int64_t total_chunks,
+                                                        const float* __restrict__ flat = nullptr,
+                                                        const int* __restrict__ steep = nullptr,
+                                                        int ntiles = 0) {
   const int lane = threadIdx.x & 63;
   const int64_t chunk_id = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (chunk_id >= total_chunks) return;
+  if (flat && steep[chunk_id] == 0) {
+    for (int q = lane; q < Q; q += 64) {
+      float s = 0.f;
+      for (int ct = 0; ct < ntiles; ++ct) s += flat[(chunk_id * ntiles + ct) * (int64_t)Q + q];
+      ddA_intra[chunk_id * Q + q] = s;
+    }
+    return;
+  }
   const int per = (Q + 63) >> 6;
   const int q0 = lane * per;
   auto val = [&](int q) {

@@ -42,7 +42,7 @@ _SIGNATURES = {
     "ema_chunk_scan_chunk_state_bwd_dx": (c_int, _SEQ + [c_int, _P, _P] + _SEQ + [_I, _I, _I, _I, _I, _P]),
     "ema_chunk_state_bwd_db": (c_int, _SEQ + [c_int, _P, _P, _P, c_int, _I, _I, _I, _I, _I, _P]),
     "ema_chunk_scan_bwd_dc": (c_int, _SEQ + [c_int, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
-    "ema_chunk_scan_bwd_ddAcs_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
+    "ema_chunk_scan_bwd_ddAcs_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I, c_int]),
     "ema_chunk_scan_bwd_ddAcs": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _P]),
     "ema_bwd_dx_dA_fused_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "ema_bwd_dx_dA_fused": (c_int, _SEQ + _SEQ + [c_int, _P, _P, _P] + _SEQ + [_P] + _SEQ + [_P, c_size_t, _I, _I, _I, _I, _P]),

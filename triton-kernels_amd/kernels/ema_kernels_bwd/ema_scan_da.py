@@ -1,5 +1,6 @@
-"""B6, intra-chunk log-decay gradient: the dout . x^T contraction over the feature axis on
-MFMA, scaled by the segsum decays and reduced by a two-dimensional prefix.
+"""B6, intra-chunk log-decay gradient.  Chunks of up to 512 rows whose cumsum never rises take the
+factored form (two chunk-local scans and one dot per row); the others the dout . x^T contraction
+over the feature axis on MFMA, scaled by the segsum decays and reduced by a two-dimensional prefix.
 
 Mirrors kernels/ema_kernels_bwd/ema_scan_da.py:113-137 of the reference."""
 import torch
@@ -19,7 +20,9 @@ def _ema_chunk_scan_bwd_ddAcs_stable(x, dA_cumsum, dout):
     cs = _lib.f32c(dA_cumsum)
     ddA_cumsum = torch.empty(batch * nh, nchunks, chunk_size, device=dev, dtype=torch.float32)
     L = _lib.lib()
-    ws_bytes = L.ema_chunk_scan_bwd_ddAcs_workspace_bytes(batch, nh, seqlen, chunk_size)
+    ws_bytes = L.ema_chunk_scan_bwd_ddAcs_workspace_bytes(
+        batch, nh, seqlen, token_dim, chunk_size, _lib.dtype_code(x)
+    )
     assert ws_bytes > 0, "unsupported shape"
     ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
     with torch.cuda.device(dev):
