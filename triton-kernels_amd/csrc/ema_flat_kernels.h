@@ -20,8 +20,11 @@
 //      thread's register from one sub-tile to the next), and, once per chunk, one thread per column
 //      chains the forward group states through all sub-tiles; then the forward values from the true
 //      state and the reverse pass with the dots.
-// Behind the last use of a row the row that takes its registers next is requested: the dy row of
-// the sub-tile before, the x row of the same sub-tile of the workgroup's next chunk.
+// Behind the last use of an x row the row that takes its registers next is requested: the same row
+// of the same sub-tile of the workgroup's next chunk, a whole chunk ahead.  The dy rows have no
+// registers to wait in: every wave copies the rows of the sub-tile before straight from global memory
+// into a place of its own in LDS while it works on this one, and moves them to registers when it gets
+// there.
 #pragma once
 #include "ema_tile_kernels.h"
 
@@ -55,13 +58,45 @@ __device__ __forceinline__ RowWords<NW> flat_load_row(__amdgpu_buffer_rsrc_t des
   return r;
 }
 
+// 64 lanes x 16 bytes from global memory into LDS without passing through registers: lane l's piece, at
+// base + lane_offset bytes, lands at lds_base + 16 * l.  base and lds_base are the same in every lane.
+// The copy counts as a vector-memory load of the wave and completes in order with its other loads.
+// First the wave's earlier LDS reads are waited for (they may read the place that is written); m0,
+// which carries the LDS address, is put back; the wait states cover a scalar base that vector
+// instructions have just written.
+typedef __attribute__((address_space(3))) void flat_lds_void_t;
+__device__ __forceinline__ void flat_copy16_to_lds(const void* base, unsigned lane_offset, void* lds_base) {
+  const unsigned lds = (unsigned)(uintptr_t)(flat_lds_void_t*)lds_base;
+  const uint64_t wide = reinterpret_cast<uint64_t>(base);
+  const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(wide >> 32));
+  const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)wide);
+  base = reinterpret_cast<const void*>(((uint64_t)hi << 32) | (uint64_t)lo);
+  unsigned keep;
+  asm volatile(
+      "s_waitcnt lgkmcnt(0)\n\ts_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %1, %2 nt\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(keep)
+      : "v"(lane_offset), "s"(base), "s"(lds)
+      : "memory");
+}
+// Waits until at most `newer` of the wave's vector-memory operations are under way: everything but
+// the `newer` most recent ones has completed.
+template <int NEWER>
+__device__ __forceinline__ void flat_wait_loads() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NEWER) : "memory");
+}
+
 template <typename T, int CPL, int RPL, int KT>
 struct FlatCfg {
   using W = TileCfg<T, CPL, RPL>;
   static constexpr int kStateFloats = KT * W::NG * W::BN;  // forward group states of every sub-tile
-  static constexpr int kRevFloats = 2 * W::NG * W::BN;     // reverse group states, double-buffered
-  static constexpr int kDecayFloats = KT * W::NG;
-  static constexpr int smem_bytes = (kStateFloats + kRevFloats + kDecayFloats) * (int)sizeof(float);
+  static constexpr int kRevFloats = W::NG * W::BN;         // reverse group states
+  static constexpr int kDecayFloats = KT * W::NG + 4;       // and the flag of a rising cumsum
+  static constexpr int kRowBytes = W::BN * (int)sizeof(T);  // a sub-tile's row: 256 or 512 bytes
+  static constexpr int kStageBytes = kTileRows * kRowBytes;  // the dy rows of one sub-tile
+  static constexpr int smem_bytes = (kStateFloats + kRevFloats + kDecayFloats) * (int)sizeof(float) + kStageBytes;
+  static_assert((kStateFloats + kRevFloats + kDecayFloats) % 4 == 0, "the staged rows start at a multiple of 16 bytes");
+  static_assert(smem_bytes <= 160 * 1024, "LDS of one compute unit");
 };
 
 // part[(chunk*ntiles + ctile)*Q + q]: the dot of row q over the columns of tile ctile, times a[q].
@@ -77,17 +112,31 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), 1) void da_flat_kernel(
   static_assert(2 * BN <= NT, "one thread per column and direction");
   extern __shared__ __attribute__((aligned(16))) float flat_smem[];
   float (*sS)[NG][BN] = reinterpret_cast<float (*)[NG][BN]>(flat_smem);
-  float (*sR)[NG][BN] = reinterpret_cast<float (*)[NG][BN]>(flat_smem + F::kStateFloats);
+  float (*sR)[BN] = reinterpret_cast<float (*)[BN]>(flat_smem + F::kStateFloats);
   float (*sD)[NG] = reinterpret_cast<float (*)[NG]>(flat_smem + F::kStateFloats + F::kRevFloats);
-  const int lane = threadIdx.x & 63;
+  int* const sFlag = reinterpret_cast<int*>(flat_smem + F::kStateFloats + F::kRevFloats + KT * NG);
   const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-  const unsigned off = (unsigned)lane * CPL;
-  const int kf = (int)threadIdx.x - BN;  // column of the threads that chain the forward group states
+  // this wave's staged dy rows
+  constexpr int ROWB = F::kRowBytes, LPR = ROWB / 16, RPI = 64 / LPR, NCOPY = RPL / RPI;
+  static_assert(RPL % RPI == 0, "whole rows per copy");
+  char* const stage = reinterpret_cast<char*>(flat_smem + F::kStateFloats + F::kRevFloats + F::kDecayFloats) +
+                      grp * (RPL * ROWB);
 
+  auto opaque = [](unsigned v) {
+    asm volatile("" : "+s"(v));
+    return v;
+  };
+  if (threadIdx.x == 0) *sFlag = 0;
+  __syncthreads();
+  // This lane's number, formed anew wherever it is asked for: what is derived from it (LDS addresses,
+  // column offsets, comparisons) is then formed where it is used instead of being kept in registers
+  // for the whole kernel, and the registers hold rows.
+  auto lane_now = [&]() {
+    return (int)__builtin_amdgcn_mbcnt_hi(opaque(~0u), __builtin_amdgcn_mbcnt_lo(opaque(~0u), 0u));
+  };
   struct Item {
     int64_t chunk_id, xbase, dbase;  // element offsets of the chunk's first row at the tile's first column
     int ctile, limit, ncols;
-    unsigned voff;  // byte offset of this lane's columns in a row
   };
   auto decode = [&](int w) {
     Item it;
@@ -100,10 +149,13 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), 1) void da_flat_kernel(
     const int col0 = it.ctile * BN;
     it.limit = min(Q, L - c * Q);
     it.ncols = min(BN, Tdim - col0);
-    it.voff = lane * CPL < it.ncols ? off * (unsigned)sizeof(T) : kFlatNoColumn;
     it.xbase = b * sx.sb + h * sx.sh + (int64_t)c * Q * sx.sl + col0;
     it.dbase = b * sd.sb + h * sd.sh + (int64_t)c * Q * sd.sl + col0;
     return it;
+  };
+  // byte offset of lane ln's columns in a row of chunk c (outside every descriptor past the tensor)
+  auto col_off = [&](const Item& c, int ln) {
+    return ln * CPL < c.ncols ? (unsigned)ln * (unsigned)(CPL * sizeof(T)) : kFlatNoColumn;
   };
   // byte offset of row i of this wave in sub-tile t, for a row pitch of pitch bytes
   auto row_off = [&](int t, int i, unsigned pitch) { return (unsigned)(kTileRows * t + RPL * grp + i) * pitch; };
@@ -111,18 +163,15 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), 1) void da_flat_kernel(
   // rows are formed where they are used and not kept for the whole kernel in scalar registers that
   // are needed for other things.
   const unsigned xpitch = (unsigned)sx.sl * (unsigned)sizeof(T), dpitch = (unsigned)sd.sl * (unsigned)sizeof(T);
-  auto opaque = [](unsigned v) {
-    asm volatile("" : "+s"(v));
-    return v;
-  };
   // Lane RPL*t + i: cs[q] - cs[q-1] for row i of this wave in sub-tile t (cs[0] itself for the
   // chunk's first row, 0 for rows at or past the limit).  One register holds the wave's coefficients
   // of the whole chunk; a row's value is read from its lane where it is used.
   static_assert(RPL * KT <= 64, "one lane per row of the wave");
   auto coef_load = [&](const Item& it) {
-    const int q = kTileRows * (lane / RPL) + RPL * grp + lane % RPL;
+    const int ln = lane_now();
+    const int q = kTileRows * (ln / RPL) + RPL * grp + ln % RPL;
     float raw = 0.f;
-    if (lane < RPL * KT && q < it.limit) {
+    if (ln < RPL * KT && q < it.limit) {
       const float* p = cs + it.chunk_id * Q + q;
       raw = p[0] - (q > 0 ? p[-1] : 0.f);
     }
@@ -130,21 +179,43 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), 1) void da_flat_kernel(
   };
   auto row_coef = [](float v, int i) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), i)); };
 
+  // Requests the dy rows of this wave in sub-tile t of chunk `c` into the wave's place in LDS.  The
+  // addresses are clamped into the chunk's valid rows and the tensor's columns (what arrives for a
+  // row at or past the limit or a column past the end is dropped when the rows are taken out).
+  auto dy_request = [&](const Item& c, int t) {
+    const T* base = dy + c.dbase;
+    const int me = lane_now();
+    const unsigned colb = min((unsigned)(me % LPR) * 16u, (unsigned)c.ncols * (unsigned)sizeof(T) - 16u);
+#pragma unroll
+    for (int j = 0; j < NCOPY; ++j) {
+      const int row = min(kTileRows * t + RPL * grp + RPI * j + me / LPR, c.limit - 1);
+      flat_copy16_to_lds(base, (unsigned)row * dpitch + colb, stage + j * 1024);
+    }
+  };
+  // Takes them out (after the wait for the copies).
+  auto dy_take = [&](RowWords<NW>* rows, const Item& c, int t) {
+    const int nrows = c.limit - (kTileRows * t + RPL * grp);
+    const int ln = lane_now();
+    const bool cok = ln * CPL < c.ncols;
+    const bool full = nrows >= RPL && __all(cok);
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+      rows[i] = *reinterpret_cast<const RowWords<NW>*>(stage + i * ROWB + ln * (CPL * (int)sizeof(T)));
+      if (!full && !(i < nrows && cok)) rows[i] = row_zero<NW>();
+    }
+  };
+
   RowWords<NW> xr[KT][RPL], dr[RPL];
   float araw = 0.f;
-  int w = blockIdx.x, buf = 0;
+  int w = blockIdx.x;
   Item it = decode(w < total ? w : 0);
   if (w < total) {
     const __amdgpu_buffer_rsrc_t xd = flat_rows_desc(x + it.xbase, sx.sl, it.limit, it.ncols);
-    const __amdgpu_buffer_rsrc_t dd = flat_rows_desc(dy + it.dbase, sd.sl, it.limit, it.ncols);
+    dy_request(it, KT - 1);
 #pragma unroll
     for (int t = KT - 1; t >= 0; --t) {
 #pragma unroll
-      for (int i = 0; i < RPL; ++i) xr[t][i] = flat_load_row<NW>(xd, it.voff + row_off(t, i, xpitch));
-      if (t == KT - 1) {
-#pragma unroll
-        for (int i = 0; i < RPL; ++i) dr[i] = flat_load_row<NW>(dd, it.voff + row_off(t, i, dpitch));
-      }
+      for (int i = 0; i < RPL; ++i) xr[t][i] = flat_load_row<NW>(xd, col_off(it, lane_now()) + row_off(t, i, xpitch));
     }
     araw = coef_load(it);
   }
@@ -152,12 +223,14 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), 1) void da_flat_kernel(
     const int wn = w + (int)gridDim.x;
     const bool more = wn < total;
     const Item nx = decode(more ? wn : 0);
-    const __amdgpu_buffer_rsrc_t dd = flat_rows_desc(dy + it.dbase, sd.sl, it.limit, it.ncols);
     const __amdgpu_buffer_rsrc_t xdn = flat_rows_desc(x + nx.xbase, sx.sl, nx.limit, nx.ncols);
-    const __amdgpu_buffer_rsrc_t ddn = flat_rows_desc(dy + nx.dbase, sd.sl, nx.limit, nx.ncols);
     // lane RPL*t + i: the decay of row i of this wave in sub-tile t
     const float av = __expf(fminf(araw, 0.f));
-    const bool rises = araw > 0.f && kTileRows * (lane / RPL) + RPL * grp + lane % RPL > 0;
+    {
+      const int ln = lane_now();
+      const bool rises = araw > 0.f && kTileRows * (ln / RPL) + RPL * grp + ln % RPL > 0;
+      if (__any(rises) && ln == 0) *sFlag = 1;
+    }
 
     // 1. local forward passes
 #pragma unroll
@@ -168,49 +241,69 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), 1) void da_flat_kernel(
       for (int e = 0; e < CPL; ++e) s[e] = 0.f;
 #pragma unroll
       for (int i = 0; i < RPL; ++i) {
-        D *= row_coef(av, RPL * t + i);
+        const float ai = row_coef(av, RPL * t + i);
+        D *= ai;
 #pragma unroll
-        for (int e = 0; e < CPL; ++e) s[e] = fmaf(row_coef(av, RPL * t + i), s[e], row_get<T, NW>(xr[t][i], e));
+        for (int e = 0; e < CPL; ++e) s[e] = fmaf(ai, s[e], row_get<T, NW>(xr[t][i], e));
       }
+      const int ln = lane_now();
 #pragma unroll
-      for (int e = 0; e < CPL; ++e) sS[t][grp][lane * CPL + e] = s[e];
-      if (lane == 0) sD[t][grp] = D;
+      for (int e = 0; e < CPL; ++e) sS[t][grp][ln * CPL + e] = s[e];
+      if (ln == 0) sD[t][grp] = D;
       rows_opaque<NW, RPL>(xr[t]);
     }
 
     float h_in = 0.f;  // chain threads: reverse state entering the sub-tile from the rows after it
-    int flagged = 0;
 #pragma unroll
     for (int t = KT - 1; t >= 0; --t) {
+      // The copies of this sub-tile's dy rows were requested one sub-tile ago, and every sub-tile
+      // requests the RPL x rows of the next chunk after them (if there is a next chunk; the very first
+      // copies are followed by the first chunk's x rows): once at most RPL newer operations are under
+      // way they have landed.  Whatever else the wave has issued since only adds to what is waited for.
+      __builtin_amdgcn_sched_barrier(0);
+      if (t == KT - 1 || more) flat_wait_loads<RPL>();
+      else flat_wait_loads<0>();
+      dy_take(dr, it, t);
+      if (t > 0) dy_request(it, t - 1);
+      else if (more) dy_request(nx, KT - 1);
       // 2a. local reverse pass over dy: what the group hands to the rows before it
       __builtin_amdgcn_sched_barrier(0);
+      float a[RPL];  // the decays of the wave's rows, in scalar registers for the rest of the sub-tile
+#pragma unroll
+      for (int i = 0; i < RPL; ++i) a[i] = row_coef(av, RPL * t + i);
       float r[CPL];
 #pragma unroll
       for (int e = 0; e < CPL; ++e) r[e] = 0.f;
 #pragma unroll
       for (int i = RPL - 1; i >= 0; --i)
 #pragma unroll
-        for (int e = 0; e < CPL; ++e) r[e] = row_coef(av, RPL * t + i) * (row_get<T, NW>(dr[i], e) + r[e]);
+        for (int e = 0; e < CPL; ++e) r[e] = a[i] * (row_get<T, NW>(dr[i], e) + r[e]);
 #pragma unroll
-      for (int e = 0; e < CPL; ++e) sR[buf][grp][lane * CPL + e] = r[e];
+      for (int e = 0; e < CPL; ++e) sR[grp][lane_now() * CPL + e] = r[e];
       rows_opaque<NW, RPL>(dr);
-      if (t == KT - 1) flagged = __syncthreads_or(rises ? 1 : 0);
-      else __syncthreads();
+      __syncthreads();
 
       // 2b. chains over the row groups
-      if (threadIdx.x < BN) {
-        const int k = threadIdx.x;
+      constexpr int CW = BN / 64;  // waves with one thread per column
+      if (grp < CW) {
+        const int k = 64 * grp + lane_now();
+        if (t == KT - 1 && k == 0) {
+          // the workgroup of column tile 0 reports whether the chunk's cumsum rises anywhere
+          if (it.ctile == 0) steep[it.chunk_id] = *sFlag;
+          *sFlag = 0;
+        }
         float rg[NG], dg[NG];
 #pragma unroll
-        for (int g = 0; g < NG; ++g) rg[g] = sR[buf][g][k];
+        for (int g = 0; g < NG; ++g) rg[g] = sR[g][k];
 #pragma unroll
         for (int g = 0; g < NG; ++g) dg[g] = wave_uniform(sD[t][g]);
 #pragma unroll
         for (int g = NG - 1; g >= 0; --g) {
-          sR[buf][g][k] = h_in;
+          sR[g][k] = h_in;
           h_in = fmaf(dg[g], h_in, rg[g]);
         }
-      } else if (t == KT - 1 && kf < BN) {
+      } else if (t == KT - 1 && grp < 2 * CW) {
+        const int kf = 64 * (grp - CW) + lane_now();
         float E = 0.f;
 #pragma unroll 1
         for (int u = 0; u < KT; ++u) {
@@ -234,22 +327,21 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), 1) void da_flat_kernel(
       // pass takes the segment's rows.  Behind the last use of a row the row that uses its registers
       // next is requested.
       constexpr int SEG = KT >= 3 ? 2 : 4;
-      const unsigned xp = opaque(xpitch), dp = opaque(dpitch);
+      const unsigned xp = opaque(xpitch);
       float dA = 0.f;  // lane i reports row i of the wave
-      // (this lane's number, formed per sub-tile so that the eight comparisons with it are not kept)
-      const unsigned me = __builtin_amdgcn_mbcnt_hi(opaque(~0u), __builtin_amdgcn_mbcnt_lo(opaque(~0u), 0u));
+      const unsigned me = (unsigned)lane_now();
 #pragma unroll
-      for (int e = 0; e < CPL; ++e) r[e] = sR[buf][grp][lane * CPL + e];
+      for (int e = 0; e < CPL; ++e) r[e] = sR[grp][me * CPL + e];
 #pragma unroll
       for (int i0 = RPL - SEG; i0 >= 0; i0 -= SEG) {
         __builtin_amdgcn_sched_barrier(0);
         float ym[CPL];  // forward value of the row before the segment
 #pragma unroll
-        for (int e = 0; e < CPL; ++e) ym[e] = sS[t][grp][lane * CPL + e];
+        for (int e = 0; e < CPL; ++e) ym[e] = sS[t][grp][me * CPL + e];
 #pragma unroll
         for (int i = 0; i < i0; ++i)
 #pragma unroll
-          for (int e = 0; e < CPL; ++e) ym[e] = fmaf(row_coef(av, RPL * t + i), ym[e], row_get<T, NW>(xr[t][i], e));
+          for (int e = 0; e < CPL; ++e) ym[e] = fmaf(a[i], ym[e], row_get<T, NW>(xr[t][i], e));
         float yv[SEG - 1][CPL];  // forward values of the segment's rows but the last
         {
           float s[CPL];
@@ -259,7 +351,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), 1) void da_flat_kernel(
           for (int i = 0; i < SEG - 1; ++i)
 #pragma unroll
             for (int e = 0; e < CPL; ++e) {
-              s[e] = fmaf(row_coef(av, RPL * t + i0 + i), s[e], row_get<T, NW>(xr[t][i0 + i], e));
+              s[e] = fmaf(a[i0 + i], s[e], row_get<T, NW>(xr[t][i0 + i], e));
               yv[i][e] = s[e];
             }
         }
@@ -272,13 +364,11 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), 1) void da_flat_kernel(
           for (int e = 0; e < CPL; ++e) {
             const float d = row_get<T, NW>(dr[i], e) + r[e];
             dot = fmaf(d, j > 0 ? yv[j - 1][e] : ym[e], dot);
-            r[e] = d * row_coef(av, RPL * t + i);
+            r[e] = d * a[i];
           }
-          if (t > 0) dr[i] = flat_load_row<NW>(dd, it.voff + row_off(t - 1, i, dp));
-          else if (more) dr[i] = flat_load_row<NW>(ddn, nx.voff + row_off(KT - 1, i, dp));
-          if (more) xr[t][i] = flat_load_row<NW>(xdn, nx.voff + row_off(t, i, xp));
+          if (more) xr[t][i] = flat_load_row<NW>(xdn, col_off(nx, (int)me) + row_off(t, i, xp));
           // the row's dot goes into lane i (rows at or past the limit have dy = 0 and give 0)
-          const float total = wave_sum(dot) * row_coef(av, RPL * t + i);
+          const float total = wave_sum(dot) * a[i];
           if (me == (unsigned)i) dA = total;
         }
       }
@@ -288,9 +378,7 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), 1) void da_flat_kernel(
         float* pb = part + ((it.chunk_id * ntiles + it.ctile) * (int64_t)Q + q0);
         if (me < (unsigned)RPL && q0 + (int)me < Q) pb[me] = dA;
       }
-      buf ^= 1;
     }
-    if (threadIdx.x == 0 && it.ctile == 0) steep[it.chunk_id] = flagged;
     if (more) {
       araw = coef_load(nx);
     }
