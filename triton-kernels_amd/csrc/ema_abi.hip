@@ -468,8 +468,8 @@ int launch_da_flat(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, 
 }
 
 // B6.  Chunks of up to 512 rows go through the factored form first; the kernel that forms the
-// product then takes the chunks in which the cumsum rises somewhere (none, for decays), and the
-// finish kernel picks per chunk.
+// product and its finish then take the chunks in which the cumsum rises somewhere (none, for decays)
+// and the finish of the factored form the others.
 int launch_da(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, int dtype,
               const float* cs, float* ddA_intra, const DaWs& w, const Dims& d, hipStream_t st) {
   const int MT = (int)((d.Q + kBM - 1) / kBM);
@@ -497,8 +497,13 @@ int launch_da(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, int d
   EMA_TRY(launched());
   const int64_t total = d.N * d.C;
   hipLaunchKernelGGL(da_finish_kernel<kBM>, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, st, w.part,
-                     w.rowsum, ddA_intra, (int)d.Q, MT, total, flat ? w.flat : nullptr, only,
-                     da_flat_tiles(d, dtype));
+                     w.rowsum, ddA_intra, (int)d.Q, MT, total, only);
+  if (flat) {
+    EMA_TRY(launched());
+    const int64_t n = total * d.Q;
+    hipLaunchKernelGGL(da_flat_finish_kernel<256>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, w.flat, w.steep,
+                       ddA_intra, (int)d.Q, da_flat_tiles(d, dtype), n);
+  }
   return launched();
 }
 

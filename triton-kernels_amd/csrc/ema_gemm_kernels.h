@@ -177,27 +177,17 @@ __global__ __launch_bounds__(256, 2) void da_gemm_kernel(const T* __restrict__ x
 
 // B6, second part: ddA_intra[j] = sum_{i<j} (colsum[i] - rowsum[i]) with
 // colsum[i] = sum over the row tiles mt >= i / 128 of part[mt][i].  One wave per (n, c).
-// With flat (may be null) the chunks whose entry in steep is 0 take their result from there instead:
-// ddA_intra[j] = sum over the ntiles column tiles of flat[(chunk*ntiles + tile)*Q + j].
+// only (may be null): the chunks whose entry is 0 are left alone.
 template <int BM>
 __global__ __launch_bounds__(256) void da_finish_kernel(const float* __restrict__ part,
                                                         const float* __restrict__ rowsum,
                                                         float* __restrict__ ddA_intra, int Q,
                                                         int MT, int64_t total_chunks,
-                                                        const float* __restrict__ flat = nullptr,
-                                                        const int* __restrict__ steep = nullptr,
-                                                        int ntiles = 0) {
+                                                        const int* __restrict__ only = nullptr) {
   const int lane = threadIdx.x & 63;
   const int64_t chunk_id = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (chunk_id >= total_chunks) return;
-  if (flat && steep[chunk_id] == 0) {
-    for (int q = lane; q < Q; q += 64) {
-      float s = 0.f;
-      for (int ct = 0; ct < ntiles; ++ct) s += flat[(chunk_id * ntiles + ct) * (int64_t)Q + q];
-      ddA_intra[chunk_id * Q + q] = s;
-    }
-    return;
-  }
+  if (only && only[chunk_id] == 0) return;
   const int per = (Q + 63) >> 6;
   const int q0 = lane * per;
   auto val = [&](int q) {
@@ -216,6 +206,24 @@ __global__ __launch_bounds__(256) void da_finish_kernel(const float* __restrict_
       run += val(q);
     }
   }
+}
+
+// The same for the factored form, whose per-column-tile dots only have to be added up:
+// ddA_intra[chunk][q] = sum over the ntiles column tiles of flat[(chunk*ntiles + tile)*Q + q], for
+// the chunks whose entry in steep is 0.  One thread per (chunk, q).
+template <int BLOCK>
+__global__ __launch_bounds__(BLOCK) void da_flat_finish_kernel(const float* __restrict__ flat,
+                                                             const int* __restrict__ steep,
+                                                             float* __restrict__ ddA_intra, int Q,
+                                                             int ntiles, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (i >= total) return;
+  const int64_t chunk_id = i / Q;
+  if (steep[chunk_id] != 0) return;
+  const int q = (int)(i - chunk_id * Q);
+  float s = 0.f;
+  for (int ct = 0; ct < ntiles; ++ct) s += flat[(chunk_id * ntiles + ct) * (int64_t)Q + q];
+  ddA_intra[i] = s;
 }
 
 }  // namespace ema
