@@ -209,6 +209,21 @@ def test_bwd_da_intra_forms(shape, rising, dtype, device):
     assert float(got[..., 0].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("Q", [128, 256, 512, 640])
+def test_bwd_da_intra_headed_layout(Q, dtype, device):
+    """B6 on (b, L, nh, d) tensors consumed in place: the rows of a head are nh * d elements apart."""
+    from kernels.ema_kernels_bwd.ema_scan_da import _ema_chunk_scan_bwd_ddAcs_stable
+
+    announce(f"bwd_da_intra headed b2 L1100 nh3 d72 Q{Q} {dtype}")
+    x, A, dy = O.make_inputs(2, 3, 1100, 72, seed=31 + Q, dtype=dtype)
+    xf, Af = O.to_flat(x.float(), A)
+    dyf, _ = O.to_flat(dy.float(), A)
+    cs = O.chunk_cumsum(Af, Q)
+    got = _ema_chunk_scan_bwd_ddAcs_stable(x.to(device), cs.to(device), dy.to(device))
+    ref = O.bwd_da_intra(xf, cs, dyf)
+    check_close("ddA_intra", _valid(got, 1100), _valid(ref, 1100), dtype)
+
+
 def test_headed_layout_stages(device):
     """(b, L, nh, d) tensors and a (b, L, nh) log-decay are consumed in place (strided)."""
     from kernels.ema_kernels.ema_cumsum import ema_chunk_cumsum_fwd

@@ -271,13 +271,16 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), 1) void da_flat_kernel(
       float a[RPL];  // the decays of the wave's rows, in scalar registers for the rest of the sub-tile
 #pragma unroll
       for (int i = 0; i < RPL; ++i) a[i] = row_coef(av, RPL * t + i);
+      // (u[i] = dy[i] + a[i+1] * u[i+1], one multiply-add per element; the group hands on a[0] * u[0])
       float r[CPL];
 #pragma unroll
-      for (int e = 0; e < CPL; ++e) r[e] = 0.f;
+      for (int e = 0; e < CPL; ++e) r[e] = row_get<T, NW>(dr[RPL - 1], e);
 #pragma unroll
-      for (int i = RPL - 1; i >= 0; --i)
+      for (int i = RPL - 2; i >= 0; --i)
 #pragma unroll
-        for (int e = 0; e < CPL; ++e) r[e] = a[i] * (row_get<T, NW>(dr[i], e) + r[e]);
+        for (int e = 0; e < CPL; ++e) r[e] = fmaf(a[i + 1], r[e], row_get<T, NW>(dr[i], e));
+#pragma unroll
+      for (int e = 0; e < CPL; ++e) r[e] *= a[0];
 #pragma unroll
       for (int e = 0; e < CPL; ++e) sR[grp][lane_now() * CPL + e] = r[e];
       rows_opaque<NW, RPL>(dr);
@@ -324,12 +327,15 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), 1) void da_flat_kernel(
       // 2c. reverse pass with the dots, in segments of SEG of the wave's rows so that few forward
       // values are held at a time: for each segment, last first, the forward recurrence runs from the
       // state entering the group to the segment, its values over the segment are kept, and the reverse
-      // pass takes the segment's rows.  Behind the last use of a row the row that uses its registers
-      // next is requested.
+      // pass takes the segment's rows.  Behind the last use of an x row the row that uses its registers
+      // next is requested (keeping all forward values and requesting the next chunk's rows before the
+      // reverse pass was measured and is no faster: 0.1037 against 0.1019 ms at chunk 128).
       constexpr int SEG = KT >= 3 ? 2 : 4;
       const unsigned xp = opaque(xpitch);
-      float dA = 0.f;  // lane i reports row i of the wave
+      float dots[RPL];  // the rows' dots, summed over the wave (the same in every lane)
       const unsigned me = (unsigned)lane_now();
+      // r: a[i+1] * d[i+1] on entry for the wave's last row (what the rows after the group hand in),
+      // d[i+1] itself for the others, where d[i] = dy[i] + a[i+1] * d[i+1] is one multiply-add
 #pragma unroll
       for (int e = 0; e < CPL; ++e) r[e] = sR[grp][me * CPL + e];
 #pragma unroll
@@ -362,21 +368,25 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), 1) void da_flat_kernel(
           float dot = 0.f;
 #pragma unroll
           for (int e = 0; e < CPL; ++e) {
-            const float d = row_get<T, NW>(dr[i], e) + r[e];
+            const float d = i == RPL - 1 ? row_get<T, NW>(dr[i], e) + r[e] : fmaf(a[i + 1 < RPL ? i + 1 : i], r[e], row_get<T, NW>(dr[i], e));
             dot = fmaf(d, j > 0 ? yv[j - 1][e] : ym[e], dot);
-            r[e] = d * a[i];
+            r[e] = d;
           }
           if (more) xr[t][i] = flat_load_row<NW>(xdn, col_off(nx, (int)me) + row_off(t, i, xp));
-          // the row's dot goes into lane i (rows at or past the limit have dy = 0 and give 0)
-          const float total = wave_sum(dot) * a[i];
-          if (me == (unsigned)i) dA = total;
+          dots[i] = wave_sum(dot) * a[i];
         }
       }
       {
-        // a scalar base and this lane's row as a 32-bit offset, formed here and not kept
+        // (rows at or past the limit have dy = 0 and give 0); a scalar base and the lane's row as a
+        // 32-bit offset, formed here and not kept
+        float total = 0.f;  // lane i reports row i of the wave
+#pragma unroll
+        for (int i = 0; i < RPL; ++i)
+          if (me == (unsigned)i) total = dots[i];
+        const int row = (int)me;
         const int q0 = kTileRows * t + RPL * grp;
         float* pb = part + ((it.chunk_id * ntiles + it.ctile) * (int64_t)Q + q0);
-        if (me < (unsigned)RPL && q0 + (int)me < Q) pb[me] = dA;
+        if (me < (unsigned)RPL && q0 + row < Q) pb[row] = total;
       }
     }
     if (more) {
