@@ -493,6 +493,19 @@ def ssd_stages(torch, steps, warmup, only=None):
                                                            pick(i)[10], pick(i)[12]),
         "bwd_ddAcs": lambda i: _chunk_scan_bwd_ddAcs_stable(pick(i)[0], pick(i)[5], pick(i)[6], pick(i)[10], pick(i)[9]),
     }
+
+    def backward_pass(i):
+        """The backward stages chained as a caller would chain them (the reference has no combined
+        backward): the reverse walk's dstates feed dx and dB; one timed region, five launchers."""
+        x, _, _, B, Cm, dt_out, dA_cs, _, states, cb, dout = pick(i)[:11]
+        dstates, _, _ = _chunk_scan_state_passing_bwd(Cm, dA_cs, dout, states)
+        dstates = dstates.view(b, C, nh, P, N)
+        _chunk_scan_chunk_state_bwd_dx(x, dt_out, dA_cs, B, cb, dout, dstates)
+        _chunk_state_bwd_db(x, dt_out, dA_cs, dstates, B=B, ngroups=g)
+        _chunk_scan_bwd_dC(states, dA_cs, dout, C=Cm, ngroups=g)
+        _chunk_scan_bwd_ddAcs_stable(x, dt_out, dA_cs, dout, cb)
+
+    stages["backward_pass"] = backward_pass
     xb = b * L * nh * P * 2
     bc = b * L * g * N * 2
     dtb = b * L * nh * 4
@@ -511,6 +524,8 @@ def ssd_stages(torch, steps, warmup, only=None):
         "bwd_db": xb + pvb + 2 * dtb + bc + 2 * bc + dtb, "bwd_dc": xb + pvb + dtb + bc + 2 * bc + dtb,
         "bwd_dx": cbb + 3 * xb + bc + pvb + 3 * dtb, "bwd_ddAcs": 2 * xb + 3 * dtb + cbb,
     }
+    # in and out of the chained backward: x, dout, B, C, cb, dt, dA, states read; dx, dB, dC, ddt, ddA (x2) written
+    nbytes["backward_pass"] = 3 * xb + 4 * bc + cbb + 5 * dtb + pvb
     units = b * C * nh
     flops = {"chunk_state": 2 * Q * P * N * units, "chunk_state_passing": 2 * Q * P * N * units, "bmm_chunk": 2 * Q * Q * N * b * C * g,
              "chunk_scan": (2 * Q * Q * P + 2 * Q * N * P) * units, "bwd_dstates": 2 * Q * P * N * units,
@@ -847,6 +862,9 @@ def main():
                         "backward_stages_sum_ms": s5["backward_stages_sum"]["ms"],
                         # with bwd_dstates and bwd_state_passing replaced by bwd_dstates_state_passing
                         "backward_sum_with_reverse_walk_ms": s5["backward_sum_with_reverse_walk"]["ms"],
+                        # the same five launchers chained in one timed region, dstates flowing from the
+                        # reverse walk into dx and dB
+                        "backward_pass_ms": s5["backward_pass"]["ms"],
                         "stages": s5}
         torch.cuda.empty_cache()
         out["configs"] = cfgs
