@@ -224,6 +224,28 @@ def test_bwd_da_intra_headed_layout(Q, dtype, device):
     check_close("ddA_intra", _valid(got, 1100), _valid(ref, 1100), dtype)
 
 
+@pytest.mark.parametrize("Q", [128, 256, 512])
+def test_bwd_da_intra_bench_shape(Q, device):
+    """B6 at the benchmark's size (b16 nh2 d1024 L4096, bfloat16): the factored form against the oracle's
+    product form, which is evaluated here with torch on the device (268 MB of Q x Q blocks at Q = 512)."""
+    from kernels.ema_kernels.ema_cumsum import ema_chunk_cumsum_fwd
+    from kernels.ema_kernels_bwd.ema_scan_da import _ema_chunk_scan_bwd_ddAcs_stable
+
+    announce(f"bwd_da_intra b16 nh2 d1024 L4096 Q{Q} bf16")
+    gen = torch.Generator(device=device).manual_seed(400 + Q)
+    N, L, T = 32, 4096, 1024
+    X = torch.randn(N, L, T, generator=gen, device=device).to(BF16)
+    dy = torch.randn(N, L, T, generator=gen, device=device).to(BF16)
+    A = torch.nn.functional.logsigmoid(torch.randn(N, L, generator=gen, device=device) + 2.0)
+    cs = ema_chunk_cumsum_fwd(A, Q)
+    got = _ema_chunk_scan_bwd_ddAcs_stable(X, cs, dy)
+    ref = torch.cat([O.bwd_da_intra(X[n0:n0 + 8].float(), cs[n0:n0 + 8], dy[n0:n0 + 8].float()) for n0 in range(0, N, 8)])
+    check_close("ddA_intra", got, ref, BF16)
+    # linearity in dy, which no chunking or tiling may break
+    got2 = _ema_chunk_scan_bwd_ddAcs_stable(X, cs, (2 * dy.float()).to(BF16))
+    check_close("ddA_intra(2 dy)", got2, 2 * got, F32)
+
+
 def test_headed_layout_stages(device):
     """(b, L, nh, d) tensors and a (b, L, nh) log-decay are consumed in place (strided)."""
     from kernels.ema_kernels.ema_cumsum import ema_chunk_cumsum_fwd
