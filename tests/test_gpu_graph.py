@@ -56,6 +56,57 @@ def test_step_in_hip_graph(dtype, device):
     check_close("last replay vs oracle", y_g, O.from_flat(O.ema_loop(xf, Af), b, nh), dtype)
 
 
+@pytest.mark.parametrize("Q", [128, 512])
+def test_da_intra_in_hip_graph(Q, device):
+    """The B6 launcher in a graph: the factored form (copies into LDS, a flag per chunk, nothing cleared
+    by memset) and, for the chunks of the replay inputs whose cumsum rises, the product form behind it.
+    Replays see new inputs, some with rising chunks and some without."""
+    from kernels.ema_kernels.ema_cumsum import ema_chunk_cumsum_fwd
+    from kernels.ema_kernels_bwd.ema_scan_da import _ema_chunk_scan_bwd_ddAcs_stable
+    from parity_util import flat_case
+
+    announce(f"hip graph: B6 Q{Q}")
+    N, L, T = 3, 1100, 264
+    dtype = torch.bfloat16
+
+    def inputs(seed, rising):
+        A, X, dy = flat_case(N, L, T, seed=seed, dtype=dtype)
+        if rising:
+            A = A.clone()
+            A[:, 5::Q] = 0.2  # one rising step in every chunk
+        return A.to(device), X.to(device), dy.to(device)
+
+    As, Xs, dys = inputs(1, False)
+
+    def run():
+        cs = ema_chunk_cumsum_fwd(As, Q)
+        return _ema_chunk_scan_bwd_ddAcs_stable(Xs, cs, dys), cs
+
+    run()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream(device)
+    side.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            run()
+    torch.cuda.current_stream(device).wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g, cs_g = run()
+    for rep, rising in enumerate([True, False, True]):
+        A2, X2, dy2 = inputs(50 + rep, rising)
+        As.copy_(A2); Xs.copy_(X2); dys.copy_(dy2)
+        ref, _ = run()
+        ref = ref.clone()
+        torch.cuda.synchronize()
+        out_g.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, ref), f"replay {rep}: differs from the eager result"
+        want = O.bwd_da_intra(X2.float().cpu(), cs_g.cpu(), dy2.float().cpu())
+        check_close(f"replay {rep} vs oracle", out_g.reshape(N, -1)[:, :L], want.reshape(N, -1)[:, :L], dtype)
+
+
 @pytest.mark.parametrize("packed", [False, True], ids=["plain", "packed"])
 def test_ssd_forward_and_backward_stages_in_hip_graph(packed, device):
     """The Mamba-2 SSD launchers enqueue kernels only as well: the five forward stages and the six
