@@ -231,9 +231,10 @@ size_t ema_chunk_scan_bwd_ddAcs_workspace_bytes(int64_t batch, int64_t nheads, i
 
 /* B6: G[m,k] = exp(min(cs[m]-cs[k],0)) * <dy[m], x[k]> for k < m;
  * ddA_intra[j] = sum_{m>=j} sum_{k<j} G[m,k], ddA_intra[0] = 0.  Output (N,C,Q).
- * Chunks of up to 512 rows in which cs never rises (every decay) are evaluated in the factored form
+ * Chunks in which cs never rises (every decay) are evaluated in the factored form
  * ddA_intra[j] = exp(cs[j]-cs[j-1]) * <r[j], y[j-1]> with the chunk-local scans y of x and r of dy,
- * in float32 and in a time that does not grow with the chunk; the others by the product itself.
+ * in float32: one pass over x and dy for chunks of up to 512 rows, x read twice for longer ones;
+ * chunks in which cs rises somewhere by the product itself, with the pairwise minimum.
  * Replaces _ema_chunk_scan_bwd_ddAcs_stable,
  * kernels/ema_kernels_bwd/ema_scan_da.py:113-137. */
 int ema_chunk_scan_bwd_ddAcs(const void* x, int64_t x_sb, int64_t x_sl, int64_t x_sh,

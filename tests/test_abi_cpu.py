@@ -50,12 +50,11 @@ def test_workspace_sizes():
     assert handle.ema_seq_bwd_workspace_bytes(16, 2, 4096, 1024) == chain + 8 * 32 * 4096 * 4  # partials per 128 (float32) columns
     assert handle.ema_state_passing_bwd_workspace_bytes(32, 32, 1024) == 32 * 32 * 16 * 4
     # B6: column sums per row tile and row sums of the product form, dots per column tile (4 of 256
-    # bfloat16 columns, 8 of 128 float32 columns) and one flag per chunk of the factored form; chunks
-    # past 512 rows take the product form only
+    # bfloat16 columns, 8 of 128 float32 columns) and one flag per chunk of the factored form
     da = 2 * 32 * 32 * 128 * 4
     assert handle.ema_chunk_scan_bwd_ddAcs_workspace_bytes(16, 2, 4096, 1024, 128, _lib.EMA_BF16) == da + 4 * 32 * 32 * 128 * 4 + 32 * 32 * 4
     assert handle.ema_chunk_scan_bwd_ddAcs_workspace_bytes(16, 2, 4096, 1024, 128, _lib.EMA_F32) == da + 8 * 32 * 32 * 128 * 4 + 32 * 32 * 4
-    assert handle.ema_chunk_scan_bwd_ddAcs_workspace_bytes(16, 2, 4096, 1024, 1024, _lib.EMA_BF16) == (8 + 1) * 32 * 4 * 1024 * 4
+    assert handle.ema_chunk_scan_bwd_ddAcs_workspace_bytes(16, 2, 4096, 1024, 1024, _lib.EMA_BF16) == (8 + 1 + 4) * 32 * 4 * 1024 * 4 + 32 * 4 * 4
     assert handle.ema_chunk_scan_bwd_ddAcs_workspace_bytes(16, 2, 4096, 1024, 128, 7) == 0
     assert handle.ema_bwd_workspace_bytes(16, 2, 4096, 1024, 128) > 4 * 32 * 32 * 1024 * 4
     assert handle.ema_bwd_workspace_bytes(16, 2, 4096, 1024, 512) == handle.ema_bwd_workspace_bytes(16, 2, 4096, 1024, 128)

@@ -56,7 +56,7 @@ def test_step_in_hip_graph(dtype, device):
     check_close("last replay vs oracle", y_g, O.from_flat(O.ema_loop(xf, Af), b, nh), dtype)
 
 
-@pytest.mark.parametrize("Q", [128, 512])
+@pytest.mark.parametrize("Q", [128, 512, 640])
 def test_da_intra_in_hip_graph(Q, device):
     """The B6 launcher in a graph: the factored form (copies into LDS, a flag per chunk, nothing cleared
     by memset) and, for the chunks of the replay inputs whose cumsum rises, the product form behind it.

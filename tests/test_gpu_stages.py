@@ -170,8 +170,9 @@ def test_bwd_da_intra(case, device):
     assert float(got[..., 0].abs().max()) == 0.0
 
 
-# (N, L, T, Q) for B6 alone: chunks of one to four 128-row sub-tiles with ragged ends, a feature
-# width that is no multiple of the column tile, and a chunk too long for the factored form
+# (N, L, T, Q) for B6 alone: chunks of one to eight 128-row sub-tiles with ragged ends (up to four
+# sub-tiles keep their x rows in registers, longer chunks read x twice) and a feature width that is
+# no multiple of the column tile
 DA_SHAPES = [
     (2, 1000, 320, 200),
     (1, 900, 1024, 300),
@@ -179,6 +180,8 @@ DA_SHAPES = [
     (2, 2048, 512, 512),
     (2, 1500, 136, 500),
     (1, 1300, 72, 640),
+    (1, 2100, 264, 1000),
+    (2, 2048, 512, 1024),
 ]
 
 
@@ -209,7 +212,7 @@ def test_bwd_da_intra_forms(shape, rising, dtype, device):
     assert float(got[..., 0].abs().max()) == 0.0
 
 
-@pytest.mark.parametrize("Q", [128, 256, 512, 640])
+@pytest.mark.parametrize("Q", [128, 256, 512, 640, 1024])
 def test_bwd_da_intra_headed_layout(Q, dtype, device):
     """B6 on (b, L, nh, d) tensors consumed in place: the rows of a head are nh * d elements apart."""
     from kernels.ema_kernels_bwd.ema_scan_da import _ema_chunk_scan_bwd_ddAcs_stable
@@ -224,7 +227,7 @@ def test_bwd_da_intra_headed_layout(Q, dtype, device):
     check_close("ddA_intra", _valid(got, 1100), _valid(ref, 1100), dtype)
 
 
-@pytest.mark.parametrize("Q", [128, 256, 512])
+@pytest.mark.parametrize("Q", [128, 256, 512, 1024])
 def test_bwd_da_intra_bench_shape(Q, device):
     """B6 at the benchmark's size (b16 nh2 d1024 L4096, bfloat16): the factored form against the oracle's
     product form, which is evaluated here with torch on the device (268 MB of Q x Q blocks at Q = 512)."""

@@ -412,13 +412,16 @@ constexpr int kFlatLongDiv = sizeof(T) == 4 ? 2 : 1;
 inline int da_flat_cols(const Dims& d, int dtype) {
   const int wide = dtype == EMA_BF16 ? 64 * TileBf16::BWD_CPL : 64 * TileF32::BWD_CPL;
   const int div = dtype == EMA_BF16 ? kFlatLongDiv<bf16_t> : kFlatLongDiv<float>;
-  return d.Q > 2 * kTileRows ? wide / div : wide;
+  return d.Q > 2 * kTileRows && d.Q <= 4 * kTileRows ? wide / div : wide;
 }
 inline int da_flat_tiles(const Dims& d, int dtype) {
   const int bn = da_flat_cols(d, dtype);
   return (int)((d.T + bn - 1) / bn);
 }
-constexpr int kFlatMaxChunk = 4 * kTileRows;  // the factored form keeps a chunk's x rows in registers
+// The factored form takes every chunk size the library does: up to four 128-row sub-tiles with the
+// chunk's x rows kept in registers, more with x read twice.
+constexpr int kFlatMaxChunk = EMA_MAX_CHUNK;
+constexpr int kFlatMaxKept = 4 * kTileRows;
 DaWs carve_da(void* base, const Dims& d, int dtype) {
   DaWs w;
   size_t off = 0;
@@ -454,10 +457,27 @@ int launch_da_flat_k(const void* x, SeqStrides sx, const void* dy, SeqStrides sd
                      ntiles, (int)total);
   return launched();
 }
+template <typename T, int CPL, int RPL>
+int launch_da_flat_long(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* cs,
+                        const DaWs& w, const Dims& d, hipStream_t st) {
+  using Cfg = TileCfg<T, CPL, RPL>;
+  constexpr int smem = FlatLongCfg<T, CPL, RPL>::smem_bytes;
+  const int ntiles = (int)((d.T + Cfg::BN - 1) / Cfg::BN);
+  const int64_t total = d.N * d.C * ntiles;
+  if (total > 0x7fffffff) return EMA_ERR_SHAPE;
+  auto kernel = da_flat_long_kernel<T, CPL, RPL>;
+  EMA_TRY(allow_smem(kernel, smem));
+  const int64_t cap = resident_blocks(kernel, Cfg::NT, smem);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(total < cap ? total : cap)), dim3(Cfg::NT), smem, st, (const T*)x, sx,
+                     (const T*)dy, sd, cs, w.flat, w.steep, (int)d.nh, (int)d.L, (int)d.T, (int)d.Q, (int)d.C,
+                     ntiles, (int)total);
+  return launched();
+}
 template <typename T, typename S>
 int launch_da_flat(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, const float* cs,
                    const DaWs& w, const Dims& d, hipStream_t st) {
   constexpr int CPL = S::BWD_CPL, RPL = S::BWD_RPL;
+  if (d.Q > kFlatMaxKept) return launch_da_flat_long<T, CPL, RPL>(x, sx, dy, sd, cs, w, d, st);
   static_assert(CPL % kFlatLongDiv<T> == 0, "long chunks take a part of the columns");
   switch ((d.Q + kTileRows - 1) / kTileRows) {
     case 1: return launch_da_flat_k<T, CPL, RPL, 1>(x, sx, dy, sd, cs, w, d, st);
@@ -467,9 +487,9 @@ int launch_da_flat(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, 
   }
 }
 
-// B6.  Chunks of up to 512 rows go through the factored form first; the kernel that forms the
-// product and its finish then take the chunks in which the cumsum rises somewhere (none, for decays)
-// and the finish of the factored form the others.
+// B6.  Every chunk goes through the factored form first; the kernel that forms the product and its
+// finish then take the chunks in which the cumsum rises somewhere (none, for decays) and the finish
+// of the factored form the others.
 int launch_da(const void* x, SeqStrides sx, const void* dy, SeqStrides sd, int dtype,
               const float* cs, float* ddA_intra, const DaWs& w, const Dims& d, hipStream_t st) {
   const int MT = (int)((d.Q + kBM - 1) / kBM);

@@ -397,4 +397,320 @@ __global__ __launch_bounds__(64 * (kTileRows / RPL), 1) void da_flat_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------
+// The same for chunks of more than four sub-tiles (up to EMA_MAX_CHUNK rows), whose x rows do not fit
+// the registers: x is read twice.  A first walk over the sub-tiles 0 .. K-2 only finds the forward
+// state at every sub-tile boundary (local pass, one chain over the row groups, nothing kept but BN
+// floats per boundary); the second walk, from the last sub-tile to the first, reads x again next to
+// dy and does what da_flat_kernel does per sub-tile, with the local forward pass and the forward
+// chain inside the step.  The decays of the whole chunk sit in LDS (one thread per row forms them
+// at the start of a chunk).  Traffic: (3 K - 1) / (2 K) of the algorithmic bytes' x + dy.
+// ------------------------------------------------------------------------------------
+template <typename T, int CPL, int RPL>
+struct FlatLongCfg {
+  using W = TileCfg<T, CPL, RPL>;
+  static constexpr int kMaxSub = EMA_MAX_CHUNK_DEV / kTileRows;
+  static constexpr int kFloats = 2 * W::NG * W::BN    // forward and reverse group states
+                                 + kMaxSub * W::BN    // forward state at the sub-tile boundaries
+                                 + EMA_MAX_CHUNK_DEV  // the chunk's decays
+                                 + W::NG + 4;         // group decays, flag
+  static constexpr int kRowBytes = W::BN * (int)sizeof(T);
+  static constexpr int smem_bytes = kFloats * (int)sizeof(float) + kTileRows * kRowBytes;
+  static_assert(kFloats % 4 == 0, "the staged rows start at a multiple of 16 bytes");
+  static_assert(smem_bytes <= 160 * 1024, "LDS of one compute unit");
+};
+
+template <typename T, int CPL, int RPL>
+__global__ __launch_bounds__(64 * (kTileRows / RPL), 1) void da_flat_long_kernel(
+    const T* __restrict__ x, SeqStrides sx, const T* __restrict__ dy, SeqStrides sd,
+    const float* __restrict__ cs, float* __restrict__ part, int* __restrict__ steep, int nh, int L, int Tdim,
+    int Q, int C, int ntiles, int total) {
+  using W = TileCfg<T, CPL, RPL>;
+  using F = FlatLongCfg<T, CPL, RPL>;
+  constexpr int BN = W::BN, NW = W::NW, NG = W::NG, NT = W::NT;
+  static_assert(2 * BN <= NT, "one thread per column and direction");
+  static_assert(NT >= EMA_MAX_CHUNK_DEV, "one thread per row of a chunk");
+  extern __shared__ __attribute__((aligned(16))) float flat_smem[];
+  float (*sS)[BN] = reinterpret_cast<float (*)[BN]>(flat_smem);
+  float (*sR)[BN] = reinterpret_cast<float (*)[BN]>(flat_smem + NG * BN);
+  float (*sY)[BN] = reinterpret_cast<float (*)[BN]>(flat_smem + 2 * NG * BN);
+  float* const sA = flat_smem + 2 * NG * BN + F::kMaxSub * BN;
+  float* const sD = sA + EMA_MAX_CHUNK_DEV;
+  int* const sFlag = reinterpret_cast<int*>(sD + NG);
+  const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  constexpr int ROWB = F::kRowBytes, LPR = ROWB / 16, RPI = 64 / LPR, NCOPY = RPL / RPI;
+  static_assert(RPL % RPI == 0, "whole rows per copy");
+  char* const stage = reinterpret_cast<char*>(flat_smem + F::kFloats) + grp * (RPL * ROWB);
+  const int K = (Q + kTileRows - 1) / kTileRows;
+
+  auto opaque = [](unsigned v) {
+    asm volatile("" : "+s"(v));
+    return v;
+  };
+  if (threadIdx.x == 0) *sFlag = 0;
+  __syncthreads();
+  auto lane_now = [&]() {
+    return (int)__builtin_amdgcn_mbcnt_hi(opaque(~0u), __builtin_amdgcn_mbcnt_lo(opaque(~0u), 0u));
+  };
+  struct Item {
+    int64_t chunk_id, xbase, dbase;
+    int ctile, limit, ncols;
+  };
+  auto decode = [&](int w) {
+    Item it;
+    it.ctile = w % ntiles;
+    it.chunk_id = w / ntiles;
+    const int64_t n = it.chunk_id / C;
+    const int c = (int)(it.chunk_id - n * C);
+    const int64_t b = n / nh;
+    const int h = (int)(n - b * nh);
+    const int col0 = it.ctile * BN;
+    it.limit = min(Q, L - c * Q);
+    it.ncols = min(BN, Tdim - col0);
+    it.xbase = b * sx.sb + h * sx.sh + (int64_t)c * Q * sx.sl + col0;
+    it.dbase = b * sd.sb + h * sd.sh + (int64_t)c * Q * sd.sl + col0;
+    return it;
+  };
+  const unsigned xpitch = (unsigned)sx.sl * (unsigned)sizeof(T), dpitch = (unsigned)sd.sl * (unsigned)sizeof(T);
+  // the x rows of this wave in sub-tile t of chunk c, through the chunk's descriptor
+  auto x_request = [&](RowWords<NW>* rows, __amdgpu_buffer_rsrc_t desc, const Item& c, int t) {
+    const int ln = lane_now();
+    const unsigned col = ln * CPL < c.ncols ? (unsigned)ln * (unsigned)(CPL * sizeof(T)) : kFlatNoColumn;
+    const unsigned row0 = (unsigned)(kTileRows * t + RPL * grp) * opaque(xpitch);
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) rows[i] = flat_load_row<NW>(desc, col + row0 + (unsigned)i * xpitch);
+  };
+  // this thread's row of the chunk: cs[q] - cs[q-1] (cs[0] itself for row 0, 0 at or past the limit)
+  auto coef_load = [&](const Item& c) {
+    const int q = 64 * grp + lane_now();
+    float raw = 0.f;
+    if (q < c.limit) {
+      const float* p = cs + c.chunk_id * Q + q;
+      raw = p[0] - (q > 0 ? p[-1] : 0.f);
+    }
+    return raw;
+  };
+  auto dy_request = [&](const Item& c, int t) {
+    const T* base = dy + c.dbase;
+    const int me = lane_now();
+    const unsigned colb = min((unsigned)(me % LPR) * 16u, (unsigned)c.ncols * (unsigned)sizeof(T) - 16u);
+#pragma unroll
+    for (int j = 0; j < NCOPY; ++j) {
+      const int row = min(kTileRows * t + RPL * grp + RPI * j + me / LPR, c.limit - 1);
+      flat_copy16_to_lds(base, (unsigned)row * dpitch + colb, stage + j * 1024);
+    }
+  };
+  auto dy_take = [&](RowWords<NW>* rows, const Item& c, int t) {
+    const int nrows = c.limit - (kTileRows * t + RPL * grp);
+    const int ln = lane_now();
+    const bool cok = ln * CPL < c.ncols;
+    const bool full = nrows >= RPL && __all(cok);
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+      rows[i] = *reinterpret_cast<const RowWords<NW>*>(stage + i * ROWB + ln * (CPL * (int)sizeof(T)));
+      if (!full && !(i < nrows && cok)) rows[i] = row_zero<NW>();
+    }
+  };
+  // the decays of this wave's rows of sub-tile t, from LDS into scalar registers
+  auto decays = [&](float* a, int t) {
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) a[i] = wave_uniform(sA[kTileRows * t + RPL * grp + i]);
+  };
+  // local forward pass over the rows of a sub-tile: the group's state and decay into LDS
+  auto local_forward = [&](const RowWords<NW>* rows, const float* a) {
+    float s[CPL], D = 1.f;
+#pragma unroll
+    for (int e = 0; e < CPL; ++e) s[e] = 0.f;
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+      D *= a[i];
+#pragma unroll
+      for (int e = 0; e < CPL; ++e) s[e] = fmaf(a[i], s[e], row_get<T, NW>(rows[i], e));
+    }
+    const int ln = lane_now();
+#pragma unroll
+    for (int e = 0; e < CPL; ++e) sS[grp][ln * CPL + e] = s[e];
+    if (ln == 0) sD[grp] = D;
+  };
+  constexpr int CW = BN / 64;  // waves with one thread per column
+
+  RowWords<NW> xr[RPL], dr[RPL];
+  float craw = 0.f;
+  int w = blockIdx.x;
+  Item it = decode(w < total ? w : 0);
+  if (w < total) {
+    x_request(xr, flat_rows_desc(x + it.xbase, sx.sl, it.limit, it.ncols), it, 0);
+    craw = coef_load(it);
+  }
+  while (w < total) {
+    const int wn = w + (int)gridDim.x;
+    const bool more = wn < total;
+    const Item nx = decode(more ? wn : 0);
+    const __amdgpu_buffer_rsrc_t xd = flat_rows_desc(x + it.xbase, sx.sl, it.limit, it.ncols);
+    const __amdgpu_buffer_rsrc_t xdn = flat_rows_desc(x + nx.xbase, sx.sl, nx.limit, nx.ncols);
+    {
+      // the chunk's decays, the flag of a rising cumsum, a zero state before the first row
+      const int ln = lane_now(), q = 64 * grp + ln;
+      sA[q] = __expf(fminf(craw, 0.f));
+      if (__any(craw > 0.f && q > 0) && ln == 0) *sFlag = 1;
+      if (q < BN) sY[0][q] = 0.f;
+    }
+    __syncthreads();
+
+    // 1. the forward state at the sub-tile boundaries
+    for (int t = 0; t < K - 1; ++t) {
+      float a[RPL];
+      decays(a, t);
+      local_forward(xr, a);
+      rows_opaque<NW, RPL>(xr);
+      // the rows of the sub-tile after this one, which the next step needs whichever walk it belongs
+      // to; before the last of them the copies of the last sub-tile's dy rows
+      if (t == K - 2) dy_request(it, K - 1);
+      x_request(xr, xd, it, t + 1);
+      __syncthreads();
+      if (grp < CW) {
+        const int k = 64 * grp + lane_now();
+        float sg[NG], dg[NG];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) sg[g] = sS[g][k];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) dg[g] = wave_uniform(sD[g]);
+        float E = sY[t][k];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) E = fmaf(dg[g], E, sg[g]);
+        sY[t + 1][k] = E;
+      }
+      __syncthreads();
+    }
+
+    // 2. sub-tiles from the last to the first
+    float h_in = 0.f;  // chain threads: reverse state entering the sub-tile from the rows after it
+    for (int t = K - 1; t >= 0; --t) {
+      // The copies of this sub-tile's dy rows were requested a step ago and the RPL x rows of this step
+      // after them: once at most RPL newer operations are under way they have landed.
+      __builtin_amdgcn_sched_barrier(0);
+      flat_wait_loads<RPL>();
+      dy_take(dr, it, t);
+      if (t > 0) dy_request(it, t - 1);
+      __builtin_amdgcn_sched_barrier(0);
+      float a[RPL];
+      decays(a, t);
+      // 2a. local passes: reverse over dy (u[i] = dy[i] + a[i+1] * u[i+1]; the group hands on a[0] * u[0]),
+      // forward over x
+      float r[CPL];
+#pragma unroll
+      for (int e = 0; e < CPL; ++e) r[e] = row_get<T, NW>(dr[RPL - 1], e);
+#pragma unroll
+      for (int i = RPL - 2; i >= 0; --i)
+#pragma unroll
+        for (int e = 0; e < CPL; ++e) r[e] = fmaf(a[i + 1], r[e], row_get<T, NW>(dr[i], e));
+      {
+        const int ln = lane_now();
+#pragma unroll
+        for (int e = 0; e < CPL; ++e) sR[grp][ln * CPL + e] = r[e] * a[0];
+      }
+      local_forward(xr, a);
+      rows_opaque<NW, RPL>(dr);
+      rows_opaque<NW, RPL>(xr);
+      __syncthreads();
+
+      // 2b. chains over the row groups
+      if (grp < CW) {
+        const int k = 64 * grp + lane_now();
+        if (t == K - 1 && k == 0) {
+          if (it.ctile == 0) steep[it.chunk_id] = *sFlag;
+          *sFlag = 0;
+        }
+        float rg[NG], dg[NG];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) rg[g] = sR[g][k];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) dg[g] = wave_uniform(sD[g]);
+#pragma unroll
+        for (int g = NG - 1; g >= 0; --g) {
+          sR[g][k] = h_in;
+          h_in = fmaf(dg[g], h_in, rg[g]);
+        }
+      } else if (grp < 2 * CW) {
+        const int kf = 64 * (grp - CW) + lane_now();
+        float sg[NG], dg[NG];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) sg[g] = sS[g][kf];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) dg[g] = wave_uniform(sD[g]);
+        float E = sY[t][kf];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+          sS[g][kf] = E;
+          E = fmaf(dg[g], E, sg[g]);
+        }
+      }
+      __syncthreads();
+
+      // 2c. reverse pass with the dots, in two segments of the wave's rows (as in da_flat_kernel);
+      // behind the last use of an x row the same row of the step after this one is requested
+      constexpr int SEG = 4;
+      const unsigned me = (unsigned)lane_now();
+      const bool next_x = t > 0 || more;
+      const __amdgpu_buffer_rsrc_t xnext = t > 0 ? xd : xdn;
+      const unsigned xcol = (t > 0 ? (int)me * CPL < it.ncols : (int)me * CPL < nx.ncols)
+                                ? me * (unsigned)(CPL * sizeof(T)) : kFlatNoColumn;
+      const unsigned xrow0 = (unsigned)(kTileRows * (t > 0 ? t - 1 : 0) + RPL * grp) * opaque(xpitch);
+      float dots[RPL];
+#pragma unroll
+      for (int e = 0; e < CPL; ++e) r[e] = sR[grp][me * CPL + e];
+#pragma unroll
+      for (int i0 = RPL - SEG; i0 >= 0; i0 -= SEG) {
+        __builtin_amdgcn_sched_barrier(0);
+        float ym[CPL];
+#pragma unroll
+        for (int e = 0; e < CPL; ++e) ym[e] = sS[grp][me * CPL + e];
+#pragma unroll
+        for (int i = 0; i < i0; ++i)
+#pragma unroll
+          for (int e = 0; e < CPL; ++e) ym[e] = fmaf(a[i], ym[e], row_get<T, NW>(xr[i], e));
+        float yv[SEG - 1][CPL];
+        {
+          float s[CPL];
+#pragma unroll
+          for (int e = 0; e < CPL; ++e) s[e] = ym[e];
+#pragma unroll
+          for (int i = 0; i < SEG - 1; ++i)
+#pragma unroll
+            for (int e = 0; e < CPL; ++e) {
+              s[e] = fmaf(a[i0 + i], s[e], row_get<T, NW>(xr[i0 + i], e));
+              yv[i][e] = s[e];
+            }
+        }
+#pragma unroll
+        for (int j = SEG - 1; j >= 0; --j) {
+          __builtin_amdgcn_sched_barrier(0);
+          const int i = i0 + j;
+          float dot = 0.f;
+#pragma unroll
+          for (int e = 0; e < CPL; ++e) {
+            const float d = i == RPL - 1 ? row_get<T, NW>(dr[i], e) + r[e] : fmaf(a[i + 1 < RPL ? i + 1 : i], r[e], row_get<T, NW>(dr[i], e));
+            dot = fmaf(d, j > 0 ? yv[j - 1][e] : ym[e], dot);
+            r[e] = d;
+          }
+          if (next_x) xr[i] = flat_load_row<NW>(xnext, xcol + xrow0 + (unsigned)i * xpitch);
+          dots[i] = wave_sum(dot) * a[i];
+        }
+      }
+      {
+        float total = 0.f;  // lane i reports row i of the wave
+#pragma unroll
+        for (int i = 0; i < RPL; ++i)
+          if (me == (unsigned)i) total = dots[i];
+        const int q0 = kTileRows * t + RPL * grp;
+        float* pb = part + ((it.chunk_id * ntiles + it.ctile) * (int64_t)Q + q0);
+        if (me < (unsigned)RPL && q0 + (int)me < Q) pb[me] = total;
+      }
+    }
+    if (more) craw = coef_load(nx);
+    w = wn;
+    it = nx;
+  }
+}
+
 }  // namespace ema

@@ -1,6 +1,6 @@
-"""B6, intra-chunk log-decay gradient.  Chunks of up to 512 rows whose cumsum never rises take the
-factored form (two chunk-local scans and one dot per row); the others the dout . x^T contraction
-over the feature axis on MFMA, scaled by the segsum decays and reduced by a two-dimensional prefix.
+"""B6, intra-chunk log-decay gradient.  Chunks whose cumsum never rises take the factored form (two
+chunk-local scans and one dot per row); the others the dout . x^T contraction over the feature axis
+on MFMA, scaled by the segsum decays and reduced by a two-dimensional prefix.
 
 Mirrors kernels/ema_kernels_bwd/ema_scan_da.py:113-137 of the reference."""
 import torch
